@@ -1,0 +1,585 @@
+/*
+ * CPU oracle for the Minerva operator layer.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file restates, in plain single-threaded C, the arithmetic of the
+ * reference's CPU "basic" operator implementation and, for the operators the
+ * reference only implements through cuDNN v2, the semantics of the cuDNN modes
+ * its CUDA path selects.  Nothing in the shipped library links, loads or calls
+ * this file; only the parity tests, the smoke check and the CPU-baseline leg of
+ * the benchmark do, and only as the checker / the timed baseline.
+ *
+ * Compile with -O2 -ffp-contract=off: MatMult is the only reference op with a
+ * multiply-add, and the reference's own bits depend on whether the host compiler
+ * contracts it, so contraction is pinned off here.
+ *
+ * Layout conventions (reference minerva/common/scale.cpp:182-191): every tensor
+ * is column-major, dimension 0 fastest.  Image batches are {W,H,C,N}, filters are
+ * {S(width),R(height),Cin,Cout}, matrices are {rows,cols}.
+ *
+ * Parity pins per function are listed next to each function ("pinned by").
+ * Functions whose arithmetic no reference test and no closed form pins carry the
+ * words "parity unpinned" and are pinned only by the mathematical identities the
+ * tests check (adjointness, finite differences, brute force).
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+#define ORA_MAX_DIMS 8
+
+/* ------------------------------------------------------------------------- */
+/* N-d index helpers: reference minerva/common/scale.cpp:98-128 and :182-191  */
+/* ------------------------------------------------------------------------- */
+
+static size_t ora_flatten(const int* idx, const int* dims, int nd) {
+  /* scale.cpp:182-191: offset = sum idx[i] * prod(dims[0..i-1]) */
+  size_t stride = 1, ret = 0;
+  for (int i = 0; i < nd; ++i) {
+    ret += (size_t)idx[i] * stride;
+    stride *= (size_t)dims[i];
+  }
+  return ret;
+}
+
+static int ora_contains(const int* set, int nset, int v) {
+  for (int i = 0; i < nset; ++i)
+    if (set[i] == v) return 1;
+  return 0;
+}
+
+/* scale.cpp:98-108 (IncrOne) */
+static int ora_incr_one(int* idx, const int* max, int nd) {
+  for (int i = 0; i < nd; ++i) {
+    if (idx[i] + 1 < max[i]) {
+      ++idx[i];
+      return 1;
+    }
+    idx[i] = 0;
+  }
+  return 0;
+}
+
+/* scale.cpp:110-128: step only dims in `sel` (pick=1) or only dims not in it */
+static int ora_incr_sel(int* idx, const int* max, int nd, const int* sel, int nsel, int pick) {
+  for (int i = 0; i < nd; ++i) {
+    if (ora_contains(sel, nsel, i) != pick) continue;
+    if (idx[i] + 1 < max[i]) {
+      ++idx[i];
+      return 1;
+    }
+    idx[i] = 0;
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Elementwise: basic.cpp:23-52, 54-107, 125-148                               */
+/* type: 0 add, 1 sub, 2 mul, 3 div (closure.h:8-13)                           */
+/* pinned by: single IEEE operation per element (closed form), reference tests */
+/* tests/unittest_arithmetic.cpp, unittest_arithmetic_const.cpp                */
+/* ------------------------------------------------------------------------- */
+
+int ora_arithmetic(int type, const float* a, const float* b, float* c, size_t n) {
+  switch (type) {
+    case 0: for (size_t i = 0; i < n; ++i) c[i] = a[i] + b[i]; break;
+    case 1: for (size_t i = 0; i < n; ++i) c[i] = a[i] - b[i]; break;
+    case 2: for (size_t i = 0; i < n; ++i) c[i] = a[i] * b[i]; break;
+    case 3: for (size_t i = 0; i < n; ++i) c[i] = a[i] / b[i]; break;
+    default: return 1;
+  }
+  return 0;
+}
+
+/* side 0: val (op) x ; side 1: x (op) val   (closure.h:94-98) */
+int ora_arithmetic_const(int type, int side, float val, const float* x, float* y, size_t n) {
+  if (side != 0 && side != 1) return 1;
+  switch (type) {
+    case 0:
+      if (side == 0) for (size_t i = 0; i < n; ++i) y[i] = val + x[i];
+      else           for (size_t i = 0; i < n; ++i) y[i] = x[i] + val;
+      break;
+    case 1:
+      if (side == 0) for (size_t i = 0; i < n; ++i) y[i] = val - x[i];
+      else           for (size_t i = 0; i < n; ++i) y[i] = x[i] - val;
+      break;
+    case 2:
+      if (side == 0) for (size_t i = 0; i < n; ++i) y[i] = val * x[i];
+      else           for (size_t i = 0; i < n; ++i) y[i] = x[i] * val;
+      break;
+    case 3:
+      if (side == 0) for (size_t i = 0; i < n; ++i) y[i] = val / x[i];
+      else           for (size_t i = 0; i < n; ++i) y[i] = x[i] / val;
+      break;
+    default: return 1;
+  }
+  return 0;
+}
+
+/* type: 0 exp, 1 ln, 2 negate (closure.h:15-19); float overloads = expf/logf.
+ * pinned by: libm closed forms of tests/unittest_elewise.cpp:7-66 */
+int ora_elewise(int type, const float* x, float* y, size_t n) {
+  switch (type) {
+    case 0: for (size_t i = 0; i < n; ++i) y[i] = expf(x[i]); break;
+    case 1: for (size_t i = 0; i < n; ++i) y[i] = logf(x[i]); break;
+    case 2: for (size_t i = 0; i < n; ++i) y[i] = -x[i]; break;
+    default: return 1;
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* MatMult: basic.cpp:150-173 (non-CBLAS branch).  C{m,n} = A{m,k} * B{k,n}     */
+/* i, j outer; k inner, sequential fp32 accumulate starting from 0.            */
+/* pinned by: textbook triple loop of tests/unittest_sgemm.cpp:19-27, fp64 ref */
+/* ------------------------------------------------------------------------- */
+int ora_matmult(const float* a, const float* b, float* c, int m, int n, int k) {
+  for (int i = 0; i < m; ++i) {
+    for (int j = 0; j < n; ++j) {
+      float s = 0;
+      for (int l = 0; l < k; ++l) {
+        float p = a[i + (size_t)l * m] * b[l + (size_t)j * k];
+        s = s + p;
+      }
+      c[i + (size_t)j * m] = s;
+    }
+  }
+  return 0;
+}
+
+/* Same product with j outer / i inner loops and a k-blocked accumulation order
+ * identical per element to ora_matmult (each c[i,j] still sums l = 0..k-1 in
+ * order), only cache friendlier: used where the timed baseline or a test needs a
+ * larger product in seconds.  Bit-identical to ora_matmult by construction; the
+ * tests assert that. */
+int ora_matmult_fast(const float* a, const float* b, float* c, int m, int n, int k) {
+  for (int j = 0; j < n; ++j) {
+    float* cj = c + (size_t)j * m;
+    for (int i = 0; i < m; ++i) cj[i] = 0;
+    for (int l = 0; l < k; ++l) {
+      const float bl = b[l + (size_t)j * k];
+      const float* al = a + (size_t)l * m;
+      for (int i = 0; i < m; ++i) {
+        float p = al[i] * bl;
+        cj[i] = cj[i] + p;
+      }
+    }
+  }
+  return 0;
+}
+
+/* Transpose: basic.cpp:175-187.  in{n,m} -> out{m,n}; out[i + j*m] = in[j + i*n] */
+int ora_transpose(const float* in, float* out, int m, int n) {
+  for (int i = 0; i < m; ++i)
+    for (int j = 0; j < n; ++j) out[i + (size_t)j * m] = in[j + (size_t)i * n];
+  return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Reduction: basic.cpp:189-217.  type 0 sum, 1 max.  N-d, any set of dims.    */
+/* For every output coordinate: start from the element with reduced dims = 0,  */
+/* then fold the rest in IncrDimensions order.                                 */
+/* pinned by: exact closed forms of tests/unittest_reduction.cpp:6-149          */
+/* ------------------------------------------------------------------------- */
+int ora_reduction(int type, const float* in, const int* dims, int nd, const int* rdims, int nr,
+                  float* out) {
+  if (nd > ORA_MAX_DIMS || (type != 0 && type != 1)) return 1;
+  int odims[ORA_MAX_DIMS], acc[ORA_MAX_DIMS], cur[ORA_MAX_DIMS];
+  for (int i = 0; i < nd; ++i) {
+    odims[i] = ora_contains(rdims, nr, i) ? 1 : dims[i];
+    acc[i] = 0;
+    if (dims[i] <= 0) return 1;
+  }
+  do {
+    memcpy(cur, acc, sizeof(int) * nd);
+    float tmp = in[ora_flatten(cur, dims, nd)];
+    while (ora_incr_sel(cur, dims, nd, rdims, nr, 1)) {
+      float t2 = in[ora_flatten(cur, dims, nd)];
+      if (type == 0) tmp += t2;
+      else if (tmp < t2) tmp = t2;
+    }
+    out[ora_flatten(acc, odims, nd)] = tmp;
+  } while (ora_incr_sel(acc, odims, nd, rdims, nr, 0));
+  return 0;
+}
+
+/* MaxIndex: basic.cpp:369-398.  Index (stored as float) of the first maximum
+ * along `dim`; strict '<' so the lowest index wins ties.
+ * pinned by: closed form (pure selection); compiled-reference value 4,4,4 on
+ * the {5,3} iota of tests/unittest_reduction.cpp recorded in the survey. */
+int ora_maxindex(const float* in, const int* dims, int nd, int dim, float* out) {
+  if (nd > ORA_MAX_DIMS || dim < 0 || dim >= nd) return 1;
+  int odims[ORA_MAX_DIMS], it[ORA_MAX_DIMS];
+  size_t interval = 1;
+  for (int i = 0; i < nd; ++i) {
+    odims[i] = (i == dim) ? 1 : dims[i];
+    it[i] = 0;
+    if (i < dim) interval *= (size_t)dims[i];
+  }
+  int strike = dims[dim];
+  do {
+    size_t off = ora_flatten(it, dims, nd);
+    float cur = in[off];
+    int index = 0;
+    for (int i = 0; i < strike; ++i) {
+      float v = in[off + (size_t)i * interval];
+      if (cur < v) {
+        cur = v;
+        index = i;
+      }
+    }
+    out[ora_flatten(it, odims, nd)] = (float)index;
+  } while (ora_incr_sel(it, odims, nd, &dim, 1, 0));
+  return 0;
+}
+
+/* NormArithmetic: basic.cpp:319-367.  out = in0 (op) broadcast(in1); in1 has
+ * size 1 on every replicated dim.  pinned by: single IEEE op per element;
+ * tests/unittest_norm_arithmetic.cpp:6-36 closed forms. */
+int ora_norm_arithmetic(int type, const float* in0, const int* dims, int nd, const float* in1,
+                        const int* rep, int nrep, float* out) {
+  if (nd > ORA_MAX_DIMS || type < 0 || type > 3) return 1;
+  int vdims[ORA_MAX_DIMS], it[ORA_MAX_DIMS], iv[ORA_MAX_DIMS];
+  size_t total = 1;
+  for (int i = 0; i < nd; ++i) {
+    vdims[i] = ora_contains(rep, nrep, i) ? 1 : dims[i];
+    it[i] = 0;
+    total *= (size_t)dims[i];
+  }
+  if (total == 0) return 0;
+  int more = 1;
+  while (more) {
+    for (int i = 0; i < nd; ++i) iv[i] = ora_contains(rep, nrep, i) ? 0 : it[i];
+    float cur = in1[ora_flatten(iv, vdims, nd)];
+    size_t f = ora_flatten(it, dims, nd);
+    switch (type) {
+      case 0: out[f] = in0[f] + cur; break;
+      case 1: out[f] = in0[f] - cur; break;
+      case 2: out[f] = in0[f] * cur; break;
+      case 3: out[f] = in0[f] / cur; break;
+    }
+    more = ora_incr_one(it, dims, nd);
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Softmax forward over dim 0: basic.cpp:219-261.                              */
+/* m = max, e_i = expf(x_i - m), s = sequential sum of e_i from 0, y = e_i / s */
+/* `len` = dims[0], `cols` = product of the remaining dims.                    */
+/* pinned by: fp64 closed form; rows sum to 1 (survey check on compiled ref).  */
+/* ------------------------------------------------------------------------- */
+int ora_softmax_dim0(const float* in, float* out, int len, size_t cols) {
+  for (size_t c = 0; c < cols; ++c) {
+    const float* x = in + c * (size_t)len;
+    float* y = out + c * (size_t)len;
+    float mx = x[0];
+    for (int i = 1; i < len; ++i)
+      if (mx < x[i]) mx = x[i];
+    float s = 0;
+    for (int i = 0; i < len; ++i) {
+      y[i] = expf(x[i] - mx);
+      s += y[i];
+    }
+    for (int i = 0; i < len; ++i) y[i] /= s;
+  }
+  return 0;
+}
+
+/* cuDNN SOFTMAX_ACCURATE with MODE_CHANNEL (cuda_perform.cu:355-369): softmax
+ * over C for every (n,h,w).  Tensor {W,H,C,N}.  parity unpinned by any reference
+ * test; pinned by fp64 closed form and by equality with ora_softmax_dim0 when
+ * H = W = 1. */
+int ora_softmax_channel_fwd(const float* in, float* out, int n, int c, int h, int w) {
+  size_t hw = (size_t)h * w;
+  for (int img = 0; img < n; ++img)
+    for (size_t p = 0; p < hw; ++p) {
+      const float* x = in + (size_t)img * c * hw + p;
+      float* y = out + (size_t)img * c * hw + p;
+      float mx = x[0];
+      for (int k = 1; k < c; ++k)
+        if (mx < x[k * hw]) mx = x[k * hw];
+      float s = 0;
+      for (int k = 0; k < c; ++k) {
+        y[k * hw] = expf(x[k * hw] - mx);
+        s += y[k * hw];
+      }
+      for (int k = 0; k < c; ++k) y[k * hw] /= s;
+    }
+  return 0;
+}
+
+/* cuDNN softmax backward (cuda_perform.cu:371-397): dx_i = y_i*(dy_i - sum_j dy_j*y_j)
+ * over the same group as the forward.  `len` elements per group, groups strided:
+ * group g, element i at offset g_off(g) + i*stride.  Instance mode: len = C*H*W,
+ * stride 1.  parity unpinned by any reference test; pinned by finite differences
+ * of the forward in the tests. */
+int ora_softmax_instance_bwd(const float* dy, const float* y, float* dx, int len, size_t groups) {
+  for (size_t g = 0; g < groups; ++g) {
+    const float* d = dy + g * (size_t)len;
+    const float* t = y + g * (size_t)len;
+    float* o = dx + g * (size_t)len;
+    float dot = 0;
+    for (int i = 0; i < len; ++i) dot += d[i] * t[i];
+    for (int i = 0; i < len; ++i) o[i] = t[i] * (d[i] - dot);
+  }
+  return 0;
+}
+
+int ora_softmax_channel_bwd(const float* dy, const float* y, float* dx, int n, int c, int h,
+                            int w) {
+  size_t hw = (size_t)h * w;
+  for (int img = 0; img < n; ++img)
+    for (size_t p = 0; p < hw; ++p) {
+      size_t base = (size_t)img * c * hw + p;
+      float dot = 0;
+      for (int k = 0; k < c; ++k) dot += dy[base + k * hw] * y[base + k * hw];
+      for (int k = 0; k < c; ++k) dx[base + k * hw] = y[base + k * hw] * (dy[base + k * hw] - dot);
+    }
+  return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Activations.  Forward: basic.cpp:406-448.  alg: 0 sigmoid, 1 relu, 2 tanh   */
+/* (convolution_info.h:51-55).  Sigmoid keeps the reference's double           */
+/* intermediate: (float)(1.0 / (1.0 + (double)expf(-x))).                       */
+/* pinned by: closed forms of tests/unittest_activation.cpp:8-94                */
+/* ------------------------------------------------------------------------- */
+int ora_activation_fwd(int alg, const float* x, float* y, size_t n) {
+  switch (alg) {
+    case 0: for (size_t i = 0; i < n; ++i) y[i] = (float)(1.0 / (1.0 + expf(-x[i]))); break;
+    case 1: for (size_t i = 0; i < n; ++i) y[i] = x[i] > 0 ? x[i] : 0; break;
+    case 2: for (size_t i = 0; i < n; ++i) y[i] = tanhf(x[i]); break;
+    default: return 1;
+  }
+  return 0;
+}
+
+/* Backward (no reference CPU implementation, bundle.h:29,32,34,42): cuDNN v2
+ * activation backward as called at cuda_perform.cu:444-487 with
+ * (top y, top_diff dy, bottom x): sigmoid dx = dy*y*(1-y); relu dx = dy*[x>0];
+ * tanh dx = dy*(1-y*y).  parity unpinned by any reference value test
+ * (tests/unittest_elewise.cpp:83-96 only cross-checks two GPU entry points);
+ * pinned by finite differences of the forward in the tests. */
+int ora_activation_bwd(int alg, const float* dy, const float* y, const float* x, float* dx,
+                       size_t n) {
+  switch (alg) {
+    case 0: for (size_t i = 0; i < n; ++i) dx[i] = dy[i] * y[i] * (1.0f - y[i]); break;
+    case 1: for (size_t i = 0; i < n; ++i) dx[i] = x[i] > 0 ? dy[i] : 0; break;
+    case 2: for (size_t i = 0; i < n; ++i) dx[i] = dy[i] * (1.0f - y[i] * y[i]); break;
+    default: return 1;
+  }
+  return 0;
+}
+
+int ora_fill(float* dst, size_t n, float v) { /* basic.cpp:292-299 */
+  for (size_t i = 0; i < n; ++i) dst[i] = v;
+  return 0;
+}
+
+int ora_copy(const float* in, float* out, size_t n) { /* basic.cpp:400-404 */
+  memcpy(out, in, n * sizeof(float));
+  return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Convolution (cuDNN v2, CUDNN_CONVOLUTION = flipped kernel; call sites        */
+/* cuda_perform.cu:227-337; argument order cuda.cpp:394-453).                   */
+/* bottom {W,H,C,N}, filter {S,R,C,K}, top {Wo,Ho,K,N};                          */
+/* Ho = (H + 2*ph - R)/sv + 1 (narray/convolution.cpp:13-18).                   */
+/* top[n,k,i,j] = bias[k] + sum_{c,r,s} bottom[n,c,i*sv-ph+r,j*sh-pw+s]          */
+/*                                   * filter[k,c,R-1-r,S-1-s]                  */
+/* Forward pinned by the golden vectors of tests/unittest_conv_forward.cpp:7-68. */
+/* ------------------------------------------------------------------------- */
+int ora_conv_fwd(const float* bottom, const float* filter, const float* bias, float* top, int N,
+                 int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S) {
+  int Ho = (H + 2 * ph - R) / sv + 1, Wo = (W + 2 * pw - S) / sh + 1;
+  if (Ho <= 0 || Wo <= 0) return 1;
+  for (int n = 0; n < N; ++n)
+    for (int k = 0; k < K; ++k)
+      for (int i = 0; i < Ho; ++i)
+        for (int j = 0; j < Wo; ++j) {
+          float acc = 0;
+          for (int c = 0; c < C; ++c)
+            for (int r = 0; r < R; ++r) {
+              int y = i * sv - ph + r;
+              if (y < 0 || y >= H) continue;
+              for (int s = 0; s < S; ++s) {
+                int x = j * sh - pw + s;
+                if (x < 0 || x >= W) continue;
+                float p = bottom[(((size_t)n * C + c) * H + y) * W + x] *
+                          filter[(((size_t)k * C + c) * R + (R - 1 - r)) * S + (S - 1 - s)];
+                acc = acc + p;
+              }
+            }
+          top[(((size_t)n * K + k) * Ho + i) * Wo + j] = acc + (bias ? bias[k] : 0.0f);
+        }
+  return 0;
+}
+
+/* Backward data: adjoint of the forward with respect to bottom; bottom_diff has
+ * the forward bottom's shape H x W (narray/convolution.cpp:47) and is written
+ * in full (positions no window touches become 0).  parity unpinned by any
+ * reference test; pinned by the adjoint identity <conv(x,w),dy> = <x,dX> and by
+ * finite differences in the tests. */
+int ora_conv_bwd_data(const float* top_diff, const float* filter, float* bottom_diff, int N,
+                      int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S) {
+  int Ho = (H + 2 * ph - R) / sv + 1, Wo = (W + 2 * pw - S) / sh + 1;
+  if (Ho <= 0 || Wo <= 0) return 1;
+  for (int n = 0; n < N; ++n)
+    for (int c = 0; c < C; ++c)
+      for (int y = 0; y < H; ++y)
+        for (int x = 0; x < W; ++x) {
+          float acc = 0;
+          for (int k = 0; k < K; ++k)
+            for (int r = 0; r < R; ++r) {
+              int t = y + ph - r;
+              if (t < 0 || t % sv) continue;
+              int i = t / sv;
+              if (i >= Ho) continue;
+              for (int s = 0; s < S; ++s) {
+                int u = x + pw - s;
+                if (u < 0 || u % sh) continue;
+                int j = u / sh;
+                if (j >= Wo) continue;
+                float p = top_diff[(((size_t)n * K + k) * Ho + i) * Wo + j] *
+                          filter[(((size_t)k * C + c) * R + (R - 1 - r)) * S + (S - 1 - s)];
+                acc = acc + p;
+              }
+            }
+          bottom_diff[(((size_t)n * C + c) * H + y) * W + x] = acc;
+        }
+  return 0;
+}
+
+/* Backward filter: adjoint with respect to the filter, beta = 0.  parity
+ * unpinned by any reference test; pinned by <conv(x,w),dy> = <w,dW>. */
+int ora_conv_bwd_filter(const float* top_diff, const float* bottom, float* filter_diff, int N,
+                        int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R,
+                        int S) {
+  int Ho = (H + 2 * ph - R) / sv + 1, Wo = (W + 2 * pw - S) / sh + 1;
+  if (Ho <= 0 || Wo <= 0) return 1;
+  for (int k = 0; k < K; ++k)
+    for (int c = 0; c < C; ++c)
+      for (int r = 0; r < R; ++r)
+        for (int s = 0; s < S; ++s) {
+          float acc = 0;
+          for (int n = 0; n < N; ++n)
+            for (int i = 0; i < Ho; ++i) {
+              int y = i * sv - ph + r;
+              if (y < 0 || y >= H) continue;
+              for (int j = 0; j < Wo; ++j) {
+                int x = j * sh - pw + s;
+                if (x < 0 || x >= W) continue;
+                float p = top_diff[(((size_t)n * K + k) * Ho + i) * Wo + j] *
+                          bottom[(((size_t)n * C + c) * H + y) * W + x];
+                acc = acc + p;
+              }
+            }
+          filter_diff[(((size_t)k * C + c) * R + (R - 1 - r)) * S + (S - 1 - s)] = acc;
+        }
+  return 0;
+}
+
+/* Backward bias: db[k] = sum_{n,i,j} dY[n,k,i,j] (cuda_perform.cu:320-337).
+ * parity unpinned by any reference test; pinned by the closed form (a sum). */
+int ora_conv_bwd_bias(const float* top_diff, float* bias_diff, int N, int K, int Ho, int Wo) {
+  size_t hw = (size_t)Ho * Wo;
+  for (int k = 0; k < K; ++k) {
+    float acc = 0;
+    for (int n = 0; n < N; ++n) {
+      const float* p = top_diff + ((size_t)n * K + k) * hw;
+      for (size_t q = 0; q < hw; ++q) acc += p[q];
+    }
+    bias_diff[k] = acc;
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Pooling (cuDNN v2 MAX / AVERAGE_COUNT_INCLUDE_PADDING, cuda_perform.cu:489-   */
+/* 615).  Pooled size: narray/convolution.cpp:107-114.  Window o covers rows     */
+/* [o*s - p, o*s - p + k) clipped to [0,H).  alg 0 max, 1 average.               */
+/* Max forward (values and output size) pinned by the four golden vectors of     */
+/* tests/unittest_pooling_forward.cpp:7-81.                                      */
+/* ------------------------------------------------------------------------- */
+int ora_pooled_size(int in, int win, int stride, int pad) {
+  int p = (in + 2 * pad - win + stride - 1) / stride + 1;
+  if (0 <= (p - 1) * stride - in - pad) --p;
+  return p;
+}
+
+int ora_pool_fwd(int alg, const float* bottom, float* top, int N, int C, int H, int W, int sv,
+                 int sh, int kh, int kw, int ph, int pw) {
+  int Ho = ora_pooled_size(H, kh, sv, ph), Wo = ora_pooled_size(W, kw, sh, pw);
+  if (Ho <= 0 || Wo <= 0 || (alg != 0 && alg != 1)) return 1;
+  for (size_t nc = 0; nc < (size_t)N * C; ++nc) {
+    const float* b = bottom + nc * H * W;
+    float* t = top + nc * Ho * Wo;
+    for (int i = 0; i < Ho; ++i)
+      for (int j = 0; j < Wo; ++j) {
+        int y0 = i * sv - ph, x0 = j * sh - pw;
+        int ys = y0 < 0 ? 0 : y0, xs = x0 < 0 ? 0 : x0;
+        int ye = y0 + kh > H ? H : y0 + kh, xe = x0 + kw > W ? W : x0 + kw;
+        if (alg == 0) {
+          float m = -INFINITY;
+          for (int y = ys; y < ye; ++y)
+            for (int x = xs; x < xe; ++x)
+              if (m < b[y * W + x]) m = b[y * W + x];
+          t[i * Wo + j] = m;
+        } else {
+          /* parity unpinned by any reference test (average mode): divisor is
+           * the full window kh*kw, padding counted as zeros. */
+          float s = 0;
+          for (int y = ys; y < ye; ++y)
+            for (int x = xs; x < xe; ++x) s += b[y * W + x];
+          t[i * Wo + j] = s / (float)(kh * kw);
+        }
+      }
+  }
+  return 0;
+}
+
+/* Backward.  Max: dY[o] goes to the first maximum of window o in (row, col)
+ * scan order; overlapping windows accumulate in window scan order.  Average:
+ * each position of window o receives dY[o] / (kh*kw).  parity unpinned by any
+ * reference test (the reference defers to cuDNN); pinned by brute force, by
+ * sum(dX) = sum(dY) for max pooling and by finite differences of the forward.
+ * `mask_idx` (optional, max only): for every output o the flat y*W+x index of
+ * the position that received its gradient, as float. */
+int ora_pool_bwd(int alg, const float* top_diff, const float* top, const float* bottom,
+                 float* bottom_diff, float* mask_idx, int N, int C, int H, int W, int sv, int sh,
+                 int kh, int kw, int ph, int pw) {
+  (void)top;
+  int Ho = ora_pooled_size(H, kh, sv, ph), Wo = ora_pooled_size(W, kw, sh, pw);
+  if (Ho <= 0 || Wo <= 0 || (alg != 0 && alg != 1)) return 1;
+  for (size_t nc = 0; nc < (size_t)N * C; ++nc) {
+    const float* b = bottom + nc * H * W;
+    const float* dt = top_diff + nc * Ho * Wo;
+    float* db = bottom_diff + nc * H * W;
+    for (int q = 0; q < H * W; ++q) db[q] = 0;
+    for (int i = 0; i < Ho; ++i)
+      for (int j = 0; j < Wo; ++j) {
+        int y0 = i * sv - ph, x0 = j * sh - pw;
+        int ys = y0 < 0 ? 0 : y0, xs = x0 < 0 ? 0 : x0;
+        int ye = y0 + kh > H ? H : y0 + kh, xe = x0 + kw > W ? W : x0 + kw;
+        if (alg == 0) {
+          float m = -INFINITY;
+          int arg = ys * W + xs;
+          for (int y = ys; y < ye; ++y)
+            for (int x = xs; x < xe; ++x)
+              if (m < b[y * W + x]) {
+                m = b[y * W + x];
+                arg = y * W + x;
+              }
+          db[arg] += dt[i * Wo + j];
+          if (mask_idx) mask_idx[nc * Ho * Wo + i * Wo + j] = (float)arg;
+        } else {
+          float g = dt[i * Wo + j] / (float)(kh * kw);
+          for (int y = ys; y < ye; ++y)
+            for (int x = xs; x < xe; ++x) db[y * W + x] += g;
+        }
+      }
+  }
+  return 0;
+}
