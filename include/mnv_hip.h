@@ -1,0 +1,233 @@
+/*
+ * mnv_hip.h - C ABI of the MI355X (gfx950) operator library that replaces the
+ * cuBLAS / cuDNN / .cu launchers behind Minerva's GPU operator layer.
+ *
+ * Every entry point mirrors one launcher of the reference's
+ * minerva/op/impl/cuda/cuda_perform.h (cited per function) with the CUDA handle
+ * types replaced by an opaque stream pointer.  Conventions:
+ *   - all tensors are fp32, column-major, dimension 0 fastest (reference
+ *     minerva/common/scale.cpp:182-191): matrices are {rows, cols} with the row
+ *     index fastest, image batches are {W,H,C,N} (= NCHW bytes), filters are
+ *     {S,R,Cin,Cout} (= KCRS bytes);
+ *   - all pointers are device pointers unless the name says host;
+ *   - inputs and outputs never alias; the callee never allocates or frees
+ *     tensors and keeps no state between calls; launches are asynchronous on
+ *     `stream` (a hipStream_t cast to void*, NULL = the default stream) and the
+ *     caller synchronises, as the reference device does after every operator
+ *     (minerva/device/device.cpp:214-222);
+ *   - return value: 0 on success, a hipError_t value (> 0) when the runtime
+ *     reports an error, MNV_ERR_INVALID (-1) for arguments the kernels cannot
+ *     take (null pointer, non-positive extent, extent beyond 2^31-1 where the
+ *     reference's int arguments are mirrored), MNV_ERR_WORKSPACE (-2) when a
+ *     caller-provided workspace is too small;
+ *   - kernels that need device scratch take it as (workspace, workspace_bytes);
+ *     the matching *_workspace_bytes function tells how much.  A NULL workspace
+ *     is always accepted and selects a path that needs none.
+ */
+#ifndef MNV_HIP_H_
+#define MNV_HIP_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MNV_OK 0
+#define MNV_ERR_INVALID (-1)
+#define MNV_ERR_WORKSPACE (-2)
+
+typedef void* mnv_stream_t;
+
+/* ---- device, streams, memory: replaces the CUDA runtime calls of
+ *      minerva/device/device.cpp:146-222 and system/minerva_system.cpp:21-33 ---- */
+int mnv_device_count(int* count);
+int mnv_device_set(int device);
+/* name_out: at least 256 bytes.  cu_count / clock_khz / hbm_bytes may be NULL. */
+int mnv_device_info(int device, char* name_out, int* cu_count, int* clock_khz, size_t* hbm_bytes);
+int mnv_stream_create(mnv_stream_t* stream);
+int mnv_stream_destroy(mnv_stream_t stream);
+int mnv_stream_sync(mnv_stream_t stream);
+int mnv_device_sync(void);
+int mnv_malloc(void** ptr, size_t bytes);
+int mnv_free(void* ptr);
+int mnv_host_malloc(void** ptr, size_t bytes); /* pinned host memory */
+int mnv_host_free(void* ptr);
+int mnv_memcpy_h2d(void* dst, const void* src_host, size_t bytes, mnv_stream_t stream);
+int mnv_memcpy_d2h(void* dst_host, const void* src, size_t bytes, mnv_stream_t stream);
+int mnv_memcpy_d2d(void* dst, const void* src, size_t bytes, mnv_stream_t stream);
+/* Events for timing on the stream the kernels run on. */
+int mnv_event_create(void** event);
+int mnv_event_destroy(void* event);
+int mnv_event_record(void* event, mnv_stream_t stream);
+int mnv_event_sync(void* event);
+int mnv_event_elapsed_ms(void* start, void* stop, float* ms);
+const char* mnv_error_string(int status);
+
+/* ---- elementwise binary: c[i] = a[i] (op) b[i]
+ * CudaPerformAdd / CudaPerformSub / CudaPerformDotMult / CudaPerformDotDiv
+ * (cuda_perform.h:12-16).  One IEEE operation per element. ---- */
+int mnv_add(const float* a, const float* b, float* c, size_t n, mnv_stream_t stream);
+int mnv_sub(const float* a, const float* b, float* c, size_t n, mnv_stream_t stream);
+int mnv_mul(const float* a, const float* b, float* c, size_t n, mnv_stream_t stream);
+int mnv_div(const float* a, const float* b, float* c, size_t n, mnv_stream_t stream);
+
+/* ---- scalar arithmetic: CudaPerformConstAdd, CudaPerformLeftConstSub,
+ * CudaPerformScale, CudaPerformLeftConstDiv (cuda_perform.h:18,21-23).
+ *   const_add y = x + v   const_sub y = x - v   const_rsub y = v - x
+ *   const_mul y = x * v   const_div y = x / v (a true division, as the CPU
+ *   implementation basic.cpp:99-103 does)   const_rdiv y = v / x ---- */
+int mnv_const_add(const float* x, float* y, float v, size_t n, mnv_stream_t stream);
+int mnv_const_sub(const float* x, float* y, float v, size_t n, mnv_stream_t stream);
+int mnv_const_rsub(const float* x, float* y, float v, size_t n, mnv_stream_t stream);
+int mnv_const_mul(const float* x, float* y, float v, size_t n, mnv_stream_t stream);
+int mnv_const_div(const float* x, float* y, float v, size_t n, mnv_stream_t stream);
+int mnv_const_rdiv(const float* x, float* y, float v, size_t n, mnv_stream_t stream);
+
+/* ---- elementwise unary: CudaPerformElewiseExp / Ln / Negative
+ * (cuda_perform.h:43-45) ---- */
+int mnv_exp(const float* x, float* y, size_t n, mnv_stream_t stream);
+int mnv_ln(const float* x, float* y, size_t n, mnv_stream_t stream);
+int mnv_neg(const float* x, float* y, size_t n, mnv_stream_t stream);
+
+/* ---- broadcast arithmetic on an {m,n} matrix: CudaPerformNorm{Add,Sub,Mult,Div}
+ * On{Col,Row} (cuda_perform.h:25-33).
+ *   *_col: vec has n entries (shape {1,n}); res[r + c*m] = matrix[r + c*m] (op) vec[c]
+ *   *_row: vec has m entries (shape {m,1}); res[r + c*m] = matrix[r + c*m] (op) vec[r] ---- */
+int mnv_norm_add_col(const float* matrix, const float* vec, float* res, int m, int n, mnv_stream_t stream);
+int mnv_norm_sub_col(const float* matrix, const float* vec, float* res, int m, int n, mnv_stream_t stream);
+int mnv_norm_mul_col(const float* matrix, const float* vec, float* res, int m, int n, mnv_stream_t stream);
+int mnv_norm_div_col(const float* matrix, const float* vec, float* res, int m, int n, mnv_stream_t stream);
+int mnv_norm_add_row(const float* matrix, const float* vec, float* res, int m, int n, mnv_stream_t stream);
+int mnv_norm_sub_row(const float* matrix, const float* vec, float* res, int m, int n, mnv_stream_t stream);
+int mnv_norm_mul_row(const float* matrix, const float* vec, float* res, int m, int n, mnv_stream_t stream);
+int mnv_norm_div_row(const float* matrix, const float* vec, float* res, int m, int n, mnv_stream_t stream);
+
+/* ---- reductions of an {m,n} matrix: CudaPerformReduction{Sum,Max}On{Col,Row}
+ * (cuda_perform.h:35-38).
+ *   *_col: reduce dimension 0; out has n entries, out[c] = reduce_r in[r + c*m]
+ *   *_row: reduce dimension 1; out has m entries, out[r] = reduce_c in[r + c*m] ---- */
+int mnv_reduce_sum_col(const float* in, float* out, int m, int n, mnv_stream_t stream);
+int mnv_reduce_max_col(const float* in, float* out, int m, int n, mnv_stream_t stream);
+int mnv_reduce_sum_row(const float* in, float* out, int m, int n, mnv_stream_t stream);
+int mnv_reduce_max_row(const float* in, float* out, int m, int n, mnv_stream_t stream);
+
+/* ---- arg-max: CudaPerformMaxIndexOn{Col,Row} (cuda_perform.h:40-41).  The index
+ * of the first maximum (lowest index wins ties, NaN never replaces the running
+ * maximum), stored as float.  *_col: along dimension 0 (out has n entries);
+ * *_row: along dimension 1 (out has m entries). ---- */
+int mnv_maxindex_col(const float* in, float* out, int m, int n, mnv_stream_t stream);
+int mnv_maxindex_row(const float* in, float* out, int m, int n, mnv_stream_t stream);
+
+/* ---- SGEMM: CudaPerformMatMult (cuda_perform.h:17; cublasSgemm N,N, alpha 1,
+ * beta 0, cuda_perform.cu:66-70).  C{m,n} = A{m,k} * B{k,n}, all column-major with
+ * leading dimensions m, k, m.  The workspace (optional) lets skinny products split
+ * the k range over more workgroups. ---- */
+size_t mnv_sgemm_nn_workspace_bytes(int m, int n, int k);
+int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k,
+                 void* workspace, size_t workspace_bytes, mnv_stream_t stream);
+
+/* ---- transpose: CudaPerformTranspose (cuda_perform.h:19; cublasSgeam T,N).
+ * a is {m,n}; c is {n,m}; c[j + i*n] = a[i + j*m]. ---- */
+int mnv_transpose(const float* a, float* c, int m, int n, mnv_stream_t stream);
+
+/* ---- copy / fill: CudaPerformReshape (cuda_perform.h:43, n counts floats here),
+ * CudaPerformFill (cuda_perform.h:69) ---- */
+int mnv_copy(const float* in, float* out, size_t n, mnv_stream_t stream);
+int mnv_fill(float* dst, size_t n, float v, mnv_stream_t stream);
+
+/* ---- activations: CudaPerform{Sigmoid,Relu,Tanh}{Forward,Backward}
+ * (cuda_perform.h:55-60).  The reference describes the tensor as n*c*h*w
+ * elements; the op is elementwise so only the count is passed.
+ *   forward : top = f(bottom); relu is x > 0 ? x : 0
+ *   backward: sigmoid bd = td*top*(1-top); relu bd = bottom > 0 ? td : 0;
+ *             tanh bd = td*(1-top*top) ---- */
+int mnv_sigmoid_fwd(const float* bottom, float* top, size_t n, mnv_stream_t stream);
+int mnv_relu_fwd(const float* bottom, float* top, size_t n, mnv_stream_t stream);
+int mnv_tanh_fwd(const float* bottom, float* top, size_t n, mnv_stream_t stream);
+int mnv_sigmoid_bwd(const float* bottom, const float* top, const float* top_diff,
+                    float* bottom_diff, size_t n, mnv_stream_t stream);
+int mnv_relu_bwd(const float* bottom, const float* top, const float* top_diff,
+                 float* bottom_diff, size_t n, mnv_stream_t stream);
+int mnv_tanh_bwd(const float* bottom, const float* top, const float* top_diff,
+                 float* bottom_diff, size_t n, mnv_stream_t stream);
+
+/* ---- softmax: CudaPerform{Instance,Channel}Softmax{Forward,Backward}
+ * (cuda_perform.h:51-54).  Tensor {W,H,C,N}.  instance: over the C*H*W values of
+ * each image; channel: over C for each (n,h,w).  backward:
+ * bottom_diff_i = top_i * (top_diff_i - sum_j top_diff_j * top_j). ---- */
+int mnv_softmax_instance_fwd(const float* bottom, float* top, int num_images, int num_channels,
+                             int height, int width, mnv_stream_t stream);
+int mnv_softmax_channel_fwd(const float* bottom, float* top, int num_images, int num_channels,
+                            int height, int width, mnv_stream_t stream);
+int mnv_softmax_instance_bwd(const float* top_diff, const float* top, float* bottom_diff,
+                             int num_images, int num_channels, int height, int width,
+                             mnv_stream_t stream);
+int mnv_softmax_channel_bwd(const float* top_diff, const float* top, float* bottom_diff,
+                            int num_images, int num_channels, int height, int width,
+                            mnv_stream_t stream);
+
+/* ---- convolution: CudaPerformConv{Forward,BackwardData,BackwardFilter,BackwardBias}
+ * (cuda_perform.h:47-50).  True convolution (flipped filter), zero padding:
+ *   top[n,k,i,j] = bias[k] + sum_{c,r,s} bottom[n,c,i*sv-ph+r,j*sh-pw+s]
+ *                                        * filter[k,c,R-1-r,S-1-s]
+ *   top_height = (bottom_height + 2*pad_height - filter_height)/stride_vertical + 1.
+ * backward_data takes the bottom extent (not the top extent the reference
+ * launcher re-derives it from, cuda_perform.cu:277) so that inexact fits work,
+ * and writes every element of bottom_diff.  backward_filter overwrites
+ * filter_diff (beta = 0). ---- */
+int mnv_conv_fwd(const float* bottom, const float* filter, const float* bias, float* top,
+                 int num_images, int bottom_num_channels, int top_num_channels,
+                 int bottom_height, int bottom_width, int pad_height, int pad_width,
+                 int stride_vertical, int stride_horizontal, int filter_height,
+                 int filter_width, mnv_stream_t stream);
+int mnv_conv_bwd_data(const float* top_diff, const float* filter, float* bottom_diff,
+                      int num_images, int bottom_num_channels, int top_num_channels,
+                      int bottom_height, int bottom_width, int pad_height, int pad_width,
+                      int stride_vertical, int stride_horizontal, int filter_height,
+                      int filter_width, mnv_stream_t stream);
+size_t mnv_conv_bwd_filter_workspace_bytes(int num_images, int bottom_num_channels,
+                                           int top_num_channels, int bottom_height,
+                                           int bottom_width, int pad_height, int pad_width,
+                                           int stride_vertical, int stride_horizontal,
+                                           int filter_height, int filter_width);
+int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filter_diff,
+                        int num_images, int bottom_num_channels, int top_num_channels,
+                        int bottom_height, int bottom_width, int pad_height, int pad_width,
+                        int stride_vertical, int stride_horizontal, int filter_height,
+                        int filter_width, void* workspace, size_t workspace_bytes,
+                        mnv_stream_t stream);
+int mnv_conv_bwd_bias(const float* top_diff, float* bias_diff, int num_images,
+                      int top_num_channels, int top_height, int top_width, mnv_stream_t stream);
+
+/* ---- pooling: CudaPerform{Max,Average}Pooling{Forward,Backward}
+ * (cuda_perform.h:61-64).  pooled = (in + 2*pad - window + stride - 1)/stride + 1,
+ * minus one if (pooled-1)*stride >= in + pad (cuda_perform.cu:491-498);
+ * mnv_pooled_size computes it.  Window o covers [o*stride - pad, o*stride - pad +
+ * window) clipped to the tensor.  max: padding never wins; average: divisor is
+ * window_height*window_width (padding counted).  max backward sends each
+ * top_diff to the first maximum of its window in (row, column) scan order. ---- */
+int mnv_pooled_size(int in, int window, int stride, int pad);
+int mnv_maxpool_fwd(const float* bottom, float* top, int num_images, int num_channels,
+                    int bottom_height, int bottom_width, int stride_vertical,
+                    int stride_horizontal, int window_height, int window_width, int pad_height,
+                    int pad_width, mnv_stream_t stream);
+int mnv_avgpool_fwd(const float* bottom, float* top, int num_images, int num_channels,
+                    int bottom_height, int bottom_width, int stride_vertical,
+                    int stride_horizontal, int window_height, int window_width, int pad_height,
+                    int pad_width, mnv_stream_t stream);
+int mnv_maxpool_bwd(const float* bottom, const float* top, const float* top_diff,
+                    float* bottom_diff, int num_images, int num_channels, int bottom_height,
+                    int bottom_width, int stride_vertical, int stride_horizontal,
+                    int window_height, int window_width, int pad_height, int pad_width,
+                    mnv_stream_t stream);
+int mnv_avgpool_bwd(const float* bottom, const float* top, const float* top_diff,
+                    float* bottom_diff, int num_images, int num_channels, int bottom_height,
+                    int bottom_width, int stride_vertical, int stride_horizontal,
+                    int window_height, int window_width, int pad_height, int pad_width,
+                    mnv_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MNV_HIP_H_ */

@@ -1,0 +1,45 @@
+// Shared helpers of the gfx950 operator library (host + device side).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "mnv_hip.h"
+
+#define MNV_WAVE 64
+
+// Propagate a HIP runtime error as the C-ABI status.
+#define MNV_HIP_TRY(expr)                      \
+  do {                                         \
+    hipError_t mnv_e_ = (expr);                \
+    if (mnv_e_ != hipSuccess) return (int)mnv_e_; \
+  } while (0)
+
+// Status of the launch that was just issued (does not synchronise).
+#define MNV_LAUNCH_STATUS() ((int)hipGetLastError())
+
+static inline hipStream_t mnv_stream(mnv_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+static inline bool mnv_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+static inline size_t mnv_ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
+
+// Upper bound on grid.x for grid-stride kernels: enough resident work for
+// 256 CUs without paying launch cost for millions of tiny blocks.
+#define MNV_MAX_STREAM_BLOCKS 16384u
+
+#ifdef __HIPCC__
+typedef float mnv_f4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float mnv_wave_sum(float v) {
+#pragma unroll
+  for (int off = MNV_WAVE / 2; off > 0; off >>= 1) v += __shfl_down(v, off, MNV_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float mnv_wave_max(float v) {
+#pragma unroll
+  for (int off = MNV_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_down(v, off, MNV_WAVE));
+  return v;
+}
+#endif

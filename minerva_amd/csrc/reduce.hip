@@ -1,0 +1,321 @@
+// Reductions of a column-major {m,n} matrix: sum / max along either dimension,
+// arg-max along either dimension, and the convolution bias gradient.
+// Roofline: HBM bandwidth, 4 algorithmic bytes per input element.
+//
+// Reference semantics (minerva/op/impl/basic.cpp:189-217, 369-398): a left fold in
+// ascending index order that starts from the first element; max / arg-max use a
+// strict '<', so the first occurrence of the maximum wins and a NaN is never
+// selected unless it is the first element.  Max and arg-max reproduce that
+// exactly under any parallel order by reducing (value, index) pairs: the larger
+// value wins, equal values keep the lower index (so the bits of a +0 / -0 tie are
+// the reference's), NaNs are skipped, and a NaN in position 0 is restored at the
+// end.  Sums are tree-ordered (fp32), which differs from the sequential fold only
+// in rounding.
+#include <math.h>
+
+#include "mnv_common.h"
+
+namespace {
+
+#define MNV_NONE 0x7fffffff
+
+struct SumAcc {
+  float s;
+  __device__ void init() { s = 0.f; }
+  __device__ void push(float v, int) { s += v; }
+  __device__ void merge(const SumAcc& o) { s += o.s; }
+  __device__ SumAcc shfl_down(int off) const {
+    SumAcc r;
+    r.s = __shfl_down(s, off, MNV_WAVE);
+    return r;
+  }
+  // first = element 0 of the reduced line (only the pair reducers need it)
+  __device__ float result_value(float) const { return s; }
+};
+
+struct ArgAcc {
+  float v;
+  int idx;
+  __device__ void init() {
+    v = -INFINITY;
+    idx = MNV_NONE;
+  }
+  // Elements reach one accumulator in ascending index order.
+  __device__ void push(float x, int i) {
+    bool take = (idx == MNV_NONE) ? (x == x) : (x > v);
+    if (take) {
+      v = x;
+      idx = i;
+    }
+  }
+  __device__ void merge(const ArgAcc& o) {
+    bool take = (o.idx != MNV_NONE) &&
+                (idx == MNV_NONE || o.v > v || (o.v == v && o.idx < idx));
+    if (take) {
+      v = o.v;
+      idx = o.idx;
+    }
+  }
+  __device__ ArgAcc shfl_down(int off) const {
+    ArgAcc r;
+    r.v = __shfl_down(v, off, MNV_WAVE);
+    r.idx = __shfl_down(idx, off, MNV_WAVE);
+    return r;
+  }
+  __device__ float result_value(float first) const { return (first != first) ? first : v; }
+  __device__ float result_index(float first) const {
+    return (first != first || idx == MNV_NONE) ? 0.f : (float)idx;
+  }
+};
+
+// What a reducer writes.
+struct EmitValue {
+  template <class Acc>
+  __device__ static float get(const Acc& a, float first) { return a.result_value(first); }
+};
+struct EmitIndex {
+  __device__ static float get(const ArgAcc& a, float first) { return a.result_index(first); }
+};
+
+// ---------------------------------------------------------------------------
+// Along dimension 0: each of the n columns is m contiguous floats.
+// GROUP threads (one wavefront, or the whole 256-thread workgroup) share a column.
+// ---------------------------------------------------------------------------
+#define MNV_RC_THREADS 256
+
+template <class Acc, class Emit, int GROUP, bool VEC4>
+__global__ __launch_bounds__(MNV_RC_THREADS) void mnv_reduce_col_kernel(
+    const float* __restrict__ in, float* __restrict__ out, int m, int n) {
+  constexpr int COLS = MNV_RC_THREADS / GROUP;
+  __shared__ Acc part[MNV_RC_THREADS / MNV_WAVE];
+  const int g = threadIdx.x / GROUP;
+  const int t = threadIdx.x % GROUP;
+  for (int c = blockIdx.x * COLS + g; c < n; c += gridDim.x * COLS) {
+    const float* col = in + (size_t)c * m;
+    Acc acc;
+    acc.init();
+    if (VEC4) {
+      const mnv_f4* col4 = reinterpret_cast<const mnv_f4*>(col);
+      const int m4 = m >> 2;
+      int i = t;
+      // two independent 16-byte loads in flight per thread
+      for (; i + GROUP < m4; i += 2 * GROUP) {
+        mnv_f4 a = col4[i], b = col4[i + GROUP];
+        acc.push(a.x, 4 * i); acc.push(a.y, 4 * i + 1); acc.push(a.z, 4 * i + 2); acc.push(a.w, 4 * i + 3);
+        int j = i + GROUP;
+        acc.push(b.x, 4 * j); acc.push(b.y, 4 * j + 1); acc.push(b.z, 4 * j + 2); acc.push(b.w, 4 * j + 3);
+      }
+      if (i < m4) {
+        mnv_f4 a = col4[i];
+        acc.push(a.x, 4 * i); acc.push(a.y, 4 * i + 1); acc.push(a.z, 4 * i + 2); acc.push(a.w, 4 * i + 3);
+      }
+    } else {
+      for (int i = t; i < m; i += GROUP) acc.push(col[i], i);
+    }
+#pragma unroll
+    for (int off = MNV_WAVE / 2; off > 0; off >>= 1) acc.merge(acc.shfl_down(off));
+    if (GROUP > MNV_WAVE) {
+      const int w = threadIdx.x / MNV_WAVE;
+      if ((threadIdx.x % MNV_WAVE) == 0) part[w] = acc;
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        for (int q = 1; q < MNV_RC_THREADS / MNV_WAVE; ++q) acc.merge(part[q]);
+        out[c] = Emit::get(acc, col[0]);
+      }
+      __syncthreads();
+    } else if (t == 0) {
+      out[c] = Emit::get(acc, col[0]);
+    }
+  }
+}
+
+template <class Acc, class Emit>
+int launch_reduce_col(const float* in, float* out, int m, int n, mnv_stream_t stream) {
+  if (n == 0) return MNV_OK;
+  if (!in || !out || m <= 0 || n < 0) return MNV_ERR_INVALID;
+  hipStream_t s = mnv_stream(stream);
+  bool vec4 = (m % 4 == 0) && mnv_aligned16(in);
+  if (m > 2048) {
+    unsigned grid = (unsigned)(n < 65536 ? n : 65536);
+    if (vec4)
+      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_RC_THREADS, true>), dim3(grid),
+                         dim3(MNV_RC_THREADS), 0, s, in, out, m, n);
+    else
+      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_RC_THREADS, false>), dim3(grid),
+                         dim3(MNV_RC_THREADS), 0, s, in, out, m, n);
+  } else {
+    size_t blocks = mnv_ceil_div((size_t)n, MNV_RC_THREADS / MNV_WAVE);
+    unsigned grid = (unsigned)(blocks < 65536 ? blocks : 65536);
+    if (vec4)
+      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_WAVE, true>), dim3(grid),
+                         dim3(MNV_RC_THREADS), 0, s, in, out, m, n);
+    else
+      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_WAVE, false>), dim3(grid),
+                         dim3(MNV_RC_THREADS), 0, s, in, out, m, n);
+  }
+  return MNV_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------
+// Along dimension 1: out[r] = reduce_c in[r + c*m] (stride m between elements).
+// A workgroup owns RL*W consecutive rows (128 contiguous bytes per column) and
+// splits the columns over CG thread groups; partial results meet in LDS.
+// ---------------------------------------------------------------------------
+template <class Acc, class Emit, int RL, int CG, bool VEC4>
+__global__ __launch_bounds__(RL* CG) void mnv_reduce_row_kernel(const float* __restrict__ in,
+                                                                float* __restrict__ out, int m,
+                                                                int n) {
+  constexpr int W = VEC4 ? 4 : 1;
+  constexpr int ROWS = RL * W;
+  __shared__ Acc part[CG][ROWS + 1];
+  const int rl = threadIdx.x % RL;
+  const int cg = threadIdx.x / RL;
+  const int r0 = blockIdx.x * ROWS + rl * W;
+  Acc acc[W];
+#pragma unroll
+  for (int q = 0; q < W; ++q) acc[q].init();
+  if (r0 < m) {
+    if (VEC4) {
+      int c = cg;
+      for (; c + CG < n; c += 2 * CG) {
+        mnv_f4 a = *reinterpret_cast<const mnv_f4*>(in + (size_t)c * m + r0);
+        mnv_f4 b = *reinterpret_cast<const mnv_f4*>(in + (size_t)(c + CG) * m + r0);
+        acc[0].push(a.x, c); acc[1 % W].push(a.y, c); acc[2 % W].push(a.z, c); acc[3 % W].push(a.w, c);
+        acc[0].push(b.x, c + CG); acc[1 % W].push(b.y, c + CG); acc[2 % W].push(b.z, c + CG); acc[3 % W].push(b.w, c + CG);
+      }
+      if (c < n) {
+        mnv_f4 a = *reinterpret_cast<const mnv_f4*>(in + (size_t)c * m + r0);
+        acc[0].push(a.x, c); acc[1 % W].push(a.y, c); acc[2 % W].push(a.z, c); acc[3 % W].push(a.w, c);
+      }
+    } else {
+      for (int c = cg; c < n; c += CG) acc[0].push(in[(size_t)c * m + r0], c);
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < W; ++q) part[cg][rl * W + q] = acc[q];
+  __syncthreads();
+  for (int sft = CG / 2; sft > 0; sft >>= 1) {
+    if (cg < sft) {
+#pragma unroll
+      for (int q = 0; q < W; ++q) {
+        Acc a = part[cg][rl * W + q];
+        a.merge(part[cg + sft][rl * W + q]);
+        part[cg][rl * W + q] = a;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x < ROWS) {
+    int r = blockIdx.x * ROWS + threadIdx.x;
+    if (r < m) out[r] = Emit::get(part[0][threadIdx.x], in[r]);
+  }
+}
+
+template <class Acc, class Emit>
+int launch_reduce_row(const float* in, float* out, int m, int n, mnv_stream_t stream) {
+  if (m == 0) return MNV_OK;
+  if (!in || !out || m < 0 || n <= 0) return MNV_ERR_INVALID;
+  hipStream_t s = mnv_stream(stream);
+  bool vec4 = (m % 4 == 0) && mnv_aligned16(in);
+  if (vec4) {
+    constexpr int RL = 8, CG = 64;
+    unsigned grid = (unsigned)mnv_ceil_div((size_t)m, RL * 4);
+    hipLaunchKernelGGL((mnv_reduce_row_kernel<Acc, Emit, RL, CG, true>), dim3(grid),
+                       dim3(RL * CG), 0, s, in, out, m, n);
+  } else {
+    constexpr int RL = 32, CG = 16;
+    unsigned grid = (unsigned)mnv_ceil_div((size_t)m, RL);
+    hipLaunchKernelGGL((mnv_reduce_row_kernel<Acc, Emit, RL, CG, false>), dim3(grid),
+                       dim3(RL * CG), 0, s, in, out, m, n);
+  }
+  return MNV_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------
+// Convolution bias gradient: db[k] = sum over images and positions of dY[n,k,:,:]
+// (reference cuda_perform.cu:320-337).  One workgroup per output channel; its 16
+// wavefronts take images round-robin and read each hw-long row contiguously.
+// ---------------------------------------------------------------------------
+#define MNV_BIAS_THREADS 1024
+
+template <bool VEC4>
+__global__ __launch_bounds__(MNV_BIAS_THREADS) void mnv_conv_bwd_bias_kernel(
+    const float* __restrict__ top_diff, float* __restrict__ bias_diff, int N, int K, int hw) {
+  __shared__ float part[MNV_BIAS_THREADS / MNV_WAVE];
+  const int k = blockIdx.x;
+  const int wave = threadIdx.x / MNV_WAVE, lane = threadIdx.x % MNV_WAVE;
+  constexpr int NW = MNV_BIAS_THREADS / MNV_WAVE;
+  float s0 = 0.f, s1 = 0.f;
+  for (int img = wave; img < N; img += NW) {
+    const float* p = top_diff + ((size_t)img * K + k) * hw;
+    if (VEC4) {
+      const mnv_f4* p4 = reinterpret_cast<const mnv_f4*>(p);
+      const int hw4 = hw >> 2;
+      int i = lane;
+      for (; i + MNV_WAVE < hw4; i += 2 * MNV_WAVE) {
+        mnv_f4 a = p4[i], b = p4[i + MNV_WAVE];
+        s0 += (a.x + a.y) + (a.z + a.w);
+        s1 += (b.x + b.y) + (b.z + b.w);
+      }
+      if (i < hw4) {
+        mnv_f4 a = p4[i];
+        s0 += (a.x + a.y) + (a.z + a.w);
+      }
+    } else {
+      for (int i = lane; i < hw; i += MNV_WAVE) s0 += p[i];
+    }
+  }
+  float s = mnv_wave_sum(s0 + s1);
+  if (lane == 0) part[wave] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = 0.f;
+    for (int q = 0; q < NW; ++q) t += part[q];
+    bias_diff[k] = t;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int mnv_reduce_sum_col(const float* in, float* out, int m, int n, mnv_stream_t s) {
+  return launch_reduce_col<SumAcc, EmitValue>(in, out, m, n, s);
+}
+int mnv_reduce_max_col(const float* in, float* out, int m, int n, mnv_stream_t s) {
+  return launch_reduce_col<ArgAcc, EmitValue>(in, out, m, n, s);
+}
+int mnv_reduce_sum_row(const float* in, float* out, int m, int n, mnv_stream_t s) {
+  return launch_reduce_row<SumAcc, EmitValue>(in, out, m, n, s);
+}
+int mnv_reduce_max_row(const float* in, float* out, int m, int n, mnv_stream_t s) {
+  return launch_reduce_row<ArgAcc, EmitValue>(in, out, m, n, s);
+}
+int mnv_maxindex_col(const float* in, float* out, int m, int n, mnv_stream_t s) {
+  return launch_reduce_col<ArgAcc, EmitIndex>(in, out, m, n, s);
+}
+int mnv_maxindex_row(const float* in, float* out, int m, int n, mnv_stream_t s) {
+  return launch_reduce_row<ArgAcc, EmitIndex>(in, out, m, n, s);
+}
+
+int mnv_conv_bwd_bias(const float* top_diff, float* bias_diff, int num_images,
+                      int top_num_channels, int top_height, int top_width, mnv_stream_t stream) {
+  if (top_num_channels == 0) return MNV_OK;
+  if (!top_diff || !bias_diff || num_images <= 0 || top_num_channels < 0 || top_height <= 0 ||
+      top_width <= 0)
+    return MNV_ERR_INVALID;
+  long long hw = (long long)top_height * top_width;
+  if (hw > 0x7fffffffLL) return MNV_ERR_INVALID;
+  bool vec4 = (hw % 4 == 0) && mnv_aligned16(top_diff);
+  if (vec4)
+    hipLaunchKernelGGL((mnv_conv_bwd_bias_kernel<true>), dim3(top_num_channels),
+                       dim3(MNV_BIAS_THREADS), 0, mnv_stream(stream), top_diff, bias_diff,
+                       num_images, top_num_channels, (int)hw);
+  else
+    hipLaunchKernelGGL((mnv_conv_bwd_bias_kernel<false>), dim3(top_num_channels),
+                       dim3(MNV_BIAS_THREADS), 0, mnv_stream(stream), top_diff, bias_diff,
+                       num_images, top_num_channels, (int)hw);
+  return MNV_LAUNCH_STATUS();
+}
+
+}  // extern "C"

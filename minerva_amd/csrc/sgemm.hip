@@ -1,0 +1,111 @@
+// SGEMM C{m,n} = A{m,k} * B{k,n}, column-major, no transposes, alpha 1 / beta 0:
+// the product Minerva's MatMult asks for (reference minerva/op/impl/basic.cpp:150-173;
+// cublasSgemm call at minerva/op/impl/cuda/cuda_perform.cu:66-70).
+// Built on the fp32 MFMA core in gemm_core.h; A is fetched x-fast (m contiguous),
+// B k-fast (k contiguous).  Products with too few output tiles to fill 256 CUs split
+// the k range over blockIdx.z when the caller lends a workspace.
+#include "gemm_core.h"
+
+namespace {
+
+template <bool VEC>
+struct SgemmNN {
+  static constexpr bool A_KFAST = false, B_KFAST = true;
+  const float* __restrict__ A;
+  const float* __restrict__ B;
+  float* __restrict__ C;
+  int M, N, K;
+  struct AState {};
+  struct BState {};
+  __device__ void a_init(AState&, int) const {}
+  __device__ void b_init(BState&, int) const {}
+  // A[m..m+3, k]
+  __device__ void a_fetch(const AState&, int m, int k, float (&v)[4]) const {
+    if (VEC) {
+      if (m < M && k < K) {
+        mnv_f4 t = *reinterpret_cast<const mnv_f4*>(A + (size_t)k * M + m);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+      } else {
+        v[0] = v[1] = v[2] = v[3] = 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = (m + q < M && k < K) ? A[(size_t)k * M + m + q] : 0.f;
+    }
+  }
+  // B[k..k+3, n]
+  __device__ void b_fetch(const BState&, int n, int k, float (&v)[4]) const {
+    if (VEC) {
+      if (n < N && k < K) {
+        mnv_f4 t = *reinterpret_cast<const mnv_f4*>(B + (size_t)n * K + k);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+      } else {
+        v[0] = v[1] = v[2] = v[3] = 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = (n < N && k + q < K) ? B[(size_t)n * K + k + q] : 0.f;
+    }
+  }
+  __device__ void c_store(int m, int n, float x) const { C[(size_t)n * M + m] = x; }
+};
+
+typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
+typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
+
+#define MNV_SGEMM_MAX_SPLITS 16
+
+// How many k ranges to use for an (m,n,k) product given `ws_floats` floats of scratch.
+int pick_splits(int tiles, int slabs, size_t mn, size_t ws_floats) {
+  if (tiles >= 256 || slabs < 8) return 1;
+  int want = (512 + tiles - 1) / tiles;
+  if (want > MNV_SGEMM_MAX_SPLITS) want = MNV_SGEMM_MAX_SPLITS;
+  if (want > slabs / 4) want = slabs / 4;
+  size_t fit = mn ? ws_floats / mn : 0;
+  if ((size_t)want > fit) want = (int)fit;
+  return want < 1 ? 1 : want;
+}
+
+bool use_small_tile(int m, int n) {
+  // few, partly empty 128x128 tiles: smaller tiles give more workgroups and less padding
+  long long big_tiles = (long long)((m + 127) / 128) * ((n + 127) / 128);
+  return big_tiles < 128 || m <= 64 || n <= 64;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t mnv_sgemm_nn_workspace_bytes(int m, int n, int k) {
+  if (m <= 0 || n <= 0 || k <= 0) return 0;
+  bool small = use_small_tile(m, n);
+  int bm = small ? 64 : 128;
+  int tiles = ((m + bm - 1) / bm) * ((n + bm - 1) / bm);
+  int slabs = (k + 15) / 16;
+  int splits = pick_splits(tiles, slabs, (size_t)m * n, (size_t)-1);
+  return splits > 1 ? (size_t)splits * m * n * sizeof(float) : 0;
+}
+
+int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k, void* workspace,
+                 size_t workspace_bytes, mnv_stream_t stream) {
+  if (m == 0 || n == 0) return MNV_OK;
+  if (!a || !b || !c || m < 0 || n < 0 || k <= 0) return MNV_ERR_INVALID;
+  hipStream_t s = mnv_stream(stream);
+  bool vec = (m % 4 == 0) && (k % 4 == 0) && mnv_aligned16(a) && mnv_aligned16(b);
+  bool small = use_small_tile(m, n);
+  int bm = small ? 64 : 128;
+  int tiles = ((m + bm - 1) / bm) * ((n + bm - 1) / bm);
+  int slabs = (k + 15) / 16;
+  size_t ws_floats = workspace ? workspace_bytes / sizeof(float) : 0;
+  int splits = pick_splits(tiles, slabs, (size_t)m * n, ws_floats);
+  if (vec) {
+    SgemmNN<true> p{a, b, c, m, n, k};
+    return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
+                 : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
+  }
+  SgemmNN<false> p{a, b, c, m, n, k};
+  return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
+               : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
+}
+
+}  // extern "C"

@@ -1,0 +1,327 @@
+// Softmax forward / backward over an image batch {W,H,C,N}
+// (reference CPU forward minerva/op/impl/basic.cpp:219-261; cuDNN modes selected at
+// minerva/op/impl/cuda/cuda_perform.cu:339-397).
+//   instance: one softmax over the C*H*W contiguous values of each image;
+//   channel : one softmax over the C values (stride H*W) at each (n,h,w).
+// forward : y_i = exp(x_i - max) / sum_j exp(x_j - max)
+// backward: dx_i = y_i * (dy_i - sum_j dy_j*y_j)
+// Roofline: HBM bandwidth, 8 bytes per element forward and 12 backward: a line of
+// up to 8192 values is held in registers between the passes, so it is read once.
+#include <math.h>
+
+#include "mnv_common.h"
+
+namespace {
+
+#define MNV_SM_THREADS 256
+#define MNV_SM_CACHE 8  // 16-byte vectors cached per thread
+
+template <int GROUP>
+__device__ __forceinline__ float group_max(float v, float* lds) {
+  v = mnv_wave_max(v);
+  v = __shfl(v, 0, MNV_WAVE);
+  if (GROUP > MNV_WAVE) {
+    const int w = threadIdx.x / MNV_WAVE;
+    __syncthreads();
+    if ((threadIdx.x % MNV_WAVE) == 0) lds[w] = v;
+    __syncthreads();
+    v = lds[0];
+#pragma unroll
+    for (int q = 1; q < GROUP / MNV_WAVE; ++q) v = fmaxf(v, lds[q]);
+  }
+  return v;
+}
+
+template <int GROUP>
+__device__ __forceinline__ float group_sum(float v, float* lds) {
+  v = mnv_wave_sum(v);
+  v = __shfl(v, 0, MNV_WAVE);
+  if (GROUP > MNV_WAVE) {
+    const int w = threadIdx.x / MNV_WAVE;
+    __syncthreads();
+    if ((threadIdx.x % MNV_WAVE) == 0) lds[w] = v;
+    __syncthreads();
+    v = lds[0];
+#pragma unroll
+    for (int q = 1; q < GROUP / MNV_WAVE; ++q) v += lds[q];
+  }
+  return v;
+}
+
+// One line per GROUP threads; the line (len % 4 == 0, len <= GROUP*4*MNV_SM_CACHE)
+// is cached in registers.
+template <int GROUP>
+__global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_cached_kernel(
+    const float* __restrict__ in, float* __restrict__ out, int len, int lines) {
+  __shared__ float lds[MNV_SM_THREADS / MNV_WAVE];
+  constexpr int LPB = MNV_SM_THREADS / GROUP;
+  const int t = threadIdx.x % GROUP;
+  const int len4 = len >> 2;
+  // the trip count is block-uniform when GROUP spans the block; with one wavefront per
+  // line no barrier is used
+  for (int line = blockIdx.x * LPB + threadIdx.x / GROUP; line < lines; line += gridDim.x * LPB) {
+    const mnv_f4* x4 = reinterpret_cast<const mnv_f4*>(in + (size_t)line * len);
+    mnv_f4* y4 = reinterpret_cast<mnv_f4*>(out + (size_t)line * len);
+    mnv_f4 v[MNV_SM_CACHE];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < MNV_SM_CACHE; ++u) {
+      int i = t + u * GROUP;
+      if (i < len4) {
+        v[u] = x4[i];
+        mx = fmaxf(mx, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
+      }
+    }
+    mx = group_max<GROUP>(mx, lds);
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < MNV_SM_CACHE; ++u) {
+      int i = t + u * GROUP;
+      if (i < len4) {
+        v[u].x = expf(v[u].x - mx);
+        v[u].y = expf(v[u].y - mx);
+        v[u].z = expf(v[u].z - mx);
+        v[u].w = expf(v[u].w - mx);
+        s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+      }
+    }
+    s = group_sum<GROUP>(s, lds);
+#pragma unroll
+    for (int u = 0; u < MNV_SM_CACHE; ++u) {
+      int i = t + u * GROUP;
+      if (i < len4) {
+        mnv_f4 o;
+        o.x = v[u].x / s;
+        o.y = v[u].y / s;
+        o.z = v[u].z / s;
+        o.w = v[u].w / s;
+        y4[i] = o;
+      }
+    }
+  }
+}
+
+// Any length / alignment / stride: three passes over the line.  Element i of line
+// (a, b) lives at in[a*outer + b + i*stride]; `inner` = number of b values.
+template <int GROUP>
+__global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_generic_kernel(
+    const float* __restrict__ in, float* __restrict__ out, int len, int lines, int inner,
+    size_t outer, size_t stride) {
+  __shared__ float lds[MNV_SM_THREADS / MNV_WAVE];
+  constexpr int LPB = MNV_SM_THREADS / GROUP;
+  const int t = threadIdx.x % GROUP;
+  for (int line = blockIdx.x * LPB + threadIdx.x / GROUP; line < lines; line += gridDim.x * LPB) {
+    size_t base = (size_t)(line / inner) * outer + (size_t)(line % inner);
+    const float* x = in + base;
+    float* y = out + base;
+    float mx = -INFINITY;
+    for (int i = t; i < len; i += GROUP) mx = fmaxf(mx, x[i * stride]);
+    mx = group_max<GROUP>(mx, lds);
+    float s = 0.f;
+    for (int i = t; i < len; i += GROUP) {
+      float e = expf(x[i * stride] - mx);
+      y[i * stride] = e;
+      s += e;
+    }
+    s = group_sum<GROUP>(s, lds);
+    for (int i = t; i < len; i += GROUP) y[i * stride] = y[i * stride] / s;
+  }
+}
+
+template <int GROUP>
+__global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_bwd_cached_kernel(
+    const float* __restrict__ dy, const float* __restrict__ y, float* __restrict__ dx, int len,
+    int lines) {
+  __shared__ float lds[MNV_SM_THREADS / MNV_WAVE];
+  constexpr int LPB = MNV_SM_THREADS / GROUP;
+  const int t = threadIdx.x % GROUP;
+  const int len4 = len >> 2;
+  for (int line = blockIdx.x * LPB + threadIdx.x / GROUP; line < lines; line += gridDim.x * LPB) {
+    const mnv_f4* d4 = reinterpret_cast<const mnv_f4*>(dy + (size_t)line * len);
+    const mnv_f4* t4 = reinterpret_cast<const mnv_f4*>(y + (size_t)line * len);
+    mnv_f4* o4 = reinterpret_cast<mnv_f4*>(dx + (size_t)line * len);
+    mnv_f4 d[MNV_SM_CACHE], p[MNV_SM_CACHE];
+    float dot = 0.f;
+#pragma unroll
+    for (int u = 0; u < MNV_SM_CACHE; ++u) {
+      int i = t + u * GROUP;
+      if (i < len4) {
+        d[u] = d4[i];
+        p[u] = t4[i];
+        dot += (d[u].x * p[u].x + d[u].y * p[u].y) + (d[u].z * p[u].z + d[u].w * p[u].w);
+      }
+    }
+    dot = group_sum<GROUP>(dot, lds);
+#pragma unroll
+    for (int u = 0; u < MNV_SM_CACHE; ++u) {
+      int i = t + u * GROUP;
+      if (i < len4) {
+        mnv_f4 o;
+        o.x = p[u].x * (d[u].x - dot);
+        o.y = p[u].y * (d[u].y - dot);
+        o.z = p[u].z * (d[u].z - dot);
+        o.w = p[u].w * (d[u].w - dot);
+        o4[i] = o;
+      }
+    }
+  }
+}
+
+template <int GROUP>
+__global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_bwd_generic_kernel(
+    const float* __restrict__ dy, const float* __restrict__ y, float* __restrict__ dx, int len,
+    int lines, int inner, size_t outer, size_t stride) {
+  __shared__ float lds[MNV_SM_THREADS / MNV_WAVE];
+  constexpr int LPB = MNV_SM_THREADS / GROUP;
+  const int t = threadIdx.x % GROUP;
+  for (int line = blockIdx.x * LPB + threadIdx.x / GROUP; line < lines; line += gridDim.x * LPB) {
+    size_t base = (size_t)(line / inner) * outer + (size_t)(line % inner);
+    float dot = 0.f;
+    for (int i = t; i < len; i += GROUP) dot += dy[base + i * stride] * y[base + i * stride];
+    dot = group_sum<GROUP>(dot, lds);
+    for (int i = t; i < len; i += GROUP)
+      dx[base + i * stride] = y[base + i * stride] * (dy[base + i * stride] - dot);
+  }
+}
+
+// Channel mode with H*W > 1: adjacent threads own adjacent (h,w) positions, so the
+// stride-H*W walk over channels is coalesced across the wavefront.
+__global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_channel_fwd_kernel(
+    const float* __restrict__ in, float* __restrict__ out, int n, int c, int hw) {
+  size_t total = (size_t)n * hw;
+  for (size_t q = (size_t)blockIdx.x * MNV_SM_THREADS + threadIdx.x; q < total;
+       q += (size_t)gridDim.x * MNV_SM_THREADS) {
+    size_t base = (q / hw) * (size_t)c * hw + (q % hw);
+    float mx = -INFINITY;
+    for (int k = 0; k < c; ++k) mx = fmaxf(mx, in[base + (size_t)k * hw]);
+    float s = 0.f;
+    for (int k = 0; k < c; ++k) {
+      float e = expf(in[base + (size_t)k * hw] - mx);
+      out[base + (size_t)k * hw] = e;
+      s += e;
+    }
+    for (int k = 0; k < c; ++k) out[base + (size_t)k * hw] = out[base + (size_t)k * hw] / s;
+  }
+}
+
+__global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_channel_bwd_kernel(
+    const float* __restrict__ dy, const float* __restrict__ y, float* __restrict__ dx, int n,
+    int c, int hw) {
+  size_t total = (size_t)n * hw;
+  for (size_t q = (size_t)blockIdx.x * MNV_SM_THREADS + threadIdx.x; q < total;
+       q += (size_t)gridDim.x * MNV_SM_THREADS) {
+    size_t base = (q / hw) * (size_t)c * hw + (q % hw);
+    float dot = 0.f;
+    for (int k = 0; k < c; ++k) dot += dy[base + (size_t)k * hw] * y[base + (size_t)k * hw];
+    for (int k = 0; k < c; ++k)
+      dx[base + (size_t)k * hw] = y[base + (size_t)k * hw] * (dy[base + (size_t)k * hw] - dot);
+  }
+}
+
+bool dims_ok(int n, int c, int h, int w, long long* len) {
+  if (n <= 0 || c <= 0 || h <= 0 || w <= 0) return false;
+  long long l = (long long)c * h * w;
+  if (l > 0x7fffffffLL) return false;
+  *len = l;
+  return true;
+}
+
+unsigned line_grid(int lines, int lpb) {
+  size_t b = mnv_ceil_div((size_t)lines, lpb);
+  return (unsigned)(b < 65536 ? b : 65536);
+}
+
+// Contiguous lines of `len` floats (instance mode, or channel mode with H*W == 1).
+int softmax_lines_fwd(const float* in, float* out, int len, int lines, hipStream_t s) {
+  bool vec = (len % 4 == 0) && mnv_aligned16(in) && mnv_aligned16(out);
+  if (vec && len <= MNV_WAVE * 4 * MNV_SM_CACHE)
+    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_WAVE>), dim3(line_grid(lines, 4)),
+                       dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
+  else if (vec && len <= MNV_SM_THREADS * 4 * MNV_SM_CACHE)
+    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_SM_THREADS>), dim3(line_grid(lines, 1)),
+                       dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
+  else if (len <= 1024)
+    hipLaunchKernelGGL((mnv_softmax_fwd_generic_kernel<MNV_WAVE>), dim3(line_grid(lines, 4)),
+                       dim3(MNV_SM_THREADS), 0, s, in, out, len, lines, 1, (size_t)len, (size_t)1);
+  else
+    hipLaunchKernelGGL((mnv_softmax_fwd_generic_kernel<MNV_SM_THREADS>), dim3(line_grid(lines, 1)),
+                       dim3(MNV_SM_THREADS), 0, s, in, out, len, lines, 1, (size_t)len, (size_t)1);
+  return MNV_LAUNCH_STATUS();
+}
+
+int softmax_lines_bwd(const float* dy, const float* y, float* dx, int len, int lines,
+                      hipStream_t s) {
+  bool vec = (len % 4 == 0) && mnv_aligned16(dy) && mnv_aligned16(y) && mnv_aligned16(dx);
+  if (vec && len <= MNV_WAVE * 4 * MNV_SM_CACHE)
+    hipLaunchKernelGGL((mnv_softmax_bwd_cached_kernel<MNV_WAVE>), dim3(line_grid(lines, 4)),
+                       dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines);
+  else if (vec && len <= MNV_SM_THREADS * 4 * MNV_SM_CACHE)
+    hipLaunchKernelGGL((mnv_softmax_bwd_cached_kernel<MNV_SM_THREADS>), dim3(line_grid(lines, 1)),
+                       dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines);
+  else if (len <= 1024)
+    hipLaunchKernelGGL((mnv_softmax_bwd_generic_kernel<MNV_WAVE>), dim3(line_grid(lines, 4)),
+                       dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines, 1, (size_t)len, (size_t)1);
+  else
+    hipLaunchKernelGGL((mnv_softmax_bwd_generic_kernel<MNV_SM_THREADS>), dim3(line_grid(lines, 1)),
+                       dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines, 1, (size_t)len, (size_t)1);
+  return MNV_LAUNCH_STATUS();
+}
+
+}  // namespace
+
+extern "C" {
+
+int mnv_softmax_instance_fwd(const float* bottom, float* top, int num_images, int num_channels,
+                             int height, int width, mnv_stream_t stream) {
+  long long len;
+  if (!bottom || !top || !dims_ok(num_images, num_channels, height, width, &len))
+    return MNV_ERR_INVALID;
+  return softmax_lines_fwd(bottom, top, (int)len, num_images, mnv_stream(stream));
+}
+
+int mnv_softmax_channel_fwd(const float* bottom, float* top, int num_images, int num_channels,
+                            int height, int width, mnv_stream_t stream) {
+  long long len;
+  if (!bottom || !top || !dims_ok(num_images, num_channels, height, width, &len))
+    return MNV_ERR_INVALID;
+  long long hw = (long long)height * width;
+  if (hw == 1) return softmax_lines_fwd(bottom, top, num_channels, num_images, mnv_stream(stream));
+  size_t total = (size_t)num_images * hw;
+  size_t blocks = mnv_ceil_div(total, MNV_SM_THREADS);
+  if (blocks > MNV_MAX_STREAM_BLOCKS) blocks = MNV_MAX_STREAM_BLOCKS;
+  hipLaunchKernelGGL(mnv_softmax_channel_fwd_kernel, dim3((unsigned)blocks), dim3(MNV_SM_THREADS),
+                     0, mnv_stream(stream), bottom, top, num_images, num_channels, (int)hw);
+  return MNV_LAUNCH_STATUS();
+}
+
+int mnv_softmax_instance_bwd(const float* top_diff, const float* top, float* bottom_diff,
+                             int num_images, int num_channels, int height, int width,
+                             mnv_stream_t stream) {
+  long long len;
+  if (!top_diff || !top || !bottom_diff ||
+      !dims_ok(num_images, num_channels, height, width, &len))
+    return MNV_ERR_INVALID;
+  return softmax_lines_bwd(top_diff, top, bottom_diff, (int)len, num_images, mnv_stream(stream));
+}
+
+int mnv_softmax_channel_bwd(const float* top_diff, const float* top, float* bottom_diff,
+                            int num_images, int num_channels, int height, int width,
+                            mnv_stream_t stream) {
+  long long len;
+  if (!top_diff || !top || !bottom_diff ||
+      !dims_ok(num_images, num_channels, height, width, &len))
+    return MNV_ERR_INVALID;
+  long long hw = (long long)height * width;
+  if (hw == 1)
+    return softmax_lines_bwd(top_diff, top, bottom_diff, num_channels, num_images,
+                             mnv_stream(stream));
+  size_t total = (size_t)num_images * hw;
+  size_t blocks = mnv_ceil_div(total, MNV_SM_THREADS);
+  if (blocks > MNV_MAX_STREAM_BLOCKS) blocks = MNV_MAX_STREAM_BLOCKS;
+  hipLaunchKernelGGL(mnv_softmax_channel_bwd_kernel, dim3((unsigned)blocks), dim3(MNV_SM_THREADS),
+                     0, mnv_stream(stream), top_diff, top, bottom_diff, num_images, num_channels,
+                     (int)hw);
+  return MNV_LAUNCH_STATUS();
+}
+
+}  // extern "C"

@@ -1,0 +1,55 @@
+"""The C ABI library loads and exports every symbol that include/mnv_hip.h declares,
+and the ctypes binding covers all of them (no compute calls: runs without a GPU)."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "mnv_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mnv_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_a_sane_number_of_entry_points():
+    names = _declared()
+    assert len(names) >= 70
+    for must in ("mnv_sgemm_nn", "mnv_conv_fwd", "mnv_conv_bwd_data", "mnv_conv_bwd_filter",
+                 "mnv_conv_bwd_bias", "mnv_maxpool_bwd", "mnv_softmax_instance_fwd",
+                 "mnv_maxindex_col", "mnv_norm_add_row", "mnv_reduce_sum_row"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from minerva_amd import capi
+    assert os.path.exists(capi.LIB_PATH), "build the library first: python -m minerva_amd.build"
+    lib = ctypes.CDLL(capi.LIB_PATH)
+    missing = [n for n in _declared() if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_binding_covers_every_declared_symbol():
+    from minerva_amd import capi
+    declared = set(_declared())
+    bound = set(capi.PROTOTYPES)
+    assert declared == bound, (sorted(declared - bound), sorted(bound - declared))
+    capi.load()  # attaches argtypes; raises if a symbol is absent
+
+
+def test_pure_host_entry_points():
+    from minerva_amd import capi
+    L = capi.lib()
+    # pooled-size rule of narray/convolution.cpp:107-114 (golden sizes of the reference tests)
+    assert L.mnv_pooled_size(4, 3, 1, 0) == 2
+    assert L.mnv_pooled_size(4, 3, 1, 1) == 4
+    assert L.mnv_pooled_size(4, 3, 2, 1) == 3
+    assert L.mnv_pooled_size(4, 4, 3, 2) == 2
+    assert L.mnv_pooled_size(55, 3, 2, 0) == 27
+    assert L.mnv_error_string(0) == b"ok"
+    assert b"invalid" in L.mnv_error_string(-1)
+    # workspace queries are pure arithmetic
+    assert L.mnv_sgemm_nn_workspace_bytes(4096, 4096, 4096) == 0
+    assert L.mnv_sgemm_nn_workspace_bytes(1000, 256, 4096) > 0
+    assert L.mnv_conv_bwd_filter_workspace_bytes(256, 256, 384, 13, 13, 1, 1, 1, 1, 3, 3) > 0

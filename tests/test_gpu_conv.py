@@ -1,0 +1,276 @@
+"""GPU parity of the implicit-GEMM convolutions and of pooling, through the C ABI:
+the reference's golden vectors, the CPU oracle on small and AlexNet-layer shapes
+(normwise <= 1e-4; bit-exact for max pooling values and gradient routing), and at
+batch 256 the adjoint identities and sampled fp64 dot products."""
+import ctypes
+import json
+import os
+
+import numpy as np
+import pytest
+
+from gpu_util import Gpu, TOL, assert_bits_equal, normwise, say
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    return Gpu()
+
+
+def _rand(n, seed, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal(n) * scale).astype(np.float32)
+
+
+def _out(H, R, s, p):
+    return (H + 2 * p - R) // s + 1
+
+
+class Conv:
+    """Runs the three convolution passes of one geometry on the GPU."""
+
+    def __init__(self, gpu, N, C, K, H, W, ph, pw, sv, sh, R, S):
+        self.gpu, self.p = gpu, (N, C, K, H, W, ph, pw, sv, sh, R, S)
+        self.Ho, self.Wo = _out(H, R, sv, ph), _out(W, S, sh, pw)
+
+    def fwd(self, x, w, b):
+        g, p = self.gpu, self.p
+        N, C, K = p[0], p[1], p[2]
+        dx, dw, db = g.up(x), g.up(w), g.up(b)
+        dt = g.empty(N * K * self.Ho * self.Wo)
+        g.call("mnv_conv_fwd", dx.p, dw.p, db.p, dt.p, *p)
+        return g.down(dt)
+
+    def bwd_data(self, dy, w):
+        g, p = self.gpu, self.p
+        N, C, K, H, W = p[:5]
+        ddy, dw = g.up(dy), g.up(w)
+        dbd = g.up(np.full(N * C * H * W, np.nan, np.float32))  # every element must be written
+        g.call("mnv_conv_bwd_data", ddy.p, dw.p, dbd.p, *p)
+        return g.down(dbd)
+
+    def bwd_filter(self, dy, x, workspace=True):
+        g, p = self.gpu, self.p
+        N, C, K, H, W, ph, pw, sv, sh, R, S = p
+        ddy, dx = g.up(dy), g.up(x)
+        dfd = g.up(np.full(K * C * R * S, np.nan, np.float32))
+        nbytes = g.L.mnv_conv_bwd_filter_workspace_bytes(*p) if workspace else 0
+        ws = g.empty(nbytes // 4 + 1) if nbytes else None
+        g.call("mnv_conv_bwd_filter", dx.p, ddy.p, dfd.p, *p, ws.p if ws else None,
+               ctypes.c_size_t(nbytes))
+        return g.down(dfd)
+
+    def bwd_bias(self, dy):
+        g, p = self.gpu, self.p
+        ddy, db = g.up(dy), g.empty(p[2])
+        g.call("mnv_conv_bwd_bias", ddy.p, db.p, p[0], p[2], self.Ho, self.Wo)
+        return g.down(db)
+
+
+@pytest.mark.parametrize("case", json.load(open(os.path.join(GOLD, "conv_forward.json"))),
+                         ids=lambda c: c["name"])
+def test_conv_forward_golden(gpu, case):
+    W, H, C, N = case["input_size"]
+    S, R, _, K = case["weight_size"]
+    x = np.array(case["input"], np.float32)
+    w = np.array(case["weight"], np.float32)
+    b = np.array(case["bias"] or [0] * K, np.float32)
+    cv = Conv(gpu, N, C, K, H, W, case["pad_height"], case["pad_width"], case["stride_vertical"],
+              case["stride_horizontal"], R, S)
+    got = cv.fwd(x, w, b)
+    Wo, Ho, _, _ = case["correct_size"]
+    idx = np.arange(got.size)
+    want = np.array(case["correct_without_bias"], np.float32) + b[(idx // (Wo * Ho)) % K]
+    assert np.max(np.abs(got - want)) < 1e-3   # tests/unittest_conv_forward.cpp:32,66
+    assert np.max(np.abs(got - want)) < 2e-5
+
+
+CASES = [
+    # N, C, K, H, W, ph, pw, sv, sh, R, S
+    (2, 3, 4, 7, 9, 0, 0, 1, 1, 3, 5),
+    (2, 2, 3, 8, 7, 2, 1, 2, 3, 3, 2),      # strided, padded, ragged fit
+    (1, 4, 2, 6, 6, 1, 1, 1, 1, 3, 3),
+    (3, 5, 7, 11, 13, 2, 3, 1, 2, 5, 4),
+    (1, 1, 1, 1, 1, 0, 0, 1, 1, 1, 1),
+    (2, 1, 16, 28, 28, 0, 0, 1, 1, 5, 5),   # MNIST CNN layer 1
+    (2, 16, 32, 12, 12, 0, 0, 1, 1, 5, 5),  # MNIST CNN layer 2
+    (2, 16, 32, 12, 12, 2, 2, 1, 1, 5, 5),  # same with the reference app's padding
+    (5, 130, 70, 9, 9, 1, 1, 1, 1, 3, 3),   # more than one tile in both GEMM dimensions
+    (2, 8, 140, 20, 20, 1, 1, 2, 2, 3, 3),
+]
+
+
+@pytest.mark.parametrize("p", CASES)
+def test_conv_all_passes_against_oracle(gpu, ora, p):
+    N, C, K, H, W, ph, pw, sv, sh, R, S = p
+    cv = Conv(gpu, *p)
+    x, w, b = _rand(N * C * H * W, 40), _rand(K * C * R * S, 41), _rand(K, 42)
+    dy = _rand(N * K * cv.Ho * cv.Wo, 43)
+    say("conv fwd", p)
+    assert normwise(cv.fwd(x, w, b), ora.conv_fwd(x, w, b, *p)) <= TOL
+    say("conv bwd data", p)
+    assert normwise(cv.bwd_data(dy, w), ora.conv_bwd_data(dy, w, *p)) <= TOL
+    ref = ora.conv_bwd_filter(dy, x, *p)
+    for ws in (True, False):
+        say("conv bwd filter", p, ws)
+        assert normwise(cv.bwd_filter(dy, x, ws), ref) <= TOL
+    say("conv bwd bias", p)
+    assert normwise(cv.bwd_bias(dy), ora.conv_bwd_bias(dy, N, K, cv.Ho, cv.Wo)) <= TOL
+
+
+ALEXNET = [
+    # name, N, C, K, H, W, ph, pw, sv, sh, R, S   (owl/apps/imagenet_alexnet/alexnet.py:9-32)
+    ("conv1", 1, 3, 96, 227, 227, 0, 0, 4, 4, 11, 11),
+    ("conv2", 1, 96, 256, 27, 27, 2, 2, 1, 1, 5, 5),
+    ("conv3", 1, 256, 384, 13, 13, 1, 1, 1, 1, 3, 3),
+    ("conv4", 1, 384, 384, 13, 13, 1, 1, 1, 1, 3, 3),
+    ("conv5", 2, 384, 256, 13, 13, 1, 1, 1, 1, 3, 3),
+]
+
+
+@pytest.mark.parametrize("case", ALEXNET, ids=lambda c: c[0])
+def test_conv_alexnet_layers_small_batch_against_oracle(gpu, ora, case):
+    name, p = case[0], case[1:]
+    N, C, K, H, W, ph, pw, sv, sh, R, S = p
+    cv = Conv(gpu, *p)
+    x, w = _rand(N * C * H * W, 44), _rand(K * C * R * S, 45, 0.01)
+    b = _rand(K, 46, 0.1)
+    dy = _rand(N * K * cv.Ho * cv.Wo, 47)
+    say(name, "fwd")
+    assert normwise(cv.fwd(x, w, b), ora.conv_fwd(x, w, b, *p)) <= TOL
+    say(name, "bwd filter")
+    assert normwise(cv.bwd_filter(dy, x), ora.conv_bwd_filter(dy, x, *p)) <= TOL
+    say(name, "bwd data")
+    assert normwise(cv.bwd_data(dy, w), ora.conv_bwd_data(dy, w, *p)) <= TOL
+
+
+@pytest.mark.parametrize("case", [ALEXNET[1], ALEXNET[4], ALEXNET[0]], ids=lambda c: c[0])
+def test_conv_batch_256_properties(gpu, case):
+    name, p = case[0], (256,) + case[2:]
+    N, C, K, H, W, ph, pw, sv, sh, R, S = p
+    cv = Conv(gpu, *p)
+    x, w = _rand(N * C * H * W, 48), _rand(K * C * R * S, 49, 0.05)
+    b = np.zeros(K, np.float32)
+    dy = _rand(N * K * cv.Ho * cv.Wo, 50)
+    say(name, "b256 fwd")
+    y = cv.fwd(x, w, b)
+    # sampled outputs against an fp64 dot product written from the definition
+    X = x.reshape(N, C, H, W)
+    Wt = w.reshape(K, C, R, S)[:, :, ::-1, ::-1].astype(np.float64)
+    Y = y.reshape(N, K, cv.Ho, cv.Wo)
+    rng = np.random.default_rng(51)
+    worst = 0.0
+    for _ in range(40):
+        n, k = rng.integers(N), rng.integers(K)
+        i, j = rng.integers(cv.Ho), rng.integers(cv.Wo)
+        if _ < 8:  # borders, where padding and the last tile live
+            n, i, j = (N - 1, cv.Ho - 1, cv.Wo - 1) if _ % 2 else (0, 0, 0)
+        acc = 0.0
+        for r in range(R):
+            yy = i * sv - ph + r
+            if not 0 <= yy < H:
+                continue
+            xs = np.arange(S) + j * sh - pw
+            ok = (xs >= 0) & (xs < W)
+            acc += float(np.sum(X[n, :, yy, xs[ok]].astype(np.float64).T * Wt[k, :, r, ok].T))
+        worst = max(worst, abs(Y[n, k, i, j] - acc))
+    assert worst <= TOL * np.max(np.abs(y))
+    lhs = float(np.dot(y.astype(np.float64), dy.astype(np.float64)))
+    scale = float(np.linalg.norm(y.astype(np.float64)) * np.linalg.norm(dy.astype(np.float64)))
+    say(name, "b256 bwd filter")
+    dw = cv.bwd_filter(dy, x)
+    assert abs(float(np.dot(dw.astype(np.float64), w.astype(np.float64))) - lhs) <= 1e-5 * scale
+    if name != "conv1":  # the network never asks for conv1's data gradient
+        say(name, "b256 bwd data")
+        dx = cv.bwd_data(dy, w)
+        assert abs(float(np.dot(dx.astype(np.float64), x.astype(np.float64))) - lhs) <= 1e-5 * scale
+    db = cv.bwd_bias(dy)
+    assert normwise(db, dy.reshape(N, K, -1).astype(np.float64).sum(axis=(0, 2))) <= TOL
+
+
+# ------------------------------------------------------------------- pooling
+
+@pytest.mark.parametrize("case", json.load(open(os.path.join(GOLD, "pooling_forward.json"))),
+                         ids=lambda c: c["name"])
+def test_pooling_forward_golden(gpu, case):
+    W, H, C, N = case["input_size"]
+    Wo, Ho, _, _ = case["correct_size"]
+    geo = (N, C, H, W, case["stride_vertical"], case["stride_horizontal"], case["height"],
+           case["width"], case["pad_height"], case["pad_width"])
+    assert gpu.L.mnv_pooled_size(H, case["height"], case["stride_vertical"], case["pad_height"]) == Ho
+    assert gpu.L.mnv_pooled_size(W, case["width"], case["stride_horizontal"], case["pad_width"]) == Wo
+    dx, dt = gpu.up(np.array(case["input"], np.float32)), gpu.empty(Wo * Ho * C * N)
+    gpu.call("mnv_maxpool_fwd", dx.p, dt.p, *geo)
+    np.testing.assert_array_equal(gpu.down(dt), np.array(case["correct"], np.float32))
+
+
+POOL = [
+    # N, C, H, W, sv, sh, kh, kw, ph, pw
+    (2, 3, 7, 9, 2, 2, 3, 3, 0, 0),
+    (1, 2, 6, 5, 2, 3, 3, 2, 1, 1),
+    (2, 2, 8, 8, 2, 2, 2, 2, 0, 0),
+    (1, 1, 5, 5, 1, 1, 3, 3, 1, 1),
+    (2, 96, 55, 55, 2, 2, 3, 3, 0, 0),    # AlexNet pool1
+    (2, 256, 27, 27, 2, 2, 3, 3, 0, 0),   # pool2
+    (3, 256, 13, 13, 2, 2, 3, 3, 0, 0),   # pool5
+    (4, 16, 24, 24, 2, 2, 2, 2, 0, 0),    # MNIST CNN pools
+    (4, 32, 12, 12, 3, 3, 3, 3, 0, 0),
+]
+
+
+@pytest.mark.parametrize("p", POOL)
+@pytest.mark.parametrize("ties", [False, True])
+def test_pooling_against_oracle(gpu, ora, p, ties):
+    N, C, H, W, sv, sh, kh, kw, ph, pw = p
+    rng = np.random.default_rng(52)
+    if ties:   # relu-like data: many equal values, whole windows of zeros
+        x = np.maximum(rng.integers(-3, 3, size=N * C * H * W), 0).astype(np.float32)
+    else:
+        x = rng.standard_normal(N * C * H * W).astype(np.float32)
+    Ho, Wo = ora.pooled_size(H, kh, sv, ph), ora.pooled_size(W, kw, sh, pw)
+    dy = rng.standard_normal(N * C * Ho * Wo).astype(np.float32)
+    dx, dt = gpu.up(x), gpu.empty(dy.size)
+    say("pool", p, "ties" if ties else "")
+    gpu.call("mnv_maxpool_fwd", dx.p, dt.p, *p)
+    top = gpu.down(dt)
+    assert_bits_equal(top, ora.pool_fwd(ora.POOL_MAX, x, *p), "maxpool fwd")
+    ddy, dbd = gpu.up(dy), gpu.up(np.full(x.size, np.nan, np.float32))
+    gpu.call("mnv_maxpool_bwd", dx.p, dt.p, ddy.p, dbd.p, *p)
+    ref, mask = ora.pool_bwd(ora.POOL_MAX, dy, top, x, *p, want_mask=True)
+    assert_bits_equal(gpu.down(dbd), ref, "maxpool bwd (same accumulation order)")
+    # routing mask: a gradient of all ones counts, per position, the windows it wins
+    ones = gpu.up(np.ones(dy.size, np.float32))
+    gpu.call("mnv_maxpool_bwd", dx.p, dt.p, ones.p, dbd.p, *p)
+    counts = np.zeros(x.size, np.float32)
+    plane = np.repeat(np.arange(N * C), Ho * Wo) * (H * W)
+    np.add.at(counts, plane + mask.astype(np.int64), 1.0)
+    assert_bits_equal(gpu.down(dbd), counts, "maxpool routing mask")
+    gpu.call("mnv_avgpool_fwd", dx.p, dt.p, *p)
+    avg = gpu.down(dt)
+    assert normwise(avg, ora.pool_fwd(ora.POOL_AVG, x, *p)) <= TOL
+    gpu.call("mnv_avgpool_bwd", dx.p, dt.p, ddy.p, dbd.p, *p)
+    assert normwise(gpu.down(dbd), ora.pool_bwd(ora.POOL_AVG, dy, avg, x, *p)) <= TOL
+
+
+def test_pooling_batch_256_properties(gpu):
+    p = (256, 96, 55, 55, 2, 2, 3, 3, 0, 0)
+    N, C, H, W = p[:4]
+    x = _rand(N * C * H * W, 53)
+    dx, dt = gpu.up(x), gpu.empty(N * C * 27 * 27)
+    gpu.call("mnv_maxpool_fwd", dx.p, dt.p, *p)
+    top = gpu.down(dt).reshape(N * C, 27, 27)
+    X = x.reshape(N * C, H, W)
+    want = np.full((N * C, 27, 27), -np.inf, np.float32)
+    for r in range(3):
+        for s in range(3):
+            want = np.maximum(want, X[:, r:r + 53:2, s:s + 53:2])
+    assert_bits_equal(top, want, "pool1 b256")
+    dy = _rand(top.size, 54)
+    ddy, dbd = gpu.up(dy), gpu.empty(x.size)
+    gpu.call("mnv_maxpool_bwd", dx.p, dt.p, ddy.p, dbd.p, *p)
+    g = gpu.down(dbd)
+    # continuous data has no ties: every window routes to exactly one position
+    assert abs(float(g.astype(np.float64).sum()) - float(dy.astype(np.float64).sum())) < 1e-2
+    assert np.count_nonzero(g) <= dy.size

@@ -1,0 +1,176 @@
+"""GPU parity of the HBM-streaming ops against the CPU oracle, through the C ABI.
+Bit-exact: add/sub/mul/div, scalar ops, neg, relu forward/backward, fill, copy,
+broadcast add/sub/mul/div.  Normwise <= 1e-4: exp, ln, sigmoid, tanh and the sigmoid /
+tanh gradients."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from gpu_util import Gpu, TOL, assert_bits_equal, normwise, say
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [1, 3, 4, 255, 1024, 4097, 1 << 20, (1 << 20) + 3]
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    return Gpu()
+
+
+def _rand(n, seed, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal(n) * scale).astype(np.float32)
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_binary_ops_bit_exact(gpu, ora, n):
+    a, b = _rand(n, 1), _rand(n, 2)
+    b[b == 0] = 1
+    da, db, dc = gpu.up(a), gpu.up(b), gpu.empty(n)
+    for name, typ in (("mnv_add", ora.ADD), ("mnv_sub", ora.SUB), ("mnv_mul", ora.MUL),
+                      ("mnv_div", ora.DIV)):
+        say(name, n)
+        gpu.call(name, da.p, db.p, dc.p, n)
+        assert_bits_equal(gpu.down(dc), ora.arithmetic(typ, a, b), name)
+
+
+def test_binary_ops_unaligned_pointers(gpu, ora):
+    n = 10001
+    a, b = _rand(n + 1, 3), _rand(n + 1, 4)
+    da, db, dc = gpu.up(a), gpu.up(b), gpu.empty(n + 1)
+    gpu.call("mnv_add", da.offset(1), db.offset(1), dc.offset(1), n)
+    assert_bits_equal(gpu.down(dc)[1:], ora.arithmetic(ora.ADD, a[1:], b[1:]), "add+1")
+
+
+def test_binary_ops_special_values(gpu, ora):
+    sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 3.4e38, 1.17e-38, 1, -1],
+                  np.float32)
+    a = np.repeat(sp, sp.size)
+    b = np.tile(sp, sp.size)
+    da, db, dc = gpu.up(a), gpu.up(b), gpu.empty(a.size)
+    for name, typ in (("mnv_add", ora.ADD), ("mnv_sub", ora.SUB), ("mnv_mul", ora.MUL),
+                      ("mnv_div", ora.DIV)):
+        gpu.call(name, da.p, db.p, dc.p, a.size)
+        assert_bits_equal(gpu.down(dc), ora.arithmetic(typ, a, b), name + " specials")
+
+
+def test_binary_full_size_8192x8192(gpu, ora):
+    n = 8192 * 8192
+    a, b = _rand(n, 5), _rand(n, 6)
+    da, db, dc = gpu.up(a), gpu.up(b), gpu.empty(n)
+    for name, typ in (("mnv_add", ora.ADD), ("mnv_mul", ora.MUL), ("mnv_sub", ora.SUB)):
+        say(name, "8192x8192")
+        gpu.call(name, da.p, db.p, dc.p, n)
+        assert_bits_equal(gpu.down(dc), ora.arithmetic(typ, a, b), name)
+
+
+@pytest.mark.parametrize("n", [1, 5, 4099, 1 << 18])
+def test_scalar_ops_bit_exact(gpu, ora, n):
+    x = _rand(n, 7)
+    x[x == 0] = 2
+    v = 3.291  # tests/unittest_arithmetic_const.cpp:75
+    dx, dy = gpu.up(x), gpu.empty(n)
+    table = [("mnv_const_add", ora.ADD, 1), ("mnv_const_sub", ora.SUB, 1),
+             ("mnv_const_rsub", ora.SUB, 0), ("mnv_const_mul", ora.MUL, 1),
+             ("mnv_const_div", ora.DIV, 1), ("mnv_const_rdiv", ora.DIV, 0)]
+    for name, typ, side in table:
+        say(name, n)
+        gpu.call(name, dx.p, dy.p, ctypes.c_float(v), n)
+        assert_bits_equal(gpu.down(dy), ora.arithmetic_const(typ, side, v, x), name)
+
+
+def test_left_const_chain(gpu, ora):
+    # tests/unittest_leftconst.cpp:7-49: chained (c - x)
+    x = _rand(720, 8)
+    dx, d1, d2 = gpu.up(x), gpu.empty(720), gpu.empty(720)
+    gpu.call("mnv_const_rsub", dx.p, d1.p, ctypes.c_float(2.5), 720)
+    gpu.call("mnv_const_rsub", d1.p, d2.p, ctypes.c_float(-1.25), 720)
+    want = ora.arithmetic_const(ora.SUB, 0, -1.25, ora.arithmetic_const(ora.SUB, 0, 2.5, x))
+    assert_bits_equal(gpu.down(d2), want, "left const chain")
+
+
+@pytest.mark.parametrize("n", [1, 7, 4098, 1 << 20])
+def test_unary_ops(gpu, ora, n):
+    x = _rand(n, 9, 3.0)
+    dx, dy = gpu.up(x), gpu.empty(n)
+    gpu.call("mnv_neg", dx.p, dy.p, n)
+    assert_bits_equal(gpu.down(dy), ora.elewise(ora.NEG, x), "neg")
+    gpu.call("mnv_exp", dx.p, dy.p, n)
+    got, ref = gpu.down(dy), ora.elewise(ora.EXP, x)
+    assert np.max(np.abs(got / ref - 1)) <= TOL  # elementwise relative, stricter than normwise
+    pos = np.abs(x) + np.float32(500)  # tests/unittest_elewise.cpp: ln on N(500,1)
+    dp = gpu.up(pos)
+    gpu.call("mnv_ln", dp.p, dy.p, n)
+    assert normwise(gpu.down(dy), ora.elewise(ora.LN, pos)) <= TOL
+    gpu.call("mnv_copy", dx.p, dy.p, n)
+    assert_bits_equal(gpu.down(dy), x, "copy")
+    gpu.call("mnv_fill", dy.p, n, ctypes.c_float(-1.5))
+    assert_bits_equal(gpu.down(dy), np.full(n, -1.5, np.float32), "fill")
+
+
+@pytest.mark.parametrize("n", [1, 6, 7 * 6 * 3 * 2, 4099, 1 << 20])
+def test_activation_forward(gpu, ora, n):
+    x = _rand(n, 10, 2.0)
+    if n >= 6:
+        x[:6] = [0.0, -0.0, np.nan, -1.0, 1.0, 1e-30]
+    dx, dy = gpu.up(x), gpu.empty(n)
+    gpu.call("mnv_relu_fwd", dx.p, dy.p, n)
+    assert_bits_equal(gpu.down(dy), ora.activation_fwd(ora.RELU, x), "relu")
+    x = np.nan_to_num(x)
+    dx = gpu.up(x)
+    gpu.call("mnv_sigmoid_fwd", dx.p, dy.p, n)
+    assert normwise(gpu.down(dy), ora.activation_fwd(ora.SIGMOID, x)) <= TOL
+    gpu.call("mnv_tanh_fwd", dx.p, dy.p, n)
+    assert normwise(gpu.down(dy), ora.activation_fwd(ora.TANH, x)) <= TOL
+
+
+@pytest.mark.parametrize("n", [1, 5, 4099, 1 << 20])
+def test_activation_backward(gpu, ora, n):
+    x = _rand(n, 11, 2.0)
+    if n >= 5:
+        x[:5] = [0.0, -0.0, -2.0, 2.0, 1e-30]
+    dy = _rand(n, 12)
+    dxb, ddy, dout = gpu.up(x), gpu.up(dy), gpu.empty(n)
+    for name, alg in (("mnv_relu_bwd", ora.RELU), ("mnv_sigmoid_bwd", ora.SIGMOID),
+                      ("mnv_tanh_bwd", ora.TANH)):
+        y = ora.activation_fwd(alg, x)
+        dyt = gpu.up(y)
+        say(name, n)
+        gpu.call(name, dxb.p, dyt.p, ddy.p, dout.p, n)
+        ref = ora.activation_bwd(alg, dy, y, x)
+        if alg == ora.RELU:
+            assert_bits_equal(gpu.down(dout), ref, name)
+        else:
+            assert normwise(gpu.down(dout), ref) <= TOL
+
+
+NORM_SHAPES = [(9, 7), (1, 5), (5, 1), (1000, 33), (4096, 256), (8192, 64), (10, 256)]
+
+
+@pytest.mark.parametrize("m,n", NORM_SHAPES)
+def test_norm_arithmetic_bit_exact(gpu, ora, m, n):
+    x = _rand(m * n, 13)
+    row = _rand(n, 14)  # shape {1,n}: replicated along dim 0
+    col = _rand(m, 15)  # shape {m,1}: replicated along dim 1
+    row[row == 0] = 1
+    col[col == 0] = 1
+    dx, dr, dc, do = gpu.up(x), gpu.up(row), gpu.up(col), gpu.empty(m * n)
+    for op, typ in (("add", ora.ADD), ("sub", ora.SUB), ("mul", ora.MUL), ("div", ora.DIV)):
+        say("norm", op, m, n)
+        gpu.call("mnv_norm_%s_col" % op, dx.p, dr.p, do.p, m, n)
+        assert_bits_equal(gpu.down(do), ora.norm_arithmetic(typ, x, [m, n], row, [0]), op + "_col")
+        gpu.call("mnv_norm_%s_row" % op, dx.p, dc.p, do.p, m, n)
+        assert_bits_equal(gpu.down(do), ora.norm_arithmetic(typ, x, [m, n], col, [1]), op + "_row")
+
+
+def test_invalid_arguments_are_rejected(gpu):
+    L = gpu.L
+    d = gpu.empty(16)
+    assert L.mnv_add(None, d.p, d.p, 16, gpu.dev.stream) == -1
+    assert L.mnv_add(None, None, None, 0, gpu.dev.stream) == 0  # empty input is a no-op
+    assert L.mnv_norm_add_col(d.p, d.p, d.p, -1, 4, gpu.dev.stream) == -1
+    assert L.mnv_reduce_sum_col(d.p, d.p, 0, 4, gpu.dev.stream) == -1
+    assert L.mnv_sgemm_nn(d.p, d.p, d.p, 4, 4, 0, None, 0, gpu.dev.stream) == -1
+    assert L.mnv_conv_fwd(d.p, d.p, d.p, d.p, 1, 1, 1, 2, 2, 0, 0, 1, 1, 3, 3, gpu.dev.stream) == -1
+    assert L.mnv_maxpool_fwd(d.p, d.p, 1, 1, 4, 4, 0, 1, 2, 2, 0, 0, gpu.dev.stream) == -1

@@ -1,0 +1,161 @@
+"""GPU parity of reductions, arg-max, softmax and transpose against the CPU oracle.
+Bit-exact: max, arg-max indices (ties, NaN), transpose.  Normwise <= 1e-4: sums and
+softmax forward/backward."""
+import numpy as np
+import pytest
+
+from gpu_util import Gpu, TOL, assert_bits_equal, normwise, say
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    return Gpu()
+
+
+def _rand(n, seed):
+    return np.random.default_rng(seed).standard_normal(n).astype(np.float32)
+
+
+def test_reference_closed_forms(gpu):
+    # tests/unittest_reduction.cpp:6-149, {5,3} iota
+    x = np.arange(15, dtype=np.float32)
+    dx, do = gpu.up(x), gpu.empty(5)
+    gpu.call("mnv_reduce_max_col", dx.p, do.p, 5, 3)
+    np.testing.assert_array_equal(gpu.down(do, 3), [4, 9, 14])
+    gpu.call("mnv_reduce_max_row", dx.p, do.p, 5, 3)
+    np.testing.assert_array_equal(gpu.down(do, 5), [10, 11, 12, 13, 14])
+    gpu.call("mnv_reduce_sum_col", dx.p, do.p, 5, 3)
+    np.testing.assert_array_equal(gpu.down(do, 3), [10, 35, 60])
+    gpu.call("mnv_reduce_sum_row", dx.p, do.p, 5, 3)
+    np.testing.assert_array_equal(gpu.down(do, 5), [15, 18, 21, 24, 27])
+    gpu.call("mnv_maxindex_col", dx.p, do.p, 5, 3)
+    np.testing.assert_array_equal(gpu.down(do, 3), [4, 4, 4])
+    gpu.call("mnv_maxindex_row", dx.p, do.p, 5, 3)
+    np.testing.assert_array_equal(gpu.down(do, 5), [2, 2, 2, 2, 2])
+
+
+SHAPES = [(1, 1), (1, 9), (9, 1), (5, 3), (10, 256), (1000, 256), (1000, 37), (4096, 256),
+          (2050, 130), (64, 3000), (8192, 512), (515, 8192)]
+
+
+@pytest.mark.parametrize("m,n", SHAPES)
+def test_reductions(gpu, ora, m, n):
+    x = _rand(m * n, 20)
+    dx = gpu.up(x)
+    dcol, drow = gpu.empty(n), gpu.empty(m)
+    say("reduce", m, n)
+    gpu.call("mnv_reduce_max_col", dx.p, dcol.p, m, n)
+    assert_bits_equal(gpu.down(dcol), ora.reduction(ora.MAX, x, [m, n], [0]), "max_col")
+    gpu.call("mnv_reduce_max_row", dx.p, drow.p, m, n)
+    assert_bits_equal(gpu.down(drow), ora.reduction(ora.MAX, x, [m, n], [1]), "max_row")
+    gpu.call("mnv_maxindex_col", dx.p, dcol.p, m, n)
+    assert_bits_equal(gpu.down(dcol), ora.maxindex(x, [m, n], 0), "maxindex_col")
+    gpu.call("mnv_maxindex_row", dx.p, drow.p, m, n)
+    assert_bits_equal(gpu.down(drow), ora.maxindex(x, [m, n], 1), "maxindex_row")
+    gpu.call("mnv_reduce_sum_col", dx.p, dcol.p, m, n)
+    ref = ora.reduction(ora.SUM, x, [m, n], [0])
+    x64 = x.reshape(n, m).astype(np.float64)
+    assert normwise(gpu.down(dcol), ref) <= TOL
+    assert normwise(gpu.down(dcol), x64.sum(axis=1)) <= TOL
+    gpu.call("mnv_reduce_sum_row", dx.p, drow.p, m, n)
+    ref = ora.reduction(ora.SUM, x, [m, n], [1])
+    assert normwise(gpu.down(drow), ref) <= TOL
+    assert normwise(gpu.down(drow), x64.sum(axis=0)) <= TOL
+
+
+@pytest.mark.parametrize("m,n", [(8, 4), (1024, 64), (4100, 67), (300, 5000)])
+def test_max_and_argmax_with_ties_nan_and_signed_zero(gpu, ora, m, n):
+    rng = np.random.default_rng(21)
+    x = rng.integers(-2, 3, size=m * n).astype(np.float32)  # heavy ties
+    x[x == 0] = np.where(rng.random(np.count_nonzero(x == 0)) < 0.5, 0.0, -0.0)
+    x[rng.random(m * n) < 0.05] = np.nan
+    a = x.reshape(n, m)
+    a[0, :] = np.nan           # a whole column of NaN; NaN first in every row
+    if n > 2:
+        a[1, 0] = np.nan       # NaN first in a column whose rest is finite
+        a[2, :] = -np.inf      # all -inf column
+    x = a.ravel().copy()
+    dx, dcol, drow = gpu.up(x), gpu.empty(n), gpu.empty(m)
+    for name, out, ref in (
+            ("mnv_reduce_max_col", dcol, ora.reduction(ora.MAX, x, [m, n], [0])),
+            ("mnv_reduce_max_row", drow, ora.reduction(ora.MAX, x, [m, n], [1])),
+            ("mnv_maxindex_col", dcol, ora.maxindex(x, [m, n], 0)),
+            ("mnv_maxindex_row", drow, ora.maxindex(x, [m, n], 1))):
+        say(name, m, n)
+        gpu.call(name, dx.p, out.p, m, n)
+        assert_bits_equal(gpu.down(out), ref, name)
+
+
+def test_max_and_argmax_full_size(gpu, ora):
+    m = n = 8192
+    x = _rand(m * n, 22)
+    dx, dcol, drow = gpu.up(x), gpu.empty(n), gpu.empty(m)
+    a = x.reshape(n, m)
+    gpu.call("mnv_reduce_max_col", dx.p, dcol.p, m, n)
+    assert_bits_equal(gpu.down(dcol), a.max(axis=1), "max_col 8192")
+    gpu.call("mnv_reduce_max_row", dx.p, drow.p, m, n)
+    assert_bits_equal(gpu.down(drow), a.max(axis=0), "max_row 8192")
+    gpu.call("mnv_maxindex_col", dx.p, dcol.p, m, n)
+    assert_bits_equal(gpu.down(dcol), ora.maxindex(x, [m, n], 0), "maxindex_col 8192")
+    gpu.call("mnv_maxindex_row", dx.p, drow.p, m, n)
+    assert_bits_equal(gpu.down(drow), a.argmax(axis=0).astype(np.float32), "maxindex_row 8192")
+    gpu.call("mnv_reduce_sum_col", dx.p, dcol.p, m, n)
+    assert normwise(gpu.down(dcol), a.astype(np.float64).sum(axis=1)) <= TOL
+    gpu.call("mnv_reduce_sum_row", dx.p, drow.p, m, n)
+    assert normwise(gpu.down(drow), a.astype(np.float64).sum(axis=0)) <= TOL
+
+
+SOFTMAX = [(1, 1), (10, 256), (1000, 256), (7, 33), (256, 100), (2048, 64), (8192, 48),
+           (8193, 5), (9000, 3), (40000, 2)]
+
+
+@pytest.mark.parametrize("length,lines", SOFTMAX)
+def test_softmax_instance(gpu, ora, length, lines):
+    x = _rand(length * lines, 23) * 4
+    dy = _rand(length * lines, 24)
+    dx, dout = gpu.up(x), gpu.empty(x.size)
+    say("softmax instance", length, lines)
+    gpu.call("mnv_softmax_instance_fwd", dx.p, dout.p, lines, length, 1, 1)
+    y = gpu.down(dout)
+    ref = ora.softmax_instance_fwd(x, lines, length, 1, 1)
+    assert normwise(y, ref) <= TOL
+    assert np.max(np.abs(y.reshape(lines, length).astype(np.float64).sum(axis=1) - 1)) < 1e-4
+    # {W,H,C,N} with H, W > 1 is the same contiguous line
+    if length % 6 == 0:
+        gpu.call("mnv_softmax_instance_fwd", dx.p, dout.p, lines, length // 6, 2, 3)
+        assert_bits_equal(gpu.down(dout), y, "instance chw")
+    gpu.call("mnv_softmax_channel_fwd", dx.p, dout.p, lines, length, 1, 1)
+    assert_bits_equal(gpu.down(dout), y, "channel with H=W=1 equals instance")
+    dyd, dtop = gpu.up(dy), gpu.up(ref)
+    gpu.call("mnv_softmax_instance_bwd", dyd.p, dtop.p, dout.p, lines, length, 1, 1)
+    assert normwise(gpu.down(dout), ora.softmax_instance_bwd(dy, ref, lines, length, 1, 1)) <= TOL
+
+
+@pytest.mark.parametrize("n,c,h,w", [(2, 5, 3, 4), (3, 10, 1, 7), (4, 21, 13, 13), (1, 2, 1, 2)])
+def test_softmax_channel(gpu, ora, n, c, h, w):
+    x = _rand(n * c * h * w, 25) * 3
+    dy = _rand(x.size, 26)
+    dx, dout = gpu.up(x), gpu.empty(x.size)
+    gpu.call("mnv_softmax_channel_fwd", dx.p, dout.p, n, c, h, w)
+    ref = ora.softmax_channel_fwd(x, n, c, h, w)
+    assert normwise(gpu.down(dout), ref) <= TOL
+    dyd, dtop = gpu.up(dy), gpu.up(ref)
+    gpu.call("mnv_softmax_channel_bwd", dyd.p, dtop.p, dout.p, n, c, h, w)
+    assert normwise(gpu.down(dout), ora.softmax_channel_bwd(dy, ref, n, c, h, w)) <= TOL
+
+
+@pytest.mark.parametrize("m,n", [(1, 1), (3, 4), (64, 64), (65, 63), (1000, 37), (256, 784),
+                                 (4096, 9216), (10, 256)])
+def test_transpose_bit_exact(gpu, ora, m, n):
+    x = _rand(m * n, 27)       # a is {m,n}
+    dx, dout = gpu.up(x), gpu.empty(m * n)
+    say("transpose", m, n)
+    gpu.call("mnv_transpose", dx.p, dout.p, m, n)
+    # oracle: in{n_o,m_o} -> out{m_o,n_o}; here in = {m,n} so m_o = n, n_o = m
+    assert_bits_equal(gpu.down(dout), ora.transpose(x, n, m), "transpose")
+    # involution: transposing back restores the input
+    dback = gpu.empty(m * n)
+    gpu.call("mnv_transpose", dout.p, dback.p, n, m)
+    assert_bits_equal(gpu.down(dback), x, "transpose twice")

@@ -1,0 +1,99 @@
+"""GPU parity of the MFMA SGEMM against the CPU oracle (normwise <= 1e-4) and, at
+sizes the oracle cannot reach, against properties: an fp64 reference on sampled
+entries, exact reproduction of a permuted operand, and linearity."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from gpu_util import Gpu, TOL, assert_bits_equal, normwise, say
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    return Gpu()
+
+
+def _rand(n, seed):
+    return np.random.default_rng(seed).standard_normal(n).astype(np.float32)
+
+
+def _gemm(gpu, a, b, m, n, k, workspace=True):
+    da, db, dc = gpu.up(a), gpu.up(b), gpu.empty(m * n)
+    ws_bytes = gpu.L.mnv_sgemm_nn_workspace_bytes(m, n, k) if workspace else 0
+    ws = gpu.empty(ws_bytes // 4 + 1) if ws_bytes else None
+    gpu.call("mnv_sgemm_nn", da.p, db.p, dc.p, m, n, k, ws.p if ws else None,
+             ctypes.c_size_t(ws_bytes))
+    return gpu.down(dc)
+
+
+SMALL = [(3, 5, 2), (1, 1, 1), (37, 29, 53), (64, 64, 16), (128, 128, 128), (130, 70, 19),
+         (256, 256, 784), (10, 256, 256), (256, 10, 256), (257, 129, 65), (1000, 256, 512),
+         (4, 4, 4096), (512, 384, 100)]
+
+
+@pytest.mark.parametrize("m,n,k", SMALL)
+@pytest.mark.parametrize("workspace", [True, False])
+def test_sgemm_against_oracle(gpu, ora, m, n, k, workspace):
+    a, b = _rand(m * k, 30), _rand(k * n, 31)
+    say("sgemm", m, n, k, "workspace" if workspace else "no workspace")
+    got = _gemm(gpu, a, b, m, n, k, workspace)
+    ref = ora.matmult(a, b, m, n, k, fast=True)
+    assert normwise(got, ref) <= TOL
+    A = a.reshape(k, m).T.astype(np.float64)
+    B = b.reshape(n, k).T.astype(np.float64)
+    assert normwise(got.reshape(n, m).T, A @ B) <= TOL
+
+
+def test_sgemm_reference_unit_test_shape(gpu):
+    # tests/unittest_sgemm.cpp:7-28: {3,2} x {2,5} against the triple loop
+    a = np.arange(6, dtype=np.float32)
+    b = np.arange(10, dtype=np.float32) - 4
+    want = np.array([[sum((i + 3 * l) * (l + 2 * j - 4) for l in range(2)) for j in range(5)]
+                     for i in range(3)], np.float32)
+    np.testing.assert_array_equal(_gemm(gpu, a, b, 3, 5, 2).reshape(5, 3).T, want)
+
+
+BIG = [(4096, 4096, 4096), (4096, 256, 9216), (4096, 256, 4096), (1000, 256, 4096),
+       (9216, 256, 4096), (4096, 9216, 256)]
+
+
+@pytest.mark.parametrize("m,n,k", BIG)
+def test_sgemm_config_shapes_sampled_fp64(gpu, m, n, k):
+    a, b = _rand(m * k, 32), _rand(k * n, 33)
+    say("sgemm big", m, n, k)
+    got = _gemm(gpu, a, b, m, n, k).reshape(n, m)
+    A = a.reshape(k, m)   # A[l, i]
+    B = b.reshape(n, k)   # B[j, l]
+    rng = np.random.default_rng(34)
+    rows = rng.integers(0, m, 48)
+    cols = rng.integers(0, n, 48)
+    want = (B[cols].astype(np.float64) @ A[:, rows].astype(np.float64))  # [cols, rows]
+    sub = got[np.ix_(cols, rows)]
+    assert normwise(sub, want) <= TOL
+    # the corners and edges of the tile grid are where indexing slips show
+    for (i, j) in ((0, 0), (m - 1, 0), (0, n - 1), (m - 1, n - 1)):
+        w = float(B[j].astype(np.float64) @ A[:, i].astype(np.float64))
+        assert abs(got[j, i] - w) <= TOL * np.sqrt(k) * 4
+
+
+def test_sgemm_permutation_is_exact(gpu):
+    # B = permutation matrix: C = A with permuted columns, exactly (x*1 + 0s)
+    m, k = 1024, 1024
+    a = _rand(m * k, 35)
+    perm = np.random.default_rng(36).permutation(k)
+    B = np.zeros((k, k), np.float32)      # B[j, l] (numpy view of column-major {k,n})
+    B[np.arange(k), perm] = 1.0           # column j picks row perm[j]
+    got = _gemm(gpu, a, B.ravel(), m, k, k).reshape(k, m)
+    assert_bits_equal(got, a.reshape(k, m)[perm], "A * P")
+
+
+def test_sgemm_linearity_full_size(gpu):
+    m = n = k = 2048
+    a, b1, b2 = _rand(m * k, 37), _rand(k * n, 38), _rand(k * n, 39)
+    c1 = _gemm(gpu, a, b1, m, n, k)
+    c2 = _gemm(gpu, a, b2, m, n, k)
+    c12 = _gemm(gpu, a, b1 + b2, m, n, k)
+    assert normwise(c12, c1.astype(np.float64) + c2) <= TOL
