@@ -1,0 +1,98 @@
+/*
+ * mnv_host.h - C entry points of the C++ host layer (libmnv_host.so).
+ *
+ * The host layer is the C++ mirror of Minerva's operator and device interface
+ * (namespace minerva: Scale, DataShard, closures, Context, hip::<Op> functions with
+ * the parameter lists of minerva/op/impl/cuda.h:10-48, FnBundle dispatch, HipDevice
+ * with a pooled allocator and four streams, and a sequential graph runner).  C++
+ * callers include minerva_amd/host/*.h directly.  These few C functions exist so that
+ * tests, the benchmark and foreign-language bindings can drive that C++ layer without
+ * a C++ compiler: they create a runtime (device + runner), run one operator through
+ * the full Task -> HipDevice -> FnBundle -> hip::<Op> -> C ABI path on host tensors,
+ * and run the training graphs of the benchmark configurations.
+ *
+ * Every function returns 0 on success and -1 on failure; mnvh_last_error() then
+ * describes the failed check (the reference aborts the process instead).
+ */
+#ifndef MNV_HOST_H_
+#define MNV_HOST_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MNVH_MAX_DIMS 8
+
+/* A host tensor: column-major data, extent dims[0..ndims-1], dimension 0 fastest. */
+typedef struct {
+  const float* data;
+  int ndims;
+  int dims[MNVH_MAX_DIMS];
+} mnvh_tensor;
+
+const char* mnvh_last_error(void);
+
+/* sync_each_op != 0: synchronise the stream after every operator, as the reference
+ * device does (minerva/device/device.cpp:221); 0: operators stay in flight and the
+ * caller synchronises with mnvh_runtime_sync. */
+int mnvh_runtime_create(int gpu_id, int sync_each_op, void** runtime);
+int mnvh_runtime_destroy(void* runtime);
+int mnvh_runtime_sync(void* runtime);
+int mnvh_runtime_ops_issued(void* runtime, unsigned long long* count);
+int mnvh_runtime_pool_stats(void* runtime, size_t* total_bytes, size_t* cached_blocks);
+
+/*
+ * Runs one operator on host tensors through the whole host stack.  `op` and
+ * `params` (all passed as doubles):
+ *   "arithmetic" [type]                 "arithmetic_const" [type, val, side]
+ *   "elewise" [type]                    "norm_arithmetic" [type]        (vector = input 1)
+ *   "matmult"  "trans"                  "reshape" [d0, d1, ...]
+ *   "reduction" [type, dim]             "maxindex" [dim]
+ *   "sigmoid_forward" "relu_forward" "tanh_forward"
+ *   "sigmoid_backward" "relu_backward" "tanh_backward"      inputs: diff, top, bottom
+ *   "activation_forward" [alg]          "activation_backward" [alg]
+ *   "softmax_forward" [alg]             "softmax_backward" [alg]        inputs: diff, top
+ *   "conv_forward" [ph, pw, sv, sh]             inputs: bottom, filter, bias
+ *   "conv_backward_data" [ph, pw, sv, sh]       inputs: diff, bottom, filter
+ *   "conv_backward_filter" [ph, pw, sv, sh]     inputs: diff, bottom, filter
+ *   "conv_backward_bias"                        inputs: diff
+ *   "pooling_forward" [alg, h, w, sv, sh, ph, pw]      inputs: bottom
+ *   "pooling_backward" [alg, h, w, sv, sh, ph, pw]     inputs: diff, top, bottom
+ *   "fill" [val, d0, d1, ...]
+ * Enum values follow minerva/op/closure.h:8-24 and narray/convolution_info.h:19-57
+ * (arithmetic 0 add 1 sub 2 mult 3 div; elewise 0 exp 1 ln 2 negative; reduction 0 sum
+ * 1 max; softmax 0 instance 1 channel; activation 0 sigmoid 1 relu 2 tanh; pooling 0 max
+ * 1 average).  The result is written to `out` (capacity out_capacity floats) and its
+ * extent to out_ndims / out_dims.
+ */
+int mnvh_op(void* runtime, const char* op, const mnvh_tensor* inputs, int n_inputs,
+            const double* params, int n_params, float* out, size_t out_capacity,
+            int* out_ndims, int* out_dims);
+
+/* Runs `count` independent element-wise additions through the device's thread pool
+ * (four workers, four streams) and returns the results; exercises PushTask with
+ * non-light tasks and the completion listener. */
+int mnvh_concurrent_adds(void* runtime, const float* a, const float* b, size_t n, int count,
+                         float* out /* count * n floats */);
+
+/* Training graphs.  kind: "mlp" (784-256-10), "cnn" (MNIST CNN; variant 0 = conv2 pad 0
+ * + 2x2/2 pooling, 1 = the reference app's pad 2 + 3x3/3), "alexnet". */
+int mnvh_net_create(void* runtime, const char* kind, int batch, int variant, void** net);
+int mnvh_net_destroy(void* net);
+int mnvh_net_num_params(void* net, int* count);
+int mnvh_net_param_info(void* net, int index, char* name_out /* >= 16 bytes */, size_t* floats);
+int mnvh_net_set_param(void* net, const char* name, const float* host, size_t floats);
+/* name: a parameter ("w0"...), "prob", or "g_<param>" (gradient of the last step) */
+int mnvh_net_read(void* net, const char* name, float* host_out, size_t floats);
+/* Uploads one batch; it stays resident in HBM for the following steps. */
+int mnvh_net_load_batch(void* net, const float* data, size_t data_floats, const float* label,
+                        size_t label_floats);
+/* One forward + backward + SGD step on the resident batch. */
+int mnvh_net_step(void* net, float lr);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MNV_HOST_H_ */

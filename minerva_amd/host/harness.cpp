@@ -1,0 +1,315 @@
+// C entry points of the host layer (include/mnv_host.h).
+#include <cstring>
+#include <string>
+
+#include "mnv_host.h"
+#include "nets.h"
+
+using namespace minerva;
+
+namespace {
+
+thread_local std::string g_error;
+
+struct NetHandle {
+  Runner* rt;
+  std::unique_ptr<Net> net;
+  Tensor data, label;
+};
+
+template <class F> int Guard(F&& f) {
+  try {
+    f();
+    return 0;
+  } catch (const std::exception& e) {
+    g_error = e.what();
+  } catch (...) {
+    g_error = "unknown exception";
+  }
+  return -1;
+}
+
+Scale ToScale(const mnvh_tensor& t) {
+  MNV_CHECK(t.ndims >= 1 && t.ndims <= MNVH_MAX_DIMS) << "bad tensor rank";
+  return Scale(std::vector<int>(t.dims, t.dims + t.ndims));
+}
+
+int P(const double* p, int n, int i) {
+  MNV_CHECK(i < n) << "missing operator parameter " << i;
+  return static_cast<int>(p[i]);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* mnvh_last_error(void) { return g_error.c_str(); }
+
+int mnvh_runtime_create(int gpu_id, int sync_each_op, void** runtime) {
+  return Guard([&] {
+    MNV_CHECK(runtime) << "null out pointer";
+    *runtime = new Runner(gpu_id, sync_each_op != 0);
+  });
+}
+
+int mnvh_runtime_destroy(void* runtime) {
+  return Guard([&] { delete static_cast<Runner*>(runtime); });
+}
+
+int mnvh_runtime_sync(void* runtime) {
+  return Guard([&] { static_cast<Runner*>(runtime)->Sync(); });
+}
+
+int mnvh_runtime_ops_issued(void* runtime, unsigned long long* count) {
+  return Guard([&] { *count = static_cast<Runner*>(runtime)->ops_issued(); });
+}
+
+int mnvh_runtime_pool_stats(void* runtime, size_t* total_bytes, size_t* cached_blocks) {
+  return Guard([&] {
+    auto& ds = static_cast<Runner*>(runtime)->device().data_store();
+    if (total_bytes) *total_bytes = ds.GetTotalBytes();
+    if (cached_blocks) *cached_blocks = ds.NumCachedBlocks();
+  });
+}
+
+int mnvh_op(void* runtime, const char* op_name, const mnvh_tensor* inputs, int n_inputs,
+            const double* params, int n_params, float* out, size_t out_capacity,
+            int* out_ndims, int* out_dims) {
+  return Guard([&] {
+    Runner* rt = static_cast<Runner*>(runtime);
+    MNV_CHECK(rt && op_name && out) << "null argument";
+    std::string op(op_name);
+    std::vector<Tensor> in;
+    for (int i = 0; i < n_inputs; ++i) {
+      MNV_CHECK(inputs[i].data) << "null input data";
+      in.push_back(rt->MakeNArray(ToScale(inputs[i]), inputs[i].data));
+    }
+    auto need = [&](int n) { MNV_CHECK_EQ(n_inputs, n) << op << " takes " << n << " inputs"; };
+    auto conv_info = [&] {
+      return ConvInfo(P(params, n_params, 0), P(params, n_params, 1), P(params, n_params, 2),
+                      P(params, n_params, 3));
+    };
+    auto pool_info = [&] {
+      return PoolingInfo(static_cast<PoolingInfo::Algorithm>(P(params, n_params, 0)),
+                         P(params, n_params, 1), P(params, n_params, 2), P(params, n_params, 3),
+                         P(params, n_params, 4), P(params, n_params, 5), P(params, n_params, 6));
+    };
+    Tensor r;
+    if (op == "arithmetic") {
+      need(2);
+      r = rt->Arithmetic(in[0], in[1], static_cast<ArithmeticType>(P(params, n_params, 0)));
+    } else if (op == "arithmetic_const") {
+      need(1);
+      MNV_CHECK(n_params >= 3) << "arithmetic_const takes type, val, side";
+      r = rt->ArithmeticConst(in[0], static_cast<float>(params[1]),
+                              static_cast<ArithmeticType>(P(params, n_params, 0)),
+                              P(params, n_params, 2));
+    } else if (op == "elewise") {
+      need(1);
+      r = rt->Elewise(in[0], static_cast<ElewiseType>(P(params, n_params, 0)));
+    } else if (op == "norm_arithmetic") {
+      need(2);
+      r = rt->NormArithmetic(in[0], in[1], static_cast<ArithmeticType>(P(params, n_params, 0)));
+    } else if (op == "matmult") {
+      need(2);
+      r = rt->MatMult(in[0], in[1]);
+    } else if (op == "trans") {
+      need(1);
+      r = rt->Trans(in[0]);
+    } else if (op == "reshape") {
+      need(1);
+      std::vector<int> d;
+      for (int i = 0; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
+      r = rt->Reshape(in[0], Scale(d));
+    } else if (op == "reduction") {
+      need(1);
+      r = rt->Reduce(in[0], P(params, n_params, 1),
+                     static_cast<ReductionType>(P(params, n_params, 0)));
+    } else if (op == "maxindex") {
+      need(1);
+      r = rt->MaxIndex(in[0], P(params, n_params, 0));
+    } else if (op == "sigmoid_forward") {
+      need(1);
+      r = rt->SigmoidForward(in[0]);
+    } else if (op == "relu_forward") {
+      need(1);
+      r = rt->ReluForward(in[0]);
+    } else if (op == "tanh_forward") {
+      need(1);
+      r = rt->TanhForward(in[0]);
+    } else if (op == "sigmoid_backward") {
+      need(3);
+      r = rt->SigmoidBackward(in[0], in[1], in[2]);
+    } else if (op == "relu_backward") {
+      need(3);
+      r = rt->ReluBackward(in[0], in[1], in[2]);
+    } else if (op == "tanh_backward") {
+      need(3);
+      r = rt->TanhBackward(in[0], in[1], in[2]);
+    } else if (op == "activation_forward") {
+      need(1);
+      r = rt->ActivationForward(in[0], static_cast<ActivationAlgorithm>(P(params, n_params, 0)));
+    } else if (op == "activation_backward") {
+      need(3);
+      r = rt->ActivationBackward(in[0], in[1], in[2],
+                                 static_cast<ActivationAlgorithm>(P(params, n_params, 0)));
+    } else if (op == "softmax_forward") {
+      need(1);
+      r = rt->SoftmaxForward(in[0], static_cast<SoftmaxAlgorithm>(P(params, n_params, 0)));
+    } else if (op == "softmax_backward") {
+      need(2);
+      r = rt->SoftmaxBackward(in[0], in[1], static_cast<SoftmaxAlgorithm>(P(params, n_params, 0)));
+    } else if (op == "conv_forward") {
+      need(3);
+      r = rt->ConvForward(in[0], in[1], in[2], conv_info());
+    } else if (op == "conv_backward_data") {
+      need(3);
+      r = rt->ConvBackwardData(in[0], in[1], in[2], conv_info());
+    } else if (op == "conv_backward_filter") {
+      need(3);
+      r = rt->ConvBackwardFilter(in[0], in[1], in[2], conv_info());
+    } else if (op == "conv_backward_bias") {
+      need(1);
+      r = rt->ConvBackwardBias(in[0]);
+    } else if (op == "pooling_forward") {
+      need(1);
+      r = rt->PoolingForward(in[0], pool_info());
+    } else if (op == "pooling_backward") {
+      need(3);
+      r = rt->PoolingBackward(in[0], in[1], in[2], pool_info());
+    } else if (op == "fill") {
+      need(0);
+      std::vector<int> d;
+      for (int i = 1; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
+      MNV_CHECK(n_params >= 2) << "fill takes val, d0, ...";
+      r = rt->Constant(Scale(d), static_cast<float>(params[0]));
+    } else {
+      MNV_FATAL() << "unknown operator '" << op << "'";
+    }
+    size_t n = r->size.Prod();
+    MNV_CHECK(n <= out_capacity) << "output needs " << n << " floats, capacity " << out_capacity;
+    std::vector<float> host = rt->Get(r);
+    std::memcpy(out, host.data(), n * sizeof(float));
+    if (out_ndims) *out_ndims = static_cast<int>(r->size.NumDims());
+    if (out_dims)
+      for (size_t i = 0; i < r->size.NumDims(); ++i) out_dims[i] = r->size[i];
+  });
+}
+
+int mnvh_concurrent_adds(void* runtime, const float* a, const float* b, size_t n, int count,
+                         float* out) {
+  return Guard([&] {
+    Runner* rt = static_cast<Runner*>(runtime);
+    HipDevice& dev = rt->device();
+    Scale size{static_cast<int>(n)};
+    Tensor ta = rt->MakeNArray(size, a), tb = rt->MakeNArray(size, b);
+    // tasks and their output ids live until every worker is done
+    std::vector<Task> tasks(count);
+    const uint64_t base_id = (1ull << 40);
+    for (int i = 0; i < count; ++i) {
+      auto op = std::make_shared<ArithmeticOp>();
+      op->closure.type = ArithmeticType::kAdd;
+      Task& t = tasks[i];
+      t.inputs.emplace_back(PhysicalData(size, dev.device_id(), ta->id), ta->id);
+      t.inputs.emplace_back(PhysicalData(size, dev.device_id(), tb->id), tb->id);
+      t.outputs.emplace_back(PhysicalData(size, dev.device_id(), base_id + i), base_id + i);
+      t.op.compute_fn = op;
+      t.id = i;
+      t.light = false;
+    }
+    for (int i = 0; i < count; ++i) dev.PushTask(&tasks[i]);
+    dev.WaitForAllFinished();
+    std::string err = dev.TakeAsyncError();
+    for (int i = 0; i < count; ++i) {
+      if (err.empty()) dev.CopyToHost(out + (size_t)i * n, base_id + i, n);
+      dev.FreeDataIfExist(base_id + i);
+    }
+    MNV_CHECK(err.empty()) << err;
+  });
+}
+
+int mnvh_net_create(void* runtime, const char* kind, int batch, int variant, void** net) {
+  return Guard([&] {
+    Runner* rt = static_cast<Runner*>(runtime);
+    MNV_CHECK(rt && kind && net && batch > 0) << "bad argument";
+    std::unique_ptr<NetHandle> h(new NetHandle);
+    h->rt = rt;
+    std::string k(kind);
+    if (k == "mlp") h->net.reset(new MlpNet(rt, batch));
+    else if (k == "cnn") h->net.reset(variant == 1 ? new CnnNet(rt, batch, 2, 3) : new CnnNet(rt, batch));
+    else if (k == "alexnet") h->net.reset(new AlexNet(rt, batch));
+    else MNV_FATAL() << "unknown net '" << k << "'";
+    *net = h.release();
+  });
+}
+
+int mnvh_net_destroy(void* net) {
+  return Guard([&] { delete static_cast<NetHandle*>(net); });
+}
+
+int mnvh_net_num_params(void* net, int* count) {
+  return Guard([&] { *count = static_cast<int>(static_cast<NetHandle*>(net)->net->param_names.size()); });
+}
+
+int mnvh_net_param_info(void* net, int index, char* name_out, size_t* floats) {
+  return Guard([&] {
+    Net& n = *static_cast<NetHandle*>(net)->net;
+    MNV_CHECK(index >= 0 && index < static_cast<int>(n.param_names.size())) << "bad index";
+    const std::string& name = n.param_names[index];
+    if (name_out) {
+      std::strncpy(name_out, name.c_str(), 15);
+      name_out[15] = 0;
+    }
+    if (floats) *floats = n.params[name]->size.Prod();
+  });
+}
+
+int mnvh_net_set_param(void* net, const char* name, const float* host, size_t floats) {
+  return Guard([&] {
+    NetHandle* h = static_cast<NetHandle*>(net);
+    auto it = h->net->params.find(name);
+    MNV_CHECK(it != h->net->params.end()) << "no parameter '" << name << "'";
+    Scale size = it->second->size;
+    MNV_CHECK_EQ(static_cast<size_t>(size.Prod()), floats) << "size of '" << name << "'";
+    it->second = h->rt->MakeNArray(size, host);
+  });
+}
+
+int mnvh_net_read(void* net, const char* name, float* host_out, size_t floats) {
+  return Guard([&] {
+    NetHandle* h = static_cast<NetHandle*>(net);
+    Tensor t;
+    auto it = h->net->params.find(name);
+    if (it != h->net->params.end()) t = it->second;
+    else {
+      auto jt = h->net->results.find(name);
+      MNV_CHECK(jt != h->net->results.end()) << "no tensor '" << name << "'";
+      t = jt->second;
+    }
+    MNV_CHECK_EQ(static_cast<size_t>(t->size.Prod()), floats) << "size of '" << name << "'";
+    std::vector<float> v = h->rt->Get(t);
+    std::memcpy(host_out, v.data(), floats * sizeof(float));
+  });
+}
+
+int mnvh_net_load_batch(void* net, const float* data, size_t data_floats, const float* label,
+                        size_t label_floats) {
+  return Guard([&] {
+    NetHandle* h = static_cast<NetHandle*>(net);
+    Scale ds = h->net->DataSize(), ls = h->net->LabelSize();
+    MNV_CHECK_EQ(static_cast<size_t>(ds.Prod()), data_floats) << "data size";
+    MNV_CHECK_EQ(static_cast<size_t>(ls.Prod()), label_floats) << "label size";
+    h->data = h->rt->MakeNArray(ds, data);
+    h->label = h->rt->MakeNArray(ls, label);
+  });
+}
+
+int mnvh_net_step(void* net, float lr) {
+  return Guard([&] {
+    NetHandle* h = static_cast<NetHandle*>(net);
+    MNV_CHECK(h->data && h->label) << "load a batch first";
+    h->net->Step(h->data, h->label, lr);
+  });
+}
+
+}  // extern "C"

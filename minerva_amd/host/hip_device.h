@@ -1,0 +1,148 @@
+// The HIP device: the replacement for the reference's GpuDevice
+// (minerva/device/device.h:18-78, device.cpp:129-222) and its allocator
+// (minerva/device/pooled_data_store.cpp:19-65), with the same public surface the
+// engine calls: PushTask / GetPtr / FreeDataIfExist and DeviceListener::OnOperationComplete.
+//
+//  - kParallelism (4) worker threads, each with its own HIP stream and its own
+//    grow-only scratch arena; a task runs on worker `thrid` and is synchronised before
+//    completion is reported, as the reference does after every operator.
+//  - PooledDataStore: exact-size free lists over mnv_malloc / mnv_free; when the bytes
+//    held exceed the threshold every cached block is released.
+#pragma once
+#include <array>
+#include <condition_variable>
+#include <deque>
+#include <functional>
+#include <map>
+#include <mutex>
+#include <queue>
+#include <thread>
+#include <unordered_map>
+#include <unordered_set>
+
+#include "op_dispatch.h"
+
+namespace minerva {
+
+struct PhysicalData {
+  PhysicalData(const Scale& s, uint64_t d, uint64_t id) : size(s), device_id(d), data_id(id) {}
+  Scale size;
+  uint64_t device_id;
+  uint64_t data_id;
+};
+
+struct PhysicalOp {
+  std::shared_ptr<ComputeFn> compute_fn;
+  uint64_t device_id = 0;
+};
+
+struct TaskData {
+  TaskData(const PhysicalData& p, uint64_t i) : physical_data(p), id(i) {}
+  PhysicalData physical_data;
+  uint64_t id;
+};
+
+struct Task {
+  std::vector<TaskData> inputs;
+  std::vector<TaskData> outputs;
+  PhysicalOp op;
+  uint64_t id = 0;
+  bool light = false;  // run on the caller's thread (stream 0) instead of the pool
+};
+
+class DeviceListener {
+ public:
+  virtual ~DeviceListener() = default;
+  virtual void OnOperationComplete(Task*) = 0;
+};
+
+class PooledDataStore {
+ public:
+  PooledDataStore(size_t threshold, std::function<void*(size_t)> a, std::function<void(void*)> d);
+  ~PooledDataStore();
+  PooledDataStore(const PooledDataStore&) = delete;
+  PooledDataStore& operator=(const PooledDataStore&) = delete;
+  float* CreateData(uint64_t id, size_t length);
+  float* GetData(uint64_t id);
+  bool ExistData(uint64_t id) const;
+  void FreeData(uint64_t id);
+  size_t GetTotalBytes() const;
+  size_t NumCachedBlocks() const;
+
+ private:
+  void ReleaseFreeSpace();
+  struct DataState {
+    void* ptr;
+    size_t length;
+  };
+  mutable std::mutex access_mutex_;
+  std::unordered_map<uint64_t, DataState> data_states_;
+  std::unordered_map<size_t, std::queue<void*>> free_space_;
+  std::function<void*(size_t)> allocator_;
+  std::function<void(void*)> deallocator_;
+  size_t threshold_;
+  size_t total_ = 0;
+};
+
+class HipDevice {
+ public:
+  enum class MemType { kCpu, kGpu };
+  static constexpr size_t kParallelism = 4;
+  // 288 GB of HBM: keep up to 200 GiB in the pool before dropping cached blocks.
+  static constexpr size_t kDefaultPoolBytes = (size_t)200 << 30;
+
+  HipDevice(uint64_t device_id, DeviceListener* listener, int gpu_id,
+            size_t pool_bytes = kDefaultPoolBytes);
+  ~HipDevice();
+  HipDevice(const HipDevice&) = delete;
+  HipDevice& operator=(const HipDevice&) = delete;
+
+  void PushTask(Task* task);
+  std::pair<MemType, float*> GetPtr(uint64_t data_id);
+  void FreeDataIfExist(uint64_t data_id);
+  std::string GetMemUsage() const;
+  std::string Name() const;
+  MemType GetMemType() const { return MemType::kGpu; }
+  void WaitForAllFinished();
+
+  // When false, operators are left in flight on their stream and the caller decides
+  // when to synchronise (Barrier); the reference always synchronises per operator.
+  void set_sync_each_op(bool v) { sync_each_op_ = v; }
+  void Barrier(int thrid);
+  void* stream(int thrid) const { return streams_[thrid]; }
+  uint64_t device_id() const { return device_id_; }
+  PooledDataStore& data_store() { return *data_store_; }
+  // Host <-> device copies on worker stream 0, synchronised.
+  void CopyToHost(float* dst, uint64_t data_id, size_t floats);
+  // First error raised by an operator on a pool thread (empty if none).
+  std::string TakeAsyncError();
+
+ private:
+  void Execute(Task* task, int thrid);
+  void DoExecute(const DataList& in, const DataList& out, PhysicalOp& op, int thrid);
+  void Activate() const;
+  void EnsureWorkspace(int thrid, size_t bytes);
+  void WorkerLoop(int thrid);
+
+  uint64_t device_id_;
+  DeviceListener* listener_;
+  int gpu_id_;
+  bool sync_each_op_ = true;
+  std::array<void*, kParallelism> streams_{};
+  std::array<void*, kParallelism> workspace_{};
+  std::array<size_t, kParallelism> workspace_bytes_{};
+  std::unique_ptr<PooledDataStore> data_store_;
+  std::mutex local_mutex_;
+  std::unordered_set<uint64_t> local_data_;
+  // thread pool
+  std::vector<std::thread> workers_;
+  std::mutex q_mutex_;
+  std::condition_variable q_cv_, idle_cv_;
+  std::deque<Task*> queue_;
+  size_t busy_ = 0;
+  bool stop_ = false;
+  std::mutex err_mutex_;
+  std::string async_error_;
+};
+
+}  // namespace minerva

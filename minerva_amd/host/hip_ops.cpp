@@ -1,0 +1,378 @@
+#include "hip_ops.h"
+
+#include "mnv_hip.h"
+
+namespace minerva {
+namespace hip {
+
+namespace {
+
+void Ok(int status, const char* what) {
+  MNV_CHECK(status == MNV_OK) << what << ": " << mnv_error_string(status);
+}
+
+// Collapses an N-d extent around one dimension into the {m, n} matrix the library
+// reduces or broadcasts over.  Dimension 0 is the contiguous one ("col" kernels);
+// the last dimension is the strided one ("row" kernels).  The reference's GPU path
+// only accepts 2-D (minerva/op/impl/cuda.cpp:222-223,268-269); higher ranks are
+// accepted here when the dimension is the first or the last, and rejected otherwise.
+struct Collapsed {
+  bool on_first;
+  int m, n;
+};
+
+Collapsed Collapse(const Scale& size, int dim, const char* what) {
+  const int nd = static_cast<int>(size.NumDims());
+  MNV_CHECK(nd >= 1 && dim >= 0 && dim < nd) << what << ": dimension out of range";
+  long long total = size.Prod();
+  Collapsed c;
+  if (dim == 0) {
+    c.on_first = true;
+    c.m = size[0];
+    c.n = static_cast<int>(total / size[0]);
+  } else {
+    MNV_CHECK(dim == nd - 1) << what << ": only the first or the last dimension is supported";
+    c.on_first = false;
+    c.n = size[nd - 1];
+    c.m = static_cast<int>(total / size[nd - 1]);
+  }
+  return c;
+}
+
+}  // namespace
+
+void Arithmetic(const DataList& inputs, const DataList& outputs, ArithmeticClosure& closure,
+                const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 2u) << "Arithmetic takes 2 inputs";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "Arithmetic takes 1 output";
+  const float* l = inputs[0].data_;
+  const float* r = inputs[1].data_;
+  float* o = outputs[0].data_;
+  size_t n = outputs[0].size_.Prod();
+  switch (closure.type) {
+    case ArithmeticType::kAdd: Ok(mnv_add(l, r, o, n, ctx.stream), "add"); break;
+    case ArithmeticType::kSub: Ok(mnv_sub(l, r, o, n, ctx.stream), "sub"); break;
+    case ArithmeticType::kMult: Ok(mnv_mul(l, r, o, n, ctx.stream), "mul"); break;
+    case ArithmeticType::kDiv: Ok(mnv_div(l, r, o, n, ctx.stream), "div"); break;
+  }
+}
+
+void ArithmeticConst(const DataList& inputs, const DataList& outputs,
+                     ArithmeticConstClosure& closure, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "(arithmetic const) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(arithmetic const) #outputs is wrong!";
+  const float* x = inputs[0].data_;
+  float* y = outputs[0].data_;
+  const float v = closure.val;
+  size_t n = inputs[0].size_.Prod();
+  const bool left = closure.side == 0;
+  switch (closure.type) {
+    case ArithmeticType::kAdd: Ok(mnv_const_add(x, y, v, n, ctx.stream), "const add"); break;
+    case ArithmeticType::kSub:
+      Ok(left ? mnv_const_rsub(x, y, v, n, ctx.stream) : mnv_const_sub(x, y, v, n, ctx.stream),
+         "const sub");
+      break;
+    case ArithmeticType::kMult: Ok(mnv_const_mul(x, y, v, n, ctx.stream), "const mul"); break;
+    case ArithmeticType::kDiv:
+      // x / v is a true division here, as on the CPU (basic.cpp:99-103); the CUDA path
+      // multiplies by 1/v instead (cuda.cpp:196), which is not the same rounding.
+      Ok(left ? mnv_const_rdiv(x, y, v, n, ctx.stream) : mnv_const_div(x, y, v, n, ctx.stream),
+         "const div");
+      break;
+  }
+}
+
+void Elewise(const DataList& inputs, const DataList& outputs, ElewiseClosure& closure,
+             const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "(elewise) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(elewise) #outputs is wrong!";
+  const float* x = inputs[0].data_;
+  float* y = outputs[0].data_;
+  size_t n = outputs[0].size_.Prod();
+  switch (closure.type) {
+    case ElewiseType::kExp: Ok(mnv_exp(x, y, n, ctx.stream), "exp"); break;
+    case ElewiseType::kLn: Ok(mnv_ln(x, y, n, ctx.stream), "ln"); break;
+    case ElewiseType::kNegative: Ok(mnv_neg(x, y, n, ctx.stream), "neg"); break;
+    default: MNV_FATAL() << "elewise algorithm not supported";
+  }
+}
+
+void MatMult(const DataList& inputs, const DataList& outputs, MatMultClosure&,
+             const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 2u) << "(matmult) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(matmult) #outputs is wrong!";
+  int m = inputs[0].size_[0];
+  int k = inputs[0].size_[1];
+  int n = outputs[0].size_[1];
+  MNV_CHECK_EQ(inputs[1].size_[0], k) << "(matmult) inner dimensions differ";
+  Ok(mnv_sgemm_nn(inputs[0].data_, inputs[1].data_, outputs[0].data_, m, n, k, ctx.workspace,
+                  ctx.workspace_bytes, ctx.stream),
+     "sgemm");
+}
+
+void Transpose(const DataList& inputs, const DataList& outputs, TransposeClosure&,
+               const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "(transpose) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(transpose) #outputs is wrong!";
+  int m = inputs[0].size_[0];
+  int n = inputs[0].size_[1];
+  Ok(mnv_transpose(inputs[0].data_, outputs[0].data_, m, n, ctx.stream), "transpose");
+}
+
+void NormArithmetic(const DataList& inputs, const DataList& outputs,
+                    NormArithmeticClosure& closure, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 2u) << "NormArithmetic kernel wrong #input";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "NormArithmetic kernel wrong #output";
+  MNV_CHECK_EQ(closure.dims_to_replicate.NumDims(), 1u)
+      << "currently do norm on one dimension only";
+  Collapsed c = Collapse(inputs[0].size_, closure.dims_to_replicate[0], "NormArithmetic");
+  const float* mat = inputs[0].data_;
+  const float* vec = inputs[1].data_;
+  float* res = outputs[0].data_;
+  int (*fn)(const float*, const float*, float*, int, int, mnv_stream_t) = nullptr;
+  // replicated along dim 0 => the vector has one entry per column ("OnCol")
+  switch (closure.type) {
+    case ArithmeticType::kAdd: fn = c.on_first ? mnv_norm_add_col : mnv_norm_add_row; break;
+    case ArithmeticType::kSub: fn = c.on_first ? mnv_norm_sub_col : mnv_norm_sub_row; break;
+    case ArithmeticType::kMult: fn = c.on_first ? mnv_norm_mul_col : mnv_norm_mul_row; break;
+    case ArithmeticType::kDiv: fn = c.on_first ? mnv_norm_div_col : mnv_norm_div_row; break;
+  }
+  Ok(fn(mat, vec, res, c.m, c.n, ctx.stream), "norm arithmetic");
+}
+
+void Reduction(const DataList& inputs, const DataList& outputs, ReductionClosure& closure,
+               const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "Reduction kernel wrong #input";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "Reduction kernel wrong #output";
+  MNV_CHECK_EQ(closure.dims_to_reduce.NumDims(), 1u)
+      << "currently do reduction on one dimension only";
+  Collapsed c = Collapse(inputs[0].size_, closure.dims_to_reduce[0], "Reduction");
+  const float* in = inputs[0].data_;
+  float* out = outputs[0].data_;
+  const bool sum = closure.type == ReductionType::kSum;
+  int rc = c.on_first ? (sum ? mnv_reduce_sum_col(in, out, c.m, c.n, ctx.stream)
+                             : mnv_reduce_max_col(in, out, c.m, c.n, ctx.stream))
+                      : (sum ? mnv_reduce_sum_row(in, out, c.m, c.n, ctx.stream)
+                             : mnv_reduce_max_row(in, out, c.m, c.n, ctx.stream));
+  Ok(rc, "reduction");
+}
+
+void MaxIndex(const DataList& inputs, const DataList& outputs, MaxIndexClosure& closure,
+              const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "MaxIndex kernel wrong #input";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "MaxIndex kernel wrong #output";
+  Collapsed c = Collapse(inputs[0].size_, closure.dim, "MaxIndex");
+  int rc = c.on_first
+               ? mnv_maxindex_col(inputs[0].data_, outputs[0].data_, c.m, c.n, ctx.stream)
+               : mnv_maxindex_row(inputs[0].data_, outputs[0].data_, c.m, c.n, ctx.stream);
+  Ok(rc, "maxindex");
+}
+
+void Reshape(const DataList& inputs, const DataList& outputs, ReshapeClosure&,
+             const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u);
+  MNV_CHECK_EQ(outputs.size(), 1u);
+  MNV_CHECK_EQ(inputs[0].size_.Prod(), outputs[0].size_.Prod()) << "reshape changes the size";
+  Ok(mnv_copy(inputs[0].data_, outputs[0].data_, inputs[0].size_.Prod(), ctx.stream), "reshape");
+}
+
+#define MNV_ACT_FWD(Name, fn)                                                             \
+  void Name(const DataList& inputs, const DataList& outputs, Name##Closure&,              \
+            const Context& ctx) {                                                         \
+    MNV_CHECK_EQ(inputs.size(), 1u) << #Name " #inputs wrong";                            \
+    MNV_CHECK_EQ(outputs.size(), 1u) << #Name " #outputs wrong";                          \
+    Ok(fn(inputs[0].data_, outputs[0].data_, inputs[0].size_.Prod(), ctx.stream), #Name); \
+  }
+MNV_ACT_FWD(SigmoidForward, mnv_sigmoid_fwd)
+MNV_ACT_FWD(ReluForward, mnv_relu_fwd)
+MNV_ACT_FWD(TanhForward, mnv_tanh_fwd)
+
+// inputs: [top_diff, top, bottom] (cuda.cpp:348-392)
+#define MNV_ACT_BWD(Name, fn)                                                              \
+  void Name(const DataList& inputs, const DataList& outputs, Name##Closure&,               \
+            const Context& ctx) {                                                          \
+    MNV_CHECK_EQ(inputs.size(), 3u) << #Name " #inputs wrong";                             \
+    MNV_CHECK_EQ(outputs.size(), 1u) << #Name " #outputs wrong";                           \
+    Ok(fn(inputs[2].data_, inputs[1].data_, inputs[0].data_, outputs[0].data_,             \
+          inputs[0].size_.Prod(), ctx.stream),                                             \
+       #Name);                                                                             \
+  }
+MNV_ACT_BWD(SigmoidBackward, mnv_sigmoid_bwd)
+MNV_ACT_BWD(ReluBackward, mnv_relu_bwd)
+MNV_ACT_BWD(TanhBackward, mnv_tanh_bwd)
+
+void ActivationForward(const DataList& inputs, const DataList& outputs,
+                       ActivationForwardClosure& closure, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "(activation forward) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(activation forward) #outputs wrong";
+  const float* b = inputs[0].data_;
+  float* t = outputs[0].data_;
+  size_t n = inputs[0].size_.Prod();
+  switch (closure.algorithm) {
+    case ActivationAlgorithm::kSigmoid: Ok(mnv_sigmoid_fwd(b, t, n, ctx.stream), "sigmoid"); break;
+    case ActivationAlgorithm::kRelu: Ok(mnv_relu_fwd(b, t, n, ctx.stream), "relu"); break;
+    case ActivationAlgorithm::kTanh: Ok(mnv_tanh_fwd(b, t, n, ctx.stream), "tanh"); break;
+    default: MNV_FATAL() << "activation algorithm not supported";
+  }
+}
+
+void ActivationBackward(const DataList& inputs, const DataList& outputs,
+                        ActivationBackwardClosure& closure, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 3u) << "(activation backward) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(activation backward) #outputs wrong";
+  const float* td = inputs[0].data_;
+  const float* top = inputs[1].data_;
+  const float* bot = inputs[2].data_;
+  float* bd = outputs[0].data_;
+  size_t n = inputs[0].size_.Prod();
+  switch (closure.algorithm) {
+    case ActivationAlgorithm::kSigmoid:
+      Ok(mnv_sigmoid_bwd(bot, top, td, bd, n, ctx.stream), "sigmoid bwd");
+      break;
+    case ActivationAlgorithm::kRelu: Ok(mnv_relu_bwd(bot, top, td, bd, n, ctx.stream), "relu bwd"); break;
+    case ActivationAlgorithm::kTanh: Ok(mnv_tanh_bwd(bot, top, td, bd, n, ctx.stream), "tanh bwd"); break;
+    default: MNV_FATAL() << "activation algorithm not supported";
+  }
+}
+
+// Image batches are {W,H,C,N}; filters {S,R,Cin,Cout} (minerva/narray/image_batch.cpp:35-93)
+void ConvForward(const DataList& inputs, const DataList& outputs, ConvForwardClosure& c,
+                 const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 3u) << "(conv forward) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(conv forward) #outputs wrong";
+  auto& bottom = inputs[0];
+  auto& filter = inputs[1];
+  auto& bias = inputs[2];
+  auto& top = outputs[0];
+  MNV_CHECK_EQ(bottom.size_[2], filter.size_[2]) << "#input channels mismatch";
+  Ok(mnv_conv_fwd(bottom.data_, filter.data_, bias.data_, top.data_, bottom.size_[3],
+                  bottom.size_[2], top.size_[2], bottom.size_[1], bottom.size_[0], c.pad_height,
+                  c.pad_width, c.stride_vertical, c.stride_horizontal, filter.size_[1],
+                  filter.size_[0], ctx.stream),
+     "conv forward");
+}
+
+void ConvBackwardData(const DataList& inputs, const DataList& outputs,
+                      ConvBackwardDataClosure& c, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 2u) << "(conv backward data) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(conv backward data) #outputs wrong";
+  auto& top_diff = inputs[0];
+  auto& filter = inputs[1];
+  auto& bottom_diff = outputs[0];
+  // The extent of bottom_diff comes from the output shard (the forward bottom's size,
+  // narray/convolution.cpp:47), not from a formula that only holds for exact fits.
+  Ok(mnv_conv_bwd_data(top_diff.data_, filter.data_, bottom_diff.data_, top_diff.size_[3],
+                       bottom_diff.size_[2], top_diff.size_[2], bottom_diff.size_[1],
+                       bottom_diff.size_[0], c.pad_height, c.pad_width, c.stride_vertical,
+                       c.stride_horizontal, filter.size_[1], filter.size_[0], ctx.stream),
+     "conv backward data");
+}
+
+void ConvBackwardFilter(const DataList& inputs, const DataList& outputs,
+                        ConvBackwardFilterClosure& c, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 2u) << "(conv backward filter) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(conv backward filter) #outputs wrong";
+  auto& top_diff = inputs[0];
+  auto& bottom = inputs[1];
+  auto& filter_diff = outputs[0];
+  Ok(mnv_conv_bwd_filter(bottom.data_, top_diff.data_, filter_diff.data_, top_diff.size_[3],
+                         bottom.size_[2], top_diff.size_[2], bottom.size_[1], bottom.size_[0],
+                         c.pad_height, c.pad_width, c.stride_vertical, c.stride_horizontal,
+                         filter_diff.size_[1], filter_diff.size_[0], ctx.workspace,
+                         ctx.workspace_bytes, ctx.stream),
+     "conv backward filter");
+}
+
+void ConvBackwardBias(const DataList& inputs, const DataList& outputs, ConvBackwardBiasClosure&,
+                      const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "(conv backward bias) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(conv backward bias) #outputs wrong";
+  auto& top_diff = inputs[0];
+  Ok(mnv_conv_bwd_bias(top_diff.data_, outputs[0].data_, top_diff.size_[3], top_diff.size_[2],
+                       top_diff.size_[1], top_diff.size_[0], ctx.stream),
+     "conv backward bias");
+}
+
+void SoftmaxForward(const DataList& inputs, const DataList& outputs,
+                    SoftmaxForwardClosure& closure, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "(softmax forward) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(softmax forward) #outputs wrong";
+  auto& b = inputs[0];
+  MNV_CHECK_EQ(b.size_.NumDims(), 4u) << "softmax takes an image batch";
+  switch (closure.algorithm) {
+    case SoftmaxAlgorithm::kInstance:
+      Ok(mnv_softmax_instance_fwd(b.data_, outputs[0].data_, b.size_[3], b.size_[2], b.size_[1],
+                                  b.size_[0], ctx.stream), "softmax instance");
+      break;
+    case SoftmaxAlgorithm::kChannel:
+      Ok(mnv_softmax_channel_fwd(b.data_, outputs[0].data_, b.size_[3], b.size_[2], b.size_[1],
+                                 b.size_[0], ctx.stream), "softmax channel");
+      break;
+    default: MNV_FATAL() << "softmax algorithm not supported";
+  }
+}
+
+void SoftmaxBackward(const DataList& inputs, const DataList& outputs,
+                     SoftmaxBackwardClosure& closure, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 2u) << "(softmax backward) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(softmax backward) #outputs wrong";
+  auto& td = inputs[0];
+  auto& top = inputs[1];
+  MNV_CHECK_EQ(td.size_.NumDims(), 4u) << "softmax takes an image batch";
+  switch (closure.algorithm) {
+    case SoftmaxAlgorithm::kInstance:
+      Ok(mnv_softmax_instance_bwd(td.data_, top.data_, outputs[0].data_, td.size_[3], td.size_[2],
+                                  td.size_[1], td.size_[0], ctx.stream), "softmax instance bwd");
+      break;
+    case SoftmaxAlgorithm::kChannel:
+      Ok(mnv_softmax_channel_bwd(td.data_, top.data_, outputs[0].data_, td.size_[3], td.size_[2],
+                                 td.size_[1], td.size_[0], ctx.stream), "softmax channel bwd");
+      break;
+    default: MNV_FATAL() << "softmax algorithm not supported";
+  }
+}
+
+void PoolingForward(const DataList& inputs, const DataList& outputs, PoolingForwardClosure& c,
+                    const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "(pooling forward) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(pooling forward) #outputs wrong";
+  auto& b = inputs[0];
+  auto fn = c.algorithm == PoolingInfo::Algorithm::kMax ? mnv_maxpool_fwd : mnv_avgpool_fwd;
+  Ok(fn(b.data_, outputs[0].data_, b.size_[3], b.size_[2], b.size_[1], b.size_[0],
+        c.stride_vertical, c.stride_horizontal, c.height, c.width, c.pad_height, c.pad_width,
+        ctx.stream),
+     "pooling forward");
+}
+
+void PoolingBackward(const DataList& inputs, const DataList& outputs, PoolingBackwardClosure& c,
+                     const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 3u) << "(pooling backward) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(pooling backward) #outputs wrong";
+  auto& td = inputs[0];
+  auto& top = inputs[1];
+  auto& b = inputs[2];
+  auto fn = c.algorithm == PoolingInfo::Algorithm::kMax ? mnv_maxpool_bwd : mnv_avgpool_bwd;
+  Ok(fn(b.data_, top.data_, td.data_, outputs[0].data_, td.size_[3], td.size_[2], b.size_[1],
+        b.size_[0], c.stride_vertical, c.stride_horizontal, c.height, c.width, c.pad_height,
+        c.pad_width, ctx.stream),
+     "pooling backward");
+}
+
+void ArrayLoader(const DataList& outputs, ArrayLoaderClosure& closure, const Context& ctx) {
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(array loader) #outputs wrong";
+  MNV_CHECK(closure.data) << "probably already executed";
+  // on the operator's own stream (the reference uses the default stream, cuda.cpp:595)
+  Ok(mnv_memcpy_h2d(outputs[0].data_, closure.data.get(),
+                    outputs[0].size_.Prod() * sizeof(float), ctx.stream), "array loader");
+  // the host buffer must outlive the asynchronous copy
+  Ok(mnv_stream_sync(ctx.stream), "array loader sync");
+  closure.data.reset();
+}
+
+void Fill(const DataList& outputs, FillClosure& closure, const Context& ctx) {
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(fill) #outputs wrong";
+  Ok(mnv_fill(outputs[0].data_, outputs[0].size_.Prod(), closure.val, ctx.stream), "fill");
+}
+
+}  // namespace hip
+}  // namespace minerva

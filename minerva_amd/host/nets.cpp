@@ -1,0 +1,181 @@
+#include "nets.h"
+
+namespace minerva {
+
+void Net::AddParam(const std::string& name, const Scale& size) {
+  param_names.push_back(name);
+  params[name] = rt->Zeros(size);
+}
+
+void Net::Sgd(const std::string& name, const Tensor& grad, float lr) {
+  results["g_" + name] = grad;
+  Tensor step = rt->ArithmeticConst(grad, lr / static_cast<float>(batch_), ArithmeticType::kMult, 0);
+  params[name] = rt->Sub(params[name], step);
+}
+
+// ------------------------------------------------------------------------- MLP
+
+MlpNet::MlpNet(Runner* r, int batch, int in, int hidden, int out)
+    : Net(r, batch), in_(in), hidden_(hidden), out_(out) {
+  AddParam("w0", Scale{hidden, in});
+  AddParam("b0", Scale{hidden, 1});
+  AddParam("w1", Scale{out, hidden});
+  AddParam("b1", Scale{out, 1});
+}
+
+void MlpNet::Step(const Tensor& data, const Tensor& label, float lr) {
+  Tensor& w0 = params["w0"]; Tensor& b0 = params["b0"];
+  Tensor& w1 = params["w1"]; Tensor& b1 = params["b1"];
+  // FF
+  Tensor a1 = rt->ReluForward(rt->NormArithmetic(rt->MatMult(w0, data), b0, ArithmeticType::kAdd));
+  Tensor a2 = rt->NormArithmetic(rt->MatMult(w1, a1), b1, ArithmeticType::kAdd);
+  Tensor a3 = rt->Reshape(
+      rt->SoftmaxForward(rt->Reshape(a2, Scale{out_, 1, 1, batch_}), SoftmaxAlgorithm::kInstance),
+      Scale{out_, batch_});
+  results["prob"] = a3;
+  // BP
+  Tensor s2 = rt->Sub(a3, label);
+  Tensor s1 = rt->ReluBackward(rt->MatMult(rt->Trans(w1), s2), a1, a1);
+  Tensor gw0 = rt->MatMult(s1, rt->Trans(data));
+  Tensor gb0 = rt->Sum(s1, 1);
+  Tensor gw1 = rt->MatMult(s2, rt->Trans(a1));
+  Tensor gb1 = rt->Sum(s2, 1);
+  // update
+  Sgd("w0", gw0, lr); Sgd("b0", gb0, lr); Sgd("w1", gw1, lr); Sgd("b1", gb1, lr);
+}
+
+// ------------------------------------------------------------------------- CNN
+
+CnnNet::CnnNet(Runner* r, int batch, int pad2, int pool2) : Net(r, batch) {
+  conv_info[0] = ConvInfo(0, 0, 1, 1);
+  conv_info[1] = ConvInfo(pad2, pad2, 1, 1);
+  pool_info[0] = PoolingInfo(PoolingInfo::Algorithm::kMax, 2, 2, 2, 2);
+  pool_info[1] = PoolingInfo(PoolingInfo::Algorithm::kMax, pool2, pool2, pool2, pool2);
+  AddParam("w0", Scale{5, 5, 1, 16});
+  AddParam("b0", Scale{16});
+  AddParam("w1", Scale{5, 5, 16, 32});
+  AddParam("b1", Scale{32});
+  AddParam("w2", Scale{10, 512});
+  AddParam("b2", Scale{10, 1});
+}
+
+void CnnNet::Step(const Tensor& data, const Tensor& label, float lr) {
+  const int b = batch_;
+  Tensor a0 = data;
+  Tensor a1 = rt->ConvForward(a0, params["w0"], params["b0"], conv_info[0]);
+  Tensor a2 = rt->ActivationForward(a1, ActivationAlgorithm::kRelu);
+  Tensor a3 = rt->PoolingForward(a2, pool_info[0]);
+  Tensor a4 = rt->ConvForward(a3, params["w1"], params["b1"], conv_info[1]);
+  Tensor a5 = rt->ActivationForward(a4, ActivationAlgorithm::kRelu);
+  Tensor a6 = rt->PoolingForward(a5, pool_info[1]);
+  Tensor re6 = rt->Reshape(a6, Scale{a6->size.Prod() / b, b});
+  MNV_CHECK_EQ(re6->size[0], 512) << "the classifier expects 512 features";
+  Tensor a7 = rt->NormArithmetic(rt->MatMult(params["w2"], re6), params["b2"], ArithmeticType::kAdd);
+  Tensor a8 = rt->SoftmaxForward(rt->Reshape(a7, Scale{10, 1, 1, b}), SoftmaxAlgorithm::kInstance);
+  results["prob"] = a8;
+  // BP
+  Tensor s8 = rt->Sub(a8, label);
+  Tensor s7 = rt->Reshape(s8, Scale{10, b});
+  Tensor s6 = rt->Reshape(rt->MatMult(rt->Trans(params["w2"]), s7), a6->size);
+  Tensor s5 = rt->PoolingBackward(s6, a6, a5, pool_info[1]);
+  Tensor s4 = rt->ActivationBackward(s5, a5, a4, ActivationAlgorithm::kRelu);
+  Tensor s3 = rt->ConvBackwardData(s4, a3, params["w1"], conv_info[1]);
+  Tensor s2 = rt->PoolingBackward(s3, a3, a2, pool_info[0]);
+  Tensor s1 = rt->ActivationBackward(s2, a2, a1, ActivationAlgorithm::kRelu);
+  Tensor gw0 = rt->ConvBackwardFilter(s1, a0, params["w0"], conv_info[0]);
+  Tensor gb0 = rt->ConvBackwardBias(s1);
+  Tensor gw1 = rt->ConvBackwardFilter(s4, a3, params["w1"], conv_info[1]);
+  Tensor gb1 = rt->ConvBackwardBias(s4);
+  Tensor gw2 = rt->MatMult(s7, rt->Trans(re6));
+  Tensor gb2 = rt->Sum(s7, 1);
+  Sgd("w0", gw0, lr); Sgd("b0", gb0, lr); Sgd("w1", gw1, lr); Sgd("b1", gb1, lr);
+  Sgd("w2", gw2, lr); Sgd("b2", gb2, lr);
+}
+
+// --------------------------------------------------------------------- AlexNet
+
+AlexNet::AlexNet(Runner* r, int batch, int num_classes) : Net(r, batch), classes_(num_classes) {
+  convs[0] = ConvInfo(0, 0, 4, 4);
+  convs[1] = ConvInfo(2, 2, 1, 1);
+  convs[2] = convs[3] = convs[4] = ConvInfo(1, 1, 1, 1);
+  for (auto& p : poolings) p = PoolingInfo(PoolingInfo::Algorithm::kMax, 3, 3, 2, 2);
+  AddParam("w0", Scale{11, 11, 3, 96});
+  AddParam("w1", Scale{5, 5, 96, 256});
+  AddParam("w2", Scale{3, 3, 256, 384});
+  AddParam("w3", Scale{3, 3, 384, 384});
+  AddParam("w4", Scale{3, 3, 384, 256});
+  AddParam("w5", Scale{4096, 9216});
+  AddParam("w6", Scale{4096, 4096});
+  AddParam("w7", Scale{num_classes, 4096});
+  AddParam("b0", Scale{96});
+  AddParam("b1", Scale{256});
+  AddParam("b2", Scale{384});
+  AddParam("b3", Scale{384});
+  AddParam("b4", Scale{256});
+  AddParam("b5", Scale{4096, 1});
+  AddParam("b6", Scale{4096, 1});
+  AddParam("b7", Scale{num_classes, 1});
+}
+
+void AlexNet::Step(const Tensor& data, const Tensor& label, float lr) {
+  const int n = batch_;
+  auto W = [&](int i) -> Tensor& { return params["w" + std::to_string(i)]; };
+  auto B = [&](int i) -> Tensor& { return params["b" + std::to_string(i)]; };
+  auto fc = [&](int i, const Tensor& x) {
+    return rt->NormArithmetic(rt->MatMult(W(i), x), B(i), ArithmeticType::kAdd);
+  };
+  Tensor acts[12], sens[12];
+  // FF
+  acts[0] = data;
+  acts[1] = rt->ReluForward(rt->ConvForward(acts[0], W(0), B(0), convs[0]));   // conv1
+  acts[2] = rt->PoolingForward(acts[1], poolings[0]);                           // pool1
+  acts[3] = rt->ReluForward(rt->ConvForward(acts[2], W(1), B(1), convs[1]));   // conv2
+  acts[4] = rt->PoolingForward(acts[3], poolings[1]);                           // pool2
+  acts[5] = rt->ReluForward(rt->ConvForward(acts[4], W(2), B(2), convs[2]));   // conv3
+  acts[6] = rt->ReluForward(rt->ConvForward(acts[5], W(3), B(3), convs[3]));   // conv4
+  acts[7] = rt->ReluForward(rt->ConvForward(acts[6], W(4), B(4), convs[4]));   // conv5
+  acts[8] = rt->PoolingForward(acts[7], poolings[2]);                           // pool5
+  Tensor re8 = rt->Reshape(acts[8], Scale{acts[8]->size.Prod() / n, n});
+  acts[9] = rt->ReluForward(fc(5, re8));                                        // fc6
+  acts[10] = rt->ReluForward(fc(6, acts[9]));                                   // fc7
+  acts[11] = fc(7, acts[10]);                                                   // fc8
+  Tensor out = rt->Reshape(
+      rt->SoftmaxForward(rt->Reshape(acts[11], Scale{classes_, 1, 1, n}), SoftmaxAlgorithm::kInstance),
+      Scale{classes_, n});
+  results["prob"] = out;
+  // BP
+  sens[11] = rt->Sub(out, label);
+  sens[10] = rt->ReluBackward(rt->MatMult(rt->Trans(W(7)), sens[11]), acts[10], acts[10]);
+  sens[9] = rt->ReluBackward(rt->MatMult(rt->Trans(W(6)), sens[10]), acts[9], acts[9]);
+  sens[8] = rt->Reshape(rt->MatMult(rt->Trans(W(5)), sens[9]), acts[8]->size);
+  sens[7] = rt->ReluBackward(rt->PoolingBackward(sens[8], acts[8], acts[7], poolings[2]), acts[7], acts[7]);
+  sens[6] = rt->ReluBackward(rt->ConvBackwardData(sens[7], acts[6], W(4), convs[4]), acts[6], acts[6]);
+  sens[5] = rt->ReluBackward(rt->ConvBackwardData(sens[6], acts[5], W(3), convs[3]), acts[5], acts[5]);
+  sens[4] = rt->ConvBackwardData(sens[5], acts[4], W(2), convs[2]);
+  sens[3] = rt->ReluBackward(rt->PoolingBackward(sens[4], acts[4], acts[3], poolings[1]), acts[3], acts[3]);
+  sens[2] = rt->ConvBackwardData(sens[3], acts[2], W(1), convs[1]);
+  sens[1] = rt->ReluBackward(rt->PoolingBackward(sens[2], acts[2], acts[1], poolings[0]), acts[1], acts[1]);
+  Tensor gw[8], gb[8];
+  gw[7] = rt->MatMult(sens[11], rt->Trans(acts[10]));
+  gw[6] = rt->MatMult(sens[10], rt->Trans(acts[9]));
+  gw[5] = rt->MatMult(sens[9], rt->Trans(re8));
+  gw[4] = rt->ConvBackwardFilter(sens[7], acts[6], W(4), convs[4]);
+  gw[3] = rt->ConvBackwardFilter(sens[6], acts[5], W(3), convs[3]);
+  gw[2] = rt->ConvBackwardFilter(sens[5], acts[4], W(2), convs[2]);
+  gw[1] = rt->ConvBackwardFilter(sens[3], acts[2], W(1), convs[1]);
+  gw[0] = rt->ConvBackwardFilter(sens[1], acts[0], W(0), convs[0]);
+  gb[7] = rt->Sum(sens[11], 1);
+  gb[6] = rt->Sum(sens[10], 1);
+  gb[5] = rt->Sum(sens[9], 1);
+  gb[4] = rt->ConvBackwardBias(sens[7]);
+  gb[3] = rt->ConvBackwardBias(sens[6]);
+  gb[2] = rt->ConvBackwardBias(sens[5]);
+  gb[1] = rt->ConvBackwardBias(sens[3]);
+  gb[0] = rt->ConvBackwardBias(sens[1]);
+  for (int i = 0; i < 8; ++i) {
+    Sgd("w" + std::to_string(i), gw[i], lr);
+    Sgd("b" + std::to_string(i), gb[i], lr);
+  }
+}
+
+}  // namespace minerva

@@ -1,0 +1,74 @@
+// The three training graphs of the benchmark configurations, written against the
+// Runner exactly as the reference applications write them against NArray:
+//   MLP 784-256-10          apps/mnist_common.h:213-288 (MnistMlpAlgo)
+//   MNIST CNN               apps/mnist_common.h:123-211 (MnistCnnAlgo)
+//   AlexNet-shaped network  owl/apps/imagenet_alexnet/alexnet.py:7-133 (no dropout / LRN,
+//                           single group), plain SGD w -= lr/batch * grad
+// One Step = forward + backward + parameter update, one operator at a time; nothing is
+// fused across operator boundaries.
+#pragma once
+#include <map>
+
+#include "runner.h"
+
+namespace minerva {
+
+class Net {
+ public:
+  Net(Runner* r, int batch) : rt(r), batch_(batch) {}
+  virtual ~Net() {}
+  virtual void Step(const Tensor& data, const Tensor& label, float lr) = 0;
+  virtual Scale DataSize() const = 0;
+  virtual Scale LabelSize() const = 0;
+  int batch() const { return batch_; }
+
+  std::vector<std::string> param_names;   // "w0", "b0", ...
+  std::map<std::string, Tensor> params;   // current parameters
+  std::map<std::string, Tensor> results;  // "prob" and "g_<param>" of the last Step
+
+ protected:
+  // w <- w - (lr / batch) * g : ArithmeticConst(mult, const on the left) + Arithmetic(sub)
+  void Sgd(const std::string& name, const Tensor& grad, float lr);
+  void AddParam(const std::string& name, const Scale& size);
+  Runner* rt;
+  int batch_;
+};
+
+class MlpNet : public Net {
+ public:
+  MlpNet(Runner* r, int batch, int in = 784, int hidden = 256, int out = 10);
+  void Step(const Tensor& data, const Tensor& label, float lr) override;
+  Scale DataSize() const override { return Scale{in_, batch_}; }
+  Scale LabelSize() const override { return Scale{out_, batch_}; }
+
+ private:
+  int in_, hidden_, out_;
+};
+
+class CnnNet : public Net {
+ public:
+  // pad2 / pool2: 0 and 2x2/2 (benchmark configuration) or 2 and 3x3/3 (reference app)
+  CnnNet(Runner* r, int batch, int pad2 = 0, int pool2 = 2);
+  void Step(const Tensor& data, const Tensor& label, float lr) override;
+  Scale DataSize() const override { return Scale{28, 28, 1, batch_}; }
+  Scale LabelSize() const override { return Scale{10, 1, 1, batch_}; }
+
+ private:
+  ConvInfo conv_info[2];
+  PoolingInfo pool_info[2];
+};
+
+class AlexNet : public Net {
+ public:
+  AlexNet(Runner* r, int batch, int num_classes = 1000);
+  void Step(const Tensor& data, const Tensor& label, float lr) override;
+  Scale DataSize() const override { return Scale{227, 227, 3, batch_}; }
+  Scale LabelSize() const override { return Scale{classes_, batch_}; }
+
+ private:
+  int classes_;
+  ConvInfo convs[5];
+  PoolingInfo poolings[3];
+};
+
+}  // namespace minerva

@@ -1,0 +1,242 @@
+#include "runner.h"
+
+#include <cstring>
+
+namespace minerva {
+
+TensorNode::~TensorNode() {
+  if (runner && runner->device_) runner->device_->FreeDataIfExist(id);
+}
+
+Runner::Runner(int gpu_id, bool sync_each_op) {
+  device_.reset(new HipDevice(0, this, gpu_id));
+  device_->set_sync_each_op(sync_each_op);
+}
+
+Runner::~Runner() {
+  device_->WaitForAllFinished();
+}
+
+Tensor Runner::Compute(const std::vector<Tensor>& inputs, const Scale& out_size,
+                       std::shared_ptr<ComputeFn> fn) {
+  Task task;
+  for (auto& t : inputs) {
+    MNV_CHECK(t) << "null tensor";
+    task.inputs.emplace_back(PhysicalData(t->size, device_->device_id(), t->id), t->id);
+  }
+  Tensor out = std::make_shared<TensorNode>(this, next_id_++, out_size);
+  task.outputs.emplace_back(PhysicalData(out_size, device_->device_id(), out->id), out->id);
+  task.op.compute_fn = std::move(fn);
+  task.op.device_id = device_->device_id();
+  task.id = ops_issued_++;
+  task.light = true;  // sequential: run on the caller's thread, worker stream 0
+  device_->PushTask(&task);
+  return out;
+}
+
+std::vector<float> Runner::Get(const Tensor& t) {
+  std::vector<float> host(t->size.Prod());
+  device_->Barrier(0);
+  device_->CopyToHost(host.data(), t->id, host.size());
+  return host;
+}
+
+Tensor Runner::MakeNArray(const Scale& size, std::shared_ptr<float> host) {
+  auto op = std::make_shared<ArrayLoaderOp>();
+  op->closure.data = std::move(host);
+  return Compute({}, size, op);
+}
+
+Tensor Runner::MakeNArray(const Scale& size, const float* host) {
+  size_t n = size.Prod();
+  std::shared_ptr<float> copy(new float[n], [](float* p) { delete[] p; });
+  std::memcpy(copy.get(), host, n * sizeof(float));
+  return MakeNArray(size, copy);
+}
+
+Tensor Runner::Constant(const Scale& size, float v) {
+  auto op = std::make_shared<FillOp>();
+  op->closure.val = v;
+  return Compute({}, size, op);
+}
+
+Tensor Runner::Arithmetic(const Tensor& a, const Tensor& b, ArithmeticType t) {
+  MNV_CHECK(a->size == b->size) << "size must match " << a->size << " " << b->size;
+  auto op = std::make_shared<ArithmeticOp>();
+  op->closure.type = t;
+  return Compute({a, b}, a->size, op);
+}
+
+Tensor Runner::ArithmeticConst(const Tensor& a, float v, ArithmeticType t, int side) {
+  auto op = std::make_shared<ArithmeticConstOp>();
+  op->closure = {t, v, side};
+  return Compute({a}, a->size, op);
+}
+
+Tensor Runner::Elewise(const Tensor& a, ElewiseType t) {
+  auto op = std::make_shared<ElewiseOp>();
+  op->closure.type = t;
+  return Compute({a}, a->size, op);
+}
+
+Tensor Runner::NormArithmetic(const Tensor& lhs, const Tensor& rhs, ArithmeticType t) {
+  MNV_CHECK_EQ(lhs->size.NumDims(), rhs->size.NumDims()) << "#dimension mismatch";
+  std::vector<int> rep;
+  for (size_t i = 0; i < lhs->size.NumDims(); ++i) {
+    if (lhs->size[i] == rhs->size[i]) continue;
+    MNV_CHECK_EQ(rhs->size[i], 1) << "NormArithmetic cannot replicate a dimension that is not 1";
+    rep.push_back(static_cast<int>(i));
+  }
+  MNV_CHECK(!rep.empty()) << "nothing to replicate";
+  auto op = std::make_shared<NormArithmeticOp>();
+  op->closure.type = t;
+  op->closure.dims_to_replicate = Scale(rep);
+  return Compute({lhs, rhs}, lhs->size, op);
+}
+
+Tensor Runner::MatMult(const Tensor& a, const Tensor& b) {
+  MNV_CHECK_EQ(a->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(b->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(a->size[1], b->size[0]) << "size must match";
+  return Compute({a, b}, Scale{a->size[0], b->size[1]}, std::make_shared<MatMultOp>());
+}
+
+Tensor Runner::Trans(const Tensor& a) {
+  MNV_CHECK_EQ(a->size.NumDims(), 2u) << "eligible only for 2D";
+  return Compute({a}, Scale{a->size[1], a->size[0]}, std::make_shared<TransOp>());
+}
+
+Tensor Runner::Reshape(const Tensor& a, const Scale& size) {
+  MNV_CHECK_EQ(a->size.Prod(), size.Prod()) << "reshape must keep the element count";
+  return Compute({a}, size, std::make_shared<ReshapeOp>());
+}
+
+Tensor Runner::Reduce(const Tensor& a, int dim, ReductionType t) {
+  MNV_CHECK(0 <= dim && dim < static_cast<int>(a->size.NumDims())) << "dim out of bound";
+  Scale size = a->size;
+  size[dim] = 1;
+  auto op = std::make_shared<ReductionOp>();
+  op->closure.type = t;
+  op->closure.dims_to_reduce = Scale{dim};
+  return Compute({a}, size, op);
+}
+
+Tensor Runner::MaxIndex(const Tensor& a, int dim) {
+  MNV_CHECK(0 <= dim && dim < static_cast<int>(a->size.NumDims())) << "dim out of bound";
+  Scale size = a->size;
+  size[dim] = 1;
+  auto op = std::make_shared<MaxIndexOp>();
+  op->closure.dim = dim;
+  return Compute({a}, size, op);
+}
+
+Tensor Runner::SigmoidForward(const Tensor& a) { return Compute({a}, a->size, std::make_shared<SigmoidForwardOp>()); }
+Tensor Runner::ReluForward(const Tensor& a) { return Compute({a}, a->size, std::make_shared<ReluForwardOp>()); }
+Tensor Runner::TanhForward(const Tensor& a) { return Compute({a}, a->size, std::make_shared<TanhForwardOp>()); }
+
+static void CheckSame(const Tensor& a, const Tensor& b) {
+  MNV_CHECK(a->size == b->size) << "inputs sizes mismatch";
+}
+
+Tensor Runner::SigmoidBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom) {
+  CheckSame(diff, top); CheckSame(diff, bottom);
+  return Compute({diff, top, bottom}, diff->size, std::make_shared<SigmoidBackwardOp>());
+}
+Tensor Runner::ReluBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom) {
+  CheckSame(diff, top); CheckSame(diff, bottom);
+  return Compute({diff, top, bottom}, diff->size, std::make_shared<ReluBackwardOp>());
+}
+Tensor Runner::TanhBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom) {
+  CheckSame(diff, top); CheckSame(diff, bottom);
+  return Compute({diff, top, bottom}, diff->size, std::make_shared<TanhBackwardOp>());
+}
+
+Tensor Runner::ActivationForward(const Tensor& a, ActivationAlgorithm alg) {
+  auto op = std::make_shared<ActivationForwardOp>();
+  op->closure.algorithm = alg;
+  return Compute({a}, a->size, op);
+}
+
+Tensor Runner::ActivationBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom,
+                                  ActivationAlgorithm alg) {
+  CheckSame(diff, top); CheckSame(diff, bottom);
+  auto op = std::make_shared<ActivationBackwardOp>();
+  op->closure.algorithm = alg;
+  return Compute({diff, top, bottom}, diff->size, op);
+}
+
+Tensor Runner::SoftmaxForward(const Tensor& a, SoftmaxAlgorithm alg) {
+  auto op = std::make_shared<SoftmaxForwardOp>();
+  op->closure.algorithm = alg;
+  return Compute({a}, a->size, op);
+}
+
+Tensor Runner::SoftmaxBackward(const Tensor& diff, const Tensor& top, SoftmaxAlgorithm alg) {
+  CheckSame(diff, top);
+  auto op = std::make_shared<SoftmaxBackwardOp>();
+  op->closure.algorithm = alg;
+  return Compute({diff, top}, diff->size, op);
+}
+
+Tensor Runner::ConvForward(const Tensor& src, const Tensor& filter, const Tensor& bias,
+                           ConvInfo info) {
+  MNV_CHECK_EQ(src->size.NumDims(), 4u);
+  MNV_CHECK_EQ(filter->size.NumDims(), 4u);
+  MNV_CHECK_EQ(src->size[2], filter->size[2]) << "#input channels mismatch";
+  MNV_CHECK_EQ(bias->size.NumDims(), 1u) << "bias dimension mismatch";
+  MNV_CHECK_EQ(bias->size[0], filter->size[3]) << "bias size mismatch";
+  Scale out{(src->size[0] + 2 * info.pad_width - filter->size[0]) / info.stride_horizontal + 1,
+            (src->size[1] + 2 * info.pad_height - filter->size[1]) / info.stride_vertical + 1,
+            filter->size[3], src->size[3]};
+  auto op = std::make_shared<ConvForwardOp>();
+  op->closure = {info.pad_height, info.pad_width, info.stride_vertical, info.stride_horizontal};
+  return Compute({src, filter, bias}, out, op);
+}
+
+Tensor Runner::ConvBackwardData(const Tensor& diff, const Tensor& bottom, const Tensor& filter,
+                                ConvInfo info) {
+  MNV_CHECK_EQ(diff->size[2], filter->size[3]) << "#output channels mismatch";
+  auto op = std::make_shared<ConvBackwardDataOp>();
+  op->closure = {info.pad_height, info.pad_width, info.stride_vertical, info.stride_horizontal};
+  return Compute({diff, filter}, bottom->size, op);
+}
+
+Tensor Runner::ConvBackwardFilter(const Tensor& diff, const Tensor& bottom, const Tensor& filter,
+                                  ConvInfo info) {
+  MNV_CHECK_EQ(diff->size[3], bottom->size[3]) << "#images mismatch";
+  auto op = std::make_shared<ConvBackwardFilterOp>();
+  op->closure = {info.pad_height, info.pad_width, info.stride_vertical, info.stride_horizontal};
+  return Compute({diff, bottom}, filter->size, op);
+}
+
+Tensor Runner::ConvBackwardBias(const Tensor& diff) {
+  return Compute({diff}, Scale{diff->size[2]}, std::make_shared<ConvBackwardBiasOp>());
+}
+
+static int PooledSize(int in, int win, int stride, int pad) {
+  int p = (in + 2 * pad - win + stride - 1) / stride + 1;
+  if (0 <= (p - 1) * stride - in - pad) --p;
+  return p;
+}
+
+Tensor Runner::PoolingForward(const Tensor& src, PoolingInfo info) {
+  MNV_CHECK_EQ(src->size.NumDims(), 4u);
+  Scale out{PooledSize(src->size[0], info.width, info.stride_horizontal, info.pad_width),
+            PooledSize(src->size[1], info.height, info.stride_vertical, info.pad_height),
+            src->size[2], src->size[3]};
+  auto op = std::make_shared<PoolingForwardOp>();
+  op->closure = {info.algorithm, info.height, info.width, info.stride_vertical,
+                 info.stride_horizontal, info.pad_height, info.pad_width};
+  return Compute({src}, out, op);
+}
+
+Tensor Runner::PoolingBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom,
+                               PoolingInfo info) {
+  CheckSame(diff, top);
+  auto op = std::make_shared<PoolingBackwardOp>();
+  op->closure = {info.algorithm, info.height, info.width, info.stride_vertical,
+                 info.stride_horizontal, info.pad_height, info.pad_width};
+  return Compute({diff, top, bottom}, bottom->size, op);
+}
+
+}  // namespace minerva

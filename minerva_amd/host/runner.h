@@ -1,0 +1,95 @@
+// A small sequential graph runner: the eager stand-in for Minerva's NArray front end
+// and DAG scheduler, enough to drive the operator layer exactly the way the reference
+// applications do.  Every call builds the same closure the reference's NArray method
+// builds, derives the output extent with the same rule, wraps it in a Task and hands it
+// to the HipDevice; a tensor frees its device data when its last handle dies, which is
+// what the DAG's reference counting does.  Output-extent rules follow
+//   convolution floor formula   minerva/narray/convolution.cpp:13-18
+//   pooling ceil + clip         minerva/narray/convolution.cpp:107-114
+//   broadcast dim detection     minerva/narray/narray.cpp:195-214
+//   reductions                  minerva/narray/narray_reduction.cpp:14-51
+#pragma once
+#include <atomic>
+
+#include "hip_device.h"
+
+namespace minerva {
+
+class Runner;
+
+struct TensorNode {
+  TensorNode(Runner* r, uint64_t i, const Scale& s) : runner(r), id(i), size(s) {}
+  ~TensorNode();
+  Runner* runner;
+  uint64_t id;
+  Scale size;
+};
+using Tensor = std::shared_ptr<TensorNode>;
+
+class Runner : public DeviceListener {
+ public:
+  explicit Runner(int gpu_id, bool sync_each_op = true);
+  ~Runner() override;
+  void OnOperationComplete(Task*) override { ++ops_completed_; }
+
+  HipDevice& device() { return *device_; }
+  uint64_t ops_issued() const { return ops_issued_; }
+  void Sync() { device_->Barrier(0); }
+
+  Tensor Compute(const std::vector<Tensor>& inputs, const Scale& out_size,
+                 std::shared_ptr<ComputeFn> fn);
+  std::vector<float> Get(const Tensor& t);
+
+  // data generators
+  Tensor MakeNArray(const Scale& size, std::shared_ptr<float> host);
+  Tensor MakeNArray(const Scale& size, const float* host);  // copies the host data first
+  Tensor Constant(const Scale& size, float v);
+  Tensor Zeros(const Scale& size) { return Constant(size, 0.f); }
+
+  // NArray arithmetic
+  Tensor Arithmetic(const Tensor& a, const Tensor& b, ArithmeticType t);
+  Tensor Add(const Tensor& a, const Tensor& b) { return Arithmetic(a, b, ArithmeticType::kAdd); }
+  Tensor Sub(const Tensor& a, const Tensor& b) { return Arithmetic(a, b, ArithmeticType::kSub); }
+  Tensor Mult(const Tensor& a, const Tensor& b) { return Arithmetic(a, b, ArithmeticType::kMult); }
+  Tensor Div(const Tensor& a, const Tensor& b) { return Arithmetic(a, b, ArithmeticType::kDiv); }
+  Tensor ArithmeticConst(const Tensor& a, float v, ArithmeticType t, int side);
+  Tensor Elewise(const Tensor& a, ElewiseType t);
+  Tensor NormArithmetic(const Tensor& lhs, const Tensor& rhs, ArithmeticType t);
+  Tensor MatMult(const Tensor& a, const Tensor& b);
+  Tensor Trans(const Tensor& a);
+  Tensor Reshape(const Tensor& a, const Scale& size);
+  Tensor Reduce(const Tensor& a, int dim, ReductionType t);
+  Tensor Sum(const Tensor& a, int dim) { return Reduce(a, dim, ReductionType::kSum); }
+  Tensor Max(const Tensor& a, int dim) { return Reduce(a, dim, ReductionType::kMax); }
+  Tensor MaxIndex(const Tensor& a, int dim);
+
+  // Elewise:: and Convolution::
+  Tensor SigmoidForward(const Tensor& a);
+  Tensor ReluForward(const Tensor& a);
+  Tensor TanhForward(const Tensor& a);
+  Tensor SigmoidBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom);
+  Tensor ReluBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom);
+  Tensor TanhBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom);
+  Tensor ActivationForward(const Tensor& a, ActivationAlgorithm alg);
+  Tensor ActivationBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom,
+                            ActivationAlgorithm alg);
+  Tensor SoftmaxForward(const Tensor& a, SoftmaxAlgorithm alg);
+  Tensor SoftmaxBackward(const Tensor& diff, const Tensor& top, SoftmaxAlgorithm alg);
+  Tensor ConvForward(const Tensor& src, const Tensor& filter, const Tensor& bias, ConvInfo info);
+  Tensor ConvBackwardData(const Tensor& diff, const Tensor& bottom, const Tensor& filter,
+                          ConvInfo info);
+  Tensor ConvBackwardFilter(const Tensor& diff, const Tensor& bottom, const Tensor& filter,
+                            ConvInfo info);
+  Tensor ConvBackwardBias(const Tensor& diff);
+  Tensor PoolingForward(const Tensor& src, PoolingInfo info);
+  Tensor PoolingBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom,
+                         PoolingInfo info);
+
+ private:
+  friend struct TensorNode;
+  std::unique_ptr<HipDevice> device_;
+  std::atomic<uint64_t> next_id_{1};
+  std::atomic<uint64_t> ops_issued_{0}, ops_completed_{0};
+};
+
+}  // namespace minerva

@@ -1,0 +1,149 @@
+"""ctypes binding of the C++ host layer (include/mnv_host.h -> lib/libmnv_host.so).
+
+`Runtime.op` runs one Minerva operator on numpy tensors through the complete host
+stack (closure -> Task -> HipDevice -> FnBundle -> hip::<Op> -> C ABI -> HIP kernel);
+`Net` drives the training graphs.  Tensors are (flat float32 data, Minerva dims) pairs:
+dims[0] is the fastest dimension, so a numpy array of shape dims[::-1] has the same bytes.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from . import capi
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libmnv_host.so")
+MAX_DIMS = 8
+
+
+class _Tensor(ctypes.Structure):
+    _fields_ = [("data", ctypes.POINTER(ctypes.c_float)), ("ndims", ctypes.c_int),
+                ("dims", ctypes.c_int * MAX_DIMS)]
+
+
+class HostError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise OSError("%s is missing: run `python -m minerva_amd.build`" % LIB_PATH)
+        capi.lib()  # libmnv_hip.so first, from the same directory
+        L = ctypes.CDLL(LIB_PATH)
+        L.mnvh_last_error.restype = ctypes.c_char_p
+        _lib = L
+    return _lib
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise HostError("%s: %s" % (what, lib().mnvh_last_error().decode()))
+
+
+class Runtime:
+    def __init__(self, gpu=0, sync_each_op=True):
+        self.h = ctypes.c_void_p()
+        _check(lib().mnvh_runtime_create(gpu, 1 if sync_each_op else 0, ctypes.byref(self.h)),
+               "runtime_create")
+
+    def close(self):
+        if self.h:
+            _check(lib().mnvh_runtime_destroy(self.h), "runtime_destroy")
+            self.h = None
+
+    def sync(self):
+        _check(lib().mnvh_runtime_sync(self.h), "runtime_sync")
+
+    def ops_issued(self):
+        n = ctypes.c_ulonglong()
+        _check(lib().mnvh_runtime_ops_issued(self.h, ctypes.byref(n)), "ops_issued")
+        return n.value
+
+    def pool_stats(self):
+        t, c = ctypes.c_size_t(), ctypes.c_size_t()
+        _check(lib().mnvh_runtime_pool_stats(self.h, ctypes.byref(t), ctypes.byref(c)), "pool_stats")
+        return t.value, c.value
+
+    def op(self, name, inputs, params=(), out_capacity=None):
+        """inputs: list of (array, dims).  Returns (flat float32 result, dims)."""
+        keep = []
+        arr = (_Tensor * max(len(inputs), 1))()
+        for i, (a, dims) in enumerate(inputs):
+            a = np.ascontiguousarray(a, dtype=np.float32).ravel()
+            assert a.size == int(np.prod(dims)), (name, a.size, dims)
+            keep.append(a)
+            arr[i].data = a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+            arr[i].ndims = len(dims)
+            for j, d in enumerate(dims):
+                arr[i].dims[j] = int(d)
+        if out_capacity is None:
+            out_capacity = max([int(np.prod(d)) for _, d in inputs] + [1]) * 4 + 1024
+        out = np.empty(out_capacity, dtype=np.float32)
+        nd = ctypes.c_int()
+        od = (ctypes.c_int * MAX_DIMS)()
+        p = (ctypes.c_double * max(len(params), 1))(*[float(x) for x in params])
+        _check(lib().mnvh_op(self.h, name.encode(), arr, len(inputs), p, len(params),
+                             out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                             ctypes.c_size_t(out_capacity), ctypes.byref(nd), od), name)
+        dims = [od[i] for i in range(nd.value)]
+        return out[:int(np.prod(dims))].copy(), dims
+
+    def concurrent_adds(self, a, b, count):
+        a = np.ascontiguousarray(a, np.float32)
+        b = np.ascontiguousarray(b, np.float32)
+        out = np.empty(count * a.size, np.float32)
+        fp = ctypes.POINTER(ctypes.c_float)
+        _check(lib().mnvh_concurrent_adds(self.h, a.ctypes.data_as(fp), b.ctypes.data_as(fp),
+                                          ctypes.c_size_t(a.size), count, out.ctypes.data_as(fp)),
+               "concurrent_adds")
+        return out.reshape(count, a.size)
+
+
+class Net:
+    def __init__(self, runtime, kind, batch, variant=0):
+        self.rt = runtime
+        self.h = ctypes.c_void_p()
+        _check(lib().mnvh_net_create(runtime.h, kind.encode(), batch, variant, ctypes.byref(self.h)),
+               "net_create")
+        n = ctypes.c_int()
+        _check(lib().mnvh_net_num_params(self.h, ctypes.byref(n)), "net_num_params")
+        self.params = {}
+        for i in range(n.value):
+            name = ctypes.create_string_buffer(16)
+            sz = ctypes.c_size_t()
+            _check(lib().mnvh_net_param_info(self.h, i, name, ctypes.byref(sz)), "net_param_info")
+            self.params[name.value.decode()] = sz.value
+
+    def close(self):
+        if self.h:
+            _check(lib().mnvh_net_destroy(self.h), "net_destroy")
+            self.h = None
+
+    def set_param(self, name, a):
+        a = np.ascontiguousarray(a, np.float32).ravel()
+        _check(lib().mnvh_net_set_param(self.h, name.encode(),
+                                        a.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                                        ctypes.c_size_t(a.size)), "net_set_param " + name)
+
+    def read(self, name, floats):
+        out = np.empty(floats, np.float32)
+        _check(lib().mnvh_net_read(self.h, name.encode(),
+                                   out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                                   ctypes.c_size_t(floats)), "net_read " + name)
+        return out
+
+    def load_batch(self, data, label):
+        d = np.ascontiguousarray(data, np.float32).ravel()
+        l = np.ascontiguousarray(label, np.float32).ravel()
+        fp = ctypes.POINTER(ctypes.c_float)
+        _check(lib().mnvh_net_load_batch(self.h, d.ctypes.data_as(fp), ctypes.c_size_t(d.size),
+                                         l.ctypes.data_as(fp), ctypes.c_size_t(l.size)),
+               "net_load_batch")
+
+    def step(self, lr):
+        _check(lib().mnvh_net_step(self.h, ctypes.c_float(lr)), "net_step")

@@ -1,0 +1,266 @@
+"""The C++ host layer on the GPU: every Minerva operator through closure -> Task ->
+HipDevice -> FnBundle -> hip::<Op> -> C ABI, checked against the CPU oracle in the style
+of the reference's own unit tests (tests/unittest_*.cpp), plus the device's allocator,
+its four-stream thread pool, its error convention, and the three training graphs."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from gpu_util import TOL, assert_bits_equal, normwise, say
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from minerva_amd import hostapi
+    r = hostapi.Runtime(0, sync_each_op=True)
+    yield r
+    r.close()
+
+
+def _rand(n, seed, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal(n) * scale).astype(np.float32)
+
+
+def test_arithmetic_like_reference_unit_tests(rt, ora):
+    dims = [2, 3, 4, 5, 6]   # tests/unittest_arithmetic.cpp
+    a, b = _rand(720, 60), _rand(720, 61)
+    for typ in (ora.ADD, ora.SUB, ora.MUL, ora.DIV):
+        got, od = rt.op("arithmetic", [(a, dims), (b, dims)], [typ])
+        assert od == dims
+        assert_bits_equal(got, ora.arithmetic(typ, a, b), "arithmetic %d" % typ)
+        for side in (0, 1):
+            got, _ = rt.op("arithmetic_const", [(a, dims)], [typ, 3.291, side])
+            assert_bits_equal(got, ora.arithmetic_const(typ, side, 3.291, a), "const")
+    for typ in (ora.EXP, ora.NEG):
+        got, _ = rt.op("elewise", [(a, dims)], [typ])
+        assert normwise(got, ora.elewise(typ, a)) <= TOL
+    got, _ = rt.op("elewise", [(np.abs(a) + 500, dims)], [ora.LN])
+    assert normwise(got, ora.elewise(ora.LN, np.abs(a) + np.float32(500))) <= TOL
+
+
+def test_norm_arithmetic_and_reductions(rt, ora):
+    x = _rand(63, 62)
+    row, col = _rand(7, 63), _rand(9, 64)
+    got, _ = rt.op("norm_arithmetic", [(x, [9, 7]), (row, [1, 7])], [ora.ADD])
+    assert_bits_equal(got, ora.norm_arithmetic(ora.ADD, x, [9, 7], row, [0]), "{9,7}+{1,7}")
+    got, _ = rt.op("norm_arithmetic", [(x, [9, 7]), (col, [9, 1])], [ora.MUL])
+    assert_bits_equal(got, ora.norm_arithmetic(ora.MUL, x, [9, 7], col, [1]), "{9,7}*{9,1}")
+    iota = np.arange(15, dtype=np.float32)
+    for typ, dim, want in ((ora.MAX, 0, [4, 9, 14]), (ora.MAX, 1, [10, 11, 12, 13, 14]),
+                           (ora.SUM, 0, [10, 35, 60]), (ora.SUM, 1, [15, 18, 21, 24, 27])):
+        got, od = rt.op("reduction", [(iota, [5, 3])], [typ, dim])
+        np.testing.assert_array_equal(got, want)
+        assert od == ([1, 3] if dim == 0 else [5, 1])
+    got, od = rt.op("maxindex", [(iota, [5, 3])], [0])
+    np.testing.assert_array_equal(got, [4, 4, 4])
+    # higher rank, first and last dimension (the CPU implementation is N-d)
+    y = _rand(4 * 3 * 5, 65)
+    for dim in (0, 2):
+        got, _ = rt.op("reduction", [(y, [4, 3, 5])], [ora.MAX, dim])
+        assert_bits_equal(got, ora.reduction(ora.MAX, y, [4, 3, 5], [dim]), "3-d max")
+        got, _ = rt.op("maxindex", [(y, [4, 3, 5])], [dim])
+        assert_bits_equal(got, ora.maxindex(y, [4, 3, 5], dim), "3-d maxindex")
+    v = _rand(15, 66)
+    got, _ = rt.op("norm_arithmetic", [(y, [4, 3, 5]), (v, [1, 3, 5])], [ora.SUB])
+    assert_bits_equal(got, ora.norm_arithmetic(ora.SUB, y, [4, 3, 5], v, [0]), "3-d norm")
+
+
+def test_matmult_transpose_reshape(rt, ora):
+    a, b = _rand(6, 67), _rand(10, 68)   # tests/unittest_sgemm.cpp: {3,2} x {2,5}
+    got, od = rt.op("matmult", [(a, [3, 2]), (b, [2, 5])])
+    assert od == [3, 5]
+    assert normwise(got, ora.matmult(a, b, 3, 5, 2)) <= TOL
+    x = _rand(35, 69)
+    got, od = rt.op("trans", [(x, [5, 7])])
+    assert od == [7, 5]
+    assert_bits_equal(got, ora.transpose(x, 7, 5), "trans")
+    got, od = rt.op("reshape", [(x, [5, 7])], [7, 5, 1])
+    assert od == [7, 5, 1]
+    assert_bits_equal(got, x, "reshape")
+
+
+def test_activations_and_softmax(rt, ora):
+    dims = [7, 6, 3, 2]  # tests/unittest_activation.cpp
+    x, dy = _rand(252, 70), _rand(252, 71)
+    names = {ora.SIGMOID: "sigmoid", ora.RELU: "relu", ora.TANH: "tanh"}
+    for alg, nm in names.items():
+        y_ref = ora.activation_fwd(alg, x)
+        got, _ = rt.op(nm + "_forward", [(x, dims)])
+        got2, _ = rt.op("activation_forward", [(x, dims)], [alg])
+        assert_bits_equal(got, got2, "Elewise:: and Convolution:: entry points agree")
+        assert normwise(got, y_ref) <= TOL
+        back, _ = rt.op(nm + "_backward", [(dy, dims), (y_ref, dims), (x, dims)])
+        back2, _ = rt.op("activation_backward", [(dy, dims), (y_ref, dims), (x, dims)], [alg])
+        assert_bits_equal(back, back2, "backward entry points agree")
+        assert normwise(back, ora.activation_bwd(alg, dy, y_ref, x)) <= TOL
+    z = _rand(10 * 256, 72) * 3
+    y, od = rt.op("softmax_forward", [(z, [10, 1, 1, 256])], [0])
+    ref = ora.softmax_instance_fwd(z, 256, 10, 1, 1)
+    assert normwise(y, ref) <= TOL
+    d, _ = rt.op("softmax_backward", [(_rand(2560, 73), [10, 1, 1, 256]), (ref, [10, 1, 1, 256])], [0])
+    assert normwise(d, ora.softmax_instance_bwd(_rand(2560, 73), ref, 256, 10, 1, 1)) <= TOL
+    c, _ = rt.op("softmax_forward", [(z[:120], [4, 3, 5, 2])], [1])
+    assert normwise(c, ora.softmax_channel_fwd(z[:120], 2, 5, 3, 4)) <= TOL
+
+
+def test_convolution_golden_and_gradients(rt, ora):
+    for case in json.load(open(os.path.join(GOLD, "conv_forward.json"))):
+        W, H, C, N = case["input_size"]
+        S, R, _, K = case["weight_size"]
+        x = np.array(case["input"], np.float32)
+        w = np.array(case["weight"], np.float32)
+        b = np.array(case["bias"] or [0] * K, np.float32)
+        info = [case["pad_height"], case["pad_width"], case["stride_vertical"],
+                case["stride_horizontal"]]
+        got, od = rt.op("conv_forward", [(x, case["input_size"]), (w, case["weight_size"]), (b, [K])],
+                        info)
+        assert od == case["correct_size"]
+        idx = np.arange(got.size)
+        want = np.array(case["correct_without_bias"], np.float32) + b[(idx // 16) % K]
+        assert np.max(np.abs(got - want)) < 1e-3
+        p = (N, C, K, H, W, *info, R, S)
+        dy = _rand(got.size, 74)
+        gd, od = rt.op("conv_backward_data", [(dy, od), (x, case["input_size"]), (w, case["weight_size"])], info)
+        assert od == case["input_size"]
+        assert normwise(gd, ora.conv_bwd_data(dy, w, *p)) <= TOL
+        gf, od = rt.op("conv_backward_filter", [(dy, case["correct_size"]), (x, case["input_size"]),
+                                                (w, case["weight_size"])], info)
+        assert od == case["weight_size"]
+        assert normwise(gf, ora.conv_bwd_filter(dy, x, *p)) <= TOL
+        gb, od = rt.op("conv_backward_bias", [(dy, case["correct_size"])])
+        assert od == [K]
+        assert normwise(gb, ora.conv_bwd_bias(dy, N, K, case["correct_size"][1], case["correct_size"][0])) <= TOL
+
+
+def test_pooling_golden_and_gradient(rt, ora):
+    for case in json.load(open(os.path.join(GOLD, "pooling_forward.json"))):
+        x = np.array(case["input"], np.float32)
+        prm = [0, case["height"], case["width"], case["stride_vertical"], case["stride_horizontal"],
+               case["pad_height"], case["pad_width"]]
+        got, od = rt.op("pooling_forward", [(x, case["input_size"])], prm)
+        assert od == case["correct_size"]          # EXPECT_EQ(output.Size(), correct_size)
+        np.testing.assert_array_equal(got, np.array(case["correct"], np.float32))
+        dy = _rand(got.size, 75)
+        back, od = rt.op("pooling_backward", [(dy, od), (got, od), (x, case["input_size"])], prm)
+        assert od == case["input_size"]
+        W, H, C, N = case["input_size"]
+        ref = ora.pool_bwd(ora.POOL_MAX, dy, got, x, N, C, H, W, *prm[3:5], *prm[1:3], *prm[5:7])
+        assert_bits_equal(back, ref, "pool bwd")
+
+
+def test_error_convention(rt):
+    from minerva_amd import hostapi
+    a = _rand(6, 76)
+    with pytest.raises(hostapi.HostError, match="size must match"):
+        rt.op("arithmetic", [(a, [2, 3]), (a, [3, 2])], [0])
+    with pytest.raises(hostapi.HostError, match="size must match"):
+        rt.op("matmult", [(a, [2, 3]), (a, [2, 3])])
+    with pytest.raises(hostapi.HostError, match="cannot replicate"):
+        rt.op("norm_arithmetic", [(a, [2, 3]), (a[:4], [2, 2])], [0])
+    with pytest.raises(hostapi.HostError, match="first or the last"):
+        rt.op("reduction", [(_rand(24, 77), [2, 3, 4])], [0, 1])
+    with pytest.raises(hostapi.HostError, match="channels mismatch"):
+        rt.op("conv_forward", [(_rand(36, 78), [3, 3, 2, 2]), (a[:4], [2, 2, 1, 1]), (a[:1], [1])],
+              [0, 0, 1, 1])
+    with pytest.raises(hostapi.HostError, match="unknown operator"):
+        rt.op("lrn_forward", [(a, [6])])
+    # the runtime is still usable after a failed check
+    got, _ = rt.op("arithmetic", [(a, [6]), (a, [6])], [0])
+    assert_bits_equal(got, a + a, "after error")
+
+
+def test_pooled_allocator_reuses_exact_sizes(rt):
+    a = _rand(5000, 79)
+    rt.op("arithmetic", [(a, [5000]), (a, [5000])], [0])
+    total0, cached0 = rt.pool_stats()
+    for _ in range(5):
+        rt.op("arithmetic", [(a, [5000]), (a, [5000])], [0])
+    total1, cached1 = rt.pool_stats()
+    assert total1 == total0, "same-size requests must be served from the free lists"
+    assert cached1 >= 3  # two inputs and one output went back to the pool
+
+
+def test_four_stream_thread_pool(rt):
+    a, b = _rand(100003, 80), _rand(100003, 81)
+    out = rt.concurrent_adds(a, b, 24)
+    for i in range(24):
+        assert_bits_equal(out[i], a + b, "concurrent add %d" % i)
+
+
+def _run_net(kind, batch, steps, sync_each_op, variant=0, lr=0.01):
+    from minerva_amd import hostapi
+    from oracle import nets
+    params, data, label = nets.make_inputs(kind, batch)
+    r = hostapi.Runtime(0, sync_each_op=sync_each_op)
+    net = hostapi.Net(r, kind, batch, variant)
+    for k, v in params.items():
+        net.set_param(k, v)
+    net.load_batch(data, label)
+    for _ in range(steps):
+        net.step(lr)
+    r.sync()
+    out = {k: net.read(k, n) for k, n in net.params.items()}
+    out.update({"g_" + k: net.read("g_" + k, n) for k, n in net.params.items()})
+    out["prob"] = net.read("prob", label.size)
+    ops = r.ops_issued()
+    net.close()
+    r.close()
+    return out, ops
+
+
+# A whole training step chains ~20 fp32 operators, and both sides round at every one of
+# them (the oracle's sequential sums included), so gradients that end in a cancelling sum
+# (the bias gradients) are compared at 5e-4 normwise; single operators stay at 1e-4.
+TOL_STEP = 5e-4
+
+
+def _compare(got, newp, res, grad_tol=TOL):
+    for k, v in newp.items():
+        assert normwise(got["g_" + k], res["g_" + k]) <= grad_tol, "gradient " + k
+        assert normwise(got[k], v) <= TOL, "updated " + k
+    assert normwise(got["prob"], res["prob"]) <= TOL
+
+
+def test_mlp_step_matches_oracle(ora):
+    from oracle import nets
+    params, data, label = nets.make_inputs("mlp", 256)
+    p = dict(params)
+    for _ in range(2):
+        p, res = nets.mlp_step(p, data, label, 0.01, 256)
+    say("mlp 2 steps, per-op sync")
+    got, ops = _run_net("mlp", 256, 2, True)
+    _compare(got, p, res)
+    say("mlp 2 steps, one sync per step")
+    got2, _ = _run_net("mlp", 256, 2, False)
+    for k in got:
+        assert_bits_equal(got[k], got2[k], "sync mode must not change " + k)
+    assert ops >= 2 * 25
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_cnn_step_matches_oracle(ora, variant):
+    from oracle import nets
+    batch = 16
+    params, data, label = nets.make_inputs("cnn", batch)
+    kw = dict(pad2=2, pool2=3) if variant else {}
+    p, res = nets.cnn_step(dict(params), data, label, 0.01, batch, **kw)
+    say("cnn step variant", variant)
+    got, _ = _run_net("cnn", batch, 1, True, variant)
+    _compare(got, p, res)
+
+
+def test_alexnet_step_matches_oracle_small_batch(ora):
+    from oracle import nets
+    batch = 2
+    params, data, label = nets.make_inputs("alexnet", batch)
+    say("alexnet oracle step b=2 (CPU)")
+    p, res = nets.alexnet_step(dict(params), data, label, 0.01, batch)
+    say("alexnet GPU step b=2")
+    got, ops = _run_net("alexnet", batch, 1, False)
+    _compare(got, p, res, TOL_STEP)
+    assert ops > 80
