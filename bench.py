@@ -1,0 +1,197 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X operator layer on BASELINE.json's metric:
+"AlexNet-shape fp32 train images/s at b=256; SGEMM TFLOP/s; eltwise HBM GB/s".
+
+One step = one forward + backward + SGD pass of the AlexNet-shaped network
+(BASELINE.json configs[4]) at batch 256 on one GPU, every operator issued separately
+through the C++ host layer (Task -> HipDevice -> hip::<Op> -> C ABI -> HIP kernel),
+synthetic seeded inputs already resident in HBM.  `value` is images/s with one stream
+synchronisation per step; the same step with the reference device's per-operator
+synchronisation is reported beside it.  The dominant kernel (the MFMA implicit-GEMM
+filter-gradient kernel) is timed with HIP events on its own stream inside the timed
+steps and priced against the fp32 MFMA peak.  SGEMM 4096^3 and the 8192^2 elementwise add
+are measured the same way and reported in the same JSON line, and the CPU oracle is
+timed on a bounded sample of the same workload on the host cores.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+BATCH = 256
+
+# 2*N*Ho*Wo*K*C*R*S per convolution pass at batch 256, in GFLOP (conv1..conv5)
+CONV_GFLOP = [53.97, 229.32, 76.55, 114.83, 76.55]
+STEP_GFLOP = 1689.8  # convolutions (fwd, bwd-filter, bwd-data except conv1) + three FC layers
+
+
+def log(*a):
+    print(*a, file=sys.stderr)
+    sys.stderr.flush()
+
+
+def alexnet_bench(steps, warmup):
+    from minerva_amd import hostapi
+    from oracle import nets  # input generator only (seeded host data)
+    params, data, label = nets.make_inputs("alexnet", BATCH)
+    out = {}
+    for mode, sync_each in (("per_step_sync", False), ("per_op_sync", True)):
+        rt = hostapi.Runtime(0, sync_each_op=sync_each)
+        net = hostapi.Net(rt, "alexnet", BATCH)
+        for k, v in params.items():
+            net.set_param(k, v)
+        net.load_batch(data, label)
+        for _ in range(warmup):
+            net.step(0.01)
+        rt.sync()
+        ops0 = rt.ops_issued()
+        rt.profile(not sync_each)
+        rt.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            net.step(0.01)
+            rt.sync()
+        t1 = time.perf_counter()
+        prof = rt.profile_read() if not sync_each else {}
+        rt.profile(False)
+        prob = net.read("prob", 1000 * BATCH)
+        ms = (t1 - t0) * 1e3 / steps
+        out[mode] = {"ms_per_step": ms, "images_per_s": BATCH / (ms / 1e3),
+                     "ops_per_step": (rt.ops_issued() - ops0) // steps,
+                     "finite": bool(np.isfinite(prob).all()), "profile": prof}
+        log("alexnet b=%d %s: %.3f ms/step, %.1f img/s, %d ops/step" %
+            (BATCH, mode, ms, out[mode]["images_per_s"], out[mode]["ops_per_step"]))
+        net.close()
+        rt.close()
+    return out
+
+
+def dominant_kernel_roofline(prof, steps):
+    """The filter-gradient operators of conv2..conv5 run the 128x128 MFMA kernel
+    (mnv_gemm_kernel<128x128x16, ConvBwdFilter>) followed by its split-k reduction; the
+    event pair brackets both, so the figure is slightly conservative."""
+    names = [n for n in prof if n.endswith("conv bp filter") and "stride:1*1" in n]
+    launches = sum(prof[n][0] for n in names)
+    total_ms = sum(prof[n][1] for n in names)
+    if not launches:
+        return None
+    gflop_per_step = sum(CONV_GFLOP[1:])
+    flops_per_launch = gflop_per_step * 1e9 * steps / launches
+    avg_ms = total_ms / launches
+    achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
+    return {"bound": "mfma", "kernel": "mnv_gemm_kernel<128x128x16,ConvBwdFilter> (conv2-5 filter gradient)",
+            "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+            "avg_launch_ms": round(avg_ms, 4), "launches": launches,
+            "algorithmic_gflop_per_launch": round(flops_per_launch / 1e9, 2)}
+
+
+def op_table(prof, steps):
+    rows = sorted(prof.items(), key=lambda kv: -kv[1][1])
+    return [{"op": n, "launches_per_step": c // steps, "ms_per_step": round(ms / steps, 4)}
+            for n, (c, ms) in rows[:12]]
+
+
+def micro_bench():
+    """SGEMM 4096^3 (N(0,1) inputs) and the 8192^2 elementwise add, events on the stream."""
+    from minerva_amd import capi
+    L = capi.lib()
+    dev = capi.Device(0)
+    rng = np.random.default_rng(7)
+    m = n = k = 4096
+    a = dev.upload(rng.standard_normal(m * k, dtype=np.float32))
+    b = dev.upload(rng.standard_normal(k * n, dtype=np.float32))
+    c = dev.empty(m * n)
+    ms = dev.time_ms(lambda: L.mnv_sgemm_nn(a.p, b.p, c.p, m, n, k, None, 0, dev.stream), iters=20, warmup=5)
+    tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+    sgemm = {"shape": "4096x4096x4096", "ms": round(ms, 4), "tflops": round(tf, 2),
+             "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
+                          "unit": "TFLOP/s", "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}}
+    log("sgemm 4096^3: %.3f ms, %.1f TFLOP/s" % (ms, tf))
+    ne = 8192 * 8192
+    # three distinct 256 MiB buffers: 768 MiB per pass, larger than the 256 MB last-level cache
+    x = dev.upload(rng.standard_normal(ne, dtype=np.float32))
+    y = dev.upload(rng.standard_normal(ne, dtype=np.float32))
+    z = dev.empty(ne)
+    ms = dev.time_ms(lambda: L.mnv_add(x.p, y.p, z.p, ne, dev.stream), iters=50, warmup=5)
+    gbs = 12.0 * ne / (ms * 1e-3) / 1e9
+    elt = {"op": "add 8192x8192", "ms": round(ms, 4), "gbs": round(gbs, 1),
+           "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+                        "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}}
+    log("add 8192^2: %.4f ms, %.0f GB/s" % (ms, gbs))
+    return sgemm, elt
+
+
+def cpu_baseline(batch=4):
+    """The CPU oracle's AlexNet step on a bounded sample (batch 4 instead of 256): naive
+    single-threaded loops; convolution and pooling have no reference CPU implementation,
+    so this is the repository's restatement ("port"), timed on one host core."""
+    from oracle import nets
+    params, data, label = nets.make_inputs("alexnet", batch)
+    t0 = time.perf_counter()
+    nets.alexnet_step(params, data, label, 0.01, batch)
+    dt = time.perf_counter() - t0
+    log("cpu oracle alexnet b=%d: %.2f s" % (batch, dt))
+    return {"value": round(batch / dt, 4), "unit": "images/s", "cores": 1, "kind": "port",
+            "sample": "one AlexNet-shaped train step at batch %d (of 256) with the naive "
+                      "single-threaded CPU oracle, %.1f s" % (batch, dt),
+            "host_cpus": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures the one-GPU operator path only: run with --gpus 1 "
+                 "(nothing in this build uses a second GPU)")
+    from minerva_amd import capi
+    dev_info = capi.Device(0, own_stream=False).info()
+    log("device:", dev_info)
+    res = alexnet_bench(args.steps, args.warmup)
+    main_run = res["per_step_sync"]
+    roof = dominant_kernel_roofline(main_run["profile"], args.steps)
+    sgemm, elt = micro_bench()
+    line = {
+        "metric": "AlexNet-shape fp32 train images/s at b=256; SGEMM TFLOP/s; eltwise HBM GB/s",
+        "value": round(main_run["images_per_s"], 1),
+        "unit": "images/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(main_run["ms_per_step"], 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "AlexNet-shaped single-group network (BASELINE.json configs[4]): "
+                               "NCHW fp32, batch 256, 3x227x227 input, forward + backward + SGD, "
+                               "one operator per launch, one stream sync per step",
+                   "global_batch": BATCH, "ops_per_step": main_run["ops_per_step"],
+                   "algorithmic_gflop_per_step": STEP_GFLOP},
+        "step_mfma_frac": round(STEP_GFLOP / main_run["ms_per_step"] / PEAK_FP32_MFMA_TFLOPS, 4),
+        "per_op_sync": {"images_per_s": round(res["per_op_sync"]["images_per_s"], 1),
+                        "ms_per_step": round(res["per_op_sync"]["ms_per_step"], 3)},
+        "roofline": roof,
+        "sgemm": sgemm,
+        "eltwise": elt,
+        "top_ops": op_table(main_run["profile"], args.steps),
+        "device": dev_info,
+        "outputs_finite": main_run["finite"] and res["per_op_sync"]["finite"],
+    }
+    line["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

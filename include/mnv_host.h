@@ -43,6 +43,12 @@ int mnvh_runtime_sync(void* runtime);
 int mnvh_runtime_ops_issued(void* runtime, unsigned long long* count);
 int mnvh_runtime_pool_stats(void* runtime, size_t* total_bytes, size_t* cached_blocks);
 
+/* Per-operator device timing (two events per operator on its own stream).  The read
+ * synchronises, writes one "name<TAB>launches<TAB>total_ms" line per operator name and
+ * clears the record. */
+int mnvh_runtime_profile(void* runtime, int enable);
+int mnvh_runtime_profile_read(void* runtime, char* text_out, size_t capacity);
+
 /*
  * Runs one operator on host tensors through the whole host stack.  `op` and
  * `params` (all passed as doubles):

@@ -72,6 +72,21 @@ int mnvh_runtime_pool_stats(void* runtime, size_t* total_bytes, size_t* cached_b
   });
 }
 
+int mnvh_runtime_profile(void* runtime, int enable) {
+  return Guard([&] { static_cast<Runner*>(runtime)->device().set_profile(enable != 0); });
+}
+
+int mnvh_runtime_profile_read(void* runtime, char* text_out, size_t capacity) {
+  return Guard([&] {
+    auto prof = static_cast<Runner*>(runtime)->device().CollectProfile();
+    std::ostringstream ss;
+    for (auto& kv : prof) ss << kv.first << "\t" << kv.second.first << "\t" << kv.second.second << "\n";
+    std::string s = ss.str();
+    MNV_CHECK(text_out && s.size() + 1 <= capacity) << "profile text needs " << s.size() + 1 << " bytes";
+    std::memcpy(text_out, s.c_str(), s.size() + 1);
+  });
+}
+
 int mnvh_op(void* runtime, const char* op_name, const mnvh_tensor* inputs, int n_inputs,
             const double* params, int n_params, float* out, size_t out_capacity,
             int* out_ndims, int* out_dims) {

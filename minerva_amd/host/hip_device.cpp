@@ -254,11 +254,44 @@ void HipDevice::DoExecute(const DataList& in, const DataList& out, PhysicalOp& o
   ctx.stream = streams_[thrid];
   ctx.workspace = workspace_[thrid];
   ctx.workspace_bytes = workspace_bytes_[thrid];
+  Timed t{std::string(), nullptr, nullptr};
+  if (profile_) {
+    t.name = op.compute_fn->Name();
+    Ok(mnv_event_create(&t.start), "event create");
+    Ok(mnv_event_create(&t.stop), "event create");
+    Ok(mnv_event_record(t.start, streams_[thrid]), "event record");
+  }
   op.compute_fn->Execute(in, out, ctx);
+  if (profile_) {
+    Ok(mnv_event_record(t.stop, streams_[thrid]), "event record");
+    std::lock_guard<std::mutex> lck(prof_mutex_);
+    timed_.push_back(t);
+  }
   if (sync_each_op_) {
     int rc = mnv_stream_sync(streams_[thrid]);
     MNV_CHECK(rc == MNV_OK) << op.compute_fn->Name() << ": " << mnv_error_string(rc);
   }
+}
+
+std::map<std::string, std::pair<int, double>> HipDevice::CollectProfile() {
+  Activate();
+  for (size_t i = 0; i < kParallelism; ++i) Ok(mnv_stream_sync(streams_[i]), "profile sync");
+  std::vector<Timed> rec;
+  {
+    std::lock_guard<std::mutex> lck(prof_mutex_);
+    rec.swap(timed_);
+  }
+  std::map<std::string, std::pair<int, double>> out;
+  for (auto& t : rec) {
+    float ms = 0.f;
+    Ok(mnv_event_elapsed_ms(t.start, t.stop, &ms), "event elapsed");
+    auto& e = out[t.name];
+    e.first += 1;
+    e.second += ms;
+    mnv_event_destroy(t.start);
+    mnv_event_destroy(t.stop);
+  }
+  return out;
 }
 
 void HipDevice::Barrier(int thrid) { Ok(mnv_stream_sync(streams_[thrid]), "barrier"); }

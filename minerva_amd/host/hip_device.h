@@ -117,6 +117,13 @@ class HipDevice {
   // First error raised by an operator on a pool thread (empty if none).
   std::string TakeAsyncError();
 
+  // Per-operator timing, the counterpart of the reference's ExecutionProfiler
+  // (minerva/profiler/execution_profiler.cpp:17-53): while enabled, every operator is
+  // bracketed by two events on its own stream; CollectProfile synchronises and returns
+  // name -> (launch count, total device milliseconds), then clears the record.
+  void set_profile(bool v) { profile_ = v; }
+  std::map<std::string, std::pair<int, double>> CollectProfile();
+
  private:
   void Execute(Task* task, int thrid);
   void DoExecute(const DataList& in, const DataList& out, PhysicalOp& op, int thrid);
@@ -143,6 +150,14 @@ class HipDevice {
   bool stop_ = false;
   std::mutex err_mutex_;
   std::string async_error_;
+  struct Timed {
+    std::string name;
+    void* start;
+    void* stop;
+  };
+  bool profile_ = false;
+  std::mutex prof_mutex_;
+  std::vector<Timed> timed_;
 };
 
 }  // namespace minerva

@@ -69,6 +69,19 @@ class Runtime:
         _check(lib().mnvh_runtime_pool_stats(self.h, ctypes.byref(t), ctypes.byref(c)), "pool_stats")
         return t.value, c.value
 
+    def profile(self, enable):
+        _check(lib().mnvh_runtime_profile(self.h, 1 if enable else 0), "profile")
+
+    def profile_read(self):
+        """{operator name: (launches, total device ms)} since the last read."""
+        buf = ctypes.create_string_buffer(1 << 16)
+        _check(lib().mnvh_runtime_profile_read(self.h, buf, ctypes.c_size_t(len(buf))), "profile_read")
+        out = {}
+        for line in buf.value.decode().splitlines():
+            name, cnt, ms = line.split("\t")
+            out[name] = (int(cnt), float(ms))
+        return out
+
     def op(self, name, inputs, params=(), out_capacity=None):
         """inputs: list of (array, dims).  Returns (flat float32 result, dims)."""
         keep = []
