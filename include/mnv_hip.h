@@ -175,17 +175,31 @@ int mnv_softmax_channel_bwd(const float* top_diff, const float* top, float* bott
  * backward_data takes the bottom extent (not the top extent the reference
  * launcher re-derives it from, cuda_perform.cu:277) so that inexact fits work,
  * and writes every element of bottom_diff.  backward_filter overwrites
- * filter_diff (beta = 0). ---- */
+ * filter_diff (beta = 0).  The workspace (optional everywhere) holds a re-ordered copy of
+ * the filter for forward / backward_data (which then read the reduction dimension as
+ * (tap, channel) and spend no address arithmetic per 16-channel slab) and the split
+ * partial sums for backward_filter; without it a slower, equally exact path runs. ---- */
+size_t mnv_conv_fwd_workspace_bytes(int num_images, int bottom_num_channels,
+                                   int top_num_channels, int bottom_height, int bottom_width,
+                                   int pad_height, int pad_width, int stride_vertical,
+                                   int stride_horizontal, int filter_height, int filter_width);
 int mnv_conv_fwd(const float* bottom, const float* filter, const float* bias, float* top,
                  int num_images, int bottom_num_channels, int top_num_channels,
                  int bottom_height, int bottom_width, int pad_height, int pad_width,
                  int stride_vertical, int stride_horizontal, int filter_height,
-                 int filter_width, mnv_stream_t stream);
+                 int filter_width, void* workspace, size_t workspace_bytes,
+                 mnv_stream_t stream);
+size_t mnv_conv_bwd_data_workspace_bytes(int num_images, int bottom_num_channels,
+                                        int top_num_channels, int bottom_height,
+                                        int bottom_width, int pad_height, int pad_width,
+                                        int stride_vertical, int stride_horizontal,
+                                        int filter_height, int filter_width);
 int mnv_conv_bwd_data(const float* top_diff, const float* filter, float* bottom_diff,
                       int num_images, int bottom_num_channels, int top_num_channels,
                       int bottom_height, int bottom_width, int pad_height, int pad_width,
                       int stride_vertical, int stride_horizontal, int filter_height,
-                      int filter_width, mnv_stream_t stream);
+                      int filter_width, void* workspace, size_t workspace_bytes,
+                      mnv_stream_t stream);
 size_t mnv_conv_bwd_filter_workspace_bytes(int num_images, int bottom_num_channels,
                                            int top_num_channels, int bottom_height,
                                            int bottom_width, int pad_height, int pad_width,

@@ -49,8 +49,10 @@ PROTOTYPES = {
     "mnv_transpose": [_P, _P, _I, _I, _S],
     "mnv_copy": [_P, _P, c_sz, _S],
     "mnv_fill": [_P, c_sz, c_f, _S],
-    "mnv_conv_fwd": [_P, _P, _P, _P] + [_I] * 11 + [_S],
-    "mnv_conv_bwd_data": [_P, _P, _P] + [_I] * 11 + [_S],
+    "mnv_conv_fwd_workspace_bytes": [_I] * 11,
+    "mnv_conv_fwd": [_P, _P, _P, _P] + [_I] * 11 + [_P, c_sz, _S],
+    "mnv_conv_bwd_data_workspace_bytes": [_I] * 11,
+    "mnv_conv_bwd_data": [_P, _P, _P] + [_I] * 11 + [_P, c_sz, _S],
     "mnv_conv_bwd_filter_workspace_bytes": [_I] * 11,
     "mnv_conv_bwd_filter": [_P, _P, _P] + [_I] * 11 + [_P, c_sz, _S],
     "mnv_conv_bwd_bias": [_P, _P, _I, _I, _I, _I, _S],
@@ -81,6 +83,8 @@ _RESTYPES = {
     "mnv_error_string": ctypes.c_char_p,
     "mnv_sgemm_nn_workspace_bytes": c_sz,
     "mnv_conv_bwd_filter_workspace_bytes": c_sz,
+    "mnv_conv_fwd_workspace_bytes": c_sz,
+    "mnv_conv_bwd_data_workspace_bytes": c_sz,
 }
 
 

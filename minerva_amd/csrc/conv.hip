@@ -12,6 +12,8 @@
 // In every case the GEMM "m" dimension is the one that is contiguous in the output
 // tensor, so result stores are coalesced, and no im2col buffer exists in HBM.
 // Roofline: fp32 MFMA, 2*N*Ho*Wo*K*C*R*S algorithmic flops per pass.
+#include <stdlib.h>
+
 #include "gemm_core.h"
 
 namespace {
@@ -28,46 +30,63 @@ __device__ __forceinline__ int pack_yx(int y, int x) { return (y << 16) | (x & 0
 __device__ __forceinline__ int unpack_y(int p) { return p >> 16; }
 __device__ __forceinline__ int unpack_x(int p) { return (int)(short)(p & 0xffff); }
 
+// Every policy comes in two addressing flavours (see the contract in gemm_core.h):
+//   FAST   : the reduction index is ordered (filter tap, channel) and a period is one tap,
+//            so the im2col offsets and their bounds tests are computed once per tap and a
+//            slab of 16 channels only advances a uniform scalar offset.  Needs the channel
+//            count of the reduction to be a multiple of 16 (and unit stride for the data
+//            gradient).
+//   generic: the reduction index is the flat (channel, tap) order, one period per slab.
+// The two orders only differ in the order the products are summed.
+
 // ------------------------------------------------------------------ forward
-template <bool VECB>
+template <bool FAST>
 struct ConvFwd {
   static constexpr bool A_KFAST = false, B_KFAST = true;
+  static constexpr int A_NOFF = 4, B_NOFF = FAST ? 1 : 4;
   const float* __restrict__ bottom;
   const float* __restrict__ filter;
   const float* __restrict__ bias;
   float* __restrict__ top;
   ConvGeom g;
-  int M, N, K;  // GEMM extents: N*Ho*Wo, Kout, C*R*S
+  int M, N, K, total_slabs, spp;  // GEMM extents: N*Ho*Wo, Kout, C*R*S
+  struct Res {
+    mnv_rsrc a, b;
+  };
   struct AState {
     int off[4], yx[4];
   };
   struct BState {};
+  __device__ void make_res(Res& r) const {
+    r.a = mnv_make_rsrc(bottom, (unsigned)(g.N * g.C * g.HW) * 4u);
+    r.b = mnv_make_rsrc(filter, (unsigned)(g.K * g.CRS) * 4u);
+  }
   __device__ void a_init(AState& st, int m) const {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       int mm = m + q;
-      if (mm < M) {
-        int img = mnv_fastdiv(mm, g.d_HoWo);
-        int pos = mm - img * g.HoWo;
-        int i = mnv_fastdiv(pos, g.d_Wo);
-        int j = pos - i * g.Wo;
-        int y0 = i * g.sv - g.ph, x0 = j * g.sh - g.pw;
-        st.off[q] = img * g.C * g.HW + y0 * g.W + x0;
-        st.yx[q] = pack_yx(y0, x0);
-      } else {
-        st.off[q] = 0;
-        st.yx[q] = pack_yx(MNV_FAR, MNV_FAR);
-      }
+      int img = mnv_fastdiv(mm, g.d_HoWo);
+      int pos = mm - img * g.HoWo;
+      int i = mnv_fastdiv(pos, g.d_Wo);
+      int j = pos - i * g.Wo;
+      int y0 = i * g.sv - g.ph, x0 = j * g.sh - g.pw;
+      st.off[q] = img * g.C * g.HW + y0 * g.W + x0;
+      st.yx[q] = mm < M ? pack_yx(y0, x0) : pack_yx(MNV_FAR, MNV_FAR);
     }
   }
   __device__ void b_init(BState&, int) const {}
-  __device__ void a_fetch(const AState& st, int, int k, float (&v)[4]) const {
-    if (k >= K) {
-      v[0] = v[1] = v[2] = v[3] = 0.f;
-      return;
+  __device__ void a_period(const AState& st, unsigned (&off)[4], int, int kl, int period) const {
+    int c, rs;
+    bool kok = true;
+    if (FAST) {  // period = tap, kl = channel within the slab
+      rs = period;
+      c = kl;
+    } else {  // period = slab, flat k = (c, r', s')
+      int k = period * 16 + kl;
+      kok = k < K;
+      c = mnv_fastdiv(k, g.d_RS);
+      rs = k - c * g.RS;
     }
-    int c = mnv_fastdiv(k, g.d_RS);
-    int rs = k - c * g.RS;
     int rp = mnv_fastdiv(rs, g.d_S);
     int sp = rs - rp * g.S;
     int r = g.R - 1 - rp, s = g.S - 1 - sp;  // flipped tap
@@ -75,23 +94,29 @@ struct ConvFwd {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       int y = unpack_y(st.yx[q]) + r, x = unpack_x(st.yx[q]) + s;
-      bool ok = (unsigned)y < (unsigned)g.H && (unsigned)x < (unsigned)g.W;
-      v[q] = ok ? bottom[st.off[q] + koff] : 0.f;
+      bool ok = kok & ((unsigned)y < (unsigned)g.H) & ((unsigned)x < (unsigned)g.W);
+      off[q] = ok ? (unsigned)(st.off[q] + koff) * 4u : MNV_OOB;
     }
   }
-  __device__ void b_fetch(const BState&, int n, int k, float (&v)[4]) const {
-    if (VECB) {
-      if (n < N && k < K) {
-        mnv_f4 t = *reinterpret_cast<const mnv_f4*>(filter + (size_t)n * K + k);
-        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-      } else {
-        v[0] = v[1] = v[2] = v[3] = 0.f;
-      }
+  __device__ unsigned a_soff(int, int s) const {
+    return FAST ? (unsigned)s * 16u * (unsigned)g.HW * 4u : 0u;
+  }
+  // generic: `filter` is the caller's tensor [n][c][r'][s'], element (k, n) at n*CRS + k.
+  // FAST: `filter` is the permuted copy [n][r's'][c], so the 4 channels of a vector are
+  // one 16-byte load and consecutive slabs are consecutive memory.
+  __device__ void b_period(const BState&, unsigned (&off)[B_NOFF], int n, int kl,
+                           int period) const {
+    if (FAST) {
+      off[0] = (n < N) ? (unsigned)(n * g.CRS + period * g.C + kl) * 4u : MNV_OOB;
     } else {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) v[q] = (n < N && k + q < K) ? filter[(size_t)n * K + k + q] : 0.f;
+      for (int q = 0; q < B_NOFF; ++q) {
+        int k = period * 16 + kl + q;
+        off[q] = ((n < N) & (k < K)) ? (unsigned)(n * K + k) * 4u : MNV_OOB;
+      }
     }
   }
+  __device__ unsigned b_soff(int, int s) const { return FAST ? (unsigned)s * 64u : 0u; }
   __device__ void c_store(int m, int n, float x) const {
     int img = mnv_fastdiv(m, g.d_HoWo);
     int pos = m - img * g.HoWo;
@@ -100,70 +125,95 @@ struct ConvFwd {
 };
 
 // ------------------------------------------------------------ backward data
+// FAST additionally means both strides are 1, so every (row, col) of the shifted window
+// is a real output position.
+template <bool FAST>
 struct ConvBwdData {
   static constexpr bool A_KFAST = false, B_KFAST = true;
+  static constexpr int A_NOFF = 4, B_NOFF = FAST ? 1 : 4;
   const float* __restrict__ top_diff;
   const float* __restrict__ filter;
   float* __restrict__ bottom_diff;
   ConvGeom g;
-  int M, N, K;  // N*H*W, C, Kout*R*S
+  int M, N, K, total_slabs, spp;  // N*H*W, C, Kout*R*S
+  struct Res {
+    mnv_rsrc a, b;
+  };
   struct AState {
     int off[4], yx[4];  // image offset into top_diff; (y+ph-R+1, x+pw-S+1)
   };
   struct BState {};
+  __device__ void make_res(Res& r) const {
+    r.a = mnv_make_rsrc(top_diff, (unsigned)(g.N * g.K * g.HoWo) * 4u);
+    r.b = mnv_make_rsrc(filter, (unsigned)(g.K * g.CRS) * 4u);
+  }
   __device__ void a_init(AState& st, int m) const {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       int mm = m + q;
-      if (mm < M) {
-        int img = mnv_fastdiv(mm, g.d_HW);
-        int pos = mm - img * g.HW;
-        int y = mnv_fastdiv(pos, g.d_W);
-        int x = pos - y * g.W;
-        st.off[q] = img * g.K * g.HoWo;
-        st.yx[q] = pack_yx(y + g.ph - g.R + 1, x + g.pw - g.S + 1);
-      } else {
-        st.off[q] = 0;
-        st.yx[q] = pack_yx(MNV_FAR, MNV_FAR);
-      }
+      int img = mnv_fastdiv(mm, g.d_HW);
+      int pos = mm - img * g.HW;
+      int y = mnv_fastdiv(pos, g.d_W);
+      int x = pos - y * g.W;
+      int ty0 = y + g.ph - g.R + 1, tx0 = x + g.pw - g.S + 1;
+      st.off[q] = img * g.K * g.HoWo + (FAST ? ty0 * g.Wo + tx0 : 0);
+      st.yx[q] = mm < M ? pack_yx(ty0, tx0) : pack_yx(MNV_FAR, MNV_FAR);
     }
   }
   __device__ void b_init(BState&, int) const {}
-  __device__ void a_fetch(const AState& st, int, int k, float (&v)[4]) const {
-    if (k >= K) {
-      v[0] = v[1] = v[2] = v[3] = 0.f;
-      return;
-    }
-    int ko = mnv_fastdiv(k, g.d_RS);
-    int rs = k - ko * g.RS;
-    int rp = mnv_fastdiv(rs, g.d_S);
-    int sp = rs - rp * g.S;
-    int koff = ko * g.HoWo;
+  __device__ void a_period(const AState& st, unsigned (&off)[4], int, int kl, int period) const {
+    if (FAST) {  // period = tap (r', s'), kl = output channel within the slab
+      int rp = mnv_fastdiv(period, g.d_S);
+      int sp = period - rp * g.S;
+      int koff = kl * g.HoWo + rp * g.Wo + sp;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      int ty = unpack_y(st.yx[q]) + rp, tx = unpack_x(st.yx[q]) + sp;
-      float val = 0.f;
-      if (ty >= 0 && tx >= 0) {
-        int i = mnv_fastdiv(ty, g.d_sv), j = mnv_fastdiv(tx, g.d_sh);
-        if (i * g.sv == ty && j * g.sh == tx && i < g.Ho && j < g.Wo)
-          val = top_diff[st.off[q] + koff + i * g.Wo + j];
+      for (int q = 0; q < 4; ++q) {
+        int i = unpack_y(st.yx[q]) + rp, j = unpack_x(st.yx[q]) + sp;
+        bool ok = ((unsigned)i < (unsigned)g.Ho) & ((unsigned)j < (unsigned)g.Wo);
+        off[q] = ok ? (unsigned)(st.off[q] + koff) * 4u : MNV_OOB;
       }
-      v[q] = val;
-    }
-  }
-  // B[kk, c] = filter[ko, c, r', s'] for kk = (ko, r', s')
-  __device__ void b_fetch(const BState&, int n, int k, float (&v)[4]) const {
-    int ko = mnv_fastdiv(k, g.d_RS);
-    int rs = k - ko * g.RS;
+    } else {  // flat k = (ko, r', s')
+      int k = period * 16 + kl;
+      int ko = mnv_fastdiv(k, g.d_RS);
+      int rs = k - ko * g.RS;
+      int rp = mnv_fastdiv(rs, g.d_S);
+      int sp = rs - rp * g.S;
+      int koff = ko * g.HoWo;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      v[q] = (n < N && k + q < K) ? filter[(size_t)ko * g.CRS + n * g.RS + rs] : 0.f;
-      if (++rs == g.RS) {
-        rs = 0;
-        ++ko;
+      for (int q = 0; q < 4; ++q) {
+        int ty = unpack_y(st.yx[q]) + rp, tx = unpack_x(st.yx[q]) + sp;
+        int tyc = ty < 0 ? 0 : ty, txc = tx < 0 ? 0 : tx;
+        int i = mnv_fastdiv(tyc, g.d_sv), j = mnv_fastdiv(txc, g.d_sh);
+        bool ok = (k < K) & (ty >= 0) & (tx >= 0) & (i * g.sv == ty) & (j * g.sh == tx) &
+                  (i < g.Ho) & (j < g.Wo);
+        off[q] = ok ? (unsigned)(st.off[q] + koff + i * g.Wo + j) * 4u : MNV_OOB;
       }
     }
   }
+  __device__ unsigned a_soff(int, int s) const {
+    return FAST ? (unsigned)s * 16u * (unsigned)g.HoWo * 4u : 0u;
+  }
+  // B[kk, c] = filter[ko, c, r', s'].  FAST reads the permuted copy [c][r's'][ko].
+  __device__ void b_period(const BState&, unsigned (&off)[B_NOFF], int n, int kl,
+                           int period) const {
+    if (FAST) {
+      off[0] = (n < N) ? (unsigned)((n * g.RS + period) * g.K + kl) * 4u : MNV_OOB;
+    } else {
+      int k = period * 16 + kl;
+      int ko = mnv_fastdiv(k, g.d_RS);
+      int rs = k - ko * g.RS;
+#pragma unroll
+      for (int q = 0; q < B_NOFF; ++q) {
+        bool ok = (n < N) & (k + q < K);
+        off[q] = ok ? (unsigned)(ko * g.CRS + n * g.RS + rs) * 4u : MNV_OOB;
+        ++rs;
+        bool wrap = rs == g.RS;
+        rs = wrap ? 0 : rs;
+        ko += wrap ? 1 : 0;
+      }
+    }
+  }
+  __device__ unsigned b_soff(int, int s) const { return FAST ? (unsigned)s * 64u : 0u; }
   __device__ void c_store(int m, int n, float x) const {
     int img = mnv_fastdiv(m, g.d_HW);
     int pos = m - img * g.HW;
@@ -174,32 +224,36 @@ struct ConvBwdData {
 // ---------------------------------------------------------- backward filter
 struct ConvBwdFilter {
   static constexpr bool A_KFAST = true, B_KFAST = true;
+  static constexpr int A_NOFF = 4, B_NOFF = 4;
   const float* __restrict__ bottom;
   const float* __restrict__ top_diff;
   float* __restrict__ filter_diff;
   ConvGeom g;
-  int M, N, K;  // C*R*S, Kout, N*Ho*Wo
+  int M, N, K, total_slabs, spp;  // C*R*S, Kout, N*Ho*Wo
+  struct Res {
+    mnv_rsrc a, b;
+  };
   struct AState {
     int off, dyx;  // c*H*W + dy*W + dx ; (dy, dx) = (R-1-r'-ph, S-1-s'-pw)
   };
   struct BState {};
+  __device__ void make_res(Res& r) const {
+    r.a = mnv_make_rsrc(bottom, (unsigned)(g.N * g.C * g.HW) * 4u);
+    r.b = mnv_make_rsrc(top_diff, (unsigned)(g.N * g.K * g.HoWo) * 4u);
+  }
   __device__ void a_init(AState& st, int m) const {
-    if (m < M) {
-      int c = mnv_fastdiv(m, g.d_RS);
-      int rs = m - c * g.RS;
-      int rp = mnv_fastdiv(rs, g.d_S);
-      int sp = rs - rp * g.S;
-      int dy = g.R - 1 - rp - g.ph, dx = g.S - 1 - sp - g.pw;
-      st.off = c * g.HW + dy * g.W + dx;
-      st.dyx = pack_yx(dy, dx);
-    } else {
-      st.off = 0;
-      st.dyx = pack_yx(MNV_FAR, MNV_FAR);
-    }
+    int c = mnv_fastdiv(m, g.d_RS);
+    int rs = m - c * g.RS;
+    int rp = mnv_fastdiv(rs, g.d_S);
+    int sp = rs - rp * g.S;
+    int dy = g.R - 1 - rp - g.ph, dx = g.S - 1 - sp - g.pw;
+    st.off = c * g.HW + dy * g.W + dx;
+    st.dyx = m < M ? pack_yx(dy, dx) : pack_yx(MNV_FAR, MNV_FAR);
   }
   __device__ void b_init(BState&, int) const {}
   // A[m, kk..kk+3] = bottom[img, c, i*sv + dy, j*sh + dx] for kk = (img, i, j)
-  __device__ void a_fetch(const AState& st, int, int k, float (&v)[4]) const {
+  __device__ void a_period(const AState& st, unsigned (&off)[4], int, int kl, int period) const {
+    int k = period * 16 + kl;
     int img = mnv_fastdiv(k, g.d_HoWo);
     int pos = k - img * g.HoWo;
     int i = mnv_fastdiv(pos, g.d_Wo);
@@ -208,35 +262,88 @@ struct ConvBwdFilter {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       int y = i * g.sv + dy, x = j * g.sh + dx;
-      bool ok = (k + q < K) && (unsigned)y < (unsigned)g.H && (unsigned)x < (unsigned)g.W;
-      v[q] = ok ? bottom[img * g.C * g.HW + st.off + i * g.sv * g.W + j * g.sh] : 0.f;
-      if (++j == g.Wo) {
-        j = 0;
-        if (++i == g.Ho) {
-          i = 0;
-          ++img;
-        }
-      }
+      bool ok = (k + q < K) & ((unsigned)y < (unsigned)g.H) & ((unsigned)x < (unsigned)g.W);
+      unsigned o = (unsigned)(img * g.C * g.HW + st.off + i * g.sv * g.W + j * g.sh) * 4u;
+      off[q] = ok ? o : MNV_OOB;
+      ++j;
+      bool wj = j == g.Wo;
+      j = wj ? 0 : j;
+      i += wj ? 1 : 0;
+      bool wi = i == g.Ho;
+      i = wi ? 0 : i;
+      img += wi ? 1 : 0;
     }
   }
+  __device__ unsigned a_soff(int, int) const { return 0u; }
   // B[kk..kk+3, ko] = top_diff[img, ko, i, j]
-  __device__ void b_fetch(const BState&, int n, int k, float (&v)[4]) const {
+  __device__ void b_period(const BState&, unsigned (&off)[4], int n, int kl, int period) const {
+    int k = period * 16 + kl;
     int img = mnv_fastdiv(k, g.d_HoWo);
     int pos = k - img * g.HoWo;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      v[q] = (n < N && k + q < K) ? top_diff[((size_t)img * N + n) * g.HoWo + pos] : 0.f;
-      if (++pos == g.HoWo) {
-        pos = 0;
-        ++img;
-      }
+      bool ok = (n < N) & (k + q < K);
+      off[q] = ok ? (unsigned)((img * N + n) * g.HoWo + pos) * 4u : MNV_OOB;
+      ++pos;
+      bool wrap = pos == g.HoWo;
+      pos = wrap ? 0 : pos;
+      img += wrap ? 1 : 0;
     }
   }
+  __device__ unsigned b_soff(int, int) const { return 0u; }
   __device__ void c_store(int m, int n, float x) const { filter_diff[(size_t)n * M + m] = x; }
 };
 
+// Filter permutations for the FAST policies (a few MB at most, one pass):
+//   to_rsc: out[k][r's'][c] = in[k][c][r's']      (forward)
+//   to_crk: out[c][r's'][k] = in[k][c][r's']      (data gradient)
+__global__ __launch_bounds__(256) void mnv_filter_permute_kernel(const float* __restrict__ in,
+                                                                 float* __restrict__ out, int K,
+                                                                 int C, int RS, bool to_crk) {
+  const int total = K * C * RS;
+  for (int o = blockIdx.x * 256 + threadIdx.x; o < total; o += gridDim.x * 256) {
+    int k, c, rs;
+    if (to_crk) {
+      k = o % K;
+      rs = (o / K) % RS;
+      c = o / (K * RS);
+    } else {
+      c = o % C;
+      rs = (o / C) % RS;
+      k = o / (C * RS);
+    }
+    out[o] = in[(k * C + c) * RS + rs];
+  }
+}
+
+int permute_filter(const float* in, float* out, int K, int C, int RS, bool to_crk, hipStream_t s) {
+  int total = K * C * RS;
+  int blocks = (total + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(mnv_filter_permute_kernel, dim3(blocks), dim3(256), 0, s, in, out, K, C, RS,
+                     to_crk);
+  return MNV_LAUNCH_STATUS();
+}
+
 typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
+typedef MnvGemmTile<128, 256, 16, 2, 4> TileWide8;   // 8 wavefronts of 64x64
+typedef MnvGemmTile<128, 256, 16, 2, 2> TileWide4;   // 4 wavefronts of 64x128
+typedef MnvGemmTile<256, 128, 16, 4, 2> TileTall8;
+typedef MnvGemmTile<256, 128, 16, 2, 2> TileTall4;
+
+template <class P>
+int launch_tile(int tile, const P& p, int splits, void* ws, hipStream_t s) {
+  if (const char* e = getenv("MNV_CONV_TILE")) tile = atoi(e);
+  switch (tile) {
+    case 0: return mnv_gemm_launch<TileSmall>(p, splits, ws, s);
+    case 2: return mnv_gemm_launch<TileWide8>(p, splits, ws, s);
+    case 3: return mnv_gemm_launch<TileWide4>(p, splits, ws, s);
+    case 4: return mnv_gemm_launch<TileTall8>(p, splits, ws, s);
+    case 5: return mnv_gemm_launch<TileTall4>(p, splits, ws, s);
+    default: return mnv_gemm_launch<TileBig>(p, splits, ws, s);
+  }
+}
 
 int make_geom(ConvGeom* g, int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh,
               int R, int S) {
@@ -247,7 +354,7 @@ int make_geom(ConvGeom* g, int N, int C, int K, int H, int W, int ph, int pw, in
   if (H + 2 * ph < R || W + 2 * pw < S || Ho <= 0 || Wo <= 0) return MNV_ERR_INVALID;
   // 16-bit packed coordinates and 32-bit element offsets
   if (H + ph + R >= 16000 || W + pw + S >= 16000) return MNV_ERR_INVALID;
-  const long long lim = 0x7fffffffLL;
+  const long long lim = (1LL << 29) - 1;  // 32-bit byte offsets into each tensor
   if ((long long)N * C * H * W > lim || (long long)N * K * Ho * Wo > lim ||
       (long long)K * C * R * S > lim)
     return MNV_ERR_INVALID;
@@ -272,8 +379,12 @@ bool small_tiles(int m, int n) {
 
 #define MNV_BWDF_MAX_SPLITS 256
 
+// The filter gradient gets its parallelism from splitting the long N*Ho*Wo reduction,
+// so it keeps the 128x128 tile (twice the operand reuse) unless the output is tiny.
+bool bwd_filter_small_tiles(int m, int n) { return m <= 64 || n <= 64; }
+
 int bwd_filter_splits(int m, int n, int k, size_t ws_floats) {
-  bool small = small_tiles(m, n);
+  bool small = bwd_filter_small_tiles(m, n);
   int bm = small ? 64 : 128;
   long long tiles = (long long)((m + bm - 1) / bm) * ((n + bm - 1) / bm);
   int slabs = (k + 15) / 16;
@@ -289,39 +400,61 @@ int bwd_filter_splits(int m, int n, int k, size_t ws_floats) {
 
 extern "C" {
 
+size_t mnv_conv_fwd_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw, int sv,
+                                   int sh, int R, int S) {
+  ConvGeom g;
+  if (make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S)) return 0;
+  return C % 16 == 0 ? (size_t)K * g.CRS * sizeof(float) : 0;
+}
+
 int mnv_conv_fwd(const float* bottom, const float* filter, const float* bias, float* top, int N,
                  int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S,
-                 mnv_stream_t stream) {
+                 void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
   ConvGeom g;
   if (!bottom || !filter || !bias || !top) return MNV_ERR_INVALID;
   int rc = make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S);
   if (rc) return rc;
   int gm = N * g.HoWo, gn = K, gk = g.CRS;
   hipStream_t s = mnv_stream(stream);
-  bool vecb = (gk % 4 == 0) && mnv_aligned16(filter);
-  bool small = small_tiles(gm, gn);
-  if (vecb) {
-    ConvFwd<true> p{bottom, filter, bias, top, g, gm, gn, gk};
-    return small ? mnv_gemm_launch<TileSmall>(p, 1, nullptr, s)
-                 : mnv_gemm_launch<TileBig>(p, 1, nullptr, s);
+  const int tile = small_tiles(gm, gn) ? 0 : 1;
+  if (C % 16 == 0 && workspace && workspace_bytes >= (size_t)K * g.CRS * sizeof(float)) {
+    float* wp = static_cast<float*>(workspace);
+    rc = permute_filter(filter, wp, K, C, g.RS, false, s);
+    if (rc) return rc;
+    ConvFwd<true> p{bottom, wp, bias, top, g, gm, gn, gk, g.RS * (C / 16), C / 16};
+    return launch_tile(tile, p, 1, nullptr, s);
   }
-  ConvFwd<false> p{bottom, filter, bias, top, g, gm, gn, gk};
-  return small ? mnv_gemm_launch<TileSmall>(p, 1, nullptr, s)
-               : mnv_gemm_launch<TileBig>(p, 1, nullptr, s);
+  ConvFwd<false> p{bottom, filter, bias, top, g, gm, gn, gk, (gk + 15) / 16, 1};
+  return launch_tile(tile, p, 1, nullptr, s);
+}
+
+size_t mnv_conv_bwd_data_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw,
+                                        int sv, int sh, int R, int S) {
+  ConvGeom g;
+  if (make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S)) return 0;
+  return (sv == 1 && sh == 1 && K % 16 == 0) ? (size_t)K * g.CRS * sizeof(float) : 0;
 }
 
 int mnv_conv_bwd_data(const float* top_diff, const float* filter, float* bottom_diff, int N,
                       int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S,
-                      mnv_stream_t stream) {
+                      void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
   ConvGeom g;
   if (!top_diff || !filter || !bottom_diff) return MNV_ERR_INVALID;
   int rc = make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S);
   if (rc) return rc;
   int gm = N * g.HW, gn = C, gk = K * g.RS;
-  ConvBwdData p{top_diff, filter, bottom_diff, g, gm, gn, gk};
   hipStream_t s = mnv_stream(stream);
-  return small_tiles(gm, gn) ? mnv_gemm_launch<TileSmall>(p, 1, nullptr, s)
-                             : mnv_gemm_launch<TileBig>(p, 1, nullptr, s);
+  const int tile = small_tiles(gm, gn) ? 0 : 1;
+  if (sv == 1 && sh == 1 && K % 16 == 0 && workspace &&
+      workspace_bytes >= (size_t)K * g.CRS * sizeof(float)) {
+    float* wq = static_cast<float*>(workspace);
+    rc = permute_filter(filter, wq, K, C, g.RS, true, s);
+    if (rc) return rc;
+    ConvBwdData<true> p{top_diff, wq, bottom_diff, g, gm, gn, gk, g.RS * (K / 16), K / 16};
+    return launch_tile(tile, p, 1, nullptr, s);
+  }
+  ConvBwdData<false> p{top_diff, filter, bottom_diff, g, gm, gn, gk, (gk + 15) / 16, 1};
+  return launch_tile(tile, p, 1, nullptr, s);
 }
 
 size_t mnv_conv_bwd_filter_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw,
@@ -340,11 +473,10 @@ int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filte
   int rc = make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S);
   if (rc) return rc;
   int gm = g.CRS, gn = K, gk = N * g.HoWo;
-  ConvBwdFilter p{bottom, top_diff, filter_diff, g, gm, gn, gk};
+  ConvBwdFilter p{bottom, top_diff, filter_diff, g, gm, gn, gk, (gk + 15) / 16, 1};
   hipStream_t s = mnv_stream(stream);
   int splits = bwd_filter_splits(gm, gn, gk, workspace ? workspace_bytes / sizeof(float) : 0);
-  return small_tiles(gm, gn) ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
-                             : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
+  return launch_tile(bwd_filter_small_tiles(gm, gn) ? 0 : 1, p, splits, workspace, s);
 }
 
 }  // extern "C"

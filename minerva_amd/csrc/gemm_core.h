@@ -22,31 +22,43 @@
 
 typedef float mnv_f16v __attribute__((ext_vector_type(16)));
 
-// Division by a run-time constant, prepared on the host (valid for 0 <= n < 2^31).
+// Division by a run-time constant d >= 1, prepared on the host; valid for 0 <= n < 2^31
+// and branch-free (d == 1 gives mul == 0, shift == 0):  n / d == (mulhi(n, mul) + n) >> shift.
 struct MnvFastDiv {
   unsigned mul, shift;
-  int d;
 };
 
 static inline MnvFastDiv mnv_fastdiv_make(int d) {
   MnvFastDiv f;
-  f.d = d;
-  if (d <= 1) {
-    f.mul = 0;
-    f.shift = 0;
-    return f;
-  }
-  unsigned lg = 0;
-  while ((1ull << lg) < (unsigned long long)d) ++lg;  // ceil(log2 d)
-  unsigned p = 31 + lg;
-  f.mul = (unsigned)(((1ull << p) + (unsigned)d - 1) / (unsigned)d);
-  f.shift = p - 32;
+  unsigned s = 0;
+  while ((1ull << s) < (unsigned long long)d) ++s;  // ceil(log2 d)
+  f.shift = s;
+  f.mul = (unsigned)((((1ull << s) - (unsigned long long)d) << 32) / (unsigned long long)d + 1);
+  if (d <= 1) f.mul = 0;
   return f;
 }
 
 #ifdef __HIPCC__
 __device__ __forceinline__ int mnv_fastdiv(int n, const MnvFastDiv& f) {
-  return f.d == 1 ? n : (int)(__umulhi((unsigned)n, f.mul) >> f.shift);
+  return (int)((__umulhi((unsigned)n, f.mul) + (unsigned)n) >> f.shift);
+}
+
+// Buffer addressing: every operand is read through a raw buffer resource whose extent is
+// the tensor's byte size, so a masked-off element is fetched with an offset past the end
+// and the hardware returns 0 for it: no divergent branch, no address clamp, no fault.
+// Operands are therefore limited to 2^31 - 1 bytes.
+#define MNV_OOB 0x80000000u
+typedef __amdgpu_buffer_rsrc_t mnv_rsrc;
+
+__device__ __forceinline__ mnv_rsrc mnv_make_rsrc(const float* p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ float mnv_buf_load(mnv_rsrc r, unsigned byte_off) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0));
+}
+__device__ __forceinline__ void mnv_buf_load4(mnv_rsrc r, unsigned byte_off, float (&v)[4]) {
+  mnv_f4 t = __builtin_bit_cast(mnv_f4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0));
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
 }
 
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int PAD_ = 0>
@@ -59,6 +71,10 @@ struct MnvGemmTile {
   static constexpr int AV = BM * BK / (4 * NT);  // 4-vectors of A per thread per slab
   static constexpr int BV = BN * BK / (4 * NT);
   static constexpr size_t LDS_BYTES = (size_t)2 * BK * (LDA + LDB) * sizeof(float);
+  // Wavefronts per SIMD the register allocation must allow: four 4-wavefront workgroups
+  // per CU make 1024 resident tiles, which lets tile counts just under a multiple of
+  // 1024 finish in whole rounds.
+  static constexpr int MIN_WAVES = (NT == 256 && BM * BN <= 128 * 128) ? 4 : 1;
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
   static_assert(BK % 4 == 0 && (BM * BK) % (4 * NT) == 0 && (BN * BK) % (4 * NT) == 0, "tile/thread mismatch");
 };
@@ -76,18 +92,43 @@ struct MnvFetchMap {
   __device__ static int k(int tid, int p) { return KFAST ? (tid % GK) * 4 : (tid / GX + p * RP); }
 };
 
-// Problem policy contract (all __device__):
+// Problem policy contract (all __device__ unless noted).  The k dimension is cut into
+// slabs of BK and the slabs into "periods" of `spp` consecutive slabs: within a period
+// every thread's byte offsets into A and B are constant and only a wavefront-uniform
+// scalar offset advances, so a slab costs no address arithmetic at all (fp32 MFMA and
+// VALU instructions do not overlap on gfx950: every VALU instruction in the main loop is
+// matrix-pipe time lost).  Offsets are recomputed once per period.  A policy whose
+// addressing has no such structure uses spp = 1.
 //   static constexpr bool A_KFAST, B_KFAST;
-//   struct AState / BState;                          per-thread, per-fetch-vector state
-//   void a_init(AState&, int x /*m, global*/) const;   called once per vector slot
-//   void a_fetch(const AState&, int m, int k, float (&v)[4]) const;   zero-fills out of range
+//   static constexpr int A_NOFF, B_NOFF;      1: one 16-byte load per vector; 4: four 4-byte loads
+//   int M, N, total_slabs, spp;               (host-set members)
+//   struct Res;  void make_res(Res&) const;   buffer resources
+//   struct AState / BState;                   per-thread, per-vector state set once
+//   void a_init(AState&, int m) const;
+//   void a_period(const AState&, unsigned (&off)[A_NOFF], int m, int kl, int period) const;
+//        byte offsets of this vector's elements for slab 0 of `period`; kl = the vector's
+//        first k index inside a slab; an element that must read as 0 gets MNV_OOB
+//   unsigned a_soff(int period, int s) const; uniform byte offset of slab s of the period
 //   (same for b with n)
-//   void c_store(int m, int n, float v) const;         only called for m < M, n < N
-//   int M, N, K;
+//   void c_store(int m, int n, float v) const;   only called for m < M, n < N
+template <int NOFF>
+__device__ __forceinline__ void mnv_fetch_vec(mnv_rsrc r, const unsigned (&off)[NOFF],
+                                              unsigned soff, float (&v)[4]) {
+  if (NOFF == 1) {
+    mnv_f4 t = __builtin_bit_cast(
+        mnv_f4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off[0], (int)soff, 0));
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  } else {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      v[q] = __builtin_bit_cast(
+          float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)off[q % NOFF], (int)soff, 0));
+  }
+}
+
 template <class T, class P>
-__global__ __launch_bounds__(T::NT) void mnv_gemm_kernel(P prob, int tiles_m, int tiles_n,
-                                                         int slabs_per_split,
-                                                         float* __restrict__ partial) {
+__global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
+    P prob, int tiles_m, int tiles_n, int slabs_per_split, float* __restrict__ partial) {
   extern __shared__ float mnv_gemm_lds[];
   float* As = mnv_gemm_lds;                       // [2][BK][LDA]
   float* Bs = mnv_gemm_lds + 2 * T::BK * T::LDA;  // [2][BK][LDB]
@@ -104,13 +145,15 @@ __global__ __launch_bounds__(T::NT) void mnv_gemm_kernel(P prob, int tiles_m, in
   const int tile_m = b % tiles_m, tile_n = b / tiles_m;
   const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
 
-  const int total_slabs = (prob.K + T::BK - 1) / T::BK;
   const int slab_begin = blockIdx.z * slabs_per_split;
   int slab_end = slab_begin + slabs_per_split;
-  if (slab_end > total_slabs) slab_end = total_slabs;
+  if (slab_end > prob.total_slabs) slab_end = prob.total_slabs;
 
+  typename P::Res res;
+  prob.make_res(res);
   typename P::AState ast[T::AV];
   typename P::BState bst[T::BV];
+  unsigned aoff[T::AV][P::A_NOFF], boff[T::BV][P::B_NOFF];
 #pragma unroll
   for (int p = 0; p < T::AV; ++p) prob.a_init(ast[p], m0 + MapA::x(tid, p));
 #pragma unroll
@@ -118,14 +161,20 @@ __global__ __launch_bounds__(T::NT) void mnv_gemm_kernel(P prob, int tiles_m, in
 
   float ra[T::AV][4], rb[T::BV][4];
 
-  auto fetch = [&](int slab) {
-    const int k0 = slab * T::BK;
+  auto new_period = [&](int period) {
 #pragma unroll
     for (int p = 0; p < T::AV; ++p)
-      prob.a_fetch(ast[p], m0 + MapA::x(tid, p), k0 + MapA::k(tid, p), ra[p]);
+      prob.a_period(ast[p], aoff[p], m0 + MapA::x(tid, p), MapA::k(tid, p), period);
 #pragma unroll
     for (int p = 0; p < T::BV; ++p)
-      prob.b_fetch(bst[p], n0 + MapB::x(tid, p), k0 + MapB::k(tid, p), rb[p]);
+      prob.b_period(bst[p], boff[p], n0 + MapB::x(tid, p), MapB::k(tid, p), period);
+  };
+  auto fetch = [&](int period, int s) {
+    const unsigned sa = prob.a_soff(period, s), sb = prob.b_soff(period, s);
+#pragma unroll
+    for (int p = 0; p < T::AV; ++p) mnv_fetch_vec<P::A_NOFF>(res.a, aoff[p], sa, ra[p]);
+#pragma unroll
+    for (int p = 0; p < T::BV; ++p) mnv_fetch_vec<P::B_NOFF>(res.b, boff[p], sb, rb[p]);
   };
   auto stash = [&](int buf) {
     float* a = As + buf * T::BK * T::LDA;
@@ -166,16 +215,25 @@ __global__ __launch_bounds__(T::NT) void mnv_gemm_kernel(P prob, int tiles_m, in
   const int wm = (wave % T::WGM) * T::WM, wn = (wave / T::WGM) * T::WN;
   const int lm = lane % 32, lk = lane / 32;
 
+  // (period, s) of the slab whose loads are issued next
+  int period = slab_begin / prob.spp, s = slab_begin - period * prob.spp;
   if (slab_begin < slab_end) {
-    fetch(slab_begin);
+    new_period(period);
+    fetch(period, s);
     stash(0);
   }
   __syncthreads();
 
   for (int slab = slab_begin; slab < slab_end; ++slab) {
     const int buf = (slab - slab_begin) & 1;
-    const bool more = slab + 1 < slab_end;
-    if (more) fetch(slab + 1);  // global loads in flight while this slab is multiplied
+    // Loads of the next slab are in flight while this one is multiplied.  Past the end of
+    // the k range the loads run past the tensors and read as 0 (or fetch a slab of the
+    // next split, which is never multiplied).
+    if (++s == prob.spp) {
+      s = 0;
+      new_period(++period);
+    }
+    fetch(period, s);
     const float* a = As + buf * T::BK * T::LDA + wm + lm;
     const float* bb = Bs + buf * T::BK * T::LDB + wn + lm;
 #pragma unroll
@@ -191,7 +249,7 @@ __global__ __launch_bounds__(T::NT) void mnv_gemm_kernel(P prob, int tiles_m, in
         for (int j = 0; j < T::TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[i][j], 0, 0, 0);
     }
-    if (more) stash(buf ^ 1);
+    stash(buf ^ 1);
     __syncthreads();
   }
 
@@ -235,7 +293,7 @@ __global__ __launch_bounds__(256) void mnv_gemm_splitk_reduce_kernel(P prob,
 template <class T, class P>
 static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream_t s) {
   const int tiles_m = (prob.M + T::BM - 1) / T::BM, tiles_n = (prob.N + T::BN - 1) / T::BN;
-  const int total_slabs = (prob.K + T::BK - 1) / T::BK;
+  const int total_slabs = prob.total_slabs;
   if (splits < 1) splits = 1;
   if (splits > total_slabs) splits = total_slabs > 0 ? total_slabs : 1;
   int per = (total_slabs + splits - 1) / splits;

@@ -8,47 +8,55 @@
 
 namespace {
 
+// Period 0 holds every full 16-deep slab: the per-thread byte offsets are fixed and only
+// the uniform slab offset moves.  A k extent that is not a multiple of 16 leaves one
+// partial slab, which is period 1 and gets its own masked offsets.
 template <bool VEC>
 struct SgemmNN {
   static constexpr bool A_KFAST = false, B_KFAST = true;
+  static constexpr int A_NOFF = VEC ? 1 : 4, B_NOFF = VEC ? 1 : 4;
   const float* __restrict__ A;
   const float* __restrict__ B;
   float* __restrict__ C;
-  int M, N, K;
+  int M, N, K, total_slabs, spp;
+  struct Res {
+    mnv_rsrc a, b;
+  };
   struct AState {};
   struct BState {};
+  __device__ void make_res(Res& r) const {
+    r.a = mnv_make_rsrc(A, (unsigned)M * (unsigned)K * 4u);
+    r.b = mnv_make_rsrc(B, (unsigned)K * (unsigned)N * 4u);
+  }
   __device__ void a_init(AState&, int) const {}
   __device__ void b_init(BState&, int) const {}
-  // A[m..m+3, k]
-  __device__ void a_fetch(const AState&, int m, int k, float (&v)[4]) const {
-    if (VEC) {
-      if (m < M && k < K) {
-        mnv_f4 t = *reinterpret_cast<const mnv_f4*>(A + (size_t)k * M + m);
-        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-      } else {
-        v[0] = v[1] = v[2] = v[3] = 0.f;
-      }
-    } else {
+  // A[m..m+3, k]: x-fast
+  __device__ void a_period(const AState&, unsigned (&off)[A_NOFF], int m, int kl, int period) const {
+    const int k = period * spp * 16 + kl;
+    const unsigned base = ((unsigned)k * (unsigned)M + (unsigned)m) * 4u;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) v[q] = (m + q < M && k < K) ? A[(size_t)k * M + m + q] : 0.f;
-    }
+    for (int q = 0; q < A_NOFF; ++q) off[q] = ((m + q < M) & (k < K)) ? base + 4u * q : MNV_OOB;
   }
-  // B[k..k+3, n]
-  __device__ void b_fetch(const BState&, int n, int k, float (&v)[4]) const {
-    if (VEC) {
-      if (n < N && k < K) {
-        mnv_f4 t = *reinterpret_cast<const mnv_f4*>(B + (size_t)n * K + k);
-        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-      } else {
-        v[0] = v[1] = v[2] = v[3] = 0.f;
-      }
-    } else {
+  __device__ unsigned a_soff(int, int s) const { return (unsigned)s * 16u * (unsigned)M * 4u; }
+  // B[k..k+3, n]: k-fast
+  __device__ void b_period(const BState&, unsigned (&off)[B_NOFF], int n, int kl, int period) const {
+    const int k = period * spp * 16 + kl;
+    const unsigned base = ((unsigned)n * (unsigned)K + (unsigned)k) * 4u;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) v[q] = (n < N && k + q < K) ? B[(size_t)n * K + k + q] : 0.f;
-    }
+    for (int q = 0; q < B_NOFF; ++q) off[q] = ((n < N) & (k + q < K)) ? base + 4u * q : MNV_OOB;
   }
+  __device__ unsigned b_soff(int, int s) const { return (unsigned)s * 64u; }
   __device__ void c_store(int m, int n, float x) const { C[(size_t)n * M + m] = x; }
 };
+
+template <bool VEC>
+SgemmNN<VEC> make_sgemm(const float* a, const float* b, float* c, int m, int n, int k) {
+  SgemmNN<VEC> p;
+  p.A = a; p.B = b; p.C = c; p.M = m; p.N = n; p.K = k;
+  p.spp = k >= 16 ? k / 16 : 1;
+  p.total_slabs = (k + 15) / 16;
+  return p;
+}
 
 typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
@@ -90,6 +98,8 @@ int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k, 
                  size_t workspace_bytes, mnv_stream_t stream) {
   if (m == 0 || n == 0) return MNV_OK;
   if (!a || !b || !c || m < 0 || n < 0 || k <= 0) return MNV_ERR_INVALID;
+  // operands are addressed through 32-bit buffer offsets: at most 2^31 - 1 bytes each
+  if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
   hipStream_t s = mnv_stream(stream);
   bool vec = (m % 4 == 0) && (k % 4 == 0) && mnv_aligned16(a) && mnv_aligned16(b);
   bool small = use_small_tile(m, n);
@@ -99,11 +109,11 @@ int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k, 
   size_t ws_floats = workspace ? workspace_bytes / sizeof(float) : 0;
   int splits = pick_splits(tiles, slabs, (size_t)m * n, ws_floats);
   if (vec) {
-    SgemmNN<true> p{a, b, c, m, n, k};
+    SgemmNN<true> p = make_sgemm<true>(a, b, c, m, n, k);
     return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
                  : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
   }
-  SgemmNN<false> p{a, b, c, m, n, k};
+  SgemmNN<false> p = make_sgemm<false>(a, b, c, m, n, k);
   return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
                : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
 }

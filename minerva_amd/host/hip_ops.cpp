@@ -248,7 +248,7 @@ void ConvForward(const DataList& inputs, const DataList& outputs, ConvForwardClo
   Ok(mnv_conv_fwd(bottom.data_, filter.data_, bias.data_, top.data_, bottom.size_[3],
                   bottom.size_[2], top.size_[2], bottom.size_[1], bottom.size_[0], c.pad_height,
                   c.pad_width, c.stride_vertical, c.stride_horizontal, filter.size_[1],
-                  filter.size_[0], ctx.stream),
+                  filter.size_[0], ctx.workspace, ctx.workspace_bytes, ctx.stream),
      "conv forward");
 }
 
@@ -264,7 +264,8 @@ void ConvBackwardData(const DataList& inputs, const DataList& outputs,
   Ok(mnv_conv_bwd_data(top_diff.data_, filter.data_, bottom_diff.data_, top_diff.size_[3],
                        bottom_diff.size_[2], top_diff.size_[2], bottom_diff.size_[1],
                        bottom_diff.size_[0], c.pad_height, c.pad_width, c.stride_vertical,
-                       c.stride_horizontal, filter.size_[1], filter.size_[0], ctx.stream),
+                       c.stride_horizontal, filter.size_[1], filter.size_[0], ctx.workspace,
+                       ctx.workspace_bytes, ctx.stream),
      "conv backward data");
 }
 

@@ -35,20 +35,27 @@ class Conv:
         self.gpu, self.p = gpu, (N, C, K, H, W, ph, pw, sv, sh, R, S)
         self.Ho, self.Wo = _out(H, R, sv, ph), _out(W, S, sh, pw)
 
-    def fwd(self, x, w, b):
+    def _ws(self, query, workspace):
+        nbytes = getattr(self.gpu.L, query)(*self.p) if workspace else 0
+        ws = self.gpu.empty(nbytes // 4 + 1) if nbytes else None
+        return (ws.p if ws else None), ctypes.c_size_t(nbytes), ws
+
+    def fwd(self, x, w, b, workspace=True):
         g, p = self.gpu, self.p
         N, C, K = p[0], p[1], p[2]
         dx, dw, db = g.up(x), g.up(w), g.up(b)
         dt = g.empty(N * K * self.Ho * self.Wo)
-        g.call("mnv_conv_fwd", dx.p, dw.p, db.p, dt.p, *p)
+        wp, wb, keep = self._ws("mnv_conv_fwd_workspace_bytes", workspace)
+        g.call("mnv_conv_fwd", dx.p, dw.p, db.p, dt.p, *p, wp, wb)
         return g.down(dt)
 
-    def bwd_data(self, dy, w):
+    def bwd_data(self, dy, w, workspace=True):
         g, p = self.gpu, self.p
         N, C, K, H, W = p[:5]
         ddy, dw = g.up(dy), g.up(w)
         dbd = g.up(np.full(N * C * H * W, np.nan, np.float32))  # every element must be written
-        g.call("mnv_conv_bwd_data", ddy.p, dw.p, dbd.p, *p)
+        wp, wb, keep = self._ws("mnv_conv_bwd_data_workspace_bytes", workspace)
+        g.call("mnv_conv_bwd_data", ddy.p, dw.p, dbd.p, *p, wp, wb)
         return g.down(dbd)
 
     def bwd_filter(self, dy, x, workspace=True):
@@ -99,6 +106,9 @@ CASES = [
     (2, 16, 32, 12, 12, 2, 2, 1, 1, 5, 5),  # same with the reference app's padding
     (5, 130, 70, 9, 9, 1, 1, 1, 1, 3, 3),   # more than one tile in both GEMM dimensions
     (2, 8, 140, 20, 20, 1, 1, 2, 2, 3, 3),
+    (3, 32, 48, 10, 11, 1, 2, 1, 1, 3, 5),  # channel counts that take the (tap, channel) order
+    (2, 16, 16, 9, 9, 2, 2, 1, 1, 5, 5),
+    (2, 48, 32, 12, 12, 1, 1, 2, 1, 3, 3),  # 16-multiple channels but a strided data gradient
 ]
 
 
@@ -108,10 +118,14 @@ def test_conv_all_passes_against_oracle(gpu, ora, p):
     cv = Conv(gpu, *p)
     x, w, b = _rand(N * C * H * W, 40), _rand(K * C * R * S, 41), _rand(K, 42)
     dy = _rand(N * K * cv.Ho * cv.Wo, 43)
-    say("conv fwd", p)
-    assert normwise(cv.fwd(x, w, b), ora.conv_fwd(x, w, b, *p)) <= TOL
-    say("conv bwd data", p)
-    assert normwise(cv.bwd_data(dy, w), ora.conv_bwd_data(dy, w, *p)) <= TOL
+    ref = ora.conv_fwd(x, w, b, *p)
+    for ws in (True, False):
+        say("conv fwd", p, ws)
+        assert normwise(cv.fwd(x, w, b, ws), ref) <= TOL
+    ref = ora.conv_bwd_data(dy, w, *p)
+    for ws in (True, False):
+        say("conv bwd data", p, ws)
+        assert normwise(cv.bwd_data(dy, w, ws), ref) <= TOL
     ref = ora.conv_bwd_filter(dy, x, *p)
     for ws in (True, False):
         say("conv bwd filter", p, ws)

@@ -172,5 +172,5 @@ def test_invalid_arguments_are_rejected(gpu):
     assert L.mnv_norm_add_col(d.p, d.p, d.p, -1, 4, gpu.dev.stream) == -1
     assert L.mnv_reduce_sum_col(d.p, d.p, 0, 4, gpu.dev.stream) == -1
     assert L.mnv_sgemm_nn(d.p, d.p, d.p, 4, 4, 0, None, 0, gpu.dev.stream) == -1
-    assert L.mnv_conv_fwd(d.p, d.p, d.p, d.p, 1, 1, 1, 2, 2, 0, 0, 1, 1, 3, 3, gpu.dev.stream) == -1
+    assert L.mnv_conv_fwd(d.p, d.p, d.p, d.p, 1, 1, 1, 2, 2, 0, 0, 1, 1, 3, 3, None, 0, gpu.dev.stream) == -1
     assert L.mnv_maxpool_fwd(d.p, d.p, 1, 1, 4, 4, 0, 1, 2, 2, 0, 0, gpu.dev.stream) == -1

@@ -222,7 +222,7 @@ TOL_STEP = 5e-4
 def _compare(got, newp, res, grad_tol=TOL):
     for k, v in newp.items():
         assert normwise(got["g_" + k], res["g_" + k]) <= grad_tol, "gradient " + k
-        assert normwise(got[k], v) <= TOL, "updated " + k
+        assert normwise(got[k], v) <= grad_tol, "updated " + k
     assert normwise(got["prob"], res["prob"]) <= TOL
 
 
