@@ -61,7 +61,7 @@ struct ConvFwd {
     r.a = mnv_make_rsrc(bottom, (unsigned)(g.N * g.C * g.HW) * 4u);
     r.b = mnv_make_rsrc(filter, (unsigned)(g.K * g.CRS) * 4u);
   }
-  __device__ void a_init(AState& st, int m) const {
+  __device__ void a_init(const Res& res, AState& st, int m) const {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       int mm = m + q;
@@ -74,7 +74,7 @@ struct ConvFwd {
       st.yx[q] = mm < M ? pack_yx(y0, x0) : pack_yx(MNV_FAR, MNV_FAR);
     }
   }
-  __device__ void b_init(BState&, int) const {}
+  __device__ void b_init(const Res&, BState&, int) const {}
   __device__ void a_period(const AState& st, unsigned (&off)[4], int, int kl, int period) const {
     int c, rs;
     bool kok = true;
@@ -98,9 +98,12 @@ struct ConvFwd {
       off[q] = ok ? (unsigned)(st.off[q] + koff) * 4u : MNV_OOB;
     }
   }
-  __device__ unsigned a_soff(int, int s) const {
-    return FAST ? (unsigned)s * 16u * (unsigned)g.HW * 4u : 0u;
+  __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[4], int, int s, int,
+                         float (&v)[4]) const {
+    mnv_fetch_vec<4>(r.a, off, FAST ? (unsigned)s * 16u * (unsigned)g.HW * 4u : 0u, v);
   }
+  size_t extra_lds_bytes() const { return 0; }
+  __device__ void block_init(Res&, float*, int, int) const {}
   // generic: `filter` is the caller's tensor [n][c][r'][s'], element (k, n) at n*CRS + k.
   // FAST: `filter` is the permuted copy [n][r's'][c], so the 4 channels of a vector are
   // one 16-byte load and consecutive slabs are consecutive memory.
@@ -116,7 +119,10 @@ struct ConvFwd {
       }
     }
   }
-  __device__ unsigned b_soff(int, int s) const { return FAST ? (unsigned)s * 64u : 0u; }
+  __device__ void b_load(const Res& r, const BState&, const unsigned (&off)[B_NOFF], int, int s,
+                         int, float (&v)[4]) const {
+    mnv_fetch_vec<B_NOFF>(r.b, off, FAST ? (unsigned)s * 64u : 0u, v);
+  }
   __device__ void c_store(int m, int n, float x) const {
     int img = mnv_fastdiv(m, g.d_HoWo);
     int pos = m - img * g.HoWo;
@@ -147,7 +153,7 @@ struct ConvBwdData {
     r.a = mnv_make_rsrc(top_diff, (unsigned)(g.N * g.K * g.HoWo) * 4u);
     r.b = mnv_make_rsrc(filter, (unsigned)(g.K * g.CRS) * 4u);
   }
-  __device__ void a_init(AState& st, int m) const {
+  __device__ void a_init(const Res& res, AState& st, int m) const {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       int mm = m + q;
@@ -160,7 +166,7 @@ struct ConvBwdData {
       st.yx[q] = mm < M ? pack_yx(ty0, tx0) : pack_yx(MNV_FAR, MNV_FAR);
     }
   }
-  __device__ void b_init(BState&, int) const {}
+  __device__ void b_init(const Res&, BState&, int) const {}
   __device__ void a_period(const AState& st, unsigned (&off)[4], int, int kl, int period) const {
     if (FAST) {  // period = tap (r', s'), kl = output channel within the slab
       int rp = mnv_fastdiv(period, g.d_S);
@@ -190,9 +196,12 @@ struct ConvBwdData {
       }
     }
   }
-  __device__ unsigned a_soff(int, int s) const {
-    return FAST ? (unsigned)s * 16u * (unsigned)g.HoWo * 4u : 0u;
+  __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[4], int, int s, int,
+                         float (&v)[4]) const {
+    mnv_fetch_vec<4>(r.a, off, FAST ? (unsigned)s * 16u * (unsigned)g.HoWo * 4u : 0u, v);
   }
+  size_t extra_lds_bytes() const { return 0; }
+  __device__ void block_init(Res&, float*, int, int) const {}
   // B[kk, c] = filter[ko, c, r', s'].  FAST reads the permuted copy [c][r's'][ko].
   __device__ void b_period(const BState&, unsigned (&off)[B_NOFF], int n, int kl,
                            int period) const {
@@ -213,7 +222,10 @@ struct ConvBwdData {
       }
     }
   }
-  __device__ unsigned b_soff(int, int s) const { return FAST ? (unsigned)s * 64u : 0u; }
+  __device__ void b_load(const Res& r, const BState&, const unsigned (&off)[B_NOFF], int, int s,
+                         int, float (&v)[4]) const {
+    mnv_fetch_vec<B_NOFF>(r.b, off, FAST ? (unsigned)s * 64u : 0u, v);
+  }
   __device__ void c_store(int m, int n, float x) const {
     int img = mnv_fastdiv(m, g.d_HW);
     int pos = m - img * g.HW;
@@ -241,7 +253,7 @@ struct ConvBwdFilter {
     r.a = mnv_make_rsrc(bottom, (unsigned)(g.N * g.C * g.HW) * 4u);
     r.b = mnv_make_rsrc(top_diff, (unsigned)(g.N * g.K * g.HoWo) * 4u);
   }
-  __device__ void a_init(AState& st, int m) const {
+  __device__ void a_init(const Res& res, AState& st, int m) const {
     int c = mnv_fastdiv(m, g.d_RS);
     int rs = m - c * g.RS;
     int rp = mnv_fastdiv(rs, g.d_S);
@@ -250,7 +262,7 @@ struct ConvBwdFilter {
     st.off = c * g.HW + dy * g.W + dx;
     st.dyx = m < M ? pack_yx(dy, dx) : pack_yx(MNV_FAR, MNV_FAR);
   }
-  __device__ void b_init(BState&, int) const {}
+  __device__ void b_init(const Res&, BState&, int) const {}
   // A[m, kk..kk+3] = bottom[img, c, i*sv + dy, j*sh + dx] for kk = (img, i, j)
   __device__ void a_period(const AState& st, unsigned (&off)[4], int, int kl, int period) const {
     int k = period * 16 + kl;
@@ -274,7 +286,12 @@ struct ConvBwdFilter {
       img += wi ? 1 : 0;
     }
   }
-  __device__ unsigned a_soff(int, int) const { return 0u; }
+  __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[4], int, int, int,
+                         float (&v)[4]) const {
+    mnv_fetch_vec<4>(r.a, off, 0u, v);
+  }
+  size_t extra_lds_bytes() const { return 0; }
+  __device__ void block_init(Res&, float*, int, int) const {}
   // B[kk..kk+3, ko] = top_diff[img, ko, i, j]
   __device__ void b_period(const BState&, unsigned (&off)[4], int n, int kl, int period) const {
     int k = period * 16 + kl;
@@ -290,8 +307,108 @@ struct ConvBwdFilter {
       img += wrap ? 1 : 0;
     }
   }
-  __device__ unsigned b_soff(int, int) const { return 0u; }
+  __device__ void b_load(const Res& r, const BState&, const unsigned (&off)[4], int, int, int,
+                         float (&v)[4]) const {
+    mnv_fetch_vec<4>(r.b, off, 0u, v);
+  }
   __device__ void c_store(int m, int n, float x) const { filter_diff[(size_t)n * M + m] = x; }
+};
+
+// Filter gradient, fast addressing.  The GEMM rows are ordered (tap, channel) instead of
+// (channel, tap), so a thread's tap is fixed and the only thing that changes from slab to
+// slab is which 16 output positions are reduced.  The reduction runs image by image
+// (one period per image, positions padded to a multiple of 16).  A workgroup first writes,
+// for every tap its rows touch, a table pos -> byte offset of the input pixel that the tap
+// pairs with output position pos (or MNV_OOB when that pixel is padding or pos is past the
+// image); a slab's im2col offsets are then one 16-byte LDS read and four adds per vector.
+// top_diff is read with 16-byte loads of 4 consecutive positions; only the last, partial
+// slab of an image needs per-element masking.
+struct ConvBwdFilterFast {
+  static constexpr bool A_KFAST = true, B_KFAST = true;
+  static constexpr int A_NOFF = 1, B_NOFF = 1;
+  const float* __restrict__ bottom;
+  const float* __restrict__ top_diff;
+  float* __restrict__ filter_diff;
+  ConvGeom g;
+  int M, N, K, total_slabs, spp;  // C*R*S rows in (tap, c) order, Kout, N*Ho*Wo
+  int PP, taps_per_block;         // padded positions per image, table rows per workgroup
+  MnvFastDiv d_C;
+  struct Res {
+    mnv_rsrc a, b;
+    const unsigned* tab;  // LDS: [taps_per_block][PP]
+    int tap0;             // first tap of the workgroup's rows
+  };
+  struct AState {
+    unsigned cbase;  // c*H*W*4, or MNV_OOB for rows past M
+    int trow;        // (tap - first tap of the workgroup) * PP
+  };
+  struct BState {};
+  __device__ void make_res(Res& r) const {
+    r.a = mnv_make_rsrc(bottom, (unsigned)(g.N * g.C * g.HW) * 4u);
+    r.b = mnv_make_rsrc(top_diff, (unsigned)(g.N * g.K * g.HoWo) * 4u);
+    r.tab = nullptr;
+    r.tap0 = 0;
+  }
+  size_t extra_lds_bytes() const { return (size_t)taps_per_block * PP * sizeof(unsigned); }
+  __device__ void block_init(Res& r, float* extra, int m0, int) const {
+    unsigned* tab = reinterpret_cast<unsigned*>(extra);
+    r.tab = tab;
+    const int tap0 = mnv_fastdiv(m0, d_C);
+    r.tap0 = tap0;
+    for (int e = threadIdx.x; e < taps_per_block * PP; e += blockDim.x) {
+      int t = e / PP, pos = e - t * PP;
+      int tap = tap0 + t;
+      int rp = mnv_fastdiv(tap, g.d_S), sp = tap - rp * g.S;
+      int dy = g.R - 1 - rp - g.ph, dx = g.S - 1 - sp - g.pw;
+      int i = mnv_fastdiv(pos, g.d_Wo), j = pos - i * g.Wo;
+      int y = i * g.sv + dy, x = j * g.sh + dx;
+      bool ok = (pos < g.HoWo) & (tap < g.RS) & ((unsigned)y < (unsigned)g.H) &
+                ((unsigned)x < (unsigned)g.W);
+      tab[e] = ok ? (unsigned)(y * g.W + x) * 4u : MNV_OOB;
+    }
+  }
+  __device__ void a_init(const Res& res, AState& st, int m) const {
+    int tap = mnv_fastdiv(m, d_C);
+    int c = m - tap * g.C;
+    st.cbase = m < M ? (unsigned)(c * g.HW) * 4u : MNV_OOB;
+    int t = tap - res.tap0;
+    st.trow = (t < taps_per_block ? t : 0) * PP;  // rows past M read a valid table row; cbase masks them
+  }
+  __device__ void b_init(const Res&, BState&, int) const {}
+  __device__ void a_period(const AState&, unsigned (&off)[1], int, int, int) const { off[0] = 0; }
+  // off[0] is unused for A: the offsets come from the table every slab.
+  __device__ void a_load(const Res& r, const AState& st, const unsigned (&)[1], int period, int s,
+                         int kl, float (&v)[4]) const {
+    const unsigned* t = r.tab + st.trow + s * 16 + kl;
+    const unsigned soff = (unsigned)period * (unsigned)(g.C * g.HW) * 4u;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      v[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                           r.a, (int)(st.cbase + t[q]), (int)soff, 0));
+  }
+  __device__ void b_period(const BState&, unsigned (&off)[1], int n, int kl, int) const {
+    off[0] = n < N ? (unsigned)(n * g.HoWo + kl) * 4u : MNV_OOB;
+  }
+  __device__ void b_load(const Res& r, const BState&, const unsigned (&off)[1], int period, int s,
+                         int kl, float (&v)[4]) const {
+    const unsigned soff = ((unsigned)period * (unsigned)(g.K * g.HoWo) + (unsigned)s * 16u) * 4u;
+    if (s * 16 + 16 <= g.HoWo) {  // uniform: every position of the slab is inside the image
+      mnv_fetch_vec<1>(r.b, off, soff, v);
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        bool ok = s * 16 + kl + q < g.HoWo;
+        v[q] = __builtin_bit_cast(
+            float, __builtin_amdgcn_raw_buffer_load_b32(r.b, (int)(ok ? off[0] + 4u * q : MNV_OOB),
+                                                        (int)soff, 0));
+      }
+    }
+  }
+  __device__ void c_store(int m, int n, float x) const {
+    int tap = mnv_fastdiv(m, d_C);
+    int c = m - tap * g.C;
+    filter_diff[(size_t)n * M + c * g.RS + tap] = x;
+  }
 };
 
 // Filter permutations for the FAST policies (a few MB at most, one pass):
@@ -473,10 +590,20 @@ int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filte
   int rc = make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S);
   if (rc) return rc;
   int gm = g.CRS, gn = K, gk = N * g.HoWo;
-  ConvBwdFilter p{bottom, top_diff, filter_diff, g, gm, gn, gk, (gk + 15) / 16, 1};
   hipStream_t s = mnv_stream(stream);
   int splits = bwd_filter_splits(gm, gn, gk, workspace ? workspace_bytes / sizeof(float) : 0);
-  return launch_tile(bwd_filter_small_tiles(gm, gn) ? 0 : 1, p, splits, workspace, s);
+  const bool small = bwd_filter_small_tiles(gm, gn);
+  // Fast addressing: rows in (tap, channel) order with per-tap offset tables in LDS.  The
+  // tables of all taps a 128-row tile touches must fit beside the tiles.
+  const int PP = (g.HoWo + 15) / 16 * 16;
+  const int taps_per_block = (128 + C - 1) / C + 1;
+  if (!small && (size_t)taps_per_block * PP * 4 <= 24 * 1024) {
+    ConvBwdFilterFast p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16), PP / 16,
+                        PP, taps_per_block, mnv_fastdiv_make(C)};
+    return launch_tile(1, p, splits, workspace, s);
+  }
+  ConvBwdFilter p{bottom, top_diff, filter_diff, g, gm, gn, gk, (gk + 15) / 16, 1};
+  return launch_tile(small ? 0 : 1, p, splits, workspace, s);
 }
 
 }  // extern "C"

@@ -104,12 +104,18 @@ struct MnvFetchMap {
 //   int M, N, total_slabs, spp;               (host-set members)
 //   struct Res;  void make_res(Res&) const;   buffer resources
 //   struct AState / BState;                   per-thread, per-vector state set once
-//   void a_init(AState&, int m) const;
+//   void a_init(const Res&, AState&, int m) const;    after block_init
 //   void a_period(const AState&, unsigned (&off)[A_NOFF], int m, int kl, int period) const;
 //        byte offsets of this vector's elements for slab 0 of `period`; kl = the vector's
 //        first k index inside a slab; an element that must read as 0 gets MNV_OOB
-//   unsigned a_soff(int period, int s) const; uniform byte offset of slab s of the period
+//   void a_load(const Res&, const AState&, const unsigned (&off)[A_NOFF], int period, int s,
+//               int kl, float (&v)[4]) const;
+//        issues the loads of slab s of the period; the usual body is
+//        mnv_fetch_vec(res.a, off, <uniform byte offset of the slab>, v)
 //   (same for b with n)
+//   size_t extra_lds_bytes() const;           (host) LDS the policy wants after the tiles
+//   void block_init(Res&, float* extra_lds, int m0, int n0) const;   once per workgroup,
+//        before the first load; a barrier follows it
 //   void c_store(int m, int n, float v) const;   only called for m < M, n < N
 template <int NOFF>
 __device__ __forceinline__ void mnv_fetch_vec(mnv_rsrc r, const unsigned (&off)[NOFF],
@@ -151,13 +157,14 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
 
   typename P::Res res;
   prob.make_res(res);
+  prob.block_init(res, mnv_gemm_lds + 2 * T::BK * (T::LDA + T::LDB), m0, n0);
   typename P::AState ast[T::AV];
   typename P::BState bst[T::BV];
   unsigned aoff[T::AV][P::A_NOFF], boff[T::BV][P::B_NOFF];
 #pragma unroll
-  for (int p = 0; p < T::AV; ++p) prob.a_init(ast[p], m0 + MapA::x(tid, p));
+  for (int p = 0; p < T::AV; ++p) prob.a_init(res, ast[p], m0 + MapA::x(tid, p));
 #pragma unroll
-  for (int p = 0; p < T::BV; ++p) prob.b_init(bst[p], n0 + MapB::x(tid, p));
+  for (int p = 0; p < T::BV; ++p) prob.b_init(res, bst[p], n0 + MapB::x(tid, p));
 
   float ra[T::AV][4], rb[T::BV][4];
 
@@ -170,11 +177,12 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
       prob.b_period(bst[p], boff[p], n0 + MapB::x(tid, p), MapB::k(tid, p), period);
   };
   auto fetch = [&](int period, int s) {
-    const unsigned sa = prob.a_soff(period, s), sb = prob.b_soff(period, s);
 #pragma unroll
-    for (int p = 0; p < T::AV; ++p) mnv_fetch_vec<P::A_NOFF>(res.a, aoff[p], sa, ra[p]);
+    for (int p = 0; p < T::AV; ++p)
+      prob.a_load(res, ast[p], aoff[p], period, s, MapA::k(tid, p), ra[p]);
 #pragma unroll
-    for (int p = 0; p < T::BV; ++p) mnv_fetch_vec<P::B_NOFF>(res.b, boff[p], sb, rb[p]);
+    for (int p = 0; p < T::BV; ++p)
+      prob.b_load(res, bst[p], boff[p], period, s, MapB::k(tid, p), rb[p]);
   };
   auto stash = [&](int buf) {
     float* a = As + buf * T::BK * T::LDA;
@@ -217,6 +225,7 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
 
   // (period, s) of the slab whose loads are issued next
   int period = slab_begin / prob.spp, s = slab_begin - period * prob.spp;
+  __syncthreads();  // block_init may have written LDS
   if (slab_begin < slab_end) {
     new_period(period);
     fetch(period, s);
@@ -307,8 +316,10 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
                                     (int)T::LDS_BYTES));
     attr_set = true;
   }
+  const size_t lds_bytes = T::LDS_BYTES + prob.extra_lds_bytes();
+  if (lds_bytes > 64 * 1024) return MNV_ERR_INVALID;
   hipLaunchKernelGGL((mnv_gemm_kernel<T, P>), dim3(tiles_m * tiles_n, 1, splits), dim3(T::NT),
-                     T::LDS_BYTES, s, prob, tiles_m, tiles_n, per,
+                     lds_bytes, s, prob, tiles_m, tiles_n, per,
                      reinterpret_cast<float*>(workspace));
   int rc = MNV_LAUNCH_STATUS();
   if (rc) return rc;

@@ -2,15 +2,19 @@
 // (cuDNN v2 modes selected at reference minerva/op/impl/cuda/cuda_perform.cu:489-615;
 // output extent rule minerva/narray/convolution.cpp:107-114).
 // Roofline: HBM bandwidth; forward moves 4*(in + out) bytes, backward
-// 4*(top_diff + bottom + bottom_diff) (the overlapping window re-reads hit in cache).
+// 4*(top_diff + bottom + bottom_diff).
 //
 // Window o covers rows [o*stride - pad, o*stride - pad + window) clipped to the
 // tensor.  max: padding never wins.  average: divisor is the full window area.
-// max backward is a gather: every bottom position revisits the (few) windows that
-// contain it, recomputes each window's first maximum in (row, column) scan order and
-// adds that window's gradient if the maximum is itself; windows are visited in
-// ascending order so overlapping contributions add up in the same order as a
-// sequential scatter, and no atomics are needed.
+// max backward sends each top_diff to the first maximum of its window in (row, column)
+// scan order; a position that wins several overlapping windows adds their gradients in
+// ascending window order, which is the order a sequential scatter would use, so the
+// result is bit-identical to it and no atomics are needed.
+//
+// Main path: a workgroup stages whole (n,c) planes in LDS with contiguous 16-byte loads,
+// finds every window's arg-max once from LDS, then walks the plane's positions and
+// gathers the gradients of the (at most ceil(k/s)^2) windows each one can win.  HBM sees
+// every tensor exactly once.  Planes too large for LDS take the direct kernels below.
 #include <math.h>
 
 #include "mnv_common.h"
@@ -18,11 +22,131 @@
 namespace {
 
 #define MNV_POOL_THREADS 256
+#define MNV_POOL_LDS_FLOATS 8192  // plane data staged per workgroup (32 KiB)
 
 struct PoolGeom {
   int H, W, Ho, Wo, sv, sh, kh, kw, ph, pw;
 };
 
+__device__ __forceinline__ int ceil_div_pos(int a, int b) {  // b > 0, any a
+  return a >= 0 ? (a + b - 1) / b : -((-a) / b);
+}
+
+// Loads `count` floats starting at src (any alignment) into LDS.
+__device__ __forceinline__ void stage(const float* __restrict__ src, float* dst, int count) {
+  // align the global side to 16 bytes, then copy vectors
+  int head = (int)(((16 - (reinterpret_cast<uintptr_t>(src) & 15)) & 15) >> 2);
+  if (head > count) head = count;
+  for (int i = threadIdx.x; i < head; i += MNV_POOL_THREADS) dst[i] = src[i];
+  const int n4 = (count - head) >> 2;
+  const mnv_f4* s4 = reinterpret_cast<const mnv_f4*>(src + head);
+  for (int i = threadIdx.x; i < n4; i += MNV_POOL_THREADS) {
+    mnv_f4 v = s4[i];
+    float* d = dst + head + 4 * i;
+    d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+  }
+  for (int i = head + 4 * n4 + threadIdx.x; i < count; i += MNV_POOL_THREADS) dst[i] = src[i];
+}
+
+// ---- LDS-staged kernels: `ppb` planes per workgroup --------------------------------
+template <bool MAX>
+__global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_fwd_lds_kernel(
+    const float* __restrict__ bottom, float* __restrict__ top, int planes, int ppb, PoolGeom g) {
+  extern __shared__ float lds[];
+  const int hw = g.H * g.W, howo = g.Ho * g.Wo;
+  for (int p0 = blockIdx.x * ppb; p0 < planes; p0 += gridDim.x * ppb) {
+    const int np = min(ppb, planes - p0);
+    __syncthreads();
+    stage(bottom + (size_t)p0 * hw, lds, np * hw);
+    __syncthreads();
+    for (int q = threadIdx.x; q < np * howo; q += MNV_POOL_THREADS) {
+      int pl = q / howo, o = q - pl * howo;
+      int i = o / g.Wo, j = o - i * g.Wo;
+      int y0 = i * g.sv - g.ph, x0 = j * g.sh - g.pw;
+      int ys = max(y0, 0), xs = max(x0, 0);
+      int ye = min(y0 + g.kh, g.H), xe = min(x0 + g.kw, g.W);
+      const float* b = lds + pl * hw;
+      float r;
+      if (MAX) {
+        r = -INFINITY;
+        for (int y = ys; y < ye; ++y)
+          for (int x = xs; x < xe; ++x) {
+            float v = b[y * g.W + x];
+            if (r < v) r = v;
+          }
+      } else {
+        float s = 0.f;
+        for (int y = ys; y < ye; ++y)
+          for (int x = xs; x < xe; ++x) s += b[y * g.W + x];
+        r = s / (float)(g.kh * g.kw);
+      }
+      top[(size_t)p0 * howo + q] = r;
+    }
+  }
+}
+
+// LDS: [ppb*hw] plane data, then [ppb*howo] top_diff, then [ppb*howo] arg-max positions.
+template <bool MAX>
+__global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_lds_kernel(
+    const float* __restrict__ bottom, const float* __restrict__ top_diff,
+    float* __restrict__ bottom_diff, int planes, int ppb, PoolGeom g) {
+  extern __shared__ float lds[];
+  const int hw = g.H * g.W, howo = g.Ho * g.Wo;
+  float* sx = lds;
+  float* sd = lds + ppb * hw;
+  int* sarg = reinterpret_cast<int*>(sd + ppb * howo);
+  for (int p0 = blockIdx.x * ppb; p0 < planes; p0 += gridDim.x * ppb) {
+    const int np = min(ppb, planes - p0);
+    __syncthreads();
+    if (MAX) stage(bottom + (size_t)p0 * hw, sx, np * hw);
+    stage(top_diff + (size_t)p0 * howo, sd, np * howo);
+    __syncthreads();
+    if (MAX) {
+      // first maximum of every window in scan order (strict '<'), as a flat position
+      for (int q = threadIdx.x; q < np * howo; q += MNV_POOL_THREADS) {
+        int pl = q / howo, o = q - pl * howo;
+        int i = o / g.Wo, j = o - i * g.Wo;
+        int y0 = i * g.sv - g.ph, x0 = j * g.sh - g.pw;
+        int ys = max(y0, 0), xs = max(x0, 0);
+        int ye = min(y0 + g.kh, g.H), xe = min(x0 + g.kw, g.W);
+        const float* b = sx + pl * hw;
+        float mx = -INFINITY;
+        int arg = ys * g.W + xs;
+        for (int y = ys; y < ye; ++y)
+          for (int x = xs; x < xe; ++x) {
+            float v = b[y * g.W + x];
+            if (mx < v) {
+              mx = v;
+              arg = y * g.W + x;
+            }
+          }
+        sarg[q] = arg;
+      }
+      __syncthreads();
+    }
+    for (int q = threadIdx.x; q < np * hw; q += MNV_POOL_THREADS) {
+      int pl = q / hw, pos = q - pl * hw;
+      int y = pos / g.W, x = pos - y * g.W;
+      int i_lo = max(ceil_div_pos(y + g.ph - g.kh + 1, g.sv), 0);
+      int i_hi = min((y + g.ph) / g.sv, g.Ho - 1);
+      int j_lo = max(ceil_div_pos(x + g.pw - g.kw + 1, g.sh), 0);
+      int j_hi = min((x + g.pw) / g.sh, g.Wo - 1);
+      float acc = 0.f;
+      for (int i = i_lo; i <= i_hi; ++i)
+        for (int j = j_lo; j <= j_hi; ++j) {
+          int o = pl * howo + i * g.Wo + j;
+          if (MAX) {
+            if (sarg[o] == pos) acc += sd[o];
+          } else {
+            acc += sd[o] / (float)(g.kh * g.kw);
+          }
+        }
+      bottom_diff[(size_t)p0 * hw + q] = acc;
+    }
+  }
+}
+
+// ---- direct kernels for planes that do not fit in LDS -------------------------------
 template <bool MAX>
 __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_fwd_kernel(
     const float* __restrict__ bottom, float* __restrict__ top, size_t planes, PoolGeom g) {
@@ -54,10 +178,6 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_fwd_kernel(
   }
 }
 
-__device__ __forceinline__ int ceil_div_pos(int a, int b) {  // b > 0, any a
-  return a >= 0 ? (a + b - 1) / b : -((-a) / b);
-}
-
 template <bool MAX>
 __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_kernel(
     const float* __restrict__ bottom, const float* __restrict__ top_diff,
@@ -77,14 +197,12 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_kernel(
     const float* b = bottom + plane * per_plane;
     const float* dt = top_diff + plane * (size_t)g.Ho * g.Wo;
     float acc = 0.f;
-    const float mine = MAX ? b[pos] : 0.f;
     for (int i = i_lo; i <= i_hi; ++i)
       for (int j = j_lo; j <= j_hi; ++j) {
         if (MAX) {
           int y0 = i * g.sv - g.ph, x0 = j * g.sh - g.pw;
           int ys = max(y0, 0), xs = max(x0, 0);
           int ye = min(y0 + g.kh, g.H), xe = min(x0 + g.kw, g.W);
-          // first maximum in scan order (strict '<'), as a flat position
           float mx = -INFINITY;
           int arg = ys * g.W + xs;
           for (int yy = ys; yy < ye; ++yy)
@@ -95,7 +213,6 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_kernel(
                 arg = yy * g.W + xx;
               }
             }
-          (void)mine;
           if (arg == pos) acc += dt[i * g.Wo + j];
         } else {
           acc += dt[i * g.Wo + j] / (float)(g.kh * g.kw);
@@ -110,7 +227,7 @@ int make_geom(PoolGeom* g, int n, int c, int h, int w, int sv, int sh, int kh, i
   if (n <= 0 || c <= 0 || h <= 0 || w <= 0 || sv <= 0 || sh <= 0 || kh <= 0 || kw <= 0 ||
       ph < 0 || pw < 0)
     return MNV_ERR_INVALID;
-  if ((long long)h * w > 0x7fffffffLL) return MNV_ERR_INVALID;
+  if ((long long)h * w > 0x7fffffffLL || (long long)n * c > 0x7fffffffLL) return MNV_ERR_INVALID;
   g->H = h; g->W = w; g->sv = sv; g->sh = sh; g->kh = kh; g->kw = kw; g->ph = ph; g->pw = pw;
   g->Ho = mnv_pooled_size(h, kh, sv, ph);
   g->Wo = mnv_pooled_size(w, kw, sh, pw);
@@ -124,6 +241,19 @@ unsigned pool_grid(size_t total) {
   return (unsigned)blocks;
 }
 
+// Planes per workgroup for the LDS path: as many as fit the staging area, but no more
+// than leaves every CU several workgroups.  0 = plane too large, use the direct kernels.
+int planes_per_block(const PoolGeom& g, long long planes, bool bwd) {
+  long long per_plane = (long long)g.H * g.W + (bwd ? 2LL * g.Ho * g.Wo : 0);
+  if (per_plane > MNV_POOL_LDS_FLOATS) return 0;
+  long long ppb = MNV_POOL_LDS_FLOATS / per_plane;
+  long long cap = planes / 2048;  // keep at least ~2048 workgroups
+  if (cap < 1) cap = 1;
+  if (ppb > cap) ppb = cap;
+  if (ppb > 64) ppb = 64;
+  return (int)ppb;
+}
+
 template <bool MAX>
 int pool_fwd(const float* bottom, float* top, int n, int c, int h, int w, int sv, int sh, int kh,
              int kw, int ph, int pw, mnv_stream_t stream) {
@@ -131,9 +261,20 @@ int pool_fwd(const float* bottom, float* top, int n, int c, int h, int w, int sv
   if (!bottom || !top) return MNV_ERR_INVALID;
   int rc = make_geom(&g, n, c, h, w, sv, sh, kh, kw, ph, pw);
   if (rc) return rc;
-  size_t planes = (size_t)n * c;
-  hipLaunchKernelGGL((mnv_pool_fwd_kernel<MAX>), dim3(pool_grid(planes * g.Ho * g.Wo)),
-                     dim3(MNV_POOL_THREADS), 0, mnv_stream(stream), bottom, top, planes, g);
+  long long planes = (long long)n * c;
+  int ppb = planes_per_block(g, planes, false);
+  if (ppb > 0) {
+    size_t lds = (size_t)ppb * h * w * sizeof(float);
+    long long blocks = (planes + ppb - 1) / ppb;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL((mnv_pool_fwd_lds_kernel<MAX>), dim3((unsigned)blocks),
+                       dim3(MNV_POOL_THREADS), lds, mnv_stream(stream), bottom, top, (int)planes,
+                       ppb, g);
+  } else {
+    hipLaunchKernelGGL((mnv_pool_fwd_kernel<MAX>), dim3(pool_grid((size_t)planes * g.Ho * g.Wo)),
+                       dim3(MNV_POOL_THREADS), 0, mnv_stream(stream), bottom, top, (size_t)planes,
+                       g);
+  }
   return MNV_LAUNCH_STATUS();
 }
 
@@ -144,10 +285,20 @@ int pool_bwd(const float* bottom, const float* top_diff, float* bottom_diff, int
   if (!bottom || !top_diff || !bottom_diff) return MNV_ERR_INVALID;
   int rc = make_geom(&g, n, c, h, w, sv, sh, kh, kw, ph, pw);
   if (rc) return rc;
-  size_t planes = (size_t)n * c;
-  hipLaunchKernelGGL((mnv_pool_bwd_kernel<MAX>), dim3(pool_grid(planes * h * w)),
-                     dim3(MNV_POOL_THREADS), 0, mnv_stream(stream), bottom, top_diff, bottom_diff,
-                     planes, g);
+  long long planes = (long long)n * c;
+  int ppb = planes_per_block(g, planes, true);
+  if (ppb > 0) {
+    size_t lds = (size_t)ppb * ((size_t)h * w + 2 * (size_t)g.Ho * g.Wo) * sizeof(float);
+    long long blocks = (planes + ppb - 1) / ppb;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL((mnv_pool_bwd_lds_kernel<MAX>), dim3((unsigned)blocks),
+                       dim3(MNV_POOL_THREADS), lds, mnv_stream(stream), bottom, top_diff,
+                       bottom_diff, (int)planes, ppb, g);
+  } else {
+    hipLaunchKernelGGL((mnv_pool_bwd_kernel<MAX>), dim3(pool_grid((size_t)planes * h * w)),
+                       dim3(MNV_POOL_THREADS), 0, mnv_stream(stream), bottom, top_diff,
+                       bottom_diff, (size_t)planes, g);
+  }
   return MNV_LAUNCH_STATUS();
 }
 

@@ -28,8 +28,8 @@ struct SgemmNN {
     r.a = mnv_make_rsrc(A, (unsigned)M * (unsigned)K * 4u);
     r.b = mnv_make_rsrc(B, (unsigned)K * (unsigned)N * 4u);
   }
-  __device__ void a_init(AState&, int) const {}
-  __device__ void b_init(BState&, int) const {}
+  __device__ void a_init(const Res&, AState&, int) const {}
+  __device__ void b_init(const Res&, BState&, int) const {}
   // A[m..m+3, k]: x-fast
   __device__ void a_period(const AState&, unsigned (&off)[A_NOFF], int m, int kl, int period) const {
     const int k = period * spp * 16 + kl;
@@ -37,7 +37,10 @@ struct SgemmNN {
 #pragma unroll
     for (int q = 0; q < A_NOFF; ++q) off[q] = ((m + q < M) & (k < K)) ? base + 4u * q : MNV_OOB;
   }
-  __device__ unsigned a_soff(int, int s) const { return (unsigned)s * 16u * (unsigned)M * 4u; }
+  __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[A_NOFF], int, int s,
+                         int, float (&v)[4]) const {
+    mnv_fetch_vec<A_NOFF>(r.a, off, (unsigned)s * 16u * (unsigned)M * 4u, v);
+  }
   // B[k..k+3, n]: k-fast
   __device__ void b_period(const BState&, unsigned (&off)[B_NOFF], int n, int kl, int period) const {
     const int k = period * spp * 16 + kl;
@@ -45,7 +48,12 @@ struct SgemmNN {
 #pragma unroll
     for (int q = 0; q < B_NOFF; ++q) off[q] = ((n < N) & (k + q < K)) ? base + 4u * q : MNV_OOB;
   }
-  __device__ unsigned b_soff(int, int s) const { return (unsigned)s * 64u; }
+  __device__ void b_load(const Res& r, const BState&, const unsigned (&off)[B_NOFF], int, int s,
+                         int, float (&v)[4]) const {
+    mnv_fetch_vec<B_NOFF>(r.b, off, (unsigned)s * 64u, v);
+  }
+  size_t extra_lds_bytes() const { return 0; }
+  __device__ void block_init(Res&, float*, int, int) const {}
   __device__ void c_store(int m, int n, float x) const { C[(size_t)n * M + m] = x; }
 };
 

@@ -231,6 +231,8 @@ POOL = [
     (3, 256, 13, 13, 2, 2, 3, 3, 0, 0),   # pool5
     (4, 16, 24, 24, 2, 2, 2, 2, 0, 0),    # MNIST CNN pools
     (4, 32, 12, 12, 3, 3, 3, 3, 0, 0),
+    (1, 3, 100, 95, 2, 2, 3, 3, 1, 1),    # planes too large for the LDS-staged kernels
+    (70, 33, 5, 7, 1, 2, 2, 3, 1, 1),     # many tiny planes per workgroup, odd plane size
 ]
 
 
