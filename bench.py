@@ -51,7 +51,9 @@ def alexnet_bench(steps, warmup):
         net = hostapi.Net(rt, "alexnet", BATCH)
         for k, v in params.items():
             net.set_param(k, v)
-        net.load_batch(data, label)
+        t_h2d = time.perf_counter()
+        net.load_batch(data, label)  # ArrayLoader: pageable host memory -> HBM, synchronous
+        t_h2d = (time.perf_counter() - t_h2d) * 1e3
         for _ in range(warmup):
             net.step(0.01)
         rt.sync()
@@ -69,7 +71,8 @@ def alexnet_bench(steps, warmup):
         ms = (t1 - t0) * 1e3 / steps
         out[mode] = {"ms_per_step": ms, "images_per_s": BATCH / (ms / 1e3),
                      "ops_per_step": (rt.ops_issued() - ops0) // steps,
-                     "finite": bool(np.isfinite(prob).all()), "profile": prof}
+                     "finite": bool(np.isfinite(prob).all()), "profile": prof,
+                     "h2d_batch_ms": t_h2d}
         log("alexnet b=%d %s: %.3f ms/step, %.1f img/s, %d ops/step" %
             (BATCH, mode, ms, out[mode]["images_per_s"], out[mode]["ops_per_step"]))
         net.close()
@@ -77,9 +80,16 @@ def alexnet_bench(steps, warmup):
     return out
 
 
+# HBM bytes per launch of the dominant kernel (average over the conv2..conv5 filter
+# gradients), from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB
+# per dispatch), each scaled by what the same counter reads for the 8192^2 copy kernel
+# (256 MiB read, 256 MiB written).  None until measured.
+DOMINANT_KERNEL_TRAFFIC_BYTES = None
+
+
 def dominant_kernel_roofline(prof, steps):
     """The filter-gradient operators of conv2..conv5 run the 128x128 MFMA kernel
-    (mnv_gemm_kernel<128x128x16, ConvBwdFilter>) followed by its split-k reduction; the
+    (mnv_gemm_kernel<128x128x16, ConvBwdFilterFast>) followed by its split-k reduction; the
     event pair brackets both, so the figure is slightly conservative."""
     names = [n for n in prof if n.endswith("conv bp filter") and "stride:1*1" in n]
     launches = sum(prof[n][0] for n in names)
@@ -90,9 +100,11 @@ def dominant_kernel_roofline(prof, steps):
     flops_per_launch = gflop_per_step * 1e9 * steps / launches
     avg_ms = total_ms / launches
     achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
-    return {"bound": "mfma", "kernel": "mnv_gemm_kernel<128x128x16,ConvBwdFilter> (conv2-5 filter gradient)",
+    return {"bound": "mfma",
+            "kernel": "mnv_gemm_kernel<128x128x16,ConvBwdFilterFast> (conv2-5 filter gradient)",
             "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+            "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+            "traffic": DOMINANT_KERNEL_TRAFFIC_BYTES,
             "avg_launch_ms": round(avg_ms, 4), "launches": launches,
             "algorithmic_gflop_per_launch": round(flops_per_launch / 1e9, 2)}
 
@@ -130,7 +142,45 @@ def micro_bench():
            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
                         "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}}
     log("add 8192^2: %.4f ms, %.0f GB/s" % (ms, gbs))
+    elt["ops"] = bandwidth_table(L, dev, x, y, z, ne)
     return sgemm, elt
+
+
+def bandwidth_table(L, dev, x, y, z, ne):
+    """The 8192^2 bandwidth microbenchmark (BASELINE.json configs[1]): GB/s from the
+    algorithmic bytes per element of each operator."""
+    m = n = 8192
+    S = dev.stream
+    vec = dev.upload(np.random.default_rng(8).standard_normal(m, dtype=np.float32))
+    small = dev.empty(m)
+    f = ctypes.c_float
+    ops = [
+        ("copy", 8, lambda: L.mnv_copy(x.p, z.p, ne, S)),
+        ("mul", 12, lambda: L.mnv_mul(x.p, y.p, z.p, ne, S)),
+        ("sub", 12, lambda: L.mnv_sub(x.p, y.p, z.p, ne, S)),
+        ("scalar mul", 8, lambda: L.mnv_const_mul(x.p, z.p, f(3.291), ne, S)),
+        ("broadcast add {1,n}", 8, lambda: L.mnv_norm_add_col(x.p, vec.p, z.p, m, n, S)),
+        ("broadcast add {m,1}", 8, lambda: L.mnv_norm_add_row(x.p, vec.p, z.p, m, n, S)),
+        ("sigmoid fwd", 8, lambda: L.mnv_sigmoid_fwd(x.p, z.p, ne, S)),
+        ("relu fwd", 8, lambda: L.mnv_relu_fwd(x.p, z.p, ne, S)),
+        ("tanh fwd", 8, lambda: L.mnv_tanh_fwd(x.p, z.p, ne, S)),
+        ("sigmoid bwd", 12, lambda: L.mnv_sigmoid_bwd(x.p, x.p, y.p, z.p, ne, S)),
+        ("relu bwd", 12, lambda: L.mnv_relu_bwd(x.p, x.p, y.p, z.p, ne, S)),
+        ("tanh bwd", 12, lambda: L.mnv_tanh_bwd(x.p, x.p, y.p, z.p, ne, S)),
+        ("sum dim 0", 4, lambda: L.mnv_reduce_sum_col(x.p, small.p, m, n, S)),
+        ("sum dim 1", 4, lambda: L.mnv_reduce_sum_row(x.p, small.p, m, n, S)),
+        ("max dim 0", 4, lambda: L.mnv_reduce_max_col(x.p, small.p, m, n, S)),
+        ("max dim 1", 4, lambda: L.mnv_reduce_max_row(x.p, small.p, m, n, S)),
+        ("maxindex dim 0", 4, lambda: L.mnv_maxindex_col(x.p, small.p, m, n, S)),
+        ("softmax rows", 8, lambda: L.mnv_softmax_instance_fwd(x.p, z.p, n, m, 1, 1, S)),
+    ]
+    table = []
+    for name, bpe, fn in ops:
+        ms = dev.time_ms(fn, iters=20, warmup=3)
+        gbs = bpe * ne / (ms * 1e-3) / 1e9
+        table.append({"op": name, "ms": round(ms, 4), "gbs": round(gbs, 1),
+                      "frac": round(gbs / PEAK_HBM_GBS, 4)})
+    return table
 
 
 def cpu_baseline(batch=4):
@@ -182,6 +232,7 @@ def main():
         "step_mfma_frac": round(STEP_GFLOP / main_run["ms_per_step"] / PEAK_FP32_MFMA_TFLOPS, 4),
         "per_op_sync": {"images_per_s": round(res["per_op_sync"]["images_per_s"], 1),
                         "ms_per_step": round(res["per_op_sync"]["ms_per_step"], 3)},
+        "h2d_batch_ms": round(main_run["h2d_batch_ms"], 2),
         "roofline": roof,
         "sgemm": sgemm,
         "eltwise": elt,

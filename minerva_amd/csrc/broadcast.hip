@@ -19,7 +19,7 @@ struct OpDiv { __device__ float operator()(float a, float b) const { return a / 
 #define MNV_BC_COLS 4  // columns per workgroup iteration: 4 independent 16-byte loads in flight
 
 // ROWVEC = true: vector indexed by row (shape {m,1}); false: by column ({1,n}).
-template <class Op, bool ROWVEC, bool VEC4>
+template <class Op, bool ROWVEC, bool VEC4, bool NT>
 __global__ __launch_bounds__(MNV_BC_THREADS) void mnv_norm_kernel(
     const float* __restrict__ mat, const float* __restrict__ vec, float* __restrict__ res, int m,
     int n, Op op) {
@@ -38,7 +38,9 @@ __global__ __launch_bounds__(MNV_BC_THREADS) void mnv_norm_kernel(
 #pragma unroll
       for (int u = 0; u < MNV_BC_COLS; ++u)
         if (c0 + u < n)
-          v[u] = *reinterpret_cast<const mnv_f4*>(mat + (size_t)(c0 + u) * m + r0);
+          v[u] = NT ? __builtin_nontemporal_load(
+                          reinterpret_cast<const mnv_f4*>(mat + (size_t)(c0 + u) * m + r0))
+                    : *reinterpret_cast<const mnv_f4*>(mat + (size_t)(c0 + u) * m + r0);
 #pragma unroll
       for (int u = 0; u < MNV_BC_COLS; ++u)
         if (c0 + u < n) {
@@ -48,7 +50,8 @@ __global__ __launch_bounds__(MNV_BC_THREADS) void mnv_norm_kernel(
           o.y = op(v[u].y, ROWVEC ? rv[1 % W] : cv);
           o.z = op(v[u].z, ROWVEC ? rv[2 % W] : cv);
           o.w = op(v[u].w, ROWVEC ? rv[3 % W] : cv);
-          *reinterpret_cast<mnv_f4*>(res + (size_t)(c0 + u) * m + r0) = o;
+          if (NT) __builtin_nontemporal_store(o, reinterpret_cast<mnv_f4*>(res + (size_t)(c0 + u) * m + r0));
+          else *reinterpret_cast<mnv_f4*>(res + (size_t)(c0 + u) * m + r0) = o;
         }
     } else {
 #pragma unroll
@@ -74,11 +77,16 @@ int launch_norm(const float* mat, const float* vec, float* res, int m, int n, mn
   if (gy > want) gy = want ? want : 1u;
   if (gy > 65535u) gy = 65535u;
   dim3 grid(gx, gy);
-  if (vec4)
-    hipLaunchKernelGGL((mnv_norm_kernel<Op, ROWVEC, true>), grid, dim3(MNV_BC_THREADS), 0,
+  // past the 256 MB last-level cache the matrix streams with non-temporal accesses
+  const bool nt = (size_t)m * n * 8 >= ((size_t)512 << 20);
+  if (vec4 && nt)
+    hipLaunchKernelGGL((mnv_norm_kernel<Op, ROWVEC, true, true>), grid, dim3(MNV_BC_THREADS), 0,
+                       mnv_stream(stream), mat, vec, res, m, n, Op());
+  else if (vec4)
+    hipLaunchKernelGGL((mnv_norm_kernel<Op, ROWVEC, true, false>), grid, dim3(MNV_BC_THREADS), 0,
                        mnv_stream(stream), mat, vec, res, m, n, Op());
   else
-    hipLaunchKernelGGL((mnv_norm_kernel<Op, ROWVEC, false>), grid, dim3(MNV_BC_THREADS), 0,
+    hipLaunchKernelGGL((mnv_norm_kernel<Op, ROWVEC, false, false>), grid, dim3(MNV_BC_THREADS), 0,
                        mnv_stream(stream), mat, vec, res, m, n, Op());
   return MNV_LAUNCH_STATUS();
 }

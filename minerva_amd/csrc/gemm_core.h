@@ -74,7 +74,7 @@ struct MnvGemmTile {
   // Wavefronts per SIMD the register allocation must allow: four 4-wavefront workgroups
   // per CU make 1024 resident tiles, which lets tile counts just under a multiple of
   // 1024 finish in whole rounds.
-  static constexpr int MIN_WAVES = (NT == 256 && BM * BN <= 128 * 128) ? 4 : 1;
+  static constexpr int MIN_WAVES = (NT == 256 && BM * BN <= 128 * 128 && BK <= 16) ? 4 : 1;
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
   static_assert(BK % 4 == 0 && (BM * BK) % (4 * NT) == 0 && (BN * BK) % (4 * NT) == 0, "tile/thread mismatch");
 };
@@ -310,10 +310,9 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
   splits = total_slabs > 0 ? (total_slabs + per - 1) / per : 1;
   if ((long long)tiles_m * tiles_n > 0x7fffffffLL || splits > 65535) return MNV_ERR_INVALID;
   static bool attr_set = false;  // idempotent; a race only repeats the same call
-  if (!attr_set && T::LDS_BYTES > 48 * 1024) {
+  if (!attr_set && T::LDS_BYTES + prob.extra_lds_bytes() > 48 * 1024) {
     MNV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&mnv_gemm_kernel<T, P>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)T::LDS_BYTES));
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
     attr_set = true;
   }
   const size_t lds_bytes = T::LDS_BYTES + prob.extra_lds_bytes();

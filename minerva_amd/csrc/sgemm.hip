@@ -4,6 +4,8 @@
 // Built on the fp32 MFMA core in gemm_core.h; A is fetched x-fast (m contiguous),
 // B k-fast (k contiguous).  Products with too few output tiles to fill 256 CUs split
 // the k range over blockIdx.z when the caller lends a workspace.
+#include <stdlib.h>
+
 #include "gemm_core.h"
 
 namespace {
@@ -18,7 +20,7 @@ struct SgemmNN {
   const float* __restrict__ A;
   const float* __restrict__ B;
   float* __restrict__ C;
-  int M, N, K, total_slabs, spp;
+  int M, N, K, total_slabs, spp, bk;
   struct Res {
     mnv_rsrc a, b;
   };
@@ -32,27 +34,32 @@ struct SgemmNN {
   __device__ void b_init(const Res&, BState&, int) const {}
   // A[m..m+3, k]: x-fast
   __device__ void a_period(const AState&, unsigned (&off)[A_NOFF], int m, int kl, int period) const {
-    const int k = period * spp * 16 + kl;
+    const int k = period * spp * bk + kl;
     const unsigned base = ((unsigned)k * (unsigned)M + (unsigned)m) * 4u;
 #pragma unroll
     for (int q = 0; q < A_NOFF; ++q) off[q] = ((m + q < M) & (k < K)) ? base + 4u * q : MNV_OOB;
   }
   __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[A_NOFF], int, int s,
                          int, float (&v)[4]) const {
-    mnv_fetch_vec<A_NOFF>(r.a, off, (unsigned)s * 16u * (unsigned)M * 4u, v);
+    mnv_fetch_vec<A_NOFF>(r.a, off, (unsigned)s * (unsigned)bk * (unsigned)M * 4u, v);
   }
   // B[k..k+3, n]: k-fast
   __device__ void b_period(const BState&, unsigned (&off)[B_NOFF], int n, int kl, int period) const {
-    const int k = period * spp * 16 + kl;
+    const int k = period * spp * bk + kl;
     const unsigned base = ((unsigned)n * (unsigned)K + (unsigned)k) * 4u;
 #pragma unroll
     for (int q = 0; q < B_NOFF; ++q) off[q] = ((n < N) & (k + q < K)) ? base + 4u * q : MNV_OOB;
   }
   __device__ void b_load(const Res& r, const BState&, const unsigned (&off)[B_NOFF], int, int s,
                          int, float (&v)[4]) const {
-    mnv_fetch_vec<B_NOFF>(r.b, off, (unsigned)s * 64u, v);
+    mnv_fetch_vec<B_NOFF>(r.b, off, (unsigned)s * (unsigned)bk * 4u, v);
   }
   size_t extra_lds_bytes() const { return 0; }
+  void set_bk(int b) {
+    bk = b;
+    spp = K >= b ? K / b : 1;
+    total_slabs = (K + b - 1) / b;
+  }
   __device__ void block_init(Res&, float*, int, int) const {}
   __device__ void c_store(int m, int n, float x) const { C[(size_t)n * M + m] = x; }
 };
@@ -61,13 +68,29 @@ template <bool VEC>
 SgemmNN<VEC> make_sgemm(const float* a, const float* b, float* c, int m, int n, int k) {
   SgemmNN<VEC> p;
   p.A = a; p.B = b; p.C = c; p.M = m; p.N = n; p.K = k;
-  p.spp = k >= 16 ? k / 16 : 1;
-  p.total_slabs = (k + 15) / 16;
+  p.set_bk(16);
   return p;
 }
 
 typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
+typedef MnvGemmTile<128, 128, 32, 2, 2> TileBig32;
+typedef MnvGemmTile<128, 128, 16, 2, 2, 32> TileBigPad32;
+typedef MnvGemmTile<128, 128, 16, 2, 2, 4> TileBigPad4;
+typedef MnvGemmTile<256, 128, 16, 4, 2> TileTall8;
+typedef MnvGemmTile<256, 256, 16, 4, 2> TileHuge8;
+
+template <class P>
+int sgemm_launch_exp(int tile, P p, int splits, void* ws, hipStream_t s) {
+  switch (tile) {
+    case 2: p.set_bk(32); return mnv_gemm_launch<TileBig32>(p, splits, ws, s);
+    case 3: return mnv_gemm_launch<TileBigPad32>(p, splits, ws, s);
+    case 4: return mnv_gemm_launch<TileBigPad4>(p, splits, ws, s);
+    case 5: return mnv_gemm_launch<TileTall8>(p, splits, ws, s);
+    case 6: return mnv_gemm_launch<TileHuge8>(p, splits, ws, s);
+    default: return mnv_gemm_launch<TileBig>(p, splits, ws, s);
+  }
+}
 
 #define MNV_SGEMM_MAX_SPLITS 16
 
@@ -118,6 +141,7 @@ int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k, 
   int splits = pick_splits(tiles, slabs, (size_t)m * n, ws_floats);
   if (vec) {
     SgemmNN<true> p = make_sgemm<true>(a, b, c, m, n, k);
+    if (const char* e = getenv("MNV_SGEMM_TILE")) return sgemm_launch_exp(atoi(e), p, 1, nullptr, s);
     return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
                  : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
   }

@@ -50,7 +50,7 @@ __device__ __forceinline__ float group_sum(float v, float* lds) {
 
 // One line per GROUP threads; the line (len % 4 == 0, len <= GROUP*4*MNV_SM_CACHE)
 // is cached in registers.
-template <int GROUP>
+template <int GROUP, int CACHE>
 __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_cached_kernel(
     const float* __restrict__ in, float* __restrict__ out, int len, int lines) {
   __shared__ float lds[MNV_SM_THREADS / MNV_WAVE];
@@ -62,20 +62,20 @@ __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_cached_kernel(
   for (int line = blockIdx.x * LPB + threadIdx.x / GROUP; line < lines; line += gridDim.x * LPB) {
     const mnv_f4* x4 = reinterpret_cast<const mnv_f4*>(in + (size_t)line * len);
     mnv_f4* y4 = reinterpret_cast<mnv_f4*>(out + (size_t)line * len);
-    mnv_f4 v[MNV_SM_CACHE];
+    mnv_f4 v[CACHE];
     float mx = -INFINITY;
 #pragma unroll
-    for (int u = 0; u < MNV_SM_CACHE; ++u) {
+    for (int u = 0; u < CACHE; ++u) {
       int i = t + u * GROUP;
       if (i < len4) {
-        v[u] = x4[i];
+        v[u] = __builtin_nontemporal_load(x4 + i);
         mx = fmaxf(mx, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
       }
     }
     mx = group_max<GROUP>(mx, lds);
     float s = 0.f;
 #pragma unroll
-    for (int u = 0; u < MNV_SM_CACHE; ++u) {
+    for (int u = 0; u < CACHE; ++u) {
       int i = t + u * GROUP;
       if (i < len4) {
         v[u].x = expf(v[u].x - mx);
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_cached_kernel(
     }
     s = group_sum<GROUP>(s, lds);
 #pragma unroll
-    for (int u = 0; u < MNV_SM_CACHE; ++u) {
+    for (int u = 0; u < CACHE; ++u) {
       int i = t + u * GROUP;
       if (i < len4) {
         mnv_f4 o;
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_cached_kernel(
         o.y = v[u].y / s;
         o.z = v[u].z / s;
         o.w = v[u].w / s;
-        y4[i] = o;
+        __builtin_nontemporal_store(o, y4 + i);
       }
     }
   }
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_generic_kernel
   }
 }
 
-template <int GROUP>
+template <int GROUP, int CACHE>
 __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_bwd_cached_kernel(
     const float* __restrict__ dy, const float* __restrict__ y, float* __restrict__ dx, int len,
     int lines) {
@@ -140,20 +140,20 @@ __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_bwd_cached_kernel(
     const mnv_f4* d4 = reinterpret_cast<const mnv_f4*>(dy + (size_t)line * len);
     const mnv_f4* t4 = reinterpret_cast<const mnv_f4*>(y + (size_t)line * len);
     mnv_f4* o4 = reinterpret_cast<mnv_f4*>(dx + (size_t)line * len);
-    mnv_f4 d[MNV_SM_CACHE], p[MNV_SM_CACHE];
+    mnv_f4 d[CACHE], p[CACHE];
     float dot = 0.f;
 #pragma unroll
-    for (int u = 0; u < MNV_SM_CACHE; ++u) {
+    for (int u = 0; u < CACHE; ++u) {
       int i = t + u * GROUP;
       if (i < len4) {
-        d[u] = d4[i];
-        p[u] = t4[i];
+        d[u] = __builtin_nontemporal_load(d4 + i);
+        p[u] = __builtin_nontemporal_load(t4 + i);
         dot += (d[u].x * p[u].x + d[u].y * p[u].y) + (d[u].z * p[u].z + d[u].w * p[u].w);
       }
     }
     dot = group_sum<GROUP>(dot, lds);
 #pragma unroll
-    for (int u = 0; u < MNV_SM_CACHE; ++u) {
+    for (int u = 0; u < CACHE; ++u) {
       int i = t + u * GROUP;
       if (i < len4) {
         mnv_f4 o;
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_bwd_cached_kernel(
         o.y = p[u].y * (d[u].y - dot);
         o.z = p[u].z * (d[u].z - dot);
         o.w = p[u].w * (d[u].w - dot);
-        o4[i] = o;
+        __builtin_nontemporal_store(o, o4 + i);
       }
     }
   }
@@ -235,11 +235,11 @@ unsigned line_grid(int lines, int lpb) {
 int softmax_lines_fwd(const float* in, float* out, int len, int lines, hipStream_t s) {
   bool vec = (len % 4 == 0) && mnv_aligned16(in) && mnv_aligned16(out);
   if (vec && len <= MNV_WAVE * 4 * MNV_SM_CACHE)
-    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_WAVE>), dim3(line_grid(lines, 4)),
-                       dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
+    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_WAVE, MNV_SM_CACHE>),
+                       dim3(line_grid(lines, 4)), dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
   else if (vec && len <= MNV_SM_THREADS * 4 * MNV_SM_CACHE)
-    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_SM_THREADS>), dim3(line_grid(lines, 1)),
-                       dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
+    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_SM_THREADS, MNV_SM_CACHE>),
+                       dim3(line_grid(lines, 1)), dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
   else if (len <= 1024)
     hipLaunchKernelGGL((mnv_softmax_fwd_generic_kernel<MNV_WAVE>), dim3(line_grid(lines, 4)),
                        dim3(MNV_SM_THREADS), 0, s, in, out, len, lines, 1, (size_t)len, (size_t)1);
@@ -253,11 +253,11 @@ int softmax_lines_bwd(const float* dy, const float* y, float* dx, int len, int l
                       hipStream_t s) {
   bool vec = (len % 4 == 0) && mnv_aligned16(dy) && mnv_aligned16(y) && mnv_aligned16(dx);
   if (vec && len <= MNV_WAVE * 4 * MNV_SM_CACHE)
-    hipLaunchKernelGGL((mnv_softmax_bwd_cached_kernel<MNV_WAVE>), dim3(line_grid(lines, 4)),
-                       dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines);
+    hipLaunchKernelGGL((mnv_softmax_bwd_cached_kernel<MNV_WAVE, MNV_SM_CACHE>),
+                       dim3(line_grid(lines, 4)), dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines);
   else if (vec && len <= MNV_SM_THREADS * 4 * MNV_SM_CACHE)
-    hipLaunchKernelGGL((mnv_softmax_bwd_cached_kernel<MNV_SM_THREADS>), dim3(line_grid(lines, 1)),
-                       dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines);
+    hipLaunchKernelGGL((mnv_softmax_bwd_cached_kernel<MNV_SM_THREADS, MNV_SM_CACHE>),
+                       dim3(line_grid(lines, 1)), dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines);
   else if (len <= 1024)
     hipLaunchKernelGGL((mnv_softmax_bwd_generic_kernel<MNV_WAVE>), dim3(line_grid(lines, 4)),
                        dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines, 1, (size_t)len, (size_t)1);
