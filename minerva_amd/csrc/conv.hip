@@ -12,7 +12,6 @@
 // In every case the GEMM "m" dimension is the one that is contiguous in the output
 // tensor, so result stores are coalesced, and no im2col buffer exists in HBM.
 // Roofline: fp32 MFMA, 2*N*Ho*Wo*K*C*R*S algorithmic flops per pass.
-#include <stdlib.h>
 
 #include "gemm_core.h"
 
@@ -444,22 +443,12 @@ int permute_filter(const float* in, float* out, int K, int C, int RS, bool to_cr
 
 typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
-typedef MnvGemmTile<128, 256, 16, 2, 4> TileWide8;   // 8 wavefronts of 64x64
-typedef MnvGemmTile<128, 256, 16, 2, 2> TileWide4;   // 4 wavefronts of 64x128
-typedef MnvGemmTile<256, 128, 16, 4, 2> TileTall8;
-typedef MnvGemmTile<256, 128, 16, 2, 2> TileTall4;
 
+// tile 0: 64x64 output tiles, tile 1: 128x128
 template <class P>
 int launch_tile(int tile, const P& p, int splits, void* ws, hipStream_t s) {
-  if (const char* e = getenv("MNV_CONV_TILE")) tile = atoi(e);
-  switch (tile) {
-    case 0: return mnv_gemm_launch<TileSmall>(p, splits, ws, s);
-    case 2: return mnv_gemm_launch<TileWide8>(p, splits, ws, s);
-    case 3: return mnv_gemm_launch<TileWide4>(p, splits, ws, s);
-    case 4: return mnv_gemm_launch<TileTall8>(p, splits, ws, s);
-    case 5: return mnv_gemm_launch<TileTall4>(p, splits, ws, s);
-    default: return mnv_gemm_launch<TileBig>(p, splits, ws, s);
-  }
+  return tile == 0 ? mnv_gemm_launch<TileSmall>(p, splits, ws, s)
+                   : mnv_gemm_launch<TileBig>(p, splits, ws, s);
 }
 
 int make_geom(ConvGeom* g, int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh,

@@ -70,13 +70,22 @@ struct MnvGemmTile {
   static constexpr int LDA = BM + PAD_, LDB = BN + PAD_;
   static constexpr int AV = BM * BK / (4 * NT);  // 4-vectors of A per thread per slab
   static constexpr int BV = BN * BK / (4 * NT);
-  static constexpr size_t LDS_BYTES = (size_t)2 * BK * (LDA + LDB) * sizeof(float);
+  // LDS floats of one operand tile (one of two buffers).  An x-fast operand is stored
+  // [k][x] (pitch LDA / LDB); a k-fast operand is stored [x][k] with a pitch of BK + 4 so
+  // that a fetched 4-vector is one 16-byte LDS write and the MFMA side reads four k values
+  // per 16-byte LDS read.
+  static constexpr int KP = BK + 4;
+  static constexpr int a_tile(bool kfast) { return kfast ? BM * KP : BK * LDA; }
+  static constexpr int b_tile(bool kfast) { return kfast ? BN * KP : BK * LDB; }
+  static constexpr size_t lds_bytes(bool a_kfast, bool b_kfast) {
+    return (size_t)2 * (a_tile(a_kfast) + b_tile(b_kfast)) * sizeof(float);
+  }
   // Wavefronts per SIMD the register allocation must allow: four 4-wavefront workgroups
   // per CU make 1024 resident tiles, which lets tile counts just under a multiple of
   // 1024 finish in whole rounds.
   static constexpr int MIN_WAVES = (NT == 256 && BM * BN <= 128 * 128 && BK <= 16) ? 4 : 1;
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
-  static_assert(BK % 4 == 0 && (BM * BK) % (4 * NT) == 0 && (BN * BK) % (4 * NT) == 0, "tile/thread mismatch");
+  static_assert(BK % 8 == 0 && (BM * BK) % (4 * NT) == 0 && (BN * BK) % (4 * NT) == 0, "tile/thread mismatch");
 };
 
 // Per-thread position of its fetches inside an operand tile (BX x BK).
@@ -136,8 +145,9 @@ template <class T, class P>
 __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
     P prob, int tiles_m, int tiles_n, int slabs_per_split, float* __restrict__ partial) {
   extern __shared__ float mnv_gemm_lds[];
-  float* As = mnv_gemm_lds;                       // [2][BK][LDA]
-  float* Bs = mnv_gemm_lds + 2 * T::BK * T::LDA;  // [2][BK][LDB]
+  constexpr int ATILE = T::a_tile(P::A_KFAST), BTILE = T::b_tile(P::B_KFAST);
+  float* As = mnv_gemm_lds;              // two buffers of ATILE floats
+  float* Bs = mnv_gemm_lds + 2 * ATILE;  // two buffers of BTILE floats
   typedef MnvFetchMap<T::BM, T::BK, T::NT, P::A_KFAST> MapA;
   typedef MnvFetchMap<T::BN, T::BK, T::NT, P::B_KFAST> MapB;
 
@@ -157,7 +167,7 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
 
   typename P::Res res;
   prob.make_res(res);
-  prob.block_init(res, mnv_gemm_lds + 2 * T::BK * (T::LDA + T::LDB), m0, n0);
+  prob.block_init(res, mnv_gemm_lds + 2 * (ATILE + BTILE), m0, n0);
   typename P::AState ast[T::AV];
   typename P::BState bst[T::BV];
   unsigned aoff[T::AV][P::A_NOFF], boff[T::BV][P::B_NOFF];
@@ -185,29 +195,19 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
       prob.b_load(res, bst[p], boff[p], period, s, MapB::k(tid, p), rb[p]);
   };
   auto stash = [&](int buf) {
-    float* a = As + buf * T::BK * T::LDA;
-    float* bb = Bs + buf * T::BK * T::LDB;
+    float* a = As + buf * ATILE;
+    float* bb = Bs + buf * BTILE;
 #pragma unroll
     for (int p = 0; p < T::AV; ++p) {
       const int x = MapA::x(tid, p), k = MapA::k(tid, p);
-      if (P::A_KFAST) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) a[(k + q) * T::LDA + x] = ra[p][q];
-      } else {
-        mnv_f4 v = {ra[p][0], ra[p][1], ra[p][2], ra[p][3]};
-        *reinterpret_cast<mnv_f4*>(a + k * T::LDA + x) = v;
-      }
+      mnv_f4 v = {ra[p][0], ra[p][1], ra[p][2], ra[p][3]};
+      *reinterpret_cast<mnv_f4*>(a + (P::A_KFAST ? x * T::KP + k : k * T::LDA + x)) = v;
     }
 #pragma unroll
     for (int p = 0; p < T::BV; ++p) {
       const int x = MapB::x(tid, p), k = MapB::k(tid, p);
-      if (P::B_KFAST) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) bb[(k + q) * T::LDB + x] = rb[p][q];
-      } else {
-        mnv_f4 v = {rb[p][0], rb[p][1], rb[p][2], rb[p][3]};
-        *reinterpret_cast<mnv_f4*>(bb + k * T::LDB + x) = v;
-      }
+      mnv_f4 v = {rb[p][0], rb[p][1], rb[p][2], rb[p][3]};
+      *reinterpret_cast<mnv_f4*>(bb + (P::B_KFAST ? x * T::KP + k : k * T::LDB + x)) = v;
     }
   };
 
@@ -243,20 +243,43 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
       new_period(++period);
     }
     fetch(period, s);
-    const float* a = As + buf * T::BK * T::LDA + wm + lm;
-    const float* bb = Bs + buf * T::BK * T::LDB + wn + lm;
+    // A round multiplies 8 k values: MFMA step t pairs k = 8h + t (lanes 0..31) with
+    // k = 8h + 4 + t (lanes 32..63), so a lane's four steps use four consecutive k.
+    const float* a = As + buf * ATILE;
+    const float* bb = Bs + buf * BTILE;
 #pragma unroll
-    for (int kk = 0; kk < T::BK / 2; ++kk) {
-      float av[T::TM], bv[T::TN];
+    for (int h = 0; h < T::BK / 8; ++h) {
+      float av[T::TM][4], bv[T::TN][4];
+      const int kq = 8 * h + 4 * lk;
 #pragma unroll
-      for (int i = 0; i < T::TM; ++i) av[i] = a[(kk * 2 + lk) * T::LDA + i * 32];
+      for (int i = 0; i < T::TM; ++i) {
+        const int x = wm + i * 32 + lm;
+        if (P::A_KFAST) {
+          mnv_f4 v = *reinterpret_cast<const mnv_f4*>(a + x * T::KP + kq);
+          av[i][0] = v.x; av[i][1] = v.y; av[i][2] = v.z; av[i][3] = v.w;
+        } else {
 #pragma unroll
-      for (int j = 0; j < T::TN; ++j) bv[j] = bb[(kk * 2 + lk) * T::LDB + j * 32];
+          for (int t = 0; t < 4; ++t) av[i][t] = a[(kq + t) * T::LDA + x];
+        }
+      }
 #pragma unroll
-      for (int i = 0; i < T::TM; ++i)
+      for (int j = 0; j < T::TN; ++j) {
+        const int x = wn + j * 32 + lm;
+        if (P::B_KFAST) {
+          mnv_f4 v = *reinterpret_cast<const mnv_f4*>(bb + x * T::KP + kq);
+          bv[j][0] = v.x; bv[j][1] = v.y; bv[j][2] = v.z; bv[j][3] = v.w;
+        } else {
 #pragma unroll
-        for (int j = 0; j < T::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j], av[i], acc[i][j], 0, 0, 0);
+          for (int t = 0; t < 4; ++t) bv[j][t] = bb[(kq + t) * T::LDB + x];
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+          for (int j = 0; j < T::TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j][t], av[i][t], acc[i][j], 0, 0, 0);
     }
     stash(buf ^ 1);
     __syncthreads();
@@ -310,12 +333,13 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
   splits = total_slabs > 0 ? (total_slabs + per - 1) / per : 1;
   if ((long long)tiles_m * tiles_n > 0x7fffffffLL || splits > 65535) return MNV_ERR_INVALID;
   static bool attr_set = false;  // idempotent; a race only repeats the same call
-  if (!attr_set && T::LDS_BYTES + prob.extra_lds_bytes() > 48 * 1024) {
+  const size_t tile_bytes = T::lds_bytes(P::A_KFAST, P::B_KFAST);
+  if (!attr_set && tile_bytes + prob.extra_lds_bytes() > 48 * 1024) {
     MNV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&mnv_gemm_kernel<T, P>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
     attr_set = true;
   }
-  const size_t lds_bytes = T::LDS_BYTES + prob.extra_lds_bytes();
+  const size_t lds_bytes = tile_bytes + prob.extra_lds_bytes();
   if (lds_bytes > 64 * 1024) return MNV_ERR_INVALID;
   hipLaunchKernelGGL((mnv_gemm_kernel<T, P>), dim3(tiles_m * tiles_n, 1, splits), dim3(T::NT),
                      lds_bytes, s, prob, tiles_m, tiles_n, per,

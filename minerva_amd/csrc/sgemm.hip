@@ -4,8 +4,6 @@
 // Built on the fp32 MFMA core in gemm_core.h; A is fetched x-fast (m contiguous),
 // B k-fast (k contiguous).  Products with too few output tiles to fill 256 CUs split
 // the k range over blockIdx.z when the caller lends a workspace.
-#include <stdlib.h>
-
 #include "gemm_core.h"
 
 namespace {
@@ -74,24 +72,6 @@ SgemmNN<VEC> make_sgemm(const float* a, const float* b, float* c, int m, int n, 
 
 typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
-typedef MnvGemmTile<128, 128, 32, 2, 2> TileBig32;
-typedef MnvGemmTile<128, 128, 16, 2, 2, 32> TileBigPad32;
-typedef MnvGemmTile<128, 128, 16, 2, 2, 4> TileBigPad4;
-typedef MnvGemmTile<256, 128, 16, 4, 2> TileTall8;
-typedef MnvGemmTile<256, 256, 16, 4, 2> TileHuge8;
-
-template <class P>
-int sgemm_launch_exp(int tile, P p, int splits, void* ws, hipStream_t s) {
-  switch (tile) {
-    case 2: p.set_bk(32); return mnv_gemm_launch<TileBig32>(p, splits, ws, s);
-    case 3: return mnv_gemm_launch<TileBigPad32>(p, splits, ws, s);
-    case 4: return mnv_gemm_launch<TileBigPad4>(p, splits, ws, s);
-    case 5: return mnv_gemm_launch<TileTall8>(p, splits, ws, s);
-    case 6: return mnv_gemm_launch<TileHuge8>(p, splits, ws, s);
-    default: return mnv_gemm_launch<TileBig>(p, splits, ws, s);
-  }
-}
-
 #define MNV_SGEMM_MAX_SPLITS 16
 
 // How many k ranges to use for an (m,n,k) product given `ws_floats` floats of scratch.
@@ -141,7 +121,6 @@ int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k, 
   int splits = pick_splits(tiles, slabs, (size_t)m * n, ws_floats);
   if (vec) {
     SgemmNN<true> p = make_sgemm<true>(a, b, c, m, n, k);
-    if (const char* e = getenv("MNV_SGEMM_TILE")) return sgemm_launch_exp(atoi(e), p, 1, nullptr, s);
     return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
                  : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
   }

@@ -48,6 +48,8 @@ def mlp_step(p, data, label, lr, batch, din=784, hid=256, dout=10):
     newp = {k: _sgd(p[k], g[k], lr, batch) for k in p}
     res = {"prob": a3}
     res.update({"g_" + k: v for k, v in g.items()})
+    res["l1_b0"] = ora.reduction(ora.SUM, np.abs(s1), [hid, batch], [1])
+    res["l1_b1"] = ora.reduction(ora.SUM, np.abs(s2), [dout, batch], [1])
     return newp, res
 
 
@@ -85,6 +87,9 @@ def cnn_step(p, data, label, lr, batch, pad2=0, pool2=2):
     newp = {k: _sgd(p[k], g[k], lr, batch) for k in p}
     res = {"prob": a8}
     res.update({"g_" + k: v for k, v in g.items()})
+    res["l1_b0"] = ora.conv_bwd_bias(np.abs(s1), N, 16, 24, 24)
+    res["l1_b1"] = ora.conv_bwd_bias(np.abs(s4), N, 32, h2, h2)
+    res["l1_b2"] = ora.reduction(ora.SUM, np.abs(s7), [10, N], [1])
     return newp, res
 
 
@@ -159,6 +164,15 @@ def alexnet_step(p, data, label, lr, batch, classes=1000):
     newp = {k: _sgd(p[k], g[k], lr, batch) for k in p}
     res = {"prob": out}
     res.update({"g_" + k: v for k, v in g.items()})
+    # L1 mass behind every bias gradient: the scale its rounding error is measured against
+    res["l1_b7"] = ora.reduction(ora.SUM, np.abs(sens[11]), [classes, N], [1])
+    res["l1_b6"] = ora.reduction(ora.SUM, np.abs(sens[10]), [4096, N], [1])
+    res["l1_b5"] = ora.reduction(ora.SUM, np.abs(sens[9]), [4096, N], [1])
+    res["l1_b4"] = ora.conv_bwd_bias(np.abs(sens[7]), N, 256, 13, 13)
+    res["l1_b3"] = ora.conv_bwd_bias(np.abs(sens[6]), N, 384, 13, 13)
+    res["l1_b2"] = ora.conv_bwd_bias(np.abs(sens[5]), N, 384, 13, 13)
+    res["l1_b1"] = ora.conv_bwd_bias(np.abs(sens[3]), N, 256, 27, 27)
+    res["l1_b0"] = ora.conv_bwd_bias(np.abs(sens[1]), N, 96, 55, 55)
     return newp, res
 
 
