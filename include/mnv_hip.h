@@ -211,8 +211,12 @@ int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filte
                         int stride_vertical, int stride_horizontal, int filter_height,
                         int filter_width, void* workspace, size_t workspace_bytes,
                         mnv_stream_t stream);
+/* workspace (optional; 0 bytes = one workgroup per channel) lets each channel's sum be split
+ * over image groups whose partial sums are added in a fixed order. */
+size_t mnv_conv_bwd_bias_workspace_bytes(int num_images, int top_num_channels);
 int mnv_conv_bwd_bias(const float* top_diff, float* bias_diff, int num_images,
-                      int top_num_channels, int top_height, int top_width, mnv_stream_t stream);
+                      int top_num_channels, int top_height, int top_width, void* workspace,
+                      size_t workspace_bytes, mnv_stream_t stream);
 
 /* ---- pooling: CudaPerform{Max,Average}Pooling{Forward,Backward}
  * (cuda_perform.h:61-64).  pooled = (in + 2*pad - window + stride - 1)/stride + 1,

@@ -55,7 +55,8 @@ PROTOTYPES = {
     "mnv_conv_bwd_data": [_P, _P, _P] + [_I] * 11 + [_P, c_sz, _S],
     "mnv_conv_bwd_filter_workspace_bytes": [_I] * 11,
     "mnv_conv_bwd_filter": [_P, _P, _P] + [_I] * 11 + [_P, c_sz, _S],
-    "mnv_conv_bwd_bias": [_P, _P, _I, _I, _I, _I, _S],
+    "mnv_conv_bwd_bias": [_P, _P, _I, _I, _I, _I, _P, c_sz, _S],
+    "mnv_conv_bwd_bias_workspace_bytes": [_I, _I],
     "mnv_pooled_size": [_I, _I, _I, _I],
 }
 for _n in ("add", "sub", "mul", "div"):
@@ -85,6 +86,7 @@ _RESTYPES = {
     "mnv_conv_bwd_filter_workspace_bytes": c_sz,
     "mnv_conv_fwd_workspace_bytes": c_sz,
     "mnv_conv_bwd_data_workspace_bytes": c_sz,
+    "mnv_conv_bwd_bias_workspace_bytes": c_sz,
 }
 
 

@@ -22,27 +22,7 @@
 
 typedef float mnv_f16v __attribute__((ext_vector_type(16)));
 
-// Division by a run-time constant d >= 1, prepared on the host; valid for 0 <= n < 2^31
-// and branch-free (d == 1 gives mul == 0, shift == 0):  n / d == (mulhi(n, mul) + n) >> shift.
-struct MnvFastDiv {
-  unsigned mul, shift;
-};
-
-static inline MnvFastDiv mnv_fastdiv_make(int d) {
-  MnvFastDiv f;
-  unsigned s = 0;
-  while ((1ull << s) < (unsigned long long)d) ++s;  // ceil(log2 d)
-  f.shift = s;
-  f.mul = (unsigned)((((1ull << s) - (unsigned long long)d) << 32) / (unsigned long long)d + 1);
-  if (d <= 1) f.mul = 0;
-  return f;
-}
-
 #ifdef __HIPCC__
-__device__ __forceinline__ int mnv_fastdiv(int n, const MnvFastDiv& f) {
-  return (int)((__umulhi((unsigned)n, f.mul) + (unsigned)n) >> f.shift);
-}
-
 // Buffer addressing: every operand is read through a raw buffer resource whose extent is
 // the tensor's byte size, so a masked-off element is fetched with an offset past the end
 // and the hardware returns 0 for it: no divergent branch, no address clamp, no fault.

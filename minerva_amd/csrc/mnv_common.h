@@ -28,7 +28,27 @@ static inline size_t mnv_ceil_div(size_t a, size_t b) { return (a + b - 1) / b; 
 // 256 CUs without paying launch cost for millions of tiny blocks.
 #define MNV_MAX_STREAM_BLOCKS 16384u
 
+// Division by a run-time constant d >= 1, prepared on the host; valid for 0 <= n < 2^31
+// and branch-free (d == 1 gives mul == 0, shift == 0):  n / d == (mulhi(n, mul) + n) >> shift.
+struct MnvFastDiv {
+  unsigned mul, shift;
+};
+
+static inline MnvFastDiv mnv_fastdiv_make(int d) {
+  MnvFastDiv f;
+  unsigned s = 0;
+  while ((1ull << s) < (unsigned long long)d) ++s;  // ceil(log2 d)
+  f.shift = s;
+  f.mul = (unsigned)((((1ull << s) - (unsigned long long)d) << 32) / (unsigned long long)d + 1);
+  if (d <= 1) f.mul = 0;
+  return f;
+}
+
 #ifdef __HIPCC__
+__device__ __forceinline__ int mnv_fastdiv(int n, const MnvFastDiv& f) {
+  return (int)((__umulhi((unsigned)n, f.mul) + (unsigned)n) >> f.shift);
+}
+
 typedef float mnv_f4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float mnv_wave_sum(float v) {

@@ -26,6 +26,7 @@ namespace {
 
 struct PoolGeom {
   int H, W, Ho, Wo, sv, sh, kh, kw, ph, pw;
+  MnvFastDiv d_hw, d_howo, d_W, d_Wo, d_sv, d_sh;  // run-time integer division is ~40 instructions
 };
 
 __device__ __forceinline__ int ceil_div_pos(int a, int b) {  // b > 0, any a
@@ -60,8 +61,8 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_fwd_lds_kernel(
     stage(bottom + (size_t)p0 * hw, lds, np * hw);
     __syncthreads();
     for (int q = threadIdx.x; q < np * howo; q += MNV_POOL_THREADS) {
-      int pl = q / howo, o = q - pl * howo;
-      int i = o / g.Wo, j = o - i * g.Wo;
+      int pl = mnv_fastdiv(q, g.d_howo), o = q - pl * howo;
+      int i = mnv_fastdiv(o, g.d_Wo), j = o - i * g.Wo;
       int y0 = i * g.sv - g.ph, x0 = j * g.sh - g.pw;
       int ys = max(y0, 0), xs = max(x0, 0);
       int ye = min(y0 + g.kh, g.H), xe = min(x0 + g.kw, g.W);
@@ -104,8 +105,8 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_lds_kernel(
     if (MAX) {
       // first maximum of every window in scan order (strict '<'), as a flat position
       for (int q = threadIdx.x; q < np * howo; q += MNV_POOL_THREADS) {
-        int pl = q / howo, o = q - pl * howo;
-        int i = o / g.Wo, j = o - i * g.Wo;
+        int pl = mnv_fastdiv(q, g.d_howo), o = q - pl * howo;
+        int i = mnv_fastdiv(o, g.d_Wo), j = o - i * g.Wo;
         int y0 = i * g.sv - g.ph, x0 = j * g.sh - g.pw;
         int ys = max(y0, 0), xs = max(x0, 0);
         int ye = min(y0 + g.kh, g.H), xe = min(x0 + g.kw, g.W);
@@ -125,12 +126,14 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_lds_kernel(
       __syncthreads();
     }
     for (int q = threadIdx.x; q < np * hw; q += MNV_POOL_THREADS) {
-      int pl = q / hw, pos = q - pl * hw;
-      int y = pos / g.W, x = pos - y * g.W;
-      int i_lo = max(ceil_div_pos(y + g.ph - g.kh + 1, g.sv), 0);
-      int i_hi = min((y + g.ph) / g.sv, g.Ho - 1);
-      int j_lo = max(ceil_div_pos(x + g.pw - g.kw + 1, g.sh), 0);
-      int j_hi = min((x + g.pw) / g.sh, g.Wo - 1);
+      int pl = mnv_fastdiv(q, g.d_hw), pos = q - pl * hw;
+      int y = mnv_fastdiv(pos, g.d_W), x = pos - y * g.W;
+      // windows i with i*sv - ph <= y < i*sv - ph + kh, clipped to [0, Ho)
+      int ay = y + g.ph - g.kh + g.sv, ax = x + g.pw - g.kw + g.sh;  // ceil((y+ph-kh+1)/sv)
+      int i_lo = ay > 0 ? mnv_fastdiv(ay, g.d_sv) : 0;
+      int i_hi = min(mnv_fastdiv(y + g.ph, g.d_sv), g.Ho - 1);
+      int j_lo = ax > 0 ? mnv_fastdiv(ax, g.d_sh) : 0;
+      int j_hi = min(mnv_fastdiv(x + g.pw, g.d_sh), g.Wo - 1);
       float acc = 0.f;
       for (int i = i_lo; i <= i_hi; ++i)
         for (int j = j_lo; j <= j_hi; ++j) {
@@ -232,6 +235,12 @@ int make_geom(PoolGeom* g, int n, int c, int h, int w, int sv, int sh, int kh, i
   g->Ho = mnv_pooled_size(h, kh, sv, ph);
   g->Wo = mnv_pooled_size(w, kw, sh, pw);
   if (g->Ho <= 0 || g->Wo <= 0) return MNV_ERR_INVALID;
+  g->d_hw = mnv_fastdiv_make(h * w);
+  g->d_howo = mnv_fastdiv_make(g->Ho * g->Wo);
+  g->d_W = mnv_fastdiv_make(w);
+  g->d_Wo = mnv_fastdiv_make(g->Wo);
+  g->d_sv = mnv_fastdiv_make(sv);
+  g->d_sh = mnv_fastdiv_make(sh);
   return MNV_OK;
 }
 

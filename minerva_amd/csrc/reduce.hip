@@ -233,46 +233,73 @@ int launch_reduce_row(const float* in, float* out, int m, int n, mnv_stream_t st
 
 // ---------------------------------------------------------------------------
 // Convolution bias gradient: db[k] = sum over images and positions of dY[n,k,:,:]
-// (reference cuda_perform.cu:320-337).  One workgroup per output channel; its 16
-// wavefronts take images round-robin and read each hw-long row contiguously.
+// (reference cuda_perform.cu:320-337).  A channel's data is N runs of hw contiguous
+// floats, one per image.  Workgroup (k, g) sums channel k over image group g: its four
+// wavefronts take the group's images round-robin and read each run with 16-byte loads
+// from its first aligned address (at most three single floats on either side).  With
+// several groups per channel the group sums go to a scratch area and a second, tiny
+// kernel adds them in group order, so the result does not depend on scheduling.
 // ---------------------------------------------------------------------------
-#define MNV_BIAS_THREADS 1024
+#define MNV_BIAS_THREADS 256
 
-template <bool VEC4>
 __global__ __launch_bounds__(MNV_BIAS_THREADS) void mnv_conv_bwd_bias_kernel(
-    const float* __restrict__ top_diff, float* __restrict__ bias_diff, int N, int K, int hw) {
-  __shared__ float part[MNV_BIAS_THREADS / MNV_WAVE];
-  const int k = blockIdx.x;
-  const int wave = threadIdx.x / MNV_WAVE, lane = threadIdx.x % MNV_WAVE;
+    const float* __restrict__ top_diff, float* __restrict__ out, int N, int K, int hw,
+    int images_per_group) {
   constexpr int NW = MNV_BIAS_THREADS / MNV_WAVE;
-  float s0 = 0.f, s1 = 0.f;
-  for (int img = wave; img < N; img += NW) {
+  __shared__ float part[NW];
+  const int k = blockIdx.x, g = blockIdx.y;
+  const int wave = threadIdx.x / MNV_WAVE, lane = threadIdx.x % MNV_WAVE;
+  const int img_end = min(N, (g + 1) * images_per_group);
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  for (int img = g * images_per_group + wave; img < img_end; img += NW) {
     const float* p = top_diff + ((size_t)img * K + k) * hw;
-    if (VEC4) {
-      const mnv_f4* p4 = reinterpret_cast<const mnv_f4*>(p);
-      const int hw4 = hw >> 2;
-      int i = lane;
-      for (; i + MNV_WAVE < hw4; i += 2 * MNV_WAVE) {
-        mnv_f4 a = p4[i], b = p4[i + MNV_WAVE];
-        s0 += (a.x + a.y) + (a.z + a.w);
-        s1 += (b.x + b.y) + (b.z + b.w);
-      }
-      if (i < hw4) {
-        mnv_f4 a = p4[i];
-        s0 += (a.x + a.y) + (a.z + a.w);
-      }
-    } else {
-      for (int i = lane; i < hw; i += MNV_WAVE) s0 += p[i];
+    int head = (int)((4 - ((reinterpret_cast<uintptr_t>(p) >> 2) & 3)) & 3);
+    if (head > hw) head = hw;
+    const int n4 = (hw - head) >> 2, tail = (hw - head) & 3;
+    const mnv_f4* p4 = reinterpret_cast<const mnv_f4*>(p + head);
+    if (lane < head) s0 += p[lane];
+    if (lane < tail) s1 += p[head + 4 * n4 + lane];
+    int i = lane;
+    for (; i + 3 * MNV_WAVE < n4; i += 4 * MNV_WAVE) {
+      mnv_f4 a = p4[i], b = p4[i + MNV_WAVE], c = p4[i + 2 * MNV_WAVE], d = p4[i + 3 * MNV_WAVE];
+      s0 += (a.x + a.y) + (a.z + a.w);
+      s1 += (b.x + b.y) + (b.z + b.w);
+      s2 += (c.x + c.y) + (c.z + c.w);
+      s3 += (d.x + d.y) + (d.z + d.w);
+    }
+    for (; i < n4; i += MNV_WAVE) {
+      mnv_f4 a = p4[i];
+      s0 += (a.x + a.y) + (a.z + a.w);
     }
   }
-  float s = mnv_wave_sum(s0 + s1);
+  float s = mnv_wave_sum((s0 + s1) + (s2 + s3));
   if (lane == 0) part[wave] = s;
   __syncthreads();
   if (threadIdx.x == 0) {
     float t = 0.f;
     for (int q = 0; q < NW; ++q) t += part[q];
-    bias_diff[k] = t;
+    out[(size_t)k * gridDim.y + g] = t;
   }
+}
+
+__global__ __launch_bounds__(256) void mnv_conv_bwd_bias_finish_kernel(
+    const float* __restrict__ partial, float* __restrict__ bias_diff, int K, int groups) {
+  const int k = blockIdx.x * 256 + threadIdx.x;
+  if (k >= K) return;
+  float t = 0.f;
+  for (int g = 0; g < groups; ++g) t += partial[(size_t)k * groups + g];
+  bias_diff[k] = t;
+}
+
+// Image groups per channel: enough workgroups to fill the chip, at least four images
+// per wavefront's worth of work in each.
+int bias_groups(int num_images, int channels) {
+  int want = (2048 + channels - 1) / channels;
+  int max_groups = (num_images + 3) / 4;
+  if (want > max_groups) want = max_groups;
+  if (want < 1) want = 1;
+  int per = (num_images + want - 1) / want;
+  return (num_images + per - 1) / per;
 }
 
 }  // namespace
@@ -298,23 +325,35 @@ int mnv_maxindex_row(const float* in, float* out, int m, int n, mnv_stream_t s) 
   return launch_reduce_row<ArgAcc, EmitIndex>(in, out, m, n, s);
 }
 
+size_t mnv_conv_bwd_bias_workspace_bytes(int num_images, int top_num_channels) {
+  if (num_images <= 0 || top_num_channels <= 0) return 0;
+  int groups = bias_groups(num_images, top_num_channels);
+  return groups > 1 ? (size_t)groups * top_num_channels * sizeof(float) : 0;
+}
+
 int mnv_conv_bwd_bias(const float* top_diff, float* bias_diff, int num_images,
-                      int top_num_channels, int top_height, int top_width, mnv_stream_t stream) {
+                      int top_num_channels, int top_height, int top_width, void* workspace,
+                      size_t workspace_bytes, mnv_stream_t stream) {
   if (top_num_channels == 0) return MNV_OK;
   if (!top_diff || !bias_diff || num_images <= 0 || top_num_channels < 0 || top_height <= 0 ||
       top_width <= 0)
     return MNV_ERR_INVALID;
   long long hw = (long long)top_height * top_width;
-  if (hw > 0x7fffffffLL) return MNV_ERR_INVALID;
-  bool vec4 = (hw % 4 == 0) && mnv_aligned16(top_diff);
-  if (vec4)
-    hipLaunchKernelGGL((mnv_conv_bwd_bias_kernel<true>), dim3(top_num_channels),
-                       dim3(MNV_BIAS_THREADS), 0, mnv_stream(stream), top_diff, bias_diff,
-                       num_images, top_num_channels, (int)hw);
-  else
-    hipLaunchKernelGGL((mnv_conv_bwd_bias_kernel<false>), dim3(top_num_channels),
-                       dim3(MNV_BIAS_THREADS), 0, mnv_stream(stream), top_diff, bias_diff,
-                       num_images, top_num_channels, (int)hw);
+  if (hw > 0x7fffffffLL || top_num_channels > 0x7fffffff / 2) return MNV_ERR_INVALID;
+  int groups = bias_groups(num_images, top_num_channels);
+  if (groups > 65535) groups = 65535;
+  if (!workspace || workspace_bytes < (size_t)groups * top_num_channels * sizeof(float)) groups = 1;
+  int per = (num_images + groups - 1) / groups;
+  hipStream_t s = mnv_stream(stream);
+  float* out = groups > 1 ? reinterpret_cast<float*>(workspace) : bias_diff;
+  hipLaunchKernelGGL(mnv_conv_bwd_bias_kernel, dim3(top_num_channels, groups),
+                     dim3(MNV_BIAS_THREADS), 0, s, top_diff, out, num_images, top_num_channels,
+                     (int)hw, per);
+  int rc = MNV_LAUNCH_STATUS();
+  if (rc || groups == 1) return rc;
+  hipLaunchKernelGGL(mnv_conv_bwd_bias_finish_kernel, dim3((top_num_channels + 255) / 256),
+                     dim3(256), 0, s, reinterpret_cast<const float*>(workspace), bias_diff,
+                     top_num_channels, groups);
   return MNV_LAUNCH_STATUS();
 }
 

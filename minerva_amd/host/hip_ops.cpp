@@ -290,7 +290,8 @@ void ConvBackwardBias(const DataList& inputs, const DataList& outputs, ConvBackw
   MNV_CHECK_EQ(outputs.size(), 1u) << "(conv backward bias) #outputs wrong";
   auto& top_diff = inputs[0];
   Ok(mnv_conv_bwd_bias(top_diff.data_, outputs[0].data_, top_diff.size_[3], top_diff.size_[2],
-                       top_diff.size_[1], top_diff.size_[0], ctx.stream),
+                       top_diff.size_[1], top_diff.size_[0], ctx.workspace, ctx.workspace_bytes,
+                       ctx.stream),
      "conv backward bias");
 }
 

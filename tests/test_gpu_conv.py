@@ -69,10 +69,13 @@ class Conv:
                ctypes.c_size_t(nbytes))
         return g.down(dfd)
 
-    def bwd_bias(self, dy):
+    def bwd_bias(self, dy, workspace=True):
         g, p = self.gpu, self.p
         ddy, db = g.up(dy), g.empty(p[2])
-        g.call("mnv_conv_bwd_bias", ddy.p, db.p, p[0], p[2], self.Ho, self.Wo)
+        nbytes = g.L.mnv_conv_bwd_bias_workspace_bytes(p[0], p[2]) if workspace else 0
+        ws = g.empty(nbytes // 4 + 1) if nbytes else None
+        g.call("mnv_conv_bwd_bias", ddy.p, db.p, p[0], p[2], self.Ho, self.Wo,
+               ws.p if ws else None, ctypes.c_size_t(nbytes))
         return g.down(db)
 
 
@@ -130,8 +133,10 @@ def test_conv_all_passes_against_oracle(gpu, ora, p):
     for ws in (True, False):
         say("conv bwd filter", p, ws)
         assert normwise(cv.bwd_filter(dy, x, ws), ref) <= TOL
-    say("conv bwd bias", p)
-    assert normwise(cv.bwd_bias(dy), ora.conv_bwd_bias(dy, N, K, cv.Ho, cv.Wo)) <= TOL
+    ref = ora.conv_bwd_bias(dy, N, K, cv.Ho, cv.Wo)
+    for ws in (True, False):
+        say("conv bwd bias", p, ws)
+        assert normwise(cv.bwd_bias(dy, ws), ref) <= TOL
 
 
 ALEXNET = [
