@@ -494,12 +494,11 @@ int bwd_filter_splits(int m, int n, int k, size_t ws_floats) {
   int bm = small ? 64 : 128;
   long long tiles = (long long)((m + bm - 1) / bm) * ((n + bm - 1) / bm);
   int slabs = (k + 15) / 16;
-  long long want = (1024 + tiles - 1) / tiles;
-  if (want > MNV_BWDF_MAX_SPLITS) want = MNV_BWDF_MAX_SPLITS;
-  if (want > slabs / 8) want = slabs / 8;
+  int max_splits = MNV_BWDF_MAX_SPLITS;
+  if (max_splits > slabs / 8) max_splits = slabs / 8;
   size_t fit = ws_floats / ((size_t)m * n);
-  if ((size_t)want > fit) want = (long long)fit;
-  return want < 1 ? 1 : (int)want;
+  if ((size_t)max_splits > fit) max_splits = (int)fit;
+  return mnv_pick_splits(tiles, slabs, max_splits);
 }
 
 }  // namespace

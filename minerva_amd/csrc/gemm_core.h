@@ -51,12 +51,18 @@ struct MnvGemmTile {
   static constexpr int AV = BM * BK / (4 * NT);  // 4-vectors of A per thread per slab
   static constexpr int BV = BN * BK / (4 * NT);
   // LDS floats of one operand tile (one of two buffers).  An x-fast operand is stored
-  // [k][x] (pitch LDA / LDB); a k-fast operand is stored [x][k] with a pitch of BK + 4 so
-  // that a fetched 4-vector is one 16-byte LDS write and the MFMA side reads four k values
-  // per 16-byte LDS read.
-  static constexpr int KP = BK + 4;
-  static constexpr int a_tile(bool kfast) { return kfast ? BM * KP : BK * LDA; }
-  static constexpr int b_tile(bool kfast) { return kfast ? BN * KP : BK * LDB; }
+  // [k][x] (pitch LDA / LDB).  A k-fast operand is stored [x][k] with no padding, so that a
+  // fetched 4-vector is one 16-byte LDS write and the MFMA side reads four k values per
+  // 16-byte LDS read; the 16-byte chunks of row x are permuted by XOR with kswz(x), which
+  // spreads both the writes (consecutive chunks of two rows per eight lanes) and the reads
+  // (one chunk of eight consecutive rows) over all 32 banks.
+  static constexpr int KCH = BK / 4;  // 16-byte chunks per row
+  __host__ __device__ static constexpr int kswz(int x) { return (x / (32 / BK)) & (KCH - 1); }
+  __host__ __device__ static constexpr int kaddr(int x, int chunk) {
+    return x * BK + ((chunk ^ kswz(x)) << 2);
+  }
+  static constexpr int a_tile(bool kfast) { return kfast ? BM * BK : BK * LDA; }
+  static constexpr int b_tile(bool kfast) { return kfast ? BN * BK : BK * LDB; }
   static constexpr size_t lds_bytes(bool a_kfast, bool b_kfast) {
     return (size_t)2 * (a_tile(a_kfast) + b_tile(b_kfast)) * sizeof(float);
   }
@@ -65,7 +71,9 @@ struct MnvGemmTile {
   // 1024 finish in whole rounds.
   static constexpr int MIN_WAVES = (NT == 256 && BM * BN <= 128 * 128 && BK <= 16) ? 4 : 1;
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
-  static_assert(BK % 8 == 0 && (BM * BK) % (4 * NT) == 0 && (BN * BK) % (4 * NT) == 0, "tile/thread mismatch");
+  static_assert((BK == 8 || BK == 16 || BK == 32) && (BM * BK) % (4 * NT) == 0 &&
+                    (BN * BK) % (4 * NT) == 0,
+                "tile/thread mismatch");
 };
 
 // Per-thread position of its fetches inside an operand tile (BX x BK).
@@ -181,13 +189,13 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
     for (int p = 0; p < T::AV; ++p) {
       const int x = MapA::x(tid, p), k = MapA::k(tid, p);
       mnv_f4 v = {ra[p][0], ra[p][1], ra[p][2], ra[p][3]};
-      *reinterpret_cast<mnv_f4*>(a + (P::A_KFAST ? x * T::KP + k : k * T::LDA + x)) = v;
+      *reinterpret_cast<mnv_f4*>(a + (P::A_KFAST ? T::kaddr(x, k >> 2) : k * T::LDA + x)) = v;
     }
 #pragma unroll
     for (int p = 0; p < T::BV; ++p) {
       const int x = MapB::x(tid, p), k = MapB::k(tid, p);
       mnv_f4 v = {rb[p][0], rb[p][1], rb[p][2], rb[p][3]};
-      *reinterpret_cast<mnv_f4*>(bb + (P::B_KFAST ? x * T::KP + k : k * T::LDB + x)) = v;
+      *reinterpret_cast<mnv_f4*>(bb + (P::B_KFAST ? T::kaddr(x, k >> 2) : k * T::LDB + x)) = v;
     }
   };
 
@@ -235,7 +243,7 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
       for (int i = 0; i < T::TM; ++i) {
         const int x = wm + i * 32 + lm;
         if (P::A_KFAST) {
-          mnv_f4 v = *reinterpret_cast<const mnv_f4*>(a + x * T::KP + kq);
+          mnv_f4 v = *reinterpret_cast<const mnv_f4*>(a + T::kaddr(x, kq >> 2));
           av[i][0] = v.x; av[i][1] = v.y; av[i][2] = v.z; av[i][3] = v.w;
         } else {
 #pragma unroll
@@ -246,7 +254,7 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
       for (int j = 0; j < T::TN; ++j) {
         const int x = wn + j * 32 + lm;
         if (P::B_KFAST) {
-          mnv_f4 v = *reinterpret_cast<const mnv_f4*>(bb + x * T::KP + kq);
+          mnv_f4 v = *reinterpret_cast<const mnv_f4*>(bb + T::kaddr(x, kq >> 2));
           bv[j][0] = v.x; bv[j][1] = v.y; bv[j][2] = v.z; bv[j][3] = v.w;
         } else {
 #pragma unroll
@@ -298,6 +306,29 @@ __global__ __launch_bounds__(256) void mnv_gemm_splitk_reduce_kernel(P prob,
     for (int z = 1; z < splits; ++z) s += partial[(size_t)z * mn + q];
     prob.c_store((int)(q % prob.M), (int)(q / prob.M), s);
   }
+}
+
+// Number of k ranges for `tiles` output tiles of `slabs` k-slabs each.  Workgroups are
+// dealt evenly to 256 CUs that hold four of them at a time, and the kernel ends when the
+// fullest CU does: a split count that puts a few workgroups past a multiple of 1024 costs a
+// whole extra round, so the estimate below (workgroups on the fullest CU x slabs each,
+// corrected for the matrix pipe running below its rate with fewer than four workgroups in
+// residence) is minimised rather than the count simply rounded up.
+static inline int mnv_pick_splits(long long tiles, int slabs, int max_splits) {
+  static const double rate[5] = {1.0, 0.45, 0.75, 0.92, 1.0};
+  if (max_splits < 1) max_splits = 1;
+  int best = 1;
+  double best_cost = 0;
+  for (int s = 1; s <= max_splits; ++s) {
+    long long per_cu = (tiles * s + 255) / 256;
+    int len = (slabs + s - 1) / s;
+    double cost = (double)per_cu * (len + 4) / rate[per_cu < 4 ? per_cu : 4];
+    if (s == 1 || cost < best_cost * 0.98) {  // prefer fewer partial results on a near tie
+      best = s;
+      best_cost = cost;
+    }
+  }
+  return best;
 }
 
 // Host-side launch of one tile configuration.  `splits` > 1 needs

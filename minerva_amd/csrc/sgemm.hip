@@ -76,13 +76,12 @@ typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
 
 // How many k ranges to use for an (m,n,k) product given `ws_floats` floats of scratch.
 int pick_splits(int tiles, int slabs, size_t mn, size_t ws_floats) {
-  if (tiles >= 256 || slabs < 8) return 1;
-  int want = (512 + tiles - 1) / tiles;
-  if (want > MNV_SGEMM_MAX_SPLITS) want = MNV_SGEMM_MAX_SPLITS;
-  if (want > slabs / 4) want = slabs / 4;
+  if (tiles >= 1024 || slabs < 8) return 1;
+  int max_splits = MNV_SGEMM_MAX_SPLITS;
+  if (max_splits > slabs / 4) max_splits = slabs / 4;
   size_t fit = mn ? ws_floats / mn : 0;
-  if ((size_t)want > fit) want = (int)fit;
-  return want < 1 ? 1 : want;
+  if ((size_t)max_splits > fit) max_splits = (int)fit;
+  return mnv_pick_splits(tiles, slabs, max_splits);
 }
 
 bool use_small_tile(int m, int n) {
