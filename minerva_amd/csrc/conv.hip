@@ -443,12 +443,25 @@ int permute_filter(const float* in, float* out, int K, int C, int RS, bool to_cr
 
 typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
+typedef MnvGemmTile<128, 128, 16, 4, 1, 0, 96> Tile96;  // four wavefronts of 32 x 96
 
-// tile 0: 64x64 output tiles, tile 1: 128x128
+// tile 0: 64x64 output tiles, tile 1: 128x128, tile 2: 128x96
 template <class P>
 int launch_tile(int tile, const P& p, int splits, void* ws, hipStream_t s) {
-  return tile == 0 ? mnv_gemm_launch<TileSmall>(p, splits, ws, s)
-                   : mnv_gemm_launch<TileBig>(p, splits, ws, s);
+  switch (tile) {
+    case 0: return mnv_gemm_launch<TileSmall>(p, splits, ws, s);
+    case 2: return mnv_gemm_launch<Tile96>(p, splits, ws, s);
+    default: return mnv_gemm_launch<TileBig>(p, splits, ws, s);
+  }
+}
+const int kTileM[3] = {64, 128, 128}, kTileN[3] = {64, 128, 96};
+
+// 128-row tiles: 96 columns wide when that leaves clearly fewer idle columns than 128
+// (an output 96 or 192 wide), since the narrower tile does a little less work per byte
+// staged.
+int wide_tile(int n) {
+  int pad128 = (n + 127) / 128 * 128, pad96 = (n + 95) / 96 * 96;
+  return pad96 * 10 < pad128 * 9 ? 2 : 1;
 }
 
 int make_geom(ConvGeom* g, int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh,
@@ -478,21 +491,22 @@ int make_geom(ConvGeom* g, int N, int C, int K, int H, int W, int ph, int pw, in
   return MNV_OK;
 }
 
-bool small_tiles(int m, int n) {
+int pick_tile(int m, int n) {
   long long big = (long long)((m + 127) / 128) * ((n + 127) / 128);
-  return big < 128 || m <= 64 || n <= 64;
+  if (big < 128 || m <= 64 || n <= 64) return 0;
+  return wide_tile(n);
 }
 
 #define MNV_BWDF_MAX_SPLITS 256
 
 // The filter gradient gets its parallelism from splitting the long N*Ho*Wo reduction,
 // so it keeps the 128x128 tile (twice the operand reuse) unless the output is tiny.
-bool bwd_filter_small_tiles(int m, int n) { return m <= 64 || n <= 64; }
+int bwd_filter_tile(int m, int n) { return (m <= 64 || n <= 64) ? 0 : wide_tile(n); }
 
 int bwd_filter_splits(int m, int n, int k, size_t ws_floats) {
-  bool small = bwd_filter_small_tiles(m, n);
-  int bm = small ? 64 : 128;
-  long long tiles = (long long)((m + bm - 1) / bm) * ((n + bm - 1) / bm);
+  const int tile = bwd_filter_tile(m, n);
+  const int bm = kTileM[tile], bn = kTileN[tile];
+  long long tiles = (long long)((m + bm - 1) / bm) * ((n + bn - 1) / bn);
   int slabs = (k + 15) / 16;
   int max_splits = MNV_BWDF_MAX_SPLITS;
   if (max_splits > slabs / 8) max_splits = slabs / 8;
@@ -521,7 +535,7 @@ int mnv_conv_fwd(const float* bottom, const float* filter, const float* bias, fl
   if (rc) return rc;
   int gm = N * g.HoWo, gn = K, gk = g.CRS;
   hipStream_t s = mnv_stream(stream);
-  const int tile = small_tiles(gm, gn) ? 0 : 1;
+  const int tile = pick_tile(gm, gn);
   if (C % 16 == 0 && workspace && workspace_bytes >= (size_t)K * g.CRS * sizeof(float)) {
     float* wp = static_cast<float*>(workspace);
     rc = permute_filter(filter, wp, K, C, g.RS, false, s);
@@ -549,7 +563,7 @@ int mnv_conv_bwd_data(const float* top_diff, const float* filter, float* bottom_
   if (rc) return rc;
   int gm = N * g.HW, gn = C, gk = K * g.RS;
   hipStream_t s = mnv_stream(stream);
-  const int tile = small_tiles(gm, gn) ? 0 : 1;
+  const int tile = pick_tile(gm, gn);
   if (sv == 1 && sh == 1 && K % 16 == 0 && workspace &&
       workspace_bytes >= (size_t)K * g.CRS * sizeof(float)) {
     float* wq = static_cast<float*>(workspace);
@@ -580,18 +594,18 @@ int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filte
   int gm = g.CRS, gn = K, gk = N * g.HoWo;
   hipStream_t s = mnv_stream(stream);
   int splits = bwd_filter_splits(gm, gn, gk, workspace ? workspace_bytes / sizeof(float) : 0);
-  const bool small = bwd_filter_small_tiles(gm, gn);
+  const int tile = bwd_filter_tile(gm, gn);
   // Fast addressing: rows in (tap, channel) order with per-tap offset tables in LDS.  The
   // tables of all taps a 128-row tile touches must fit beside the tiles.
   const int PP = (g.HoWo + 15) / 16 * 16;
   const int taps_per_block = (128 + C - 1) / C + 1;
-  if (!small && (size_t)taps_per_block * PP * 4 <= 24 * 1024) {
+  if (tile != 0 && (size_t)taps_per_block * PP * 4 <= 24 * 1024) {
     ConvBwdFilterFast p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16), PP / 16,
                         PP, taps_per_block, mnv_fastdiv_make(C)};
-    return launch_tile(1, p, splits, workspace, s);
+    return launch_tile(tile, p, splits, workspace, s);
   }
   ConvBwdFilter p{bottom, top_diff, filter_diff, g, gm, gn, gk, (gk + 15) / 16, 1};
-  return launch_tile(small ? 0 : 1, p, splits, workspace, s);
+  return launch_tile(tile, p, splits, workspace, s);
 }
 
 }  // extern "C"

@@ -41,11 +41,14 @@ __device__ __forceinline__ void mnv_buf_load4(mnv_rsrc r, unsigned byte_off, flo
   v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
 }
 
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int PAD_ = 0>
+// BNU_ (default BN_): columns of the tile that are actually multiplied.  A tile fetches and
+// stages BN columns but may compute only the first BNU of them (and tiles then advance by
+// BNU), which lets a 96-wide output use three 32-column MFMA blocks instead of four.
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int PAD_ = 0, int BNU_ = BN_>
 struct MnvGemmTile {
-  static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_, BNU = BNU_;
   static constexpr int NT = MNV_WAVE * WGM * WGN;
-  static constexpr int WM = BM / WGM, WN = BN / WGN;
+  static constexpr int WM = BM / WGM, WN = BNU / WGN;
   static constexpr int TM = WM / 32, TN = WN / 32;
   static constexpr int LDA = BM + PAD_, LDB = BN + PAD_;
   static constexpr int AV = BM * BK / (4 * NT);  // 4-vectors of A per thread per slab
@@ -70,7 +73,7 @@ struct MnvGemmTile {
   // per CU make 1024 resident tiles, which lets tile counts just under a multiple of
   // 1024 finish in whole rounds.
   static constexpr int MIN_WAVES = (NT == 256 && BM * BN <= 128 * 128 && BK <= 16) ? 4 : 1;
-  static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
+  static_assert(WM % 32 == 0 && WN % 32 == 0 && BNU <= BN, "wave tile must be a multiple of 32x32");
   static_assert((BK == 8 || BK == 16 || BK == 32) && (BM * BK) % (4 * NT) == 0 &&
                     (BN * BK) % (4 * NT) == 0,
                 "tile/thread mismatch");
@@ -147,7 +150,7 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
   const int per_xcd = total / 8;
   if (b < per_xcd * 8) b = (b % 8) * per_xcd + b / 8;
   const int tile_m = b % tiles_m, tile_n = b / tiles_m;
-  const int m0 = tile_m * T::BM, n0 = tile_n * T::BN;
+  const int m0 = tile_m * T::BM, n0 = tile_n * T::BNU;
 
   const int slab_begin = blockIdx.z * slabs_per_split;
   int slab_end = slab_begin + slabs_per_split;
@@ -335,7 +338,7 @@ static inline int mnv_pick_splits(long long tiles, int slabs, int max_splits) {
 // splits*M*N*sizeof(float) bytes at `workspace`.
 template <class T, class P>
 static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream_t s) {
-  const int tiles_m = (prob.M + T::BM - 1) / T::BM, tiles_n = (prob.N + T::BN - 1) / T::BN;
+  const int tiles_m = (prob.M + T::BM - 1) / T::BM, tiles_n = (prob.N + T::BNU - 1) / T::BNU;
   const int total_slabs = prob.total_slabs;
   if (splits < 1) splits = 1;
   if (splits > total_slabs) splits = total_slabs > 0 ? total_slabs : 1;

@@ -112,6 +112,10 @@ CASES = [
     (3, 32, 48, 10, 11, 1, 2, 1, 1, 3, 5),  # channel counts that take the (tap, channel) order
     (2, 16, 16, 9, 9, 2, 2, 1, 1, 5, 5),
     (2, 48, 32, 12, 12, 1, 1, 2, 1, 3, 3),  # 16-multiple channels but a strided data gradient
+    (8, 16, 96, 48, 48, 1, 1, 1, 1, 3, 3),  # 96 output channels on many tiles: 96-column tiles
+    (8, 96, 16, 48, 48, 1, 1, 1, 1, 3, 3),  # 96 input channels: the same for the data gradient
+    (4, 64, 96, 20, 20, 1, 1, 1, 1, 3, 3),  # 96-column tiles in the table-driven filter gradient
+    (8, 4, 192, 46, 46, 0, 0, 1, 1, 3, 3),  # two 96-column tiles, channel-major reduction order
 ]
 
 
