@@ -112,7 +112,7 @@ def dominant_kernel_roofline(prof, steps):
 def op_table(prof, steps):
     rows = sorted(prof.items(), key=lambda kv: -kv[1][1])
     return [{"op": n, "launches_per_step": c // steps, "ms_per_step": round(ms / steps, 4)}
-            for n, (c, ms) in rows[:12]]
+            for n, (c, ms) in rows]
 
 
 def micro_bench():

@@ -33,6 +33,12 @@ __device__ __forceinline__ int ceil_div_pos(int a, int b) {  // b > 0, any a
   return a >= 0 ? (a + b - 1) / b : -((-a) / b);
 }
 
+// a / stride for a >= 0; ST = 1 or 2 when both strides are that constant, 0 otherwise
+template <int ST>
+__device__ __forceinline__ int div_stride(int a, const MnvFastDiv& d) {
+  return ST == 1 ? a : ST == 2 ? (a >> 1) : mnv_fastdiv(a, d);
+}
+
 // Loads `count` floats starting at src (any alignment) into LDS.
 __device__ __forceinline__ void stage(const float* __restrict__ src, float* dst, int count) {
   // align the global side to 16 bytes, then copy vectors
@@ -87,7 +93,7 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_fwd_lds_kernel(
 }
 
 // LDS: [ppb*hw] plane data, then [ppb*howo] top_diff, then [ppb*howo] arg-max positions.
-template <bool MAX>
+template <bool MAX, int ST>
 __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_lds_kernel(
     const float* __restrict__ bottom, const float* __restrict__ top_diff,
     float* __restrict__ bottom_diff, int planes, int ppb, PoolGeom g) {
@@ -130,10 +136,10 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_lds_kernel(
       int y = mnv_fastdiv(pos, g.d_W), x = pos - y * g.W;
       // windows i with i*sv - ph <= y < i*sv - ph + kh, clipped to [0, Ho)
       int ay = y + g.ph - g.kh + g.sv, ax = x + g.pw - g.kw + g.sh;  // ceil((y+ph-kh+1)/sv)
-      int i_lo = ay > 0 ? mnv_fastdiv(ay, g.d_sv) : 0;
-      int i_hi = min(mnv_fastdiv(y + g.ph, g.d_sv), g.Ho - 1);
-      int j_lo = ax > 0 ? mnv_fastdiv(ax, g.d_sh) : 0;
-      int j_hi = min(mnv_fastdiv(x + g.pw, g.d_sh), g.Wo - 1);
+      int i_lo = ay > 0 ? div_stride<ST>(ay, g.d_sv) : 0;
+      int i_hi = min(div_stride<ST>(y + g.ph, g.d_sv), g.Ho - 1);
+      int j_lo = ax > 0 ? div_stride<ST>(ax, g.d_sh) : 0;
+      int j_hi = min(div_stride<ST>(x + g.pw, g.d_sh), g.Wo - 1);
       float acc = 0.f;
       for (int i = i_lo; i <= i_hi; ++i)
         for (int j = j_lo; j <= j_hi; ++j) {
@@ -300,9 +306,12 @@ int pool_bwd(const float* bottom, const float* top_diff, float* bottom_diff, int
     size_t lds = (size_t)ppb * ((size_t)h * w + 2 * (size_t)g.Ho * g.Wo) * sizeof(float);
     long long blocks = (planes + ppb - 1) / ppb;
     if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL((mnv_pool_bwd_lds_kernel<MAX>), dim3((unsigned)blocks),
-                       dim3(MNV_POOL_THREADS), lds, mnv_stream(stream), bottom, top_diff,
-                       bottom_diff, (int)planes, ppb, g);
+    const int st = (sv == sh && (sv == 1 || sv == 2)) ? sv : 0;
+    auto kernel = st == 1   ? mnv_pool_bwd_lds_kernel<MAX, 1>
+                  : st == 2 ? mnv_pool_bwd_lds_kernel<MAX, 2>
+                            : mnv_pool_bwd_lds_kernel<MAX, 0>;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(MNV_POOL_THREADS), lds,
+                       mnv_stream(stream), bottom, top_diff, bottom_diff, (int)planes, ppb, g);
   } else {
     hipLaunchKernelGGL((mnv_pool_bwd_kernel<MAX>), dim3(pool_grid((size_t)planes * h * w)),
                        dim3(MNV_POOL_THREADS), 0, mnv_stream(stream), bottom, top_diff,

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(MNV_TR_THREADS) void mnv_transpose_vec4_kernel(
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     int i = i0 + tx * 4, j = j0 + ty + 16 * p;
-    if (i < m && j < n) v[p] = __builtin_nontemporal_load(reinterpret_cast<const mnv_f4*>(a + (size_t)j * m + i));
+    if (i < m && j < n) v[p] = *reinterpret_cast<const mnv_f4*>(a + (size_t)j * m + i);
   }
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
