@@ -84,7 +84,7 @@ def alexnet_bench(steps, warmup):
 # gradients), from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB
 # per dispatch), each scaled by what the same counter reads for the 8192^2 copy kernel
 # (256 MiB read, 256 MiB written).  None until measured.
-DOMINANT_KERNEL_TRAFFIC_BYTES = 1.50e9
+DOMINANT_KERNEL_TRAFFIC_BYTES = 1.44e9
 
 
 def dominant_kernel_roofline(prof, steps):
