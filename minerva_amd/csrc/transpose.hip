@@ -3,7 +3,10 @@
 // c[j + i*n] = a[i + j*m].  Roofline: HBM bandwidth, 8 bytes per element.  A 64x64
 // tile goes through LDS so that both the read (along i) and the write (along j) are
 // contiguous 256-byte runs per 64 threads; the LDS row pitch of 65 floats keeps the
-// transposed reads off a single bank.
+// transposed reads off a single bank.  Tiles are visited along diagonals: workgroups that
+// run together then differ in both their row and their column offset, so neither their
+// reads nor their writes (whose addresses would otherwise differ by multiples of 64 rows
+// of a power-of-two pitch) pile onto a few memory channels.
 #include "mnv_common.h"
 
 namespace {
@@ -12,9 +15,9 @@ namespace {
 #define MNV_TR_THREADS 256
 
 __global__ __launch_bounds__(MNV_TR_THREADS) void mnv_transpose_kernel(
-    const float* __restrict__ a, float* __restrict__ c, int m, int n, int tiles_i) {
+    const float* __restrict__ a, float* __restrict__ c, int m, int n, int tiles_i, int tiles_j) {
   __shared__ float tile[MNV_TR_TILE][MNV_TR_TILE + 1];
-  const int ti = blockIdx.x % tiles_i, tj = blockIdx.x / tiles_i;
+  const int ti = blockIdx.x % tiles_i, tj = (blockIdx.x / tiles_i + ti) % tiles_j;
   const int i0 = ti * MNV_TR_TILE, j0 = tj * MNV_TR_TILE;
   const int tx = threadIdx.x % MNV_TR_TILE, ty = threadIdx.x / MNV_TR_TILE;
   // read: tx runs along i (contiguous in a)
@@ -36,9 +39,9 @@ __global__ __launch_bounds__(MNV_TR_THREADS) void mnv_transpose_kernel(
 // and writes four consecutive j of one output column; the 64x64 tile is transposed
 // through LDS with 4-byte accesses.  Needs m % 4 == 0, n % 4 == 0 and aligned pointers.
 __global__ __launch_bounds__(MNV_TR_THREADS) void mnv_transpose_vec4_kernel(
-    const float* __restrict__ a, float* __restrict__ c, int m, int n, int tiles_i) {
+    const float* __restrict__ a, float* __restrict__ c, int m, int n, int tiles_i, int tiles_j) {
   __shared__ float tile[MNV_TR_TILE][MNV_TR_TILE + 1];
-  const int ti = blockIdx.x % tiles_i, tj = blockIdx.x / tiles_i;
+  const int ti = blockIdx.x % tiles_i, tj = (blockIdx.x / tiles_i + ti) % tiles_j;
   const int i0 = ti * MNV_TR_TILE, j0 = tj * MNV_TR_TILE;
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
   mnv_f4 v[4];
@@ -76,9 +79,9 @@ extern "C" int mnv_transpose(const float* a, float* c, int m, int n, mnv_stream_
   if (tiles_i * tiles_j > 0x7fffffffULL) return MNV_ERR_INVALID;
   if (m % 4 == 0 && n % 4 == 0 && mnv_aligned16(a) && mnv_aligned16(c))
     hipLaunchKernelGGL(mnv_transpose_vec4_kernel, dim3((unsigned)(tiles_i * tiles_j)),
-                       dim3(MNV_TR_THREADS), 0, mnv_stream(stream), a, c, m, n, (int)tiles_i);
+                       dim3(MNV_TR_THREADS), 0, mnv_stream(stream), a, c, m, n, (int)tiles_i, (int)tiles_j);
   else
     hipLaunchKernelGGL(mnv_transpose_kernel, dim3((unsigned)(tiles_i * tiles_j)),
-                       dim3(MNV_TR_THREADS), 0, mnv_stream(stream), a, c, m, n, (int)tiles_i);
+                       dim3(MNV_TR_THREADS), 0, mnv_stream(stream), a, c, m, n, (int)tiles_i, (int)tiles_j);
   return MNV_LAUNCH_STATUS();
 }
