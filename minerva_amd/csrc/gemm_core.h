@@ -23,24 +23,6 @@
 typedef float mnv_f16v __attribute__((ext_vector_type(16)));
 
 #ifdef __HIPCC__
-// Buffer addressing: every operand is read through a raw buffer resource whose extent is
-// the tensor's byte size, so a masked-off element is fetched with an offset past the end
-// and the hardware returns 0 for it: no divergent branch, no address clamp, no fault.
-// Operands are therefore limited to 2^31 - 1 bytes.
-#define MNV_OOB 0x80000000u
-typedef __amdgpu_buffer_rsrc_t mnv_rsrc;
-
-__device__ __forceinline__ mnv_rsrc mnv_make_rsrc(const float* p, unsigned bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p), 0, bytes, 0x00020000);
-}
-__device__ __forceinline__ float mnv_buf_load(mnv_rsrc r, unsigned byte_off) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0));
-}
-__device__ __forceinline__ void mnv_buf_load4(mnv_rsrc r, unsigned byte_off, float (&v)[4]) {
-  mnv_f4 t = __builtin_bit_cast(mnv_f4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0));
-  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-}
-
 // BNU_ (default BN_): columns of the tile that are actually multiplied.  A tile fetches and
 // stages BN columns but may compute only the first BNU of them (and tiles then advance by
 // BNU), which lets a 96-wide output use three 32-column MFMA blocks instead of four.
@@ -234,6 +216,10 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
       new_period(++period);
     }
     fetch(period, s);
+    // Keep the loads up here: left alone, the scheduler sinks them below most of the
+    // multiplies to shorten register lifetimes, and each wavefront then waits out the
+    // full memory latency once per slab.
+    __builtin_amdgcn_sched_barrier(0);
     // A round multiplies 8 k values: MFMA step t pairs k = 8h + t (lanes 0..31) with
     // k = 8h + 4 + t (lanes 32..63), so a lane's four steps use four consecutive k.
     const float* a = As + buf * ATILE;

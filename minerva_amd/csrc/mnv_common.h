@@ -51,6 +51,25 @@ __device__ __forceinline__ int mnv_fastdiv(int n, const MnvFastDiv& f) {
 
 typedef float mnv_f4 __attribute__((ext_vector_type(4)));
 
+// Buffer addressing: every operand is read through a raw buffer resource whose extent is
+// the tensor's byte size, so a masked-off element is fetched with an offset past the end
+// and the hardware returns 0 for it: no divergent branch, no address clamp, no fault.
+// Operands are therefore limited to 2^31 - 1 bytes.
+#define MNV_OOB 0x80000000u
+typedef __amdgpu_buffer_rsrc_t mnv_rsrc;
+
+__device__ __forceinline__ mnv_rsrc mnv_make_rsrc(const float* p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ float mnv_buf_load(mnv_rsrc r, unsigned byte_off) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0));
+}
+__device__ __forceinline__ void mnv_buf_load4(mnv_rsrc r, unsigned byte_off, float (&v)[4]) {
+  mnv_f4 t = __builtin_bit_cast(mnv_f4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0));
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+
+
 __device__ __forceinline__ float mnv_wave_sum(float v) {
 #pragma unroll
   for (int off = MNV_WAVE / 2; off > 0; off >>= 1) v += __shfl_down(v, off, MNV_WAVE);

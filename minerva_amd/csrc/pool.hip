@@ -11,146 +11,338 @@
 // ascending window order, which is the order a sequential scatter would use, so the
 // result is bit-identical to it and no atomics are needed.
 //
-// Main path: a workgroup stages whole (n,c) planes in LDS with contiguous 16-byte loads,
-// finds every window's arg-max once from LDS, then walks the plane's positions and
+// Main path: a workgroup stages groups of whole (n,c) planes in LDS with aligned 16-byte
+// loads, finds every window's arg-max once from LDS, then walks the planes' positions and
 // gathers the gradients of the (at most ceil(k/s)^2) windows each one can win.  HBM sees
-// every tensor exactly once.  Planes too large for LDS take the direct kernels below.
+// every tensor exactly once.  The workgroups are persistent and keep the next group's
+// loads in flight (in registers) while they work on the current one; 3x3/2 and 2x2/2
+// windows are unrolled at compile time.  Planes too large for LDS take the direct kernels.
 #include <math.h>
+
+#include <algorithm>
 
 #include "mnv_common.h"
 
 namespace {
 
 #define MNV_POOL_THREADS 256
-#define MNV_POOL_LDS_FLOATS 8192  // plane data staged per workgroup (32 KiB)
+#define MNV_POOL_XV 8  // 16-byte vectors of plane data a thread holds for the next group
+#define MNV_POOL_DV 4  // ... of top_diff
+#define MNV_POOL_X_FLOATS (MNV_POOL_THREADS * 4 * MNV_POOL_XV)
+#define MNV_POOL_D_FLOATS (MNV_POOL_THREADS * 4 * MNV_POOL_DV)
 
 struct PoolGeom {
   int H, W, Ho, Wo, sv, sh, kh, kw, ph, pw;
   MnvFastDiv d_hw, d_howo, d_W, d_Wo, d_sv, d_sh;  // run-time integer division is ~40 instructions
+  // stride-2 backward: 2x2 blocks of padded coordinates (rows 2a, 2a+1) that meet the plane
+  int a0, b0, NA, NB;
+  MnvFastDiv d_nab, d_nb;
 };
 
 __device__ __forceinline__ int ceil_div_pos(int a, int b) {  // b > 0, any a
   return a >= 0 ? (a + b - 1) / b : -((-a) / b);
 }
 
-// a / stride for a >= 0; ST = 1 or 2 when both strides are that constant, 0 otherwise
+// Products of small indices (LDS offsets, plane coordinates: far below 2^23) on the
+// full-rate 24-bit multiplier; the 32-bit integer multiply runs at a quarter of that.
+__device__ __forceinline__ int m24(int a, int b) { return __mul24(a, b); }
+
+// a / stride for a >= 0; ST = the compile-time stride, or 0 for a run-time one
 template <int ST>
 __device__ __forceinline__ int div_stride(int a, const MnvFastDiv& d) {
   return ST == 1 ? a : ST == 2 ? (a >> 1) : mnv_fastdiv(a, d);
 }
 
-// Loads `count` floats starting at src (any alignment) into LDS.
-__device__ __forceinline__ void stage(const float* __restrict__ src, float* dst, int count) {
-  // align the global side to 16 bytes, then copy vectors
-  int head = (int)(((16 - (reinterpret_cast<uintptr_t>(src) & 15)) & 15) >> 2);
-  if (head > count) head = count;
-  for (int i = threadIdx.x; i < head; i += MNV_POOL_THREADS) dst[i] = src[i];
-  const int n4 = (count - head) >> 2;
-  const mnv_f4* s4 = reinterpret_cast<const mnv_f4*>(src + head);
-  for (int i = threadIdx.x; i < n4; i += MNV_POOL_THREADS) {
-    mnv_f4 v = s4[i];
-    float* d = dst + head + 4 * i;
-    d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+// A run of `count` floats starting `first` floats into a 16-byte aligned tensor of `total`
+// floats, moved HBM -> registers -> LDS in aligned 16-byte pieces.  The run is widened down
+// to the previous 16-byte boundary (element e of the run lands at lds[(first & 3) + e]) and
+// read through a buffer resource that ends with the tensor, so the last piece may hang over
+// the end and reads zeros there.  issue() and commit() are separate so that the loads of
+// the next group stay in flight while the current one is being worked on.
+template <int NV>
+struct PoolStage {
+  mnv_f4 r[NV];
+  int nvec;
+  __device__ __forceinline__ void issue(const float* base, size_t total, size_t first, int count) {
+    const size_t a0 = first & ~(size_t)3;
+    nvec = (int)((first + count - a0 + 3) >> 2);
+    size_t left = (total - a0) * sizeof(float);
+    if (left > 0x7fffffffu) left = 0x7fffffffu;
+    mnv_rsrc rs = mnv_make_rsrc(base + a0, (unsigned)left);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int v = threadIdx.x + u * MNV_POOL_THREADS;
+      if (v < nvec)
+        r[u] = __builtin_bit_cast(mnv_f4, __builtin_amdgcn_raw_buffer_load_b128(rs, v * 16, 0, 0));
+    }
   }
-  for (int i = head + 4 * n4 + threadIdx.x; i < count; i += MNV_POOL_THREADS) dst[i] = src[i];
+  __device__ __forceinline__ void commit(float* lds) const {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int v = threadIdx.x + u * MNV_POOL_THREADS;
+      if (v < nvec) *reinterpret_cast<mnv_f4*>(lds + 4 * v) = r[u];
+    }
+  }
+};
+
+// Value (and position) of window (i, j) of the plane at b.  KS / ST are the compile-time
+// square window and stride, or 0 for the run-time ones in g.  Maximum: strict '<' from
+// -inf in scan order, so the first maximum wins and a NaN never does; `arg` starts at the
+// first in-range position.  Average: scan-order sum over the in-range part / full area.
+template <bool MAX, int KS, int ST>
+__device__ __forceinline__ float pool_window(const float* b, const PoolGeom& g, int i, int j,
+                                            int* arg) {
+  const int sv = ST ? ST : g.sv, sh = ST ? ST : g.sh;
+  const int kh = KS ? KS : g.kh, kw = KS ? KS : g.kw;
+  const int y0 = i * sv - g.ph, x0 = j * sh - g.pw;
+  float r = MAX ? -INFINITY : 0.f;
+  int at = m24(max(y0, 0), g.W) + max(x0, 0);
+  if (KS && y0 >= 0 && x0 >= 0 && y0 + KS <= g.H && x0 + KS <= g.W) {
+    // window inside the plane (all of them when nothing is padded or clipped): no checks
+    const int base = m24(y0, g.W) + x0;
+#pragma unroll
+    for (int dy = 0; dy < KS; ++dy)
+#pragma unroll
+      for (int dx = 0; dx < KS; ++dx) {
+        const float v = b[base + dy * g.W + dx];
+        if (MAX) {
+          if (r < v) {
+            r = v;
+            at = base + dy * g.W + dx;
+          }
+        } else {
+          r += v;
+        }
+      }
+  } else if (KS) {
+#pragma unroll
+    for (int dy = 0; dy < KS; ++dy)
+#pragma unroll
+      for (int dx = 0; dx < KS; ++dx) {
+        const int y = y0 + dy, x = x0 + dx;
+        const bool ok = ((unsigned)y < (unsigned)g.H) & ((unsigned)x < (unsigned)g.W);
+        const float v = ok ? b[y * g.W + x] : (MAX ? -INFINITY : 0.f);
+        if (MAX) {
+          if (r < v) {
+            r = v;
+            at = y * g.W + x;
+          }
+        } else {
+          r += v;
+        }
+      }
+  } else {
+    const int ys = max(y0, 0), xs = max(x0, 0);
+    const int ye = min(y0 + kh, g.H), xe = min(x0 + kw, g.W);
+    for (int y = ys; y < ye; ++y)
+      for (int x = xs; x < xe; ++x) {
+        const float v = b[y * g.W + x];
+        if (MAX) {
+          if (r < v) {
+            r = v;
+            at = y * g.W + x;
+          }
+        } else {
+          r += v;
+        }
+      }
+  }
+  if (arg) *arg = at;
+  return MAX ? r : r / (float)(kh * kw);
 }
 
-// ---- LDS-staged kernels: `ppb` planes per workgroup --------------------------------
-template <bool MAX>
+// ---- LDS-staged kernels: groups of `ppb` planes per workgroup, software pipelined ------
+template <bool MAX, int KS, int ST>
 __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_fwd_lds_kernel(
     const float* __restrict__ bottom, float* __restrict__ top, int planes, int ppb, PoolGeom g) {
   extern __shared__ float lds[];
   const int hw = g.H * g.W, howo = g.Ho * g.Wo;
-  for (int p0 = blockIdx.x * ppb; p0 < planes; p0 += gridDim.x * ppb) {
-    const int np = min(ppb, planes - p0);
+  const size_t total = (size_t)planes * hw;
+  const int groups = (planes + ppb - 1) / ppb;
+  PoolStage<MNV_POOL_XV> sx;
+  int grp = blockIdx.x;
+  if (grp < groups) {
+    const int p0 = grp * ppb;
+    sx.issue(bottom, total, (size_t)p0 * hw, min(ppb, planes - p0) * hw);
+  }
+  for (; grp < groups; grp += gridDim.x) {
+    const int p0 = grp * ppb, np = min(ppb, planes - p0);
+    const int shift = (int)(((size_t)p0 * hw) & 3);
+    __syncthreads();  // the previous group's windows have been read
+    sx.commit(lds);
+    const int nxt = grp + gridDim.x;
+    if (nxt < groups) {
+      const int q0 = nxt * ppb;
+      sx.issue(bottom, total, (size_t)q0 * hw, min(ppb, planes - q0) * hw);
+    }
     __syncthreads();
-    stage(bottom + (size_t)p0 * hw, lds, np * hw);
-    __syncthreads();
+    float* topg = top + (size_t)p0 * howo;  // uniform base, 32-bit per-thread offsets
     for (int q = threadIdx.x; q < np * howo; q += MNV_POOL_THREADS) {
-      int pl = mnv_fastdiv(q, g.d_howo), o = q - pl * howo;
-      int i = mnv_fastdiv(o, g.d_Wo), j = o - i * g.Wo;
-      int y0 = i * g.sv - g.ph, x0 = j * g.sh - g.pw;
-      int ys = max(y0, 0), xs = max(x0, 0);
-      int ye = min(y0 + g.kh, g.H), xe = min(x0 + g.kw, g.W);
-      const float* b = lds + pl * hw;
-      float r;
-      if (MAX) {
-        r = -INFINITY;
-        for (int y = ys; y < ye; ++y)
-          for (int x = xs; x < xe; ++x) {
-            float v = b[y * g.W + x];
-            if (r < v) r = v;
-          }
-      } else {
-        float s = 0.f;
-        for (int y = ys; y < ye; ++y)
-          for (int x = xs; x < xe; ++x) s += b[y * g.W + x];
-        r = s / (float)(g.kh * g.kw);
-      }
-      top[(size_t)p0 * howo + q] = r;
+      const int pl = mnv_fastdiv(q, g.d_howo), o = q - m24(pl, howo);
+      const int i = mnv_fastdiv(o, g.d_Wo), j = o - m24(i, g.Wo);
+      __builtin_nontemporal_store(pool_window<MAX, KS, ST>(lds + shift + m24(pl, hw), g, i, j, nullptr),
+                                  &topg[(unsigned)q]);
     }
   }
 }
 
-// LDS: [ppb*hw] plane data, then [ppb*howo] top_diff, then [ppb*howo] arg-max positions.
-template <bool MAX, int ST>
+// LDS: plane data [ppb*hw + 8], top_diff [ppb*howo + 8], arg-max positions [ppb*howo].
+template <bool MAX, int KS, int ST>
 __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_lds_kernel(
     const float* __restrict__ bottom, const float* __restrict__ top_diff,
     float* __restrict__ bottom_diff, int planes, int ppb, PoolGeom g) {
   extern __shared__ float lds[];
   const int hw = g.H * g.W, howo = g.Ho * g.Wo;
-  float* sx = lds;
-  float* sd = lds + ppb * hw;
-  int* sarg = reinterpret_cast<int*>(sd + ppb * howo);
-  for (int p0 = blockIdx.x * ppb; p0 < planes; p0 += gridDim.x * ppb) {
-    const int np = min(ppb, planes - p0);
-    __syncthreads();
-    if (MAX) stage(bottom + (size_t)p0 * hw, sx, np * hw);
-    stage(top_diff + (size_t)p0 * howo, sd, np * howo);
+  const size_t total_x = (size_t)planes * hw, total_d = (size_t)planes * howo;
+  const int groups = (planes + ppb - 1) / ppb;
+  float* lx = lds;
+  float* ld = lds + ((ppb * hw + 8 + 3) & ~3);
+  int* sarg = reinterpret_cast<int*>(ld + ((ppb * howo + 8 + 3) & ~3));
+  const int sv = ST ? ST : g.sv, sh = ST ? ST : g.sh;
+  const int kh = KS ? KS : g.kh, kw = KS ? KS : g.kw;
+  PoolStage<MAX ? MNV_POOL_XV : 1> sx;
+  PoolStage<MNV_POOL_DV> sd;
+  int grp = blockIdx.x;
+  if (grp < groups) {
+    const int p0 = grp * ppb, np = min(ppb, planes - p0);
+    if (MAX) sx.issue(bottom, total_x, (size_t)p0 * hw, np * hw);
+    sd.issue(top_diff, total_d, (size_t)p0 * howo, np * howo);
+  }
+  for (; grp < groups; grp += gridDim.x) {
+    const int p0 = grp * ppb, np = min(ppb, planes - p0);
+    const int shift_x = (int)(((size_t)p0 * hw) & 3);
+    const float* bx = lx + shift_x;
+    const float* bd = ld + (int)(((size_t)p0 * howo) & 3);
+    __syncthreads();  // the previous group has been read
+    if (MAX) sx.commit(lx);
+    sd.commit(ld);
+    const int nxt = grp + gridDim.x;
+    if (nxt < groups) {
+      const int q0 = nxt * ppb, nq = min(ppb, planes - q0);
+      if (MAX) sx.issue(bottom, total_x, (size_t)q0 * hw, nq * hw);
+      sd.issue(top_diff, total_d, (size_t)q0 * howo, nq * howo);
+    }
     __syncthreads();
     if (MAX) {
-      // first maximum of every window in scan order (strict '<'), as a flat position
+      // first maximum of every window in scan order, as a flat position in its plane
       for (int q = threadIdx.x; q < np * howo; q += MNV_POOL_THREADS) {
-        int pl = mnv_fastdiv(q, g.d_howo), o = q - pl * howo;
-        int i = mnv_fastdiv(o, g.d_Wo), j = o - i * g.Wo;
-        int y0 = i * g.sv - g.ph, x0 = j * g.sh - g.pw;
-        int ys = max(y0, 0), xs = max(x0, 0);
-        int ye = min(y0 + g.kh, g.H), xe = min(x0 + g.kw, g.W);
-        const float* b = sx + pl * hw;
-        float mx = -INFINITY;
-        int arg = ys * g.W + xs;
-        for (int y = ys; y < ye; ++y)
-          for (int x = xs; x < xe; ++x) {
-            float v = b[y * g.W + x];
-            if (mx < v) {
-              mx = v;
-              arg = y * g.W + x;
-            }
-          }
+        const int pl = mnv_fastdiv(q, g.d_howo), o = q - m24(pl, howo);
+        const int i = mnv_fastdiv(o, g.d_Wo), j = o - m24(i, g.Wo);
+        int arg;
+        pool_window<true, KS, ST>(bx + m24(pl, hw), g, i, j, &arg);
         sarg[q] = arg;
       }
       __syncthreads();
     }
-    for (int q = threadIdx.x; q < np * hw; q += MNV_POOL_THREADS) {
-      int pl = mnv_fastdiv(q, g.d_hw), pos = q - pl * hw;
-      int y = mnv_fastdiv(pos, g.d_W), x = pos - y * g.W;
-      // windows i with i*sv - ph <= y < i*sv - ph + kh, clipped to [0, Ho)
-      int ay = y + g.ph - g.kh + g.sv, ax = x + g.pw - g.kw + g.sh;  // ceil((y+ph-kh+1)/sv)
-      int i_lo = ay > 0 ? div_stride<ST>(ay, g.d_sv) : 0;
-      int i_hi = min(div_stride<ST>(y + g.ph, g.d_sv), g.Ho - 1);
-      int j_lo = ax > 0 ? div_stride<ST>(ax, g.d_sh) : 0;
-      int j_hi = min(div_stride<ST>(x + g.pw, g.d_sh), g.Wo - 1);
-      float acc = 0.f;
-      for (int i = i_lo; i <= i_hi; ++i)
-        for (int j = j_lo; j <= j_hi; ++j) {
-          int o = pl * howo + i * g.Wo + j;
-          if (MAX) {
-            if (sarg[o] == pos) acc += sd[o];
-          } else {
-            acc += sd[o] / (float)(g.kh * g.kw);
-          }
+    // The gradients go to LDS first, over the plane data (dead once the arg-max positions
+    // are known), and leave as dense 16-byte stores: written straight from the loop below
+    // they would be 4-byte stores at a stride of two.
+    float* lout = lx + shift_x;
+    if constexpr (ST == 2 && (KS == 2 || KS == 3)) {
+      // A thread owns a 2x2 block of padded coordinates (rows 2a, 2a+1; columns 2b, 2b+1).
+      // Row 2a lies in windows a-1 (3-wide only) and a, row 2a+1 in window a alone, so the
+      // block's four positions draw on the same four windows: their arg-max positions and
+      // gradients are read once, and each position adds the ones it wins in ascending
+      // window order, like a sequential scatter.
+      const int nblk = g.NA * g.NB;
+      for (int q = threadIdx.x; q < np * nblk; q += MNV_POOL_THREADS) {
+        const int pl = mnv_fastdiv(q, g.d_nab), r = q - m24(pl, nblk);
+        const int ai = mnv_fastdiv(r, g.d_nb), bi = r - m24(ai, g.NB);
+        const int a = g.a0 + ai, b = g.b0 + bi;
+        const int y = 2 * a - g.ph, x = 2 * b - g.pw;
+        const float* d = bd + m24(pl, howo);
+        const int* sa = sarg + m24(pl, howo);
+        const bool vi0 = KS == 3 && a >= 1 && a - 1 < g.Ho, vi1 = a < g.Ho;
+        const bool vj0 = KS == 3 && b >= 1 && b - 1 < g.Wo, vj1 = b < g.Wo;
+        const int o11 = m24(a, g.Wo) + b, o10 = o11 - 1, o01 = o11 - g.Wo, o00 = o01 - 1;
+        // a window that does not exist contributes +0.0f, which changes no sum
+        float d00 = (vi0 && vj0) ? d[o00] : 0.f, d01 = (vi0 && vj1) ? d[o01] : 0.f;
+        float d10 = (vi1 && vj0) ? d[o10] : 0.f, d11 = (vi1 && vj1) ? d[o11] : 0.f;
+        const int p00 = m24(y, g.W) + x, p01 = p00 + 1, p10 = p00 + g.W, p11 = p10 + 1;
+        float g00, g01, g10, g11;
+        if (MAX) {
+          const int s00 = (vi0 && vj0) ? sa[o00] : -1, s01 = (vi0 && vj1) ? sa[o01] : -1;
+          const int s10 = (vi1 && vj0) ? sa[o10] : -1, s11 = (vi1 && vj1) ? sa[o11] : -1;
+          g00 = (((0.f + (s00 == p00 ? d00 : 0.f)) + (s01 == p00 ? d01 : 0.f)) +
+                 (s10 == p00 ? d10 : 0.f)) + (s11 == p00 ? d11 : 0.f);
+          g01 = (0.f + (s01 == p01 ? d01 : 0.f)) + (s11 == p01 ? d11 : 0.f);
+          g10 = (0.f + (s10 == p10 ? d10 : 0.f)) + (s11 == p10 ? d11 : 0.f);
+          g11 = 0.f + (s11 == p11 ? d11 : 0.f);
+        } else {
+          const float area = (float)(KS * KS);
+          d00 = d00 / area; d01 = d01 / area; d10 = d10 / area; d11 = d11 / area;
+          g00 = (((0.f + d00) + d01) + d10) + d11;
+          g01 = (0.f + d01) + d11;
+          g10 = (0.f + d10) + d11;
+          g11 = 0.f + d11;
         }
-      bottom_diff[(size_t)p0 * hw + q] = acc;
+        const bool y0ok = (unsigned)y < (unsigned)g.H, y1ok = (unsigned)(y + 1) < (unsigned)g.H;
+        const bool x0ok = (unsigned)x < (unsigned)g.W, x1ok = (unsigned)(x + 1) < (unsigned)g.W;
+        const int po = m24(pl, hw);
+        if (y0ok && x0ok) lout[po + p00] = g00;
+        if (y0ok && x1ok) lout[po + p01] = g01;
+        if (y1ok && x0ok) lout[po + p10] = g10;
+        if (y1ok && x1ok) lout[po + p11] = g11;
+      }
+    } else {
+      for (int q = threadIdx.x; q < np * hw; q += MNV_POOL_THREADS) {
+        const int pl = mnv_fastdiv(q, g.d_hw), pos = q - pl * hw;
+        const int y = mnv_fastdiv(pos, g.d_W), x = pos - y * g.W;
+        // windows i with i*sv - ph <= y < i*sv - ph + kh, clipped to [0, Ho); likewise j
+        const int ay = y + g.ph - kh + sv, ax = x + g.pw - kw + sh;  // ceil((y+ph-kh+1)/sv)
+        const int i_lo = ay > 0 ? div_stride<ST>(ay, g.d_sv) : 0;
+        const int i_hi = min(div_stride<ST>(y + g.ph, g.d_sv), g.Ho - 1);
+        const int j_lo = ax > 0 ? div_stride<ST>(ax, g.d_sh) : 0;
+        const int j_hi = min(div_stride<ST>(x + g.pw, g.d_sh), g.Wo - 1);
+        const float* d = bd + pl * howo;
+        const int* sa = sarg + pl * howo;
+        float acc = 0.f;
+        // gradients are added in ascending window order, like a sequential scatter
+        if (KS && ST) {
+          constexpr int CNT = (KS && ST) ? (KS + ST - 1) / (ST ? ST : 1) : 1;
+  #pragma unroll
+          for (int a = 0; a < CNT; ++a)
+  #pragma unroll
+            for (int c = 0; c < CNT; ++c) {
+              const int i = i_lo + a, j = j_lo + c;
+              if ((i <= i_hi) & (j <= j_hi)) {
+                const int o = i * g.Wo + j;
+                if (MAX) {
+                  if (sa[o] == pos) acc += d[o];
+                } else {
+                  acc += d[o] / (float)(kh * kw);
+                }
+              }
+            }
+        } else {
+          for (int i = i_lo; i <= i_hi; ++i)
+            for (int j = j_lo; j <= j_hi; ++j) {
+              const int o = i * g.Wo + j;
+              if (MAX) {
+                if (sa[o] == pos) acc += d[o];
+              } else {
+                acc += d[o] / (float)(kh * kw);
+              }
+            }
+        }
+        lout[q] = acc;
+      }
+    }
+    __syncthreads();
+    {
+      const int cnt = np * hw;
+      float* gout = bottom_diff + (((size_t)p0 * hw) & ~(size_t)3);  // 16-byte aligned
+      const int nv = (shift_x + cnt + 3) >> 2;
+      for (int v = threadIdx.x; v < nv; v += MNV_POOL_THREADS) {
+        const int e0 = 4 * v - shift_x;  // position of the vector's first float in the group
+        if (e0 >= 0 && e0 + 4 <= cnt) {
+          __builtin_nontemporal_store(*reinterpret_cast<const mnv_f4*>(lx + 4 * v),
+                                      reinterpret_cast<mnv_f4*>(gout) + v);
+        } else {  // the group's first and last vector may be shared with its neighbours
+          for (int k = 0; k < 4; ++k)
+            if (e0 + k >= 0 && e0 + k < cnt) gout[4 * v + k] = lx[4 * v + k];
+        }
+      }
     }
   }
 }
@@ -247,6 +439,12 @@ int make_geom(PoolGeom* g, int n, int c, int h, int w, int sv, int sh, int kh, i
   g->d_Wo = mnv_fastdiv_make(g->Wo);
   g->d_sv = mnv_fastdiv_make(sv);
   g->d_sh = mnv_fastdiv_make(sh);
+  g->a0 = ph >> 1;
+  g->b0 = pw >> 1;
+  g->NA = ((ph + h - 1) >> 1) - g->a0 + 1;
+  g->NB = ((pw + w - 1) >> 1) - g->b0 + 1;
+  g->d_nab = mnv_fastdiv_make(g->NA * g->NB);
+  g->d_nb = mnv_fastdiv_make(g->NB);
   return MNV_OK;
 }
 
@@ -256,17 +454,32 @@ unsigned pool_grid(size_t total) {
   return (unsigned)blocks;
 }
 
-// Planes per workgroup for the LDS path: as many as fit the staging area, but no more
-// than leaves every CU several workgroups.  0 = plane too large, use the direct kernels.
+// Planes per workgroup for the LDS path: as many as fit the register staging and 48 KiB of
+// LDS, but few enough that every workgroup gets several groups to pipeline.  0 = a plane is
+// too large (or a pointer not 16-byte aligned): use the direct kernels.
 int planes_per_block(const PoolGeom& g, long long planes, bool bwd) {
-  long long per_plane = (long long)g.H * g.W + (bwd ? 2LL * g.Ho * g.Wo : 0);
-  if (per_plane > MNV_POOL_LDS_FLOATS) return 0;
-  long long ppb = MNV_POOL_LDS_FLOATS / per_plane;
-  long long cap = planes / 2048;  // keep at least ~2048 workgroups
+  const long long hw = (long long)g.H * g.W, howo = (long long)g.Ho * g.Wo;
+  long long ppb = (MNV_POOL_X_FLOATS - 6) / hw;
+  if (bwd) {
+    ppb = std::min(ppb, (MNV_POOL_D_FLOATS - 6) / howo);
+    ppb = std::min(ppb, (12288 - 24) / (hw + 2 * howo));
+  }
+  if (ppb < 1) return 0;
+  long long cap = planes / 4096;
   if (cap < 1) cap = 1;
   if (ppb > cap) ppb = cap;
   if (ppb > 64) ppb = 64;
   return (int)ppb;
+}
+
+// Workgroups of a pipelined launch: all that fit on the chip at once, each looping over
+// its share of the groups.
+unsigned lds_grid(long long groups, size_t lds_bytes) {
+  long long per_cu = (160 * 1024) / (long long)(lds_bytes + 512);
+  if (per_cu > 8) per_cu = 8;
+  if (per_cu < 1) per_cu = 1;
+  long long blocks = 256 * per_cu;
+  return (unsigned)(groups < blocks ? groups : blocks);
 }
 
 template <bool MAX>
@@ -277,14 +490,16 @@ int pool_fwd(const float* bottom, float* top, int n, int c, int h, int w, int sv
   int rc = make_geom(&g, n, c, h, w, sv, sh, kh, kw, ph, pw);
   if (rc) return rc;
   long long planes = (long long)n * c;
-  int ppb = planes_per_block(g, planes, false);
+  int ppb = mnv_aligned16(bottom) ? planes_per_block(g, planes, false) : 0;
   if (ppb > 0) {
-    size_t lds = (size_t)ppb * h * w * sizeof(float);
-    long long blocks = (planes + ppb - 1) / ppb;
-    if (blocks > 65536) blocks = 65536;
-    hipLaunchKernelGGL((mnv_pool_fwd_lds_kernel<MAX>), dim3((unsigned)blocks),
-                       dim3(MNV_POOL_THREADS), lds, mnv_stream(stream), bottom, top, (int)planes,
-                       ppb, g);
+    size_t lds = ((size_t)ppb * h * w + 8) * sizeof(float);
+    long long groups = (planes + ppb - 1) / ppb;
+    const bool sq = kh == kw && sv == sh;
+    auto kernel = (sq && kh == 3 && sv == 2)   ? mnv_pool_fwd_lds_kernel<MAX, 3, 2>
+                  : (sq && kh == 2 && sv == 2) ? mnv_pool_fwd_lds_kernel<MAX, 2, 2>
+                                               : mnv_pool_fwd_lds_kernel<MAX, 0, 0>;
+    hipLaunchKernelGGL(kernel, dim3(lds_grid(groups, lds)), dim3(MNV_POOL_THREADS), lds,
+                       mnv_stream(stream), bottom, top, (int)planes, ppb, g);
   } else {
     hipLaunchKernelGGL((mnv_pool_fwd_kernel<MAX>), dim3(pool_grid((size_t)planes * g.Ho * g.Wo)),
                        dim3(MNV_POOL_THREADS), 0, mnv_stream(stream), bottom, top, (size_t)planes,
@@ -301,16 +516,19 @@ int pool_bwd(const float* bottom, const float* top_diff, float* bottom_diff, int
   int rc = make_geom(&g, n, c, h, w, sv, sh, kh, kw, ph, pw);
   if (rc) return rc;
   long long planes = (long long)n * c;
-  int ppb = planes_per_block(g, planes, true);
+  int ppb = (mnv_aligned16(bottom) && mnv_aligned16(top_diff) && mnv_aligned16(bottom_diff))
+                ? planes_per_block(g, planes, true)
+                : 0;
   if (ppb > 0) {
-    size_t lds = (size_t)ppb * ((size_t)h * w + 2 * (size_t)g.Ho * g.Wo) * sizeof(float);
-    long long blocks = (planes + ppb - 1) / ppb;
-    if (blocks > 65536) blocks = 65536;
-    const int st = (sv == sh && (sv == 1 || sv == 2)) ? sv : 0;
-    auto kernel = st == 1   ? mnv_pool_bwd_lds_kernel<MAX, 1>
-                  : st == 2 ? mnv_pool_bwd_lds_kernel<MAX, 2>
-                            : mnv_pool_bwd_lds_kernel<MAX, 0>;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(MNV_POOL_THREADS), lds,
+    const size_t hw = (size_t)h * w, howo = (size_t)g.Ho * g.Wo;
+    size_t lds = (((ppb * hw + 8 + 3) & ~(size_t)3) + ((ppb * howo + 8 + 3) & ~(size_t)3) +
+                  ppb * howo) * sizeof(float);
+    long long groups = (planes + ppb - 1) / ppb;
+    const bool sq = kh == kw && sv == sh;
+    auto kernel = (sq && kh == 3 && sv == 2)   ? mnv_pool_bwd_lds_kernel<MAX, 3, 2>
+                  : (sq && kh == 2 && sv == 2) ? mnv_pool_bwd_lds_kernel<MAX, 2, 2>
+                                               : mnv_pool_bwd_lds_kernel<MAX, 0, 0>;
+    hipLaunchKernelGGL(kernel, dim3(lds_grid(groups, lds)), dim3(MNV_POOL_THREADS), lds,
                        mnv_stream(stream), bottom, top_diff, bottom_diff, (int)planes, ppb, g);
   } else {
     hipLaunchKernelGGL((mnv_pool_bwd_kernel<MAX>), dim3(pool_grid((size_t)planes * h * w)),

@@ -242,6 +242,10 @@ POOL = [
     (4, 32, 12, 12, 3, 3, 3, 3, 0, 0),
     (1, 3, 100, 95, 2, 2, 3, 3, 1, 1),    # planes too large for the LDS-staged kernels
     (70, 33, 5, 7, 1, 2, 2, 3, 1, 1),     # many tiny planes per workgroup, odd plane size
+    (3, 5, 9, 11, 2, 2, 3, 3, 1, 1),      # padded 3x3/2 and 2x2/2: the 2x2-block gradient
+    (3, 5, 8, 10, 2, 2, 2, 2, 1, 1),      #   path with blocks that start outside the plane
+    (2, 7, 10, 9, 2, 2, 3, 3, 0, 0),      # even height: clipped last window
+    (5000, 1, 6, 6, 2, 2, 3, 3, 0, 0),    # more groups than resident workgroups
 ]
 
 
