@@ -129,6 +129,90 @@ struct ConvFwd {
   }
 };
 
+// Forward without padding (ph == pw == 0, any channel count and stride).  Every tap of
+// every output position is a real pixel, so the pixel offset is base(position) + koff(k)
+// with koff(k) = ((c*H + R-1-r')*W + S-1-s')*4 for the flat reduction index k = (c, r', s').
+// koff is tabulated in LDS once per workgroup; a slab then costs one LDS read and four
+// adds per vector, and nothing is decomposed or bounds-tested in the main loop.  The
+// filter needs no copy: in this order it already is the column-major K x Kout operand.
+// Period 0 holds the full slabs, period 1 the last, partial one (masked filter loads).
+struct ConvFwdNP {
+  static constexpr bool A_KFAST = false, B_KFAST = true;
+  static constexpr int A_NOFF = 4, B_NOFF = 4;
+  const float* __restrict__ bottom;
+  const float* __restrict__ filter;
+  const float* __restrict__ bias;
+  float* __restrict__ top;
+  ConvGeom g;
+  int M, N, K, total_slabs, spp;  // GEMM extents: N*Ho*Wo, Kout, C*R*S
+  struct Res {
+    mnv_rsrc a, b;
+    const unsigned* tab;  // LDS: [total_slabs*16] byte offsets, MNV_OOB past K
+  };
+  struct AState {};
+  struct BState {};
+  __device__ void make_res(Res& r) const {
+    r.a = mnv_make_rsrc(bottom, (unsigned)(g.N * g.C * g.HW) * 4u);
+    r.b = mnv_make_rsrc(filter, (unsigned)(g.K * g.CRS) * 4u);
+    r.tab = nullptr;
+  }
+  size_t extra_lds_bytes() const { return (size_t)total_slabs * 16 * sizeof(unsigned); }
+  __device__ void block_init(Res& r, float* extra, int, int) const {
+    unsigned* tab = reinterpret_cast<unsigned*>(extra);
+    r.tab = tab;
+    for (int k = threadIdx.x; k < total_slabs * 16; k += blockDim.x) {
+      int c = mnv_fastdiv(k, g.d_RS);
+      int rs = k - c * g.RS;
+      int rp = mnv_fastdiv(rs, g.d_S), sp = rs - rp * g.S;
+      tab[k] = k < K ? (unsigned)(c * g.HW + (g.R - 1 - rp) * g.W + (g.S - 1 - sp)) * 4u : MNV_OOB;
+    }
+  }
+  __device__ void a_init(const Res&, AState&, int) const {}
+  __device__ void b_init(const Res&, BState&, int) const {}
+  // rows past M are never stored, so they may read any valid pixel
+  __device__ void a_period(const AState&, unsigned (&off)[4], int m, int, int) const {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      int mm = m + q < M ? m + q : 0;
+      int img = mnv_fastdiv(mm, g.d_HoWo);
+      int pos = mm - img * g.HoWo;
+      int i = mnv_fastdiv(pos, g.d_Wo);
+      int j = pos - i * g.Wo;
+      off[q] = (unsigned)(img * g.C * g.HW + i * g.sv * g.W + j * g.sh) * 4u;
+    }
+  }
+  __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[4], int period, int s,
+                         int kl, float (&v)[4]) const {
+    const unsigned t = r.tab[(period * spp + s) * 16 + kl];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      v[q] = __builtin_bit_cast(float,
+                                __builtin_amdgcn_raw_buffer_load_b32(r.a, (int)(off[q] + t), 0, 0));
+  }
+  // filter element (k, n) at n*K + k: four consecutive k are one 16-byte load (4-byte
+  // aligned is enough for a buffer load)
+  __device__ void b_period(const BState&, unsigned (&off)[4], int n, int kl, int period) const {
+    int k = period * spp * 16 + kl;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      off[q] = ((n < N) & (k + q < K)) ? (unsigned)(n * K + k + q) * 4u : MNV_OOB;
+  }
+  __device__ void b_load(const Res& r, const BState&, const unsigned (&off)[4], int period, int s,
+                         int, float (&v)[4]) const {
+    if (period == 0 && spp * 16 <= K) {  // uniform: a full slab
+      const unsigned one[1] = {off[0]};
+      mnv_fetch_vec<1>(r.b, one, (unsigned)s * 64u, v);
+    } else {
+      mnv_fetch_vec<4>(r.b, off, (unsigned)s * 64u, v);
+    }
+  }
+  __device__ void c_store(int m, int n, float x) const {
+    int img = mnv_fastdiv(m, g.d_HoWo);
+    int pos = m - img * g.HoWo;
+    top[((size_t)img * N + n) * g.HoWo + pos] = x + bias[n];
+  }
+};
+
 // ------------------------------------------------------------ backward data
 // FAST additionally means both strides are 1, so every (row, col) of the shifted window
 // is a real output position.
@@ -322,6 +406,11 @@ struct ConvBwdFilter {
 // image); a slab's im2col offsets are then one 16-byte LDS read and four adds per vector.
 // top_diff is read with 16-byte loads of 4 consecutive positions; only the last, partial
 // slab of an image needs per-element masking.
+//
+// NP ("no padding", any channel count): with ph == pw == 0 every tap of every output
+// position is a real pixel, so the pixel offset splits into a row part (channel, tap) and a
+// position part: one position table serves all rows, which stay in (channel, tap) order.
+template <bool NP>
 struct ConvBwdFilterFast {
   static constexpr bool A_KFAST = true, B_KFAST = true;
   static constexpr int A_NOFF = 1, B_NOFF = 1;
@@ -358,15 +447,23 @@ struct ConvBwdFilterFast {
       int t = e / PP, pos = e - t * PP;
       int tap = tap0 + t;
       int rp = mnv_fastdiv(tap, g.d_S), sp = tap - rp * g.S;
-      int dy = g.R - 1 - rp - g.ph, dx = g.S - 1 - sp - g.pw;
+      int dy = NP ? 0 : g.R - 1 - rp - g.ph, dx = NP ? 0 : g.S - 1 - sp - g.pw;
       int i = mnv_fastdiv(pos, g.d_Wo), j = pos - i * g.Wo;
       int y = i * g.sv + dy, x = j * g.sh + dx;
-      bool ok = (pos < g.HoWo) & (tap < g.RS) & ((unsigned)y < (unsigned)g.H) &
+      bool ok = (pos < g.HoWo) & (NP | (tap < g.RS)) & ((unsigned)y < (unsigned)g.H) &
                 ((unsigned)x < (unsigned)g.W);
       tab[e] = ok ? (unsigned)(y * g.W + x) * 4u : MNV_OOB;
     }
   }
   __device__ void a_init(const Res& res, AState& st, int m) const {
+    if (NP) {  // m = (c, r', s'); the tap's shift is part of the row offset
+      int c = mnv_fastdiv(m, g.d_RS);
+      int rs = m - c * g.RS;
+      int rp = mnv_fastdiv(rs, g.d_S), sp = rs - rp * g.S;
+      st.cbase = m < M ? (unsigned)(c * g.HW + (g.R - 1 - rp) * g.W + (g.S - 1 - sp)) * 4u : MNV_OOB;
+      st.trow = 0;
+      return;
+    }
     int tap = mnv_fastdiv(m, d_C);
     int c = m - tap * g.C;
     st.cbase = m < M ? (unsigned)(c * g.HW) * 4u : MNV_OOB;
@@ -404,6 +501,10 @@ struct ConvBwdFilterFast {
     }
   }
   __device__ void c_store(int m, int n, float x) const {
+    if (NP) {
+      filter_diff[(size_t)n * M + m] = x;
+      return;
+    }
     int tap = mnv_fastdiv(m, d_C);
     int c = m - tap * g.C;
     filter_diff[(size_t)n * M + c * g.RS + tap] = x;
@@ -543,6 +644,10 @@ int mnv_conv_fwd(const float* bottom, const float* filter, const float* bias, fl
     ConvFwd<true> p{bottom, wp, bias, top, g, gm, gn, gk, g.RS * (C / 16), C / 16};
     return launch_tile(tile, p, 1, nullptr, s);
   }
+  if (ph == 0 && pw == 0 && gk <= 4096) {
+    ConvFwdNP p{bottom, filter, bias, top, g, gm, gn, gk, (gk + 15) / 16, gk >= 16 ? gk / 16 : 1};
+    return launch_tile(tile, p, 1, nullptr, s);
+  }
   ConvFwd<false> p{bottom, filter, bias, top, g, gm, gn, gk, (gk + 15) / 16, 1};
   return launch_tile(tile, p, 1, nullptr, s);
 }
@@ -599,9 +704,14 @@ int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filte
   // tables of all taps a 128-row tile touches must fit beside the tiles.
   const int PP = (g.HoWo + 15) / 16 * 16;
   const int taps_per_block = (128 + C - 1) / C + 1;
+  if (tile != 0 && ph == 0 && pw == 0 && (size_t)PP * 4 <= 24 * 1024) {
+    ConvBwdFilterFast<true> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
+                              PP / 16, PP, 1, mnv_fastdiv_make(C)};
+    return launch_tile(tile, p, splits, workspace, s);
+  }
   if (tile != 0 && (size_t)taps_per_block * PP * 4 <= 24 * 1024) {
-    ConvBwdFilterFast p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16), PP / 16,
-                        PP, taps_per_block, mnv_fastdiv_make(C)};
+    ConvBwdFilterFast<false> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
+                               PP / 16, PP, taps_per_block, mnv_fastdiv_make(C)};
     return launch_tile(tile, p, splits, workspace, s);
   }
   ConvBwdFilter p{bottom, top_diff, filter_diff, g, gm, gn, gk, (gk + 15) / 16, 1};
