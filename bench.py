@@ -131,6 +131,19 @@ def micro_bench():
              "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
                           "unit": "TFLOP/s", "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}}
     log("sgemm 4096^3: %.3f ms, %.1f TFLOP/s" % (ms, tf))
+    # the other shapes of BASELINE.json configs[2], with the split-k workspace the host layer lends
+    shapes = []
+    for (mm, kk, nn) in ((256, 9216, 4096), (4096, 4096, 256), (1000, 4096, 256)):
+        aa = dev.upload(rng.standard_normal(mm * kk, dtype=np.float32))
+        bb = dev.upload(rng.standard_normal(kk * nn, dtype=np.float32))
+        cc = dev.empty(mm * nn)
+        wsb = L.mnv_sgemm_nn_workspace_bytes(mm, nn, kk)
+        ws = dev.empty(wsb // 4 + 1)
+        t = dev.time_ms(lambda: L.mnv_sgemm_nn(aa.p, bb.p, cc.p, mm, nn, kk, ws.p,
+                                               ctypes.c_size_t(wsb), dev.stream), iters=20, warmup=5)
+        shapes.append({"MxKxN": "%dx%dx%d" % (mm, kk, nn), "ms": round(t, 4),
+                       "tflops": round(2.0 * mm * nn * kk / (t * 1e-3) / 1e12, 2)})
+    sgemm["other_shapes"] = shapes
     ne = 8192 * 8192
     # three distinct 256 MiB buffers: 768 MiB per pass, larger than the 256 MB last-level cache
     x = dev.upload(rng.standard_normal(ne, dtype=np.float32))
@@ -181,6 +194,36 @@ def bandwidth_table(L, dev, x, y, z, ne):
         table.append({"op": name, "ms": round(ms, 4), "gbs": round(gbs, 1),
                       "frac": round(gbs / PEAK_HBM_GBS, 4)})
     return table
+
+
+def small_nets(steps=20, warmup=3):
+    """BASELINE.json configs[0] (MLP) and configs[3] (CNN) at batch 256: latency-bound
+    graphs, reported as ms/step and operators/step without a roofline claim."""
+    from minerva_amd import hostapi
+    from oracle import nets  # input generator only
+    out = {}
+    for name in ("mlp", "cnn"):
+        params, data, label = nets.make_inputs(name, BATCH)
+        rt = hostapi.Runtime(0, sync_each_op=False)
+        net = hostapi.Net(rt, name, BATCH)
+        for k, v in params.items():
+            net.set_param(k, v)
+        net.load_batch(data, label)
+        for _ in range(warmup):
+            net.step(0.01)
+        rt.sync()
+        ops0 = rt.ops_issued()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            net.step(0.01)
+            rt.sync()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        out[name + "_b256"] = {"ms_per_step": round(ms, 4), "images_per_s": round(BATCH / ms * 1e3, 1),
+                               "ops_per_step": (rt.ops_issued() - ops0) // steps}
+        log("%s b=%d: %.3f ms/step" % (name, BATCH, ms))
+        net.close()
+        rt.close()
+    return out
 
 
 def cpu_baseline(batch=4):
@@ -236,6 +279,7 @@ def main():
         "roofline": roof,
         "sgemm": sgemm,
         "eltwise": elt,
+        "small_nets": small_nets(),
         "top_ops": op_table(main_run["profile"], args.steps),
         "device": dev_info,
         "outputs_finite": main_run["finite"] and res["per_op_sync"]["finite"],
