@@ -186,11 +186,35 @@ def bandwidth_table(L, dev, x, y, z, ne):
         ("max dim 1", 4, lambda: L.mnv_reduce_max_row(x.p, small.p, m, n, S)),
         ("maxindex dim 0", 4, lambda: L.mnv_maxindex_col(x.p, small.p, m, n, S)),
         ("softmax rows", 8, lambda: L.mnv_softmax_instance_fwd(x.p, z.p, n, m, 1, 1, S)),
+        ("softmax rows bwd", 12, lambda: L.mnv_softmax_instance_bwd(x.p, y.p, z.p, n, m, 1, 1, S)),
+        ("transpose", 8, lambda: L.mnv_transpose(x.p, z.p, m, n, S)),
     ]
     table = []
     for name, bpe, fn in ops:
         ms = dev.time_ms(fn, iters=20, warmup=3)
         gbs = bpe * ne / (ms * 1e-3) / 1e9
+        table.append({"op": name, "ms": round(ms, 4), "gbs": round(gbs, 1),
+                      "frac": round(gbs / PEAK_HBM_GBS, 4)})
+    # AlexNet pool1 at batch 256 ({55,55,96,256} -> {27,27,96,256}, 3x3 stride 2) and the
+    # conv1 bias gradient, in the same buffers: bytes = every tensor once
+    geo = (256, 96, 55, 55, 2, 2, 3, 3, 0, 0)
+    nin, nout = 256 * 96 * 55 * 55, 256 * 96 * 27 * 27
+    px = dev.upload(np.random.default_rng(9).standard_normal(nin, dtype=np.float32))
+    py, pdy, pdx = dev.empty(nout), dev.empty(nout), dev.empty(nin)
+    L.mnv_fill(pdy.p, nout, f(0.5), S)
+    bias_ws = dev.empty(1 << 18)  # 1 MiB
+    assert px.n == nin and pdx.n == nin and py.n == nout and pdy.n == nout and small.n >= 96
+    extra = [
+        ("maxpool 3x3/2 fwd (pool1)", 4 * (nin + nout), lambda: L.mnv_maxpool_fwd(px.p, py.p, *geo, S)),
+        ("maxpool 3x3/2 bwd (pool1)", 4 * (2 * nin + nout),
+         lambda: L.mnv_maxpool_bwd(px.p, py.p, pdy.p, pdx.p, *geo, S)),
+        ("conv bias gradient (conv1)", 4 * nin,
+         lambda: L.mnv_conv_bwd_bias(px.p, small.p, 256, 96, 55, 55, bias_ws.p,
+                                     ctypes.c_size_t(1 << 20), S)),
+    ]
+    for name, nbytes, fn in extra:
+        ms = dev.time_ms(fn, iters=20, warmup=3)
+        gbs = nbytes / (ms * 1e-3) / 1e9
         table.append({"op": name, "ms": round(ms, 4), "gbs": round(gbs, 1),
                       "frac": round(gbs / PEAK_HBM_GBS, 4)})
     return table
