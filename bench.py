@@ -203,6 +203,7 @@ def bandwidth_table(L, dev, x, y, z, ne):
     py, pdy, pdx = dev.empty(nout), dev.empty(nout), dev.empty(nin)
     L.mnv_fill(pdy.p, nout, f(0.5), S)
     bias_ws = dev.empty(1 << 18)  # 1 MiB
+    z2 = dev.empty(nin)
     assert px.n == nin and pdx.n == nin and py.n == nout and pdy.n == nout and small.n >= 96
     extra = [
         ("maxpool 3x3/2 fwd (pool1)", 4 * (nin + nout), lambda: L.mnv_maxpool_fwd(px.p, py.p, *geo, S)),
@@ -211,6 +212,15 @@ def bandwidth_table(L, dev, x, y, z, ne):
         ("conv bias gradient (conv1)", 4 * nin,
          lambda: L.mnv_conv_bwd_bias(px.p, small.p, 256, 96, 55, 55, bias_ws.p,
                                      ctypes.c_size_t(1 << 20), S)),
+    ]
+    # LRN over the same {55,55,96,256} tensor (Caffe-style norm1: local_size 5, alpha 1e-4,
+    # beta 0.75): forward reads bottom and writes scale and top, backward reads four tensors
+    lsc, ltop = dev.empty(nin), dev.empty(nin)
+    lrn = (5, f(1e-4), f(0.75), 256, 96, 55, 55)
+    extra += [
+        ("lrn fwd (norm1)", 12 * nin, lambda: L.mnv_lrn_fwd(px.p, lsc.p, ltop.p, *lrn, S)),
+        ("lrn bwd (norm1)", 20 * nin,
+         lambda: L.mnv_lrn_bwd(px.p, ltop.p, lsc.p, pdx.p, z2.p, *lrn, S)),
     ]
     for name, nbytes, fn in extra:
         ms = dev.time_ms(fn, iters=20, warmup=3)

@@ -248,6 +248,23 @@ int mnv_avgpool_bwd(const float* bottom, const float* top, const float* top_diff
                     int window_height, int window_width, int pad_height, int pad_width,
                     mnv_stream_t stream);
 
+/* ---- local response normalisation across channels: CudaPerformLRN{Forward,Backward}
+ * (cuda_perform.h:72-76; kernels cuda_kernel.h:223-331).  Tensor {W,H,C,N}.
+ *   scale = 1 + alpha/local_size * (sum of bottom^2 over the channel window)
+ *   top   = bottom * scale^(-beta)
+ * forward writes both `scale` and `top` (the reference passes `scale` as an input
+ * tensor and fills it, cuda.cpp:45-59); backward reads them:
+ *   bottom_diff = top_diff * scale^(-beta)
+ *                 - 2*alpha*beta/local_size * bottom * (sum of top_diff*top/scale over the window)
+ * The window of channel c is [c - (local_size-1)/2, c + local_size/2] forward and its
+ * mirror image backward, clipped to the channels. ---- */
+int mnv_lrn_fwd(const float* bottom, float* scale, float* top, int local_size, float alpha,
+                float beta, int num_images, int num_channels, int height, int width,
+                mnv_stream_t stream);
+int mnv_lrn_bwd(const float* bottom, const float* top, const float* scale, const float* top_diff,
+                float* bottom_diff, int local_size, float alpha, float beta, int num_images,
+                int num_channels, int height, int width, mnv_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -79,6 +79,8 @@ for _m in ("instance", "channel"):
 for _k in ("max", "avg"):
     PROTOTYPES["mnv_%spool_fwd" % _k] = [_P, _P] + [_I] * 10 + [_S]
     PROTOTYPES["mnv_%spool_bwd" % _k] = [_P, _P, _P, _P] + [_I] * 10 + [_S]
+PROTOTYPES["mnv_lrn_fwd"] = [_P, _P, _P, _I, c_f, c_f, _I, _I, _I, _I, _S]
+PROTOTYPES["mnv_lrn_bwd"] = [_P, _P, _P, _P, _P, _I, c_f, c_f, _I, _I, _I, _I, _S]
 
 _RESTYPES = {
     "mnv_error_string": ctypes.c_char_p,

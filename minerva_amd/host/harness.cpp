@@ -192,6 +192,16 @@ int mnvh_op(void* runtime, const char* op_name, const mnvh_tensor* inputs, int n
     } else if (op == "pooling_backward") {
       need(3);
       r = rt->PoolingBackward(in[0], in[1], in[2], pool_info());
+    } else if (op == "lrn_forward") {  // params: local_size, alpha, beta; inputs: bottom, scale
+      need(2);
+      MNV_CHECK(n_params >= 3) << "lrn_forward takes local_size, alpha, beta";
+      r = rt->LRNForward(in[0], in[1], static_cast<int>(params[0]), static_cast<float>(params[1]),
+                         static_cast<float>(params[2]));
+    } else if (op == "lrn_backward") {  // inputs: bottom, top, scale, top_diff
+      need(4);
+      MNV_CHECK(n_params >= 3) << "lrn_backward takes local_size, alpha, beta";
+      r = rt->LRNBackward(in[0], in[1], in[2], in[3], static_cast<int>(params[0]),
+                          static_cast<float>(params[1]), static_cast<float>(params[2]));
     } else if (op == "fill") {
       need(0);
       std::vector<int> d;

@@ -360,6 +360,30 @@ void PoolingBackward(const DataList& inputs, const DataList& outputs, PoolingBac
      "pooling backward");
 }
 
+// inputs {bottom, scale}: `scale` arrives as an input and is filled by the operator, as in
+// the reference (cuda.cpp:45-59); data_shape is the {W,H,C,N} extent of bottom.
+void LRNForward(const DataList& inputs, const DataList& outputs, LRNForwardClosure& c,
+                const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 2u) << "(LRNForward) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(LRNForward) #outputs is wrong!";
+  MNV_CHECK_EQ(c.data_shape.NumDims(), 4u) << "(LRNForward) data shape must be {W,H,C,N}";
+  Ok(mnv_lrn_fwd(inputs[0].data_, inputs[1].data_, outputs[0].data_, c.local_size, c.alpha, c.beta,
+                 c.data_shape[3], c.data_shape[2], c.data_shape[1], c.data_shape[0], ctx.stream),
+     "LRN forward");
+}
+
+// inputs {bottom, top, scale, top_diff} (cuda.cpp:61-77)
+void LRNBackward(const DataList& inputs, const DataList& outputs, LRNBackwardClosure& c,
+                 const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 4u) << "(LRNBackward) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(LRNBackward) #outputs is wrong!";
+  MNV_CHECK_EQ(c.data_shape.NumDims(), 4u) << "(LRNBackward) data shape must be {W,H,C,N}";
+  Ok(mnv_lrn_bwd(inputs[0].data_, inputs[1].data_, inputs[2].data_, inputs[3].data_,
+                 outputs[0].data_, c.local_size, c.alpha, c.beta, c.data_shape[3], c.data_shape[2],
+                 c.data_shape[1], c.data_shape[0], ctx.stream),
+     "LRN backward");
+}
+
 void ArrayLoader(const DataList& outputs, ArrayLoaderClosure& closure, const Context& ctx) {
   MNV_CHECK_EQ(outputs.size(), 1u) << "(array loader) #outputs wrong";
   MNV_CHECK(closure.data) << "probably already executed";

@@ -34,6 +34,8 @@ void ActivationForward(const DataList&, const DataList&, ActivationForwardClosur
 void ActivationBackward(const DataList&, const DataList&, ActivationBackwardClosure&, const Context&);
 void PoolingForward(const DataList&, const DataList&, PoolingForwardClosure&, const Context&);
 void PoolingBackward(const DataList&, const DataList&, PoolingBackwardClosure&, const Context&);
+void LRNForward(const DataList&, const DataList&, LRNForwardClosure&, const Context&);
+void LRNBackward(const DataList&, const DataList&, LRNBackwardClosure&, const Context&);
 
 void ArrayLoader(const DataList&, ArrayLoaderClosure&, const Context&);
 void Fill(const DataList&, FillClosure&, const Context&);

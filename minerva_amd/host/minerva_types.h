@@ -187,4 +187,13 @@ template <int i> struct PoolingClosure {
 typedef PoolingClosure<0> PoolingForwardClosure;
 typedef PoolingClosure<1> PoolingBackwardClosure;
 
+// reference minerva/op/closure.h:151-158
+template <int i> struct LRNClosure {
+  int local_size;
+  float alpha, beta;
+  Scale data_shape;
+};
+typedef LRNClosure<0> LRNForwardClosure;
+typedef LRNClosure<1> LRNBackwardClosure;
+
 }  // namespace minerva

@@ -65,6 +65,8 @@ MNV_INSTALL_COMPUTE_FN(ActivationForwardClosure, hip::ActivationForward)
 MNV_INSTALL_COMPUTE_FN(ActivationBackwardClosure, hip::ActivationBackward)
 MNV_INSTALL_COMPUTE_FN(PoolingForwardClosure, hip::PoolingForward)
 MNV_INSTALL_COMPUTE_FN(PoolingBackwardClosure, hip::PoolingBackward)
+MNV_INSTALL_COMPUTE_FN(LRNForwardClosure, hip::LRNForward)
+MNV_INSTALL_COMPUTE_FN(LRNBackwardClosure, hip::LRNBackward)
 MNV_INSTALL_DATAGEN_FN(ArrayLoaderClosure, hip::ArrayLoader)
 MNV_INSTALL_DATAGEN_FN(FillClosure, hip::Fill)
 
@@ -112,6 +114,8 @@ MNV_SIMPLE_OP(ReluBackwardOp, ComputeFnWithClosure, ReluBackwardClosure, "relu b
 MNV_SIMPLE_OP(TanhForwardOp, ComputeFnWithClosure, TanhForwardClosure, "tanh forward")
 MNV_SIMPLE_OP(TanhBackwardOp, ComputeFnWithClosure, TanhBackwardClosure, "tanh backward")
 MNV_SIMPLE_OP(ConvBackwardBiasOp, ComputeFnWithClosure, ConvBackwardBiasClosure, "conv bp bias")
+MNV_SIMPLE_OP(LRNForwardOp, ComputeFnWithClosure, LRNForwardClosure, "LRN Forward")
+MNV_SIMPLE_OP(LRNBackwardOp, ComputeFnWithClosure, LRNBackwardClosure, "LRN Backward")
 
 class FillOp : public PhyDataGenFnWithClosure<FillClosure> {
  public:

@@ -239,4 +239,24 @@ Tensor Runner::PoolingBackward(const Tensor& diff, const Tensor& top, const Tens
   return Compute({diff, top, bottom}, bottom->size, op);
 }
 
+Tensor Runner::LRNForward(const Tensor& src, const Tensor& scale, int local_size, float alpha,
+                          float beta) {
+  MNV_CHECK_EQ(src->size.NumDims(), 4u);
+  CheckSame(src, scale);
+  auto op = std::make_shared<LRNForwardOp>();
+  op->closure = {local_size, alpha, beta, src->size};
+  return Compute({src, scale}, src->size, op);
+}
+
+Tensor Runner::LRNBackward(const Tensor& bottom, const Tensor& top, const Tensor& scale,
+                           const Tensor& top_diff, int local_size, float alpha, float beta) {
+  MNV_CHECK_EQ(bottom->size.NumDims(), 4u);
+  CheckSame(bottom, top);
+  CheckSame(bottom, scale);
+  CheckSame(bottom, top_diff);
+  auto op = std::make_shared<LRNBackwardOp>();
+  op->closure = {local_size, alpha, beta, bottom->size};
+  return Compute({bottom, top, scale, top_diff}, bottom->size, op);
+}
+
 }  // namespace minerva

@@ -84,6 +84,11 @@ class Runner : public DeviceListener {
   Tensor PoolingForward(const Tensor& src, PoolingInfo info);
   Tensor PoolingBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom,
                          PoolingInfo info);
+  // reference minerva/narray/convolution.cpp:165-175; `scale` is filled by the forward pass
+  Tensor LRNForward(const Tensor& src, const Tensor& scale, int local_size, float alpha,
+                    float beta);
+  Tensor LRNBackward(const Tensor& bottom, const Tensor& top, const Tensor& scale,
+                     const Tensor& top_diff, int local_size, float alpha, float beta);
 
  private:
   friend struct TensorNode;

@@ -583,3 +583,65 @@ int ora_pool_bwd(int alg, const float* top_diff, const float* top, const float* 
   }
   return 0;
 }
+
+/* ------------------------------------------------------------------------- */
+/* Local response normalisation across channels.  The reference has no CPU     */
+/* implementation; this restates its CUDA kernels LRNFillScale /                */
+/* LRNComputeOutput / LRNComputeDiff (minerva/op/impl/cuda/cuda_kernel.h:223-331,*/
+/* launch arguments minerva/op/impl/cuda/cuda_perform.cu:643-667): one sequential*/
+/* walk over the channels of every (image, position) with an fp32 running sum   */
+/* (add the entering channel, then subtract the leaving one).  The walk is       */
+/* written as one loop; for channels >= local_size it performs the reference's   */
+/* operations in the reference's order, for channels < local_size (where the     */
+/* reference reads past the tensor) the window is clipped to the channels.       */
+/* parity unpinned: no reference test covers LRN; pinned by the closed form in   */
+/* fp64 and, for the backward pass, by finite differences of the forward one.    */
+/* ------------------------------------------------------------------------- */
+int ora_lrn_fwd(const float* bottom, float* scale, float* top, int size, float alpha, float beta,
+                int N, int C, int H, int W) {
+  if (size <= 0) return -1;
+  const size_t step = (size_t)H * W;
+  const float alpha_over_size = alpha / size; /* cuda_perform.cu:649 */
+  const int pre_pad = (size - 1) / 2, post_pad = size - pre_pad - 1; /* cuda_kernel.h:234-235 */
+  for (int n = 0; n < N; ++n)
+    for (size_t p = 0; p < step; ++p) {
+      const size_t off = (size_t)n * C * step + p;
+      const float* in = bottom + off;
+      float accum = 0.f;
+      for (int head = 0; head < C + post_pad; ++head) {
+        if (head < C) accum += in[head * step] * in[head * step];
+        if (head >= size) accum -= in[(head - size) * step] * in[(head - size) * step];
+        if (head >= post_pad)
+          scale[off + (head - post_pad) * step] = 1.f + accum * alpha_over_size;
+      }
+    }
+  const size_t total = (size_t)N * C * step;
+  for (size_t i = 0; i < total; ++i) /* cuda_kernel.h:265-270 */
+    top[i] = bottom[i] * powf(scale[i], -beta);
+  return 0;
+}
+
+int ora_lrn_bwd(const float* bottom, const float* top, const float* scale, const float* top_diff,
+                float* bottom_diff, int size, float alpha, float beta, int N, int C, int H,
+                int W) {
+  if (size <= 0) return -1;
+  const size_t step = (size_t)H * W;
+  const float cache_ratio = (float)(2. * alpha * beta / size); /* cuda_perform.cu:665 */
+  const int pre_pad = size - (size + 1) / 2, post_pad = size - pre_pad - 1; /* cuda_kernel.h:291-292 */
+  for (int n = 0; n < N; ++n)
+    for (size_t p = 0; p < step; ++p) {
+      const size_t off = (size_t)n * C * step + p;
+      const float *x = bottom + off, *y = top + off, *sc = scale + off, *dy = top_diff + off;
+      float accum = 0.f;
+      for (int head = 0; head < C + post_pad; ++head) {
+        if (head < C) accum += dy[head * step] * y[head * step] / sc[head * step];
+        if (head >= size)
+          accum -= dy[(head - size) * step] * y[(head - size) * step] / sc[(head - size) * step];
+        if (head >= post_pad) {
+          const size_t o = (head - post_pad) * step;
+          bottom_diff[off + o] = dy[o] * powf(sc[o], -beta) - cache_ratio * x[o] * accum;
+        }
+      }
+    }
+  return 0;
+}

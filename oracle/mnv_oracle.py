@@ -245,3 +245,21 @@ def pool_bwd(alg, top_diff, top, bottom, N, C, H, W, sv, sh, kh, kw, ph, pw, wan
                             _p(mask) if want_mask else None, N, C, H, W, sv, sh, kh, kw, ph,
                             pw), "pool_bwd")
     return (out, mask) if want_mask else out
+
+
+def lrn_fwd(bottom, local_size, alpha, beta, N, C, H, W):
+    """Returns (top, scale)."""
+    bottom = _f(bottom)
+    scale = np.empty(bottom.size, dtype=np.float32)
+    top = np.empty(bottom.size, dtype=np.float32)
+    _chk(lib().ora_lrn_fwd(_p(bottom), _p(scale), _p(top), local_size, ctypes.c_float(alpha),
+                           ctypes.c_float(beta), N, C, H, W), "lrn_fwd")
+    return top, scale
+
+
+def lrn_bwd(bottom, top, scale, top_diff, local_size, alpha, beta, N, C, H, W):
+    bottom, top, scale, top_diff = _f(bottom), _f(top), _f(scale), _f(top_diff)
+    out = np.empty(bottom.size, dtype=np.float32)
+    _chk(lib().ora_lrn_bwd(_p(bottom), _p(top), _p(scale), _p(top_diff), _p(out), local_size,
+                           ctypes.c_float(alpha), ctypes.c_float(beta), N, C, H, W), "lrn_bwd")
+    return out

@@ -303,3 +303,54 @@ def test_pooling_batch_256_properties(gpu):
     # continuous data has no ties: every window routes to exactly one position
     assert abs(float(g.astype(np.float64).sum()) - float(dy.astype(np.float64).sum())) < 1e-2
     assert np.count_nonzero(g) <= dy.size
+
+
+# ----------------------------------------------------------------------- LRN
+LRN = [
+    # N, C, H, W, local_size, alpha, beta
+    (2, 8, 3, 5, 5, 1e-1, 0.75),
+    (3, 7, 4, 4, 3, 1e-2, 0.5),
+    (2, 9, 5, 3, 4, 2e-1, 0.75),      # even window: forward and backward windows differ
+    (1, 3, 6, 6, 5, 1e-1, 0.75),      # fewer channels than the window
+    (2, 4, 2, 2, 1, 1e-1, 0.75),
+    (2, 96, 27, 27, 5, 1e-4, 0.75),   # AlexNet norm1 (after pool1) and its constants
+    (2, 256, 13, 13, 5, 1e-4, 0.75),  # norm2
+    (70, 5, 9, 7, 5, 1e-1, 0.75),     # image boundaries inside a wavefront
+]
+
+
+@pytest.mark.parametrize("p", LRN)
+def test_lrn_against_oracle(gpu, ora, p):
+    N, C, H, W, size, alpha, beta = p
+    x = _rand(N * C * H * W, 60) * 3
+    dy = _rand(x.size, 61)
+    say("lrn", p)
+    dx, ds, dt = gpu.up(x), gpu.up(np.full(x.size, np.nan, np.float32)), gpu.up(np.full(x.size, np.nan, np.float32))
+    gpu.call("mnv_lrn_fwd", dx.p, ds.p, dt.p, size, ctypes.c_float(alpha), ctypes.c_float(beta), N, C, H, W)
+    top, scale = ora.lrn_fwd(x, size, alpha, beta, N, C, H, W)
+    assert normwise(gpu.down(ds), scale) <= 1e-6      # same operations in the same order
+    assert normwise(gpu.down(dt), top) <= TOL
+    # backward from the oracle's forward results, so that only the backward kernel is compared
+    dtop, dsc, ddy = gpu.up(top), gpu.up(scale), gpu.up(dy)
+    dbd = gpu.up(np.full(x.size, np.nan, np.float32))
+    gpu.call("mnv_lrn_bwd", dx.p, dtop.p, dsc.p, ddy.p, dbd.p, size, ctypes.c_float(alpha),
+             ctypes.c_float(beta), N, C, H, W)
+    assert normwise(gpu.down(dbd), ora.lrn_bwd(x, top, scale, dy, size, alpha, beta, N, C, H, W)) <= TOL
+
+
+def test_lrn_batch_256_properties(gpu):
+    """AlexNet norm1 at batch 256: the closed form in fp64 on sampled positions."""
+    N, C, H, W, size, alpha, beta = 256, 96, 27, 27, 5, 1e-4, 0.75
+    x = _rand(N * C * H * W, 62) * 10
+    dxb, ds, dt = gpu.up(x), gpu.empty(x.size), gpu.empty(x.size)
+    gpu.call("mnv_lrn_fwd", dxb.p, ds.p, dt.p, size, ctypes.c_float(alpha), ctypes.c_float(beta), N, C, H, W)
+    top = gpu.down(dt).reshape(N, C, H * W)
+    X = x.reshape(N, C, H * W).astype(np.float64)
+    rng = np.random.default_rng(63)
+    worst = 0.0
+    for _ in range(400):
+        n, c, p = int(rng.integers(N)), int(rng.integers(C)), int(rng.integers(H * W))
+        lo, hi = max(c - 2, 0), min(c + 2, C - 1)
+        s = 1.0 + alpha / size * np.sum(X[n, lo:hi + 1, p] ** 2)
+        worst = max(worst, abs(top[n, c, p] - X[n, c, p] * s ** (-beta)))
+    assert worst <= TOL * np.max(np.abs(top))

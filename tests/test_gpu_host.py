@@ -153,6 +153,21 @@ def test_pooling_golden_and_gradient(rt, ora):
         assert_bits_equal(back, ref, "pool bwd")
 
 
+def test_lrn_forward_and_backward(rt, ora):
+    W, H, C, N = 6, 5, 12, 3
+    size = [W, H, C, N]
+    x = _rand(W * H * C * N, 76) * 3
+    prm = [5, 1e-2, 0.75]
+    top, scale = ora.lrn_fwd(x, 5, 1e-2, 0.75, N, C, H, W)
+    got, od = rt.op("lrn_forward", [(x, size), (np.zeros_like(x), size)], prm)
+    assert od == size
+    assert normwise(got, top) <= TOL
+    dy = _rand(x.size, 77)
+    back, od = rt.op("lrn_backward", [(x, size), (top, size), (scale, size), (dy, size)], prm)
+    assert od == size
+    assert normwise(back, ora.lrn_bwd(x, top, scale, dy, 5, 1e-2, 0.75, N, C, H, W)) <= TOL
+
+
 def test_error_convention(rt):
     from minerva_amd import hostapi
     a = _rand(6, 76)
@@ -168,7 +183,7 @@ def test_error_convention(rt):
         rt.op("conv_forward", [(_rand(36, 78), [3, 3, 2, 2]), (a[:4], [2, 2, 1, 1]), (a[:1], [1])],
               [0, 0, 1, 1])
     with pytest.raises(hostapi.HostError, match="unknown operator"):
-        rt.op("lrn_forward", [(a, [6])])
+        rt.op("no_such_operator", [(a, [6])])
     # the runtime is still usable after a failed check
     got, _ = rt.op("arithmetic", [(a, [6]), (a, [6])], [0])
     assert_bits_equal(got, a + a, "after error")

@@ -380,3 +380,57 @@ def test_pooled_size_matches_ceil_mode_formula(ora):
                     if (want - 1) * s >= H + p:
                         want -= 1
                     assert ora.pooled_size(H, k, s, p) == want
+
+
+# ------------------------------------------------------------------------ LRN
+def _lrn64(x, size, alpha, beta, n, c, h, w, backward_window=False):
+    """fp64 closed form: (top, scale) with the window written out as a direct sum."""
+    X = x.reshape(n, c, h * w).astype(np.float64)
+    pre = size - (size + 1) // 2 if backward_window else (size - 1) // 2
+    post = size - pre - 1
+    scale = np.empty_like(X)
+    for k in range(c):
+        lo, hi = max(k - pre, 0), min(k + post, c - 1)
+        scale[:, k] = 1.0 + alpha / size * (X[:, lo:hi + 1] ** 2).sum(axis=1)
+    return (X * scale ** (-beta)).ravel(), scale.ravel()
+
+
+@pytest.mark.parametrize("size,c", [(5, 8), (3, 7), (1, 4), (5, 96), (4, 9), (5, 3)])
+def test_lrn_forward_closed_form(ora, size, c):
+    rng = np.random.default_rng(70 + size + c)
+    n, h, w = 2, 3, 4
+    alpha, beta = 1e-1, 0.75   # a large alpha makes the normalisation visible
+    x = (rng.standard_normal(n * c * h * w) * 3).astype(np.float32)
+    top, scale = ora.lrn_fwd(x, size, alpha, beta, n, c, h, w)
+    want_top, want_scale = _lrn64(x, size, alpha, beta, n, c, h, w)
+    assert np.max(np.abs(scale - want_scale) / want_scale) < 2e-6
+    assert np.max(np.abs(top - want_top)) <= 2e-6 * np.max(np.abs(want_top))
+    # a window shifted by one channel (the plausible off-by-one) must not pass
+    if size > 1 and c >= size:
+        X = x.reshape(n, c, h * w).astype(np.float64)
+        wrong = np.empty_like(X)
+        pre, post = (size - 1) // 2 + 1, size - (size - 1) // 2 - 2
+        for k in range(c):
+            lo, hi = max(k - pre, 0), min(k + post, c - 1)
+            wrong[:, k] = 1.0 + alpha / size * (X[:, lo:hi + 1] ** 2).sum(axis=1)
+        assert np.max(np.abs(scale - wrong.ravel()) / wrong.ravel()) > 1e-3
+
+
+@pytest.mark.parametrize("size,c", [(5, 8), (3, 5), (4, 7), (5, 3)])
+def test_lrn_backward_finite_difference(ora, size, c):
+    rng = np.random.default_rng(80 + size + c)
+    n, h, w = 1, 2, 2
+    alpha, beta = 2e-1, 0.75
+    x = rng.standard_normal(n * c * h * w).astype(np.float32)
+    dy = rng.standard_normal(x.size).astype(np.float32)
+    top, scale = ora.lrn_fwd(x, size, alpha, beta, n, c, h, w)
+    got = ora.lrn_bwd(x, top, scale, dy, size, alpha, beta, n, c, h, w)
+
+    def fwd(v):
+        return _lrn64(v, size, alpha, beta, n, c, h, w)[0]
+
+    # the backward window (cuda_kernel.h:291-292: pre_pad = size - (size+1)/2) is the adjoint
+    # of the forward one (cuda_kernel.h:234-235) for even sizes too, so the finite difference
+    # of the forward pass pins it
+    want = _fd(fwd, x.astype(np.float64), dy.astype(np.float64), eps=1e-4)
+    assert np.max(np.abs(got - want)) < 2e-5 * max(1.0, np.max(np.abs(want)))
