@@ -265,6 +265,23 @@ int mnv_lrn_bwd(const float* bottom, const float* top, const float* scale, const
                 float* bottom_diff, int local_size, float alpha, float beta, int num_images,
                 int num_channels, int height, int width, mnv_stream_t stream);
 
+/* ---- Concat / Slice / Select data movement (reference cuda.cpp:80-155, 644-655).
+ * The reference builds Concat and Slice from one CudaPerformCopy (cuda_perform.h:20) per
+ * image; here one 2-D copy per input tensor does it: `rows` rows of `row_elems` floats,
+ * row r read at src + r*src_pitch and written at dst + r*dst_pitch (pitches in floats,
+ * >= row_elems).  Concatenating along dimension d: rows = product of the dimensions above
+ * d, row_elems = (extent of this input along d) * (product of the dimensions below d),
+ * dst_pitch = the same with the output's extent, dst advanced by the extents of the inputs
+ * before it.  mnv_select replaces CudaPerformSelect (cuda_perform.h:76): dst{rows, n} takes
+ * columns indices[0..n) of the column-major src{rows, cols}.  The indices are host memory
+ * (the closure's vector); they are staged in `workspace` (mnv_select_workspace_bytes,
+ * required) instead of the reference's per-call cudaMalloc (cuda_perform.cu:674). ---- */
+int mnv_copy_2d(const float* src, float* dst, size_t row_elems, size_t rows, size_t src_pitch,
+                size_t dst_pitch, mnv_stream_t stream);
+size_t mnv_select_workspace_bytes(int num_indices);
+int mnv_select(const float* src, float* dst, const int* indices_host, int num_indices, int rows,
+               int cols, void* workspace, size_t workspace_bytes, mnv_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

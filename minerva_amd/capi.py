@@ -79,6 +79,9 @@ for _m in ("instance", "channel"):
 for _k in ("max", "avg"):
     PROTOTYPES["mnv_%spool_fwd" % _k] = [_P, _P] + [_I] * 10 + [_S]
     PROTOTYPES["mnv_%spool_bwd" % _k] = [_P, _P, _P, _P] + [_I] * 10 + [_S]
+PROTOTYPES["mnv_copy_2d"] = [_P, _P, c_sz, c_sz, c_sz, c_sz, _S]
+PROTOTYPES["mnv_select_workspace_bytes"] = [_I]
+PROTOTYPES["mnv_select"] = [_P, _P, _P, _I, _I, _I, _P, c_sz, _S]
 PROTOTYPES["mnv_lrn_fwd"] = [_P, _P, _P, _I, c_f, c_f, _I, _I, _I, _I, _S]
 PROTOTYPES["mnv_lrn_bwd"] = [_P, _P, _P, _P, _P, _I, c_f, c_f, _I, _I, _I, _I, _S]
 
@@ -89,6 +92,7 @@ _RESTYPES = {
     "mnv_conv_fwd_workspace_bytes": c_sz,
     "mnv_conv_bwd_data_workspace_bytes": c_sz,
     "mnv_conv_bwd_bias_workspace_bytes": c_sz,
+    "mnv_select_workspace_bytes": c_sz,
 }
 
 

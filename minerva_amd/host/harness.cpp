@@ -192,6 +192,16 @@ int mnvh_op(void* runtime, const char* op_name, const mnvh_tensor* inputs, int n
     } else if (op == "pooling_backward") {
       need(3);
       r = rt->PoolingBackward(in[0], in[1], in[2], pool_info());
+    } else if (op == "concat") {  // params: catdim; any number (> 1) of inputs
+      r = rt->Concat(in, P(params, n_params, 0));
+    } else if (op == "slice") {  // params: slice_dim, st_off, slice_count
+      need(1);
+      r = rt->Slice(in[0], P(params, n_params, 0), P(params, n_params, 1), P(params, n_params, 2));
+    } else if (op == "select") {  // params: the column indices
+      need(1);
+      std::vector<int> idx;
+      for (int i = 0; i < n_params; ++i) idx.push_back(static_cast<int>(params[i]));
+      r = rt->Select(in[0], idx);
     } else if (op == "lrn_forward") {  // params: local_size, alpha, beta; inputs: bottom, scale
       need(2);
       MNV_CHECK(n_params >= 3) << "lrn_forward takes local_size, alpha, beta";

@@ -384,6 +384,74 @@ void LRNBackward(const DataList& inputs, const DataList& outputs, LRNBackwardClo
      "LRN backward");
 }
 
+namespace {
+// product of the dimensions below / above d
+size_t Inner(const Scale& s, size_t d) {
+  size_t p = 1;
+  for (size_t i = 0; i < d; ++i) p *= static_cast<size_t>(s[i]);
+  return p;
+}
+size_t Outer(const Scale& s, size_t d) {
+  size_t p = 1;
+  for (size_t i = d + 1; i < s.NumDims(); ++i) p *= static_cast<size_t>(s[i]);
+  return p;
+}
+}  // namespace
+
+// Any dimension is accepted (the reference CHECKs for the last three and then treats every
+// dimension but the last as the second to last, cuda.cpp:83,97-118).
+void Concat(const DataList& inputs, const DataList& outputs, ConcatClosure& c, const Context& ctx) {
+  MNV_CHECK_GT(inputs.size(), 1u) << "(Concat) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(Concat) #outputs is wrong!";
+  const Scale& os = outputs[0].size_;
+  MNV_CHECK(c.catdim >= 0 && static_cast<size_t>(c.catdim) < os.NumDims()) << "(Concat) bad dimension";
+  const size_t d = static_cast<size_t>(c.catdim);
+  const size_t inner = Inner(os, d), outer = Outer(os, d);
+  size_t offset = 0;
+  for (auto& in : inputs) {
+    MNV_CHECK_EQ(in.size_.NumDims(), os.NumDims()) << "(Concat) rank mismatch";
+    for (size_t i = 0; i < os.NumDims(); ++i)
+      if (i != d) MNV_CHECK_EQ(in.size_[i], os[i]) << "(Concat) extent mismatch in dimension " << i;
+    const size_t e = static_cast<size_t>(in.size_[d]);
+    MNV_CHECK_LE(offset + e, static_cast<size_t>(os[d])) << "(Concat) inputs exceed the output";
+    Ok(mnv_copy_2d(in.data_, outputs[0].data_ + offset * inner, e * inner, outer, e * inner,
+                   static_cast<size_t>(os[d]) * inner, ctx.stream), "concat");
+    offset += e;
+  }
+  MNV_CHECK_EQ(offset, static_cast<size_t>(os[d])) << "(Concat) inputs do not fill the output";
+}
+
+void Slice(const DataList& inputs, const DataList& outputs, SliceClosure& c, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "(Slice) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(Slice) #outputs is wrong!";
+  const Scale& is = inputs[0].size_;
+  MNV_CHECK(c.slice_dim >= 0 && static_cast<size_t>(c.slice_dim) < is.NumDims()) << "(Slice) bad dimension";
+  const size_t d = static_cast<size_t>(c.slice_dim);
+  MNV_CHECK(c.st_off >= 0 && c.slice_count > 0 && c.st_off + c.slice_count <= is[d])
+      << "(Slice) range outside the tensor";
+  MNV_CHECK_EQ(outputs[0].size_[d], c.slice_count) << "(Slice) output extent";
+  const size_t inner = Inner(is, d), outer = Outer(is, d);
+  Ok(mnv_copy_2d(inputs[0].data_ + static_cast<size_t>(c.st_off) * inner, outputs[0].data_,
+                 static_cast<size_t>(c.slice_count) * inner, outer,
+                 static_cast<size_t>(is[d]) * inner, static_cast<size_t>(c.slice_count) * inner,
+                 ctx.stream), "slice");
+}
+
+void Select(const DataList& inputs, const DataList& outputs, SelectClosure& c, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u);
+  MNV_CHECK_EQ(outputs.size(), 1u);
+  MNV_CHECK_EQ(inputs[0].size_.NumDims(), 2u);
+  MNV_CHECK_EQ(outputs[0].size_.NumDims(), 2u);
+  MNV_CHECK_EQ(inputs[0].size_[0], outputs[0].size_[0]);
+  MNV_CHECK_EQ(static_cast<size_t>(outputs[0].size_[1]), c.indices.size());
+  for (auto i : c.indices) MNV_CHECK(i >= 0 && i < inputs[0].size_[1]) << "(Select) index " << i;
+  Ok(mnv_select(inputs[0].data_, outputs[0].data_, c.indices.data(),
+                static_cast<int>(c.indices.size()), inputs[0].size_[0], inputs[0].size_[1],
+                ctx.workspace, ctx.workspace_bytes, ctx.stream), "select");
+  // the index vector belongs to the closure: it must outlive the staging copy
+  Ok(mnv_stream_sync(ctx.stream), "select sync");
+}
+
 void ArrayLoader(const DataList& outputs, ArrayLoaderClosure& closure, const Context& ctx) {
   MNV_CHECK_EQ(outputs.size(), 1u) << "(array loader) #outputs wrong";
   MNV_CHECK(closure.data) << "probably already executed";

@@ -39,6 +39,9 @@ struct Thrower {
   } else                \
     ::minerva::detail::Thrower(__FILE__, __LINE__, #cond).os
 #define MNV_CHECK_EQ(a, b) MNV_CHECK((a) == (b)) << "(" << (a) << " vs " << (b) << ") "
+#define MNV_CHECK_GT(a, b) MNV_CHECK((a) > (b)) << "(" << (a) << " vs " << (b) << ") "
+#define MNV_CHECK_LT(a, b) MNV_CHECK((a) < (b)) << "(" << (a) << " vs " << (b) << ") "
+#define MNV_CHECK_LE(a, b) MNV_CHECK((a) <= (b)) << "(" << (a) << " vs " << (b) << ") "
 #define MNV_FATAL() ::minerva::detail::Thrower(__FILE__, __LINE__, "fatal").os
 
 // ---- Scale: an N-d extent or index; dimension 0 is the fastest in memory.
@@ -195,5 +198,10 @@ template <int i> struct LRNClosure {
 };
 typedef LRNClosure<0> LRNForwardClosure;
 typedef LRNClosure<1> LRNBackwardClosure;
+
+// reference minerva/op/closure.h:160-176
+struct ConcatClosure { int catdim; };
+struct SliceClosure { int slice_dim, st_off, slice_count; };
+struct SelectClosure { std::vector<int> indices; };
 
 }  // namespace minerva

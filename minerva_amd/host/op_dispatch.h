@@ -67,6 +67,9 @@ MNV_INSTALL_COMPUTE_FN(PoolingForwardClosure, hip::PoolingForward)
 MNV_INSTALL_COMPUTE_FN(PoolingBackwardClosure, hip::PoolingBackward)
 MNV_INSTALL_COMPUTE_FN(LRNForwardClosure, hip::LRNForward)
 MNV_INSTALL_COMPUTE_FN(LRNBackwardClosure, hip::LRNBackward)
+MNV_INSTALL_COMPUTE_FN(ConcatClosure, hip::Concat)
+MNV_INSTALL_COMPUTE_FN(SliceClosure, hip::Slice)
+MNV_INSTALL_COMPUTE_FN(SelectClosure, hip::Select)
 MNV_INSTALL_DATAGEN_FN(ArrayLoaderClosure, hip::ArrayLoader)
 MNV_INSTALL_DATAGEN_FN(FillClosure, hip::Fill)
 
@@ -116,6 +119,9 @@ MNV_SIMPLE_OP(TanhBackwardOp, ComputeFnWithClosure, TanhBackwardClosure, "tanh b
 MNV_SIMPLE_OP(ConvBackwardBiasOp, ComputeFnWithClosure, ConvBackwardBiasClosure, "conv bp bias")
 MNV_SIMPLE_OP(LRNForwardOp, ComputeFnWithClosure, LRNForwardClosure, "LRN Forward")
 MNV_SIMPLE_OP(LRNBackwardOp, ComputeFnWithClosure, LRNBackwardClosure, "LRN Backward")
+MNV_SIMPLE_OP(ConcatOp, ComputeFnWithClosure, ConcatClosure, "Concat")
+MNV_SIMPLE_OP(SliceOp, ComputeFnWithClosure, SliceClosure, "Slice")
+MNV_SIMPLE_OP(SelectOp, ComputeFnWithClosure, SelectClosure, "select")
 
 class FillOp : public PhyDataGenFnWithClosure<FillClosure> {
  public:

@@ -239,6 +239,45 @@ Tensor Runner::PoolingBackward(const Tensor& diff, const Tensor& top, const Tens
   return Compute({diff, top, bottom}, bottom->size, op);
 }
 
+Tensor Runner::Concat(const std::vector<Tensor>& arrays, int catdim) {
+  MNV_CHECK_GT(arrays.size(), 1u) << "Concat more than one narray";
+  MNV_CHECK(catdim >= 0 && arrays[0]->size.NumDims() > static_cast<size_t>(catdim))
+      << "can't concat on non-sense dim";
+  std::vector<int> dims(arrays[0]->size.NumDims());
+  int target = 0;
+  for (auto& a : arrays) {
+    MNV_CHECK_EQ(a->size.NumDims(), dims.size()) << "rank mismatch";
+    target += a->size[catdim];
+  }
+  for (size_t i = 0; i < dims.size(); ++i)
+    dims[i] = i == static_cast<size_t>(catdim) ? target : arrays[0]->size[i];
+  auto op = std::make_shared<ConcatOp>();
+  op->closure = {catdim};
+  return Compute(arrays, Scale(dims), op);
+}
+
+Tensor Runner::Slice(const Tensor& src, int slice_dim, int st_off, int slice_count) {
+  MNV_CHECK(slice_dim >= 0 && src->size.NumDims() > static_cast<size_t>(slice_dim))
+      << "can't slice on non-sense dim";
+  std::vector<int> dims(src->size.NumDims());
+  for (size_t i = 0; i < dims.size(); ++i)
+    dims[i] = i == static_cast<size_t>(slice_dim) ? slice_count : src->size[i];
+  auto op = std::make_shared<SliceOp>();
+  op->closure = {slice_dim, st_off, slice_count};
+  return Compute({src}, Scale(dims), op);
+}
+
+// The reference's NArray::Select never hands its indices to the operator (narray.cpp:190
+// leaves the closure empty); here they are.
+Tensor Runner::Select(const Tensor& src, const std::vector<int>& indices) {
+  MNV_CHECK_EQ(src->size.NumDims(), 2u);
+  MNV_CHECK_LT(0u, indices.size());
+  for (auto i : indices) MNV_CHECK(i >= 0 && i < src->size[1]) << "index " << i << " out of range";
+  auto op = std::make_shared<SelectOp>();
+  op->closure = {indices};
+  return Compute({src}, Scale{src->size[0], static_cast<int>(indices.size())}, op);
+}
+
 Tensor Runner::LRNForward(const Tensor& src, const Tensor& scale, int local_size, float alpha,
                           float beta) {
   MNV_CHECK_EQ(src->size.NumDims(), 4u);

@@ -84,6 +84,10 @@ class Runner : public DeviceListener {
   Tensor PoolingForward(const Tensor& src, PoolingInfo info);
   Tensor PoolingBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom,
                          PoolingInfo info);
+  // reference minerva/narray/narray.cpp:129-160, 183-192
+  Tensor Concat(const std::vector<Tensor>& arrays, int catdim);
+  Tensor Slice(const Tensor& src, int slice_dim, int st_off, int slice_count);
+  Tensor Select(const Tensor& src, const std::vector<int>& indices);
   // reference minerva/narray/convolution.cpp:165-175; `scale` is filled by the forward pass
   Tensor LRNForward(const Tensor& src, const Tensor& scale, int local_size, float alpha,
                     float beta);

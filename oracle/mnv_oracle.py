@@ -263,3 +263,22 @@ def lrn_bwd(bottom, top, scale, top_diff, local_size, alpha, beta, N, C, H, W):
     _chk(lib().ora_lrn_bwd(_p(bottom), _p(top), _p(scale), _p(top_diff), _p(out), local_size,
                            ctypes.c_float(alpha), ctypes.c_float(beta), N, C, H, W), "lrn_bwd")
     return out
+
+
+# Concat / Slice / Select are pure data movement on column-major tensors (reference
+# minerva/op/impl/cuda.cpp:80-155, 644-655; extents minerva/narray/narray.cpp:129-192):
+# numpy's own indexing on Fortran-ordered views is the closed form.
+def concat(arrays, dims_list, catdim):
+    views = [_f(a).reshape(d, order="F") for a, d in zip(arrays, dims_list)]
+    return np.concatenate(views, axis=catdim).ravel(order="F")
+
+
+def slice_(x, dims, slice_dim, st_off, slice_count):
+    v = _f(x).reshape(dims, order="F")
+    idx = [slice(None)] * len(dims)
+    idx[slice_dim] = slice(st_off, st_off + slice_count)
+    return v[tuple(idx)].ravel(order="F")
+
+
+def select(x, rows, cols, indices):
+    return _f(x).reshape((rows, cols), order="F")[:, list(indices)].ravel(order="F")

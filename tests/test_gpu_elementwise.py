@@ -174,3 +174,40 @@ def test_invalid_arguments_are_rejected(gpu):
     assert L.mnv_sgemm_nn(d.p, d.p, d.p, 4, 4, 0, None, 0, gpu.dev.stream) == -1
     assert L.mnv_conv_fwd(d.p, d.p, d.p, d.p, 1, 1, 1, 2, 2, 0, 0, 1, 1, 3, 3, None, 0, gpu.dev.stream) == -1
     assert L.mnv_maxpool_fwd(d.p, d.p, 1, 1, 4, 4, 0, 1, 2, 2, 0, 0, gpu.dev.stream) == -1
+
+
+# ------------------------------------------------- Concat / Slice / Select movement
+@pytest.mark.parametrize("row_elems,rows,sp,dp,shift", [
+    (64, 5, 64, 200, 0),        # 16-byte path
+    (64, 5, 128, 64, 0),
+    (63, 7, 70, 91, 0),         # scalar path: odd run length
+    (64, 3, 64, 64, 1),         # scalar path: unaligned pointers
+    (1, 1000, 3, 2, 0),         # many one-float rows
+    (70000, 3, 70000, 140000, 0),
+])
+def test_copy_2d(gpu, row_elems, rows, sp, dp, shift):
+    src = _rand(rows * sp + shift, 90)
+    dst0 = _rand(rows * dp + shift, 91)
+    dsrc, ddst = gpu.up(src), gpu.up(dst0)
+    gpu.call("mnv_copy_2d", ctypes.c_void_p(dsrc.ptr + 4 * shift), ctypes.c_void_p(ddst.ptr + 4 * shift),
+             ctypes.c_size_t(row_elems), ctypes.c_size_t(rows), ctypes.c_size_t(sp), ctypes.c_size_t(dp))
+    want = dst0.copy()
+    for r in range(rows):
+        want[shift + r * dp: shift + r * dp + row_elems] = src[shift + r * sp: shift + r * sp + row_elems]
+    assert_bits_equal(gpu.down(ddst), want, "copy_2d (elements between rows untouched)")
+
+
+def test_select_columns(gpu, ora):
+    rows, cols = 37, 11
+    x = _rand(rows * cols, 92)
+    idx = [3, 0, 10, 3, 7]
+    dx, dd = gpu.up(x), gpu.up(np.full(rows * len(idx), np.nan, np.float32))
+    arr = (ctypes.c_int * len(idx))(*idx)
+    nbytes = gpu.L.mnv_select_workspace_bytes(len(idx))
+    ws = gpu.empty(nbytes // 4 + 1)
+    gpu.call("mnv_select", dx.p, dd.p, arr, len(idx), rows, cols, ws.p, ctypes.c_size_t(nbytes))
+    assert_bits_equal(gpu.down(dd), ora.select(x, rows, cols, idx), "select")
+    # out-of-range index and missing workspace are refused
+    bad = (ctypes.c_int * 1)(cols)
+    assert gpu.L.mnv_select(dx.p, dd.p, bad, 1, rows, cols, ws.p, ctypes.c_size_t(nbytes), gpu.dev.stream) == -1
+    assert gpu.L.mnv_select(dx.p, dd.p, arr, len(idx), rows, cols, None, ctypes.c_size_t(0), gpu.dev.stream) == -2

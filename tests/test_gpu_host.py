@@ -168,6 +168,41 @@ def test_lrn_forward_and_backward(rt, ora):
     assert normwise(back, ora.lrn_bwd(x, top, scale, dy, 5, 1e-2, 0.75, N, C, H, W)) <= TOL
 
 
+def test_concat_slice_select(rt, ora):
+    # channel concat of image batches {W,H,C,N}, the reference's main use (cuda.cpp:97-118)
+    a, b, c = _rand(5 * 4 * 3 * 2, 80), _rand(5 * 4 * 6 * 2, 81), _rand(5 * 4 * 1 * 2, 82)
+    da, db, dc = [5, 4, 3, 2], [5, 4, 6, 2], [5, 4, 1, 2]
+    got, od = rt.op("concat", [(a, da), (b, db), (c, dc)], [2])
+    assert od == [5, 4, 10, 2]
+    assert_bits_equal(got, ora.concat([a, b, c], [da, db, dc], 2), "concat channels")
+    # along the last dimension (plain append) and along dimension 0 (not in the reference)
+    got, od = rt.op("concat", [(a, da), (a, da)], [3])
+    assert od == [5, 4, 3, 4]
+    assert_bits_equal(got, ora.concat([a, a], [da, da], 3), "concat images")
+    m1, m2 = _rand(6, 83), _rand(9, 84)
+    got, od = rt.op("concat", [(m1, [2, 3]), (m2, [3, 3])], [0])
+    assert od == [5, 3]
+    assert_bits_equal(got, ora.concat([m1, m2], [[2, 3], [3, 3]], 0), "concat rows")
+    # slices undo the concat
+    cat = ora.concat([a, b, c], [da, db, dc], 2)
+    got, od = rt.op("slice", [(cat, [5, 4, 10, 2])], [2, 3, 6])
+    assert od == db
+    assert_bits_equal(got, b, "slice channels")
+    got, od = rt.op("slice", [(cat, [5, 4, 10, 2])], [3, 1, 1])
+    assert od == [5, 4, 10, 1]
+    assert_bits_equal(got, ora.slice_(cat, [5, 4, 10, 2], 3, 1, 1), "slice images")
+    got, od = rt.op("select", [(m2, [3, 3])], [2, 0, 2])
+    assert od == [3, 3]
+    assert_bits_equal(got, ora.select(m2, 3, 3, [2, 0, 2]), "select")
+    from minerva_amd import hostapi
+    with pytest.raises(hostapi.HostError, match="extent mismatch"):
+        rt.op("concat", [(a, da), (_rand(4 * 4 * 3 * 2, 85), [4, 4, 3, 2])], [2])
+    with pytest.raises(hostapi.HostError, match="range outside"):
+        rt.op("slice", [(a, da)], [2, 2, 2])
+    with pytest.raises(hostapi.HostError, match="out of range"):
+        rt.op("select", [(m2, [3, 3])], [3])
+
+
 def test_error_convention(rt):
     from minerva_amd import hostapi
     a = _rand(6, 76)
