@@ -282,6 +282,17 @@ size_t mnv_select_workspace_bytes(int num_indices);
 int mnv_select(const float* src, float* dst, const int* indices_host, int num_indices, int rows,
                int cols, void* workspace, size_t workspace_bytes, mnv_stream_t stream);
 
+/* ---- random tensors: CudaPerformRandn / CudaPerformRandBernoulli (cuda_perform.h:66-67).
+ * The reference seeds cuRAND from the wall clock per call (cuda.cpp:601,606); here the seed
+ * is an argument and the generator is counter based (Philox4x32-10): element block i/4
+ * uses counter (lo32, hi32, 0, 0) and key = seed, so equal seeds give equal tensors.
+ * mnv_randn: mean + stddev * N(0,1) by Box-Muller (the reference passes its `var` closure
+ * field as cuRAND's stddev argument).  mnv_rand_bernoulli: 1.0f with probability p, else 0. ---- */
+int mnv_randn(float* dst, size_t n, unsigned long long seed, float mean, float stddev,
+              mnv_stream_t stream);
+int mnv_rand_bernoulli(float* dst, size_t n, unsigned long long seed, float p,
+                       mnv_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -77,6 +77,9 @@ int mnvh_op(void* runtime, const char* op, const mnvh_tensor* inputs, int n_inpu
             const double* params, int n_params, float* out, size_t out_capacity,
             int* out_ndims, int* out_dims);
 
+/* Restarts the sequence the seeds of the "randn" / "rand_bernoulli" operators are drawn from. */
+int mnvh_set_random_seed(unsigned long long seed);
+
 /* Runs `count` independent element-wise additions through the device's thread pool
  * (four workers, four streams) and returns the results; exercises PushTask with
  * non-light tasks and the completion listener. */

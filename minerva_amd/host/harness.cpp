@@ -212,6 +212,14 @@ int mnvh_op(void* runtime, const char* op_name, const mnvh_tensor* inputs, int n
       MNV_CHECK(n_params >= 3) << "lrn_backward takes local_size, alpha, beta";
       r = rt->LRNBackward(in[0], in[1], in[2], in[3], static_cast<int>(params[0]),
                           static_cast<float>(params[1]), static_cast<float>(params[2]));
+    } else if (op == "randn" || op == "rand_bernoulli") {  // params: mu, var | p ; then d0, d1, ...
+      need(0);
+      const int lead = op == "randn" ? 2 : 1;
+      MNV_CHECK(n_params > lead) << op << " takes its parameters, then the extents";
+      std::vector<int> d;
+      for (int i = lead; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
+      r = op == "randn" ? rt->Randn(Scale(d), static_cast<float>(params[0]), static_cast<float>(params[1]))
+                        : rt->RandBernoulli(Scale(d), static_cast<float>(params[0]));
     } else if (op == "fill") {
       need(0);
       std::vector<int> d;
@@ -229,6 +237,11 @@ int mnvh_op(void* runtime, const char* op_name, const mnvh_tensor* inputs, int n
     if (out_dims)
       for (size_t i = 0; i < r->size.NumDims(); ++i) out_dims[i] = r->size[i];
   });
+}
+
+int mnvh_set_random_seed(unsigned long long seed) {
+  minerva::hip::SetRandomSeed(seed);
+  return 0;
 }
 
 int mnvh_concurrent_adds(void* runtime, const float* a, const float* b, size_t n, int count,

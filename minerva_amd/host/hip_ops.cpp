@@ -1,5 +1,7 @@
 #include "hip_ops.h"
 
+#include <atomic>
+
 #include "mnv_hip.h"
 
 namespace minerva {
@@ -461,6 +463,33 @@ void ArrayLoader(const DataList& outputs, ArrayLoaderClosure& closure, const Con
   // the host buffer must outlive the asynchronous copy
   Ok(mnv_stream_sync(ctx.stream), "array loader sync");
   closure.data.reset();
+}
+
+namespace {
+std::atomic<uint64_t> g_seed_base{0x243F6A8885A308D3ull}, g_seed_count{0};
+uint64_t NextSeed() {  // splitmix64 of (base + call number)
+  uint64_t z = g_seed_base.load() + 0x9E3779B97F4A7C15ull * (g_seed_count.fetch_add(1) + 1);
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+}  // namespace
+
+void SetRandomSeed(uint64_t seed) {
+  g_seed_base.store(seed);
+  g_seed_count.store(0);
+}
+
+void Randn(const DataList& outputs, RandnClosure& closure, const Context& ctx) {
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(normal) #outputs wrong";
+  Ok(mnv_randn(outputs[0].data_, outputs[0].size_.Prod(), NextSeed(), closure.mu, closure.var,
+               ctx.stream), "randn");
+}
+
+void RandBernoulli(const DataList& outputs, RandBernoulliClosure& closure, const Context& ctx) {
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(bernoulli) #outputs wrong";
+  Ok(mnv_rand_bernoulli(outputs[0].data_, outputs[0].size_.Prod(), NextSeed(), closure.p,
+                        ctx.stream), "rand bernoulli");
 }
 
 void Fill(const DataList& outputs, FillClosure& closure, const Context& ctx) {

@@ -4,6 +4,7 @@
 // the closure (as minerva/op/impl/cuda.cpp does) and calls one launcher of the C ABI
 // in include/mnv_hip.h; a non-zero status from the library fails a check.
 #pragma once
+#include <cstdint>
 #include "minerva_types.h"
 
 namespace minerva {
@@ -42,6 +43,11 @@ void Select(const DataList&, const DataList&, SelectClosure&, const Context&);
 
 void ArrayLoader(const DataList&, ArrayLoaderClosure&, const Context&);
 void Fill(const DataList&, FillClosure&, const Context&);
+void Randn(const DataList&, RandnClosure&, const Context&);
+void RandBernoulli(const DataList&, RandBernoulliClosure&, const Context&);
+// Seeds of successive Randn / RandBernoulli calls are drawn from one process-wide sequence;
+// this restarts it (the reference seeds from the clock and cannot be replayed).
+void SetRandomSeed(uint64_t seed);
 
 }  // namespace hip
 }  // namespace minerva

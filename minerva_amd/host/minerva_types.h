@@ -147,6 +147,10 @@ struct PoolingInfo {
 
 struct ArrayLoaderClosure { std::shared_ptr<float> data; };
 struct FillClosure { float val; };
+// reference minerva/op/closure.h:30-36; `var` is handed to the generator as the standard
+// deviation, as the reference does (cuda_perform.cu:621, basic.cpp:275)
+struct RandnClosure { float mu, var; };
+struct RandBernoulliClosure { float p; };
 struct MatMultClosure {};
 struct TransposeClosure {};
 struct ReshapeClosure {};

@@ -72,6 +72,8 @@ MNV_INSTALL_COMPUTE_FN(SliceClosure, hip::Slice)
 MNV_INSTALL_COMPUTE_FN(SelectClosure, hip::Select)
 MNV_INSTALL_DATAGEN_FN(ArrayLoaderClosure, hip::ArrayLoader)
 MNV_INSTALL_DATAGEN_FN(FillClosure, hip::Fill)
+MNV_INSTALL_DATAGEN_FN(RandnClosure, hip::Randn)
+MNV_INSTALL_DATAGEN_FN(RandBernoulliClosure, hip::RandBernoulli)
 
 template <typename C> class ComputeFnWithClosure : public ComputeFn {
  public:
@@ -106,6 +108,8 @@ inline const char* ArithSym(ArithmeticType t) {
   };
 
 MNV_SIMPLE_OP(ArrayLoaderOp, PhyDataGenFnWithClosure, ArrayLoaderClosure, ":array loader")
+MNV_SIMPLE_OP(RandnOp, PhyDataGenFnWithClosure, RandnClosure, ":normal")
+MNV_SIMPLE_OP(RandBernoulliOp, PhyDataGenFnWithClosure, RandBernoulliClosure, ":bernoulli")
 MNV_SIMPLE_OP(MatMultOp, ComputeFnWithClosure, MatMultClosure, "*")
 MNV_SIMPLE_OP(TransOp, ComputeFnWithClosure, TransposeClosure, "trans")
 MNV_SIMPLE_OP(MaxIndexOp, ComputeFnWithClosure, MaxIndexClosure, "max index")

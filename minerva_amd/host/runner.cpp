@@ -60,6 +60,19 @@ Tensor Runner::Constant(const Scale& size, float v) {
   return Compute({}, size, op);
 }
 
+Tensor Runner::Randn(const Scale& size, float mu, float var) {
+  auto op = std::make_shared<RandnOp>();
+  op->closure = {mu, var};
+  return Compute({}, size, op);
+}
+
+Tensor Runner::RandBernoulli(const Scale& size, float p) {
+  MNV_CHECK(p >= 0.f && p <= 1.f) << "probability out of range: " << p;
+  auto op = std::make_shared<RandBernoulliOp>();
+  op->closure = {p};
+  return Compute({}, size, op);
+}
+
 Tensor Runner::Arithmetic(const Tensor& a, const Tensor& b, ArithmeticType t) {
   MNV_CHECK(a->size == b->size) << "size must match " << a->size << " " << b->size;
   auto op = std::make_shared<ArithmeticOp>();

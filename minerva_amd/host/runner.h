@@ -45,6 +45,9 @@ class Runner : public DeviceListener {
   Tensor MakeNArray(const Scale& size, const float* host);  // copies the host data first
   Tensor Constant(const Scale& size, float v);
   Tensor Zeros(const Scale& size) { return Constant(size, 0.f); }
+  // reference minerva/narray/narray.cpp:21-33
+  Tensor Randn(const Scale& size, float mu, float var);
+  Tensor RandBernoulli(const Scale& size, float p);
 
   // NArray arithmetic
   Tensor Arithmetic(const Tensor& a, const Tensor& b, ArithmeticType t);

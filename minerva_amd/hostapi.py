@@ -106,6 +106,10 @@ class Runtime:
         dims = [od[i] for i in range(nd.value)]
         return out[:int(np.prod(dims))].copy(), dims
 
+    @staticmethod
+    def set_random_seed(seed):
+        _check(lib().mnvh_set_random_seed(ctypes.c_uint64(seed)), "set_random_seed")
+
     def concurrent_adds(self, a, b, count):
         a = np.ascontiguousarray(a, np.float32)
         b = np.ascontiguousarray(b, np.float32)

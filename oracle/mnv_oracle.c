@@ -645,3 +645,67 @@ int ora_lrn_bwd(const float* bottom, const float* top, const float* scale, const
     }
   return 0;
 }
+
+/* ------------------------------------------------------------------------- */
+/* Random generators.  The reference draws from a clock-seeded engine          */
+/* (basic.cpp:270-290, cuda.cpp:599-607), so there is nothing of its output to  */
+/* reproduce; what is restated here is the published counter-based generator    */
+/* the library uses instead, Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel*/
+/* random numbers: as easy as 1, 2, 3", SC'11; constants and round function as   */
+/* in the paper and the Random123 distribution), and the element mapping:        */
+/*   block b = i / 4: counter (lo32 b, hi32 b, 0, 0), key (lo32 seed, hi32 seed) */
+/*   normal:    Box-Muller on (x0,x1) and (x2,x3), u1 = ((x>>8)+1)*2^-24,        */
+/*              u2 = (x>>8)*2^-24, out = mean + stddev * z                       */
+/*   bernoulli: out = ((x>>8)*2^-24 < p)                                         */
+/* pinned by: the Random123 known-answer vectors for philox4x32_10 (tests), and  */
+/* the moments / distribution of the outputs.                                    */
+/* ------------------------------------------------------------------------- */
+void ora_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+  uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+  for (int round = 0; round < 10; ++round) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+static void ora_box_muller(uint32_t a, uint32_t b, float* z0, float* z1) {
+  const float u1 = (float)((a >> 8) + 1u) * 5.9604644775390625e-8f;
+  const float u2 = (float)(b >> 8) * 5.9604644775390625e-8f;
+  const float r = sqrtf(-2.0f * logf(u1));
+  const float t = 6.283185307179586f * u2;
+  *z0 = r * cosf(t);
+  *z1 = r * sinf(t);
+}
+
+int ora_randn(float* dst, size_t n, uint64_t seed, float mean, float stddev) {
+  const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  for (size_t b = 0; 4 * b < n; ++b) {
+    const uint32_t ctr[4] = {(uint32_t)b, (uint32_t)((uint64_t)b >> 32), 0u, 0u};
+    uint32_t x[4];
+    float v[4];
+    ora_philox4x32_10(ctr, key, x);
+    ora_box_muller(x[0], x[1], &v[0], &v[1]);
+    ora_box_muller(x[2], x[3], &v[2], &v[3]);
+    for (int t = 0; t < 4; ++t)
+      if (4 * b + t < n) dst[4 * b + t] = mean + stddev * v[t];
+  }
+  return 0;
+}
+
+int ora_rand_bernoulli(float* dst, size_t n, uint64_t seed, float p) {
+  const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  for (size_t b = 0; 4 * b < n; ++b) {
+    const uint32_t ctr[4] = {(uint32_t)b, (uint32_t)((uint64_t)b >> 32), 0u, 0u};
+    uint32_t x[4];
+    ora_philox4x32_10(ctr, key, x);
+    for (int t = 0; t < 4; ++t)
+      if (4 * b + t < n)
+        dst[4 * b + t] = ((float)(x[t] >> 8) * 5.9604644775390625e-8f < p) ? 1.f : 0.f;
+  }
+  return 0;
+}

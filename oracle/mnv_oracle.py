@@ -282,3 +282,25 @@ def slice_(x, dims, slice_dim, st_off, slice_count):
 
 def select(x, rows, cols, indices):
     return _f(x).reshape((rows, cols), order="F")[:, list(indices)].ravel(order="F")
+
+
+def philox4x32_10(ctr, key):
+    c = (ctypes.c_uint32 * 4)(*ctr)
+    k = (ctypes.c_uint32 * 2)(*key)
+    out = (ctypes.c_uint32 * 4)()
+    lib().ora_philox4x32_10(c, k, out)
+    return [int(v) for v in out]
+
+
+def randn(n, seed, mean, stddev):
+    out = np.empty(n, dtype=np.float32)
+    _chk(lib().ora_randn(_p(out), ctypes.c_size_t(n), ctypes.c_uint64(seed), ctypes.c_float(mean),
+                         ctypes.c_float(stddev)), "randn")
+    return out
+
+
+def rand_bernoulli(n, seed, p):
+    out = np.empty(n, dtype=np.float32)
+    _chk(lib().ora_rand_bernoulli(_p(out), ctypes.c_size_t(n), ctypes.c_uint64(seed),
+                                  ctypes.c_float(p)), "rand_bernoulli")
+    return out

@@ -211,3 +211,37 @@ def test_select_columns(gpu, ora):
     bad = (ctypes.c_int * 1)(cols)
     assert gpu.L.mnv_select(dx.p, dd.p, bad, 1, rows, cols, ws.p, ctypes.c_size_t(nbytes), gpu.dev.stream) == -1
     assert gpu.L.mnv_select(dx.p, dd.p, arr, len(idx), rows, cols, None, ctypes.c_size_t(0), gpu.dev.stream) == -2
+
+
+# ----------------------------------------------------------------------- random
+@pytest.mark.parametrize("n", [1, 3, 4, 1001, 1 << 20])
+def test_random_generators_match_oracle(gpu, ora, n):
+    seed = 0x0123456789abcdef
+    d = gpu.up(np.full(n + 1, np.nan, np.float32))
+    gpu.call("mnv_rand_bernoulli", d.p, ctypes.c_size_t(n), ctypes.c_uint64(seed), ctypes.c_float(0.3))
+    out = gpu.down(d)
+    assert_bits_equal(out[:n], ora.rand_bernoulli(n, seed, 0.3), "bernoulli: same bits as the oracle")
+    assert np.isnan(out[n])
+    gpu.call("mnv_randn", d.p, ctypes.c_size_t(n), ctypes.c_uint64(seed), ctypes.c_float(-1.0),
+             ctypes.c_float(0.5))
+    out = gpu.down(d)
+    # same uniforms, device log / sin / cos instead of libm: absolute agreement of the normals
+    assert np.max(np.abs(out[:n] - ora.randn(n, seed, -1.0, 0.5))) <= 2e-5
+    assert np.isnan(out[n])
+    # an unaligned destination takes the scalar stores
+    gpu.call("mnv_rand_bernoulli", ctypes.c_void_p(d.ptr + 4), ctypes.c_size_t(n), ctypes.c_uint64(seed),
+             ctypes.c_float(0.3))
+    assert_bits_equal(gpu.down(d)[1:n + 1], ora.rand_bernoulli(n, seed, 0.3), "bernoulli, unaligned")
+    assert gpu.L.mnv_rand_bernoulli(d.p, ctypes.c_size_t(n), ctypes.c_uint64(1), ctypes.c_float(1.5),
+                                    gpu.dev.stream) == -1
+
+
+def test_randn_distribution_at_full_size(gpu):
+    n = 8192 * 8192
+    d = gpu.empty(n)
+    gpu.call("mnv_randn", d.p, ctypes.c_size_t(n), ctypes.c_uint64(99), ctypes.c_float(0.0), ctypes.c_float(1.0))
+    z = gpu.down(d)
+    assert np.isfinite(z).all()
+    assert abs(float(z.mean(dtype=np.float64))) < 1e-3 and abs(float(z.std(dtype=np.float64)) - 1.0) < 1e-3
+    # tails: P(|z| > 4) = 6.33e-5
+    assert abs(np.count_nonzero(np.abs(z) > 4) / n - 6.334e-5) < 5e-6

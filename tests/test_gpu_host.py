@@ -203,6 +203,23 @@ def test_concat_slice_select(rt, ora):
         rt.op("select", [(m2, [3, 3])], [3])
 
 
+def test_random_operators(rt, ora):
+    from minerva_amd import hostapi
+    hostapi.Runtime.set_random_seed(5)
+    a, od = rt.op("randn", [], [0.0, 0.01, 64, 33], out_capacity=64 * 33)
+    b, _ = rt.op("randn", [], [0.0, 0.01, 64, 33], out_capacity=64 * 33)
+    assert od == [64, 33]
+    assert abs(a.mean()) < 1e-3 and abs(a.std() - 0.01) < 1e-3      # the "var" field is the deviation
+    assert not np.array_equal(a, b)                                  # successive calls differ
+    hostapi.Runtime.set_random_seed(5)
+    a2, _ = rt.op("randn", [], [0.0, 0.01, 64, 33], out_capacity=64 * 33)
+    assert_bits_equal(a2, a, "same seed sequence, same tensor")
+    m, _ = rt.op("rand_bernoulli", [], [0.25, 100, 100], out_capacity=10000)
+    assert set(np.unique(m)) <= {0.0, 1.0} and abs(m.mean() - 0.25) < 0.02
+    with pytest.raises(hostapi.HostError, match="probability out of range"):
+        rt.op("rand_bernoulli", [], [1.5, 4], out_capacity=4)
+
+
 def test_error_convention(rt):
     from minerva_amd import hostapi
     a = _rand(6, 76)

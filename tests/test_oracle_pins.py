@@ -434,3 +434,40 @@ def test_lrn_backward_finite_difference(ora, size, c):
     # of the forward pass pins it
     want = _fd(fwd, x.astype(np.float64), dy.astype(np.float64), eps=1e-4)
     assert np.max(np.abs(got - want)) < 2e-5 * max(1.0, np.max(np.abs(want)))
+
+
+# ------------------------------------------------------------------------ RNG
+def test_philox_known_answer_vectors(ora):
+    # philox4x32_10 known-answer vectors of the Random123 distribution (kat_vectors)
+    kat = [
+        ((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+        ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+        ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
+         (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1)),
+    ]
+    for ctr, key, want in kat:
+        assert tuple(ora.philox4x32_10(ctr, key)) == want
+
+
+def test_random_tensors_mapping_and_distribution(ora):
+    from scipy import stats
+    n, seed = 400003, 0x1234567890abcdef
+    z = ora.randn(n, seed, 1.5, 2.0)
+    # element 4b+t comes from counter (b, 0, 0, 0) and the two halves of the seed as key
+    x = ora.philox4x32_10((7, 0, 0, 0), (seed & 0xffffffff, seed >> 32))
+    u1 = np.float32((x[0] >> 8) + 1) * np.float32(2.0 ** -24)
+    u2 = np.float32(x[1] >> 8) * np.float32(2.0 ** -24)
+    r = np.sqrt(-2.0 * np.log(np.float64(u1)))
+    assert abs(z[28] - (1.5 + 2.0 * r * np.cos(2 * np.pi * np.float64(u2)))) < 1e-5
+    assert abs(z[29] - (1.5 + 2.0 * r * np.sin(2 * np.pi * np.float64(u2)))) < 1e-5
+    # distribution: mean, deviation, and a Kolmogorov-Smirnov test against N(1.5, 2)
+    assert abs(z.mean() - 1.5) < 0.02 and abs(z.std() - 2.0) < 0.02
+    assert stats.kstest((z[:100000] - 1.5) / 2.0, "norm").pvalue > 1e-3
+    assert np.array_equal(ora.randn(n, seed, 1.5, 2.0), z)          # a function of the seed
+    assert not np.array_equal(ora.randn(n, seed + 1, 1.5, 2.0), z)
+    assert np.array_equal(ora.randn(1001, seed, 1.5, 2.0), z[:1001])  # and not of the length
+    b = ora.rand_bernoulli(n, seed, 0.3)
+    assert set(np.unique(b)) == {0.0, 1.0}
+    assert abs(b.mean() - 0.3) < 0.005
+    assert b[28] == (1.0 if np.float32(x[0] >> 8) * np.float32(2.0 ** -24) < np.float32(0.3) else 0.0)
+    assert ora.rand_bernoulli(1000, 3, 0.0).sum() == 0 and ora.rand_bernoulli(1000, 3, 1.0).sum() == 1000
