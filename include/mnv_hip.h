@@ -89,6 +89,9 @@ int mnv_const_rdiv(const float* x, float* y, float v, size_t n, mnv_stream_t str
 int mnv_exp(const float* x, float* y, size_t n, mnv_stream_t stream);
 int mnv_ln(const float* x, float* y, size_t n, mnv_stream_t stream);
 int mnv_neg(const float* x, float* y, size_t n, mnv_stream_t stream);
+/* ThresholdNorm (CPU-only in the reference, basic.cpp:110-123):
+ * y = |x| > threshold ? |x| / x * threshold : x, i.e. x clipped to [-threshold, threshold]. */
+int mnv_threshold_norm(const float* x, float* y, float threshold, size_t n, mnv_stream_t stream);
 
 /* ---- broadcast arithmetic on an {m,n} matrix: CudaPerformNorm{Add,Sub,Mult,Div}
  * On{Col,Row} (cuda_perform.h:25-33).

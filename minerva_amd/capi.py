@@ -82,6 +82,7 @@ for _k in ("max", "avg"):
 PROTOTYPES["mnv_copy_2d"] = [_P, _P, c_sz, c_sz, c_sz, c_sz, _S]
 PROTOTYPES["mnv_select_workspace_bytes"] = [_I]
 PROTOTYPES["mnv_select"] = [_P, _P, _P, _I, _I, _I, _P, c_sz, _S]
+PROTOTYPES["mnv_threshold_norm"] = [_P, _P, c_f, c_sz, _S]
 PROTOTYPES["mnv_randn"] = [_P, c_sz, ctypes.c_uint64, c_f, c_f, _S]
 PROTOTYPES["mnv_rand_bernoulli"] = [_P, c_sz, ctypes.c_uint64, c_f, _S]
 PROTOTYPES["mnv_lrn_fwd"] = [_P, _P, _P, _I, c_f, c_f, _I, _I, _I, _I, _S]

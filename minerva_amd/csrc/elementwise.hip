@@ -23,6 +23,11 @@ struct OpConstRdiv { float v; __device__ float operator()(float x, float) const 
 struct OpExp { __device__ float operator()(float x, float) const { return expf(x); } };
 struct OpLn  { __device__ float operator()(float x, float) const { return logf(x); } };
 struct OpNeg { __device__ float operator()(float x, float) const { return -x; } };
+// basic.cpp:116-122, the operations as written there (|x| / x is exactly +-1)
+struct OpThresholdNorm {
+  float t;
+  __device__ float operator()(float x, float) const { return fabsf(x) > t ? fabsf(x) / x * t : x; }
+};
 struct OpCopy { __device__ float operator()(float x, float) const { return x; } };
 struct OpFill { float v; __device__ float operator()(float, float) const { return v; } };
 
@@ -95,6 +100,9 @@ int mnv_neg(const float* x, float* y, size_t n, mnv_stream_t s) {
   return mnv_stream_launch<OpNeg, 1>(x, nullptr, y, n, OpNeg(), s);
 }
 
+int mnv_threshold_norm(const float* x, float* y, float threshold, size_t n, mnv_stream_t s) {
+  return mnv_stream_launch<OpThresholdNorm, 1>(x, nullptr, y, n, OpThresholdNorm{threshold}, s);
+}
 int mnv_copy(const float* in, float* out, size_t n, mnv_stream_t s) {
   return mnv_stream_launch<OpCopy, 1>(in, nullptr, out, n, OpCopy(), s);
 }

@@ -192,6 +192,16 @@ int mnvh_op(void* runtime, const char* op_name, const mnvh_tensor* inputs, int n
     } else if (op == "pooling_backward") {
       need(3);
       r = rt->PoolingBackward(in[0], in[1], in[2], pool_info());
+    } else if (op == "threshold_norm") {  // params: threshold
+      need(1);
+      MNV_CHECK(n_params >= 1) << "threshold_norm takes the threshold";
+      r = rt->ThresholdNorm(in[0], static_cast<float>(params[0]));
+    } else if (op == "index") {  // params: idx, then the extents of one block
+      need(1);
+      std::vector<int> d;
+      for (int i = 1; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
+      MNV_CHECK(!d.empty()) << "index takes idx, d0, ...";
+      r = rt->Index(in[0], P(params, n_params, 0), Scale(d));
     } else if (op == "concat") {  // params: catdim; any number (> 1) of inputs
       r = rt->Concat(in, P(params, n_params, 0));
     } else if (op == "slice") {  // params: slice_dim, st_off, slice_count

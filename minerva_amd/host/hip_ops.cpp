@@ -400,6 +400,27 @@ size_t Outer(const Scale& s, size_t d) {
 }
 }  // namespace
 
+// CPU-only in the reference (bundle.h:31, basic.cpp:110-123)
+void ThresholdNorm(const DataList& inputs, const DataList& outputs, ThresholdNormClosure& c,
+                   const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "(elewise) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(elewise) #outputs is wrong!";
+  Ok(mnv_threshold_norm(inputs[0].data_, outputs[0].data_, c.threshold, outputs[0].size_.Prod(),
+                        ctx.stream), "threshold norm");
+}
+
+// CPU-only in the reference (bundle.h:55, basic.cpp:473-488): the idx-th block of
+// output-sized data
+void Index(const DataList& inputs, const DataList& outputs, IndexClosure& c, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 1u) << "(index) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(index) #outputs wrong";
+  const size_t len = outputs[0].size_.Prod();
+  MNV_CHECK(c.idx >= 0 && (static_cast<size_t>(c.idx) + 1) * len <= inputs[0].size_.Prod())
+      << "(index) block " << c.idx << " outside the input";
+  Ok(mnv_copy(inputs[0].data_ + static_cast<size_t>(c.idx) * len, outputs[0].data_, len, ctx.stream),
+     "index");
+}
+
 // Any dimension is accepted (the reference CHECKs for the last three and then treats every
 // dimension but the last as the second to last, cuda.cpp:83,97-118).
 void Concat(const DataList& inputs, const DataList& outputs, ConcatClosure& c, const Context& ctx) {

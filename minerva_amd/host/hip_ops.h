@@ -37,6 +37,8 @@ void PoolingForward(const DataList&, const DataList&, PoolingForwardClosure&, co
 void PoolingBackward(const DataList&, const DataList&, PoolingBackwardClosure&, const Context&);
 void LRNForward(const DataList&, const DataList&, LRNForwardClosure&, const Context&);
 void LRNBackward(const DataList&, const DataList&, LRNBackwardClosure&, const Context&);
+void ThresholdNorm(const DataList&, const DataList&, ThresholdNormClosure&, const Context&);
+void Index(const DataList&, const DataList&, IndexClosure&, const Context&);
 void Concat(const DataList&, const DataList&, ConcatClosure&, const Context&);
 void Slice(const DataList&, const DataList&, SliceClosure&, const Context&);
 void Select(const DataList&, const DataList&, SelectClosure&, const Context&);

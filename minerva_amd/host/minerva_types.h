@@ -203,7 +203,9 @@ template <int i> struct LRNClosure {
 typedef LRNClosure<0> LRNForwardClosure;
 typedef LRNClosure<1> LRNBackwardClosure;
 
-// reference minerva/op/closure.h:160-176
+// reference minerva/op/closure.h:74-76, 160-176
+struct ThresholdNormClosure { float threshold; };
+struct IndexClosure { int idx; };
 struct ConcatClosure { int catdim; };
 struct SliceClosure { int slice_dim, st_off, slice_count; };
 struct SelectClosure { std::vector<int> indices; };

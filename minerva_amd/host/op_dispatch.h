@@ -67,6 +67,8 @@ MNV_INSTALL_COMPUTE_FN(PoolingForwardClosure, hip::PoolingForward)
 MNV_INSTALL_COMPUTE_FN(PoolingBackwardClosure, hip::PoolingBackward)
 MNV_INSTALL_COMPUTE_FN(LRNForwardClosure, hip::LRNForward)
 MNV_INSTALL_COMPUTE_FN(LRNBackwardClosure, hip::LRNBackward)
+MNV_INSTALL_COMPUTE_FN(ThresholdNormClosure, hip::ThresholdNorm)
+MNV_INSTALL_COMPUTE_FN(IndexClosure, hip::Index)
 MNV_INSTALL_COMPUTE_FN(ConcatClosure, hip::Concat)
 MNV_INSTALL_COMPUTE_FN(SliceClosure, hip::Slice)
 MNV_INSTALL_COMPUTE_FN(SelectClosure, hip::Select)
@@ -123,6 +125,8 @@ MNV_SIMPLE_OP(TanhBackwardOp, ComputeFnWithClosure, TanhBackwardClosure, "tanh b
 MNV_SIMPLE_OP(ConvBackwardBiasOp, ComputeFnWithClosure, ConvBackwardBiasClosure, "conv bp bias")
 MNV_SIMPLE_OP(LRNForwardOp, ComputeFnWithClosure, LRNForwardClosure, "LRN Forward")
 MNV_SIMPLE_OP(LRNBackwardOp, ComputeFnWithClosure, LRNBackwardClosure, "LRN Backward")
+MNV_SIMPLE_OP(ThresholdNormOp, ComputeFnWithClosure, ThresholdNormClosure, "threshold norm")
+MNV_SIMPLE_OP(IndexOp, ComputeFnWithClosure, IndexClosure, "index")
 MNV_SIMPLE_OP(ConcatOp, ComputeFnWithClosure, ConcatClosure, "Concat")
 MNV_SIMPLE_OP(SliceOp, ComputeFnWithClosure, SliceClosure, "Slice")
 MNV_SIMPLE_OP(SelectOp, ComputeFnWithClosure, SelectClosure, "select")

@@ -252,6 +252,18 @@ Tensor Runner::PoolingBackward(const Tensor& diff, const Tensor& top, const Tens
   return Compute({diff, top, bottom}, bottom->size, op);
 }
 
+Tensor Runner::ThresholdNorm(const Tensor& a, float threshold) {
+  auto op = std::make_shared<ThresholdNormOp>();
+  op->closure = {threshold};
+  return Compute({a}, a->size, op);
+}
+
+Tensor Runner::Index(const Tensor& a, int idx, const Scale& block) {
+  auto op = std::make_shared<IndexOp>();
+  op->closure = {idx};
+  return Compute({a}, block, op);
+}
+
 Tensor Runner::Concat(const std::vector<Tensor>& arrays, int catdim) {
   MNV_CHECK_GT(arrays.size(), 1u) << "Concat more than one narray";
   MNV_CHECK(catdim >= 0 && arrays[0]->size.NumDims() > static_cast<size_t>(catdim))

@@ -88,6 +88,8 @@ class Runner : public DeviceListener {
   Tensor PoolingBackward(const Tensor& diff, const Tensor& top, const Tensor& bottom,
                          PoolingInfo info);
   // reference minerva/narray/narray.cpp:129-160, 183-192
+  Tensor ThresholdNorm(const Tensor& a, float threshold);
+  Tensor Index(const Tensor& a, int idx, const Scale& block);  // the idx-th `block`-sized piece
   Tensor Concat(const std::vector<Tensor>& arrays, int catdim);
   Tensor Slice(const Tensor& src, int slice_dim, int st_off, int slice_count);
   Tensor Select(const Tensor& src, const std::vector<int>& indices);

@@ -709,3 +709,10 @@ int ora_rand_bernoulli(float* dst, size_t n, uint64_t seed, float p) {
   }
   return 0;
 }
+
+/* ThresholdNorm: basic.cpp:110-123, the expression as written there. */
+int ora_threshold_norm(const float* x, float* y, size_t n, float threshold) {
+  for (size_t i = 0; i < n; ++i)
+    y[i] = fabsf(x[i]) > threshold ? fabsf(x[i]) / x[i] * threshold : x[i];
+  return 0;
+}

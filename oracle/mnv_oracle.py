@@ -304,3 +304,11 @@ def rand_bernoulli(n, seed, p):
     _chk(lib().ora_rand_bernoulli(_p(out), ctypes.c_size_t(n), ctypes.c_uint64(seed),
                                   ctypes.c_float(p)), "rand_bernoulli")
     return out
+
+
+def threshold_norm(x, threshold):
+    x = _f(x)
+    out = np.empty(x.size, dtype=np.float32)
+    _chk(lib().ora_threshold_norm(_p(x), _p(out), ctypes.c_size_t(x.size), ctypes.c_float(threshold)),
+         "threshold_norm")
+    return out

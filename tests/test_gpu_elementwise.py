@@ -245,3 +245,12 @@ def test_randn_distribution_at_full_size(gpu):
     assert abs(float(z.mean(dtype=np.float64))) < 1e-3 and abs(float(z.std(dtype=np.float64)) - 1.0) < 1e-3
     # tails: P(|z| > 4) = 6.33e-5
     assert abs(np.count_nonzero(np.abs(z) > 4) / n - 6.334e-5) < 5e-6
+
+
+def test_threshold_norm_bit_exact(gpu, ora):
+    n = 100003
+    x = _rand(n, 95) * 2
+    x[:4] = [0.0, -0.0, 0.7, -0.7]
+    dx, dy = gpu.up(x), gpu.empty(n)
+    gpu.call("mnv_threshold_norm", dx.p, dy.p, ctypes.c_float(0.7), ctypes.c_size_t(n))
+    assert_bits_equal(gpu.down(dy), ora.threshold_norm(x, 0.7), "threshold norm")

@@ -203,6 +203,19 @@ def test_concat_slice_select(rt, ora):
         rt.op("select", [(m2, [3, 3])], [3])
 
 
+def test_threshold_norm_and_index(rt, ora):
+    x = _rand(24, 86) * 2
+    got, od = rt.op("threshold_norm", [(x, [4, 6])], [0.5])
+    assert od == [4, 6]
+    assert_bits_equal(got, ora.threshold_norm(x, 0.5), "threshold norm")
+    got, od = rt.op("index", [(x, [4, 6])], [2, 4, 2])      # third {4,2} block
+    assert od == [4, 2]
+    assert_bits_equal(got, x[16:24], "index")
+    from minerva_amd import hostapi
+    with pytest.raises(hostapi.HostError, match="outside the input"):
+        rt.op("index", [(x, [4, 6])], [3, 4, 2])
+
+
 def test_random_operators(rt, ora):
     from minerva_amd import hostapi
     hostapi.Runtime.set_random_seed(5)

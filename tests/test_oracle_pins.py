@@ -471,3 +471,12 @@ def test_random_tensors_mapping_and_distribution(ora):
     assert abs(b.mean() - 0.3) < 0.005
     assert b[28] == (1.0 if np.float32(x[0] >> 8) * np.float32(2.0 ** -24) < np.float32(0.3) else 0.0)
     assert ora.rand_bernoulli(1000, 3, 0.0).sum() == 0 and ora.rand_bernoulli(1000, 3, 1.0).sum() == 1000
+
+
+def test_threshold_norm_is_a_clip(ora):
+    x = np.array([-3.0, -1.0, -0.5, 0.0, 0.25, 1.0, 2.5, np.inf, -np.inf], np.float32)
+    got = ora.threshold_norm(x, 1.0)
+    # |x| / x * t is exactly sign(x) * t, so the operator is a clip to [-t, t] (inf/inf = nan)
+    want = np.clip(x, -1.0, 1.0)
+    assert np.array_equal(got[:7], want[:7])
+    assert np.isnan(got[7]) and np.isnan(got[8])
