@@ -15,10 +15,11 @@
 // running sum (add the entering channel, then subtract the leaving one, in fp32), kept in
 // a register.  For the common window sizes (3, 5, 7) the walk is unrolled by the window size:
 // the last `size` values then sit in a register ring with compile-time indices, so nothing is
-// read twice, and the loads of the next `size` channels are issued before the current ones
-// are consumed.  Other sizes take the generic kernels, which re-read the value that leaves
-// the window and the one needed for the output (cache hits).  All accesses are ordinary:
-// non-temporal 4-byte stores measured 35% slower here.
+// read twice, the loads of the next channels are issued before the current ones are
+// consumed, and a thread handles several neighbouring positions per access.  Other sizes
+// (and tensors of 2 GiB or more) take the generic kernels, which re-read the value that
+// leaves the window and the one needed for the output (cache hits).  All accesses are
+// ordinary: non-temporal 4-byte stores measured 35% slower here.
 #include <math.h>
 
 #include "mnv_common.h"
@@ -26,6 +27,7 @@
 namespace {
 
 #define MNV_LRN_THREADS 256
+#define MNV_LRN_ST_AUX 2  // nt bit of the 16-byte stores
 
 // s^e for s >= 1 through the hardware log2 / exp2: relative error ~1e-6
 __device__ __forceinline__ float pow_ge1(float s, float e) { return __expf(e * __logf(s)); }
@@ -94,115 +96,205 @@ __global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_bwd_kernel(
 }
 
 // ---- window size known at compile time ---------------------------------------------
+// A thread owns V consecutive positions of one image (V = 4 forward, 2 backward: the
+// backward pass keeps four tensors in flight) and reads / writes them with one buffer
+// access of 4*V bytes per channel; buffer accesses need only 4-byte alignment, which is
+// all an odd plane size leaves.  Its byte offset is fixed and the channel advances through
+// the wavefront-uniform scalar offset, so the walk costs no address arithmetic.  A group
+// that hangs over the end of its plane reads a few floats of the next channel into lanes
+// whose results are dropped, and stores its valid elements one by one.
+//
 // Slot u of a ring holds the value of channel head with head % SIZE == u; the value that
 // leaves the window when channel `head` enters is the one already in slot head % SIZE.
 // Slots start at zero, and channels past the end enter as zero: adding or subtracting
 // 0*0 leaves the running sum bit-for-bit unchanged, so the partial windows at both ends
-// need no special case.
-// G = a multiple of SIZE channels are handled per iteration and the next G loaded ahead: a
-// thread keeps G 4-byte loads in flight, which is what it takes to cover the memory latency.
-template <int SIZE, int G>
+// need no special case.  G (a multiple of SIZE) channels are handled per iteration and the
+// next G loaded ahead.
+template <int V>
+struct LrnVec {
+  float v[V];
+};
+template <int V>
+__device__ __forceinline__ LrnVec<V> lrn_load(mnv_rsrc r, unsigned voff, unsigned soff);
+template <>
+__device__ __forceinline__ LrnVec<4> lrn_load<4>(mnv_rsrc r, unsigned voff, unsigned soff) {
+  mnv_f4 t = __builtin_bit_cast(mnv_f4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0));
+  return LrnVec<4>{{t.x, t.y, t.z, t.w}};
+}
+template <>
+__device__ __forceinline__ LrnVec<2> lrn_load<2>(mnv_rsrc r, unsigned voff, unsigned soff) {
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  f2 t = __builtin_bit_cast(f2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, (int)soff, 0));
+  return LrnVec<2>{{t.x, t.y}};
+}
+template <int V>
+__device__ __forceinline__ void lrn_store(mnv_rsrc r, unsigned voff, unsigned soff, const float (&o)[V],
+                                          int valid) {
+  if (valid == V) {
+    if (V == 4) {
+      mnv_f4 t = {o[0], o[1], o[2], o[3 % V]};
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, t),
+                                             r, (int)voff, (int)soff, MNV_LRN_ST_AUX);
+    } else {
+      typedef float f2 __attribute__((ext_vector_type(2)));
+      f2 t = {o[0], o[1]};
+      __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(__attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned, t),
+                                            r, (int)voff, (int)soff, 0);
+    }
+  } else {
+#pragma unroll
+    for (int t = 0; t < V; ++t)
+      if (t < valid)
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, o[t]), r, (int)(voff + 4u * t),
+                                              (int)soff, 0);
+  }
+}
+
+template <int SIZE, int G, int V>
 __global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_fwd_ring_kernel(
     const float* __restrict__ bottom, float* __restrict__ scale, float* __restrict__ top,
-    float alpha_over_size, float negative_beta, int channels, int hw, size_t positions,
-    MnvFastDiv d_hw) {
+    float alpha_over_size, float negative_beta, int channels, int hw, int groups_per_image,
+    size_t groups, unsigned bytes, MnvFastDiv d_gpi) {
+  static_assert(G % SIZE == 0, "group must be whole windows");
   constexpr int pre_pad = (SIZE - 1) / 2, post_pad = SIZE - pre_pad - 1;
-  for (size_t q = (size_t)blockIdx.x * MNV_LRN_THREADS + threadIdx.x; q < positions;
+  const mnv_rsrc rin = mnv_make_rsrc(bottom, bytes), rsc = mnv_make_rsrc(scale, bytes),
+                 rtop = mnv_make_rsrc(top, bytes);
+  const unsigned cstep = (unsigned)hw * 4u;  // bytes from one channel to the next
+  for (size_t q = (size_t)blockIdx.x * MNV_LRN_THREADS + threadIdx.x; q < groups;
        q += (size_t)gridDim.x * MNV_LRN_THREADS) {
-    const int n = mnv_fastdiv((int)q, d_hw), p = (int)q - n * hw;
-    const size_t base = (size_t)n * channels * hw + p;
-    const float* in = bottom + base;
-    static_assert(G % SIZE == 0, "group must be whole windows");
-    float win[SIZE], nxt[G];
+    const int n = mnv_fastdiv((int)q, d_gpi), p0 = ((int)q - n * groups_per_image) * V;
+    const int valid = min(V, hw - p0);
+    const unsigned voff = ((unsigned)n * (unsigned)channels * (unsigned)hw + (unsigned)p0) * 4u;
+    LrnVec<V> win[SIZE], nxt[G];
 #pragma unroll
-    for (int u = 0; u < SIZE; ++u) win[u] = 0.f;
+    for (int u = 0; u < SIZE; ++u)
 #pragma unroll
-    for (int u = 0; u < G; ++u) nxt[u] = u < channels ? in[(size_t)u * hw] : 0.f;
-    float accum = 0.f;
+      for (int t = 0; t < V; ++t) win[u].v[t] = 0.f;
+#pragma unroll
+    for (int u = 0; u < G; ++u) {
+      if (u < channels) {
+        nxt[u] = lrn_load<V>(rin, voff, (unsigned)u * cstep);
+      } else {
+#pragma unroll
+        for (int t = 0; t < V; ++t) nxt[u].v[t] = 0.f;
+      }
+    }
+    float accum[V];
+#pragma unroll
+    for (int t = 0; t < V; ++t) accum[t] = 0.f;
     for (int h0 = 0; h0 < channels + post_pad; h0 += G) {
-      float cur[G];
+      LrnVec<V> cur[G];
 #pragma unroll
       for (int u = 0; u < G; ++u) {
         cur[u] = nxt[u];
         const int h = h0 + G + u;
-        nxt[u] = h < channels ? in[(size_t)h * hw] : 0.f;
+        if (h < channels) {
+          nxt[u] = lrn_load<V>(rin, voff, (unsigned)h * cstep);
+        } else {
+#pragma unroll
+          for (int t = 0; t < V; ++t) nxt[u].v[t] = 0.f;
+        }
       }
 #pragma unroll
       for (int u = 0; u < G; ++u) {
-        const int head = h0 + u;
-        accum += cur[u] * cur[u];
-        accum -= win[u % SIZE] * win[u % SIZE];
+        const int c = h0 + u - post_pad;
+#pragma unroll
+        for (int t = 0; t < V; ++t) {
+          accum[t] += cur[u].v[t] * cur[u].v[t];
+          accum[t] -= win[u % SIZE].v[t] * win[u % SIZE].v[t];
+        }
         win[u % SIZE] = cur[u];
-        const int c = head - post_pad;
         if (c >= 0 && c < channels) {
-          const float s = 1.f + accum * alpha_over_size;
-          const float self = win[(u - post_pad + SIZE) % SIZE];
-          scale[base + (size_t)c * hw] = s;
-          top[base + (size_t)c * hw] = self * pow_ge1(s, negative_beta);
+          float s[V], o[V];
+#pragma unroll
+          for (int t = 0; t < V; ++t) {
+            s[t] = 1.f + accum[t] * alpha_over_size;
+            o[t] = win[(u - post_pad + SIZE) % SIZE].v[t] * pow_ge1(s[t], negative_beta);
+          }
+          lrn_store<V>(rsc, voff, (unsigned)c * cstep, s, valid);
+          lrn_store<V>(rtop, voff, (unsigned)c * cstep, o, valid);
         }
       }
     }
   }
 }
 
-template <int SIZE, int G>
+template <int SIZE, int G, int V>
 __global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_bwd_ring_kernel(
     const float* __restrict__ bottom, const float* __restrict__ top,
     const float* __restrict__ scale, const float* __restrict__ top_diff,
     float* __restrict__ bottom_diff, float negative_beta, float cache_ratio, int channels, int hw,
-    size_t positions, MnvFastDiv d_hw) {
+    int groups_per_image, size_t groups, unsigned bytes, MnvFastDiv d_gpi) {
+  static_assert(G % SIZE == 0, "group must be whole windows");
   constexpr int pre_pad = SIZE - (SIZE + 1) / 2, post_pad = SIZE - pre_pad - 1;
-  for (size_t q = (size_t)blockIdx.x * MNV_LRN_THREADS + threadIdx.x; q < positions;
+  const mnv_rsrc rx = mnv_make_rsrc(bottom, bytes), ry = mnv_make_rsrc(top, bytes),
+                 rs = mnv_make_rsrc(scale, bytes), rdy = mnv_make_rsrc(top_diff, bytes),
+                 rdx = mnv_make_rsrc(bottom_diff, bytes);
+  const unsigned cstep = (unsigned)hw * 4u;
+  for (size_t q = (size_t)blockIdx.x * MNV_LRN_THREADS + threadIdx.x; q < groups;
        q += (size_t)gridDim.x * MNV_LRN_THREADS) {
-    const int n = mnv_fastdiv((int)q, d_hw), p = (int)q - n * hw;
-    const size_t base = (size_t)n * channels * hw + p;
-    const float* x = bottom + base;
-    const float* y = top + base;
-    const float* sc = scale + base;
-    const float* dy = top_diff + base;
+    const int n = mnv_fastdiv((int)q, d_gpi), p0 = ((int)q - n * groups_per_image) * V;
+    const int valid = min(V, hw - p0);
+    const unsigned voff = ((unsigned)n * (unsigned)channels * (unsigned)hw + (unsigned)p0) * 4u;
     // rings: ratio = dy*y/scale (the summed quantity), and dy, scale for the output term
-    static_assert(G % SIZE == 0, "group must be whole windows");
-    float rwin[SIZE], dwin[SIZE], swin[SIZE];
-    float ndy[G], ny[G], nsc[G], nx[G];  // next group; nx is bottom at the output channel
+    LrnVec<V> rwin[SIZE], dwin[SIZE], swin[SIZE];
+    LrnVec<V> ndy[G], ny[G], nsc[G], nx[G];  // next group; nx is bottom at the output channel
 #pragma unroll
-    for (int u = 0; u < SIZE; ++u) {
-      rwin[u] = 0.f; dwin[u] = 0.f; swin[u] = 1.f;
-    }
+    for (int u = 0; u < SIZE; ++u)
 #pragma unroll
-    for (int u = 0; u < G; ++u) {
-      const bool in_range = u < channels;
-      ndy[u] = in_range ? dy[(size_t)u * hw] : 0.f;
-      ny[u] = in_range ? y[(size_t)u * hw] : 0.f;
-      nsc[u] = in_range ? sc[(size_t)u * hw] : 1.f;
-      const int c = u - post_pad;
-      nx[u] = (c >= 0 && c < channels) ? x[(size_t)c * hw] : 0.f;
-    }
-    float accum = 0.f;
+      for (int t = 0; t < V; ++t) {
+        rwin[u].v[t] = 0.f; dwin[u].v[t] = 0.f; swin[u].v[t] = 1.f;
+      }
+    auto fetch = [&](int h, int u) {
+      if (h < channels) {
+        ndy[u] = lrn_load<V>(rdy, voff, (unsigned)h * cstep);
+        ny[u] = lrn_load<V>(ry, voff, (unsigned)h * cstep);
+        nsc[u] = lrn_load<V>(rs, voff, (unsigned)h * cstep);
+      } else {
+#pragma unroll
+        for (int t = 0; t < V; ++t) {
+          ndy[u].v[t] = 0.f; ny[u].v[t] = 0.f; nsc[u].v[t] = 1.f;
+        }
+      }
+      const int c = h - post_pad;
+      if (c >= 0 && c < channels) {
+        nx[u] = lrn_load<V>(rx, voff, (unsigned)c * cstep);
+      } else {
+#pragma unroll
+        for (int t = 0; t < V; ++t) nx[u].v[t] = 0.f;
+      }
+    };
+#pragma unroll
+    for (int u = 0; u < G; ++u) fetch(u, u);
+    float accum[V];
+#pragma unroll
+    for (int t = 0; t < V; ++t) accum[t] = 0.f;
     for (int h0 = 0; h0 < channels + post_pad; h0 += G) {
-      float cdy[G], cy[G], csc[G], cx[G];
+      LrnVec<V> cdy[G], cy[G], csc[G], cx[G];
 #pragma unroll
       for (int u = 0; u < G; ++u) {
         cdy[u] = ndy[u]; cy[u] = ny[u]; csc[u] = nsc[u]; cx[u] = nx[u];
-        const int h = h0 + G + u;
-        const bool in_range = h < channels;
-        ndy[u] = in_range ? dy[(size_t)h * hw] : 0.f;
-        ny[u] = in_range ? y[(size_t)h * hw] : 0.f;
-        nsc[u] = in_range ? sc[(size_t)h * hw] : 1.f;
-        const int c = h - post_pad;
-        nx[u] = (c >= 0 && c < channels) ? x[(size_t)c * hw] : 0.f;
+        fetch(h0 + G + u, u);
       }
 #pragma unroll
       for (int u = 0; u < G; ++u) {
-        const int head = h0 + u;
-        const float r = cdy[u] * cy[u] / csc[u];  // 0 past the last channel
-        accum += r;
-        accum -= rwin[u % SIZE];
+        const int c = h0 + u - post_pad;
+        LrnVec<V> r;
+#pragma unroll
+        for (int t = 0; t < V; ++t) {
+          r.v[t] = cdy[u].v[t] * cy[u].v[t] / csc[u].v[t];  // 0 past the last channel
+          accum[t] += r.v[t];
+          accum[t] -= rwin[u % SIZE].v[t];
+        }
         rwin[u % SIZE] = r; dwin[u % SIZE] = cdy[u]; swin[u % SIZE] = csc[u];
-        const int c = head - post_pad;
         if (c >= 0 && c < channels) {
           const int slot = (u - post_pad + SIZE) % SIZE;
-          const float out = dwin[slot] * pow_ge1(swin[slot], negative_beta) - cache_ratio * cx[u] * accum;
-          bottom_diff[base + (size_t)c * hw] = out;
+          float o[V];
+#pragma unroll
+          for (int t = 0; t < V; ++t)
+            o[t] = dwin[slot].v[t] * pow_ge1(swin[slot].v[t], negative_beta) -
+                   cache_ratio * cx[u].v[t] * accum[t];
+          lrn_store<V>(rdx, voff, (unsigned)c * cstep, o, valid);
         }
       }
     }
@@ -236,26 +328,27 @@ int mnv_lrn_fwd(const float* bottom, float* scale, float* top, int local_size, f
   int hw;
   int rc = check_dims(local_size, num_images, channels, height, width, &positions, &hw);
   if (rc) return rc;
-  const dim3 grid(lrn_grid(positions)), block(MNV_LRN_THREADS);
+  const dim3 block(MNV_LRN_THREADS);
   hipStream_t s = mnv_stream(stream);
   const float aos = alpha / local_size;
-  const MnvFastDiv d = mnv_fastdiv_make(hw);
-  switch (local_size) {
-    case 3:
-      hipLaunchKernelGGL((mnv_lrn_fwd_ring_kernel<3, 18>), grid, block, 0, s, bottom, scale, top, aos,
-                         -beta, channels, hw, positions, d);
-      break;
-    case 5:
-      hipLaunchKernelGGL((mnv_lrn_fwd_ring_kernel<5, 20>), grid, block, 0, s, bottom, scale, top, aos,
-                         -beta, channels, hw, positions, d);
-      break;
-    case 7:
-      hipLaunchKernelGGL((mnv_lrn_fwd_ring_kernel<7, 21>), grid, block, 0, s, bottom, scale, top, aos,
-                         -beta, channels, hw, positions, d);
-      break;
-    default:
-      hipLaunchKernelGGL(mnv_lrn_fwd_kernel, grid, block, 0, s, bottom, scale, top, local_size,
-                         aos, -beta, channels, hw, positions, d);
+  const size_t bytes = positions * channels * sizeof(float);
+  constexpr int V = 4;
+  const int gpi = (hw + V - 1) / V;
+  const size_t groups = (size_t)gpi * num_images;
+  const bool ring = bytes < 0x80000000ull && (local_size == 3 || local_size == 5 || local_size == 7);
+  if (ring) {
+    const dim3 grid(lrn_grid(groups));
+    const MnvFastDiv d = mnv_fastdiv_make(gpi);
+#define MNV_LRN_FWD(SIZE, G)                                                                       \
+  hipLaunchKernelGGL((mnv_lrn_fwd_ring_kernel<SIZE, G, V>), grid, block, 0, s, bottom, scale, top, \
+                     aos, -beta, channels, hw, gpi, groups, (unsigned)bytes, d)
+    if (local_size == 3) MNV_LRN_FWD(3, 6);
+    else if (local_size == 5) MNV_LRN_FWD(5, 5);
+    else MNV_LRN_FWD(7, 7);
+#undef MNV_LRN_FWD
+  } else {
+    hipLaunchKernelGGL(mnv_lrn_fwd_kernel, dim3(lrn_grid(positions)), block, 0, s, bottom, scale, top,
+                       local_size, aos, -beta, channels, hw, positions, mnv_fastdiv_make(hw));
   }
   return MNV_LAUNCH_STATUS();
 }
@@ -268,26 +361,29 @@ int mnv_lrn_bwd(const float* bottom, const float* top, const float* scale, const
   int hw;
   int rc = check_dims(local_size, num_images, channels, height, width, &positions, &hw);
   if (rc) return rc;
-  const dim3 grid(lrn_grid(positions)), block(MNV_LRN_THREADS);
+  const dim3 block(MNV_LRN_THREADS);
   hipStream_t s = mnv_stream(stream);
   const float ratio = (float)(2. * alpha * beta / local_size);
-  const MnvFastDiv d = mnv_fastdiv_make(hw);
-  switch (local_size) {
-    case 3:
-      hipLaunchKernelGGL((mnv_lrn_bwd_ring_kernel<3, 9>), grid, block, 0, s, bottom, top, scale,
-                         top_diff, bottom_diff, -beta, ratio, channels, hw, positions, d);
-      break;
-    case 5:
-      hipLaunchKernelGGL((mnv_lrn_bwd_ring_kernel<5, 10>), grid, block, 0, s, bottom, top, scale,
-                         top_diff, bottom_diff, -beta, ratio, channels, hw, positions, d);
-      break;
-    case 7:
-      hipLaunchKernelGGL((mnv_lrn_bwd_ring_kernel<7, 14>), grid, block, 0, s, bottom, top, scale,
-                         top_diff, bottom_diff, -beta, ratio, channels, hw, positions, d);
-      break;
-    default:
-      hipLaunchKernelGGL(mnv_lrn_bwd_kernel, grid, block, 0, s, bottom, top, scale, top_diff,
-                         bottom_diff, local_size, -beta, ratio, channels, hw, positions, d);
+  const size_t bytes = positions * channels * sizeof(float);
+  constexpr int V = 2;
+  const int gpi = (hw + V - 1) / V;
+  const size_t groups = (size_t)gpi * num_images;
+  const bool ring = bytes < 0x80000000ull && (local_size == 3 || local_size == 5 || local_size == 7);
+  if (ring) {
+    const dim3 grid(lrn_grid(groups));
+    const MnvFastDiv d = mnv_fastdiv_make(gpi);
+#define MNV_LRN_BWD(SIZE, G)                                                                     \
+  hipLaunchKernelGGL((mnv_lrn_bwd_ring_kernel<SIZE, G, V>), grid, block, 0, s, bottom, top, scale, \
+                     top_diff, bottom_diff, -beta, ratio, channels, hw, gpi, groups,             \
+                     (unsigned)bytes, d)
+    if (local_size == 3) MNV_LRN_BWD(3, 6);
+    else if (local_size == 5) MNV_LRN_BWD(5, 5);
+    else MNV_LRN_BWD(7, 7);
+#undef MNV_LRN_BWD
+  } else {
+    hipLaunchKernelGGL(mnv_lrn_bwd_kernel, dim3(lrn_grid(positions)), block, 0, s, bottom, top, scale,
+                       top_diff, bottom_diff, local_size, -beta, ratio, channels, hw, positions,
+                       mnv_fastdiv_make(hw));
   }
   return MNV_LAUNCH_STATUS();
 }
