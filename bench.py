@@ -270,10 +270,36 @@ def cpu_baseline(batch=4):
     nets.alexnet_step(params, data, label, 0.01, batch)
     dt = time.perf_counter() - t0
     log("cpu oracle alexnet b=%d: %.2f s" % (batch, dt))
-    return {"value": round(batch / dt, 4), "unit": "images/s", "cores": 1, "kind": "port",
-            "sample": "one AlexNet-shaped train step at batch %d (of 256) with the naive "
-                      "single-threaded CPU oracle, %.1f s" % (batch, dt),
-            "host_cpus": os.cpu_count()}
+    out = {"value": round(batch / dt, 4), "unit": "images/s", "cores": 1, "kind": "port",
+           "sample": "one AlexNet-shaped train step at batch %d (of 256) with the naive "
+                     "single-threaded CPU oracle, %.1f s" % (batch, dt),
+           "host_cpus": os.cpu_count()}
+    # the same single-threaded restatement on the other parts of the metric (one run each,
+    # output allocation included): what the reference's CPU device would spend per operator
+    from oracle import mnv_oracle as ora
+    rng = np.random.default_rng(11)
+    ne = 8192 * 8192
+    x, y = rng.standard_normal(ne, dtype=np.float32), rng.standard_normal(ne, dtype=np.float32)
+    others = {}
+
+    def timed(name, fn, unit_work, unit):
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        others[name] = {"s": round(dt, 3), unit: round(unit_work / dt / 1e9, 3)}
+
+    timed("add 8192x8192", lambda: ora.arithmetic(ora.ADD, x, y), 12.0 * ne, "gbs")
+    timed("sum dim 0 8192x8192", lambda: ora.reduction(ora.SUM, x, [8192, 8192], [0]), 4.0 * ne, "gbs")
+    a = rng.standard_normal(1000 * 4096, dtype=np.float32)
+    b = rng.standard_normal(4096 * 256, dtype=np.float32)
+    timed("sgemm 1000x4096x256", lambda: ora.matmult(a, b, 1000, 256, 4096), 2.0 * 1000 * 4096 * 256,
+          "gflops")
+    pm, dm, lm = nets.make_inputs("mlp", BATCH)
+    t0 = time.perf_counter()
+    nets.mlp_step(pm, dm, lm, 0.01, BATCH)
+    others["mlp step b256"] = {"s": round(time.perf_counter() - t0, 3)}
+    out["other_parts"] = others
+    return out
 
 
 def main():
