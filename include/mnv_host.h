@@ -88,6 +88,8 @@ int mnvh_concurrent_adds(void* runtime, const float* a, const float* b, size_t n
 
 /* Training graphs.  kind: "mlp" (784-256-10), "cnn" (MNIST CNN; variant 0 = conv2 pad 0
  * + 2x2/2 pooling, 1 = the reference app's pad 2 + 3x3/3), "alexnet". */
+/* "alexnet": variant 0 = no dropout (the benchmark configuration), 1 = the reference
+ * application's drop6 / drop7 with rate 0.5, masks from the restartable seed sequence */
 int mnvh_net_create(void* runtime, const char* kind, int batch, int variant, void** net);
 int mnvh_net_destroy(void* net);
 int mnvh_net_num_params(void* net, int* count);

@@ -295,7 +295,7 @@ int mnvh_net_create(void* runtime, const char* kind, int batch, int variant, voi
     std::string k(kind);
     if (k == "mlp") h->net.reset(new MlpNet(rt, batch));
     else if (k == "cnn") h->net.reset(variant == 1 ? new CnnNet(rt, batch, 2, 3) : new CnnNet(rt, batch));
-    else if (k == "alexnet") h->net.reset(new AlexNet(rt, batch));
+    else if (k == "alexnet") h->net.reset(new AlexNet(rt, batch, 1000, variant == 1 ? 0.5f : 0.f));
     else MNV_FATAL() << "unknown net '" << k << "'";
     *net = h.release();
   });

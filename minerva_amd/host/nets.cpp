@@ -94,7 +94,8 @@ void CnnNet::Step(const Tensor& data, const Tensor& label, float lr) {
 
 // --------------------------------------------------------------------- AlexNet
 
-AlexNet::AlexNet(Runner* r, int batch, int num_classes) : Net(r, batch), classes_(num_classes) {
+AlexNet::AlexNet(Runner* r, int batch, int num_classes, float dropout_rate)
+    : Net(r, batch), classes_(num_classes), dropout_rate_(dropout_rate) {
   convs[0] = ConvInfo(0, 0, 4, 4);
   convs[1] = ConvInfo(2, 2, 1, 1);
   convs[2] = convs[3] = convs[4] = ConvInfo(1, 1, 1, 1);
@@ -136,8 +137,18 @@ void AlexNet::Step(const Tensor& data, const Tensor& label, float lr) {
   acts[7] = rt->ReluForward(rt->ConvForward(acts[6], W(4), B(4), convs[4]));   // conv5
   acts[8] = rt->PoolingForward(acts[7], poolings[2]);                           // pool5
   Tensor re8 = rt->Reshape(acts[8], Scale{acts[8]->size.Prod() / n, n});
+  const bool drop = dropout_rate_ > 0.f;
+  Tensor mask6, mask7;
   acts[9] = rt->ReluForward(fc(5, re8));                                        // fc6
+  if (drop) {
+    mask6 = rt->RandBernoulli(acts[9]->size, dropout_rate_);
+    acts[9] = rt->Mult(acts[9], mask6);                                         // drop6
+  }
   acts[10] = rt->ReluForward(fc(6, acts[9]));                                   // fc7
+  if (drop) {
+    mask7 = rt->RandBernoulli(acts[10]->size, dropout_rate_);
+    acts[10] = rt->Mult(acts[10], mask7);                                       // drop7
+  }
   acts[11] = fc(7, acts[10]);                                                   // fc8
   Tensor out = rt->Reshape(
       rt->SoftmaxForward(rt->Reshape(acts[11], Scale{classes_, 1, 1, n}), SoftmaxAlgorithm::kInstance),
@@ -145,8 +156,12 @@ void AlexNet::Step(const Tensor& data, const Tensor& label, float lr) {
   results["prob"] = out;
   // BP
   sens[11] = rt->Sub(out, label);
-  sens[10] = rt->ReluBackward(rt->MatMult(rt->Trans(W(7)), sens[11]), acts[10], acts[10]);
-  sens[9] = rt->ReluBackward(rt->MatMult(rt->Trans(W(6)), sens[10]), acts[9], acts[9]);
+  sens[10] = rt->MatMult(rt->Trans(W(7)), sens[11]);                            // fc8
+  if (drop) sens[10] = rt->Mult(sens[10], mask7);                               // drop7
+  sens[10] = rt->ReluBackward(sens[10], acts[10], acts[10]);                    // relu7
+  sens[9] = rt->MatMult(rt->Trans(W(6)), sens[10]);
+  if (drop) sens[9] = rt->Mult(sens[9], mask6);                                 // drop6
+  sens[9] = rt->ReluBackward(sens[9], acts[9], acts[9]);                        // relu6
   sens[8] = rt->Reshape(rt->MatMult(rt->Trans(W(5)), sens[9]), acts[8]->size);
   sens[7] = rt->ReluBackward(rt->PoolingBackward(sens[8], acts[8], acts[7], poolings[2]), acts[7], acts[7]);
   sens[6] = rt->ReluBackward(rt->ConvBackwardData(sens[7], acts[6], W(4), convs[4]), acts[6], acts[6]);

@@ -60,13 +60,16 @@ class CnnNet : public Net {
 
 class AlexNet : public Net {
  public:
-  AlexNet(Runner* r, int batch, int num_classes = 1000);
+  // dropout_rate > 0: the reference application's drop6 / drop7 (owl/apps/imagenet_alexnet/
+  // alexnet.py:86-89,97-101): activations times a Bernoulli(dropout_rate) mask, no rescaling
+  AlexNet(Runner* r, int batch, int num_classes = 1000, float dropout_rate = 0.f);
   void Step(const Tensor& data, const Tensor& label, float lr) override;
   Scale DataSize() const override { return Scale{227, 227, 3, batch_}; }
   Scale LabelSize() const override { return Scale{classes_, batch_}; }
 
  private:
   int classes_;
+  float dropout_rate_;
   ConvInfo convs[5];
   PoolingInfo poolings[3];
 };

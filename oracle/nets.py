@@ -112,8 +112,29 @@ def alexnet_param_shapes(classes=1000):
     return shapes
 
 
-def alexnet_step(p, data, label, lr, batch, classes=1000):
+def seed_sequence(base, count):
+    """The seeds the host layer hands to successive Randn / RandBernoulli calls after
+    SetRandomSeed(base): splitmix64 of base + k * golden ratio, k = 1, 2, ..."""
+    M = (1 << 64) - 1
+    out = []
+    for k in range(1, count + 1):
+        z = (base + 0x9E3779B97F4A7C15 * k) & M
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & M
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & M
+        out.append(z ^ (z >> 31))
+    return out
+
+
+def alexnet_step(p, data, label, lr, batch, classes=1000, dropout_rate=0.0, seed_base=None):
+    """dropout_rate > 0 adds the reference application's drop6 / drop7
+    (owl/apps/imagenet_alexnet/alexnet.py:86-89,97-101) with the masks the library draws for
+    the first two RandBernoulli calls after SetRandomSeed(seed_base)."""
     N = batch
+    drop = dropout_rate > 0.0
+    if drop:
+        s6, s7 = seed_sequence(seed_base, 2)
+        mask6 = ora.rand_bernoulli(4096 * N, s6, dropout_rate)
+        mask7 = ora.rand_bernoulli(4096 * N, s7, dropout_rate)
     cv = [(N,) + c for c in ALEX_CONVS]
     pool = lambda C, H: (N, C, H, H, 2, 2, 3, 3, 0, 0)
     acts = [None] * 12
@@ -127,14 +148,24 @@ def alexnet_step(p, data, label, lr, batch, classes=1000):
     acts[7] = _relu(ora.conv_fwd(acts[6], p["w4"], p["b4"], *cv[4]))     # 256 x 13 x 13
     acts[8] = ora.pool_fwd(ora.POOL_MAX, acts[7], *pool(256, 13))        # 6 -> 9216
     acts[9] = _relu(_fc(p["w5"], acts[8], p["b5"], 4096, 9216, N))
+    if drop:
+        acts[9] = ora.arithmetic(ora.MUL, acts[9], mask6)
     acts[10] = _relu(_fc(p["w6"], acts[9], p["b6"], 4096, 4096, N))
+    if drop:
+        acts[10] = ora.arithmetic(ora.MUL, acts[10], mask7)
     acts[11] = _fc(p["w7"], acts[10], p["b7"], classes, 4096, N)
     out = ora.softmax_instance_fwd(acts[11], N, classes, 1, 1)
     sens = [None] * 12
     sens[11] = ora.arithmetic(ora.SUB, out, label)
     mm = lambda a, b, m, n, k: ora.matmult(a, b, m, n, k, fast=True)
-    sens[10] = _relu_bwd(mm(ora.transpose(p["w7"], 4096, classes), sens[11], 4096, N, classes), acts[10])
-    sens[9] = _relu_bwd(mm(ora.transpose(p["w6"], 4096, 4096), sens[10], 4096, N, 4096), acts[9])
+    sens[10] = mm(ora.transpose(p["w7"], 4096, classes), sens[11], 4096, N, classes)
+    if drop:
+        sens[10] = ora.arithmetic(ora.MUL, sens[10], mask7)
+    sens[10] = _relu_bwd(sens[10], acts[10])
+    sens[9] = mm(ora.transpose(p["w6"], 4096, 4096), sens[10], 4096, N, 4096)
+    if drop:
+        sens[9] = ora.arithmetic(ora.MUL, sens[9], mask6)
+    sens[9] = _relu_bwd(sens[9], acts[9])
     sens[8] = mm(ora.transpose(p["w5"], 9216, 4096), sens[9], 9216, N, 4096)
     sens[7] = _relu_bwd(ora.pool_bwd(ora.POOL_MAX, sens[8], acts[8], acts[7], *pool(256, 13)), acts[7])
     sens[6] = _relu_bwd(ora.conv_bwd_data(sens[7], p["w4"], *cv[4]), acts[6])

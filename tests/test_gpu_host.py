@@ -377,3 +377,21 @@ def test_alexnet_step_matches_oracle_small_batch(ora):
     ce = lambda pr: -np.log(pr.reshape(batch, -1)[np.arange(batch), lab].astype(np.float64)).mean()
     assert abs(ce(got["prob"]) - ce(res["prob"])) <= 1e-5 * abs(ce(res["prob"]))
     assert ops > 80
+
+
+def test_alexnet_step_with_dropout_matches_oracle(ora):
+    """The reference application's graph including drop6 / drop7: the masks come from the
+    library's generator, which the oracle reproduces bit for bit from the seed sequence."""
+    from minerva_amd import hostapi
+    from oracle import nets
+    batch, seed = 2, 20240607
+    params, data, label = nets.make_inputs("alexnet", batch)
+    say("alexnet + dropout oracle step b=2 (CPU)")
+    p, res = nets.alexnet_step(dict(params), data, label, 0.01, batch, dropout_rate=0.5, seed_base=seed)
+    say("alexnet + dropout GPU step b=2")
+    hostapi.Runtime.set_random_seed(seed)
+    got, ops = _run_net("alexnet", batch, 1, False, variant=1)
+    _compare(got, p, res, batch=batch, deep=True)
+    # dropout changed the result: the plain graph's probabilities differ
+    _, plain = nets.alexnet_step(dict(params), data, label, 0.01, batch)
+    assert normwise(got["prob"], plain["prob"]) > 1e-3 or np.max(np.abs(got["g_w7"] - plain["g_w7"])) > 0
