@@ -303,7 +303,11 @@ __global__ __launch_bounds__(256) void mnv_gemm_splitk_reduce_kernel(P prob,
 // whole extra round, so the estimate below (workgroups on the fullest CU x slabs each,
 // corrected for the matrix pipe running below its rate with fewer than four workgroups in
 // residence) is minimised rather than the count simply rounded up.
-static inline int mnv_pick_splits(long long tiles, int slabs, int max_splits) {
+// `per_split` (optional) is what every additional k range costs for writing and re-reading
+// its partial result, in the same unit (one slab of one workgroup); `cost_out` receives the
+// estimate of the chosen count so that callers can compare tile shapes.
+static inline int mnv_pick_splits(long long tiles, int slabs, int max_splits, double per_split = 0.0,
+                                  double* cost_out = nullptr) {
   static const double rate[5] = {1.0, 0.45, 0.75, 0.92, 1.0};
   if (max_splits < 1) max_splits = 1;
   int best = 1;
@@ -311,12 +315,13 @@ static inline int mnv_pick_splits(long long tiles, int slabs, int max_splits) {
   for (int s = 1; s <= max_splits; ++s) {
     long long per_cu = (tiles * s + 255) / 256;
     int len = (slabs + s - 1) / s;
-    double cost = (double)per_cu * (len + 4) / rate[per_cu < 4 ? per_cu : 4];
+    double cost = (double)per_cu * (len + 4) / rate[per_cu < 4 ? per_cu : 4] + (s > 1 ? per_split * s : 0.0);
     if (s == 1 || cost < best_cost * 0.98) {  // prefer fewer partial results on a near tie
       best = s;
       best_cost = cost;
     }
   }
+  if (cost_out) *cost_out = best_cost;
   return best;
 }
 

@@ -74,20 +74,41 @@ typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
 #define MNV_SGEMM_MAX_SPLITS 16
 
-// How many k ranges to use for an (m,n,k) product given `ws_floats` floats of scratch.
-int pick_splits(int tiles, int slabs, size_t mn, size_t ws_floats) {
-  if (tiles >= 1024 || slabs < 8) return 1;
-  int max_splits = MNV_SGEMM_MAX_SPLITS;
-  if (max_splits > slabs / 4) max_splits = slabs / 4;
-  size_t fit = mn ? ws_floats / mn : 0;
-  if ((size_t)max_splits > fit) max_splits = (int)fit;
-  return mnv_pick_splits(tiles, slabs, max_splits);
-}
+// Tile shape and number of k ranges for an (m,n,k) product given `ws_floats` floats of
+// scratch.  Both shapes are priced with the occupancy model of mnv_pick_splits, in units of
+// one 128x128x16 slab: a 64x64 slab is a quarter of the arithmetic at about 80% of the
+// efficiency, and every extra k range writes and re-reads m*n floats (about 1.2 us per
+// slab unit, 6 TB/s for the partial sums).
+struct SgemmPlan {
+  bool small;
+  int splits;
+};
 
-bool use_small_tile(int m, int n) {
-  // few, partly empty 128x128 tiles: smaller tiles give more workgroups and less padding
-  long long big_tiles = (long long)((m + 127) / 128) * ((n + 127) / 128);
-  return big_tiles < 128 || m <= 64 || n <= 64;
+SgemmPlan plan_sgemm(int m, int n, int k, size_t ws_floats) {
+  const int slabs = (k + 15) / 16;
+  const size_t mn = (size_t)m * n;
+  const double per_split = 8.0 * (double)mn / 6e6 / 1.2;
+  SgemmPlan best{false, 1};
+  double best_cost = 0;
+  for (int small = 0; small < 2; ++small) {
+    const int bm = small ? 64 : 128;
+    const long long tiles = (long long)((m + bm - 1) / bm) * ((n + bm - 1) / bm);
+    int max_splits = MNV_SGEMM_MAX_SPLITS;
+    if (max_splits > slabs / 4) max_splits = slabs / 4;
+    const size_t fit = mn ? ws_floats / mn : 0;
+    if ((size_t)max_splits > fit) max_splits = (int)fit;
+    if (tiles >= 1024 || slabs < 8) max_splits = 1;
+    const double unit = small ? 0.31 : 1.0;
+    double cost;
+    const int splits = mnv_pick_splits(tiles, slabs, max_splits, per_split / unit, &cost);
+    cost *= unit;
+    const bool forced = small ? (m <= 64 || n <= 64) : false;
+    if (small == 0 || forced || cost < best_cost) {
+      best = SgemmPlan{small != 0, splits};
+      best_cost = cost;
+    }
+  }
+  return best;
 }
 
 }  // namespace
@@ -96,12 +117,8 @@ extern "C" {
 
 size_t mnv_sgemm_nn_workspace_bytes(int m, int n, int k) {
   if (m <= 0 || n <= 0 || k <= 0) return 0;
-  bool small = use_small_tile(m, n);
-  int bm = small ? 64 : 128;
-  int tiles = ((m + bm - 1) / bm) * ((n + bm - 1) / bm);
-  int slabs = (k + 15) / 16;
-  int splits = pick_splits(tiles, slabs, (size_t)m * n, (size_t)-1);
-  return splits > 1 ? (size_t)splits * m * n * sizeof(float) : 0;
+  const SgemmPlan plan = plan_sgemm(m, n, k, (size_t)-1);
+  return plan.splits > 1 ? (size_t)plan.splits * m * n * sizeof(float) : 0;
 }
 
 int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k, void* workspace,
@@ -112,12 +129,9 @@ int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k, 
   if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
   hipStream_t s = mnv_stream(stream);
   bool vec = (m % 4 == 0) && (k % 4 == 0) && mnv_aligned16(a) && mnv_aligned16(b);
-  bool small = use_small_tile(m, n);
-  int bm = small ? 64 : 128;
-  int tiles = ((m + bm - 1) / bm) * ((n + bm - 1) / bm);
-  int slabs = (k + 15) / 16;
-  size_t ws_floats = workspace ? workspace_bytes / sizeof(float) : 0;
-  int splits = pick_splits(tiles, slabs, (size_t)m * n, ws_floats);
+  const SgemmPlan plan = plan_sgemm(m, n, k, workspace ? workspace_bytes / sizeof(float) : 0);
+  const bool small = plan.small;
+  const int splits = plan.splits;
   if (vec) {
     SgemmNN<true> p = make_sgemm<true>(a, b, c, m, n, k);
     return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
