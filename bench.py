@@ -41,6 +41,20 @@ def log(*a):
     sys.stderr.flush()
 
 
+def graph_replay(rt, net, steps, warmup):
+    """The same step recorded once into a HIP graph and replayed, one sync per replay.  The
+    replay runs the same kernels on the same buffers plus one copy kernel per parameter
+    (new weights back over the old ones); reported beside the operator-by-operator figure,
+    never as `value`."""
+    nodes = net.capture_step(0.01)
+    net.replay(warmup)
+    t0 = time.perf_counter()
+    net.replay(steps, sync_each_step=True)
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    net.release_graph()
+    return {"nodes": nodes, "ms_per_step": round(ms, 4), "images_per_s": round(BATCH / ms * 1e3, 1)}
+
+
 def alexnet_bench(steps, warmup):
     from minerva_amd import hostapi
     from oracle import nets  # input generator only (seeded host data)
@@ -69,8 +83,14 @@ def alexnet_bench(steps, warmup):
         rt.profile(False)
         prob = net.read("prob", 1000 * BATCH)
         ms = (t1 - t0) * 1e3 / steps
-        out[mode] = {"ms_per_step": ms, "images_per_s": BATCH / (ms / 1e3),
-                     "ops_per_step": (rt.ops_issued() - ops0) // steps,
+        ops_per_step = (rt.ops_issued() - ops0) // steps
+        graph = None
+        if not sync_each:
+            graph = graph_replay(rt, net, steps, warmup)
+            log("alexnet b=%d recorded step: %d nodes, %.3f ms/replay" %
+                (BATCH, graph["nodes"], graph["ms_per_step"]))
+        out[mode] = {"graph_replay": graph,"ms_per_step": ms, "images_per_s": BATCH / (ms / 1e3),
+                     "ops_per_step": ops_per_step,
                      "finite": bool(np.isfinite(prob).all()), "profile": prof,
                      "h2d_batch_ms": t_h2d}
         log("alexnet b=%d %s: %.3f ms/step, %.1f img/s, %d ops/step" %
@@ -254,7 +274,9 @@ def small_nets(steps=20, warmup=3):
         ms = (time.perf_counter() - t0) * 1e3 / steps
         out[name + "_b256"] = {"ms_per_step": round(ms, 4), "images_per_s": round(BATCH / ms * 1e3, 1),
                                "ops_per_step": (rt.ops_issued() - ops0) // steps}
-        log("%s b=%d: %.3f ms/step" % (name, BATCH, ms))
+        out[name + "_b256"]["graph_replay"] = g = graph_replay(rt, net, steps, warmup)
+        log("%s b=%d: %.3f ms/step, recorded step %.3f ms/replay (%d nodes)" %
+            (name, BATCH, ms, g["ms_per_step"], g["nodes"]))
         net.close()
         rt.close()
     return out
@@ -335,6 +357,7 @@ def main():
         "step_mfma_frac": round(STEP_GFLOP / main_run["ms_per_step"] / PEAK_FP32_MFMA_TFLOPS, 4),
         "per_op_sync": {"images_per_s": round(res["per_op_sync"]["images_per_s"], 1),
                         "ms_per_step": round(res["per_op_sync"]["ms_per_step"], 3)},
+        "graph_replay": main_run["graph_replay"],
         "h2d_batch_ms": round(main_run["h2d_batch_ms"], 2),
         "roofline": roof,
         "sgemm": sgemm,

@@ -62,6 +62,20 @@ int mnv_event_destroy(void* event);
 int mnv_event_record(void* event, mnv_stream_t stream);
 int mnv_event_sync(void* event);
 int mnv_event_elapsed_ms(void* start, void* stop, float* ms);
+/* Stream capture into a HIP graph.  No counterpart in the reference, which launches and
+ * synchronises every operator by itself (minerva/device/device.cpp:204-221); for callers
+ * whose step is a fixed sequence of short kernels and therefore launch-bound.  Between
+ * begin and end every call of this library on `stream` (not NULL) is recorded instead of
+ * run; only kernel launches may be recorded, so the sequence must have run once before
+ * (one-time set-up), must not allocate, synchronise or copy from host memory
+ * (mnv_select, mnv_memcpy_h2d/d2h), and must use the same buffers on every replay.
+ * end_capture returns the instantiated graph and optionally its node count;
+ * abort_capture ends a capture whose recording failed and discards it. */
+int mnv_graph_begin_capture(mnv_stream_t stream);
+int mnv_graph_end_capture(mnv_stream_t stream, void** graph_exec, size_t* num_nodes);
+int mnv_graph_abort_capture(mnv_stream_t stream);
+int mnv_graph_launch(void* graph_exec, mnv_stream_t stream);
+int mnv_graph_destroy(void* graph_exec);
 const char* mnv_error_string(int status);
 
 /* ---- elementwise binary: c[i] = a[i] (op) b[i]

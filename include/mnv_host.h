@@ -102,6 +102,20 @@ int mnvh_net_load_batch(void* net, const float* data, size_t data_floats, const 
                         size_t label_floats);
 /* One forward + backward + SGD step on the resident batch. */
 int mnvh_net_step(void* net, float lr);
+/* Records one step on the resident batch into a HIP graph (nothing of it is applied:
+ * parameters are unchanged afterwards), for networks whose step is launch-bound.  The
+ * reference has no counterpart: its device launches and synchronises operator by operator.
+ * A replay runs the same kernels in the same order on the same buffers as mnvh_net_step
+ * with the recorded lr and then copies the new parameters over the old ones, so results
+ * are bit-identical to eager steps.  While the recording exists, mnvh_net_load_batch and
+ * mnvh_net_set_param overwrite the resident buffers in place, mnvh_net_step is refused,
+ * and "prob" / "g_<param>" hold the values of the latest replay.  A network with dropout
+ * is refused (its masks come from seeds drawn on the host in every step). */
+int mnvh_net_capture_step(void* net, float lr, size_t* num_nodes /* may be NULL */);
+/* Replays the recording `steps` times; sync_each_step != 0 waits after every replay,
+ * otherwise only after the last. */
+int mnvh_net_replay(void* net, int steps, int sync_each_step);
+int mnvh_net_release_graph(void* net);
 
 #ifdef __cplusplus
 }

@@ -43,6 +43,11 @@ PROTOTYPES = {
     "mnv_event_record": [_P, _S],
     "mnv_event_sync": [_P],
     "mnv_event_elapsed_ms": [_P, _P, ctypes.POINTER(c_f)],
+    "mnv_graph_begin_capture": [_S],
+    "mnv_graph_end_capture": [_S, ctypes.POINTER(_P), ctypes.POINTER(c_sz)],
+    "mnv_graph_abort_capture": [_S],
+    "mnv_graph_launch": [_P, _S],
+    "mnv_graph_destroy": [_P],
     "mnv_error_string": [_I],
     "mnv_sgemm_nn_workspace_bytes": [_I, _I, _I],
     "mnv_sgemm_nn": [_P, _P, _P, _I, _I, _I, _P, c_sz, _S],

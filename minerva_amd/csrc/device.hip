@@ -136,6 +136,60 @@ int mnv_event_elapsed_ms(void* start, void* stop, float* ms) {
   return MNV_OK;
 }
 
+// ---- stream capture.  A launch-bound sequence of operators (a whole training step of a
+// small network is a few dozen short kernels) is recorded once into a HIP graph and then
+// replayed with one launch.  Only kernel launches may be recorded: the operator entry
+// points of this library issue nothing else once their one-time set-up has run, so a
+// sequence is executed once eagerly before it is captured.
+
+int mnv_graph_begin_capture(mnv_stream_t stream) {
+  if (!stream) return MNV_ERR_INVALID;  // the default stream cannot be captured
+  MNV_HIP_TRY(hipStreamBeginCapture(mnv_stream(stream), hipStreamCaptureModeGlobal));
+  return MNV_OK;
+}
+
+int mnv_graph_end_capture(mnv_stream_t stream, void** graph_exec, size_t* num_nodes) {
+  if (!stream || !graph_exec) return MNV_ERR_INVALID;
+  *graph_exec = nullptr;
+  hipGraph_t graph = nullptr;
+  MNV_HIP_TRY(hipStreamEndCapture(mnv_stream(stream), &graph));
+  if (!graph) return MNV_ERR_INVALID;
+  if (num_nodes) {
+    hipError_t e = hipGraphGetNodes(graph, nullptr, num_nodes);
+    if (e != hipSuccess) {
+      hipGraphDestroy(graph);
+      return (int)e;
+    }
+  }
+  hipGraphExec_t exec = nullptr;
+  hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  hipGraphDestroy(graph);
+  if (e != hipSuccess) return (int)e;
+  *graph_exec = reinterpret_cast<void*>(exec);
+  return MNV_OK;
+}
+
+int mnv_graph_abort_capture(mnv_stream_t stream) {
+  if (!stream) return MNV_ERR_INVALID;
+  hipGraph_t graph = nullptr;
+  hipError_t e = hipStreamEndCapture(mnv_stream(stream), &graph);
+  if (graph) hipGraphDestroy(graph);
+  (void)hipGetLastError();  // an invalidated capture reports its error here; it is dropped
+  return e == hipSuccess || e == hipErrorStreamCaptureInvalidated ? MNV_OK : (int)e;
+}
+
+int mnv_graph_launch(void* graph_exec, mnv_stream_t stream) {
+  if (!graph_exec) return MNV_ERR_INVALID;
+  MNV_HIP_TRY(hipGraphLaunch(reinterpret_cast<hipGraphExec_t>(graph_exec), mnv_stream(stream)));
+  return MNV_OK;
+}
+
+int mnv_graph_destroy(void* graph_exec) {
+  if (!graph_exec) return MNV_OK;
+  MNV_HIP_TRY(hipGraphExecDestroy(reinterpret_cast<hipGraphExec_t>(graph_exec)));
+  return MNV_OK;
+}
+
 const char* mnv_error_string(int status) {
   if (status == MNV_OK) return "ok";
   if (status == MNV_ERR_INVALID) return "invalid argument (null pointer or non-positive extent)";

@@ -2,6 +2,7 @@
 #include <cstring>
 #include <string>
 
+#include "mnv_hip.h"
 #include "mnv_host.h"
 #include "nets.h"
 
@@ -15,6 +16,23 @@ struct NetHandle {
   Runner* rt;
   std::unique_ptr<Net> net;
   Tensor data, label;
+  // a recorded Step: the instantiated graph and every tensor its kernels read or write
+  void* graph = nullptr;
+  std::vector<Tensor> graph_tensors;
+  void ReleaseGraph() {
+    if (!graph) return;
+    rt->Sync();
+    mnv_graph_destroy(graph);
+    graph = nullptr;
+    graph_tensors.clear();
+    net->results.clear();
+  }
+  ~NetHandle() {
+    try {
+      ReleaseGraph();
+    } catch (...) {
+    }
+  }
 };
 
 template <class F> int Guard(F&& f) {
@@ -329,7 +347,8 @@ int mnvh_net_set_param(void* net, const char* name, const float* host, size_t fl
     MNV_CHECK(it != h->net->params.end()) << "no parameter '" << name << "'";
     Scale size = it->second->size;
     MNV_CHECK_EQ(static_cast<size_t>(size.Prod()), floats) << "size of '" << name << "'";
-    it->second = h->rt->MakeNArray(size, host);
+    if (h->graph) h->rt->Upload(it->second, host);  // the recording reads this address
+    else it->second = h->rt->MakeNArray(size, host);
   });
 }
 
@@ -357,8 +376,13 @@ int mnvh_net_load_batch(void* net, const float* data, size_t data_floats, const 
     Scale ds = h->net->DataSize(), ls = h->net->LabelSize();
     MNV_CHECK_EQ(static_cast<size_t>(ds.Prod()), data_floats) << "data size";
     MNV_CHECK_EQ(static_cast<size_t>(ls.Prod()), label_floats) << "label size";
-    h->data = h->rt->MakeNArray(ds, data);
-    h->label = h->rt->MakeNArray(ls, label);
+    if (h->graph) {  // the recording reads these addresses
+      h->rt->Upload(h->data, data);
+      h->rt->Upload(h->label, label);
+    } else {
+      h->data = h->rt->MakeNArray(ds, data);
+      h->label = h->rt->MakeNArray(ls, label);
+    }
   });
 }
 
@@ -366,8 +390,69 @@ int mnvh_net_step(void* net, float lr) {
   return Guard([&] {
     NetHandle* h = static_cast<NetHandle*>(net);
     MNV_CHECK(h->data && h->label) << "load a batch first";
+    MNV_CHECK(!h->graph) << "the step is recorded: replay it or release the recording first";
     h->net->Step(h->data, h->label, lr);
   });
+}
+
+int mnvh_net_capture_step(void* net, float lr, size_t* num_nodes) {
+  return Guard([&] {
+    NetHandle* h = static_cast<NetHandle*>(net);
+    MNV_CHECK(h->data && h->label) << "load a batch first";
+    MNV_CHECK(!h->graph) << "the step is already recorded";
+    MNV_CHECK(h->net->Capturable()) << "this network draws random seeds on the host in every "
+                                    << "step; a recording would repeat them";
+    Runner* rt = h->rt;
+    Net& n = *h->net;
+    const std::map<std::string, Tensor> saved = n.params;
+    auto pass = [&](bool record) {
+      rt->BeginRetain();
+      try {
+        if (record) rt->device().BeginCapture();
+        n.Step(h->data, h->label, lr);
+        // The step leaves the new parameters in new tensors; a replay must find them
+        // where it reads them, so they are copied back over the old ones.
+        if (record)
+          for (auto& name : n.param_names) rt->CopyInto(saved.at(name), n.params[name]);
+        n.params = saved;
+        if (record) {
+          h->graph = rt->device().EndCapture(num_nodes);
+          h->graph_tensors = rt->EndRetain();
+        } else {
+          rt->Sync();
+          n.results.clear();
+          rt->EndRetain();  // every block of the step goes back to the pool's free lists
+        }
+      } catch (...) {
+        rt->device().AbortCapture();
+        n.params = saved;
+        n.results.clear();
+        rt->EndRetain();
+        throw;
+      }
+    };
+    // First an eager pass that changes nothing (the new parameters are dropped): it runs
+    // the kernels' one-time set-up and leaves one cached block per tensor of the step, so
+    // that the recording pass allocates nothing.
+    pass(false);
+    pass(true);
+  });
+}
+
+int mnvh_net_replay(void* net, int steps, int sync_each_step) {
+  return Guard([&] {
+    NetHandle* h = static_cast<NetHandle*>(net);
+    MNV_CHECK(h->graph) << "record a step first";
+    for (int i = 0; i < steps; ++i) {
+      h->rt->device().LaunchGraph(h->graph);
+      if (sync_each_step) h->rt->Sync();
+    }
+    h->rt->Sync();
+  });
+}
+
+int mnvh_net_release_graph(void* net) {
+  return Guard([&] { static_cast<NetHandle*>(net)->ReleaseGraph(); });
 }
 
 }  // extern "C"

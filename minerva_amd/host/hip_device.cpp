@@ -98,6 +98,8 @@ HipDevice::HipDevice(uint64_t device_id, DeviceListener* listener, int gpu_id, s
   for (size_t i = 0; i < kParallelism; ++i) Ok(mnv_stream_create(&streams_[i]), "stream create");
   auto allocator = [this](size_t len) -> void* {
     void* p = nullptr;
+    MNV_CHECK(!capturing_) << "a block of " << len << " bytes is not cached: device memory "
+                           << "cannot be allocated while a graph is recorded";
     Activate();
     Ok(mnv_malloc(&p, len), "device malloc");
     return p;
@@ -255,19 +257,20 @@ void HipDevice::DoExecute(const DataList& in, const DataList& out, PhysicalOp& o
   ctx.workspace = workspace_[thrid];
   ctx.workspace_bytes = workspace_bytes_[thrid];
   Timed t{std::string(), nullptr, nullptr};
-  if (profile_) {
+  const bool timed = profile_ && !capturing_;
+  if (timed) {
     t.name = op.compute_fn->Name();
     Ok(mnv_event_create(&t.start), "event create");
     Ok(mnv_event_create(&t.stop), "event create");
     Ok(mnv_event_record(t.start, streams_[thrid]), "event record");
   }
   op.compute_fn->Execute(in, out, ctx);
-  if (profile_) {
+  if (timed) {
     Ok(mnv_event_record(t.stop, streams_[thrid]), "event record");
     std::lock_guard<std::mutex> lck(prof_mutex_);
     timed_.push_back(t);
   }
-  if (sync_each_op_) {
+  if (sync_each_op_ && !capturing_) {
     int rc = mnv_stream_sync(streams_[thrid]);
     MNV_CHECK(rc == MNV_OK) << op.compute_fn->Name() << ": " << mnv_error_string(rc);
   }
@@ -294,13 +297,63 @@ std::map<std::string, std::pair<int, double>> HipDevice::CollectProfile() {
   return out;
 }
 
-void HipDevice::Barrier(int thrid) { Ok(mnv_stream_sync(streams_[thrid]), "barrier"); }
+void HipDevice::BeginCapture() {
+  MNV_CHECK(!capturing_) << "a graph is already being recorded";
+  WaitForAllFinished();
+  Activate();
+  EnsureWorkspace(0, kWorkspaceBytes);
+  for (size_t i = 0; i < kParallelism; ++i) Ok(mnv_stream_sync(streams_[i]), "capture sync");
+  Ok(mnv_graph_begin_capture(streams_[0]), "begin capture");
+  capturing_ = true;
+}
+
+void* HipDevice::EndCapture(size_t* num_nodes) {
+  MNV_CHECK(capturing_) << "no graph is being recorded";
+  capturing_ = false;
+  void* exec = nullptr;
+  int rc = mnv_graph_end_capture(streams_[0], &exec, num_nodes);
+  if (rc != MNV_OK) mnv_graph_abort_capture(streams_[0]);
+  Ok(rc, "end capture");
+  return exec;
+}
+
+void HipDevice::AbortCapture() {
+  if (!capturing_) return;
+  capturing_ = false;
+  mnv_graph_abort_capture(streams_[0]);
+}
+
+void HipDevice::LaunchGraph(void* graph_exec) {
+  MNV_CHECK(!capturing_) << "a graph cannot be replayed while another is recorded";
+  Activate();
+  Ok(mnv_graph_launch(graph_exec, streams_[0]), "graph launch");
+}
+
+void HipDevice::Barrier(int thrid) {
+  MNV_CHECK(!capturing_) << "no synchronisation while a graph is recorded";
+  Ok(mnv_stream_sync(streams_[thrid]), "barrier");
+}
 
 void HipDevice::CopyToHost(float* dst, uint64_t data_id, size_t floats) {
+  MNV_CHECK(!capturing_) << "no host copies while a graph is recorded";
   Activate();
   Ok(mnv_memcpy_d2h(dst, data_store_->GetData(data_id), floats * sizeof(float), streams_[0]),
      "copy to host");
   Ok(mnv_stream_sync(streams_[0]), "copy to host sync");
+}
+
+void HipDevice::CopyFromHost(uint64_t data_id, const float* src, size_t floats) {
+  MNV_CHECK(!capturing_) << "no host copies while a graph is recorded";
+  Activate();
+  Ok(mnv_memcpy_h2d(data_store_->GetData(data_id), src, floats * sizeof(float), streams_[0]),
+     "copy from host");
+  Ok(mnv_stream_sync(streams_[0]), "copy from host sync");
+}
+
+void HipDevice::CopyOnDevice(uint64_t dst_id, uint64_t src_id, size_t floats) {
+  Activate();
+  Ok(mnv_copy(data_store_->GetData(src_id), data_store_->GetData(dst_id), floats, streams_[0]),
+     "device copy");
 }
 
 }  // namespace minerva

@@ -114,6 +114,10 @@ class HipDevice {
   PooledDataStore& data_store() { return *data_store_; }
   // Host <-> device copies on worker stream 0, synchronised.
   void CopyToHost(float* dst, uint64_t data_id, size_t floats);
+  // Overwrites existing data in place (its address does not change).
+  void CopyFromHost(uint64_t data_id, const float* src, size_t floats);
+  // dst <- src on worker stream 0, left in flight (a kernel, so it can be recorded).
+  void CopyOnDevice(uint64_t dst_id, uint64_t src_id, size_t floats);
   // First error raised by an operator on a pool thread (empty if none).
   std::string TakeAsyncError();
 
@@ -123,6 +127,18 @@ class HipDevice {
   // name -> (launch count, total device milliseconds), then clears the record.
   void set_profile(bool v) { profile_ = v; }
   std::map<std::string, std::pair<int, double>> CollectProfile();
+
+  // Records the light tasks pushed between Begin and End (they run on worker stream 0)
+  // into a HIP graph instead of executing them.  While recording, operators are neither
+  // synchronised nor timed, and the data store may only hand out cached blocks: a device
+  // allocation cannot be recorded, so the caller runs the same task sequence once before
+  // and keeps its blocks cached.  EndCapture returns the instantiated graph;
+  // AbortCapture discards a recording that failed.  LaunchGraph replays on stream 0.
+  void BeginCapture();
+  void* EndCapture(size_t* num_nodes);
+  void AbortCapture();
+  bool capturing() const { return capturing_; }
+  void LaunchGraph(void* graph_exec);
 
  private:
   void Execute(Task* task, int thrid);
@@ -135,6 +151,7 @@ class HipDevice {
   DeviceListener* listener_;
   int gpu_id_;
   bool sync_each_op_ = true;
+  bool capturing_ = false;
   std::array<void*, kParallelism> streams_{};
   std::array<void*, kParallelism> workspace_{};
   std::array<size_t, kParallelism> workspace_bytes_{};

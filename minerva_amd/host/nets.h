@@ -21,6 +21,9 @@ class Net {
   virtual Scale DataSize() const = 0;
   virtual Scale LabelSize() const = 0;
   int batch() const { return batch_; }
+  // Whether replaying a recording of one Step equals calling Step again.  Not so when the
+  // step draws fresh random seeds on the host (dropout): a recording would repeat them.
+  virtual bool Capturable() const { return true; }
 
   std::vector<std::string> param_names;   // "w0", "b0", ...
   std::map<std::string, Tensor> params;   // current parameters
@@ -66,6 +69,7 @@ class AlexNet : public Net {
   void Step(const Tensor& data, const Tensor& label, float lr) override;
   Scale DataSize() const override { return Scale{227, 227, 3, batch_}; }
   Scale LabelSize() const override { return Scale{classes_, batch_}; }
+  bool Capturable() const override { return dropout_rate_ == 0.f; }
 
  private:
   int classes_;

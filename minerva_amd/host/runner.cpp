@@ -31,7 +31,31 @@ Tensor Runner::Compute(const std::vector<Tensor>& inputs, const Scale& out_size,
   task.id = ops_issued_++;
   task.light = true;  // sequential: run on the caller's thread, worker stream 0
   device_->PushTask(&task);
+  if (retain_) retained_.push_back(out);
   return out;
+}
+
+void Runner::Upload(const Tensor& t, const float* host) {
+  MNV_CHECK(t && host) << "null argument";
+  device_->Barrier(0);
+  device_->CopyFromHost(t->id, host, t->size.Prod());
+}
+
+void Runner::CopyInto(const Tensor& dst, const Tensor& src) {
+  MNV_CHECK(dst && src && dst->size == src->size) << "extents differ";
+  device_->CopyOnDevice(dst->id, src->id, src->size.Prod());
+}
+
+void Runner::BeginRetain() {
+  MNV_CHECK(!retain_) << "already retaining";
+  retain_ = true;
+}
+
+std::vector<Tensor> Runner::EndRetain() {
+  retain_ = false;
+  std::vector<Tensor> kept;
+  kept.swap(retained_);
+  return kept;
 }
 
 std::vector<float> Runner::Get(const Tensor& t) {

@@ -39,6 +39,16 @@ class Runner : public DeviceListener {
   Tensor Compute(const std::vector<Tensor>& inputs, const Scale& out_size,
                  std::shared_ptr<ComputeFn> fn);
   std::vector<float> Get(const Tensor& t);
+  // Overwrites a tensor's device data in place (synchronous); its address is kept, which
+  // is what a recorded graph that reads it needs.
+  void Upload(const Tensor& t, const float* host);
+  // dst <- src, both alive, same extent; ordered after everything issued so far.
+  void CopyInto(const Tensor& dst, const Tensor& src);
+  // While retaining, every tensor Compute creates is kept alive by the runner, so no
+  // device block is released or reused; EndRetain hands the kept tensors to the caller.
+  // A recorded graph owns them for as long as it may be replayed.
+  void BeginRetain();
+  std::vector<Tensor> EndRetain();
 
   // data generators
   Tensor MakeNArray(const Scale& size, std::shared_ptr<float> host);
@@ -104,6 +114,8 @@ class Runner : public DeviceListener {
   std::unique_ptr<HipDevice> device_;
   std::atomic<uint64_t> next_id_{1};
   std::atomic<uint64_t> ops_issued_{0}, ops_completed_{0};
+  bool retain_ = false;
+  std::vector<Tensor> retained_;
 };
 
 }  // namespace minerva

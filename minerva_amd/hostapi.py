@@ -164,3 +164,16 @@ class Net:
 
     def step(self, lr):
         _check(lib().mnvh_net_step(self.h, ctypes.c_float(lr)), "net_step")
+
+    def capture_step(self, lr):
+        """Records one step into a HIP graph; returns the number of graph nodes."""
+        n = ctypes.c_size_t()
+        _check(lib().mnvh_net_capture_step(self.h, ctypes.c_float(lr), ctypes.byref(n)),
+               "net_capture_step")
+        return n.value
+
+    def replay(self, steps=1, sync_each_step=True):
+        _check(lib().mnvh_net_replay(self.h, int(steps), 1 if sync_each_step else 0), "net_replay")
+
+    def release_graph(self):
+        _check(lib().mnvh_net_release_graph(self.h), "net_release_graph")
