@@ -545,17 +545,22 @@ int permute_filter(const float* in, float* out, int K, int C, int RS, bool to_cr
 typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
 typedef MnvGemmTile<128, 128, 16, 4, 1, 0, 96> Tile96;  // four wavefronts of 32 x 96
+// Four wavefronts of 32 x 32 for outputs of at most 32 columns (a convolution with few
+// output channels): a 64-column tile would spend half or more of its multiplies on padding.
+// 64 columns are staged because a slab of 32 would not give every thread a vector to fetch.
+typedef MnvGemmTile<128, 64, 16, 4, 1, 0, 32> TileThin;
 
-// tile 0: 64x64 output tiles, tile 1: 128x128, tile 2: 128x96
+// tile 0: 64x64 output tiles, tile 1: 128x128, tile 2: 128x96, tile 3: 128x32
 template <class P>
 int launch_tile(int tile, const P& p, int splits, void* ws, hipStream_t s) {
   switch (tile) {
     case 0: return mnv_gemm_launch<TileSmall>(p, splits, ws, s);
     case 2: return mnv_gemm_launch<Tile96>(p, splits, ws, s);
+    case 3: return mnv_gemm_launch<TileThin>(p, splits, ws, s);
     default: return mnv_gemm_launch<TileBig>(p, splits, ws, s);
   }
 }
-const int kTileM[3] = {64, 128, 128}, kTileN[3] = {64, 128, 96};
+const int kTileM[4] = {64, 128, 128, 128}, kTileN[4] = {64, 128, 96, 32};
 
 // 128-row tiles: 96 columns wide when that leaves clearly fewer idle columns than 128
 // (an output 96 or 192 wide), since the narrower tile does a little less work per byte
@@ -593,16 +598,41 @@ int make_geom(ConvGeom* g, int N, int C, int K, int H, int W, int ph, int pw, in
 }
 
 int pick_tile(int m, int n) {
+  if (n <= 32) return 3;
   long long big = (long long)((m + 127) / 128) * ((n + 127) / 128);
   if (big < 128 || m <= 64 || n <= 64) return 0;
   return wide_tile(n);
 }
 
+// A 64x64 or 128x32 tile does little arithmetic per k-slab, so a slab costs one trip to
+// memory and back; its kernels need about 64 registers and at most 24 KB of LDS, which
+// lets a CU hold six to eight workgroups whose trips overlap.  When the output has fewer tiles than that, the
+// reduction is cut into k ranges (at least six slabs each) until about 2048 workgroups
+// are in flight.  `ws_floats`: workspace left for the partial results.
+int small_tile_splits(int tile, int m, int n, int slabs, size_t ws_floats) {
+  if (tile != 0 && tile != 3) return 1;
+  const int bm = kTileM[tile], bn = kTileN[tile];
+  long long tiles = (long long)((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+  if (tiles >= 1536) return 1;
+  long long want = (2048 + tiles - 1) / tiles;
+  if (want > slabs / 6) want = slabs / 6;
+  size_t fit = ws_floats / ((size_t)m * n);
+  if ((size_t)want > fit) want = (long long)fit;
+  return want < 2 ? 1 : (int)want;
+}
+
+// Workspace layout of the forward and data-gradient convolutions: the permuted filter
+// (when the fast policy applies) first, then, 256-byte aligned, the partial results.
+size_t align256(size_t bytes) { return (bytes + 255) & ~(size_t)255; }
+
 #define MNV_BWDF_MAX_SPLITS 256
 
 // The filter gradient gets its parallelism from splitting the long N*Ho*Wo reduction,
 // so it keeps the 128x128 tile (twice the operand reuse) unless the output is tiny.
-int bwd_filter_tile(int m, int n) { return (m <= 64 || n <= 64) ? 0 : wide_tile(n); }
+int bwd_filter_tile(int m, int n) {
+  if (n <= 32) return 3;
+  return (m <= 64 || n <= 64) ? 0 : wide_tile(n);
+}
 
 int bwd_filter_splits(int m, int n, int k, size_t ws_floats) {
   const int tile = bwd_filter_tile(m, n);
@@ -624,7 +654,10 @@ size_t mnv_conv_fwd_workspace_bytes(int N, int C, int K, int H, int W, int ph, i
                                    int sh, int R, int S) {
   ConvGeom g;
   if (make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S)) return 0;
-  return C % 16 == 0 ? (size_t)K * g.CRS * sizeof(float) : 0;
+  const size_t permuted = C % 16 == 0 ? (size_t)K * g.CRS * sizeof(float) : 0;
+  const int gm = N * g.HoWo, gn = K;
+  const int splits = small_tile_splits(pick_tile(gm, gn), gm, gn, (g.CRS + 15) / 16, (size_t)-1);
+  return splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
 }
 
 int mnv_conv_fwd(const float* bottom, const float* filter, const float* bias, float* top, int N,
@@ -637,26 +670,40 @@ int mnv_conv_fwd(const float* bottom, const float* filter, const float* bias, fl
   int gm = N * g.HoWo, gn = K, gk = g.CRS;
   hipStream_t s = mnv_stream(stream);
   const int tile = pick_tile(gm, gn);
-  if (C % 16 == 0 && workspace && workspace_bytes >= (size_t)K * g.CRS * sizeof(float)) {
+  const size_t permuted_bytes = (size_t)K * g.CRS * sizeof(float);
+  // the no-padding policy reads the filter where it is; for a small problem the extra
+  // launch that permutes the filter for the fast policy would cost more than it gains
+  const bool np = ph == 0 && pw == 0 && gk <= 4096;
+  const bool fast = C % 16 == 0 && workspace && workspace_bytes >= permuted_bytes &&
+                    !(np && (tile == 0 || tile == 3));
+  // what is left of the workspace after the permuted filter holds the partial results
+  const size_t used = fast ? align256(permuted_bytes) : 0;
+  float* part = workspace && workspace_bytes > used ? reinterpret_cast<float*>(static_cast<char*>(workspace) + used) : nullptr;
+  const int splits = small_tile_splits(tile, gm, gn, (gk + 15) / 16,
+                                       part ? (workspace_bytes - used) / sizeof(float) : 0);
+  if (fast) {
     float* wp = static_cast<float*>(workspace);
     rc = permute_filter(filter, wp, K, C, g.RS, false, s);
     if (rc) return rc;
     ConvFwd<true> p{bottom, wp, bias, top, g, gm, gn, gk, g.RS * (C / 16), C / 16};
-    return launch_tile(tile, p, 1, nullptr, s);
+    return launch_tile(tile, p, splits, part, s);
   }
-  if (ph == 0 && pw == 0 && gk <= 4096) {
+  if (np) {
     ConvFwdNP p{bottom, filter, bias, top, g, gm, gn, gk, (gk + 15) / 16, gk >= 16 ? gk / 16 : 1};
-    return launch_tile(tile, p, 1, nullptr, s);
+    return launch_tile(tile, p, splits, part, s);
   }
   ConvFwd<false> p{bottom, filter, bias, top, g, gm, gn, gk, (gk + 15) / 16, 1};
-  return launch_tile(tile, p, 1, nullptr, s);
+  return launch_tile(tile, p, splits, part, s);
 }
 
 size_t mnv_conv_bwd_data_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw,
                                         int sv, int sh, int R, int S) {
   ConvGeom g;
   if (make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S)) return 0;
-  return (sv == 1 && sh == 1 && K % 16 == 0) ? (size_t)K * g.CRS * sizeof(float) : 0;
+  const size_t permuted = (sv == 1 && sh == 1 && K % 16 == 0) ? (size_t)K * g.CRS * sizeof(float) : 0;
+  const int gm = N * g.HW, gn = C;
+  const int splits = small_tile_splits(pick_tile(gm, gn), gm, gn, (K * g.RS + 15) / 16, (size_t)-1);
+  return splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
 }
 
 int mnv_conv_bwd_data(const float* top_diff, const float* filter, float* bottom_diff, int N,
@@ -669,16 +716,21 @@ int mnv_conv_bwd_data(const float* top_diff, const float* filter, float* bottom_
   int gm = N * g.HW, gn = C, gk = K * g.RS;
   hipStream_t s = mnv_stream(stream);
   const int tile = pick_tile(gm, gn);
-  if (sv == 1 && sh == 1 && K % 16 == 0 && workspace &&
-      workspace_bytes >= (size_t)K * g.CRS * sizeof(float)) {
+  const size_t permuted_bytes = (size_t)K * g.CRS * sizeof(float);
+  const bool fast = sv == 1 && sh == 1 && K % 16 == 0 && workspace && workspace_bytes >= permuted_bytes;
+  const size_t used = fast ? align256(permuted_bytes) : 0;
+  float* part = workspace && workspace_bytes > used ? reinterpret_cast<float*>(static_cast<char*>(workspace) + used) : nullptr;
+  const int splits = small_tile_splits(tile, gm, gn, (gk + 15) / 16,
+                                       part ? (workspace_bytes - used) / sizeof(float) : 0);
+  if (fast) {
     float* wq = static_cast<float*>(workspace);
     rc = permute_filter(filter, wq, K, C, g.RS, true, s);
     if (rc) return rc;
     ConvBwdData<true> p{top_diff, wq, bottom_diff, g, gm, gn, gk, g.RS * (K / 16), K / 16};
-    return launch_tile(tile, p, 1, nullptr, s);
+    return launch_tile(tile, p, splits, part, s);
   }
   ConvBwdData<false> p{top_diff, filter, bottom_diff, g, gm, gn, gk, (gk + 15) / 16, 1};
-  return launch_tile(tile, p, 1, nullptr, s);
+  return launch_tile(tile, p, splits, part, s);
 }
 
 size_t mnv_conv_bwd_filter_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw,

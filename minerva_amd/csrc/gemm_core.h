@@ -283,18 +283,59 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
   }
 }
 
-// Sums the per-split partial results in split order (deterministic) and hands each
-// element to the policy's store.
-template <class P>
+// Sums the per-split partial results in a fixed order (deterministic) and hands each
+// element to the policy's store.  ZL threads share one output element: thread z of them
+// adds the partial results z, z + ZL, z + 2 ZL, ... and the ZL sums are added in order
+// through LDS.  A small output with many k ranges (the filter gradient of a narrow
+// convolution: a few hundred elements, hundreds of ranges) would otherwise leave the chip
+// to a few hundred threads that each walk the whole list.
+template <class P, int ZL>
 __global__ __launch_bounds__(256) void mnv_gemm_splitk_reduce_kernel(P prob,
                                                                     const float* __restrict__ partial,
                                                                     int splits) {
+  constexpr int QL = 256 / ZL;  // output elements per workgroup pass
+  __shared__ float red[ZL > 1 ? 256 : 1];
   const size_t mn = (size_t)prob.M * prob.N;
-  for (size_t q = (size_t)blockIdx.x * 256 + threadIdx.x; q < mn; q += (size_t)gridDim.x * 256) {
-    float s = partial[q];
-    for (int z = 1; z < splits; ++z) s += partial[(size_t)z * mn + q];
-    prob.c_store((int)(q % prob.M), (int)(q / prob.M), s);
+  const int tq = threadIdx.x % QL, tz = threadIdx.x / QL;
+  for (size_t q0 = (size_t)blockIdx.x * QL; q0 < mn; q0 += (size_t)gridDim.x * QL) {
+    const size_t q = q0 + tq;
+    float s = 0.f;
+    if (q < mn) {
+      const float* p = partial + q + (size_t)tz * mn;
+      const size_t step = (size_t)ZL * mn;
+      int z = tz;
+      float v0, v1, v2, v3;
+      for (; z + 3 * ZL < splits; z += 4 * ZL, p += 4 * step) {
+        v0 = p[0]; v1 = p[step]; v2 = p[2 * step]; v3 = p[3 * step];
+        s += v0; s += v1; s += v2; s += v3;
+      }
+      for (; z < splits; z += ZL, p += step) s += *p;
+    }
+    if (ZL == 1) {
+      if (q < mn) prob.c_store((int)(q % prob.M), (int)(q / prob.M), s);
+    } else {
+      __syncthreads();  // the previous pass has read its sums
+      red[threadIdx.x] = s;
+      __syncthreads();
+      if (tz == 0 && q < mn) {
+        float t = red[tq];
+#pragma unroll
+        for (int z = 1; z < ZL; ++z) t += red[z * QL + tq];
+        prob.c_store((int)(q % prob.M), (int)(q / prob.M), t);
+      }
+    }
   }
+}
+
+template <class P, int ZL>
+static int mnv_gemm_splitk_reduce_launch(const P& prob, const float* partial, int splits,
+                                         hipStream_t s) {
+  const size_t mn = (size_t)prob.M * prob.N;
+  size_t blocks = mnv_ceil_div(mn, 256 / ZL);
+  if (blocks > MNV_MAX_STREAM_BLOCKS) blocks = MNV_MAX_STREAM_BLOCKS;
+  hipLaunchKernelGGL((mnv_gemm_splitk_reduce_kernel<P, ZL>), dim3((unsigned)blocks), dim3(256), 0,
+                     s, prob, partial, splits);
+  return MNV_LAUNCH_STATUS();
 }
 
 // Number of k ranges for `tiles` output tiles of `slabs` k-slabs each.  Workgroups are
@@ -352,12 +393,14 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
   int rc = MNV_LAUNCH_STATUS();
   if (rc) return rc;
   if (splits > 1) {
-    size_t mn = (size_t)prob.M * prob.N;
-    size_t blocks = mnv_ceil_div(mn, 256);
-    if (blocks > MNV_MAX_STREAM_BLOCKS) blocks = MNV_MAX_STREAM_BLOCKS;
-    hipLaunchKernelGGL((mnv_gemm_splitk_reduce_kernel<P>), dim3((unsigned)blocks), dim3(256), 0, s,
-                       prob, reinterpret_cast<const float*>(workspace), splits);
-    rc = MNV_LAUNCH_STATUS();
+    // enough threads to cover the chip: one per element for a large output, up to 64 per
+    // element (never more than half the ranges) for a small one
+    const size_t mn = (size_t)prob.M * prob.N;
+    const float* part = reinterpret_cast<const float*>(workspace);
+    if (mn >= 65536 || splits < 8) rc = mnv_gemm_splitk_reduce_launch<P, 1>(prob, part, splits, s);
+    else if (mn >= 16384 || splits < 32) rc = mnv_gemm_splitk_reduce_launch<P, 4>(prob, part, splits, s);
+    else if (mn >= 4096 || splits < 128) rc = mnv_gemm_splitk_reduce_launch<P, 16>(prob, part, splits, s);
+    else rc = mnv_gemm_splitk_reduce_launch<P, 64>(prob, part, splits, s);
   }
   return rc;
 }

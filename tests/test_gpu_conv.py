@@ -116,6 +116,8 @@ CASES = [
     (8, 96, 16, 48, 48, 1, 1, 1, 1, 3, 3),  # 96 input channels: the same for the data gradient
     (4, 64, 96, 20, 20, 1, 1, 1, 1, 3, 3),  # 96-column tiles in the table-driven filter gradient
     (8, 4, 192, 46, 46, 0, 0, 1, 1, 3, 3),  # two 96-column tiles, channel-major reduction order
+    (3, 20, 17, 13, 13, 1, 1, 1, 1, 3, 3),  # <= 32 channels either way: 128x32 tiles, ragged rows,
+    (2, 24, 33, 15, 14, 0, 0, 1, 1, 4, 4),  #   and a reduction cut into k ranges on small tiles
 ]
 
 
