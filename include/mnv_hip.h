@@ -58,6 +58,12 @@ int mnv_memcpy_d2h(void* dst_host, const void* src, size_t bytes, mnv_stream_t s
 int mnv_memcpy_d2d(void* dst, const void* src, size_t bytes, mnv_stream_t stream);
 /* Events for timing on the stream the kernels run on. */
 int mnv_event_create(void** event);
+/* An event that carries no time stamp, for ordering only, and the wait that makes every
+ * later call on `stream` start after the work recorded before `event`: what replaces the
+ * reference's cudaStreamSynchronize after every operator (minerva/device/device.cpp:221)
+ * when operators on different streams depend on each other. */
+int mnv_event_create_ordering(void** event);
+int mnv_stream_wait_event(mnv_stream_t stream, void* event);
 int mnv_event_destroy(void* event);
 int mnv_event_record(void* event, mnv_stream_t stream);
 int mnv_event_sync(void* event);

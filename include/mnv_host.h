@@ -34,19 +34,37 @@ typedef struct {
 
 const char* mnvh_last_error(void);
 
-/* sync_each_op != 0: synchronise the stream after every operator, as the reference
- * device does (minerva/device/device.cpp:221); 0: operators stay in flight and the
- * caller synchronises with mnvh_runtime_sync. */
+/* sync_each_op: 1 = synchronise the stream after every operator, as the reference device
+ * does (minerva/device/device.cpp:221); 0 = operators stay in flight on one stream in
+ * program order and the caller synchronises with mnvh_runtime_sync; 2 = dataflow: operators
+ * stay in flight on the device's four streams (a chain of dependent operators shares a
+ * stream, independent chains get different ones), every output carries an event recorded
+ * behind its producer and a consumer on another stream waits for it on the GPU -- what the
+ * reference's scheduler achieves by waiting on the host after every operator.  Results are
+ * bit-identical in all three modes. */
 int mnvh_runtime_create(int gpu_id, int sync_each_op, void** runtime);
+/* The same with the pooled allocator's threshold (default 200 GiB): when the bytes held
+ * exceed it, every cached block is released (minerva/device/pooled_data_store.cpp:27-33);
+ * in dataflow mode a stream recycles blocks that other streams still use (and waits for
+ * them) once the pool holds half of it, instead of allocating. */
+int mnvh_runtime_create_pool(int gpu_id, int sync_each_op, size_t pool_bytes, void** runtime);
 int mnvh_runtime_destroy(void* runtime);
 int mnvh_runtime_sync(void* runtime);
 int mnvh_runtime_ops_issued(void* runtime, unsigned long long* count);
 int mnvh_runtime_pool_stats(void* runtime, size_t* total_bytes, size_t* cached_blocks);
+/* Dataflow mode, since the runtime was created: how often a consumer's stream was made to
+ * wait for a producer on another stream, and how often a stream was made to wait for other
+ * streams before it reused a recycled block. */
+int mnvh_runtime_dataflow_stats(void* runtime, unsigned long long* producer_waits,
+                                unsigned long long* recycle_waits);
 
 /* Per-operator device timing (two events per operator on its own stream).  The read
  * synchronises, writes one "name<TAB>launches<TAB>total_ms" line per operator name and
  * clears the record. */
 int mnvh_runtime_profile(void* runtime, int enable);
+/* Times only the operators whose name contains name_part (NULL or "": all).  The events
+ * cost a few microseconds of idle GPU each; a step timed with all of them runs ~5% slower. */
+int mnvh_runtime_profile_filter(void* runtime, const char* name_part);
 int mnvh_runtime_profile_read(void* runtime, char* text_out, size_t capacity);
 
 /*
@@ -76,6 +94,17 @@ int mnvh_runtime_profile_read(void* runtime, char* text_out, size_t capacity);
 int mnvh_op(void* runtime, const char* op, const mnvh_tensor* inputs, int n_inputs,
             const double* params, int n_params, float* out, size_t out_capacity,
             int* out_ndims, int* out_dims);
+
+/* Device-resident tensors, for graphs of operators that do not go through host memory
+ * between operators.  `op` / `params` as for mnvh_op; a tensor is freed (its block goes back
+ * to the device's pool) by mnvh_tensor_free even while operators that use it are queued.
+ * mnvh_tensor_info reports the extent and the worker stream the producer was placed on. */
+int mnvh_tensor_create(void* runtime, const mnvh_tensor* host, void** tensor);
+int mnvh_tensor_op(void* runtime, const char* op, void* const* inputs, int n_inputs,
+                   const double* params, int n_params, void** out);
+int mnvh_tensor_info(void* tensor, int* ndims, int* dims /* MNVH_MAX_DIMS */, int* stream);
+int mnvh_tensor_read(void* runtime, void* tensor, float* out, size_t out_capacity);
+int mnvh_tensor_free(void* tensor);
 
 /* Restarts the sequence the seeds of the "randn" / "rand_bernoulli" operators are drawn from. */
 int mnvh_set_random_seed(unsigned long long seed);

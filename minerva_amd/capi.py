@@ -39,6 +39,8 @@ PROTOTYPES = {
     "mnv_memcpy_d2h": [_P, _P, c_sz, _S],
     "mnv_memcpy_d2d": [_P, _P, c_sz, _S],
     "mnv_event_create": [ctypes.POINTER(c_p)],
+    "mnv_event_create_ordering": [ctypes.POINTER(_P)],
+    "mnv_stream_wait_event": [_S, _P],
     "mnv_event_destroy": [_P],
     "mnv_event_record": [_P, _S],
     "mnv_event_sync": [_P],

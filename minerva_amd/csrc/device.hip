@@ -111,6 +111,20 @@ int mnv_event_create(void** event) {
   return MNV_OK;
 }
 
+int mnv_event_create_ordering(void** event) {
+  if (!event) return MNV_ERR_INVALID;
+  hipEvent_t e;
+  MNV_HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  *event = reinterpret_cast<void*>(e);
+  return MNV_OK;
+}
+
+int mnv_stream_wait_event(mnv_stream_t stream, void* event) {
+  if (!event) return MNV_ERR_INVALID;
+  MNV_HIP_TRY(hipStreamWaitEvent(mnv_stream(stream), reinterpret_cast<hipEvent_t>(event), 0));
+  return MNV_OK;
+}
+
 int mnv_event_destroy(void* event) {
   if (!event) return MNV_ERR_INVALID;
   MNV_HIP_TRY(hipEventDestroy(reinterpret_cast<hipEvent_t>(event)));

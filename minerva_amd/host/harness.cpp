@@ -57,6 +57,153 @@ int P(const double* p, int n, int i) {
   return static_cast<int>(p[i]);
 }
 
+// One operator by name on device tensors: the NArray call the name stands for.
+Tensor RunNamedOp(Runner* rt, const std::string& op, const std::vector<Tensor>& in,
+                  const double* params, int n_params) {
+  const int n_inputs = static_cast<int>(in.size());
+  auto need = [&](int n) { MNV_CHECK_EQ(n_inputs, n) << op << " takes " << n << " inputs"; };
+  auto conv_info = [&] {
+    return ConvInfo(P(params, n_params, 0), P(params, n_params, 1), P(params, n_params, 2),
+                    P(params, n_params, 3));
+  };
+  auto pool_info = [&] {
+    return PoolingInfo(static_cast<PoolingInfo::Algorithm>(P(params, n_params, 0)),
+                       P(params, n_params, 1), P(params, n_params, 2), P(params, n_params, 3),
+                       P(params, n_params, 4), P(params, n_params, 5), P(params, n_params, 6));
+  };
+  Tensor r;
+  if (op == "arithmetic") {
+    need(2);
+    r = rt->Arithmetic(in[0], in[1], static_cast<ArithmeticType>(P(params, n_params, 0)));
+  } else if (op == "arithmetic_const") {
+    need(1);
+    MNV_CHECK(n_params >= 3) << "arithmetic_const takes type, val, side";
+    r = rt->ArithmeticConst(in[0], static_cast<float>(params[1]),
+                            static_cast<ArithmeticType>(P(params, n_params, 0)),
+                            P(params, n_params, 2));
+  } else if (op == "elewise") {
+    need(1);
+    r = rt->Elewise(in[0], static_cast<ElewiseType>(P(params, n_params, 0)));
+  } else if (op == "norm_arithmetic") {
+    need(2);
+    r = rt->NormArithmetic(in[0], in[1], static_cast<ArithmeticType>(P(params, n_params, 0)));
+  } else if (op == "matmult") {
+    need(2);
+    r = rt->MatMult(in[0], in[1]);
+  } else if (op == "trans") {
+    need(1);
+    r = rt->Trans(in[0]);
+  } else if (op == "reshape") {
+    need(1);
+    std::vector<int> d;
+    for (int i = 0; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
+    r = rt->Reshape(in[0], Scale(d));
+  } else if (op == "reduction") {
+    need(1);
+    r = rt->Reduce(in[0], P(params, n_params, 1),
+                   static_cast<ReductionType>(P(params, n_params, 0)));
+  } else if (op == "maxindex") {
+    need(1);
+    r = rt->MaxIndex(in[0], P(params, n_params, 0));
+  } else if (op == "sigmoid_forward") {
+    need(1);
+    r = rt->SigmoidForward(in[0]);
+  } else if (op == "relu_forward") {
+    need(1);
+    r = rt->ReluForward(in[0]);
+  } else if (op == "tanh_forward") {
+    need(1);
+    r = rt->TanhForward(in[0]);
+  } else if (op == "sigmoid_backward") {
+    need(3);
+    r = rt->SigmoidBackward(in[0], in[1], in[2]);
+  } else if (op == "relu_backward") {
+    need(3);
+    r = rt->ReluBackward(in[0], in[1], in[2]);
+  } else if (op == "tanh_backward") {
+    need(3);
+    r = rt->TanhBackward(in[0], in[1], in[2]);
+  } else if (op == "activation_forward") {
+    need(1);
+    r = rt->ActivationForward(in[0], static_cast<ActivationAlgorithm>(P(params, n_params, 0)));
+  } else if (op == "activation_backward") {
+    need(3);
+    r = rt->ActivationBackward(in[0], in[1], in[2],
+                               static_cast<ActivationAlgorithm>(P(params, n_params, 0)));
+  } else if (op == "softmax_forward") {
+    need(1);
+    r = rt->SoftmaxForward(in[0], static_cast<SoftmaxAlgorithm>(P(params, n_params, 0)));
+  } else if (op == "softmax_backward") {
+    need(2);
+    r = rt->SoftmaxBackward(in[0], in[1], static_cast<SoftmaxAlgorithm>(P(params, n_params, 0)));
+  } else if (op == "conv_forward") {
+    need(3);
+    r = rt->ConvForward(in[0], in[1], in[2], conv_info());
+  } else if (op == "conv_backward_data") {
+    need(3);
+    r = rt->ConvBackwardData(in[0], in[1], in[2], conv_info());
+  } else if (op == "conv_backward_filter") {
+    need(3);
+    r = rt->ConvBackwardFilter(in[0], in[1], in[2], conv_info());
+  } else if (op == "conv_backward_bias") {
+    need(1);
+    r = rt->ConvBackwardBias(in[0]);
+  } else if (op == "pooling_forward") {
+    need(1);
+    r = rt->PoolingForward(in[0], pool_info());
+  } else if (op == "pooling_backward") {
+    need(3);
+    r = rt->PoolingBackward(in[0], in[1], in[2], pool_info());
+  } else if (op == "threshold_norm") {  // params: threshold
+    need(1);
+    MNV_CHECK(n_params >= 1) << "threshold_norm takes the threshold";
+    r = rt->ThresholdNorm(in[0], static_cast<float>(params[0]));
+  } else if (op == "index") {  // params: idx, then the extents of one block
+    need(1);
+    std::vector<int> d;
+    for (int i = 1; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
+    MNV_CHECK(!d.empty()) << "index takes idx, d0, ...";
+    r = rt->Index(in[0], P(params, n_params, 0), Scale(d));
+  } else if (op == "concat") {  // params: catdim; any number (> 1) of inputs
+    r = rt->Concat(in, P(params, n_params, 0));
+  } else if (op == "slice") {  // params: slice_dim, st_off, slice_count
+    need(1);
+    r = rt->Slice(in[0], P(params, n_params, 0), P(params, n_params, 1), P(params, n_params, 2));
+  } else if (op == "select") {  // params: the column indices
+    need(1);
+    std::vector<int> idx;
+    for (int i = 0; i < n_params; ++i) idx.push_back(static_cast<int>(params[i]));
+    r = rt->Select(in[0], idx);
+  } else if (op == "lrn_forward") {  // params: local_size, alpha, beta; inputs: bottom, scale
+    need(2);
+    MNV_CHECK(n_params >= 3) << "lrn_forward takes local_size, alpha, beta";
+    r = rt->LRNForward(in[0], in[1], static_cast<int>(params[0]), static_cast<float>(params[1]),
+                       static_cast<float>(params[2]));
+  } else if (op == "lrn_backward") {  // inputs: bottom, top, scale, top_diff
+    need(4);
+    MNV_CHECK(n_params >= 3) << "lrn_backward takes local_size, alpha, beta";
+    r = rt->LRNBackward(in[0], in[1], in[2], in[3], static_cast<int>(params[0]),
+                        static_cast<float>(params[1]), static_cast<float>(params[2]));
+  } else if (op == "randn" || op == "rand_bernoulli") {  // params: mu, var | p ; then d0, d1, ...
+    need(0);
+    const int lead = op == "randn" ? 2 : 1;
+    MNV_CHECK(n_params > lead) << op << " takes its parameters, then the extents";
+    std::vector<int> d;
+    for (int i = lead; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
+    r = op == "randn" ? rt->Randn(Scale(d), static_cast<float>(params[0]), static_cast<float>(params[1]))
+                      : rt->RandBernoulli(Scale(d), static_cast<float>(params[0]));
+  } else if (op == "fill") {
+    need(0);
+    std::vector<int> d;
+    for (int i = 1; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
+    MNV_CHECK(n_params >= 2) << "fill takes val, d0, ...";
+    r = rt->Constant(Scale(d), static_cast<float>(params[0]));
+  } else {
+    MNV_FATAL() << "unknown operator '" << op << "'";
+  }
+  return r;
+}
+
 }  // namespace
 
 extern "C" {
@@ -66,7 +213,16 @@ const char* mnvh_last_error(void) { return g_error.c_str(); }
 int mnvh_runtime_create(int gpu_id, int sync_each_op, void** runtime) {
   return Guard([&] {
     MNV_CHECK(runtime) << "null out pointer";
-    *runtime = new Runner(gpu_id, sync_each_op != 0);
+    MNV_CHECK(sync_each_op >= 0 && sync_each_op <= 2) << "mode must be 0, 1 or 2";
+    *runtime = new Runner(gpu_id, sync_each_op == 1, sync_each_op == 2);
+  });
+}
+
+int mnvh_runtime_create_pool(int gpu_id, int sync_each_op, size_t pool_bytes, void** runtime) {
+  return Guard([&] {
+    MNV_CHECK(runtime && pool_bytes > 0) << "bad argument";
+    MNV_CHECK(sync_each_op >= 0 && sync_each_op <= 2) << "mode must be 0, 1 or 2";
+    *runtime = new Runner(gpu_id, sync_each_op == 1, sync_each_op == 2, pool_bytes);
   });
 }
 
@@ -90,8 +246,23 @@ int mnvh_runtime_pool_stats(void* runtime, size_t* total_bytes, size_t* cached_b
   });
 }
 
+int mnvh_runtime_dataflow_stats(void* runtime, unsigned long long* producer_waits,
+                                unsigned long long* recycle_waits) {
+  return Guard([&] {
+    HipDevice& d = static_cast<Runner*>(runtime)->device();
+    if (producer_waits) *producer_waits = d.producer_waits();
+    if (recycle_waits) *recycle_waits = d.recycle_waits();
+  });
+}
+
 int mnvh_runtime_profile(void* runtime, int enable) {
   return Guard([&] { static_cast<Runner*>(runtime)->device().set_profile(enable != 0); });
+}
+
+int mnvh_runtime_profile_filter(void* runtime, const char* name_part) {
+  return Guard([&] {
+    static_cast<Runner*>(runtime)->device().set_profile_filter(name_part ? name_part : "");
+  });
 }
 
 int mnvh_runtime_profile_read(void* runtime, char* text_out, size_t capacity) {
@@ -111,152 +282,12 @@ int mnvh_op(void* runtime, const char* op_name, const mnvh_tensor* inputs, int n
   return Guard([&] {
     Runner* rt = static_cast<Runner*>(runtime);
     MNV_CHECK(rt && op_name && out) << "null argument";
-    std::string op(op_name);
     std::vector<Tensor> in;
     for (int i = 0; i < n_inputs; ++i) {
       MNV_CHECK(inputs[i].data) << "null input data";
       in.push_back(rt->MakeNArray(ToScale(inputs[i]), inputs[i].data));
     }
-    auto need = [&](int n) { MNV_CHECK_EQ(n_inputs, n) << op << " takes " << n << " inputs"; };
-    auto conv_info = [&] {
-      return ConvInfo(P(params, n_params, 0), P(params, n_params, 1), P(params, n_params, 2),
-                      P(params, n_params, 3));
-    };
-    auto pool_info = [&] {
-      return PoolingInfo(static_cast<PoolingInfo::Algorithm>(P(params, n_params, 0)),
-                         P(params, n_params, 1), P(params, n_params, 2), P(params, n_params, 3),
-                         P(params, n_params, 4), P(params, n_params, 5), P(params, n_params, 6));
-    };
-    Tensor r;
-    if (op == "arithmetic") {
-      need(2);
-      r = rt->Arithmetic(in[0], in[1], static_cast<ArithmeticType>(P(params, n_params, 0)));
-    } else if (op == "arithmetic_const") {
-      need(1);
-      MNV_CHECK(n_params >= 3) << "arithmetic_const takes type, val, side";
-      r = rt->ArithmeticConst(in[0], static_cast<float>(params[1]),
-                              static_cast<ArithmeticType>(P(params, n_params, 0)),
-                              P(params, n_params, 2));
-    } else if (op == "elewise") {
-      need(1);
-      r = rt->Elewise(in[0], static_cast<ElewiseType>(P(params, n_params, 0)));
-    } else if (op == "norm_arithmetic") {
-      need(2);
-      r = rt->NormArithmetic(in[0], in[1], static_cast<ArithmeticType>(P(params, n_params, 0)));
-    } else if (op == "matmult") {
-      need(2);
-      r = rt->MatMult(in[0], in[1]);
-    } else if (op == "trans") {
-      need(1);
-      r = rt->Trans(in[0]);
-    } else if (op == "reshape") {
-      need(1);
-      std::vector<int> d;
-      for (int i = 0; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
-      r = rt->Reshape(in[0], Scale(d));
-    } else if (op == "reduction") {
-      need(1);
-      r = rt->Reduce(in[0], P(params, n_params, 1),
-                     static_cast<ReductionType>(P(params, n_params, 0)));
-    } else if (op == "maxindex") {
-      need(1);
-      r = rt->MaxIndex(in[0], P(params, n_params, 0));
-    } else if (op == "sigmoid_forward") {
-      need(1);
-      r = rt->SigmoidForward(in[0]);
-    } else if (op == "relu_forward") {
-      need(1);
-      r = rt->ReluForward(in[0]);
-    } else if (op == "tanh_forward") {
-      need(1);
-      r = rt->TanhForward(in[0]);
-    } else if (op == "sigmoid_backward") {
-      need(3);
-      r = rt->SigmoidBackward(in[0], in[1], in[2]);
-    } else if (op == "relu_backward") {
-      need(3);
-      r = rt->ReluBackward(in[0], in[1], in[2]);
-    } else if (op == "tanh_backward") {
-      need(3);
-      r = rt->TanhBackward(in[0], in[1], in[2]);
-    } else if (op == "activation_forward") {
-      need(1);
-      r = rt->ActivationForward(in[0], static_cast<ActivationAlgorithm>(P(params, n_params, 0)));
-    } else if (op == "activation_backward") {
-      need(3);
-      r = rt->ActivationBackward(in[0], in[1], in[2],
-                                 static_cast<ActivationAlgorithm>(P(params, n_params, 0)));
-    } else if (op == "softmax_forward") {
-      need(1);
-      r = rt->SoftmaxForward(in[0], static_cast<SoftmaxAlgorithm>(P(params, n_params, 0)));
-    } else if (op == "softmax_backward") {
-      need(2);
-      r = rt->SoftmaxBackward(in[0], in[1], static_cast<SoftmaxAlgorithm>(P(params, n_params, 0)));
-    } else if (op == "conv_forward") {
-      need(3);
-      r = rt->ConvForward(in[0], in[1], in[2], conv_info());
-    } else if (op == "conv_backward_data") {
-      need(3);
-      r = rt->ConvBackwardData(in[0], in[1], in[2], conv_info());
-    } else if (op == "conv_backward_filter") {
-      need(3);
-      r = rt->ConvBackwardFilter(in[0], in[1], in[2], conv_info());
-    } else if (op == "conv_backward_bias") {
-      need(1);
-      r = rt->ConvBackwardBias(in[0]);
-    } else if (op == "pooling_forward") {
-      need(1);
-      r = rt->PoolingForward(in[0], pool_info());
-    } else if (op == "pooling_backward") {
-      need(3);
-      r = rt->PoolingBackward(in[0], in[1], in[2], pool_info());
-    } else if (op == "threshold_norm") {  // params: threshold
-      need(1);
-      MNV_CHECK(n_params >= 1) << "threshold_norm takes the threshold";
-      r = rt->ThresholdNorm(in[0], static_cast<float>(params[0]));
-    } else if (op == "index") {  // params: idx, then the extents of one block
-      need(1);
-      std::vector<int> d;
-      for (int i = 1; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
-      MNV_CHECK(!d.empty()) << "index takes idx, d0, ...";
-      r = rt->Index(in[0], P(params, n_params, 0), Scale(d));
-    } else if (op == "concat") {  // params: catdim; any number (> 1) of inputs
-      r = rt->Concat(in, P(params, n_params, 0));
-    } else if (op == "slice") {  // params: slice_dim, st_off, slice_count
-      need(1);
-      r = rt->Slice(in[0], P(params, n_params, 0), P(params, n_params, 1), P(params, n_params, 2));
-    } else if (op == "select") {  // params: the column indices
-      need(1);
-      std::vector<int> idx;
-      for (int i = 0; i < n_params; ++i) idx.push_back(static_cast<int>(params[i]));
-      r = rt->Select(in[0], idx);
-    } else if (op == "lrn_forward") {  // params: local_size, alpha, beta; inputs: bottom, scale
-      need(2);
-      MNV_CHECK(n_params >= 3) << "lrn_forward takes local_size, alpha, beta";
-      r = rt->LRNForward(in[0], in[1], static_cast<int>(params[0]), static_cast<float>(params[1]),
-                         static_cast<float>(params[2]));
-    } else if (op == "lrn_backward") {  // inputs: bottom, top, scale, top_diff
-      need(4);
-      MNV_CHECK(n_params >= 3) << "lrn_backward takes local_size, alpha, beta";
-      r = rt->LRNBackward(in[0], in[1], in[2], in[3], static_cast<int>(params[0]),
-                          static_cast<float>(params[1]), static_cast<float>(params[2]));
-    } else if (op == "randn" || op == "rand_bernoulli") {  // params: mu, var | p ; then d0, d1, ...
-      need(0);
-      const int lead = op == "randn" ? 2 : 1;
-      MNV_CHECK(n_params > lead) << op << " takes its parameters, then the extents";
-      std::vector<int> d;
-      for (int i = lead; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
-      r = op == "randn" ? rt->Randn(Scale(d), static_cast<float>(params[0]), static_cast<float>(params[1]))
-                        : rt->RandBernoulli(Scale(d), static_cast<float>(params[0]));
-    } else if (op == "fill") {
-      need(0);
-      std::vector<int> d;
-      for (int i = 1; i < n_params; ++i) d.push_back(static_cast<int>(params[i]));
-      MNV_CHECK(n_params >= 2) << "fill takes val, d0, ...";
-      r = rt->Constant(Scale(d), static_cast<float>(params[0]));
-    } else {
-      MNV_FATAL() << "unknown operator '" << op << "'";
-    }
+    Tensor r = RunNamedOp(rt, op_name, in, params, n_params);
     size_t n = r->size.Prod();
     MNV_CHECK(n <= out_capacity) << "output needs " << n << " floats, capacity " << out_capacity;
     std::vector<float> host = rt->Get(r);
@@ -265,6 +296,56 @@ int mnvh_op(void* runtime, const char* op_name, const mnvh_tensor* inputs, int n
     if (out_dims)
       for (size_t i = 0; i < r->size.NumDims(); ++i) out_dims[i] = r->size[i];
   });
+}
+
+// ---- device-resident tensors: graphs of operators without a round trip to the host
+
+int mnvh_tensor_create(void* runtime, const mnvh_tensor* host, void** tensor) {
+  return Guard([&] {
+    Runner* rt = static_cast<Runner*>(runtime);
+    MNV_CHECK(rt && host && host->data && tensor) << "null argument";
+    *tensor = new Tensor(rt->MakeNArray(ToScale(*host), host->data));
+  });
+}
+
+int mnvh_tensor_op(void* runtime, const char* op_name, void* const* inputs, int n_inputs,
+                   const double* params, int n_params, void** out) {
+  return Guard([&] {
+    Runner* rt = static_cast<Runner*>(runtime);
+    MNV_CHECK(rt && op_name && out) << "null argument";
+    std::vector<Tensor> in;
+    for (int i = 0; i < n_inputs; ++i) {
+      MNV_CHECK(inputs && inputs[i]) << "null input tensor";
+      in.push_back(*static_cast<Tensor*>(inputs[i]));
+    }
+    *out = new Tensor(RunNamedOp(rt, op_name, in, params, n_params));
+  });
+}
+
+int mnvh_tensor_info(void* tensor, int* ndims, int* dims, int* stream) {
+  return Guard([&] {
+    MNV_CHECK(tensor) << "null tensor";
+    const Tensor& t = *static_cast<Tensor*>(tensor);
+    if (ndims) *ndims = static_cast<int>(t->size.NumDims());
+    if (dims)
+      for (size_t i = 0; i < t->size.NumDims(); ++i) dims[i] = t->size[i];
+    if (stream) *stream = t->stream;
+  });
+}
+
+int mnvh_tensor_read(void* runtime, void* tensor, float* out, size_t out_capacity) {
+  return Guard([&] {
+    MNV_CHECK(runtime && tensor && out) << "null argument";
+    const Tensor& t = *static_cast<Tensor*>(tensor);
+    size_t n = t->size.Prod();
+    MNV_CHECK(n <= out_capacity) << "tensor has " << n << " floats, capacity " << out_capacity;
+    std::vector<float> host = static_cast<Runner*>(runtime)->Get(t);
+    std::memcpy(out, host.data(), n * sizeof(float));
+  });
+}
+
+int mnvh_tensor_free(void* tensor) {
+  return Guard([&] { delete static_cast<Tensor*>(tensor); });
 }
 
 int mnvh_set_random_seed(unsigned long long seed) {
@@ -400,6 +481,7 @@ int mnvh_net_capture_step(void* net, float lr, size_t* num_nodes) {
     NetHandle* h = static_cast<NetHandle*>(net);
     MNV_CHECK(h->data && h->label) << "load a batch first";
     MNV_CHECK(!h->graph) << "the step is already recorded";
+    MNV_CHECK(!h->rt->device().dataflow()) << "recording needs the one-stream order, not dataflow mode";
     MNV_CHECK(h->net->Capturable()) << "this network draws random seeds on the host in every "
                                     << "step; a recording would repeat them";
     Runner* rt = h->rt;

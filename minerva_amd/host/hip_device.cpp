@@ -24,22 +24,46 @@ PooledDataStore::PooledDataStore(size_t threshold, std::function<void*(size_t)> 
 PooledDataStore::~PooledDataStore() {
   for (auto& kv : data_states_) deallocator_(kv.second.ptr);
   for (auto& kv : free_space_)
-    while (!kv.second.empty()) {
-      deallocator_(kv.second.front());
-      kv.second.pop();
-    }
+    for (auto& b : kv.second) deallocator_(b.ptr);
 }
 
-float* PooledDataStore::CreateData(uint64_t id, size_t length) {
+float* PooledDataStore::CreateData(uint64_t id, size_t length, int stream, unsigned* foreign) {
   std::lock_guard<std::mutex> lck(access_mutex_);
   auto it = data_states_.emplace(id, DataState{nullptr, length});
   MNV_CHECK(it.second) << "data already existed";
   DataState& ds = it.first->second;
+  if (foreign) *foreign = 0;
   auto hit = free_space_.find(length);
   if (hit != free_space_.end()) {  // reuse a block of exactly this size
-    ds.ptr = hit->second.front();
-    hit->second.pop();
-    if (hit->second.empty()) free_space_.erase(hit);
+    auto& blocks = hit->second;
+    size_t pick = 0;
+    bool found = stream < 0;
+    if (stream >= 0) {
+      // a block no other stream still works on needs no wait: stream order protects it
+      const unsigned mine = 1u << stream;
+      for (size_t i = 0; i < blocks.size(); ++i)
+        if ((blocks[i].users & ~mine) == 0) {
+          pick = i;
+          found = true;
+          break;
+        }
+      // Otherwise a new block is better than making this stream wait for the others (it
+      // would wait for everything queued on them, which serialises the streams); the pool
+      // grows by at most what is allocated between two synchronisations, after which
+      // every cached block is free of users again.  Past half the threshold, recycle.
+      if (!found && total_ + length > threshold_ / 2) {
+        found = true;
+        if (foreign) *foreign = blocks[0].users & ~mine;
+      }
+    }
+    if (!found) {
+      ds.ptr = allocator_(length);
+      total_ += length;
+      return static_cast<float*>(ds.ptr);
+    }
+    ds.ptr = blocks[pick].ptr;
+    blocks.erase(blocks.begin() + pick);
+    if (blocks.empty()) free_space_.erase(hit);
   } else {
     ds.ptr = allocator_(length);
     total_ += length;
@@ -60,12 +84,18 @@ bool PooledDataStore::ExistData(uint64_t id) const {
   return data_states_.count(id) != 0;
 }
 
-void PooledDataStore::FreeData(uint64_t id) {
+void PooledDataStore::FreeData(uint64_t id, unsigned users) {
   std::lock_guard<std::mutex> lck(access_mutex_);
   auto it = data_states_.find(id);
   MNV_CHECK(it != data_states_.end()) << "data #" << id << " does not exist";
-  free_space_[it->second.length].push(it->second.ptr);
+  free_space_[it->second.length].push_back(FreeBlock{it->second.ptr, users});
   data_states_.erase(it);
+}
+
+void PooledDataStore::ClearUsers() {
+  std::lock_guard<std::mutex> lck(access_mutex_);
+  for (auto& kv : free_space_)
+    for (auto& b : kv.second) b.users = 0;
 }
 
 size_t PooledDataStore::GetTotalBytes() const {
@@ -82,9 +112,8 @@ size_t PooledDataStore::NumCachedBlocks() const {
 
 void PooledDataStore::ReleaseFreeSpace() {
   for (auto& kv : free_space_)
-    while (!kv.second.empty()) {
-      deallocator_(kv.second.front());
-      kv.second.pop();
+    for (auto& b : kv.second) {
+      deallocator_(b.ptr);
       total_ -= kv.first;
     }
   free_space_.clear();
@@ -125,6 +154,8 @@ HipDevice::~HipDevice() {
   for (auto& t : workers_) t.join();
   Activate();
   for (size_t i = 0; i < kParallelism; ++i) mnv_stream_sync(streams_[i]);
+  for (auto& kv : produced_) mnv_event_destroy(kv.second.event);
+  produced_.clear();
   data_store_.reset();  // before the streams: the deallocator uses the device
   for (size_t i = 0; i < kParallelism; ++i) {
     if (workspace_[i]) mnv_free(workspace_[i]);
@@ -153,16 +184,50 @@ std::pair<HipDevice::MemType, float*> HipDevice::GetPtr(uint64_t data_id) {
 
 void HipDevice::FreeDataIfExist(uint64_t data_id) {
   size_t erased;
+  unsigned users = 0;
+  void* event = nullptr;
   {
     std::lock_guard<std::mutex> lck(local_mutex_);
     erased = local_data_.erase(data_id);
+    auto it = produced_.find(data_id);
+    if (it != produced_.end()) {
+      // The host may be far ahead of the GPU: kernels that read or write this block can
+      // still be queued on these streams when the block goes back to the pool.
+      users = it->second.users;
+      event = it->second.event;
+      produced_.erase(it);
+    }
   }
-  if (erased == 1) data_store_->FreeData(data_id);
+  if (event) mnv_event_destroy(event);  // waits already queued on it keep their meaning
+  if (erased == 1) data_store_->FreeData(data_id, users);
+}
+
+void HipDevice::set_dataflow(bool v) {
+  WaitForAllFinished();
+  Activate();
+  for (size_t i = 0; i < kParallelism; ++i) Ok(mnv_stream_sync(streams_[i]), "mode change sync");
+  dataflow_ = v;
+  if (v) sync_each_op_ = false;
+}
+
+// Makes stream `thrid` wait for everything queued so far on each of `streams`.
+void HipDevice::WaitForStreams(int thrid, unsigned streams) {
+  for (size_t s = 0; s < kParallelism; ++s) {
+    if (!(streams >> s & 1u) || static_cast<int>(s) == thrid) continue;
+    void* e = nullptr;
+    Ok(mnv_event_create_ordering(&e), "event create");
+    Ok(mnv_event_record(e, streams_[s]), "event record");
+    Ok(mnv_stream_wait_event(streams_[thrid], e), "stream wait");
+    mnv_event_destroy(e);
+    ++recycle_waits_;
+  }
 }
 
 void HipDevice::PushTask(Task* task) {
-  if (task->light) {
-    Execute(task, 0);  // light tasks skip the thread hop (device.cpp:55-61)
+  if (task->light) {  // light tasks skip the thread hop (device.cpp:55-61)
+    MNV_CHECK(task->stream >= 0 && task->stream < static_cast<int>(kParallelism)) << "bad stream";
+    MNV_CHECK(task->stream == 0 || dataflow_) << "streams other than 0 need dataflow mode";
+    Execute(task, task->stream);
     return;
   }
   {
@@ -228,16 +293,33 @@ void HipDevice::Execute(Task* task, int thrid) {
     // One GPU: every input is local.  A remote input would be copied here with
     // mnv_memcpy_d2d over xGMI, as DoCopyRemoteData does in the reference.
     MNV_CHECK_EQ(d.device_id, device_id_) << "remote inputs are not part of the one-GPU build";
+    void* wait_for = nullptr;
     {
       std::lock_guard<std::mutex> lck(local_mutex_);
       MNV_CHECK_EQ(local_data_.count(d.data_id), 1u) << "input data #" << d.data_id << " missing";
+      if (dataflow_) {
+        auto it = produced_.find(d.data_id);
+        if (it != produced_.end()) {
+          if (it->second.stream != thrid) wait_for = it->second.event;
+          it->second.users |= 1u << thrid;
+        }
+      }
+    }
+    // produced on another stream: this stream waits for the producer on the GPU
+    if (wait_for) {
+      Ok(mnv_stream_wait_event(streams_[thrid], wait_for), "stream wait");
+      ++producer_waits_;
     }
     input_shards.emplace_back(data_store_->GetData(d.data_id), d.size);
   }
   DataList output_shards;
   for (auto& o : task->outputs) {
     size_t bytes = static_cast<size_t>(o.physical_data.size.Prod()) * sizeof(float);
-    float* ptr = data_store_->CreateData(o.physical_data.data_id, bytes);
+    unsigned foreign = 0;
+    float* ptr = data_store_->CreateData(o.physical_data.data_id, bytes, dataflow_ ? thrid : -1,
+                                         &foreign);
+    // a recycled block that work queued on other streams may still touch
+    if (foreign) WaitForStreams(thrid, foreign);
     {
       std::lock_guard<std::mutex> lck(local_mutex_);
       MNV_CHECK(local_data_.insert(o.physical_data.data_id).second) << "duplicate data";
@@ -246,6 +328,15 @@ void HipDevice::Execute(Task* task, int thrid) {
   }
   MNV_CHECK(task->op.compute_fn) << "task without an operator";
   DoExecute(input_shards, output_shards, task->op, thrid);
+  if (dataflow_) {
+    for (auto& o : task->outputs) {
+      void* e = nullptr;
+      Ok(mnv_event_create_ordering(&e), "event create");
+      Ok(mnv_event_record(e, streams_[thrid]), "event record");
+      std::lock_guard<std::mutex> lck(local_mutex_);
+      produced_[o.physical_data.data_id] = Produced{e, thrid, 1u << thrid};
+    }
+  }
   if (listener_) listener_->OnOperationComplete(task);
 }
 
@@ -257,9 +348,12 @@ void HipDevice::DoExecute(const DataList& in, const DataList& out, PhysicalOp& o
   ctx.workspace = workspace_[thrid];
   ctx.workspace_bytes = workspace_bytes_[thrid];
   Timed t{std::string(), nullptr, nullptr};
-  const bool timed = profile_ && !capturing_;
+  bool timed = profile_ && !capturing_;
   if (timed) {
     t.name = op.compute_fn->Name();
+    timed = profile_filter_.empty() || t.name.find(profile_filter_) != std::string::npos;
+  }
+  if (timed) {
     Ok(mnv_event_create(&t.start), "event create");
     Ok(mnv_event_create(&t.stop), "event create");
     Ok(mnv_event_record(t.start, streams_[thrid]), "event record");
@@ -299,6 +393,7 @@ std::map<std::string, std::pair<int, double>> HipDevice::CollectProfile() {
 
 void HipDevice::BeginCapture() {
   MNV_CHECK(!capturing_) << "a graph is already being recorded";
+  MNV_CHECK(!dataflow_) << "recording needs the one-stream order, not dataflow mode";
   WaitForAllFinished();
   Activate();
   EnsureWorkspace(0, kWorkspaceBytes);
@@ -331,6 +426,13 @@ void HipDevice::LaunchGraph(void* graph_exec) {
 
 void HipDevice::Barrier(int thrid) {
   MNV_CHECK(!capturing_) << "no synchronisation while a graph is recorded";
+  if (dataflow_) {
+    Activate();
+    for (size_t i = 0; i < kParallelism; ++i) Ok(mnv_stream_sync(streams_[i]), "barrier");
+    // nothing is queued any more: every cached block may go to any stream without a wait
+    data_store_->ClearUsers();
+    return;
+  }
   Ok(mnv_stream_sync(streams_[thrid]), "barrier");
 }
 

@@ -8,8 +8,13 @@
 //    completion is reported, as the reference does after every operator.
 //  - PooledDataStore: exact-size free lists over mnv_malloc / mnv_free; when the bytes
 //    held exceed the threshold every cached block is released.
+//  - Three ways to order operators: synchronise after every one (the reference);
+//    leave them in flight on one stream (stream order); or "dataflow": operators run on
+//    any of the four streams, every output carries an event recorded behind its producer,
+//    and a consumer on another stream waits for that event on the GPU, never on the host.
 #pragma once
 #include <array>
+#include <atomic>
 #include <condition_variable>
 #include <deque>
 #include <functional>
@@ -47,7 +52,8 @@ struct Task {
   std::vector<TaskData> outputs;
   PhysicalOp op;
   uint64_t id = 0;
-  bool light = false;  // run on the caller's thread (stream 0) instead of the pool
+  bool light = false;  // run on the caller's thread instead of the pool
+  int stream = 0;      // light tasks: which worker stream (0 unless the device is in dataflow mode)
 };
 
 class DeviceListener {
@@ -62,10 +68,17 @@ class PooledDataStore {
   ~PooledDataStore();
   PooledDataStore(const PooledDataStore&) = delete;
   PooledDataStore& operator=(const PooledDataStore&) = delete;
-  float* CreateData(uint64_t id, size_t length);
+  // `stream` >= 0 (dataflow mode): prefer a cached block that only this stream has touched.
+  // *foreign receives the streams (bit per stream) other than `stream` whose queued work may
+  // still use the block handed out; the caller makes `stream` wait for them.
+  float* CreateData(uint64_t id, size_t length, int stream = -1, unsigned* foreign = nullptr);
   float* GetData(uint64_t id);
   bool ExistData(uint64_t id) const;
-  void FreeData(uint64_t id);
+  // `users`: the streams that have work queued on the block (0 when everything is known
+  // to have finished).
+  void FreeData(uint64_t id, unsigned users = 0);
+  // Every queued operator has finished: cached blocks have no users left.
+  void ClearUsers();
   size_t GetTotalBytes() const;
   size_t NumCachedBlocks() const;
 
@@ -77,7 +90,11 @@ class PooledDataStore {
   };
   mutable std::mutex access_mutex_;
   std::unordered_map<uint64_t, DataState> data_states_;
-  std::unordered_map<size_t, std::queue<void*>> free_space_;
+  struct FreeBlock {
+    void* ptr;
+    unsigned users;
+  };
+  std::unordered_map<size_t, std::deque<FreeBlock>> free_space_;
   std::function<void*(size_t)> allocator_;
   std::function<void(void*)> deallocator_;
   size_t threshold_;
@@ -108,6 +125,15 @@ class HipDevice {
   // When false, operators are left in flight on their stream and the caller decides
   // when to synchronise (Barrier); the reference always synchronises per operator.
   void set_sync_each_op(bool v) { sync_each_op_ = v; }
+  // Dataflow mode: light tasks may name any worker stream; dependencies across streams
+  // are kept by events on the GPU.  Implies no synchronisation per operator.
+  void set_dataflow(bool v);
+  bool dataflow() const { return dataflow_; }
+  // Since the device was created: waits of a consumer's stream for a producer on another
+  // stream, and waits of a stream for other streams before it reuses a recycled block.
+  uint64_t producer_waits() const { return producer_waits_; }
+  uint64_t recycle_waits() const { return recycle_waits_; }
+  // Waits for worker stream `thrid`; in dataflow mode for all of them.
   void Barrier(int thrid);
   void* stream(int thrid) const { return streams_[thrid]; }
   uint64_t device_id() const { return device_id_; }
@@ -126,6 +152,10 @@ class HipDevice {
   // bracketed by two events on its own stream; CollectProfile synchronises and returns
   // name -> (launch count, total device milliseconds), then clears the record.
   void set_profile(bool v) { profile_ = v; }
+  // Only operators whose name contains `part` are timed (empty: all).  Two events per
+  // operator cost a few microseconds of GPU idle time each, so a measurement that wants
+  // one kernel's duration inside an otherwise undisturbed step names that kernel.
+  void set_profile_filter(const std::string& part) { profile_filter_ = part; }
   std::map<std::string, std::pair<int, double>> CollectProfile();
 
   // Records the light tasks pushed between Begin and End (they run on worker stream 0)
@@ -152,6 +182,17 @@ class HipDevice {
   int gpu_id_;
   bool sync_each_op_ = true;
   bool capturing_ = false;
+  bool dataflow_ = false;
+  // dataflow mode, guarded by local_mutex_: where each datum was produced (stream, event
+  // recorded behind the producer) and which streams have work queued that touches it
+  struct Produced {
+    void* event;
+    int stream;
+    unsigned users;
+  };
+  std::unordered_map<uint64_t, Produced> produced_;
+  void WaitForStreams(int thrid, unsigned streams);
+  std::atomic<uint64_t> producer_waits_{0}, recycle_waits_{0};
   std::array<void*, kParallelism> streams_{};
   std::array<void*, kParallelism> workspace_{};
   std::array<size_t, kParallelism> workspace_bytes_{};
@@ -173,6 +214,7 @@ class HipDevice {
     void* stop;
   };
   bool profile_ = false;
+  std::string profile_filter_;
   std::mutex prof_mutex_;
   std::vector<Timed> timed_;
 };

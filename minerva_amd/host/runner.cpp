@@ -8,9 +8,32 @@ TensorNode::~TensorNode() {
   if (runner && runner->device_) runner->device_->FreeDataIfExist(id);
 }
 
-Runner::Runner(int gpu_id, bool sync_each_op) {
-  device_.reset(new HipDevice(0, this, gpu_id));
+Runner::Runner(int gpu_id, bool sync_each_op, bool dataflow, size_t pool_bytes)
+    : dataflow_(dataflow) {
+  device_.reset(new HipDevice(0, this, gpu_id, pool_bytes));
   device_->set_sync_each_op(sync_each_op);
+  if (dataflow) device_->set_dataflow(true);
+}
+
+void Runner::Sync() {
+  device_->Barrier(0);
+  for (auto& q : queued_) q = 0;
+}
+
+int Runner::PickStream(const std::vector<Tensor>& inputs) {
+  int pick = -1;
+  uint64_t newest = 0;
+  for (auto& t : inputs)
+    if (tail_[t->stream] == t->id && t->id >= newest) {
+      pick = t->stream;
+      newest = t->id;
+    }
+  if (pick < 0) {
+    pick = 0;
+    for (int s = 1; s < static_cast<int>(HipDevice::kParallelism); ++s)
+      if (queued_[s] < queued_[pick]) pick = s;
+  }
+  return pick;
 }
 
 Runner::~Runner() {
@@ -29,7 +52,12 @@ Tensor Runner::Compute(const std::vector<Tensor>& inputs, const Scale& out_size,
   task.op.compute_fn = std::move(fn);
   task.op.device_id = device_->device_id();
   task.id = ops_issued_++;
-  task.light = true;  // sequential: run on the caller's thread, worker stream 0
+  task.light = true;  // issued in program order from the caller's thread
+  if (dataflow_) {
+    task.stream = out->stream = PickStream(inputs);
+    tail_[task.stream] = out->id;
+    ++queued_[task.stream];
+  }
   device_->PushTask(&task);
   if (retain_) retained_.push_back(out);
   return out;

@@ -23,18 +23,22 @@ struct TensorNode {
   Runner* runner;
   uint64_t id;
   Scale size;
+  int stream = 0;  // the worker stream its producer ran on
 };
 using Tensor = std::shared_ptr<TensorNode>;
 
 class Runner : public DeviceListener {
  public:
-  explicit Runner(int gpu_id, bool sync_each_op = true);
+  // dataflow: operators are spread over the device's four streams and ordered by events
+  // (see PickStream); otherwise everything runs on stream 0 in program order.
+  explicit Runner(int gpu_id, bool sync_each_op = true, bool dataflow = false,
+                  size_t pool_bytes = HipDevice::kDefaultPoolBytes);
   ~Runner() override;
   void OnOperationComplete(Task*) override { ++ops_completed_; }
 
   HipDevice& device() { return *device_; }
   uint64_t ops_issued() const { return ops_issued_; }
-  void Sync() { device_->Barrier(0); }
+  void Sync();
 
   Tensor Compute(const std::vector<Tensor>& inputs, const Scale& out_size,
                  std::shared_ptr<ComputeFn> fn);
@@ -116,6 +120,15 @@ class Runner : public DeviceListener {
   std::atomic<uint64_t> ops_issued_{0}, ops_completed_{0};
   bool retain_ = false;
   std::vector<Tensor> retained_;
+  // Dataflow placement.  An operator whose newest input is the last thing queued on some
+  // stream continues that stream (a chain stays together and needs no event wait);
+  // any other operator starts a new chain on the stream with the least work queued since
+  // the last Sync.  Independent chains -- the weight-gradient branches of a backward pass
+  // against its data-gradient spine -- so end up on different streams and overlap.
+  int PickStream(const std::vector<Tensor>& inputs);
+  bool dataflow_ = false;
+  uint64_t tail_[HipDevice::kParallelism] = {};    // id of the last output queued per stream
+  uint64_t queued_[HipDevice::kParallelism] = {};  // operators queued per stream since Sync
 };
 
 }  // namespace minerva

@@ -45,11 +45,64 @@ def _check(rc, what):
         raise HostError("%s: %s" % (what, lib().mnvh_last_error().decode()))
 
 
+class DeviceTensor:
+    """A tensor resident on the device (a handle of the host layer)."""
+
+    def __init__(self, runtime, handle):
+        self.rt, self.h = runtime, handle
+        nd, st = ctypes.c_int(), ctypes.c_int()
+        dims = (ctypes.c_int * MAX_DIMS)()
+        _check(lib().mnvh_tensor_info(self.h, ctypes.byref(nd), dims, ctypes.byref(st)), "tensor_info")
+        self.dims = [dims[i] for i in range(nd.value)]
+        self.stream = st.value  # worker stream the producer was placed on
+
+    def read(self):
+        n = int(np.prod(self.dims))
+        out = np.empty(n, np.float32)
+        _check(lib().mnvh_tensor_read(self.rt.h, self.h,
+                                      out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                                      ctypes.c_size_t(n)), "tensor_read")
+        return out
+
+    def free(self):
+        if self.h:
+            _check(lib().mnvh_tensor_free(self.h), "tensor_free")
+            self.h = None
+
+
 class Runtime:
-    def __init__(self, gpu=0, sync_each_op=True):
+    def __init__(self, gpu=0, sync_each_op=True, dataflow=False, pool_bytes=None):
+        """sync_each_op: wait after every operator (the reference's behaviour); dataflow:
+        four streams ordered by events instead (implies no per-operator wait); pool_bytes:
+        threshold of the pooled allocator."""
         self.h = ctypes.c_void_p()
-        _check(lib().mnvh_runtime_create(gpu, 1 if sync_each_op else 0, ctypes.byref(self.h)),
-               "runtime_create")
+        mode = 2 if dataflow else (1 if sync_each_op else 0)
+        if pool_bytes is None:
+            _check(lib().mnvh_runtime_create(gpu, mode, ctypes.byref(self.h)), "runtime_create")
+        else:
+            _check(lib().mnvh_runtime_create_pool(gpu, mode, ctypes.c_size_t(pool_bytes),
+                                                  ctypes.byref(self.h)), "runtime_create_pool")
+
+    def tensor(self, a, dims):
+        a = np.ascontiguousarray(a, dtype=np.float32).ravel()
+        assert a.size == int(np.prod(dims))
+        t = _Tensor()
+        t.data = a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+        t.ndims = len(dims)
+        for j, d in enumerate(dims):
+            t.dims[j] = int(d)
+        h = ctypes.c_void_p()
+        _check(lib().mnvh_tensor_create(self.h, ctypes.byref(t), ctypes.byref(h)), "tensor_create")
+        return DeviceTensor(self, h)
+
+    def top(self, name, inputs, params=()):
+        """One operator on device tensors; returns a DeviceTensor (nothing is synchronised)."""
+        arr = (ctypes.c_void_p * max(len(inputs), 1))(*[t.h for t in inputs])
+        p = (ctypes.c_double * max(len(params), 1))(*[float(x) for x in params])
+        h = ctypes.c_void_p()
+        _check(lib().mnvh_tensor_op(self.h, name.encode(), arr, len(inputs), p, len(params),
+                                    ctypes.byref(h)), name)
+        return DeviceTensor(self, h)
 
     def close(self):
         if self.h:
@@ -69,7 +122,16 @@ class Runtime:
         _check(lib().mnvh_runtime_pool_stats(self.h, ctypes.byref(t), ctypes.byref(c)), "pool_stats")
         return t.value, c.value
 
-    def profile(self, enable):
+    def dataflow_stats(self):
+        """(waits for a producer on another stream, waits before reusing a recycled block)"""
+        a, b = ctypes.c_ulonglong(), ctypes.c_ulonglong()
+        _check(lib().mnvh_runtime_dataflow_stats(self.h, ctypes.byref(a), ctypes.byref(b)),
+               "dataflow_stats")
+        return a.value, b.value
+
+    def profile(self, enable, only=""):
+        """Per-operator device timing; `only`: time just the operators whose name contains it."""
+        _check(lib().mnvh_runtime_profile_filter(self.h, only.encode()), "profile_filter")
         _check(lib().mnvh_runtime_profile(self.h, 1 if enable else 0), "profile")
 
     def profile_read(self):

@@ -52,3 +52,41 @@ class Gpu:
         rc = getattr(self.L, name)(*args, self.dev.stream)
         capi.check(rc, name)
         self.dev.sync()
+
+
+def net_batches(kind, batch, count):
+    """The seeded parameters and `count` different batches of one network configuration."""
+    from oracle import nets
+    params, data, label = nets.make_inputs(kind, batch)
+    per_d, per_l = data.size // batch, label.size // batch
+    out = []
+    for i in range(count):  # rotate the images against the labels: new batches, same statistics
+        d = np.roll(data.reshape(batch, per_d), i, axis=0).ravel()
+        l = np.roll(label.reshape(batch, per_l), 2 * i, axis=0).ravel()
+        out.append((d.copy(), l.copy()))
+    return params, out
+
+
+def net_state(net, label_floats):
+    s = {k: net.read(k, n) for k, n in net.params.items()}
+    s.update({"g_" + k: net.read("g_" + k, n) for k, n in net.params.items()})
+    s["prob"] = net.read("prob", label_floats)
+    return s
+
+
+def run_steps(kind, batch, variant, lr, params, batches, **runtime_args):
+    """One step per batch, operator by operator; the state after every step."""
+    from minerva_amd import hostapi
+    runtime_args.setdefault("sync_each_op", False)
+    r = hostapi.Runtime(0, **runtime_args)
+    net = hostapi.Net(r, kind, batch, variant)
+    for k, v in params.items():
+        net.set_param(k, v)
+    states = []
+    for d, l in batches:
+        net.load_batch(d, l)
+        net.step(lr)
+        states.append(net_state(net, l.size))
+    net.close()
+    r.close()
+    return states

@@ -1,0 +1,154 @@
+"""Dataflow mode of the device: operators spread over four streams and ordered by events
+on the GPU instead of a host wait after every operator.  Results must be bit-identical to
+the one-stream order, also when a consumer sits on another stream than its producer and
+when a pool block is recycled on another stream while its last reader is still queued."""
+import numpy as np
+import pytest
+
+from gpu_util import assert_bits_equal, net_batches, run_steps, say
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand(n, seed):
+    return np.random.default_rng(seed).standard_normal(n).astype(np.float32)
+
+
+@pytest.mark.parametrize("kind,batch,variant", [("mlp", 256, 0), ("cnn", 64, 0), ("cnn", 32, 1),
+                                                ("alexnet", 2, 0)])
+def test_training_steps_identical_to_stream_order(kind, batch, variant):
+    params, batches = net_batches(kind, batch, 3)
+    say("one stream", kind, batch, variant)
+    want = run_steps(kind, batch, variant, 0.05, params, batches)
+    say("dataflow", kind, batch, variant)
+    got = run_steps(kind, batch, variant, 0.05, params, batches, dataflow=True)
+    for i, (g, w) in enumerate(zip(got, want)):
+        for k in w:
+            assert_bits_equal(g[k], w[k], "%s after step %d" % (k, i))
+
+
+def test_consumer_on_another_stream_waits_for_its_producer():
+    from minerva_amd import hostapi
+    n = 2048
+    a, b = _rand(n * n, 1) / np.float32(45), _rand(n * n, 2) / np.float32(45)
+    results = {}
+    for mode in ("order", "dataflow"):
+        r = hostapi.Runtime(0, sync_each_op=False, dataflow=(mode == "dataflow"))
+        ta, tb = r.tensor(a, [n, n]), r.tensor(b, [n, n])
+        say("producer chain", mode)
+        chain = [r.top("matmult", [ta, tb])]
+        for _ in range(7):  # ~0.15 ms each: the host is several products ahead of the GPU
+            chain.append(r.top("matmult", [chain[-1], tb]))
+        mid = chain[3]
+        # `mid` is not the last thing queued on its stream, so this starts a new chain
+        side = r.top("arithmetic", [mid, mid], [0])
+        side2 = r.top("arithmetic_const", [side], [2, 0.5, 0])
+        if mode == "dataflow":
+            assert all(c.stream == chain[0].stream for c in chain), "a chain shares one stream"
+            assert side.stream != mid.stream, "the side branch must sit on another stream"
+            assert side2.stream == side.stream
+            assert r.dataflow_stats()[0] >= 1, "the side branch must wait for its producer"
+        results[mode] = (side2.read(), chain[-1].read())
+        r.close()
+    assert_bits_equal(results["dataflow"][0], results["order"][0], "side branch")
+    assert_bits_equal(results["dataflow"][1], results["order"][1], "main chain")
+    assert np.isfinite(results["order"][1]).all() and np.abs(results["order"][0]).max() > 0
+
+
+def test_block_recycled_on_another_stream_waits_for_its_last_reader():
+    from minerva_amd import hostapi
+    n = 4096
+    x = _rand(n * n, 3) / np.float32(64)
+    results = {}
+    for mode in ("order", "dataflow"):
+        # four live 64 MiB tensors make half of this pool's threshold: from there on a
+        # stream recycles a block that another stream still uses rather than allocating
+        r = hostapi.Runtime(0, sync_each_op=False, dataflow=(mode == "dataflow"),
+                            pool_bytes=512 << 20)
+        tx = r.tensor(x, [n, n])
+        say("long reader", mode)
+        y = r.top("arithmetic_const", [tx], [2, 1.0, 0])    # y = x on the device, own block
+        prod = r.top("matmult", [y, y])                       # ~1 ms, reads y throughout
+        prod2 = r.top("matmult", [prod, tx])
+        total_before, _ = r.pool_stats()
+        y.free()                                              # y's block goes back to the pool
+        z = r.top("fill", [], [7.0, n, n])                    # same size: takes y's block
+        total_after, _ = r.pool_stats()
+        assert total_after == total_before, "the fill must recycle the freed block"
+        if mode == "dataflow":
+            assert z.stream != prod.stream, "the fill must sit on another stream than the reader"
+            assert r.dataflow_stats()[1] >= 1, "the fill's stream must have been made to wait"
+        results[mode] = (prod.read(), prod2.read())
+        assert_bits_equal(z.read(), np.full(n * n, 7.0, np.float32), "fill")
+        r.close()
+    # the reader saw y, not the fill that recycled y's block
+    assert_bits_equal(results["dataflow"][0], results["order"][0], "product that read the freed block")
+    assert_bits_equal(results["dataflow"][1], results["order"][1], "its successor")
+    s = np.float64(x[:n]) @ np.float64(x.reshape(n, n)[:, 0])  # entry (0, 0) of x @ x, column-major
+    assert abs(results["order"][0][0] - s) <= 1e-3 * max(1.0, abs(s))
+
+
+def test_random_operator_graph_with_frees():
+    """A few hundred operators over a changing set of live tensors, tensors freed while
+    their consumers are queued: dataflow placement against the one-stream order."""
+    from minerva_amd import hostapi
+    m = 192
+    rng_ops = np.random.default_rng(11)
+    plan = []
+    live = 4
+    for _ in range(300):
+        kind = int(rng_ops.integers(0, 5))
+        i, j = int(rng_ops.integers(0, live)), int(rng_ops.integers(0, live))
+        drop = int(rng_ops.integers(0, live + 1)) if live > 6 else -1
+        plan.append((kind, i, j, drop))
+        live += 1
+        if 0 <= drop < live - 1:
+            live -= 1
+    outs = {}
+    for mode in ("order", "dataflow"):
+        r = hostapi.Runtime(0, sync_each_op=False, dataflow=(mode == "dataflow"))
+        ts = [r.tensor(_rand(m * m, 20 + k) / np.float32(16), [m, m]) for k in range(4)]
+        streams = set()
+        say("random graph", mode)
+        for kind, i, j, drop in plan:
+            if kind == 0:
+                t = r.top("matmult", [ts[i], ts[j]])
+                t2 = r.top("arithmetic_const", [t], [2, 1.0 / 16, 0])  # keep magnitudes bounded
+                t.free()
+                t = t2
+            elif kind == 1:
+                t = r.top("arithmetic", [ts[i], ts[j]], [1])
+            elif kind == 2:
+                t = r.top("trans", [ts[i]])
+            elif kind == 3:
+                t = r.top("tanh_forward", [ts[i]])
+            else:
+                t = r.top("arithmetic", [ts[i], ts[j]], [2])
+            streams.add(t.stream)
+            ts.append(t)
+            if 0 <= drop < len(ts) - 1:
+                ts.pop(drop).free()
+        outs[mode] = [t.read() for t in ts]
+        if mode == "dataflow":
+            assert len(streams) >= 3, "the graph must spread over the streams: %r" % streams
+        r.close()
+    assert len(outs["order"]) == len(outs["dataflow"])
+    for k, (g, w) in enumerate(zip(outs["dataflow"], outs["order"])):
+        assert np.isfinite(w).all()
+        assert_bits_equal(g, w, "live tensor %d" % k)
+
+
+def test_recording_is_refused_in_dataflow_mode():
+    from minerva_amd import hostapi
+    params, batches = net_batches("mlp", 32, 1)
+    r = hostapi.Runtime(0, dataflow=True)
+    net = hostapi.Net(r, "mlp", 32)
+    for k, v in params.items():
+        net.set_param(k, v)
+    net.load_batch(*batches[0])
+    with pytest.raises(hostapi.HostError, match="dataflow"):
+        net.capture_step(0.1)
+    net.step(0.1)  # the refusal left the network usable
+    r.sync()
+    net.close()
+    r.close()

@@ -7,45 +7,16 @@ import ctypes
 import numpy as np
 import pytest
 
-from gpu_util import Gpu, assert_bits_equal, say
+from gpu_util import Gpu, assert_bits_equal, net_batches, net_state, run_steps, say
 
 pytestmark = pytest.mark.gpu
 
 
-def _batches(kind, batch, count):
-    """The seeded parameters and `count` different batches of one configuration."""
-    from oracle import nets
-    params, data, label = nets.make_inputs(kind, batch)
-    per_d, per_l = data.size // batch, label.size // batch
-    out = []
-    for i in range(count):  # rotate the images against the labels: new batches, same statistics
-        d = np.roll(data.reshape(batch, per_d), i, axis=0).ravel()
-        l = np.roll(label.reshape(batch, per_l), 2 * i, axis=0).ravel()
-        out.append((d.copy(), l.copy()))
-    return params, out
-
-
-def _state(net, label_floats):
-    s = {k: net.read(k, n) for k, n in net.params.items()}
-    s.update({"g_" + k: net.read("g_" + k, n) for k, n in net.params.items()})
-    s["prob"] = net.read("prob", label_floats)
-    return s
+_batches, _state = net_batches, net_state
 
 
 def _eager(kind, batch, variant, lr, params, batches):
-    from minerva_amd import hostapi
-    r = hostapi.Runtime(0, sync_each_op=False)
-    net = hostapi.Net(r, kind, batch, variant)
-    for k, v in params.items():
-        net.set_param(k, v)
-    states = []
-    for d, l in batches:
-        net.load_batch(d, l)
-        net.step(lr)
-        states.append(_state(net, l.size))
-    net.close()
-    r.close()
-    return states
+    return run_steps(kind, batch, variant, lr, params, batches)
 
 
 @pytest.mark.parametrize("kind,batch,variant", [("mlp", 256, 0), ("cnn", 64, 0), ("cnn", 32, 1),
