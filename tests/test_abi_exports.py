@@ -53,3 +53,17 @@ def test_pure_host_entry_points():
     assert L.mnv_sgemm_nn_workspace_bytes(4096, 4096, 4096) == 0
     assert L.mnv_sgemm_nn_workspace_bytes(1000, 256, 4096) > 0
     assert L.mnv_conv_bwd_filter_workspace_bytes(256, 256, 384, 13, 13, 1, 1, 1, 1, 3, 3) > 0
+
+
+def test_host_library_exports_every_declared_symbol():
+    """include/mnv_host.h against libmnv_host.so (loading it needs no GPU either)."""
+    from minerva_amd import capi, hostapi
+    text = open(os.path.join(ROOT, "include", "mnv_host.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(mnvh_[a-z0-9_]+)\s*\(", text)))
+    assert len(names) >= 30
+    assert os.path.exists(hostapi.LIB_PATH), "build the library first: python -m minerva_amd.build"
+    capi.lib()  # libmnv_hip.so first, from the same directory
+    lib = ctypes.CDLL(hostapi.LIB_PATH)
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
