@@ -60,8 +60,8 @@ DOMINANT_OP = "conv bp filter"  # operator names: "pad:1*1 stride:1*1 conv bp fi
 
 def alexnet_bench(steps, warmup, dataflow=False):
     from minerva_amd import hostapi
-    from oracle import nets  # input generator only (seeded host data)
-    params, data, label = nets.make_inputs("alexnet", BATCH)
+    from minerva_amd import configs
+    params, data, label = configs.make_inputs("alexnet", BATCH)
     out = {}
     modes = [("per_step_sync", False), ("per_op_sync", True)]
     if dataflow:  # kernels of different streams overlap: kept out of the default run so that
@@ -272,10 +272,10 @@ def small_nets(steps=20, warmup=3):
     """BASELINE.json configs[0] (MLP) and configs[3] (CNN) at batch 256: latency-bound
     graphs, reported as ms/step and operators/step without a roofline claim."""
     from minerva_amd import hostapi
-    from oracle import nets  # input generator only
+    from minerva_amd import configs
     out = {}
     for name in ("mlp", "cnn"):
-        params, data, label = nets.make_inputs(name, BATCH)
+        params, data, label = configs.make_inputs(name, BATCH)
         rt = hostapi.Runtime(0, sync_each_op=False)
         net = hostapi.Net(rt, name, BATCH)
         for k, v in params.items():

@@ -480,3 +480,17 @@ def test_threshold_norm_is_a_clip(ora):
     want = np.clip(x, -1.0, 1.0)
     assert np.array_equal(got[:7], want[:7])
     assert np.isnan(got[7]) and np.isnan(got[8])
+
+
+def test_benchmark_inputs_of_package_and_oracle_agree():
+    """The package's generator of the benchmark inputs (what bench.py feeds the GPU) and
+    the oracle's (what the parity tests feed both sides) are the same seeded data."""
+    from minerva_amd import configs
+    from oracle import nets
+    for kind, batch in (("mlp", 5), ("cnn", 3), ("alexnet", 1)):
+        pa, da, la = configs.make_inputs(kind, batch)
+        pb, db, lb = nets.make_inputs(kind, batch)
+        assert sorted(pa) == sorted(pb)
+        for k in pa:
+            assert np.array_equal(pa[k], pb[k]), (kind, k)
+        assert np.array_equal(da, db) and np.array_equal(la, lb), kind
