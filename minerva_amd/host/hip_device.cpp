@@ -13,6 +13,9 @@ void Ok(int status, const char* what) {
 // Scratch arena per worker stream: split-k partial sums of the skinny GEMMs and of the
 // convolution filter gradient.  The kernels use as many k ranges as fit.
 constexpr size_t kWorkspaceBytes = (size_t)128 << 20;
+// Pinned staging per worker stream: two halves, one filled by the CPU while the other is
+// copied to the device.
+constexpr size_t kStagingBytes = (size_t)16 << 20;
 }  // namespace
 
 // ---------------------------------------------------------------- PooledDataStore
@@ -159,6 +162,7 @@ HipDevice::~HipDevice() {
   data_store_.reset();  // before the streams: the deallocator uses the device
   for (size_t i = 0; i < kParallelism; ++i) {
     if (workspace_[i]) mnv_free(workspace_[i]);
+    if (staging_[i]) mnv_host_free(staging_[i]);
     mnv_stream_destroy(streams_[i]);
   }
 }
@@ -285,6 +289,11 @@ void HipDevice::EnsureWorkspace(int thrid, size_t bytes) {
   workspace_bytes_[thrid] = bytes;
 }
 
+void HipDevice::EnsureStaging(int thrid) {
+  if (staging_[thrid]) return;
+  Ok(mnv_host_malloc(&staging_[thrid], kStagingBytes), "pinned staging");
+}
+
 void HipDevice::Execute(Task* task, int thrid) {
   Activate();  // every task re-selects the device on its thread (device.cpp:201-203)
   DataList input_shards;
@@ -347,6 +356,11 @@ void HipDevice::DoExecute(const DataList& in, const DataList& out, PhysicalOp& o
   ctx.stream = streams_[thrid];
   ctx.workspace = workspace_[thrid];
   ctx.workspace_bytes = workspace_bytes_[thrid];
+  if (!capturing_) {
+    EnsureStaging(thrid);
+    ctx.staging = staging_[thrid];
+    ctx.staging_bytes = kStagingBytes;
+  }
   Timed t{std::string(), nullptr, nullptr};
   bool timed = profile_ && !capturing_;
   if (timed) {

@@ -175,6 +175,7 @@ class HipDevice {
   void DoExecute(const DataList& in, const DataList& out, PhysicalOp& op, int thrid);
   void Activate() const;
   void EnsureWorkspace(int thrid, size_t bytes);
+  void EnsureStaging(int thrid);
   void WorkerLoop(int thrid);
 
   uint64_t device_id_;
@@ -196,6 +197,7 @@ class HipDevice {
   std::array<void*, kParallelism> streams_{};
   std::array<void*, kParallelism> workspace_{};
   std::array<size_t, kParallelism> workspace_bytes_{};
+  std::array<void*, kParallelism> staging_{};  // pinned host memory, allocated at first use
   std::unique_ptr<PooledDataStore> data_store_;
   std::mutex local_mutex_;
   std::unordered_set<uint64_t> local_data_;

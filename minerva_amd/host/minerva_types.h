@@ -119,6 +119,9 @@ struct Context {
   void* stream = nullptr;
   void* workspace = nullptr;
   size_t workspace_bytes = 0;
+  // pinned host memory of the stream, for staging copies from pageable host buffers
+  void* staging = nullptr;
+  size_t staging_bytes = 0;
   virtual ~Context() {}
 };
 

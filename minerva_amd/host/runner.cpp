@@ -100,10 +100,9 @@ Tensor Runner::MakeNArray(const Scale& size, std::shared_ptr<float> host) {
 }
 
 Tensor Runner::MakeNArray(const Scale& size, const float* host) {
-  size_t n = size.Prod();
-  std::shared_ptr<float> copy(new float[n], [](float* p) { delete[] p; });
-  std::memcpy(copy.get(), host, n * sizeof(float));
-  return MakeNArray(size, copy);
+  MNV_CHECK(host) << "null host data";
+  std::shared_ptr<float> borrowed(const_cast<float*>(host), [](float*) {});
+  return MakeNArray(size, borrowed);
 }
 
 Tensor Runner::Constant(const Scale& size, float v) {

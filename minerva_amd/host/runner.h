@@ -56,7 +56,9 @@ class Runner : public DeviceListener {
 
   // data generators
   Tensor MakeNArray(const Scale& size, std::shared_ptr<float> host);
-  Tensor MakeNArray(const Scale& size, const float* host);  // copies the host data first
+  // The loader runs before this returns (operators are issued from the caller's thread and
+  // the loader waits for its copy), so the caller's buffer is read in place, not copied.
+  Tensor MakeNArray(const Scale& size, const float* host);
   Tensor Constant(const Scale& size, float v);
   Tensor Zeros(const Scale& size) { return Constant(size, 0.f); }
   // reference minerva/narray/narray.cpp:21-33
