@@ -290,8 +290,7 @@ int mnvh_op(void* runtime, const char* op_name, const mnvh_tensor* inputs, int n
     Tensor r = RunNamedOp(rt, op_name, in, params, n_params);
     size_t n = r->size.Prod();
     MNV_CHECK(n <= out_capacity) << "output needs " << n << " floats, capacity " << out_capacity;
-    std::vector<float> host = rt->Get(r);
-    std::memcpy(out, host.data(), n * sizeof(float));
+    rt->Read(r, out);
     if (out_ndims) *out_ndims = static_cast<int>(r->size.NumDims());
     if (out_dims)
       for (size_t i = 0; i < r->size.NumDims(); ++i) out_dims[i] = r->size[i];
@@ -339,8 +338,7 @@ int mnvh_tensor_read(void* runtime, void* tensor, float* out, size_t out_capacit
     const Tensor& t = *static_cast<Tensor*>(tensor);
     size_t n = t->size.Prod();
     MNV_CHECK(n <= out_capacity) << "tensor has " << n << " floats, capacity " << out_capacity;
-    std::vector<float> host = static_cast<Runner*>(runtime)->Get(t);
-    std::memcpy(out, host.data(), n * sizeof(float));
+    static_cast<Runner*>(runtime)->Read(t, out);
   });
 }
 
@@ -445,8 +443,7 @@ int mnvh_net_read(void* net, const char* name, float* host_out, size_t floats) {
       t = jt->second;
     }
     MNV_CHECK_EQ(static_cast<size_t>(t->size.Prod()), floats) << "size of '" << name << "'";
-    std::vector<float> v = h->rt->Get(t);
-    std::memcpy(host_out, v.data(), floats * sizeof(float));
+    h->rt->Read(t, host_out);
   });
 }
 

@@ -1,6 +1,7 @@
 #include "hip_device.h"
 
 #include <cstdio>
+#include <cstring>
 
 #include "mnv_hip.h"
 
@@ -453,9 +454,40 @@ void HipDevice::Barrier(int thrid) {
 void HipDevice::CopyToHost(float* dst, uint64_t data_id, size_t floats) {
   MNV_CHECK(!capturing_) << "no host copies while a graph is recorded";
   Activate();
-  Ok(mnv_memcpy_d2h(dst, data_store_->GetData(data_id), floats * sizeof(float), streams_[0]),
-     "copy to host");
-  Ok(mnv_stream_sync(streams_[0]), "copy to host sync");
+  const char* src = reinterpret_cast<const char*>(data_store_->GetData(data_id));
+  char* out = reinterpret_cast<char*>(dst);
+  const size_t bytes = floats * sizeof(float), half = kStagingBytes / 2;
+  if (bytes <= half) {
+    Ok(mnv_memcpy_d2h(out, src, bytes, streams_[0]), "copy to host");
+    Ok(mnv_stream_sync(streams_[0]), "copy to host sync");
+    return;
+  }
+  // large results come back through the pinned staging area, the DMA engine filling one
+  // half while the CPU empties the other into the caller's pageable buffer
+  EnsureStaging(0);
+  char* stage = static_cast<char*>(staging_[0]);
+  void* filled[2] = {nullptr, nullptr};
+  Ok(mnv_event_create_ordering(&filled[0]), "event create");
+  Ok(mnv_event_create_ordering(&filled[1]), "event create");
+  const size_t chunks = (bytes + half - 1) / half;
+  auto issue = [&](size_t i) {
+    const size_t off = i * half, n = bytes - off < half ? bytes - off : half;
+    int rc = mnv_memcpy_d2h(stage + (i & 1) * half, src + off, n, streams_[0]);
+    if (rc == MNV_OK) rc = mnv_event_record(filled[i & 1], streams_[0]);
+    return rc;
+  };
+  int rc = issue(0);
+  for (size_t i = 0; i < chunks && rc == MNV_OK; ++i) {
+    if (i + 1 < chunks) rc = issue(i + 1);  // the other half is free: chunk i-1 was emptied
+    if (rc == MNV_OK) rc = mnv_event_sync(filled[i & 1]);
+    if (rc != MNV_OK) break;
+    const size_t off = i * half, n = bytes - off < half ? bytes - off : half;
+    std::memcpy(out + off, stage + (i & 1) * half, n);
+  }
+  mnv_stream_sync(streams_[0]);
+  mnv_event_destroy(filled[0]);
+  mnv_event_destroy(filled[1]);
+  Ok(rc, "copy to host");
 }
 
 void HipDevice::CopyFromHost(uint64_t data_id, const float* src, size_t floats) {

@@ -88,9 +88,14 @@ std::vector<Tensor> Runner::EndRetain() {
 
 std::vector<float> Runner::Get(const Tensor& t) {
   std::vector<float> host(t->size.Prod());
-  device_->Barrier(0);
-  device_->CopyToHost(host.data(), t->id, host.size());
+  Read(t, host.data());
   return host;
+}
+
+void Runner::Read(const Tensor& t, float* host) {
+  MNV_CHECK(t && host) << "null argument";
+  device_->Barrier(0);
+  device_->CopyToHost(host, t->id, t->size.Prod());
 }
 
 Tensor Runner::MakeNArray(const Scale& size, std::shared_ptr<float> host) {

@@ -43,6 +43,7 @@ class Runner : public DeviceListener {
   Tensor Compute(const std::vector<Tensor>& inputs, const Scale& out_size,
                  std::shared_ptr<ComputeFn> fn);
   std::vector<float> Get(const Tensor& t);
+  void Read(const Tensor& t, float* host);  // the same into the caller's buffer
   // Overwrites a tensor's device data in place (synchronous); its address is kept, which
   // is what a recorded graph that reads it needs.
   void Upload(const Tensor& t, const float* host);
