@@ -18,6 +18,7 @@
 // loads in flight (in registers) while they work on the current one; 3x3/2 and 2x2/2
 // windows are unrolled at compile time.  Planes too large for LDS take the direct kernels.
 #include <math.h>
+#include <stdlib.h>
 
 #include <algorithm>
 
@@ -347,6 +348,158 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_lds_kernel(
   }
 }
 
+// ---- max-pooling gradient of 3x3/2 and 2x2/2 windows: an ordered scatter in LDS --------
+// Every window's first maximum is found once and noted in LDS (position and pass); the
+// plane data is then cleared and the gradients are added to it window by window.  No
+// atomics and still the sums of a sequential scatter, bit for bit:
+//  * 2x2/2 windows do not overlap: one pass.
+//  * 3x3/2: a position with an odd (padded) coordinate lies in at most two windows, and a
+//    two-term sum does not depend on its order.  A position with both coordinates even
+//    lies in four windows, whose scan order is: the one that has it at its corner (2,2),
+//    then (2,0), then (0,2), then (0,0).  So the additions are made in four passes keyed by
+//    where in its window the maximum sits -- pass = 2*[row 0] + [column 0] -- with a
+//    barrier between passes.  Within a pass no two windows write the same position (equal
+//    row parity within a pass means equal row offset, hence the same window row; likewise
+//    for columns), so plain read-add-write is safe.
+// Against the gather kernel above this halves the integer work per element, which is what
+// bounds the gradient (the bytes moved are the same).
+// XV / DV: 16-byte vectors of plane data / top_diff a thread stages for the next group;
+// WPT: windows per thread and group.  The small configuration (4, 1, 4) keeps the kernel
+// under 64 registers so that eight workgroups share a CU: the phases of a group are
+// separated by barriers and bound by LDS latency, and more resident workgroups hide that.
+template <int KS, int ST, int XV, int DV, int WPT>
+__global__ __launch_bounds__(MNV_POOL_THREADS, XV <= 4 ? 7 : 4) void mnv_maxpool_bwd_scatter_kernel(
+    const float* __restrict__ bottom, const float* __restrict__ top_diff,
+    float* __restrict__ bottom_diff, int planes, int ppb, PoolGeom g) {
+  extern __shared__ float lds[];
+  const int hw = g.H * g.W, howo = g.Ho * g.Wo;
+  const size_t total_x = (size_t)planes * hw, total_d = (size_t)planes * howo;
+  const int groups = (planes + ppb - 1) / ppb;
+  // LDS: plane data [ppb*hw + 8], top_diff [ppb*howo + 8], window codes [ppb*howo]
+  float* lx = lds;
+  float* ld = lds + ((ppb * hw + 8 + 3) & ~3);
+  int* code = reinterpret_cast<int*>(ld + ((ppb * howo + 8 + 3) & ~3));
+  PoolStage<XV> sx;
+  PoolStage<DV> sd;
+  int grp = blockIdx.x;
+  if (grp < groups) {
+    const int p0 = grp * ppb, np = min(ppb, planes - p0);
+    sx.issue(bottom, total_x, (size_t)p0 * hw, np * hw);
+    sd.issue(top_diff, total_d, (size_t)p0 * howo, np * howo);
+  }
+  for (; grp < groups; grp += gridDim.x) {
+    const int p0 = grp * ppb, np = min(ppb, planes - p0);
+    const int shift_x = (int)(((size_t)p0 * hw) & 3);
+    const float* bd = ld + (int)(((size_t)p0 * howo) & 3);
+    __syncthreads();  // the previous group's gradients have left LDS
+    sx.commit(lx);
+    sd.commit(ld);
+    const int nxt = grp + gridDim.x;
+    if (nxt < groups) {
+      const int q0 = nxt * ppb, nq = min(ppb, planes - q0);
+      sx.issue(bottom, total_x, (size_t)q0 * hw, nq * hw);
+      sd.issue(top_diff, total_d, (size_t)q0 * howo, nq * howo);
+    }
+    __syncthreads();
+    // first maximum of every window: (LDS index of the position) * 4 + pass.  Two windows
+    // per thread and iteration, so that the LDS reads of one overlap the compares of the
+    // other; when every window of the wavefront lies inside its plane (all of them when
+    // nothing is padded or clipped) the two scans are straight-line code.
+    const int nwin = np * howo;
+    for (int q0 = 0; q0 < nwin; q0 += 2 * MNV_POOL_THREADS) {
+      int q[2], base[2], i[2], j[2], po[2];
+      bool inside = true;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        q[u] = q0 + threadIdx.x + u * MNV_POOL_THREADS;
+        const int qq = min(q[u], nwin - 1);  // a window past the end repeats the last one
+        const int pl = mnv_fastdiv(qq, g.d_howo), o = qq - m24(pl, howo);
+        i[u] = mnv_fastdiv(o, g.d_Wo);
+        j[u] = o - m24(i[u], g.Wo);
+        po[u] = shift_x + m24(pl, hw);
+        const int y0 = i[u] * ST - g.ph, x0 = j[u] * ST - g.pw;
+        base[u] = m24(y0, g.W) + x0;
+        inside = inside && y0 >= 0 && x0 >= 0 && y0 + KS <= g.H && x0 + KS <= g.W;
+      }
+      int arg[2], pass[2];
+      if (__all(inside)) {
+        float v[2][KS * KS];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int dy = 0; dy < KS; ++dy)
+#pragma unroll
+            for (int dx = 0; dx < KS; ++dx) v[u][dy * KS + dx] = lx[po[u] + base[u] + dy * g.W + dx];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          float r = -INFINITY;
+          int rel = 0, ps = 3;  // offset of the maximum from the window's corner, its pass
+#pragma unroll
+          for (int dy = 0; dy < KS; ++dy)
+#pragma unroll
+            for (int dx = 0; dx < KS; ++dx)
+              if (r < v[u][dy * KS + dx]) {
+                r = v[u][dy * KS + dx];
+                rel = dy * g.W + dx;
+                ps = (dy == 0 ? 2 : 0) + (dx == 0 ? 1 : 0);
+              }
+          arg[u] = base[u] + rel;
+          pass[u] = KS == 3 ? ps : 0;
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          pool_window<true, KS, ST>(lx + po[u], g, i[u], j[u], &arg[u]);
+          pass[u] = 0;
+          if (KS == 3) {
+            const int y = mnv_fastdiv(arg[u], g.d_W), x = arg[u] - m24(y, g.W);
+            pass[u] = (y == i[u] * ST - g.ph ? 2 : 0) + (x == j[u] * ST - g.pw ? 1 : 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+        if (q[u] < nwin) code[q[u]] = ((po[u] + arg[u]) << 2) | pass[u];
+    }
+    __syncthreads();  // every window has read the plane data: the planes become the gradient
+    // this thread's windows, read once for all passes (at most WPT of them)
+    int wc[WPT];
+    float wd[WPT];
+#pragma unroll
+    for (int k = 0; k < WPT; ++k) {
+      const int q = threadIdx.x + k * MNV_POOL_THREADS;
+      const bool in = q < np * howo;
+      wc[k] = in ? code[q] : -1;
+      wd[k] = in ? bd[q] : 0.f;
+    }
+    const int nv = (shift_x + np * hw + 3) >> 2;
+    for (int v = threadIdx.x; v < nv; v += MNV_POOL_THREADS)
+      reinterpret_cast<mnv_f4*>(lx)[v] = mnv_f4{0.f, 0.f, 0.f, 0.f};
+    __syncthreads();
+#pragma unroll
+    for (int pass = 0; pass < (KS == 3 ? 4 : 1); ++pass) {
+#pragma unroll
+      for (int k = 0; k < WPT; ++k)
+        if (wc[k] >= 0 && (wc[k] & 3) == pass) lx[wc[k] >> 2] += wd[k];
+      __syncthreads();
+    }
+    {
+      const int cnt = np * hw;
+      float* gout = bottom_diff + (((size_t)p0 * hw) & ~(size_t)3);  // 16-byte aligned
+      for (int v = threadIdx.x; v < nv; v += MNV_POOL_THREADS) {
+        const int e0 = 4 * v - shift_x;  // position of the vector's first float in the group
+        if (e0 >= 0 && e0 + 4 <= cnt) {
+          __builtin_nontemporal_store(*reinterpret_cast<const mnv_f4*>(lx + 4 * v),
+                                      reinterpret_cast<mnv_f4*>(gout) + v);
+        } else {  // the group's first and last vector may be shared with its neighbours
+          for (int k = 0; k < 4; ++k)
+            if (e0 + k >= 0 && e0 + k < cnt) gout[4 * v + k] = lx[4 * v + k];
+        }
+      }
+    }
+  }
+}
+
 // ---- direct kernels for planes that do not fit in LDS -------------------------------
 template <bool MAX>
 __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_fwd_kernel(
@@ -472,13 +625,16 @@ int planes_per_block(const PoolGeom& g, long long planes, bool bwd) {
   return (int)ppb;
 }
 
-// Workgroups of a pipelined launch: all that fit on the chip at once, each looping over
-// its share of the groups.
-unsigned lds_grid(long long groups, size_t lds_bytes) {
+// Workgroups of a pipelined launch: `rounds` times what fits on the chip at once, each
+// looping over its share of the groups.  One round keeps every workgroup resident for the
+// whole kernel; several rounds let the dispatcher hand the slots of workgroups that
+// finish early to new ones, which evens out the spread between CUs (the forward kernel
+// gains 7% from six rounds, the gradient kernels nothing).
+unsigned lds_grid(long long groups, size_t lds_bytes, int rounds = 1) {
   long long per_cu = (160 * 1024) / (long long)(lds_bytes + 512);
   if (per_cu > 8) per_cu = 8;
   if (per_cu < 1) per_cu = 1;
-  long long blocks = 256 * per_cu;
+  long long blocks = 256 * per_cu * rounds;
   return (unsigned)(groups < blocks ? groups : blocks);
 }
 
@@ -498,7 +654,7 @@ int pool_fwd(const float* bottom, float* top, int n, int c, int h, int w, int sv
     auto kernel = (sq && kh == 3 && sv == 2)   ? mnv_pool_fwd_lds_kernel<MAX, 3, 2>
                   : (sq && kh == 2 && sv == 2) ? mnv_pool_fwd_lds_kernel<MAX, 2, 2>
                                                : mnv_pool_fwd_lds_kernel<MAX, 0, 0>;
-    hipLaunchKernelGGL(kernel, dim3(lds_grid(groups, lds)), dim3(MNV_POOL_THREADS), lds,
+    hipLaunchKernelGGL(kernel, dim3(lds_grid(groups, lds, 6)), dim3(MNV_POOL_THREADS), lds,
                        mnv_stream(stream), bottom, top, (int)planes, ppb, g);
   } else {
     hipLaunchKernelGGL((mnv_pool_fwd_kernel<MAX>), dim3(pool_grid((size_t)planes * g.Ho * g.Wo)),
@@ -516,9 +672,35 @@ int pool_bwd(const float* bottom, const float* top_diff, float* bottom_diff, int
   int rc = make_geom(&g, n, c, h, w, sv, sh, kh, kw, ph, pw);
   if (rc) return rc;
   long long planes = (long long)n * c;
-  int ppb = (mnv_aligned16(bottom) && mnv_aligned16(top_diff) && mnv_aligned16(bottom_diff))
-                ? planes_per_block(g, planes, true)
-                : 0;
+  const bool aligned = mnv_aligned16(bottom) && mnv_aligned16(top_diff) && mnv_aligned16(bottom_diff);
+  if (MAX && aligned && kh == kw && sv == sh && sv == 2 && (kh == 2 || kh == 3)) {
+    const long long hw = (long long)h * w, howo = (long long)g.Ho * g.Wo;
+    // small configuration first: planes that fit 4 staged vectors and 4 windows per thread
+    long long small = std::min((long long)(MNV_POOL_THREADS * 4 * 4 - 6) / hw,
+                               std::min((long long)(MNV_POOL_THREADS * 4 * 1 - 6) / howo,
+                                        (long long)(4 * MNV_POOL_THREADS) / howo));
+    long long big = std::min((long long)planes_per_block(g, planes, true),
+                             (long long)(8 * MNV_POOL_THREADS) / howo);
+    const long long cap = std::max(1LL, planes / 4096);
+    small = std::min(small, cap);
+    // one large plane per group leaves the small configuration's window slots a quarter
+    // empty: such planes go two to a group in the large one
+    const bool use_small = small >= 2 || (small == 1 && big <= 1);
+    const int spb = (int)(use_small ? small : big);
+    if (spb > 0) {
+      const size_t lds = ((((size_t)spb * hw + 8 + 3) & ~(size_t)3) + (((size_t)spb * howo + 8 + 3) & ~(size_t)3) +
+                          (size_t)spb * howo) * sizeof(float);
+      const long long groups = (planes + spb - 1) / spb;
+      auto kernel = kh == 3 ? (use_small ? mnv_maxpool_bwd_scatter_kernel<3, 2, 4, 1, 4>
+                                         : mnv_maxpool_bwd_scatter_kernel<3, 2, 8, 4, 8>)
+                            : (use_small ? mnv_maxpool_bwd_scatter_kernel<2, 2, 4, 1, 4>
+                                         : mnv_maxpool_bwd_scatter_kernel<2, 2, 8, 4, 8>);
+      hipLaunchKernelGGL(kernel, dim3(lds_grid(groups, lds)), dim3(MNV_POOL_THREADS), lds,
+                         mnv_stream(stream), bottom, top_diff, bottom_diff, (int)planes, spb, g);
+      return MNV_LAUNCH_STATUS();
+    }
+  }
+  int ppb = aligned ? planes_per_block(g, planes, true) : 0;
   if (ppb > 0) {
     const size_t hw = (size_t)h * w, howo = (size_t)g.Ho * g.Wo;
     size_t lds = (((ppb * hw + 8 + 3) & ~(size_t)3) + ((ppb * howo + 8 + 3) & ~(size_t)3) +
