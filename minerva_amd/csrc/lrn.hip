@@ -36,7 +36,6 @@ namespace {
 
 
 #define MNV_LRN_THREADS 256
-#define MNV_LRN_ST_AUX 2  // nt bit of the 16-byte stores
 
 // s^e for s >= 1 through the hardware log2 / exp2: relative error ~1e-6
 __device__ __forceinline__ float pow_ge1(float s, float e) { return __expf(e * __logf(s)); }
@@ -136,14 +135,17 @@ __device__ __forceinline__ LrnVec<2> lrn_load<2>(mnv_rsrc r, unsigned voff, unsi
   f2 t = __builtin_bit_cast(f2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)voff, (int)soff, 0));
   return LrnVec<2>{{t.x, t.y}};
 }
-template <int V>
+// NT: the 16-byte stores bypass the caches (for tensors that cannot stay in the 256 MB
+// last-level cache anyway; smaller ones are written through it: 51% -> 66% of HBM peak on
+// the norm1 shape, while 256 x 96 x 55 x 55 is 4% faster the other way).
+template <int V, bool NT>
 __device__ __forceinline__ void lrn_store(mnv_rsrc r, unsigned voff, unsigned soff, const float (&o)[V],
                                           int valid) {
   if (valid == V) {
     if (V == 4) {
       mnv_f4 t = {o[0], o[1], o[2], o[3 % V]};
       __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, t),
-                                             r, (int)voff, (int)soff, MNV_LRN_ST_AUX);
+                                             r, (int)voff, (int)soff, NT ? 2 : 0);
     } else {
       typedef float f2 __attribute__((ext_vector_type(2)));
       f2 t = {o[0], o[1]};
@@ -159,7 +161,7 @@ __device__ __forceinline__ void lrn_store(mnv_rsrc r, unsigned voff, unsigned so
   }
 }
 
-template <int SIZE, int G, int V>
+template <int SIZE, int G, int V, bool NT>
 __global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_fwd_ring_kernel(
     const float* __restrict__ bottom, float* __restrict__ scale, float* __restrict__ top,
     float alpha_over_size, float negative_beta, int channels, int hw, int groups_per_image,
@@ -222,8 +224,8 @@ __global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_fwd_ring_kernel(
             s[t] = 1.f + accum[t] * alpha_over_size;
             o[t] = win[(u - post_pad + SIZE) % SIZE].v[t] * pow_ge1(s[t], negative_beta);
           }
-          lrn_store<V>(rsc, voff, (unsigned)c * cstep, s, valid);
-          lrn_store<V>(rtop, voff, (unsigned)c * cstep, o, valid);
+          lrn_store<V, NT>(rsc, voff, (unsigned)c * cstep, s, valid);
+          lrn_store<V, NT>(rtop, voff, (unsigned)c * cstep, o, valid);
         }
       }
     }
@@ -309,7 +311,7 @@ __global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_bwd_ring_kernel(
           for (int t = 0; t < V; ++t)
             o[t] = dwin[slot].v[t] * pow_ge1(swin[slot].v[t], negative_beta) -
                    cache_ratio * cx[u].v[t] * accum[t];
-          lrn_store<V>(rdx, voff, (unsigned)c * cstep, o, valid);
+          lrn_store<V, false>(rdx, voff, (unsigned)c * cstep, o, valid);
         }
       }
     }
@@ -368,12 +370,23 @@ int mnv_lrn_fwd(const float* bottom, float* scale, float* top, int local_size, f
     lrn_segments(groups, channels, local_size, &seg_len, &nseg);
     const dim3 grid(lrn_grid(groups * nseg));
     const MnvFastDiv d = mnv_fastdiv_make(gpi), dg = mnv_fastdiv_make((int)groups);
-#define MNV_LRN_FWD(SIZE, G)                                                                       \
-  hipLaunchKernelGGL((mnv_lrn_fwd_ring_kernel<SIZE, G, V>), grid, block, 0, s, bottom, scale, top, \
-                     aos, -beta, channels, hw, gpi, groups, (unsigned)bytes, d, seg_len, nseg, dg)
-    if (local_size == 3) MNV_LRN_FWD(3, 6);
-    else if (local_size == 5) MNV_LRN_FWD(5, 5);
-    else MNV_LRN_FWD(7, 7);
+    const bool nt = 3 * bytes >= ((size_t)512 << 20);
+#define MNV_LRN_FWD(SIZE, G)                                                                        \
+  if (nt)                                                                                           \
+    hipLaunchKernelGGL((mnv_lrn_fwd_ring_kernel<SIZE, G, V, true>), grid, block, 0, s, bottom,      \
+                       scale, top, aos, -beta, channels, hw, gpi, groups, (unsigned)bytes, d,       \
+                       seg_len, nseg, dg);                                                          \
+  else                                                                                              \
+    hipLaunchKernelGGL((mnv_lrn_fwd_ring_kernel<SIZE, G, V, false>), grid, block, 0, s, bottom,     \
+                       scale, top, aos, -beta, channels, hw, gpi, groups, (unsigned)bytes, d,       \
+                       seg_len, nseg, dg)
+    if (local_size == 3) {
+      MNV_LRN_FWD(3, 6);
+    } else if (local_size == 5) {
+      MNV_LRN_FWD(5, 5);
+    } else {
+      MNV_LRN_FWD(7, 7);
+    }
 #undef MNV_LRN_FWD
   } else {
     hipLaunchKernelGGL(mnv_lrn_fwd_kernel, dim3(lrn_grid(positions)), block, 0, s, bottom, scale, top,
