@@ -255,6 +255,13 @@ def bandwidth_table(L, dev, x, y, z, ne):
     # beta 0.75): forward reads bottom and writes scale and top, backward reads four tensors
     lsc, ltop = dev.empty(nin), dev.empty(nin)
     lrn = (5, f(1e-4), f(0.75), 256, 96, 55, 55)
+    # The same copy, fill and read kernels on the 297 MB tensors used below: what plain
+    # streaming reaches once the operands are past the 256 MB last-level cache, the yardstick
+    # for the pooling and LRN rows (whose traffic is two to five such tensors)
+    extra += [
+        ("copy, 297 MB tensors", 8 * nin, lambda: L.mnv_copy(px.p, z2.p, nin, S)),
+        ("fill, 297 MB tensor", 4 * nin, lambda: L.mnv_fill(z2.p, nin, f(1.0), S)),
+    ]
     extra += [
         ("lrn fwd (norm1)", 12 * nin, lambda: L.mnv_lrn_fwd(px.p, lsc.p, ltop.p, *lrn, S)),
         ("lrn bwd (norm1)", 20 * nin,
