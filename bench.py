@@ -258,8 +258,12 @@ def bandwidth_table(L, dev, x, y, z, ne):
     # The same copy, fill and read kernels on the 297 MB tensors used below: what plain
     # streaming reaches once the operands are past the 256 MB last-level cache, the yardstick
     # for the pooling and LRN rows (whose traffic is two to five such tensors)
+    nbig = 3 * nin // 2
+    big_a, big_b = dev.empty(nbig), dev.empty(nbig)
+    L.mnv_fill(big_a.p, nbig, f(1.0), S)
     extra += [
-        ("copy, 297 MB tensors", 8 * nin, lambda: L.mnv_copy(px.p, z2.p, nin, S)),
+        ("copy, 594 MB footprint", 8 * nin, lambda: L.mnv_copy(px.p, z2.p, nin, S)),
+        ("copy, 892 MB footprint", 8 * nbig, lambda: L.mnv_copy(big_a.p, big_b.p, nbig, S)),
         ("fill, 297 MB tensor", 4 * nin, lambda: L.mnv_fill(z2.p, nin, f(1.0), S)),
     ]
     extra += [
