@@ -183,100 +183,115 @@ def micro_bench():
                        "tflops": round(2.0 * mm * nn * kk / (t * 1e-3) / 1e12, 2)})
     sgemm["other_shapes"] = shapes
     ne = 8192 * 8192
-    # three distinct 256 MiB buffers: 768 MiB per pass, larger than the 256 MB last-level cache
-    x = dev.upload(rng.standard_normal(ne, dtype=np.float32))
-    y = dev.upload(rng.standard_normal(ne, dtype=np.float32))
-    z = dev.empty(ne)
-    ms = dev.time_ms(lambda: L.mnv_add(x.p, y.p, z.p, ne, dev.stream), iters=50, warmup=5)
-    gbs = 12.0 * ne / (ms * 1e-3) / 1e9
-    elt = {"op": "add 8192x8192", "ms": round(ms, 4), "gbs": round(gbs, 1),
-           "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
-                        "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}}
-    log("add 8192^2: %.4f ms, %.0f GB/s" % (ms, gbs))
-    elt["ops"] = bandwidth_table(L, dev, x, y, z, ne)
+    elt = bandwidth_table(L, dev, rng, ne)
+    log("add 8192^2: %.4f ms, %.0f GB/s" % (elt["ms"], elt["gbs"]))
     return sgemm, elt
 
 
-def bandwidth_table(L, dev, x, y, z, ne):
+ROTATE = 4  # buffer sets an HBM-bound operator cycles through, so that no pass finds its
+            # operands in the 256 MB last-level cache left there by the previous pass
+
+
+def rotating(dev, make_call, sets):
+    """Average ms per call of an operator that takes the next of `sets` on every call."""
+    import itertools
+    count = itertools.count()
+    calls = [make_call(*s) for s in sets]
+    return dev.time_ms(lambda: calls[next(count) % len(calls)](), iters=6 * len(calls),
+                       warmup=2 * len(calls))
+
+
+def bandwidth_table(L, dev, rng, ne):
     """The 8192^2 bandwidth microbenchmark (BASELINE.json configs[1]): GB/s from the
-    algorithmic bytes per element of each operator."""
+    algorithmic bytes per element of each operator, every operator cycling through ROTATE
+    sets of operands (with one set, 30-40% of a 268 MB operand is still in the last-level
+    cache when the next pass starts, and the same kernels read 87-92% of peak instead of
+    75-80%: reported as `gbs_one_set`)."""
     m = n = 8192
     S = dev.stream
+    host_x = rng.standard_normal(ne, dtype=np.float32)
+    host_y = rng.standard_normal(ne, dtype=np.float32)
+    sets = [(dev.upload(host_x), dev.upload(host_y), dev.empty(ne)) for _ in range(ROTATE)]
     vec = dev.upload(np.random.default_rng(8).standard_normal(m, dtype=np.float32))
     small = dev.empty(m)
     f = ctypes.c_float
     ops = [
-        ("copy", 8, lambda: L.mnv_copy(x.p, z.p, ne, S)),
-        ("mul", 12, lambda: L.mnv_mul(x.p, y.p, z.p, ne, S)),
-        ("sub", 12, lambda: L.mnv_sub(x.p, y.p, z.p, ne, S)),
-        ("scalar mul", 8, lambda: L.mnv_const_mul(x.p, z.p, f(3.291), ne, S)),
-        ("broadcast add {1,n}", 8, lambda: L.mnv_norm_add_col(x.p, vec.p, z.p, m, n, S)),
-        ("broadcast add {m,1}", 8, lambda: L.mnv_norm_add_row(x.p, vec.p, z.p, m, n, S)),
-        ("sigmoid fwd", 8, lambda: L.mnv_sigmoid_fwd(x.p, z.p, ne, S)),
-        ("relu fwd", 8, lambda: L.mnv_relu_fwd(x.p, z.p, ne, S)),
-        ("tanh fwd", 8, lambda: L.mnv_tanh_fwd(x.p, z.p, ne, S)),
-        ("sigmoid bwd", 12, lambda: L.mnv_sigmoid_bwd(x.p, x.p, y.p, z.p, ne, S)),
-        ("relu bwd", 12, lambda: L.mnv_relu_bwd(x.p, x.p, y.p, z.p, ne, S)),
-        ("tanh bwd", 12, lambda: L.mnv_tanh_bwd(x.p, x.p, y.p, z.p, ne, S)),
-        ("sum dim 0", 4, lambda: L.mnv_reduce_sum_col(x.p, small.p, m, n, S)),
-        ("sum dim 1", 4, lambda: L.mnv_reduce_sum_row(x.p, small.p, m, n, S)),
-        ("max dim 0", 4, lambda: L.mnv_reduce_max_col(x.p, small.p, m, n, S)),
-        ("max dim 1", 4, lambda: L.mnv_reduce_max_row(x.p, small.p, m, n, S)),
-        ("maxindex dim 0", 4, lambda: L.mnv_maxindex_col(x.p, small.p, m, n, S)),
-        ("softmax rows", 8, lambda: L.mnv_softmax_instance_fwd(x.p, z.p, n, m, 1, 1, S)),
-        ("softmax rows bwd", 12, lambda: L.mnv_softmax_instance_bwd(x.p, y.p, z.p, n, m, 1, 1, S)),
-        ("transpose", 8, lambda: L.mnv_transpose(x.p, z.p, m, n, S)),
+        ("add", 12, lambda x, y, z: lambda: L.mnv_add(x.p, y.p, z.p, ne, S)),
+        ("copy", 8, lambda x, y, z: lambda: L.mnv_copy(x.p, z.p, ne, S)),
+        ("mul", 12, lambda x, y, z: lambda: L.mnv_mul(x.p, y.p, z.p, ne, S)),
+        ("sub", 12, lambda x, y, z: lambda: L.mnv_sub(x.p, y.p, z.p, ne, S)),
+        ("scalar mul", 8, lambda x, y, z: lambda: L.mnv_const_mul(x.p, z.p, f(3.291), ne, S)),
+        ("broadcast add {1,n}", 8, lambda x, y, z: lambda: L.mnv_norm_add_col(x.p, vec.p, z.p, m, n, S)),
+        ("broadcast add {m,1}", 8, lambda x, y, z: lambda: L.mnv_norm_add_row(x.p, vec.p, z.p, m, n, S)),
+        ("sigmoid fwd", 8, lambda x, y, z: lambda: L.mnv_sigmoid_fwd(x.p, z.p, ne, S)),
+        ("relu fwd", 8, lambda x, y, z: lambda: L.mnv_relu_fwd(x.p, z.p, ne, S)),
+        ("tanh fwd", 8, lambda x, y, z: lambda: L.mnv_tanh_fwd(x.p, z.p, ne, S)),
+        ("sigmoid bwd", 12, lambda x, y, z: lambda: L.mnv_sigmoid_bwd(x.p, x.p, y.p, z.p, ne, S)),
+        ("relu bwd", 12, lambda x, y, z: lambda: L.mnv_relu_bwd(x.p, x.p, y.p, z.p, ne, S)),
+        ("tanh bwd", 12, lambda x, y, z: lambda: L.mnv_tanh_bwd(x.p, x.p, y.p, z.p, ne, S)),
+        ("sum dim 0", 4, lambda x, y, z: lambda: L.mnv_reduce_sum_col(x.p, small.p, m, n, S)),
+        ("sum dim 1", 4, lambda x, y, z: lambda: L.mnv_reduce_sum_row(x.p, small.p, m, n, S)),
+        ("max dim 0", 4, lambda x, y, z: lambda: L.mnv_reduce_max_col(x.p, small.p, m, n, S)),
+        ("max dim 1", 4, lambda x, y, z: lambda: L.mnv_reduce_max_row(x.p, small.p, m, n, S)),
+        ("maxindex dim 0", 4, lambda x, y, z: lambda: L.mnv_maxindex_col(x.p, small.p, m, n, S)),
+        ("softmax rows", 8, lambda x, y, z: lambda: L.mnv_softmax_instance_fwd(x.p, z.p, n, m, 1, 1, S)),
+        ("softmax rows bwd", 12, lambda x, y, z: lambda: L.mnv_softmax_instance_bwd(x.p, y.p, z.p, n, m, 1, 1, S)),
+        ("transpose", 8, lambda x, y, z: lambda: L.mnv_transpose(x.p, z.p, m, n, S)),
     ]
     table = []
-    for name, bpe, fn in ops:
-        ms = dev.time_ms(fn, iters=20, warmup=3)
+    for name, bpe, make in ops:
+        ms = rotating(dev, make, sets)
+        ms_one = dev.time_ms(make(*sets[0]), iters=10, warmup=3)
         gbs = bpe * ne / (ms * 1e-3) / 1e9
         table.append({"op": name, "ms": round(ms, 4), "gbs": round(gbs, 1),
-                      "frac": round(gbs / PEAK_HBM_GBS, 4)})
-    # AlexNet pool1 at batch 256 ({55,55,96,256} -> {27,27,96,256}, 3x3 stride 2) and the
-    # conv1 bias gradient, in the same buffers: bytes = every tensor once
+                      "frac": round(gbs / PEAK_HBM_GBS, 4),
+                      "gbs_one_set": round(bpe * ne / (ms_one * 1e-3) / 1e9, 1)})
+    add = table[0]
+    elt = {"op": "add 8192x8192", "ms": add["ms"], "gbs": add["gbs"],
+           "roofline": {"bound": "hbm", "achieved": add["gbs"], "peak": PEAK_HBM_GBS,
+                        "unit": "GB/s", "frac": add["frac"]},
+           "buffer_sets": ROTATE}
+    del sets
+    # AlexNet pool1 at batch 256 ({55,55,96,256} -> {27,27,96,256}, 3x3 stride 2), the conv1
+    # bias gradient and LRN over the same tensor (Caffe-style norm1: local_size 5, alpha 1e-4,
+    # beta 0.75), two sets of 297 MB tensors each: bytes = every tensor once
     geo = (256, 96, 55, 55, 2, 2, 3, 3, 0, 0)
-    nin, nout = 256 * 96 * 55 * 55, 256 * 96 * 27 * 27
-    px = dev.upload(np.random.default_rng(9).standard_normal(nin, dtype=np.float32))
-    py, pdy, pdx = dev.empty(nout), dev.empty(nout), dev.empty(nin)
-    L.mnv_fill(pdy.p, nout, f(0.5), S)
-    bias_ws = dev.empty(1 << 18)  # 1 MiB
-    z2 = dev.empty(nin)
-    assert px.n == nin and pdx.n == nin and py.n == nout and pdy.n == nout and small.n >= 96
-    extra = [
-        ("maxpool 3x3/2 fwd (pool1)", 4 * (nin + nout), lambda: L.mnv_maxpool_fwd(px.p, py.p, *geo, S)),
-        ("maxpool 3x3/2 bwd (pool1)", 4 * (2 * nin + nout),
-         lambda: L.mnv_maxpool_bwd(px.p, py.p, pdy.p, pdx.p, *geo, S)),
-        ("conv bias gradient (conv1)", 4 * nin,
-         lambda: L.mnv_conv_bwd_bias(px.p, small.p, 256, 96, 55, 55, bias_ws.p,
-                                     ctypes.c_size_t(1 << 20), S)),
-    ]
-    # LRN over the same {55,55,96,256} tensor (Caffe-style norm1: local_size 5, alpha 1e-4,
-    # beta 0.75): forward reads bottom and writes scale and top, backward reads four tensors
-    lsc, ltop = dev.empty(nin), dev.empty(nin)
     lrn = (5, f(1e-4), f(0.75), 256, 96, 55, 55)
-    # The same copy, fill and read kernels on the 297 MB tensors used below: what plain
-    # streaming reaches once the operands are past the 256 MB last-level cache, the yardstick
-    # for the pooling and LRN rows (whose traffic is two to five such tensors)
-    nbig = 3 * nin // 2
-    big_a, big_b = dev.empty(nbig), dev.empty(nbig)
-    L.mnv_fill(big_a.p, nbig, f(1.0), S)
-    extra += [
-        ("copy, 594 MB footprint", 8 * nin, lambda: L.mnv_copy(px.p, z2.p, nin, S)),
-        ("copy, 892 MB footprint", 8 * nbig, lambda: L.mnv_copy(big_a.p, big_b.p, nbig, S)),
-        ("fill, 297 MB tensor", 4 * nin, lambda: L.mnv_fill(z2.p, nin, f(1.0), S)),
-    ]
-    extra += [
-        ("lrn fwd (norm1)", 12 * nin, lambda: L.mnv_lrn_fwd(px.p, lsc.p, ltop.p, *lrn, S)),
+    nin, nout = 256 * 96 * 55 * 55, 256 * 96 * 27 * 27
+    host_p = np.random.default_rng(9).standard_normal(nin, dtype=np.float32)
+    big = []
+    for _ in range(2):
+        px, py, pdy = dev.upload(host_p), dev.empty(nout), dev.empty(nout)
+        o1, o2, o3, o4 = dev.empty(nin), dev.empty(nin), dev.empty(nin), dev.empty(nin)
+        L.mnv_fill(o4.p, nin, f(0.25), S)  # a top_diff of its own for the LRN gradient
+        L.mnv_fill(pdy.p, nout, f(0.5), S)
+        L.mnv_maxpool_fwd(px.p, py.p, *geo, S)
+        L.mnv_lrn_fwd(px.p, o1.p, o2.p, *lrn, S)  # o1 = scale, o2 = top for the backward row
+        assert px.n == nin and o1.n == nin and py.n == nout and pdy.n == nout
+        big.append((px, py, pdy, o1, o2, o3, o4))
+    bias_ws = dev.empty(1 << 18)  # 1 MiB
+    extra = [
+        ("maxpool 3x3/2 fwd (pool1)", 4 * (nin + nout),
+         lambda px, py, pdy, o1, o2, o3, o4: lambda: L.mnv_maxpool_fwd(px.p, py.p, *geo, S)),
+        ("maxpool 3x3/2 bwd (pool1)", 4 * (2 * nin + nout),
+         lambda px, py, pdy, o1, o2, o3, o4: lambda: L.mnv_maxpool_bwd(px.p, py.p, pdy.p, o3.p, *geo, S)),
+        ("conv bias gradient (conv1)", 4 * nin,
+         lambda px, py, pdy, o1, o2, o3, o4: lambda: L.mnv_conv_bwd_bias(
+             px.p, small.p, 256, 96, 55, 55, bias_ws.p, ctypes.c_size_t(1 << 20), S)),
+        ("copy, 297 MB tensors", 8 * nin,
+         lambda px, py, pdy, o1, o2, o3, o4: lambda: L.mnv_copy(px.p, o3.p, nin, S)),
         ("lrn bwd (norm1)", 20 * nin,
-         lambda: L.mnv_lrn_bwd(px.p, ltop.p, lsc.p, pdx.p, z2.p, *lrn, S)),
+         lambda px, py, pdy, o1, o2, o3, o4: lambda: L.mnv_lrn_bwd(px.p, o2.p, o1.p, o4.p, o3.p, *lrn, S)),
+        ("lrn fwd (norm1)", 12 * nin,
+         lambda px, py, pdy, o1, o2, o3, o4: lambda: L.mnv_lrn_fwd(px.p, o1.p, o2.p, *lrn, S)),
     ]
-    for name, nbytes, fn in extra:
-        ms = dev.time_ms(fn, iters=20, warmup=3)
+    for name, nbytes, make in extra:
+        ms = rotating(dev, make, big)
         gbs = nbytes / (ms * 1e-3) / 1e9
         table.append({"op": name, "ms": round(ms, 4), "gbs": round(gbs, 1),
                       "frac": round(gbs / PEAK_HBM_GBS, 4)})
-    return table
+    elt["ops"] = table
+    return elt
 
 
 def small_nets(steps=20, warmup=3):

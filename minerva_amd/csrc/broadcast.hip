@@ -38,7 +38,7 @@ __global__ __launch_bounds__(MNV_BC_THREADS) void mnv_norm_kernel(
 #pragma unroll
       for (int u = 0; u < MNV_BC_COLS; ++u)
         if (c0 + u < n)
-          v[u] = *reinterpret_cast<const mnv_f4*>(mat + (size_t)(c0 + u) * m + r0);
+          v[u] = mnv_ldx4<NT>(reinterpret_cast<const mnv_f4*>(mat + (size_t)(c0 + u) * m + r0));
 #pragma unroll
       for (int u = 0; u < MNV_BC_COLS; ++u)
         if (c0 + u < n) {

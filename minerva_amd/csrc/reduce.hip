@@ -20,6 +20,7 @@ namespace {
 #define MNV_NONE 0x7fffffff
 
 struct SumAcc {
+  static constexpr int ROW_UNROLL = 2;  // columns in flight per thread in the row reducer
   float s;
   __device__ void init() { s = 0.f; }
   __device__ void push(float v, int) { s += v; }
@@ -34,6 +35,7 @@ struct SumAcc {
 };
 
 struct ArgAcc {
+  static constexpr int ROW_UNROLL = 4;
   float v;
   int idx;
   __device__ void init() {
@@ -83,7 +85,7 @@ struct EmitIndex {
 // ---------------------------------------------------------------------------
 #define MNV_RC_THREADS 256
 
-template <class Acc, class Emit, int GROUP, bool VEC4>
+template <class Acc, class Emit, int GROUP, bool VEC4, bool NT>
 __global__ __launch_bounds__(MNV_RC_THREADS) void mnv_reduce_col_kernel(
     const float* __restrict__ in, float* __restrict__ out, int m, int n) {
   constexpr int COLS = MNV_RC_THREADS / GROUP;
@@ -100,13 +102,13 @@ __global__ __launch_bounds__(MNV_RC_THREADS) void mnv_reduce_col_kernel(
       int i = t;
       // two independent 16-byte loads in flight per thread
       for (; i + GROUP < m4; i += 2 * GROUP) {
-        mnv_f4 a = col4[i], b = col4[i + GROUP];
+        mnv_f4 a = mnv_ldx4<NT>(col4 + i), b = mnv_ldx4<NT>(col4 + i + GROUP);
         acc.push(a.x, 4 * i); acc.push(a.y, 4 * i + 1); acc.push(a.z, 4 * i + 2); acc.push(a.w, 4 * i + 3);
         int j = i + GROUP;
         acc.push(b.x, 4 * j); acc.push(b.y, 4 * j + 1); acc.push(b.z, 4 * j + 2); acc.push(b.w, 4 * j + 3);
       }
       if (i < m4) {
-        mnv_f4 a = col4[i];
+        mnv_f4 a = mnv_ldx4<NT>(col4 + i);
         acc.push(a.x, 4 * i); acc.push(a.y, 4 * i + 1); acc.push(a.z, 4 * i + 2); acc.push(a.w, 4 * i + 3);
       }
     } else {
@@ -135,22 +137,29 @@ int launch_reduce_col(const float* in, float* out, int m, int n, mnv_stream_t st
   if (!in || !out || m <= 0 || n < 0) return MNV_ERR_INVALID;
   hipStream_t s = mnv_stream(stream);
   bool vec4 = (m % 4 == 0) && mnv_aligned16(in);
+  const bool big = (size_t)m * n * sizeof(float) >= MNV_PAST_CACHE_BYTES;
   if (m > 2048) {
     unsigned grid = (unsigned)(n < 65536 ? n : 65536);
-    if (vec4)
-      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_RC_THREADS, true>), dim3(grid),
+    if (vec4 && big)
+      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_RC_THREADS, true, true>), dim3(grid),
+                         dim3(MNV_RC_THREADS), 0, s, in, out, m, n);
+    else if (vec4)
+      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_RC_THREADS, true, false>), dim3(grid),
                          dim3(MNV_RC_THREADS), 0, s, in, out, m, n);
     else
-      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_RC_THREADS, false>), dim3(grid),
+      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_RC_THREADS, false, false>), dim3(grid),
                          dim3(MNV_RC_THREADS), 0, s, in, out, m, n);
   } else {
     size_t blocks = mnv_ceil_div((size_t)n, MNV_RC_THREADS / MNV_WAVE);
     unsigned grid = (unsigned)(blocks < 65536 ? blocks : 65536);
-    if (vec4)
-      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_WAVE, true>), dim3(grid),
+    if (vec4 && big)
+      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_WAVE, true, true>), dim3(grid),
+                         dim3(MNV_RC_THREADS), 0, s, in, out, m, n);
+    else if (vec4)
+      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_WAVE, true, false>), dim3(grid),
                          dim3(MNV_RC_THREADS), 0, s, in, out, m, n);
     else
-      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_WAVE, false>), dim3(grid),
+      hipLaunchKernelGGL((mnv_reduce_col_kernel<Acc, Emit, MNV_WAVE, false, false>), dim3(grid),
                          dim3(MNV_RC_THREADS), 0, s, in, out, m, n);
   }
   return MNV_LAUNCH_STATUS();
@@ -161,7 +170,7 @@ int launch_reduce_col(const float* in, float* out, int m, int n, mnv_stream_t st
 // A workgroup owns RL*W consecutive rows (128 contiguous bytes per column) and
 // splits the columns over CG thread groups; partial results meet in LDS.
 // ---------------------------------------------------------------------------
-template <class Acc, class Emit, int RL, int CG, bool VEC4>
+template <class Acc, class Emit, int RL, int CG, bool VEC4, bool NT>
 __global__ __launch_bounds__(RL* CG) void mnv_reduce_row_kernel(const float* __restrict__ in,
                                                                 float* __restrict__ out, int m,
                                                                 int n) {
@@ -176,15 +185,24 @@ __global__ __launch_bounds__(RL* CG) void mnv_reduce_row_kernel(const float* __r
   for (int q = 0; q < W; ++q) acc[q].init();
   if (r0 < m) {
     if (VEC4) {
+      // several columns in flight per thread: with one workgroup per 32 rows there are few
+      // wavefronts per SIMD, and the loads of a thread are what keeps HBM busy (measured:
+      // four for the (value, index) pairs, 4.9 -> 6.0 TB/s; two for sums, where four lose 7%)
+      constexpr int U = Acc::ROW_UNROLL;
       int c = cg;
-      for (; c + CG < n; c += 2 * CG) {
-        mnv_f4 a = *reinterpret_cast<const mnv_f4*>(in + (size_t)c * m + r0);
-        mnv_f4 b = *reinterpret_cast<const mnv_f4*>(in + (size_t)(c + CG) * m + r0);
-        acc[0].push(a.x, c); acc[1 % W].push(a.y, c); acc[2 % W].push(a.z, c); acc[3 % W].push(a.w, c);
-        acc[0].push(b.x, c + CG); acc[1 % W].push(b.y, c + CG); acc[2 % W].push(b.z, c + CG); acc[3 % W].push(b.w, c + CG);
+      for (; c + (U - 1) * CG < n; c += U * CG) {
+        mnv_f4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          v[u] = mnv_ldx4<NT>(reinterpret_cast<const mnv_f4*>(in + (size_t)(c + u * CG) * m + r0));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          acc[0].push(v[u].x, c + u * CG); acc[1 % W].push(v[u].y, c + u * CG);
+          acc[2 % W].push(v[u].z, c + u * CG); acc[3 % W].push(v[u].w, c + u * CG);
+        }
       }
-      if (c < n) {
-        mnv_f4 a = *reinterpret_cast<const mnv_f4*>(in + (size_t)c * m + r0);
+      for (; c < n; c += CG) {
+        mnv_f4 a = mnv_ldx4<NT>(reinterpret_cast<const mnv_f4*>(in + (size_t)c * m + r0));
         acc[0].push(a.x, c); acc[1 % W].push(a.y, c); acc[2 % W].push(a.z, c); acc[3 % W].push(a.w, c);
       }
     } else {
@@ -220,12 +238,16 @@ int launch_reduce_row(const float* in, float* out, int m, int n, mnv_stream_t st
   if (vec4) {
     constexpr int RL = 8, CG = 64;
     unsigned grid = (unsigned)mnv_ceil_div((size_t)m, RL * 4);
-    hipLaunchKernelGGL((mnv_reduce_row_kernel<Acc, Emit, RL, CG, true>), dim3(grid),
-                       dim3(RL * CG), 0, s, in, out, m, n);
+    if ((size_t)m * n * sizeof(float) >= MNV_PAST_CACHE_BYTES)
+      hipLaunchKernelGGL((mnv_reduce_row_kernel<Acc, Emit, RL, CG, true, true>), dim3(grid),
+                         dim3(RL * CG), 0, s, in, out, m, n);
+    else
+      hipLaunchKernelGGL((mnv_reduce_row_kernel<Acc, Emit, RL, CG, true, false>), dim3(grid),
+                         dim3(RL * CG), 0, s, in, out, m, n);
   } else {
     constexpr int RL = 32, CG = 16;
     unsigned grid = (unsigned)mnv_ceil_div((size_t)m, RL);
-    hipLaunchKernelGGL((mnv_reduce_row_kernel<Acc, Emit, RL, CG, false>), dim3(grid),
+    hipLaunchKernelGGL((mnv_reduce_row_kernel<Acc, Emit, RL, CG, false, false>), dim3(grid),
                        dim3(RL * CG), 0, s, in, out, m, n);
   }
   return MNV_LAUNCH_STATUS();
@@ -242,6 +264,7 @@ int launch_reduce_row(const float* in, float* out, int m, int n, mnv_stream_t st
 // ---------------------------------------------------------------------------
 #define MNV_BIAS_THREADS 256
 
+template <bool NT>
 __global__ __launch_bounds__(MNV_BIAS_THREADS) void mnv_conv_bwd_bias_kernel(
     const float* __restrict__ top_diff, float* __restrict__ out, int N, int K, int hw,
     int images_per_group) {
@@ -261,14 +284,14 @@ __global__ __launch_bounds__(MNV_BIAS_THREADS) void mnv_conv_bwd_bias_kernel(
     if (lane < tail) s1 += p[head + 4 * n4 + lane];
     int i = lane;
     for (; i + 3 * MNV_WAVE < n4; i += 4 * MNV_WAVE) {
-      mnv_f4 a = p4[i], b = p4[i + MNV_WAVE], c = p4[i + 2 * MNV_WAVE], d = p4[i + 3 * MNV_WAVE];
+      mnv_f4 a = mnv_ldx4<NT>(p4 + i), b = mnv_ldx4<NT>(p4 + i + MNV_WAVE), c = mnv_ldx4<NT>(p4 + i + 2 * MNV_WAVE), d = mnv_ldx4<NT>(p4 + i + 3 * MNV_WAVE);
       s0 += (a.x + a.y) + (a.z + a.w);
       s1 += (b.x + b.y) + (b.z + b.w);
       s2 += (c.x + c.y) + (c.z + c.w);
       s3 += (d.x + d.y) + (d.z + d.w);
     }
     for (; i < n4; i += MNV_WAVE) {
-      mnv_f4 a = p4[i];
+      mnv_f4 a = mnv_ldx4<NT>(p4 + i);
       s0 += (a.x + a.y) + (a.z + a.w);
     }
   }
@@ -346,9 +369,14 @@ int mnv_conv_bwd_bias(const float* top_diff, float* bias_diff, int num_images,
   int per = (num_images + groups - 1) / groups;
   hipStream_t s = mnv_stream(stream);
   float* out = groups > 1 ? reinterpret_cast<float*>(workspace) : bias_diff;
-  hipLaunchKernelGGL(mnv_conv_bwd_bias_kernel, dim3(top_num_channels, groups),
-                     dim3(MNV_BIAS_THREADS), 0, s, top_diff, out, num_images, top_num_channels,
-                     (int)hw, per);
+  if ((size_t)num_images * top_num_channels * hw * sizeof(float) >= MNV_PAST_CACHE_BYTES)
+    hipLaunchKernelGGL(mnv_conv_bwd_bias_kernel<true>, dim3(top_num_channels, groups),
+                       dim3(MNV_BIAS_THREADS), 0, s, top_diff, out, num_images, top_num_channels,
+                       (int)hw, per);
+  else
+    hipLaunchKernelGGL(mnv_conv_bwd_bias_kernel<false>, dim3(top_num_channels, groups),
+                       dim3(MNV_BIAS_THREADS), 0, s, top_diff, out, num_images, top_num_channels,
+                       (int)hw, per);
   int rc = MNV_LAUNCH_STATUS();
   if (rc || groups == 1) return rc;
   hipLaunchKernelGGL(mnv_conv_bwd_bias_finish_kernel, dim3((top_num_channels + 255) / 256),

@@ -51,7 +51,7 @@ __device__ __forceinline__ float group_sum(float v, float* lds) {
 // One line per GROUP threads; the line (len % 4 == 0, len <= GROUP*4*MNV_SM_CACHE)
 // is cached in registers.  Loads are ordinary, stores non-temporal: measured on 8192 lines
 // of 8192 that pairing moves 85% of peak HBM bandwidth, non-temporal loads as well 70-76%.
-template <int GROUP, int CACHE>
+template <int GROUP, int CACHE, bool NT>
 __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_cached_kernel(
     const float* __restrict__ in, float* __restrict__ out, int len, int lines) {
   __shared__ float lds[MNV_SM_THREADS / MNV_WAVE];
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_cached_kernel(
     for (int u = 0; u < CACHE; ++u) {
       int i = t + u * GROUP;
       if (i < len4) {
-        v[u] = x4[i];
+        v[u] = mnv_ldx4<NT>(x4 + i);
         mx = fmaxf(mx, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
       }
     }
@@ -237,11 +237,18 @@ unsigned line_grid(int lines, int lpb) {
 // Contiguous lines of `len` floats (instance mode, or channel mode with H*W == 1).
 int softmax_lines_fwd(const float* in, float* out, int len, int lines, hipStream_t s) {
   bool vec = (len % 4 == 0) && mnv_aligned16(in) && mnv_aligned16(out);
-  if (vec && len <= MNV_WAVE * 4 * MNV_SM_CACHE)
-    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_WAVE, MNV_SM_CACHE>),
+  const bool big = (size_t)len * lines * sizeof(float) >= MNV_PAST_CACHE_BYTES;
+  if (vec && len <= MNV_WAVE * 4 * MNV_SM_CACHE && big)
+    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_WAVE, MNV_SM_CACHE, true>),
                        dim3(line_grid(lines, 4)), dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
+  else if (vec && len <= MNV_WAVE * 4 * MNV_SM_CACHE)
+    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_WAVE, MNV_SM_CACHE, false>),
+                       dim3(line_grid(lines, 4)), dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
+  else if (vec && len <= MNV_SM_THREADS * 4 * MNV_SM_CACHE && big)
+    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_SM_THREADS, MNV_SM_CACHE, true>),
+                       dim3(line_grid(lines, 1)), dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
   else if (vec && len <= MNV_SM_THREADS * 4 * MNV_SM_CACHE)
-    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_SM_THREADS, MNV_SM_CACHE>),
+    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_SM_THREADS, MNV_SM_CACHE, false>),
                        dim3(line_grid(lines, 1)), dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
   else if (len <= 1024)
     hipLaunchKernelGGL((mnv_softmax_fwd_generic_kernel<MNV_WAVE>), dim3(line_grid(lines, 4)),

@@ -39,7 +39,7 @@ __global__ __launch_bounds__(MNV_STREAM_THREADS) void mnv_stream_vec4_kernel(
     for (int u = 0; u < MNV_STREAM_UNROLL; ++u) {
       size_t i = base + (size_t)u * MNV_STREAM_THREADS;
       if (i < n4) {
-        if (NIN >= 1) a[u] = mnv_ld4<false>(a4 + i);
+        if (NIN >= 1) a[u] = mnv_ld4<NT>(a4 + i);
         if (NIN >= 2) b[u] = mnv_ld4<NT>(b4 + i);
       }
     }
@@ -73,10 +73,12 @@ __global__ __launch_bounds__(MNV_STREAM_THREADS) void mnv_stream_scalar_kernel(
 }
 
 // Buffers above this many bytes of traffic cannot stay in the 256 MB last-level
-// cache between kernels, so they stream past it: the stores and the second input's
-// loads are non-temporal, the first input's loads ordinary.  Measured on 8192^2 operands,
-// that mix moves 88% (one input) and 92% (two inputs) of peak HBM bandwidth; everything
-// non-temporal 81% / 83%, all loads ordinary 88% / 74%.
+// cache between kernels, so they stream past it with non-temporal loads and stores.
+// Measured on 8192^2 operands, cycling through four sets of them so that no pass finds its
+// operands cached: everything non-temporal moves 6.3 TB/s (one input) / 6.5 TB/s (two
+// inputs); first input ordinary 6.0 / 6.4; everything ordinary 5.8 / 5.8.  (When one set
+// is reused, a third of it is still cached on the next pass and the ordinary first input
+// looks best: 7.0 / 7.3 TB/s.)
 #define MNV_STREAM_NT_BYTES ((size_t)512 << 20)
 
 template <class Op, int NIN>

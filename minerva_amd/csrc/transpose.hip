@@ -38,6 +38,7 @@ __global__ __launch_bounds__(MNV_TR_THREADS) void mnv_transpose_kernel(
 // 16-byte global accesses on both sides: a thread reads four consecutive i of one column
 // and writes four consecutive j of one output column; the 64x64 tile is transposed
 // through LDS with 4-byte accesses.  Needs m % 4 == 0, n % 4 == 0 and aligned pointers.
+template <bool NT>
 __global__ __launch_bounds__(MNV_TR_THREADS) void mnv_transpose_vec4_kernel(
     const float* __restrict__ a, float* __restrict__ c, int m, int n, int tiles_i, int tiles_j) {
   __shared__ float tile[MNV_TR_TILE][MNV_TR_TILE + 1];
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(MNV_TR_THREADS) void mnv_transpose_vec4_kernel(
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     int i = i0 + tx * 4, j = j0 + ty + 16 * p;
-    if (i < m && j < n) v[p] = *reinterpret_cast<const mnv_f4*>(a + (size_t)j * m + i);
+    if (i < m && j < n) v[p] = mnv_ldx4<NT>(reinterpret_cast<const mnv_f4*>(a + (size_t)j * m + i));
   }
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
@@ -77,8 +78,12 @@ extern "C" int mnv_transpose(const float* a, float* c, int m, int n, mnv_stream_
   if (!a || !c || m < 0 || n < 0) return MNV_ERR_INVALID;
   size_t tiles_i = mnv_ceil_div((size_t)m, MNV_TR_TILE), tiles_j = mnv_ceil_div((size_t)n, MNV_TR_TILE);
   if (tiles_i * tiles_j > 0x7fffffffULL) return MNV_ERR_INVALID;
-  if (m % 4 == 0 && n % 4 == 0 && mnv_aligned16(a) && mnv_aligned16(c))
-    hipLaunchKernelGGL(mnv_transpose_vec4_kernel, dim3((unsigned)(tiles_i * tiles_j)),
+  const bool vec = m % 4 == 0 && n % 4 == 0 && mnv_aligned16(a) && mnv_aligned16(c);
+  if (vec && (size_t)m * n * sizeof(float) >= MNV_PAST_CACHE_BYTES)
+    hipLaunchKernelGGL(mnv_transpose_vec4_kernel<true>, dim3((unsigned)(tiles_i * tiles_j)),
+                       dim3(MNV_TR_THREADS), 0, mnv_stream(stream), a, c, m, n, (int)tiles_i, (int)tiles_j);
+  else if (vec)
+    hipLaunchKernelGGL(mnv_transpose_vec4_kernel<false>, dim3((unsigned)(tiles_i * tiles_j)),
                        dim3(MNV_TR_THREADS), 0, mnv_stream(stream), a, c, m, n, (int)tiles_i, (int)tiles_j);
   else
     hipLaunchKernelGGL(mnv_transpose_kernel, dim3((unsigned)(tiles_i * tiles_j)),
