@@ -159,3 +159,30 @@ def test_transpose_bit_exact(gpu, ora, m, n):
     dback = gpu.empty(m * n)
     gpu.call("mnv_transpose", dout.p, dback.p, n, m)
     assert_bits_equal(gpu.down(dback), x, "transpose twice")
+
+
+def test_large_operand_paths_8192x8192(gpu):
+    """Inputs of 256 MB and more take the variants that read past the caches: softmax,
+    transpose and the broadcast add at the size of the bandwidth benchmark."""
+    m = n = 8192
+    x = _rand(m * n, 23)
+    dx, dz = gpu.up(x), gpu.empty(m * n)
+    say("softmax 8192 lines of 8192")
+    gpu.call("mnv_softmax_instance_fwd", dx.p, dz.p, n, m, 1, 1)  # lines of m contiguous floats
+    y = gpu.down(dz).reshape(n, m)
+    assert np.max(np.abs(y.astype(np.float64).sum(axis=1) - 1.0)) <= 1e-5
+    for line in (0, 1, 4095, 8191):
+        v = x.reshape(n, m)[line].astype(np.float64)
+        ref = np.exp(v - v.max())
+        ref /= ref.sum()
+        assert normwise(y[line], ref) <= TOL
+    say("transpose 8192 x 8192")
+    gpu.call("mnv_transpose", dx.p, dz.p, m, n)
+    assert_bits_equal(gpu.down(dz), np.ascontiguousarray(x.reshape(n, m).T).ravel(), "transpose 8192")
+    say("broadcast add 8192 x 8192")
+    vec = _rand(m, 24)
+    dv = gpu.up(vec)
+    gpu.call("mnv_norm_add_col", dx.p, dv.p, dz.p, m, n)   # res[r + c*m] = x[r + c*m] + vec[c]
+    assert_bits_equal(gpu.down(dz), (x.reshape(n, m) + vec[:, None]).ravel(), "norm_add_col 8192")
+    gpu.call("mnv_norm_add_row", dx.p, dv.p, dz.p, m, n)   # res[r + c*m] = x[r + c*m] + vec[r]
+    assert_bits_equal(gpu.down(dz), (x.reshape(n, m) + vec[None, :]).ravel(), "norm_add_row 8192")
