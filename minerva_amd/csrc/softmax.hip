@@ -48,39 +48,51 @@ __device__ __forceinline__ float group_sum(float v, float* lds) {
   return v;
 }
 
-// One line per GROUP threads; the line (len % 4 == 0, len <= GROUP*4*MNV_SM_CACHE)
-// is cached in registers.  Stores are non-temporal; NT: so are the loads (inputs of 256 MB
-// and more, which no cache holds until the next operator).  Measured on 8192 lines of 8192
-// with the operands cycled through four sets: 5.6 TB/s, 70% of peak HBM bandwidth (a plain
-// copy of the same operands: 6.4 TB/s).
-template <int GROUP, int CACHE, bool NT>
-__global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_cached_kernel(
+// Keeps a per-thread pointer in a pair of vector registers.  Left alone, the compiler
+// addresses the line as (scalar base + 32-bit lane offset); on gfx950 global loads and stores
+// in that form sustain less bandwidth than those that carry full 64-bit lane addresses
+// (8192 lines of 8192 floats, forward: 5.9 TB/s against 6.3 TB/s).
+template <class T>
+__device__ __forceinline__ T* lane_pointer(T* p) {
+  asm volatile("" : "+v"(p));
+  return p;
+}
+
+// One line per GROUP threads of an NTH-thread workgroup (GROUP = one wavefront or the whole
+// workgroup); the line (len % 4 == 0, len <= GROUP*4*CACHE) is cached in registers.
+// Stores are non-temporal; NT: so are the loads (inputs of 256 MB and more, which no cache
+// holds until the next operator).  Lines of up to 8192 values take 512 threads with four
+// vectors each rather than 256 with eight (more wavefronts, shorter per-thread chains): on
+// 8192 lines of 8192, operands cycled through four sets, 6.3 TB/s against 5.8 TB/s (a plain
+// copy of the same operands: 6.3 TB/s).
+template <int GROUP, int CACHE, int NTH, bool NT>
+__global__ __launch_bounds__(NTH) void mnv_softmax_fwd_cached_kernel(
     const float* __restrict__ in, float* __restrict__ out, int len, int lines) {
-  __shared__ float lds[MNV_SM_THREADS / MNV_WAVE];
-  constexpr int LPB = MNV_SM_THREADS / GROUP;
+  __shared__ float lds[NTH / MNV_WAVE];
+  constexpr int LPB = NTH / GROUP;
   const int t = threadIdx.x % GROUP;
   const int len4 = len >> 2;
-  // the trip count is block-uniform when GROUP spans the block; with one wavefront per
+  // the trip count is block-uniform when GROUP spans the block (and the line index then a
+  // scalar: the compiler cannot tell that threadIdx.x / GROUP is 0); with one wavefront per
   // line no barrier is used
-  for (int line = blockIdx.x * LPB + threadIdx.x / GROUP; line < lines; line += gridDim.x * LPB) {
-    const mnv_f4* x4 = reinterpret_cast<const mnv_f4*>(in + (size_t)line * len);
-    mnv_f4* y4 = reinterpret_cast<mnv_f4*>(out + (size_t)line * len);
+  for (int line = blockIdx.x * LPB + (LPB > 1 ? threadIdx.x / GROUP : 0); line < lines; line += gridDim.x * LPB) {
+    const mnv_f4* x4 = lane_pointer(reinterpret_cast<const mnv_f4*>(in + (size_t)line * len) + t);
+    mnv_f4* y4 = lane_pointer(reinterpret_cast<mnv_f4*>(out + (size_t)line * len) + t);
     mnv_f4 v[CACHE];
+    // all loads first, in a loop of their own: a use inside the same guarded block would
+    // make each load wait for the one before it
+#pragma unroll
+    for (int u = 0; u < CACHE; ++u)
+      if (t + u * GROUP < len4) v[u] = mnv_ldx4<NT>(x4 + u * GROUP);
     float mx = -INFINITY;
 #pragma unroll
-    for (int u = 0; u < CACHE; ++u) {
-      int i = t + u * GROUP;
-      if (i < len4) {
-        v[u] = mnv_ldx4<NT>(x4 + i);
-        mx = fmaxf(mx, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
-      }
-    }
+    for (int u = 0; u < CACHE; ++u)
+      if (t + u * GROUP < len4) mx = fmaxf(mx, fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w)));
     mx = group_max<GROUP>(mx, lds);
     float s = 0.f;
 #pragma unroll
     for (int u = 0; u < CACHE; ++u) {
-      int i = t + u * GROUP;
-      if (i < len4) {
+      if (t + u * GROUP < len4) {
         // exp through the hardware exp2: relative error ~1e-6 for the arguments <= 0 here
         v[u].x = __expf(v[u].x - mx);
         v[u].y = __expf(v[u].y - mx);
@@ -93,14 +105,13 @@ __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_cached_kernel(
     const float inv = 1.0f / s;  // one reciprocal per thread instead of a division per element
 #pragma unroll
     for (int u = 0; u < CACHE; ++u) {
-      int i = t + u * GROUP;
-      if (i < len4) {
+      if (t + u * GROUP < len4) {
         mnv_f4 o;
         o.x = v[u].x * inv;
         o.y = v[u].y * inv;
         o.z = v[u].z * inv;
         o.w = v[u].w * inv;
-        __builtin_nontemporal_store(o, y4 + i);
+        __builtin_nontemporal_store(o, y4 + u * GROUP);
       }
     }
   }
@@ -115,7 +126,7 @@ __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_generic_kernel
   __shared__ float lds[MNV_SM_THREADS / MNV_WAVE];
   constexpr int LPB = MNV_SM_THREADS / GROUP;
   const int t = threadIdx.x % GROUP;
-  for (int line = blockIdx.x * LPB + threadIdx.x / GROUP; line < lines; line += gridDim.x * LPB) {
+  for (int line = blockIdx.x * LPB + (LPB > 1 ? threadIdx.x / GROUP : 0); line < lines; line += gridDim.x * LPB) {
     size_t base = (size_t)(line / inner) * outer + (size_t)(line % inner);
     const float* x = in + base;
     float* y = out + base;
@@ -133,40 +144,41 @@ __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_fwd_generic_kernel
   }
 }
 
-template <int GROUP, int CACHE>
-__global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_bwd_cached_kernel(
+template <int GROUP, int CACHE, int NTH>
+__global__ __launch_bounds__(NTH) void mnv_softmax_bwd_cached_kernel(
     const float* __restrict__ dy, const float* __restrict__ y, float* __restrict__ dx, int len,
     int lines) {
-  __shared__ float lds[MNV_SM_THREADS / MNV_WAVE];
-  constexpr int LPB = MNV_SM_THREADS / GROUP;
+  __shared__ float lds[NTH / MNV_WAVE];
+  constexpr int LPB = NTH / GROUP;
   const int t = threadIdx.x % GROUP;
   const int len4 = len >> 2;
-  for (int line = blockIdx.x * LPB + threadIdx.x / GROUP; line < lines; line += gridDim.x * LPB) {
-    const mnv_f4* d4 = reinterpret_cast<const mnv_f4*>(dy + (size_t)line * len);
-    const mnv_f4* t4 = reinterpret_cast<const mnv_f4*>(y + (size_t)line * len);
-    mnv_f4* o4 = reinterpret_cast<mnv_f4*>(dx + (size_t)line * len);
+  for (int line = blockIdx.x * LPB + (LPB > 1 ? threadIdx.x / GROUP : 0); line < lines; line += gridDim.x * LPB) {
+    const mnv_f4* d4 = lane_pointer(reinterpret_cast<const mnv_f4*>(dy + (size_t)line * len) + t);
+    const mnv_f4* t4 = lane_pointer(reinterpret_cast<const mnv_f4*>(y + (size_t)line * len) + t);
+    mnv_f4* o4 = lane_pointer(reinterpret_cast<mnv_f4*>(dx + (size_t)line * len) + t);
     mnv_f4 d[CACHE], p[CACHE];
-    float dot = 0.f;
 #pragma unroll
-    for (int u = 0; u < CACHE; ++u) {
-      int i = t + u * GROUP;
-      if (i < len4) {
-        d[u] = d4[i];
-        p[u] = __builtin_nontemporal_load(t4 + i);
-        dot += (d[u].x * p[u].x + d[u].y * p[u].y) + (d[u].z * p[u].z + d[u].w * p[u].w);
+    for (int u = 0; u < CACHE; ++u) {  // loads only, so that none waits for another
+      if (t + u * GROUP < len4) {
+        d[u] = d4[u * GROUP];
+        p[u] = __builtin_nontemporal_load(t4 + u * GROUP);
       }
     }
+    float dot = 0.f;
+#pragma unroll
+    for (int u = 0; u < CACHE; ++u)
+      if (t + u * GROUP < len4)
+        dot += (d[u].x * p[u].x + d[u].y * p[u].y) + (d[u].z * p[u].z + d[u].w * p[u].w);
     dot = group_sum<GROUP>(dot, lds);
 #pragma unroll
     for (int u = 0; u < CACHE; ++u) {
-      int i = t + u * GROUP;
-      if (i < len4) {
+      if (t + u * GROUP < len4) {
         mnv_f4 o;
         o.x = p[u].x * (d[u].x - dot);
         o.y = p[u].y * (d[u].y - dot);
         o.z = p[u].z * (d[u].z - dot);
         o.w = p[u].w * (d[u].w - dot);
-        __builtin_nontemporal_store(o, o4 + i);
+        __builtin_nontemporal_store(o, o4 + u * GROUP);
       }
     }
   }
@@ -179,7 +191,7 @@ __global__ __launch_bounds__(MNV_SM_THREADS) void mnv_softmax_bwd_generic_kernel
   __shared__ float lds[MNV_SM_THREADS / MNV_WAVE];
   constexpr int LPB = MNV_SM_THREADS / GROUP;
   const int t = threadIdx.x % GROUP;
-  for (int line = blockIdx.x * LPB + threadIdx.x / GROUP; line < lines; line += gridDim.x * LPB) {
+  for (int line = blockIdx.x * LPB + (LPB > 1 ? threadIdx.x / GROUP : 0); line < lines; line += gridDim.x * LPB) {
     size_t base = (size_t)(line / inner) * outer + (size_t)(line % inner);
     float dot = 0.f;
     for (int i = t; i < len; i += GROUP) dot += dy[base + i * stride] * y[base + i * stride];
@@ -237,21 +249,28 @@ unsigned line_grid(int lines, int lpb) {
 }
 
 // Contiguous lines of `len` floats (instance mode, or channel mode with H*W == 1).
+#define MNV_SM_WIDE 512      // threads per line for lines of more than 4096 values
+#define MNV_SM_WIDE_CACHE 4  // 16-byte vectors cached per thread in that configuration
+template <int GROUP, int CACHE, int NTH>
+void launch_fwd_cached(const float* in, float* out, int len, int lines, bool nt, hipStream_t s) {
+  const dim3 grid(line_grid(lines, NTH / GROUP)), block(NTH);
+  if (nt)
+    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<GROUP, CACHE, NTH, true>), grid, block, 0, s, in,
+                       out, len, lines);
+  else
+    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<GROUP, CACHE, NTH, false>), grid, block, 0, s, in,
+                       out, len, lines);
+}
+
 int softmax_lines_fwd(const float* in, float* out, int len, int lines, hipStream_t s) {
   bool vec = (len % 4 == 0) && mnv_aligned16(in) && mnv_aligned16(out);
   const bool big = (size_t)len * lines * sizeof(float) >= MNV_PAST_CACHE_BYTES;
-  if (vec && len <= MNV_WAVE * 4 * MNV_SM_CACHE && big)
-    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_WAVE, MNV_SM_CACHE, true>),
-                       dim3(line_grid(lines, 4)), dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
-  else if (vec && len <= MNV_WAVE * 4 * MNV_SM_CACHE)
-    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_WAVE, MNV_SM_CACHE, false>),
-                       dim3(line_grid(lines, 4)), dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
-  else if (vec && len <= MNV_SM_THREADS * 4 * MNV_SM_CACHE && big)
-    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_SM_THREADS, MNV_SM_CACHE, true>),
-                       dim3(line_grid(lines, 1)), dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
-  else if (vec && len <= MNV_SM_THREADS * 4 * MNV_SM_CACHE)
-    hipLaunchKernelGGL((mnv_softmax_fwd_cached_kernel<MNV_SM_THREADS, MNV_SM_CACHE, false>),
-                       dim3(line_grid(lines, 1)), dim3(MNV_SM_THREADS), 0, s, in, out, len, lines);
+  if (vec && len <= MNV_WAVE * 4 * MNV_SM_CACHE)
+    launch_fwd_cached<MNV_WAVE, MNV_SM_CACHE, MNV_SM_THREADS>(in, out, len, lines, big, s);
+  else if (vec && len <= MNV_SM_THREADS * 4 * MNV_SM_WIDE_CACHE)
+    launch_fwd_cached<MNV_SM_THREADS, MNV_SM_WIDE_CACHE, MNV_SM_THREADS>(in, out, len, lines, big, s);
+  else if (vec && len <= MNV_SM_WIDE * 4 * MNV_SM_WIDE_CACHE)
+    launch_fwd_cached<MNV_SM_WIDE, MNV_SM_WIDE_CACHE, MNV_SM_WIDE>(in, out, len, lines, big, s);
   else if (len <= 1024)
     hipLaunchKernelGGL((mnv_softmax_fwd_generic_kernel<MNV_WAVE>), dim3(line_grid(lines, 4)),
                        dim3(MNV_SM_THREADS), 0, s, in, out, len, lines, 1, (size_t)len, (size_t)1);
@@ -265,11 +284,14 @@ int softmax_lines_bwd(const float* dy, const float* y, float* dx, int len, int l
                       hipStream_t s) {
   bool vec = (len % 4 == 0) && mnv_aligned16(dy) && mnv_aligned16(y) && mnv_aligned16(dx);
   if (vec && len <= MNV_WAVE * 4 * MNV_SM_CACHE)
-    hipLaunchKernelGGL((mnv_softmax_bwd_cached_kernel<MNV_WAVE, MNV_SM_CACHE>),
+    hipLaunchKernelGGL((mnv_softmax_bwd_cached_kernel<MNV_WAVE, MNV_SM_CACHE, MNV_SM_THREADS>),
                        dim3(line_grid(lines, 4)), dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines);
-  else if (vec && len <= MNV_SM_THREADS * 4 * MNV_SM_CACHE)
-    hipLaunchKernelGGL((mnv_softmax_bwd_cached_kernel<MNV_SM_THREADS, MNV_SM_CACHE>),
+  else if (vec && len <= MNV_SM_THREADS * 4 * MNV_SM_WIDE_CACHE)
+    hipLaunchKernelGGL((mnv_softmax_bwd_cached_kernel<MNV_SM_THREADS, MNV_SM_WIDE_CACHE, MNV_SM_THREADS>),
                        dim3(line_grid(lines, 1)), dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines);
+  else if (vec && len <= MNV_SM_WIDE * 4 * MNV_SM_WIDE_CACHE)
+    hipLaunchKernelGGL((mnv_softmax_bwd_cached_kernel<MNV_SM_WIDE, MNV_SM_WIDE_CACHE, MNV_SM_WIDE>),
+                       dim3(line_grid(lines, 1)), dim3(MNV_SM_WIDE), 0, s, dy, y, dx, len, lines);
   else if (len <= 1024)
     hipLaunchKernelGGL((mnv_softmax_bwd_generic_kernel<MNV_WAVE>), dim3(line_grid(lines, 4)),
                        dim3(MNV_SM_THREADS), 0, s, dy, y, dx, len, lines, 1, (size_t)len, (size_t)1);

@@ -107,8 +107,8 @@ def test_max_and_argmax_full_size(gpu, ora):
     assert normwise(gpu.down(drow), a.astype(np.float64).sum(axis=0)) <= TOL
 
 
-SOFTMAX = [(1, 1), (10, 256), (1000, 256), (7, 33), (256, 100), (2048, 64), (8192, 48),
-           (8193, 5), (9000, 3), (40000, 2)]
+SOFTMAX = [(1, 1), (10, 256), (1000, 256), (7, 33), (256, 100), (2048, 64), (2052, 7), (4096, 16),
+           (4100, 9), (8192, 48), (8193, 5), (9000, 3), (40000, 2)]
 
 
 @pytest.mark.parametrize("length,lines", SOFTMAX)
@@ -147,7 +147,8 @@ def test_softmax_channel(gpu, ora, n, c, h, w):
 
 
 @pytest.mark.parametrize("m,n", [(1, 1), (3, 4), (64, 64), (65, 63), (1000, 37), (256, 784),
-                                 (4096, 9216), (10, 256)])
+                                 (4096, 9216), (10, 256), (2052, 1500), (1500, 2052),
+                                 (132, 16388)])
 def test_transpose_bit_exact(gpu, ora, m, n):
     x = _rand(m * n, 27)       # a is {m,n}
     dx, dout = gpu.up(x), gpu.empty(m * n)
