@@ -280,20 +280,27 @@ __global__ __launch_bounds__(MNV_BIAS_THREADS) void mnv_conv_bwd_bias_kernel(
     if (head > hw) head = hw;
     const int n4 = (hw - head) >> 2, tail = (hw - head) & 3;
     const mnv_f4* p4 = reinterpret_cast<const mnv_f4*>(p + head);
-    if (lane < head) s0 += p[lane];
-    if (lane < tail) s1 += p[head + 4 * n4 + lane];
-    int i = lane;
-    for (; i + 3 * MNV_WAVE < n4; i += 4 * MNV_WAVE) {
-      mnv_f4 a = mnv_ldx4<NT>(p4 + i), b = mnv_ldx4<NT>(p4 + i + MNV_WAVE), c = mnv_ldx4<NT>(p4 + i + 2 * MNV_WAVE), d = mnv_ldx4<NT>(p4 + i + 3 * MNV_WAVE);
-      s0 += (a.x + a.y) + (a.z + a.w);
-      s1 += (b.x + b.y) + (b.z + b.w);
-      s2 += (c.x + c.y) + (c.z + c.w);
-      s3 += (d.x + d.y) + (d.z + d.w);
+    float edge0 = 0.f, edge1 = 0.f;  // used after the vectors so that they do not wait for these
+    if (lane < head) edge0 = p[lane];
+    if (lane < tail) edge1 = p[head + 4 * n4 + lane];
+    // Four loads in flight per lane in every iteration, the last one included: a vector
+    // past the end of the run is read from the run's last vector instead (a cache hit) and
+    // counted as 0, so there is no one-load-at-a-time remainder loop (a run of 55 x 55
+    // floats would spend four of its six trips to memory in it).
+    if (n4 > 0) {
+      const int last = n4 - 1;
+      for (int i = lane; i < n4; i += 4 * MNV_WAVE) {
+        const int i1 = i + MNV_WAVE, i2 = i + 2 * MNV_WAVE, i3 = i + 3 * MNV_WAVE;
+        mnv_f4 a = mnv_ldx4<NT>(p4 + i), b = mnv_ldx4<NT>(p4 + min(i1, last)),
+               c = mnv_ldx4<NT>(p4 + min(i2, last)), d = mnv_ldx4<NT>(p4 + min(i3, last));
+        s0 += (a.x + a.y) + (a.z + a.w);
+        s1 += i1 < n4 ? (b.x + b.y) + (b.z + b.w) : 0.f;
+        s2 += i2 < n4 ? (c.x + c.y) + (c.z + c.w) : 0.f;
+        s3 += i3 < n4 ? (d.x + d.y) + (d.z + d.w) : 0.f;
+      }
     }
-    for (; i < n4; i += MNV_WAVE) {
-      mnv_f4 a = mnv_ldx4<NT>(p4 + i);
-      s0 += (a.x + a.y) + (a.z + a.w);
-    }
+    s0 += edge0;
+    s1 += edge1;
   }
   float s = mnv_wave_sum((s0 + s1) + (s2 + s3));
   if (lane == 0) part[wave] = s;
