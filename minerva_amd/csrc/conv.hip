@@ -475,7 +475,11 @@ struct ConvBwdFilterFast {
   // off[0] is unused for A: the offsets come from the table every slab.
   __device__ void a_load(const Res& r, const AState& st, const unsigned (&)[1], int period, int s,
                          int kl, float (&v)[4]) const {
-    const unsigned* t = r.tab + st.trow + s * 16 + kl;
+    // the four entries are one aligned 16-byte LDS read: rows are PP (a multiple of 16)
+    // entries long and kl is a multiple of 4
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const u4 t = *reinterpret_cast<const u4*>(
+        __builtin_assume_aligned(r.tab + st.trow + s * 16 + kl, 16));
     const unsigned soff = (unsigned)period * (unsigned)(g.C * g.HW) * 4u;
 #pragma unroll
     for (int q = 0; q < 4; ++q)
