@@ -67,3 +67,30 @@ def test_host_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(hostapi.LIB_PATH)
     missing = [n for n in names if not hasattr(lib, n)]
     assert not missing, missing
+
+
+def test_narray_front_end_has_the_names_of_the_reference_binding():
+    """Every public name of the reference's Python binding that belongs to the operator path
+    (owl/owl/__init__.py, owl/owl/libowl.pyx:51-444, owl/owl/elewise.py, owl/owl/conv.py)
+    exists in minerva_amd.owl; importing it needs no GPU."""
+    from minerva_amd import owl
+    from minerva_amd.owl import conv, elewise
+    module = ("has_cuda wait_for_all create_cpu_device create_gpu_device get_gpu_device_count "
+              "set_device zeros ones randn randb from_numpy concat slice NArray").split()
+    narray = ("mult exp ln sigm sigm_back relu relu_back tanh tanh_back conv_forward "
+              "conv_backward_data conv_backward_filter conv_backward_bias softmax_forward "
+              "softmax_backward activation_forward activation_backward pooling_forward "
+              "pooling_backward lrn_forward lrn_backward sum max max_index count_zero trans "
+              "reshape wait_for_eval shape zeros ones randn randb concat slice from_numpy "
+              "to_numpy __add__ __sub__ __mul__ __truediv__ __iadd__ __isub__ __imul__ "
+              "__itruediv__ __radd__ __rsub__ __rmul__ __rtruediv__").split()
+    assert not [n for n in module if not hasattr(owl, n)]
+    assert not [n for n in narray if not hasattr(owl.NArray, n)]
+    assert not [n for n in "mult exp ln sigm relu tanh sigm_back relu_back tanh_back".split()
+                if not hasattr(elewise, n)]
+    assert not [n for n in "softmax Lrner Convolver Pooler soft_op pool_op".split()
+                if not hasattr(conv, n)]
+    assert conv.soft_op.instance != conv.soft_op.channel and conv.pool_op.max != conv.pool_op.avg
+    for cls, methods in ((conv.Convolver, "ff bp weight_grad bias_grad"), (conv.Pooler, "ff bp"),
+                         (conv.Lrner, "ff bp")):
+        assert not [m for m in methods.split() if not hasattr(cls, m)]
