@@ -118,6 +118,42 @@ def alexnet_bench(steps, warmup, dataflow=False):
     return out
 
 
+def owl_front_end_bench(steps, warmup):
+    """The same step issued operator by operator from Python through the NArray front end
+    (minerva_amd.owl, the interface of the reference's owl binding): what a Python
+    application sees.  Reported beside `value`, not as it."""
+    from minerva_amd import configs, owl
+    from minerva_amd.owl import models
+    params, data, label = configs.make_inputs("alexnet", BATCH)
+    owl.set_device(owl.create_gpu_device(0))
+    net = models.AlexNet()
+    net.load([params["w%d" % k] for k in range(8)], [params["b%d" % k] for k in range(8)])
+    x = owl.from_numpy(np.asarray(data, np.float32).reshape(BATCH, 3, 227, 227))
+    y = owl.from_numpy(np.asarray(label, np.float32).reshape(BATCH, 1000))
+    rt = owl._runtime()
+
+    def step():
+        out, wgrad, bgrad = net.train_one_mb(x, y)
+        net.sgd(wgrad, bgrad, BATCH, 0.01)
+        owl.wait_for_all()
+        return out
+
+    for _ in range(warmup):
+        step()
+    ops0 = rt.ops_issued()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = step()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    ops = (rt.ops_issued() - ops0) // steps
+    finite = bool(np.isfinite(out.to_numpy()).all())
+    del out, net, x, y
+    owl.close_devices()
+    log("alexnet b=%d through the owl front end: %.3f ms/step, %d ops/step" % (BATCH, ms, ops))
+    return {"ms_per_step": round(ms, 3), "images_per_s": round(BATCH / (ms / 1e3), 1),
+            "ops_per_step": int(ops), "finite": finite}
+
+
 # HBM bytes per launch of the dominant kernel (average over the conv2..conv5 filter
 # gradients), from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB
 # per dispatch), each scaled by what the same counter reads for the 8192^2 copy kernel
@@ -407,6 +443,7 @@ def main():
         "dataflow_4_streams": ({"images_per_s": round(res["dataflow"]["images_per_s"], 1),
                                 "ms_per_step": round(res["dataflow"]["ms_per_step"], 3)}
                                if args.dataflow else None),
+        "owl_front_end": owl_front_end_bench(args.steps, args.warmup),
         "h2d_batch_ms": round(main_run["h2d_batch_ms"], 2),
         "roofline": roof,
         "sgemm": sgemm,

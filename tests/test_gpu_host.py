@@ -8,7 +8,7 @@ import os
 import numpy as np
 import pytest
 
-from gpu_util import TOL, assert_bits_equal, normwise, say
+from gpu_util import TOL, assert_bits_equal, compare_step, normwise, say
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
@@ -293,48 +293,6 @@ def _run_net(kind, batch, steps, sync_each_op, variant=0, lr=0.01):
     return out, ops
 
 
-# A whole training step chains ~20 fp32 operators and both sides round at every one of
-# them.  Besides ordinary rounding noise there is one discontinuous effect: a pre-activation
-# that rounds to different sides of 0 on the two sides flips its ReLU gate, which adds or
-# drops one full-size term in the gradients downstream (seen on conv bias gradients: an
-# error of exactly one term).  So a step is compared this way: probabilities and updated
-# weights normwise at 1e-4; every weight gradient in relative L2 norm at 1e-3 with at least
-# 99.9 % of its entries within 1e-4 of the largest entry; every bias gradient -- a sum of
-# hundreds to thousands of signed, largely cancelling terms -- within 3e-3 of the L1 mass
-# of its terms (one flipped term of a 338-term sum is 3e-3 of that mass), the updated bias
-# within the same bound scaled by lr / batch.  The operators themselves are held to 1e-4
-# (or bit-exactness) one by one in the other test files.
-def _rel_l2(got, ref):
-    got = np.asarray(got, np.float64)
-    ref = np.asarray(ref, np.float64)
-    return float(np.linalg.norm(got - ref) / max(np.linalg.norm(ref), 1e-30))
-
-
-def _compare(got, newp, res, lr=0.01, batch=1, deep=False):
-    """deep=True (the 12-layer network at batch 2, where a handful of flipped gates among
-    ~10^6 tiny activations is a visible fraction of the gradient signal): gradients are held
-    to 1e-2 in relative L2 norm and 1e-3 in their norms instead of the entrywise rule."""
-    for k, v in newp.items():
-        g, r = got["g_" + k], res["g_" + k]
-        if k.startswith("w") and deep:
-            assert _rel_l2(g, r) <= 1e-2, "gradient %s: relative L2 error %.3e" % (k, _rel_l2(g, r))
-            ng, nr = np.linalg.norm(g.astype(np.float64)), np.linalg.norm(r.astype(np.float64))
-            assert abs(ng - nr) <= 1e-3 * nr, "gradient norm %s: %.6e vs %.6e" % (k, ng, nr)
-            assert normwise(got[k], v) <= TOL, "updated " + k
-        elif k.startswith("w"):
-            assert _rel_l2(g, r) <= 1e-3, "gradient %s: relative L2 error %.3e" % (k, _rel_l2(g, r))
-            close = np.abs(g.astype(np.float64) - r) <= TOL * np.max(np.abs(r))
-            assert close.mean() >= 0.999, "gradient %s: %.5f of entries within 1e-4" % (k, close.mean())
-            assert normwise(got[k], v) <= TOL, "updated " + k
-        else:
-            scale = 3e-3 * float(np.max(res["l1_" + k]))
-            err = float(np.max(np.abs(g.astype(np.float64) - r)))
-            assert err <= scale, "gradient %s: error %.3e, bound %.3e" % (k, err, scale)
-            err = float(np.max(np.abs(got[k].astype(np.float64) - v)))
-            assert err <= scale * lr / batch + 1e-12, "updated " + k
-    assert normwise(got["prob"], res["prob"]) <= TOL
-
-
 def test_mlp_step_matches_oracle(ora):
     from oracle import nets
     params, data, label = nets.make_inputs("mlp", 256)
@@ -343,7 +301,7 @@ def test_mlp_step_matches_oracle(ora):
         p, res = nets.mlp_step(p, data, label, 0.01, 256)
     say("mlp 2 steps, per-op sync")
     got, ops = _run_net("mlp", 256, 2, True)
-    _compare(got, p, res, batch=256)
+    compare_step(got, p, res, batch=256)
     say("mlp 2 steps, one sync per step")
     got2, _ = _run_net("mlp", 256, 2, False)
     for k in got:
@@ -360,7 +318,7 @@ def test_cnn_step_matches_oracle(ora, variant):
     p, res = nets.cnn_step(dict(params), data, label, 0.01, batch, **kw)
     say("cnn step variant", variant)
     got, _ = _run_net("cnn", batch, 1, True, variant)
-    _compare(got, p, res, batch=batch)
+    compare_step(got, p, res, batch=batch)
 
 
 def test_alexnet_step_matches_oracle_small_batch(ora):
@@ -371,7 +329,7 @@ def test_alexnet_step_matches_oracle_small_batch(ora):
     p, res = nets.alexnet_step(dict(params), data, label, 0.01, batch)
     say("alexnet GPU step b=2")
     got, ops = _run_net("alexnet", batch, 1, False)
-    _compare(got, p, res, batch=batch, deep=True)
+    compare_step(got, p, res, batch=batch, deep=True)
     # the loss itself (cross entropy of the probabilities) agrees to 1e-5
     lab = label.reshape(batch, -1).argmax(axis=1)
     ce = lambda pr: -np.log(pr.reshape(batch, -1)[np.arange(batch), lab].astype(np.float64)).mean()
@@ -391,7 +349,7 @@ def test_alexnet_step_with_dropout_matches_oracle(ora):
     say("alexnet + dropout GPU step b=2")
     hostapi.Runtime.set_random_seed(seed)
     got, ops = _run_net("alexnet", batch, 1, False, variant=1)
-    _compare(got, p, res, batch=batch, deep=True)
+    compare_step(got, p, res, batch=batch, deep=True)
     # dropout changed the result: the plain graph's probabilities differ
     _, plain = nets.alexnet_step(dict(params), data, label, 0.01, batch)
     assert normwise(got["prob"], plain["prob"]) > 1e-3 or np.max(np.abs(got["g_w7"] - plain["g_w7"])) > 0

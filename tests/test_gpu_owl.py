@@ -6,7 +6,7 @@ programs are written against the reference's binding, and checked against numpy
 import numpy as np
 import pytest
 
-from gpu_util import TOL, assert_bits_equal, normwise, say
+from gpu_util import TOL, assert_bits_equal, compare_step, normwise, say
 
 pytestmark = pytest.mark.gpu
 
@@ -268,3 +268,37 @@ def test_lrn_and_average_pooling_wrappers(owl, ora):
     assert normwise(y.to_numpy().ravel(), want_y) <= TOL
     sm = conv.softmax(owl.from_numpy(_rand((4, 3, 2, 5), 15)), conv.soft_op.channel)
     assert sm.shape == [5, 2, 3, 4]
+
+
+def test_alexnet_application_step_with_dropout(owl, ora):
+    """The AlexNet application (owl/apps/imagenet_alexnet/alexnet.py:64-126) on the front end,
+    drop6 / drop7 included: the masks are the library's first two Bernoulli draws after
+    seeding, which the oracle reproduces from the seed."""
+    from minerva_amd.owl import models
+    from oracle import nets
+    batch, lr, seed, keep = 2, 0.01, 424242, 0.5
+    params, data, label = nets.make_inputs("alexnet", batch)
+    say("alexnet + dropout oracle step b=2 (CPU)")
+    want_p, res = nets.alexnet_step(dict(params), data, label, lr, batch, dropout_rate=keep, seed_base=seed)
+    say("owl alexnet step b=2")
+    net = models.AlexNet()
+    net.load([params["w%d" % k] for k in range(8)], [params["b%d" % k] for k in range(8)])
+    owl.set_random_seed(seed)
+    out, wgrad, bgrad = net.train_one_mb(_nd(owl, data, [227, 227, 3, batch]),
+                                         _nd(owl, label, [1000, batch]), keep)
+    net.sgd(wgrad, bgrad, batch, lr)
+    owl.wait_for_all()
+    got = {"prob": out.to_numpy().ravel()}
+    for k in range(8):
+        got["g_w%d" % k] = wgrad[k].to_numpy().ravel()
+        got["g_b%d" % k] = bgrad[k].to_numpy().ravel()
+        got["w%d" % k] = net.weights[k].to_numpy().ravel()
+        got["b%d" % k] = net.bias[k].to_numpy().ravel()
+    compare_step(got, want_p, res, lr=lr, batch=batch, deep=True)
+    # the momentum / weight-decay update of the application, one step from zero deltas
+    before = [w.to_numpy().copy() for w in net.weights]
+    net.update(wgrad, bgrad, batch, 0.9, lr, 0.0005)
+    f = np.float32
+    for k in (0, 7):
+        delta = (f(0.9) * f(0)) - f(lr / batch) * wgrad[k].to_numpy() - f(lr * 0.0005) * before[k]
+        assert normwise(net.weights[k].to_numpy(), before[k] + delta) <= 1e-6
