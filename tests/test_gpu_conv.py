@@ -318,6 +318,9 @@ LRN = [
     (2, 96, 27, 27, 5, 1e-4, 0.75),   # AlexNet norm1 (after pool1) and its constants
     (2, 256, 13, 13, 5, 1e-4, 0.75),  # norm2
     (70, 5, 9, 7, 5, 1e-1, 0.75),     # image boundaries inside a wavefront
+    (3, 20, 55, 55, 5, 1e-4, 0.75),   # odd planes: whole wavefronts re-cut their runs, others straddle planes
+    (2, 33, 31, 33, 3, 1e-2, 0.75),   # every channel starts at a different offset from a 64-byte boundary
+    (2, 24, 28, 28, 7, 1e-2, 0.75),   # planes that start on 64-byte boundaries
 ]
 
 
@@ -338,6 +341,33 @@ def test_lrn_against_oracle(gpu, ora, p):
     gpu.call("mnv_lrn_bwd", dx.p, dtop.p, dsc.p, ddy.p, dbd.p, size, ctypes.c_float(alpha),
              ctypes.c_float(beta), N, C, H, W)
     assert normwise(gpu.down(dbd), ora.lrn_bwd(x, top, scale, dy, size, alpha, beta, N, C, H, W)) <= TOL
+
+
+@pytest.mark.parametrize("offset", [1, 5, 16])
+def test_lrn_tensors_off_their_natural_alignment(gpu, ora, offset):
+    """scale / top (and the inputs) `offset` floats into their allocations."""
+    N, C, H, W, size, alpha, beta = 2, 12, 23, 23, 5, 1e-2, 0.75
+    n = N * C * H * W
+    x = _rand(n, 64) * 3
+    dy = _rand(n, 65)
+    pad = np.full(offset, np.nan, np.float32)
+    say("lrn offset", offset)
+    dx = gpu.up(np.concatenate([pad, x]))
+    ds, dt = gpu.up(np.full(n + offset + 3, np.nan, np.float32)), gpu.up(np.full(n + offset + 7, np.nan, np.float32))
+    f = ctypes.c_float
+    gpu.call("mnv_lrn_fwd", dx.offset(offset), ds.offset(offset), dt.offset(offset), size, f(alpha), f(beta), N, C, H, W)
+    top, scale = ora.lrn_fwd(x, size, alpha, beta, N, C, H, W)
+    got_s, got_t = gpu.down(ds), gpu.down(dt)
+    assert normwise(got_s[offset:offset + n], scale) <= 1e-6 and normwise(got_t[offset:offset + n], top) <= TOL
+    assert np.isnan(got_s[:offset]).all() and np.isnan(got_s[offset + n:]).all(), "wrote outside scale"
+    assert np.isnan(got_t[:offset]).all() and np.isnan(got_t[offset + n:]).all(), "wrote outside top"
+    dtop, dsc, ddy = gpu.up(np.concatenate([pad, top])), gpu.up(np.concatenate([pad, scale])), gpu.up(np.concatenate([pad, dy]))
+    dbd = gpu.up(np.full(n + offset + 5, np.nan, np.float32))
+    gpu.call("mnv_lrn_bwd", dx.offset(offset), dtop.offset(offset), dsc.offset(offset), ddy.offset(offset),
+             dbd.offset(offset), size, f(alpha), f(beta), N, C, H, W)
+    got = gpu.down(dbd)
+    assert normwise(got[offset:offset + n], ora.lrn_bwd(x, top, scale, dy, size, alpha, beta, N, C, H, W)) <= TOL
+    assert np.isnan(got[:offset]).all() and np.isnan(got[offset + n:]).all(), "wrote outside bottom_diff"
 
 
 def test_lrn_batch_256_properties(gpu):
