@@ -132,13 +132,18 @@ struct ConvFwd {
 // Forward without padding (ph == pw == 0, any channel count and stride).  Every tap of
 // every output position is a real pixel, so the pixel offset is base(position) + koff(k)
 // with koff(k) = ((c*H + R-1-r')*W + S-1-s')*4 for the flat reduction index k = (c, r', s').
-// koff is tabulated in LDS once per workgroup; a slab then costs one LDS read and four
-// adds per vector, and nothing is decomposed or bounds-tested in the main loop.  The
+// koff is tabulated in LDS once per workgroup; a slab then costs one 16-byte LDS read and
+// four adds per vector, and nothing is decomposed or bounds-tested in the main loop.  The
 // filter needs no copy: in this order it already is the column-major K x Kout operand.
 // Period 0 holds the full slabs, period 1 the last, partial one (masked filter loads).
+// A vector is four consecutive k at ONE output position (k-fast): its four loads are 4-byte
+// gathers either way, but with four lanes per position a load instruction touches about 20
+// cache lines (16 positions, the taps of a vector a few floats apart) where four
+// consecutive positions per lane touched 64 at a stride of four pixels -- and conv1
+// (stride 4, C = 3) was bound by those L1 look-ups, not by the matrix pipe.
 struct ConvFwdNP {
-  static constexpr bool A_KFAST = false, B_KFAST = true;
-  static constexpr int A_NOFF = 4, B_NOFF = 4;
+  static constexpr bool A_KFAST = true, B_KFAST = true;
+  static constexpr int A_NOFF = 1, B_NOFF = 4;
   const float* __restrict__ bottom;
   const float* __restrict__ filter;
   const float* __restrict__ bias;
@@ -170,24 +175,24 @@ struct ConvFwdNP {
   __device__ void a_init(const Res&, AState&, int) const {}
   __device__ void b_init(const Res&, BState&, int) const {}
   // rows past M are never stored, so they may read any valid pixel
-  __device__ void a_period(const AState&, unsigned (&off)[4], int m, int, int) const {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      int mm = m + q < M ? m + q : 0;
-      int img = mnv_fastdiv(mm, g.d_HoWo);
-      int pos = mm - img * g.HoWo;
-      int i = mnv_fastdiv(pos, g.d_Wo);
-      int j = pos - i * g.Wo;
-      off[q] = (unsigned)(img * g.C * g.HW + i * g.sv * g.W + j * g.sh) * 4u;
-    }
+  __device__ void a_period(const AState&, unsigned (&off)[1], int m, int, int) const {
+    int mm = m < M ? m : 0;
+    int img = mnv_fastdiv(mm, g.d_HoWo);
+    int pos = mm - img * g.HoWo;
+    int i = mnv_fastdiv(pos, g.d_Wo);
+    int j = pos - i * g.Wo;
+    off[0] = (unsigned)(img * g.C * g.HW + i * g.sv * g.W + j * g.sh) * 4u;
   }
-  __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[4], int period, int s,
+  // an entry past K is MNV_OOB, and MNV_OOB plus any pixel offset is still out of range
+  __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[1], int period, int s,
                          int kl, float (&v)[4]) const {
-    const unsigned t = r.tab[(period * spp + s) * 16 + kl];
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const u4 t = *reinterpret_cast<const u4*>(
+        __builtin_assume_aligned(r.tab + (period * spp + s) * 16 + kl, 16));
 #pragma unroll
     for (int q = 0; q < 4; ++q)
       v[q] = __builtin_bit_cast(float,
-                                __builtin_amdgcn_raw_buffer_load_b32(r.a, (int)(off[q] + t), 0, 0));
+                                __builtin_amdgcn_raw_buffer_load_b32(r.a, (int)(off[0] + t[q]), 0, 0));
   }
   // filter element (k, n) at n*K + k: four consecutive k are one 16-byte load (4-byte
   // aligned is enough for a buffer load)
