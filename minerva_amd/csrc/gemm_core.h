@@ -18,6 +18,8 @@
 //
 // Roofline: fp32 MFMA, 2*M*N*K algorithmic flops; 256 flop/clk/CU.
 #pragma once
+#include <type_traits>
+
 #include "mnv_common.h"
 
 typedef float mnv_f16v __attribute__((ext_vector_type(16)));
@@ -206,8 +208,12 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
   }
   __syncthreads();
 
-  for (int slab = slab_begin; slab < slab_end; ++slab) {
-    const int buf = (slab - slab_begin) & 1;
+  // One slab out of LDS buffer BUF.  The buffer is a compile-time constant (the loop below
+  // is unrolled by two) so that the LDS addresses of both buffers are one register plus an
+  // immediate: selecting the buffer at run time cost seven address instructions per slab,
+  // and every vector instruction in this loop is time the matrix pipe stands still.
+  auto step = [&](auto BUF) {
+    constexpr int buf = decltype(BUF)::value;
     // Loads of the next slab are in flight while this one is multiplied.  Past the end of
     // the k range the loads run past the tensors and read as 0 (or fetch a slab of the
     // next split, which is never multiplied).
@@ -260,7 +266,13 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
     }
     stash(buf ^ 1);
     __syncthreads();
+  };
+  int slab = slab_begin;
+  for (; slab + 1 < slab_end; slab += 2) {
+    step(std::integral_constant<int, 0>{});
+    step(std::integral_constant<int, 1>{});
   }
+  if (slab < slab_end) step(std::integral_constant<int, 0>{});
 
   // Accumulator register r of lane (lm, lk) holds C[m = lm, n = lk*4 + r%4 + 8*(r/4)]
   // of its 32x32 block.
