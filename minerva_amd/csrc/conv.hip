@@ -476,15 +476,18 @@ struct ConvBwdFilterFast {
     st.trow = (t < taps_per_block ? t : 0) * PP;  // rows past M read a valid table row; cbase masks them
   }
   __device__ void b_init(const Res&, BState&, int) const {}
-  __device__ void a_period(const AState&, unsigned (&off)[1], int, int, int) const { off[0] = 0; }
-  // off[0] is unused for A: the offsets come from the table every slab.
-  __device__ void a_load(const Res& r, const AState& st, const unsigned (&)[1], int period, int s,
-                         int kl, float (&v)[4]) const {
+  // off[0]: byte offset of the vector's entries of slab 0 in the table (the pixel offsets
+  // come from the table every slab); a slab then adds s * 64 to it, one instruction
+  __device__ void a_period(const AState& st, unsigned (&off)[1], int, int kl, int) const {
+    off[0] = (unsigned)(st.trow + kl) * 4u;
+  }
+  __device__ void a_load(const Res& r, const AState& st, const unsigned (&off)[1], int period, int s,
+                         int, float (&v)[4]) const {
     // the four entries are one aligned 16-byte LDS read: rows are PP (a multiple of 16)
     // entries long and kl is a multiple of 4
     typedef unsigned u4 __attribute__((ext_vector_type(4)));
-    const u4 t = *reinterpret_cast<const u4*>(
-        __builtin_assume_aligned(r.tab + st.trow + s * 16 + kl, 16));
+    const u4 t = *reinterpret_cast<const u4*>(__builtin_assume_aligned(
+        reinterpret_cast<const char*>(r.tab) + (off[0] + (unsigned)s * 64u), 16));
     const unsigned soff = (unsigned)period * (unsigned)(g.C * g.HW) * 4u;
 #pragma unroll
     for (int q = 0; q < 4; ++q)
@@ -500,9 +503,13 @@ struct ConvBwdFilterFast {
     if (s * 16 + 16 <= g.HoWo) {  // uniform: every position of the slab is inside the image
       mnv_fetch_vec<1>(r.b, off, soff, v);
     } else {
+      // the last slab of an image; the empty asm keeps its index arithmetic in this branch
+      // (hoisted above the test it would run in every slab: five vector instructions)
+      int first = s * 16 + kl;
+      asm volatile("" : "+v"(first));
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        bool ok = s * 16 + kl + q < g.HoWo;
+        bool ok = first + q < g.HoWo;
         v[q] = __builtin_bit_cast(
             float, __builtin_amdgcn_raw_buffer_load_b32(r.b, (int)(ok ? off[0] + 4u * q : MNV_OOB),
                                                         (int)soff, 0));
