@@ -302,3 +302,21 @@ def test_alexnet_application_step_with_dropout(owl, ora):
     for k in (0, 7):
         delta = (f(0.9) * f(0)) - f(lr / batch) * wgrad[k].to_numpy() - f(lr * 0.0005) * before[k]
         assert normwise(net.weights[k].to_numpy(), before[k] + delta) <= 1e-6
+
+
+def test_errors_surface_as_exceptions(owl):
+    """The reference aborts the process on a failed CHECK; the front end raises instead."""
+    from minerva_amd import hostapi
+    a, b = owl.zeros([4, 3]), owl.zeros([5, 3])
+    with pytest.raises(hostapi.HostError):
+        a + b                      # neither equal shapes nor a dimension of size 1
+    with pytest.raises(hostapi.HostError):
+        a * b                      # inner dimensions differ
+    with pytest.raises(hostapi.HostError):
+        a.sum(2)                   # no such dimension
+    with pytest.raises(ValueError):
+        owl.zeros([4, 0])
+    with pytest.raises(ValueError):
+        owl.set_device(12345)
+    # the device keeps working after a refused operator
+    assert (a + 1.0).count_zero() == 0
