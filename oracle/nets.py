@@ -125,16 +125,9 @@ def seed_sequence(base, count):
     return out
 
 
-def alexnet_step(p, data, label, lr, batch, classes=1000, dropout_rate=0.0, seed_base=None):
-    """dropout_rate > 0 adds the reference application's drop6 / drop7
-    (owl/apps/imagenet_alexnet/alexnet.py:86-89,97-101) with the masks the library draws for
-    the first two RandBernoulli calls after SetRandomSeed(seed_base)."""
+def alexnet_forward(p, data, batch, classes=1000, masks=None):
+    """Forward pass only: (acts[0..11], probabilities).  masks = (mask6, mask7) for dropout."""
     N = batch
-    drop = dropout_rate > 0.0
-    if drop:
-        s6, s7 = seed_sequence(seed_base, 2)
-        mask6 = ora.rand_bernoulli(4096 * N, s6, dropout_rate)
-        mask7 = ora.rand_bernoulli(4096 * N, s7, dropout_rate)
     cv = [(N,) + c for c in ALEX_CONVS]
     pool = lambda C, H: (N, C, H, H, 2, 2, 3, 3, 0, 0)
     acts = [None] * 12
@@ -148,13 +141,33 @@ def alexnet_step(p, data, label, lr, batch, classes=1000, dropout_rate=0.0, seed
     acts[7] = _relu(ora.conv_fwd(acts[6], p["w4"], p["b4"], *cv[4]))     # 256 x 13 x 13
     acts[8] = ora.pool_fwd(ora.POOL_MAX, acts[7], *pool(256, 13))        # 6 -> 9216
     acts[9] = _relu(_fc(p["w5"], acts[8], p["b5"], 4096, 9216, N))
-    if drop:
-        acts[9] = ora.arithmetic(ora.MUL, acts[9], mask6)
+    if masks:
+        acts[9] = ora.arithmetic(ora.MUL, acts[9], masks[0])
     acts[10] = _relu(_fc(p["w6"], acts[9], p["b6"], 4096, 4096, N))
-    if drop:
-        acts[10] = ora.arithmetic(ora.MUL, acts[10], mask7)
+    if masks:
+        acts[10] = ora.arithmetic(ora.MUL, acts[10], masks[1])
     acts[11] = _fc(p["w7"], acts[10], p["b7"], classes, 4096, N)
     out = ora.softmax_instance_fwd(acts[11], N, classes, 1, 1)
+    return acts, out
+
+
+def alexnet_step(p, data, label, lr, batch, classes=1000, dropout_rate=0.0, seed_base=None,
+                 keep=False):
+    """dropout_rate > 0 adds the reference application's drop6 / drop7
+    (owl/apps/imagenet_alexnet/alexnet.py:86-89,97-101) with the masks the library draws for
+    the first two RandBernoulli calls after SetRandomSeed(seed_base).  keep=True also returns
+    the activations ("acts") and sensitivities ("sens") of every layer in the results."""
+    N = batch
+    drop = dropout_rate > 0.0
+    masks = None
+    if drop:
+        s6, s7 = seed_sequence(seed_base, 2)
+        mask6 = ora.rand_bernoulli(4096 * N, s6, dropout_rate)
+        mask7 = ora.rand_bernoulli(4096 * N, s7, dropout_rate)
+        masks = (mask6, mask7)
+    cv = [(N,) + c for c in ALEX_CONVS]
+    pool = lambda C, H: (N, C, H, H, 2, 2, 3, 3, 0, 0)
+    acts, out = alexnet_forward(p, data, N, classes, masks)
     sens = [None] * 12
     sens[11] = ora.arithmetic(ora.SUB, out, label)
     mm = lambda a, b, m, n, k: ora.matmult(a, b, m, n, k, fast=True)
@@ -204,6 +217,8 @@ def alexnet_step(p, data, label, lr, batch, classes=1000, dropout_rate=0.0, seed
     res["l1_b2"] = ora.conv_bwd_bias(np.abs(sens[5]), N, 384, 13, 13)
     res["l1_b1"] = ora.conv_bwd_bias(np.abs(sens[3]), N, 256, 27, 27)
     res["l1_b0"] = ora.conv_bwd_bias(np.abs(sens[1]), N, 96, 55, 55)
+    if keep:
+        res["acts"], res["sens"] = acts, sens
     return newp, res
 
 

@@ -171,7 +171,8 @@ def test_conv_alexnet_layers_small_batch_against_oracle(gpu, ora, case):
     assert normwise(cv.bwd_data(dy, w), ora.conv_bwd_data(dy, w, *p)) <= TOL
 
 
-@pytest.mark.parametrize("case", [ALEXNET[1], ALEXNET[4], ALEXNET[0]], ids=lambda c: c[0])
+@pytest.mark.parametrize("case", [ALEXNET[1], ALEXNET[2], ALEXNET[3], ALEXNET[4], ALEXNET[0]],
+                         ids=lambda c: c[0])
 def test_conv_batch_256_properties(gpu, case):
     name, p = case[0], (256,) + case[2:]
     N, C, K, H, W, ph, pw, sv, sh, R, S = p

@@ -145,6 +145,65 @@ def test_activation_backward(gpu, ora, n):
             assert normwise(gpu.down(dout), ref) <= TOL
 
 
+def test_non_temporal_instantiations_8192x8192(gpu, ora):
+    """Calls whose traffic reaches 512 MB run the non-temporal instantiations of the streaming
+    kernels: at 8192 x 8192 that is every one-input operator and every activation gradient of
+    the bandwidth benchmark, and the cached softmax gradient on lines of 8192.  Each is
+    compared with the oracle at that size (selections and single IEEE operations bit for bit)."""
+    m = n_lines = 8192
+    n = m * n_lines
+    x = _rand(n, 16, 2.0)
+    x[:6] = [0.0, -0.0, -2.0, 2.0, 1e-30, -1e-30]
+    dy = _rand(n, 17)
+    dx, ddy, dout = gpu.up(x), gpu.up(dy), gpu.empty(n)
+    v = 3.291
+    for name, args, ref in (
+            ("mnv_const_mul", (ctypes.c_float(v),), lambda: ora.arithmetic_const(ora.MUL, 1, v, x)),
+            ("mnv_const_div", (ctypes.c_float(v),), lambda: ora.arithmetic_const(ora.DIV, 1, v, x)),
+            ("mnv_copy", (), lambda: x),
+            ("mnv_neg", (), lambda: ora.elewise(ora.NEG, x)),
+            ("mnv_relu_fwd", (), lambda: ora.activation_fwd(ora.RELU, x))):
+        say(name, "8192x8192")
+        gpu.call(name, dx.p, dout.p, *args, n)
+        assert_bits_equal(gpu.down(dout), ref(), name + " 8192^2")
+    say("mnv_div 8192x8192")
+    den = dy.copy()
+    den[den == 0] = 1
+    dden = gpu.up(den)
+    gpu.call("mnv_div", dx.p, dden.p, dout.p, n)
+    assert_bits_equal(gpu.down(dout), ora.arithmetic(ora.DIV, x, den), "div 8192^2")
+    del dden
+    say("mnv_exp 8192x8192")
+    gpu.call("mnv_exp", dx.p, dout.p, n)
+    assert np.max(np.abs(gpu.down(dout) / ora.elewise(ora.EXP, x) - 1)) <= TOL
+    tops = {}
+    for name, alg in (("mnv_sigmoid_fwd", ora.SIGMOID), ("mnv_tanh_fwd", ora.TANH)):
+        say(name, "8192x8192")
+        gpu.call(name, dx.p, dout.p, n)
+        tops[alg] = ora.activation_fwd(alg, x)
+        assert normwise(gpu.down(dout), tops[alg]) <= TOL
+    tops[ora.RELU] = ora.activation_fwd(ora.RELU, x)
+    for name, alg in (("mnv_relu_bwd", ora.RELU), ("mnv_sigmoid_bwd", ora.SIGMOID),
+                      ("mnv_tanh_bwd", ora.TANH)):
+        say(name, "8192x8192")
+        dtop = gpu.up(tops[alg])
+        gpu.call(name, dx.p, dtop.p, ddy.p, dout.p, n)
+        ref = ora.activation_bwd(alg, dy, tops[alg], x)
+        if alg == ora.RELU:
+            assert_bits_equal(gpu.down(dout), ref, name + " 8192^2")
+        else:
+            assert normwise(gpu.down(dout), ref) <= TOL
+        del dtop
+    say("softmax_instance_bwd 8192 lines of 8192")
+    top = ora.softmax_instance_fwd(x, n_lines, m, 1, 1)
+    dtop = gpu.up(top)
+    gpu.call("mnv_softmax_instance_bwd", ddy.p, dtop.p, dout.p, n_lines, m, 1, 1)
+    got = gpu.down(dout).reshape(n_lines, m)
+    ref = ora.softmax_instance_bwd(dy, top, n_lines, m, 1, 1).reshape(n_lines, m)
+    err = np.max(np.abs(got.astype(np.float64) - ref), axis=1) / np.max(np.abs(ref), axis=1)
+    assert err.max() <= TOL, "softmax bwd: worst line %d, %.3e" % (int(err.argmax()), err.max())
+
+
 NORM_SHAPES = [(9, 7), (1, 5), (5, 1), (1000, 33), (4096, 256), (8192, 64), (10, 256)]
 
 
