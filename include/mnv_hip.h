@@ -36,6 +36,7 @@ extern "C" {
 #define MNV_OK 0
 #define MNV_ERR_INVALID (-1)
 #define MNV_ERR_WORKSPACE (-2)
+#define MNV_ERR_TOO_LARGE (-3)
 
 typedef void* mnv_stream_t;
 
@@ -150,6 +151,22 @@ int mnv_maxindex_row(const float* in, float* out, int m, int n, mnv_stream_t str
 size_t mnv_sgemm_nn_workspace_bytes(int m, int n, int k);
 int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k,
                  void* workspace, size_t workspace_bytes, mnv_stream_t stream);
+
+/* The same product for callers that cannot allocate device memory or lend a workspace (code
+ * under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  No counterpart
+ * in the reference, whose launchers allocate at will (cuda_perform.cu:253,674).  The split-k
+ * partial sums live in a device array of MNV_SGEMM_STATIC_SCRATCH_BYTES that is part of the
+ * library image on every GPU; the call allocates and frees nothing and returns the bits
+ * mnv_sgemm_nn returns with a workspace of that size.  Limit: m*n*2 floats must fit the
+ * array (m*n <= 4 Mi elements), else MNV_ERR_TOO_LARGE -- larger outputs fill the chip
+ * without splitting, call mnv_sgemm_nn with a NULL workspace for them.  All calls on one GPU
+ * share the array: calls that overlap on one GPU (different streams or threads) race; calls
+ * on one stream do not.  Nothing in the array needs clearing between calls (every partial
+ * sum that is read was written by the same call).  The first call on a device looks the
+ * array's address up (hipGetSymbolAddress): make it outside a graph capture. ---- */
+#define MNV_SGEMM_STATIC_SCRATCH_BYTES (32u << 20)
+int mnv_sgemm_nn_static(const float* a, const float* b, float* c, int m, int n, int k,
+                        mnv_stream_t stream);
 
 /* ---- transpose: CudaPerformTranspose (cuda_perform.h:19; cublasSgeam T,N).
  * a is {m,n}; c is {n,m}; c[j + i*n] = a[i + j*m]. ---- */

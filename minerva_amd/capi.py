@@ -53,6 +53,7 @@ PROTOTYPES = {
     "mnv_error_string": [_I],
     "mnv_sgemm_nn_workspace_bytes": [_I, _I, _I],
     "mnv_sgemm_nn": [_P, _P, _P, _I, _I, _I, _P, c_sz, _S],
+    "mnv_sgemm_nn_static": [_P, _P, _P, _I, _I, _I, _S],
     "mnv_transpose": [_P, _P, _I, _I, _S],
     "mnv_copy": [_P, _P, c_sz, _S],
     "mnv_fill": [_P, c_sz, c_f, _S],

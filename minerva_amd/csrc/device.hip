@@ -208,6 +208,7 @@ const char* mnv_error_string(int status) {
   if (status == MNV_OK) return "ok";
   if (status == MNV_ERR_INVALID) return "invalid argument (null pointer or non-positive extent)";
   if (status == MNV_ERR_WORKSPACE) return "workspace too small";
+  if (status == MNV_ERR_TOO_LARGE) return "problem exceeds the maximum of this entry point's fixed scratch area";
   return hipGetErrorString(static_cast<hipError_t>(status));
 }
 

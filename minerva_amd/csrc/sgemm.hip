@@ -4,7 +4,15 @@
 // Built on the fp32 MFMA core in gemm_core.h; A is fetched x-fast (m contiguous),
 // B k-fast (k contiguous).  Products with too few output tiles to fill 256 CUs split
 // the k range over blockIdx.z when the caller lends a workspace.
+#include <mutex>
+
 #include "gemm_core.h"
+
+// Split-k partial sums of mnv_sgemm_nn_static: one array per GPU the library is loaded on,
+// held until the process ends.  In host code the name `scratch` is only a handle for
+// hipGetSymbolAddress; kernels and every other use take the address it returns.
+#define MNV_SGEMM_STATIC_SCRATCH_FLOATS ((size_t)MNV_SGEMM_STATIC_SCRATCH_BYTES / sizeof(float))
+static __device__ __align__(256) float scratch[MNV_SGEMM_STATIC_SCRATCH_FLOATS];
 
 namespace {
 
@@ -111,6 +119,42 @@ SgemmPlan plan_sgemm(int m, int n, int k, size_t ws_floats) {
   return best;
 }
 
+#define MNV_MAX_DEVICES 64
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[MNV_MAX_DEVICES];  // device address of `scratch` on each GPU
+
+// The address of the current device's copy of `scratch`, looked up once per device.
+int scratch_address(float** out) {
+  int dev = -1;
+  MNV_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= MNV_MAX_DEVICES) return MNV_ERR_INVALID;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    MNV_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return MNV_ERR_INVALID;
+    g_scratch_ptr[dev] = static_cast<float*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return MNV_OK;
+}
+
+int sgemm_nn_impl(const float* a, const float* b, float* c, int m, int n, int k, void* workspace,
+                  size_t workspace_bytes, hipStream_t s) {
+  bool vec = (m % 4 == 0) && (k % 4 == 0) && mnv_aligned16(a) && mnv_aligned16(b);
+  const SgemmPlan plan = plan_sgemm(m, n, k, workspace ? workspace_bytes / sizeof(float) : 0);
+  const bool small = plan.small;
+  const int splits = plan.splits;
+  if (vec) {
+    SgemmNN<true> p = make_sgemm<true>(a, b, c, m, n, k);
+    return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
+                 : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
+  }
+  SgemmNN<false> p = make_sgemm<false>(a, b, c, m, n, k);
+  return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
+               : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
+}
+
 }  // namespace
 
 extern "C" {
@@ -127,19 +171,21 @@ int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k, 
   if (!a || !b || !c || m < 0 || n < 0 || k <= 0) return MNV_ERR_INVALID;
   // operands are addressed through 32-bit buffer offsets: at most 2^31 - 1 bytes each
   if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
-  hipStream_t s = mnv_stream(stream);
-  bool vec = (m % 4 == 0) && (k % 4 == 0) && mnv_aligned16(a) && mnv_aligned16(b);
-  const SgemmPlan plan = plan_sgemm(m, n, k, workspace ? workspace_bytes / sizeof(float) : 0);
-  const bool small = plan.small;
-  const int splits = plan.splits;
-  if (vec) {
-    SgemmNN<true> p = make_sgemm<true>(a, b, c, m, n, k);
-    return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
-                 : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
-  }
-  SgemmNN<false> p = make_sgemm<false>(a, b, c, m, n, k);
-  return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
-               : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
+  return sgemm_nn_impl(a, b, c, m, n, k, workspace, workspace_bytes, mnv_stream(stream));
+}
+
+int mnv_sgemm_nn_static(const float* a, const float* b, float* c, int m, int n, int k,
+                        mnv_stream_t stream) {
+  if (m == 0 || n == 0) return MNV_OK;
+  if (!a || !b || !c || m < 0 || n < 0 || k <= 0) return MNV_ERR_INVALID;
+  if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
+  // at least two k ranges of partial sums must fit the static array
+  if ((unsigned long long)m * (unsigned long long)n * 2ull > MNV_SGEMM_STATIC_SCRATCH_FLOATS)
+    return MNV_ERR_TOO_LARGE;
+  float* ws = nullptr;
+  int rc = scratch_address(&ws);
+  if (rc) return rc;
+  return sgemm_nn_impl(a, b, c, m, n, k, ws, MNV_SGEMM_STATIC_SCRATCH_BYTES, mnv_stream(stream));
 }
 
 }  // extern "C"
