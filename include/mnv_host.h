@@ -126,6 +126,10 @@ int mnvh_net_param_info(void* net, int index, char* name_out /* >= 16 bytes */, 
 int mnvh_net_set_param(void* net, const char* name, const float* host, size_t floats);
 /* name: a parameter ("w0"...), "prob", or "g_<param>" (gradient of the last step) */
 int mnvh_net_read(void* net, const char* name, float* host_out, size_t floats);
+/* For tests: the following steps of an "alexnet" network also keep their activations, read
+ * with mnvh_net_read as "act1" ... "act10" (the outputs of conv1+relu, pool1, conv2+relu,
+ * pool2, conv3..5+relu, pool5, fc6, fc7 after ReLU and dropout). */
+int mnvh_net_keep_activations(void* net, int on);
 /* Uploads one batch; it stays resident in HBM for the following steps. */
 int mnvh_net_load_batch(void* net, const float* data, size_t data_floats, const float* label,
                         size_t label_floats);

@@ -447,6 +447,10 @@ int mnvh_net_read(void* net, const char* name, float* host_out, size_t floats) {
   });
 }
 
+int mnvh_net_keep_activations(void* net, int on) {
+  return Guard([&] { static_cast<NetHandle*>(net)->net->keep_activations = on != 0; });
+}
+
 int mnvh_net_load_batch(void* net, const float* data, size_t data_floats, const float* label,
                         size_t label_floats) {
   return Guard([&] {

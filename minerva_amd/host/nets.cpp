@@ -154,6 +154,8 @@ void AlexNet::Step(const Tensor& data, const Tensor& label, float lr) {
       rt->SoftmaxForward(rt->Reshape(acts[11], Scale{classes_, 1, 1, n}), SoftmaxAlgorithm::kInstance),
       Scale{classes_, n});
   results["prob"] = out;
+  if (keep_activations)
+    for (int i = 1; i <= 10; ++i) results["act" + std::to_string(i)] = acts[i];
   // BP
   sens[11] = rt->Sub(out, label);
   sens[10] = rt->MatMult(rt->Trans(W(7)), sens[11]);                            // fc8

@@ -28,6 +28,9 @@ class Net {
   std::vector<std::string> param_names;   // "w0", "b0", ...
   std::map<std::string, Tensor> params;   // current parameters
   std::map<std::string, Tensor> results;  // "prob" and "g_<param>" of the last Step
+  // Tests only: the step also leaves its activations in `results` ("act1", "act2", ...),
+  // which keeps their device blocks alive until the next step.
+  bool keep_activations = false;
 
  protected:
   // w <- w - (lr / batch) * g : ArithmeticConst(mult, const on the left) + Arithmetic(sub)

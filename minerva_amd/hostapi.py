@@ -224,6 +224,10 @@ class Net:
                                          l.ctypes.data_as(fp), ctypes.c_size_t(l.size)),
                "net_load_batch")
 
+    def keep_activations(self, on=True):
+        """The following steps also keep "act1" ... "act10" readable (AlexNet only)."""
+        _check(lib().mnvh_net_keep_activations(self.h, 1 if on else 0), "net_keep_activations")
+
     def step(self, lr):
         _check(lib().mnvh_net_step(self.h, ctypes.c_float(lr)), "net_step")
 

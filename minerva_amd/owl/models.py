@@ -21,6 +21,8 @@ class AlexNet(object):
         self.bias_shapes = [[96], [256], [384], [384], [256], [4096, 1], [4096, 1], [self.classes, 1]]
         self.num_weights = len(self.weight_shapes)
         self.weights = self.bias = self.weightsdelta = self.biasdelta = None
+        self.keep_activations = False  # tests: train_one_mb leaves its activations in last_acts
+        self.last_acts = None
 
     def _zero_deltas(self):
         self.weightsdelta = [zeros(s) for s in self.weight_shapes]
@@ -67,6 +69,8 @@ class AlexNet(object):
             acts[10] = ele.mult(acts[10], mask7)
         acts[11] = w[7] * acts[10] + b[7]
         out = co.softmax(acts[11], co.soft_op.instance)
+        if self.keep_activations:
+            self.last_acts = list(acts)
 
         sens = [None] * 12
         sens[11] = out - label

@@ -151,33 +151,24 @@ def alexnet_forward(p, data, batch, classes=1000, masks=None):
     return acts, out
 
 
-def alexnet_step(p, data, label, lr, batch, classes=1000, dropout_rate=0.0, seed_base=None,
-                 keep=False):
-    """dropout_rate > 0 adds the reference application's drop6 / drop7
-    (owl/apps/imagenet_alexnet/alexnet.py:86-89,97-101) with the masks the library draws for
-    the first two RandBernoulli calls after SetRandomSeed(seed_base).  keep=True also returns
-    the activations ("acts") and sensitivities ("sens") of every layer in the results."""
+def alexnet_backward(p, acts, out, label, batch, classes=1000, masks=None):
+    """Backward pass from given forward results: (gradients, sensitivities, L1 mass behind
+    every bias gradient).  `acts` / `out` need not come from alexnet_forward: evaluated at
+    another implementation's activations it opens the gates and routes the pooling
+    gradients the way that implementation did."""
     N = batch
-    drop = dropout_rate > 0.0
-    masks = None
-    if drop:
-        s6, s7 = seed_sequence(seed_base, 2)
-        mask6 = ora.rand_bernoulli(4096 * N, s6, dropout_rate)
-        mask7 = ora.rand_bernoulli(4096 * N, s7, dropout_rate)
-        masks = (mask6, mask7)
     cv = [(N,) + c for c in ALEX_CONVS]
     pool = lambda C, H: (N, C, H, H, 2, 2, 3, 3, 0, 0)
-    acts, out = alexnet_forward(p, data, N, classes, masks)
     sens = [None] * 12
     sens[11] = ora.arithmetic(ora.SUB, out, label)
     mm = lambda a, b, m, n, k: ora.matmult(a, b, m, n, k, fast=True)
     sens[10] = mm(ora.transpose(p["w7"], 4096, classes), sens[11], 4096, N, classes)
-    if drop:
-        sens[10] = ora.arithmetic(ora.MUL, sens[10], mask7)
+    if masks:
+        sens[10] = ora.arithmetic(ora.MUL, sens[10], masks[1])
     sens[10] = _relu_bwd(sens[10], acts[10])
     sens[9] = mm(ora.transpose(p["w6"], 4096, 4096), sens[10], 4096, N, 4096)
-    if drop:
-        sens[9] = ora.arithmetic(ora.MUL, sens[9], mask6)
+    if masks:
+        sens[9] = ora.arithmetic(ora.MUL, sens[9], masks[0])
     sens[9] = _relu_bwd(sens[9], acts[9])
     sens[8] = mm(ora.transpose(p["w5"], 9216, 4096), sens[9], 9216, N, 4096)
     sens[7] = _relu_bwd(ora.pool_bwd(ora.POOL_MAX, sens[8], acts[8], acts[7], *pool(256, 13)), acts[7])
@@ -205,18 +196,41 @@ def alexnet_step(p, data, label, lr, batch, classes=1000, dropout_rate=0.0, seed
         "b1": ora.conv_bwd_bias(sens[3], N, 256, 27, 27),
         "b0": ora.conv_bwd_bias(sens[1], N, 96, 55, 55),
     }
+    # L1 mass behind every bias gradient: the scale its rounding error is measured against
+    l1 = {
+        "b7": ora.reduction(ora.SUM, np.abs(sens[11]), [classes, N], [1]),
+        "b6": ora.reduction(ora.SUM, np.abs(sens[10]), [4096, N], [1]),
+        "b5": ora.reduction(ora.SUM, np.abs(sens[9]), [4096, N], [1]),
+        "b4": ora.conv_bwd_bias(np.abs(sens[7]), N, 256, 13, 13),
+        "b3": ora.conv_bwd_bias(np.abs(sens[6]), N, 384, 13, 13),
+        "b2": ora.conv_bwd_bias(np.abs(sens[5]), N, 384, 13, 13),
+        "b1": ora.conv_bwd_bias(np.abs(sens[3]), N, 256, 27, 27),
+        "b0": ora.conv_bwd_bias(np.abs(sens[1]), N, 96, 55, 55),
+    }
+    return g, sens, l1
+
+
+def dropout_masks(batch, dropout_rate, seed_base):
+    """drop6 / drop7 masks: the library's first two RandBernoulli draws after
+    SetRandomSeed(seed_base)."""
+    s6, s7 = seed_sequence(seed_base, 2)
+    return (ora.rand_bernoulli(4096 * batch, s6, dropout_rate),
+            ora.rand_bernoulli(4096 * batch, s7, dropout_rate))
+
+
+def alexnet_step(p, data, label, lr, batch, classes=1000, dropout_rate=0.0, seed_base=None,
+                 keep=False):
+    """dropout_rate > 0 adds the reference application's drop6 / drop7
+    (owl/apps/imagenet_alexnet/alexnet.py:86-89,97-101) with the masks the library draws for
+    the first two RandBernoulli calls after SetRandomSeed(seed_base).  keep=True also returns
+    the activations ("acts") and sensitivities ("sens") of every layer in the results."""
+    masks = dropout_masks(batch, dropout_rate, seed_base) if dropout_rate > 0.0 else None
+    acts, out = alexnet_forward(p, data, batch, classes, masks)
+    g, sens, l1 = alexnet_backward(p, acts, out, label, batch, classes, masks)
     newp = {k: _sgd(p[k], g[k], lr, batch) for k in p}
     res = {"prob": out}
     res.update({"g_" + k: v for k, v in g.items()})
-    # L1 mass behind every bias gradient: the scale its rounding error is measured against
-    res["l1_b7"] = ora.reduction(ora.SUM, np.abs(sens[11]), [classes, N], [1])
-    res["l1_b6"] = ora.reduction(ora.SUM, np.abs(sens[10]), [4096, N], [1])
-    res["l1_b5"] = ora.reduction(ora.SUM, np.abs(sens[9]), [4096, N], [1])
-    res["l1_b4"] = ora.conv_bwd_bias(np.abs(sens[7]), N, 256, 13, 13)
-    res["l1_b3"] = ora.conv_bwd_bias(np.abs(sens[6]), N, 384, 13, 13)
-    res["l1_b2"] = ora.conv_bwd_bias(np.abs(sens[5]), N, 384, 13, 13)
-    res["l1_b1"] = ora.conv_bwd_bias(np.abs(sens[3]), N, 256, 27, 27)
-    res["l1_b0"] = ora.conv_bwd_bias(np.abs(sens[1]), N, 96, 55, 55)
+    res.update({"l1_" + k: v for k, v in l1.items()})
     if keep:
         res["acts"], res["sens"] = acts, sens
     return newp, res

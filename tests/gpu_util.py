@@ -92,43 +92,59 @@ def run_steps(kind, batch, variant, lr, params, batches, **runtime_args):
     return states
 
 
-# A whole training step chains ~20 fp32 operators and both sides round at every one of
-# them.  Besides ordinary rounding noise there is one discontinuous effect: a pre-activation
-# that rounds to different sides of 0 on the two sides flips its ReLU gate, which adds or
-# drops one full-size term in the gradients downstream (seen on conv bias gradients: an
-# error of exactly one term).  So a step is compared this way: probabilities and updated
-# weights normwise at 1e-4; every weight gradient in relative L2 norm at 1e-3 with at least
-# 99.9 % of its entries within 1e-4 of the largest entry; every bias gradient -- a sum of
-# hundreds to thousands of signed, largely cancelling terms -- within 3e-3 of the L1 mass
-# of its terms (one flipped term of a 338-term sum is 3e-3 of that mass), the updated bias
-# within the same bound scaled by lr / batch.  The operators themselves are held to 1e-4
-# (or bit-exactness) one by one in the other test files.
+# A whole training step chains ~20 fp32 operators and both sides round at every one of them.
+# For the shallow networks (MLP, MNIST CNN, batch 16 to 256) the chain is continuous enough
+# that every probability, gradient and updated parameter agrees with the oracle normwise to
+# 1e-4 (measured: <= 1.1e-5).
 def rel_l2(got, ref):
     got = np.asarray(got, np.float64)
     ref = np.asarray(ref, np.float64)
     return float(np.linalg.norm(got - ref) / max(np.linalg.norm(ref), 1e-30))
 
 
-def compare_step(got, newp, res, lr=0.01, batch=1, deep=False):
-    """deep=True (the 12-layer network at batch 2, where a handful of flipped gates among
-    ~10^6 tiny activations is a visible fraction of the gradient signal): gradients are held
-    to 1e-2 in relative L2 norm and 1e-3 in their norms instead of the entrywise rule."""
-    for k, v in newp.items():
-        g, r = got["g_" + k], res["g_" + k]
-        if k.startswith("w") and deep:
-            assert rel_l2(g, r) <= 1e-2, "gradient %s: relative L2 error %.3e" % (k, rel_l2(g, r))
-            ng, nr = np.linalg.norm(g.astype(np.float64)), np.linalg.norm(r.astype(np.float64))
-            assert abs(ng - nr) <= 1e-3 * nr, "gradient norm %s: %.6e vs %.6e" % (k, ng, nr)
-            assert normwise(got[k], v) <= TOL, "updated " + k
-        elif k.startswith("w"):
-            assert rel_l2(g, r) <= 1e-3, "gradient %s: relative L2 error %.3e" % (k, rel_l2(g, r))
-            close = np.abs(g.astype(np.float64) - r) <= TOL * np.max(np.abs(r))
-            assert close.mean() >= 0.999, "gradient %s: %.5f of entries within 1e-4" % (k, close.mean())
-            assert normwise(got[k], v) <= TOL, "updated " + k
-        else:
-            scale = 3e-3 * float(np.max(res["l1_" + k]))
-            err = float(np.max(np.abs(g.astype(np.float64) - r)))
-            assert err <= scale, "gradient %s: error %.3e, bound %.3e" % (k, err, scale)
-            err = float(np.max(np.abs(got[k].astype(np.float64) - v)))
-            assert err <= scale * lr / batch + 1e-12, "updated " + k
-    assert normwise(got["prob"], res["prob"]) <= TOL
+def compare_step(got, newp, res):
+    """Probabilities, every gradient and every updated parameter of one step, normwise 1e-4."""
+    worst = {"prob": normwise(got["prob"], res["prob"])}
+    for k, v in sorted(newp.items()):
+        worst["g_" + k] = normwise(got["g_" + k], res["g_" + k])
+        worst[k] = normwise(got[k], v)
+    say("  step: worst normwise error %.2e (%s)" % (max(worst.values()), max(worst, key=worst.get)))
+    bad = {k: v for k, v in worst.items() if not v <= TOL}
+    assert not bad, bad
+
+
+# The 12-layer AlexNet step is NOT continuous in that sense: a pre-activation that rounds to
+# different sides of 0 on the two sides flips its ReLU gate (and two near-equal values in a
+# pooling window can swap the arg-max), which adds or drops one full-size term in every
+# gradient below it; at batch 2 a single flipped gate among ~10^6 moves the gradients of the
+# layers below by 1e-3 to 1e-2.  So the step is compared in two halves, each at 1e-4:
+#   forward : every activation and the probabilities against the oracle's forward pass;
+#   backward: every gradient against the oracle's backward pass evaluated AT THE GPU's
+#             activations (same gates and routes on both sides);
+# and the update against w - lr/batch * g on the GPU's own gradient, bit for bit.
+ALEX_ACT_ELEMS = {1: 96 * 55 * 55, 2: 96 * 27 * 27, 3: 256 * 27 * 27, 4: 256 * 13 * 13,
+                  5: 384 * 13 * 13, 6: 384 * 13 * 13, 7: 256 * 13 * 13, 8: 9216, 9: 4096,
+                  10: 4096}
+
+
+def compare_alexnet_step(got, gpu_acts, params, data, label, batch, lr, ora_acts, ora_prob,
+                         masks=None):
+    """got: parameters, "g_*" and "prob" of the GPU step; gpu_acts: {1..10: activations}."""
+    from oracle import nets
+    worst = {"prob": normwise(got["prob"], ora_prob)}
+    flips = 0
+    for i, a in gpu_acts.items():
+        worst["act%d" % i] = normwise(a, ora_acts[i])
+        flips += int(np.count_nonzero((a > 0) != (ora_acts[i] > 0)))
+    acts = [data] + [gpu_acts[i] for i in range(1, 11)] + [None]
+    g, _, _ = nets.alexnet_backward(params, acts, got["prob"], label, batch, masks=masks)
+    for k in sorted(params):
+        worst["g_" + k] = normwise(got["g_" + k], g[k])
+        step = (np.float32(lr) / np.float32(batch)) * got["g_" + k]
+        assert_bits_equal(got[k], params[k] - step, "SGD update of " + k)
+    say("  alexnet step: %d of %d gates differ from the oracle's; worst normwise error %.2e (%s)"
+        % (flips, sum(a.size for a in gpu_acts.values()), max(worst.values()),
+           max(worst, key=worst.get)))
+    bad = {k: v for k, v in worst.items() if not v <= TOL}
+    assert not bad, bad
+    return flips

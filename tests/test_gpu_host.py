@@ -8,7 +8,8 @@ import os
 import numpy as np
 import pytest
 
-from gpu_util import TOL, assert_bits_equal, compare_step, normwise, say
+from gpu_util import (ALEX_ACT_ELEMS, TOL, assert_bits_equal, compare_alexnet_step, compare_step,
+                      normwise, say)
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
@@ -272,7 +273,7 @@ def test_four_stream_thread_pool(rt):
         assert_bits_equal(out[i], a + b, "concurrent add %d" % i)
 
 
-def _run_net(kind, batch, steps, sync_each_op, variant=0, lr=0.01):
+def _run_net(kind, batch, steps, sync_each_op, variant=0, lr=0.01, keep_acts=False):
     from minerva_amd import hostapi
     from oracle import nets
     params, data, label = nets.make_inputs(kind, batch)
@@ -281,10 +282,14 @@ def _run_net(kind, batch, steps, sync_each_op, variant=0, lr=0.01):
     for k, v in params.items():
         net.set_param(k, v)
     net.load_batch(data, label)
+    if keep_acts:
+        net.keep_activations()
     for _ in range(steps):
         net.step(lr)
     r.sync()
     out = {k: net.read(k, n) for k, n in net.params.items()}
+    if keep_acts:
+        out["acts"] = {i: net.read("act%d" % i, n * batch) for i, n in ALEX_ACT_ELEMS.items()}
     out.update({"g_" + k: net.read("g_" + k, n) for k, n in net.params.items()})
     out["prob"] = net.read("prob", label.size)
     ops = r.ops_issued()
@@ -301,7 +306,7 @@ def test_mlp_step_matches_oracle(ora):
         p, res = nets.mlp_step(p, data, label, 0.01, 256)
     say("mlp 2 steps, per-op sync")
     got, ops = _run_net("mlp", 256, 2, True)
-    compare_step(got, p, res, batch=256)
+    compare_step(got, p, res)
     say("mlp 2 steps, one sync per step")
     got2, _ = _run_net("mlp", 256, 2, False)
     for k in got:
@@ -318,7 +323,7 @@ def test_cnn_step_matches_oracle(ora, variant):
     p, res = nets.cnn_step(dict(params), data, label, 0.01, batch, **kw)
     say("cnn step variant", variant)
     got, _ = _run_net("cnn", batch, 1, True, variant)
-    compare_step(got, p, res, batch=batch)
+    compare_step(got, p, res)
 
 
 @pytest.mark.parametrize("variant", [0, 1])
@@ -332,7 +337,7 @@ def test_cnn_step_batch_256_matches_oracle(ora, variant):
     p, res = nets.cnn_step(dict(params), data, label, 0.01, batch, **kw)
     say("cnn step b=256 variant", variant)
     got, _ = _run_net("cnn", batch, 1, False, variant)
-    compare_step(got, p, res, batch=batch)
+    compare_step(got, p, res)
 
 
 _ALEX2 = {}
@@ -353,10 +358,10 @@ def _alexnet_oracle_b2():
 def test_alexnet_step_matches_oracle_small_batch(ora):
     batch = 2
     o = _alexnet_oracle_b2()
-    params, data, label, p, res = o["params"], o["data"], o["label"], o["newp"], o["res"]
+    params, data, label, res = o["params"], o["data"], o["label"], o["res"]
     say("alexnet GPU step b=2")
-    got, ops = _run_net("alexnet", batch, 1, False)
-    compare_step(got, p, res, batch=batch, deep=True)
+    got, ops = _run_net("alexnet", batch, 1, False, keep_acts=True)
+    compare_alexnet_step(got, got["acts"], params, data, label, batch, 0.01, res["acts"], res["prob"])
     # the loss itself (cross entropy of the probabilities) agrees to 1e-5
     lab = label.reshape(batch, -1).argmax(axis=1)
     ce = lambda pr: -np.log(pr.reshape(batch, -1)[np.arange(batch), lab].astype(np.float64)).mean()
@@ -463,13 +468,15 @@ def test_alexnet_step_with_dropout_matches_oracle(ora):
     from minerva_amd import hostapi
     from oracle import nets
     batch, seed = 2, 20240607
-    params, data, label = nets.make_inputs("alexnet", batch)
-    say("alexnet + dropout oracle step b=2 (CPU)")
-    p, res = nets.alexnet_step(dict(params), data, label, 0.01, batch, dropout_rate=0.5, seed_base=seed)
+    o = _alexnet_oracle_b2()
+    params, data, label = o["params"], o["data"], o["label"]
+    masks = nets.dropout_masks(batch, 0.5, seed)
+    say("alexnet + dropout oracle forward b=2 (CPU)")
+    acts, prob = nets.alexnet_forward(params, data, batch, masks=masks)
     say("alexnet + dropout GPU step b=2")
     hostapi.Runtime.set_random_seed(seed)
-    got, ops = _run_net("alexnet", batch, 1, False, variant=1)
-    compare_step(got, p, res, batch=batch, deep=True)
+    got, ops = _run_net("alexnet", batch, 1, False, variant=1, keep_acts=True)
+    compare_alexnet_step(got, got["acts"], params, data, label, batch, 0.01, acts, prob, masks=masks)
+    plain = o["res"]
     # dropout changed the result: the plain graph's probabilities differ
-    _, plain = nets.alexnet_step(dict(params), data, label, 0.01, batch)
     assert normwise(got["prob"], plain["prob"]) > 1e-3 or np.max(np.abs(got["g_w7"] - plain["g_w7"])) > 0
