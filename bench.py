@@ -36,6 +36,11 @@ CONV_GFLOP = [53.97, 229.32, 76.55, 114.83, 76.55]
 STEP_GFLOP = 1689.8  # convolutions (fwd, bwd-filter, bwd-data except conv1) + three FC layers
 
 
+def capi_check(rc):
+    from minerva_amd import capi
+    capi.check(rc, "benchmark set-up call")
+
+
 def log(*a):
     print(*a, file=sys.stderr)
     sys.stderr.flush()
@@ -58,14 +63,14 @@ def graph_replay(rt, net, steps, warmup):
 DOMINANT_OP = "conv bp filter"  # operator names: "pad:1*1 stride:1*1 conv bp filter" ...
 
 
-def alexnet_bench(steps, warmup, dataflow=False):
+def alexnet_bench(steps, warmup, dataflow=True):
     from minerva_amd import hostapi
     from minerva_amd import configs
     params, data, label = configs.make_inputs("alexnet", BATCH)
     out = {}
     modes = [("per_step_sync", False), ("per_op_sync", True)]
-    if dataflow:  # kernels of different streams overlap: kept out of the default run so that
-        modes.append(("dataflow", False))  # a kernel trace of it shows undisturbed durations
+    if dataflow:  # kernels of different streams overlap: a kernel trace that wants undisturbed
+        modes.append(("dataflow", False))  # durations runs with --no-dataflow
     for mode, sync_each in modes:
         rt = hostapi.Runtime(0, sync_each_op=sync_each, dataflow=(mode == "dataflow"))
         net = hostapi.Net(rt, "alexnet", BATCH)
@@ -84,10 +89,13 @@ def alexnet_bench(steps, warmup, dataflow=False):
         if plain:
             rt.profile(True, only=DOMINANT_OP)
         rt.sync()
+        per_step = []
         t0 = time.perf_counter()
         for _ in range(steps):
+            ts = time.perf_counter()
             net.step(0.01)
             rt.sync()
+            per_step.append((time.perf_counter() - ts) * 1e3)
         t1 = time.perf_counter()
         prof = rt.profile_read() if plain else {}
         rt.profile(False)
@@ -107,7 +115,8 @@ def alexnet_bench(steps, warmup, dataflow=False):
             graph = graph_replay(rt, net, steps, warmup)
             log("alexnet b=%d recorded step: %d nodes, %.3f ms/replay" %
                 (BATCH, graph["nodes"], graph["ms_per_step"]))
-        out[mode] = {"graph_replay": graph,"ms_per_step": ms, "images_per_s": BATCH / (ms / 1e3),
+        out[mode] = {"graph_replay": graph, "ms_per_step": ms, "images_per_s": BATCH / (ms / 1e3),
+                     "median_ms_per_step": float(np.median(per_step)),
                      "ops_per_step": ops_per_step,
                      "finite": bool(np.isfinite(prob).all()), "profile": prof, "all_ops": all_ops,
                      "h2d_batch_ms": t_h2d}
@@ -154,11 +163,23 @@ def owl_front_end_bench(steps, warmup):
             "ops_per_step": int(ops), "finite": finite}
 
 
-# HBM bytes per launch of the dominant kernel (average over the conv2..conv5 filter
-# gradients), from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB
-# per dispatch), each scaled by what the same counter reads for the 8192^2 copy kernel
-# (256 MiB read, 256 MiB written).  None until measured.
-DOMINANT_KERNEL_TRAFFIC_BYTES = 1.44e9
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_gemm_kernels_hbm_traffic_pmc.txt")
+
+
+def dominant_kernel_traffic():
+    """HBM bytes per launch of the dominant kernel (average over the conv2..conv5 filter
+    gradients), from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB
+    per dispatch, each scaled by what the same counter reads for the 8192^2 copy kernel).
+    The figure is the one recorded in the committed summary of those runs (its line
+    "dominant kernel traffic bytes per launch: X"), so that the two cannot drift apart; None
+    when the summary is absent."""
+    try:
+        for line in open(TRAFFIC_PROFILE):
+            if "dominant kernel traffic bytes per launch:" in line:
+                return float(line.split(":")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def dominant_kernel_roofline(prof, steps):
@@ -178,7 +199,7 @@ def dominant_kernel_roofline(prof, steps):
             "kernel": "mnv_gemm_kernel<128x128x16,ConvBwdFilterFast<false>> (conv2-5 filter gradient)",
             "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-            "traffic": DOMINANT_KERNEL_TRAFFIC_BYTES,
+            "traffic": dominant_kernel_traffic(),
             "avg_launch_ms": round(avg_ms, 4), "launches": launches,
             "algorithmic_gflop_per_launch": round(flops_per_launch / 1e9, 2)}
 
@@ -189,8 +210,9 @@ def op_table(prof, steps):
             for n, (c, ms) in rows]
 
 
-def micro_bench():
-    """SGEMM 4096^3 (N(0,1) inputs) and the 8192^2 elementwise add, events on the stream."""
+def sgemm_bench():
+    """SGEMM at the four shapes of BASELINE.json configs[2] (N(0,1) inputs), events on the
+    stream, median of five batches of ten calls; every call's status is checked."""
     from minerva_amd import capi
     L = capi.lib()
     dev = capi.Device(0)
@@ -199,7 +221,8 @@ def micro_bench():
     a = dev.upload(rng.standard_normal(m * k, dtype=np.float32))
     b = dev.upload(rng.standard_normal(k * n, dtype=np.float32))
     c = dev.empty(m * n)
-    ms = dev.time_ms(lambda: L.mnv_sgemm_nn(a.p, b.p, c.p, m, n, k, None, 0, dev.stream), iters=20, warmup=5)
+    ms = dev.time_ms(lambda: L.mnv_sgemm_nn(a.p, b.p, c.p, m, n, k, None, 0, dev.stream),
+                     iters=10, warmup=5, reps=5)
     tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
     sgemm = {"shape": "4096x4096x4096", "ms": round(ms, 4), "tflops": round(tf, 2),
              "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
@@ -214,14 +237,22 @@ def micro_bench():
         wsb = L.mnv_sgemm_nn_workspace_bytes(mm, nn, kk)
         ws = dev.empty(wsb // 4 + 1)
         t = dev.time_ms(lambda: L.mnv_sgemm_nn(aa.p, bb.p, cc.p, mm, nn, kk, ws.p,
-                                               ctypes.c_size_t(wsb), dev.stream), iters=20, warmup=5)
-        shapes.append({"MxKxN": "%dx%dx%d" % (mm, kk, nn), "ms": round(t, 4),
-                       "tflops": round(2.0 * mm * nn * kk / (t * 1e-3) / 1e12, 2)})
+                                               ctypes.c_size_t(wsb), dev.stream),
+                        iters=10, warmup=5, reps=5)
+        tfl = 2.0 * mm * nn * kk / (t * 1e-3) / 1e12
+        shapes.append({"MxKxN": "%dx%dx%d" % (mm, kk, nn), "ms": round(t, 4), "tflops": round(tfl, 2),
+                       "frac": round(tfl / PEAK_FP32_MFMA_TFLOPS, 4)})
+        log("sgemm %dx%dx%d: %.4f ms, %.1f TFLOP/s" % (mm, kk, nn, t, tfl))
     sgemm["other_shapes"] = shapes
-    ne = 8192 * 8192
-    elt = bandwidth_table(L, dev, rng, ne)
+    return sgemm
+
+
+def eltwise_bench():
+    from minerva_amd import capi
+    dev = capi.Device(0)
+    elt = bandwidth_table(capi.lib(), dev, np.random.default_rng(7), 8192 * 8192)
     log("add 8192^2: %.4f ms, %.0f GB/s" % (elt["ms"], elt["gbs"]))
-    return sgemm, elt
+    return elt
 
 
 ROTATE = 4  # buffer sets an HBM-bound operator cycles through, so that no pass finds its
@@ -229,12 +260,13 @@ ROTATE = 4  # buffer sets an HBM-bound operator cycles through, so that no pass 
 
 
 def rotating(dev, make_call, sets):
-    """Average ms per call of an operator that takes the next of `sets` on every call."""
+    """ms per call of an operator that takes the next of `sets` on every call: the median of
+    five batches, each two rounds through the sets."""
     import itertools
     count = itertools.count()
     calls = [make_call(*s) for s in sets]
-    return dev.time_ms(lambda: calls[next(count) % len(calls)](), iters=6 * len(calls),
-                       warmup=2 * len(calls))
+    return dev.time_ms(lambda: calls[next(count) % len(calls)](), iters=2 * len(calls),
+                       warmup=2 * len(calls), reps=5)
 
 
 def bandwidth_table(L, dev, rng, ne):
@@ -277,7 +309,7 @@ def bandwidth_table(L, dev, rng, ne):
     table = []
     for name, bpe, make in ops:
         ms = rotating(dev, make, sets)
-        ms_one = dev.time_ms(make(*sets[0]), iters=10, warmup=3)
+        ms_one = dev.time_ms(make(*sets[0]), iters=6, warmup=3, reps=3)
         gbs = bpe * ne / (ms * 1e-3) / 1e9
         table.append({"op": name, "ms": round(ms, 4), "gbs": round(gbs, 1),
                       "frac": round(gbs / PEAK_HBM_GBS, 4),
@@ -299,10 +331,10 @@ def bandwidth_table(L, dev, rng, ne):
     for _ in range(2):
         px, py, pdy = dev.upload(host_p), dev.empty(nout), dev.empty(nout)
         o1, o2, o3, o4 = dev.empty(nin), dev.empty(nin), dev.empty(nin), dev.empty(nin)
-        L.mnv_fill(o4.p, nin, f(0.25), S)  # a top_diff of its own for the LRN gradient
-        L.mnv_fill(pdy.p, nout, f(0.5), S)
-        L.mnv_maxpool_fwd(px.p, py.p, *geo, S)
-        L.mnv_lrn_fwd(px.p, o1.p, o2.p, *lrn, S)  # o1 = scale, o2 = top for the backward row
+        capi_check(L.mnv_fill(o4.p, nin, f(0.25), S))  # a top_diff of its own for the LRN gradient
+        capi_check(L.mnv_fill(pdy.p, nout, f(0.5), S))
+        capi_check(L.mnv_maxpool_fwd(px.p, py.p, *geo, S))
+        capi_check(L.mnv_lrn_fwd(px.p, o1.p, o2.p, *lrn, S))  # o1 = scale, o2 = top (backward row)
         assert px.n == nin and o1.n == nin and py.n == nout and pdy.n == nout
         big.append((px, py, pdy, o1, o2, o3, o4))
     bias_ws = dev.empty(1 << 18)  # 1 MiB
@@ -362,11 +394,48 @@ def small_nets(steps=20, warmup=3):
     return out
 
 
-def cpu_baseline(batch=4):
-    """The CPU oracle's AlexNet step on a bounded sample (batch 4 instead of 256): naive
-    single-threaded loops; convolution and pooling have no reference CPU implementation,
-    so this is the repository's restatement ("port"), timed on one host core."""
+def host_cpu():
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count()
+    return {"model": model, "nproc": os.cpu_count(), "usable": usable}
+
+
+def _median_time(fn, reps=3):
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return float(np.median(ts))
+
+
+def cpu_baseline(batch=4, full=False):
+    """The CPU oracle (the repository's restatement of Minerva's single-threaded basic
+    implementation; `kind` "port") on the host cores, one core per operator as the reference's
+    CpuDevice runs them:
+      value         one AlexNet-shaped train step at batch 4 of 256 (convolution and pooling
+                    have no reference CPU implementation: the oracle's naive loops);
+      config2       every operator of the 8192^2 bandwidth table at full size, median of 3;
+      sgemm         the reference's i,j,k loop order (basic.cpp:164-171): 1000x4096x256 and
+                    1024^3 at full size; for 4096x4096x256 and 256x9216x4096 a quarter / an
+                    eighth of the output columns (columns are independent and cost the same:
+                    full size = sample x 4 / x 8; --cpu-full runs them whole); 4096^3 is
+                    extrapolated from the 1024^3 rate; the four products run at the same time
+                    on four cores;
+      mlp / cnn     one train step at batch 256, median of 3."""
+    import concurrent.futures as cf
     from oracle import nets
+    from oracle import mnv_oracle as ora
     params, data, label = nets.make_inputs("alexnet", batch)
     t0 = time.perf_counter()
     nets.alexnet_step(params, data, label, 0.01, batch)
@@ -375,33 +444,85 @@ def cpu_baseline(batch=4):
     out = {"value": round(batch / dt, 4), "unit": "images/s", "cores": 1, "kind": "port",
            "sample": "one AlexNet-shaped train step at batch %d (of 256) with the naive "
                      "single-threaded CPU oracle, %.1f s" % (batch, dt),
-           "host_cpus": os.cpu_count()}
-    # the same single-threaded restatement on the other parts of the metric (one run each,
-    # output allocation included): what the reference's CPU device would spend per operator
-    from oracle import mnv_oracle as ora
+           "host": host_cpu()}
+    del params, data, label
     rng = np.random.default_rng(11)
-    ne = 8192 * 8192
+    m = n = 8192
+    ne = m * n
     x, y = rng.standard_normal(ne, dtype=np.float32), rng.standard_normal(ne, dtype=np.float32)
-    others = {}
+    row, col = rng.standard_normal(n, dtype=np.float32), rng.standard_normal(m, dtype=np.float32)
+    relu = ora.activation_fwd(ora.RELU, x)
+    sm = ora.softmax_instance_fwd(x, n, m, 1, 1)
+    ops = [
+        ("add", 12, lambda: ora.arithmetic(ora.ADD, x, y)),
+        ("mul", 12, lambda: ora.arithmetic(ora.MUL, x, y)),
+        ("sub", 12, lambda: ora.arithmetic(ora.SUB, x, y)),
+        ("scalar mul", 8, lambda: ora.arithmetic_const(ora.MUL, 1, 3.291, x)),
+        ("broadcast add {1,n}", 8, lambda: ora.norm_arithmetic(ora.ADD, x, [m, n], row, [0])),
+        ("broadcast add {m,1}", 8, lambda: ora.norm_arithmetic(ora.ADD, x, [m, n], col, [1])),
+        ("sigmoid fwd", 8, lambda: ora.activation_fwd(ora.SIGMOID, x)),
+        ("relu fwd", 8, lambda: ora.activation_fwd(ora.RELU, x)),
+        ("tanh fwd", 8, lambda: ora.activation_fwd(ora.TANH, x)),
+        ("sigmoid bwd", 12, lambda: ora.activation_bwd(ora.SIGMOID, y, sm, x)),
+        ("relu bwd", 12, lambda: ora.activation_bwd(ora.RELU, y, relu, x)),
+        ("tanh bwd", 12, lambda: ora.activation_bwd(ora.TANH, y, sm, x)),
+        ("sum dim 0", 4, lambda: ora.reduction(ora.SUM, x, [m, n], [0])),
+        ("sum dim 1", 4, lambda: ora.reduction(ora.SUM, x, [m, n], [1])),
+        ("max dim 0", 4, lambda: ora.reduction(ora.MAX, x, [m, n], [0])),
+        ("max dim 1", 4, lambda: ora.reduction(ora.MAX, x, [m, n], [1])),
+        ("maxindex dim 0", 4, lambda: ora.maxindex(x, [m, n], 0)),
+        ("softmax rows", 8, lambda: ora.softmax_instance_fwd(x, n, m, 1, 1)),
+        ("softmax rows bwd", 12, lambda: ora.softmax_instance_bwd(y, sm, n, m, 1, 1)),
+        ("transpose", 8, lambda: ora.transpose(x, m, n)),
+    ]
+    table = []
+    t_cfg2 = time.perf_counter()
+    for name, bpe, fn in ops:
+        t = _median_time(fn, 3)
+        table.append({"op": name, "s": round(t, 4), "gbs": round(bpe * ne / t / 1e9, 2)})
+    log("cpu oracle config-2 table: %.1f s" % (time.perf_counter() - t_cfg2))
+    out["config2_8192x8192"] = {"reps": 3, "statistic": "median", "cores": 1,
+                                "note": "output allocation included, as in the reference's "
+                                        "CPU device (malloc per operator output)",
+                                "ops": table}
+    del x, y, relu, sm
 
-    def timed(name, fn, unit_work, unit):
+    # SGEMM in the reference's loop order; (m, k, n, columns computed)
+    jobs = [(1000, 4096, 256, 256), (1024, 1024, 1024, 1024),
+            (4096, 4096, 256, 256 if full else 64), (256, 9216, 4096, 4096 if full else 512)]
+
+    def gemm(job):
+        mm, kk, nn, cols = job
+        r = np.random.default_rng(mm + kk)
+        a = r.standard_normal(mm * kk, dtype=np.float32)
+        b = r.standard_normal(kk * cols, dtype=np.float32)
         t0 = time.perf_counter()
-        fn()
-        dt = time.perf_counter() - t0
-        others[name] = {"s": round(dt, 3), unit: round(unit_work / dt / 1e9, 3)}
+        ora.matmult(a, b, mm, cols, kk)
+        t = time.perf_counter() - t0
+        return {"MxKxN": "%dx%dx%d" % (mm, kk, nn), "columns_timed": cols,
+                "s_timed": round(t, 3), "s_full_size": round(t * nn / cols, 3),
+                "gflops": round(2.0 * mm * kk * cols / t / 1e9, 4)}
 
-    timed("add 8192x8192", lambda: ora.arithmetic(ora.ADD, x, y), 12.0 * ne, "gbs")
-    timed("sum dim 0 8192x8192", lambda: ora.reduction(ora.SUM, x, [8192, 8192], [0]), 4.0 * ne, "gbs")
-    a = rng.standard_normal(1000 * 4096, dtype=np.float32)
-    b = rng.standard_normal(4096 * 256, dtype=np.float32)
-    timed("sgemm 1000x4096x256", lambda: ora.matmult(a, b, 1000, 256, 4096), 2.0 * 1000 * 4096 * 256,
-          "gflops")
-    pm, dm, lm = nets.make_inputs("mlp", BATCH)
-    t0 = time.perf_counter()
-    nets.mlp_step(pm, dm, lm, 0.01, BATCH)
-    others["mlp step b256"] = {"s": round(time.perf_counter() - t0, 3)}
-    out["other_parts"] = others
+    t_g = time.perf_counter()
+    with cf.ThreadPoolExecutor(len(jobs)) as pool:  # the C loops run outside the GIL
+        gemms = list(pool.map(gemm, jobs))
+    log("cpu oracle sgemm shapes: %.1f s" % (time.perf_counter() - t_g))
+    rate = gemms[1]["gflops"]
+    out["sgemm"] = {"loop_order": "i, j outer, k inner (minerva/op/impl/basic.cpp:164-171), -O2, no BLAS",
+                    "cores": "1 per product, the 4 products at the same time",
+                    "shapes": gemms,
+                    "4096x4096x4096": {"extrapolated_from": "1024^3", "gflops": rate,
+                                       "s_full_size": round(2.0 * 4096 ** 3 / (rate * 1e9), 1)}}
+    steps = {}
+    for kind, fn in (("mlp", nets.mlp_step), ("cnn", nets.cnn_step)):
+        pm, dm, lm = nets.make_inputs(kind, BATCH)
+        t = _median_time(lambda: fn(dict(pm), dm, lm, 0.01, BATCH), 3)
+        steps[kind + "_b256"] = {"s_per_step": round(t, 4), "images_per_s": round(BATCH / t, 1)}
+    out["small_nets"] = steps
     return out
+
+
+SECTIONS = ("alexnet", "sgemm", "eltwise", "small", "owl", "cpu")
 
 
 def main():
@@ -410,50 +531,70 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--dataflow", action="store_true",
-                    help="also time the step with operators spread over four streams")
+    ap.add_argument("--cpu-full", action="store_true",
+                    help="CPU baseline: run the two larger SGEMM shapes whole (minutes)")
+    ap.add_argument("--no-dataflow", action="store_true",
+                    help="skip the run with operators spread over four streams (their kernels "
+                         "overlap, which disturbs per-kernel durations in a trace)")
+    ap.add_argument("--sections", default="all",
+                    help="comma-separated parts to run (for profiling one part): " + ",".join(SECTIONS))
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures the one-GPU operator path only: run with --gpus 1 "
                  "(nothing in this build uses a second GPU)")
+    want = set(SECTIONS) if args.sections == "all" else set(args.sections.split(","))
+    if want - set(SECTIONS):
+        sys.exit("unknown section(s): %s" % ", ".join(sorted(want - set(SECTIONS))))
+    if args.no_cpu:
+        want.discard("cpu")
     from minerva_amd import capi
     dev_info = capi.Device(0, own_stream=False).info()
     log("device:", dev_info)
-    res = alexnet_bench(args.steps, args.warmup, args.dataflow)
-    main_run = res["per_step_sync"]
-    roof = dominant_kernel_roofline(main_run["profile"], args.steps)
-    sgemm, elt = micro_bench()
     line = {
         "metric": "AlexNet-shape fp32 train images/s at b=256; SGEMM TFLOP/s; eltwise HBM GB/s",
-        "value": round(main_run["images_per_s"], 1),
-        "unit": "images/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(main_run["ms_per_step"], 3),
+        "value": None, "unit": "images/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "AlexNet-shaped single-group network (BASELINE.json configs[4]): "
                                "NCHW fp32, batch 256, 3x227x227 input, forward + backward + SGD, "
                                "one operator per launch, one stream sync per step",
-                   "global_batch": BATCH, "ops_per_step": main_run["ops_per_step"],
-                   "algorithmic_gflop_per_step": STEP_GFLOP},
-        "step_mfma_frac": round(STEP_GFLOP / main_run["ms_per_step"] / PEAK_FP32_MFMA_TFLOPS, 4),
-        "per_op_sync": {"images_per_s": round(res["per_op_sync"]["images_per_s"], 1),
-                        "ms_per_step": round(res["per_op_sync"]["ms_per_step"], 3)},
-        "graph_replay": main_run["graph_replay"],
-        "dataflow_4_streams": ({"images_per_s": round(res["dataflow"]["images_per_s"], 1),
-                                "ms_per_step": round(res["dataflow"]["ms_per_step"], 3)}
-                               if args.dataflow else None),
-        "owl_front_end": owl_front_end_bench(args.steps, args.warmup),
-        "h2d_batch_ms": round(main_run["h2d_batch_ms"], 2),
-        "roofline": roof,
-        "sgemm": sgemm,
-        "eltwise": elt,
-        "small_nets": small_nets(),
-        "top_ops": op_table(main_run["all_ops"], args.steps),
-        "device": dev_info,
-        "outputs_finite": main_run["finite"] and res["per_op_sync"]["finite"],
+                   "global_batch": BATCH, "algorithmic_gflop_per_step": STEP_GFLOP},
+        "timing": "value / ms_per_step: mean over exactly `steps` steps; kernels: median of 5 "
+                  "batches of back-to-back calls between two events on the kernels' stream",
+        "roofline": None, "cpu_baseline": None,
     }
-    line["cpu_baseline"] = None if args.no_cpu else cpu_baseline()
+    if "alexnet" in want:
+        res = alexnet_bench(args.steps, args.warmup, not args.no_dataflow)
+        main_run = res["per_step_sync"]
+        line.update({
+            "value": round(main_run["images_per_s"], 1),
+            "ms_per_step": round(main_run["ms_per_step"], 3),
+            "median_ms_per_step": round(main_run["median_ms_per_step"], 3),
+            "step_mfma_frac": round(STEP_GFLOP / main_run["ms_per_step"] / PEAK_FP32_MFMA_TFLOPS, 4),
+            "per_op_sync": {"images_per_s": round(res["per_op_sync"]["images_per_s"], 1),
+                            "ms_per_step": round(res["per_op_sync"]["ms_per_step"], 3)},
+            "graph_replay": main_run["graph_replay"],
+            "dataflow_4_streams": ({"images_per_s": round(res["dataflow"]["images_per_s"], 1),
+                                    "ms_per_step": round(res["dataflow"]["ms_per_step"], 3)}
+                                   if "dataflow" in res else None),
+            "h2d_batch_ms": round(main_run["h2d_batch_ms"], 2),
+            "roofline": dominant_kernel_roofline(main_run["profile"], args.steps),
+            "top_ops": op_table(main_run["all_ops"], args.steps),
+            "outputs_finite": main_run["finite"] and res["per_op_sync"]["finite"],
+        })
+        line["config"]["ops_per_step"] = main_run["ops_per_step"]
+    if "owl" in want:
+        line["owl_front_end"] = owl_front_end_bench(args.steps, args.warmup)
+    if "sgemm" in want:
+        line["sgemm"] = sgemm_bench()
+    if "eltwise" in want:
+        line["eltwise"] = eltwise_bench()
+    if "small" in want:
+        line["small_nets"] = small_nets()
+    line["device"] = dev_info
+    if "cpu" in want:
+        line["cpu_baseline"] = cpu_baseline(full=args.cpu_full)
     print(json.dumps(line))
 
 

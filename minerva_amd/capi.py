@@ -232,16 +232,25 @@ class Device:
         check(lib().mnv_event_elapsed_ms(e0, e1, ctypes.byref(ms)), "mnv_event_elapsed_ms")
         return ms.value
 
-    def time_ms(self, fn, iters=20, warmup=5):
-        """Average milliseconds per call of fn() measured with events on this stream."""
-        for _ in range(warmup):
-            fn()
+    def time_ms(self, fn, iters=20, warmup=5, reps=1):
+        """Milliseconds per call of fn(), measured with events on this stream: the median over
+        `reps` batches of `iters` back-to-back calls.  fn() returns the status of the call it
+        makes (or None); any non-zero status raises instead of being timed."""
+        def run(count):
+            for _ in range(count):
+                rc = fn()
+                if rc is not None:
+                    check(rc, "timed call")
+        run(warmup)
         e0, e1 = self.event(), self.event()
-        self.record(e0)
-        for _ in range(iters):
-            fn()
-        self.record(e1)
-        ms = self.elapsed_ms(e0, e1) / iters
+        batches = []
+        for _ in range(max(reps, 1)):
+            self.record(e0)
+            run(iters)
+            self.record(e1)
+            batches.append(self.elapsed_ms(e0, e1) / iters)
         lib().mnv_event_destroy(e0)
         lib().mnv_event_destroy(e1)
-        return ms
+        batches.sort()
+        mid = len(batches) // 2
+        return batches[mid] if len(batches) % 2 else 0.5 * (batches[mid - 1] + batches[mid])
