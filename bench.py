@@ -68,12 +68,16 @@ def alexnet_bench(steps, warmup, dataflow=True):
     from minerva_amd import configs
     params, data, label = configs.make_inputs("alexnet", BATCH)
     out = {}
-    modes = [("per_step_sync", False), ("per_op_sync", True)]
+    # "fused": the same step with the opt-in fused operators (bit-identical results, fewer
+    # launches): reported beside `value`, which stays the operator-by-operator step
+    modes = [("per_step_sync", False), ("per_op_sync", True), ("fused", False)]
     if dataflow:  # kernels of different streams overlap: a kernel trace that wants undisturbed
         modes.append(("dataflow", False))  # durations runs with --no-dataflow
     for mode, sync_each in modes:
         rt = hostapi.Runtime(0, sync_each_op=sync_each, dataflow=(mode == "dataflow"))
         net = hostapi.Net(rt, "alexnet", BATCH)
+        if mode == "fused":
+            net.set_fused()
         for k, v in params.items():
             net.set_param(k, v)
         t_h2d = time.perf_counter()
@@ -575,6 +579,11 @@ def main():
             "per_op_sync": {"images_per_s": round(res["per_op_sync"]["images_per_s"], 1),
                             "ms_per_step": round(res["per_op_sync"]["ms_per_step"], 3)},
             "graph_replay": main_run["graph_replay"],
+            "fused_epilogues": {"images_per_s": round(res["fused"]["images_per_s"], 1),
+                                "ms_per_step": round(res["fused"]["ms_per_step"], 3),
+                                "ops_per_step": res["fused"]["ops_per_step"],
+                                "note": "opt-in fused operators, results bit-identical to the "
+                                        "operator-by-operator step"},
             "dataflow_4_streams": ({"images_per_s": round(res["dataflow"]["images_per_s"], 1),
                                     "ms_per_step": round(res["dataflow"]["ms_per_step"], 3)}
                                    if "dataflow" in res else None),

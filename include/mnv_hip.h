@@ -322,6 +322,49 @@ size_t mnv_select_workspace_bytes(int num_indices);
 int mnv_select(const float* src, float* dst, const int* indices_host, int num_indices, int rows,
                int cols, void* workspace, size_t workspace_bytes, mnv_stream_t stream);
 
+/* ---- fused epilogues: an opt-in fast path, never taken by the operators above.
+ * The reference launches a convolution and then a separate AddTensor for the bias
+ * (cuda_perform.cu:227-264), and its applications follow every convolution and inner
+ * product with a ReLU, every gradient with the ReLU gradient and finish with
+ * w -= lr/batch * g as a scalar multiply and a subtraction
+ * (owl/apps/imagenet_alexnet/alexnet.py:73-126, apps/mnist_common.h:185-197).  Each entry
+ * point below performs one such pair in the producing kernel's store and returns, bit for
+ * bit, what the two separate calls return (same IEEE operations in the same order):
+ *   mnv_conv_fwd_relu        = mnv_conv_fwd, then mnv_relu_fwd
+ *   mnv_conv_bwd_data_relu   = mnv_conv_bwd_data, then mnv_relu_bwd gated by `bottom`
+ *                              (the activations the convolution's input went through ReLU as)
+ *   mnv_maxpool_bwd_relu     = mnv_maxpool_bwd, then mnv_relu_bwd gated by `bottom`
+ *   mnv_sgemm_nn_bias        = mnv_sgemm_nn, then mnv_norm_add_row with bias{m}, then
+ *                              (relu != 0) mnv_relu_fwd
+ *   mnv_sgemm_nn_relu_bwd    = mnv_sgemm_nn, then mnv_relu_bwd gated by bottom{m,n}
+ *   mnv_sgd_update           = mnv_const_mul(g, scale), then mnv_sub(w, .): w_out = w - scale*g
+ * Workspaces are those of the unfused entry points (same *_workspace_bytes). ---- */
+int mnv_conv_fwd_relu(const float* bottom, const float* filter, const float* bias, float* top,
+                      int num_images, int bottom_num_channels, int top_num_channels,
+                      int bottom_height, int bottom_width, int pad_height, int pad_width,
+                      int stride_vertical, int stride_horizontal, int filter_height,
+                      int filter_width, void* workspace, size_t workspace_bytes,
+                      mnv_stream_t stream);
+int mnv_conv_bwd_data_relu(const float* top_diff, const float* filter, const float* bottom,
+                           float* bottom_diff, int num_images, int bottom_num_channels,
+                           int top_num_channels, int bottom_height, int bottom_width,
+                           int pad_height, int pad_width, int stride_vertical,
+                           int stride_horizontal, int filter_height, int filter_width,
+                           void* workspace, size_t workspace_bytes, mnv_stream_t stream);
+int mnv_maxpool_bwd_relu(const float* bottom, const float* top, const float* top_diff,
+                         float* bottom_diff, int num_images, int num_channels, int bottom_height,
+                         int bottom_width, int stride_vertical, int stride_horizontal,
+                         int window_height, int window_width, int pad_height, int pad_width,
+                         mnv_stream_t stream);
+int mnv_sgemm_nn_bias(const float* a, const float* b, const float* bias, float* c, int m, int n,
+                      int k, int relu, void* workspace, size_t workspace_bytes,
+                      mnv_stream_t stream);
+int mnv_sgemm_nn_relu_bwd(const float* a, const float* b, const float* bottom, float* c, int m,
+                          int n, int k, void* workspace, size_t workspace_bytes,
+                          mnv_stream_t stream);
+int mnv_sgd_update(const float* w, const float* g, float scale, float* w_out, size_t n,
+                   mnv_stream_t stream);
+
 /* ---- random tensors: CudaPerformRandn / CudaPerformRandBernoulli (cuda_perform.h:66-67).
  * The reference seeds cuRAND from the wall clock per call (cuda.cpp:601,606); here the seed
  * is an argument and the generator is counter based (Philox4x32-10): element block i/4

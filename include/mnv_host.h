@@ -85,6 +85,13 @@ int mnvh_runtime_profile_read(void* runtime, char* text_out, size_t capacity);
  *   "pooling_forward" [alg, h, w, sv, sh, ph, pw]      inputs: bottom
  *   "pooling_backward" [alg, h, w, sv, sh, ph, pw]     inputs: diff, top, bottom
  *   "fill" [val, d0, d1, ...]
+ * and the opt-in fused operators (minerva_amd/host/hip_fused_ops.h):
+ *   "conv_forward_relu" [ph, pw, sv, sh]          inputs: bottom, filter, bias
+ *   "conv_backward_data_relu" [ph, pw, sv, sh]    inputs: diff, bottom, filter
+ *   "pooling_backward_relu" [h, w, sv, sh, ph, pw]      inputs: diff, top, bottom
+ *   "matmult_bias" [relu]                         inputs: a, b, bias {m,1}
+ *   "matmult_relu_backward"                       inputs: a, b, bottom
+ *   "sgd_update" [scale]                          inputs: w, g
  * Enum values follow minerva/op/closure.h:8-24 and narray/convolution_info.h:19-57
  * (arithmetic 0 add 1 sub 2 mult 3 div; elewise 0 exp 1 ln 2 negative; reduction 0 sum
  * 1 max; softmax 0 instance 1 channel; activation 0 sigmoid 1 relu 2 tanh; pooling 0 max
@@ -126,6 +133,11 @@ int mnvh_net_param_info(void* net, int index, char* name_out /* >= 16 bytes */, 
 int mnvh_net_set_param(void* net, const char* name, const float* host, size_t floats);
 /* name: a parameter ("w0"...), "prob", or "g_<param>" (gradient of the last step) */
 int mnvh_net_read(void* net, const char* name, float* host_out, size_t floats);
+/* Opt-in fast path: the following steps use the fused operators (convolution + ReLU, data /
+ * pooling gradient + ReLU gradient, inner product + bias [+ ReLU], inner product + ReLU
+ * gradient, one-kernel SGD update) instead of the separate ones.  No counterpart in the
+ * reference; parameters, gradients and probabilities keep their bits. */
+int mnvh_net_set_fused(void* net, int on);
 /* For tests: the following steps of an "alexnet" network also keep their activations, read
  * with mnvh_net_read as "act1" ... "act10" (the outputs of conv1+relu, pool1, conv2+relu,
  * pool2, conv3..5+relu, pool5, fc6, fc7 after ReLU and dropout). */

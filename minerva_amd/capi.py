@@ -87,6 +87,12 @@ for _m in ("instance", "channel"):
 for _k in ("max", "avg"):
     PROTOTYPES["mnv_%spool_fwd" % _k] = [_P, _P] + [_I] * 10 + [_S]
     PROTOTYPES["mnv_%spool_bwd" % _k] = [_P, _P, _P, _P] + [_I] * 10 + [_S]
+PROTOTYPES["mnv_conv_fwd_relu"] = PROTOTYPES["mnv_conv_fwd"]
+PROTOTYPES["mnv_conv_bwd_data_relu"] = [_P, _P, _P, _P] + [_I] * 11 + [_P, c_sz, _S]
+PROTOTYPES["mnv_maxpool_bwd_relu"] = PROTOTYPES["mnv_maxpool_bwd"]
+PROTOTYPES["mnv_sgemm_nn_bias"] = [_P, _P, _P, _P, _I, _I, _I, _I, _P, c_sz, _S]
+PROTOTYPES["mnv_sgemm_nn_relu_bwd"] = [_P, _P, _P, _P, _I, _I, _I, _P, c_sz, _S]
+PROTOTYPES["mnv_sgd_update"] = [_P, _P, c_f, _P, c_sz, _S]
 PROTOTYPES["mnv_copy_2d"] = [_P, _P, c_sz, c_sz, c_sz, c_sz, _S]
 PROTOTYPES["mnv_select_workspace_bytes"] = [_I]
 PROTOTYPES["mnv_select"] = [_P, _P, _P, _I, _I, _I, _P, c_sz, _S]

@@ -49,6 +49,7 @@ struct ConvFwd {
   float* __restrict__ top;
   ConvGeom g;
   int M, N, K, total_slabs, spp;  // GEMM extents: N*Ho*Wo, Kout, C*R*S
+  int relu;                       // fused epilogue: top = max(conv + bias, 0)
   struct Res {
     mnv_rsrc a, b;
   };
@@ -122,10 +123,14 @@ struct ConvFwd {
                          int, float (&v)[4]) const {
     mnv_fetch_vec<B_NOFF>(r.b, off, FAST ? (unsigned)s * 64u : 0u, v);
   }
+  // The fused ReLU is the selection mnv_relu_fwd makes on the stored value, so the result has
+  // the bits of the two-operator sequence.
   __device__ void c_store(int m, int n, float x) const {
     int img = mnv_fastdiv(m, g.d_HoWo);
     int pos = m - img * g.HoWo;
-    top[((size_t)img * N + n) * g.HoWo + pos] = x + bias[n];
+    float v = x + bias[n];
+    if (relu) v = v > 0.f ? v : 0.f;
+    top[((size_t)img * N + n) * g.HoWo + pos] = v;
   }
 };
 
@@ -150,6 +155,7 @@ struct ConvFwdNP {
   float* __restrict__ top;
   ConvGeom g;
   int M, N, K, total_slabs, spp;  // GEMM extents: N*Ho*Wo, Kout, C*R*S
+  int relu;                       // fused epilogue: top = max(conv + bias, 0)
   struct Res {
     mnv_rsrc a, b;
     const unsigned* tab;  // LDS: [total_slabs*16] byte offsets, MNV_OOB past K
@@ -214,7 +220,9 @@ struct ConvFwdNP {
   __device__ void c_store(int m, int n, float x) const {
     int img = mnv_fastdiv(m, g.d_HoWo);
     int pos = m - img * g.HoWo;
-    top[((size_t)img * N + n) * g.HoWo + pos] = x + bias[n];
+    float v = x + bias[n];
+    if (relu) v = v > 0.f ? v : 0.f;
+    top[((size_t)img * N + n) * g.HoWo + pos] = v;
   }
 };
 
@@ -230,6 +238,9 @@ struct ConvBwdData {
   float* __restrict__ bottom_diff;
   ConvGeom g;
   int M, N, K, total_slabs, spp;  // N*H*W, C, Kout*R*S
+  // fused epilogue (or null): the activations the bottom tensor went through a ReLU with;
+  // bottom_diff = gate > 0 ? gradient : 0, the selection mnv_relu_bwd makes
+  const float* __restrict__ gate;
   struct Res {
     mnv_rsrc a, b;
   };
@@ -317,7 +328,9 @@ struct ConvBwdData {
   __device__ void c_store(int m, int n, float x) const {
     int img = mnv_fastdiv(m, g.d_HW);
     int pos = m - img * g.HW;
-    bottom_diff[((size_t)img * N + n) * g.HW + pos] = x;
+    const size_t at = ((size_t)img * N + n) * g.HW + pos;
+    if (gate) x = gate[at] > 0.f ? x : 0.f;
+    bottom_diff[at] = x;
   }
 };
 
@@ -680,9 +693,10 @@ size_t mnv_conv_fwd_workspace_bytes(int N, int C, int K, int H, int W, int ph, i
   return splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
 }
 
-int mnv_conv_fwd(const float* bottom, const float* filter, const float* bias, float* top, int N,
-                 int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S,
-                 void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
+static int conv_fwd_impl(const float* bottom, const float* filter, const float* bias, float* top,
+                         int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R,
+                         int S, void* workspace, size_t workspace_bytes, mnv_stream_t stream,
+                         int relu) {
   ConvGeom g;
   if (!bottom || !filter || !bias || !top) return MNV_ERR_INVALID;
   int rc = make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S);
@@ -705,15 +719,29 @@ int mnv_conv_fwd(const float* bottom, const float* filter, const float* bias, fl
     float* wp = static_cast<float*>(workspace);
     rc = permute_filter(filter, wp, K, C, g.RS, false, s);
     if (rc) return rc;
-    ConvFwd<true> p{bottom, wp, bias, top, g, gm, gn, gk, g.RS * (C / 16), C / 16};
+    ConvFwd<true> p{bottom, wp, bias, top, g, gm, gn, gk, g.RS * (C / 16), C / 16, relu};
     return launch_tile(tile, p, splits, part, s);
   }
   if (np) {
-    ConvFwdNP p{bottom, filter, bias, top, g, gm, gn, gk, (gk + 15) / 16, gk >= 16 ? gk / 16 : 1};
+    ConvFwdNP p{bottom, filter, bias, top, g, gm, gn, gk, (gk + 15) / 16, gk >= 16 ? gk / 16 : 1, relu};
     return launch_tile(tile, p, splits, part, s);
   }
-  ConvFwd<false> p{bottom, filter, bias, top, g, gm, gn, gk, (gk + 15) / 16, 1};
+  ConvFwd<false> p{bottom, filter, bias, top, g, gm, gn, gk, (gk + 15) / 16, 1, relu};
   return launch_tile(tile, p, splits, part, s);
+}
+
+int mnv_conv_fwd(const float* bottom, const float* filter, const float* bias, float* top, int N,
+                 int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S,
+                 void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
+  return conv_fwd_impl(bottom, filter, bias, top, N, C, K, H, W, ph, pw, sv, sh, R, S, workspace,
+                       workspace_bytes, stream, 0);
+}
+
+int mnv_conv_fwd_relu(const float* bottom, const float* filter, const float* bias, float* top,
+                      int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R,
+                      int S, void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
+  return conv_fwd_impl(bottom, filter, bias, top, N, C, K, H, W, ph, pw, sv, sh, R, S, workspace,
+                       workspace_bytes, stream, 1);
 }
 
 size_t mnv_conv_bwd_data_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw,
@@ -726,9 +754,10 @@ size_t mnv_conv_bwd_data_workspace_bytes(int N, int C, int K, int H, int W, int 
   return splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
 }
 
-int mnv_conv_bwd_data(const float* top_diff, const float* filter, float* bottom_diff, int N,
-                      int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S,
-                      void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
+static int conv_bwd_data_impl(const float* top_diff, const float* filter, const float* gate,
+                              float* bottom_diff, int N, int C, int K, int H, int W, int ph,
+                              int pw, int sv, int sh, int R, int S, void* workspace,
+                              size_t workspace_bytes, mnv_stream_t stream) {
   ConvGeom g;
   if (!top_diff || !filter || !bottom_diff) return MNV_ERR_INVALID;
   int rc = make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S);
@@ -746,11 +775,27 @@ int mnv_conv_bwd_data(const float* top_diff, const float* filter, float* bottom_
     float* wq = static_cast<float*>(workspace);
     rc = permute_filter(filter, wq, K, C, g.RS, true, s);
     if (rc) return rc;
-    ConvBwdData<true> p{top_diff, wq, bottom_diff, g, gm, gn, gk, g.RS * (K / 16), K / 16};
+    ConvBwdData<true> p{top_diff, wq, bottom_diff, g, gm, gn, gk, g.RS * (K / 16), K / 16, gate};
     return launch_tile(tile, p, splits, part, s);
   }
-  ConvBwdData<false> p{top_diff, filter, bottom_diff, g, gm, gn, gk, (gk + 15) / 16, 1};
+  ConvBwdData<false> p{top_diff, filter, bottom_diff, g, gm, gn, gk, (gk + 15) / 16, 1, gate};
   return launch_tile(tile, p, splits, part, s);
+}
+
+int mnv_conv_bwd_data(const float* top_diff, const float* filter, float* bottom_diff, int N,
+                      int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S,
+                      void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
+  return conv_bwd_data_impl(top_diff, filter, nullptr, bottom_diff, N, C, K, H, W, ph, pw, sv, sh,
+                            R, S, workspace, workspace_bytes, stream);
+}
+
+int mnv_conv_bwd_data_relu(const float* top_diff, const float* filter, const float* bottom,
+                           float* bottom_diff, int N, int C, int K, int H, int W, int ph, int pw,
+                           int sv, int sh, int R, int S, void* workspace, size_t workspace_bytes,
+                           mnv_stream_t stream) {
+  if (!bottom) return MNV_ERR_INVALID;
+  return conv_bwd_data_impl(top_diff, filter, bottom, bottom_diff, N, C, K, H, W, ph, pw, sv, sh,
+                            R, S, workspace, workspace_bytes, stream);
 }
 
 size_t mnv_conv_bwd_filter_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw,

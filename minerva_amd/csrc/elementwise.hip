@@ -54,6 +54,16 @@ struct OpTanhBwd {
   __device__ float operator()(float y, float dy) const { return dy * (1.0f - y * y); }
 };
 
+// (w, g) -> w - v*g: the product is rounded, then the difference, as the scalar multiply
+// followed by the subtraction round (the library is built without contraction into fma)
+struct OpSgd {
+  float v;
+  __device__ float operator()(float w, float g) const {
+    const float step = g * v;
+    return w - step;
+  }
+};
+
 }  // namespace
 
 extern "C" {
@@ -108,6 +118,11 @@ int mnv_copy(const float* in, float* out, size_t n, mnv_stream_t s) {
 }
 int mnv_fill(float* dst, size_t n, float v, mnv_stream_t s) {
   return mnv_stream_launch<OpFill, 0>(nullptr, nullptr, dst, n, OpFill{v}, s);
+}
+
+int mnv_sgd_update(const float* w, const float* g, float scale, float* w_out, size_t n,
+                   mnv_stream_t s) {
+  return mnv_stream_launch<OpSgd, 2>(w, g, w_out, n, OpSgd{scale}, s);
 }
 
 int mnv_sigmoid_fwd(const float* bottom, float* top, size_t n, mnv_stream_t s) {

@@ -223,7 +223,7 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_fwd_lds_kernel(
 template <bool MAX, int KS, int ST, bool NT>
 __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_lds_kernel(
     const float* __restrict__ bottom, const float* __restrict__ top_diff,
-    float* __restrict__ bottom_diff, int planes, int ppb, PoolGeom g) {
+    float* __restrict__ bottom_diff, int planes, int ppb, PoolGeom g, int relu) {
   extern __shared__ float lds[];
   const int hw = g.H * g.W, howo = g.Ho * g.Wo;
   const size_t total_x = (size_t)planes * hw, total_d = (size_t)planes * howo;
@@ -312,6 +312,12 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_lds_kernel(
         const bool y0ok = (unsigned)y < (unsigned)g.H, y1ok = (unsigned)(y + 1) < (unsigned)g.H;
         const bool x0ok = (unsigned)x < (unsigned)g.W, x1ok = (unsigned)(x + 1) < (unsigned)g.W;
         const int po = m24(pl, hw);
+        if (MAX && relu) {  // lout lies over the plane data: a position's own value is still there
+          if (y0ok && x0ok) g00 = lout[po + p00] > 0.f ? g00 : 0.f;
+          if (y0ok && x1ok) g01 = lout[po + p01] > 0.f ? g01 : 0.f;
+          if (y1ok && x0ok) g10 = lout[po + p10] > 0.f ? g10 : 0.f;
+          if (y1ok && x1ok) g11 = lout[po + p11] > 0.f ? g11 : 0.f;
+        }
         if (y0ok && x0ok) lout[po + p00] = g00;
         if (y0ok && x1ok) lout[po + p01] = g01;
         if (y1ok && x0ok) lout[po + p10] = g10;
@@ -358,6 +364,7 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_lds_kernel(
               }
             }
         }
+        if (MAX && relu) acc = lout[q] > 0.f ? acc : 0.f;
         lout[q] = acc;
       }
     }
@@ -388,7 +395,7 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_lds_kernel(
 template <int KS, int ST, int XV, int DV, int WPT, bool NT>
 __global__ __launch_bounds__(MNV_POOL_THREADS, XV <= 4 ? 7 : 4) void mnv_maxpool_bwd_scatter_kernel(
     const float* __restrict__ bottom, const float* __restrict__ top_diff,
-    float* __restrict__ bottom_diff, int planes, int ppb, PoolGeom g) {
+    float* __restrict__ bottom_diff, int planes, int ppb, PoolGeom g, int relu) {
   extern __shared__ float lds[];
   const int hw = g.H * g.W, howo = g.Ho * g.Wo;
   const size_t total_x = (size_t)planes * hw, total_d = (size_t)planes * howo;
@@ -475,9 +482,17 @@ __global__ __launch_bounds__(MNV_POOL_THREADS, XV <= 4 ? 7 : 4) void mnv_maxpool
           }
         }
       }
+      // Fused ReLU gradient: a position receives gradients only from windows whose maximum
+      // it is, and the gate tests that same value, so a window whose maximum is not positive
+      // is dropped here and its position keeps the +0 it was cleared to -- what the gate
+      // would have selected.
 #pragma unroll
       for (int u = 0; u < 2; ++u)
-        if (q[u] < nwin) code[q[u]] = ((po[u] + arg[u]) << 2) | pass[u];
+        if (q[u] < nwin) {
+          int c = ((po[u] + arg[u]) << 2) | pass[u];
+          if (relu && !(lx[po[u] + arg[u]] > 0.f)) c = -1;
+          code[q[u]] = c;
+        }
     }
     __syncthreads();  // every window has read the plane data: the planes become the gradient
     // this thread's windows, read once for all passes (at most WPT of them)
@@ -540,7 +555,7 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_fwd_kernel(
 template <bool MAX>
 __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_kernel(
     const float* __restrict__ bottom, const float* __restrict__ top_diff,
-    float* __restrict__ bottom_diff, size_t planes, PoolGeom g) {
+    float* __restrict__ bottom_diff, size_t planes, PoolGeom g, int relu) {
   const size_t per_plane = (size_t)g.H * g.W;
   const size_t total = planes * per_plane;
   for (size_t q = (size_t)blockIdx.x * MNV_POOL_THREADS + threadIdx.x; q < total;
@@ -577,6 +592,7 @@ __global__ __launch_bounds__(MNV_POOL_THREADS) void mnv_pool_bwd_kernel(
           acc += dt[i * g.Wo + j] / (float)(g.kh * g.kw);
         }
       }
+    if (MAX && relu) acc = b[pos] > 0.f ? acc : 0.f;
     bottom_diff[q] = acc;
   }
 }
@@ -674,7 +690,8 @@ int pool_fwd(const float* bottom, float* top, int n, int c, int h, int w, int sv
 
 template <bool MAX>
 int pool_bwd(const float* bottom, const float* top_diff, float* bottom_diff, int n, int c, int h,
-             int w, int sv, int sh, int kh, int kw, int ph, int pw, mnv_stream_t stream) {
+             int w, int sv, int sh, int kh, int kw, int ph, int pw, mnv_stream_t stream,
+             int relu = 0) {
   PoolGeom g;
   if (!bottom || !top_diff || !bottom_diff) return MNV_ERR_INVALID;
   int rc = make_geom(&g, n, c, h, w, sv, sh, kh, kw, ph, pw);
@@ -710,7 +727,8 @@ int pool_bwd(const float* bottom, const float* top_diff, float* bottom_diff, int
                                : (nt ? mnv_maxpool_bwd_scatter_kernel<2, 2, 8, 4, 8, true>
                                      : mnv_maxpool_bwd_scatter_kernel<2, 2, 8, 4, 8, false>));
       hipLaunchKernelGGL(kernel, dim3(lds_grid(groups, lds)), dim3(MNV_POOL_THREADS), lds,
-                         mnv_stream(stream), bottom, top_diff, bottom_diff, (int)planes, spb, g);
+                         mnv_stream(stream), bottom, top_diff, bottom_diff, (int)planes, spb, g,
+                         relu);
       return MNV_LAUNCH_STATUS();
     }
   }
@@ -728,11 +746,11 @@ int pool_bwd(const float* bottom, const float* top_diff, float* bottom_diff, int
                       ? (nt ? mnv_pool_bwd_lds_kernel<MAX, 2, 2, true> : mnv_pool_bwd_lds_kernel<MAX, 2, 2, false>)
                       : (nt ? mnv_pool_bwd_lds_kernel<MAX, 0, 0, true> : mnv_pool_bwd_lds_kernel<MAX, 0, 0, false>);
     hipLaunchKernelGGL(kernel, dim3(lds_grid(groups, lds)), dim3(MNV_POOL_THREADS), lds,
-                       mnv_stream(stream), bottom, top_diff, bottom_diff, (int)planes, ppb, g);
+                       mnv_stream(stream), bottom, top_diff, bottom_diff, (int)planes, ppb, g, relu);
   } else {
     hipLaunchKernelGGL((mnv_pool_bwd_kernel<MAX>), dim3(pool_grid((size_t)planes * h * w)),
                        dim3(MNV_POOL_THREADS), 0, mnv_stream(stream), bottom, top_diff,
-                       bottom_diff, (size_t)planes, g);
+                       bottom_diff, (size_t)planes, g, relu);
   }
   return MNV_LAUNCH_STATUS();
 }
@@ -761,6 +779,12 @@ int mnv_maxpool_bwd(const float* bottom, const float* top, const float* top_diff
                     int kw, int ph, int pw, mnv_stream_t s) {
   (void)top;  // the first-maximum rule is evaluated on bottom itself
   return pool_bwd<true>(bottom, top_diff, bottom_diff, n, c, h, w, sv, sh, kh, kw, ph, pw, s);
+}
+int mnv_maxpool_bwd_relu(const float* bottom, const float* top, const float* top_diff,
+                         float* bottom_diff, int n, int c, int h, int w, int sv, int sh, int kh,
+                         int kw, int ph, int pw, mnv_stream_t s) {
+  (void)top;
+  return pool_bwd<true>(bottom, top_diff, bottom_diff, n, c, h, w, sv, sh, kh, kw, ph, pw, s, 1);
 }
 int mnv_avgpool_bwd(const float* bottom, const float* top, const float* top_diff,
                     float* bottom_diff, int n, int c, int h, int w, int sv, int sh, int kh,

@@ -27,6 +27,13 @@ struct SgemmNN {
   const float* __restrict__ B;
   float* __restrict__ C;
   int M, N, K, total_slabs, spp, bk;
+  // Fused epilogues (all off for the plain product), applied in this order to the value
+  // stored, each the single operation the separate operator performs:
+  //   bias: + bias[m] (the broadcast add of an {m,1} vector); relu: max(., 0);
+  //   gate: gate[m,n] > 0 ? . : 0 (the ReLU gradient's selection)
+  const float* __restrict__ bias;
+  const float* __restrict__ gate;
+  int relu;
   struct Res {
     mnv_rsrc a, b;
   };
@@ -67,13 +74,27 @@ struct SgemmNN {
     total_slabs = (K + b - 1) / b;
   }
   __device__ void block_init(Res&, float*, int, int) const {}
-  __device__ void c_store(int m, int n, float x) const { C[(size_t)n * M + m] = x; }
+  __device__ void c_store(int m, int n, float x) const {
+    const size_t at = (size_t)n * M + m;
+    if (bias) x = x + bias[m];
+    if (relu) x = x > 0.f ? x : 0.f;
+    if (gate) x = gate[at] > 0.f ? x : 0.f;
+    C[at] = x;
+  }
+};
+
+struct SgemmEpilogue {
+  const float* bias;
+  const float* gate;
+  int relu;
 };
 
 template <bool VEC>
-SgemmNN<VEC> make_sgemm(const float* a, const float* b, float* c, int m, int n, int k) {
+SgemmNN<VEC> make_sgemm(const float* a, const float* b, float* c, int m, int n, int k,
+                        const SgemmEpilogue& e) {
   SgemmNN<VEC> p;
   p.A = a; p.B = b; p.C = c; p.M = m; p.N = n; p.K = k;
+  p.bias = e.bias; p.gate = e.gate; p.relu = e.relu;
   p.set_bk(16);
   return p;
 }
@@ -140,17 +161,18 @@ int scratch_address(float** out) {
 }
 
 int sgemm_nn_impl(const float* a, const float* b, float* c, int m, int n, int k, void* workspace,
-                  size_t workspace_bytes, hipStream_t s) {
+                  size_t workspace_bytes, hipStream_t s,
+                  const SgemmEpilogue& e = SgemmEpilogue{nullptr, nullptr, 0}) {
   bool vec = (m % 4 == 0) && (k % 4 == 0) && mnv_aligned16(a) && mnv_aligned16(b);
   const SgemmPlan plan = plan_sgemm(m, n, k, workspace ? workspace_bytes / sizeof(float) : 0);
   const bool small = plan.small;
   const int splits = plan.splits;
   if (vec) {
-    SgemmNN<true> p = make_sgemm<true>(a, b, c, m, n, k);
+    SgemmNN<true> p = make_sgemm<true>(a, b, c, m, n, k, e);
     return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
                  : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
   }
-  SgemmNN<false> p = make_sgemm<false>(a, b, c, m, n, k);
+  SgemmNN<false> p = make_sgemm<false>(a, b, c, m, n, k, e);
   return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
                : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
 }
@@ -172,6 +194,26 @@ int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k, 
   // operands are addressed through 32-bit buffer offsets: at most 2^31 - 1 bytes each
   if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
   return sgemm_nn_impl(a, b, c, m, n, k, workspace, workspace_bytes, mnv_stream(stream));
+}
+
+int mnv_sgemm_nn_bias(const float* a, const float* b, const float* bias, float* c, int m, int n,
+                      int k, int relu, void* workspace, size_t workspace_bytes,
+                      mnv_stream_t stream) {
+  if (m == 0 || n == 0) return MNV_OK;
+  if (!a || !b || !bias || !c || m < 0 || n < 0 || k <= 0) return MNV_ERR_INVALID;
+  if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
+  return sgemm_nn_impl(a, b, c, m, n, k, workspace, workspace_bytes, mnv_stream(stream),
+                       SgemmEpilogue{bias, nullptr, relu != 0});
+}
+
+int mnv_sgemm_nn_relu_bwd(const float* a, const float* b, const float* bottom, float* c, int m,
+                          int n, int k, void* workspace, size_t workspace_bytes,
+                          mnv_stream_t stream) {
+  if (m == 0 || n == 0) return MNV_OK;
+  if (!a || !b || !bottom || !c || m < 0 || n < 0 || k <= 0) return MNV_ERR_INVALID;
+  if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
+  return sgemm_nn_impl(a, b, c, m, n, k, workspace, workspace_bytes, mnv_stream(stream),
+                       SgemmEpilogue{nullptr, bottom, 0});
 }
 
 int mnv_sgemm_nn_static(const float* a, const float* b, float* c, int m, int n, int k,

@@ -154,6 +154,29 @@ Tensor RunNamedOp(Runner* rt, const std::string& op, const std::vector<Tensor>& 
   } else if (op == "pooling_backward") {
     need(3);
     r = rt->PoolingBackward(in[0], in[1], in[2], pool_info());
+  } else if (op == "conv_forward_relu") {
+    need(3);
+    r = rt->ConvForwardRelu(in[0], in[1], in[2], conv_info());
+  } else if (op == "conv_backward_data_relu") {  // inputs: diff, bottom, filter
+    need(3);
+    r = rt->ConvBackwardDataRelu(in[0], in[1], in[2], conv_info());
+  } else if (op == "pooling_backward_relu") {  // params: h, w, sv, sh, ph, pw (max pooling)
+    need(3);
+    r = rt->PoolingBackwardRelu(in[0], in[1], in[2],
+                                PoolingInfo(PoolingInfo::Algorithm::kMax, P(params, n_params, 0),
+                                            P(params, n_params, 1), P(params, n_params, 2),
+                                            P(params, n_params, 3), P(params, n_params, 4),
+                                            P(params, n_params, 5)));
+  } else if (op == "matmult_bias") {  // params: relu (0 / 1); inputs: a, b, bias {m,1}
+    need(3);
+    r = rt->MatMultBias(in[0], in[1], in[2], P(params, n_params, 0) != 0);
+  } else if (op == "matmult_relu_backward") {  // inputs: a, b, bottom
+    need(3);
+    r = rt->MatMultReluBackward(in[0], in[1], in[2]);
+  } else if (op == "sgd_update") {  // params: scale; inputs: w, g
+    need(2);
+    MNV_CHECK(n_params >= 1) << "sgd_update takes the scale";
+    r = rt->SgdUpdate(in[0], in[1], static_cast<float>(params[0]));
   } else if (op == "threshold_norm") {  // params: threshold
     need(1);
     MNV_CHECK(n_params >= 1) << "threshold_norm takes the threshold";
@@ -444,6 +467,14 @@ int mnvh_net_read(void* net, const char* name, float* host_out, size_t floats) {
     }
     MNV_CHECK_EQ(static_cast<size_t>(t->size.Prod()), floats) << "size of '" << name << "'";
     h->rt->Read(t, host_out);
+  });
+}
+
+int mnvh_net_set_fused(void* net, int on) {
+  return Guard([&] {
+    NetHandle* h = static_cast<NetHandle*>(net);
+    MNV_CHECK(!h->graph) << "release the recorded step before switching operator sets";
+    h->net->fused = on != 0;
   });
 }
 

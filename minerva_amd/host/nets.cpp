@@ -9,8 +9,41 @@ void Net::AddParam(const std::string& name, const Scale& size) {
 
 void Net::Sgd(const std::string& name, const Tensor& grad, float lr) {
   results["g_" + name] = grad;
-  Tensor step = rt->ArithmeticConst(grad, lr / static_cast<float>(batch_), ArithmeticType::kMult, 0);
+  const float scale = lr / static_cast<float>(batch_);
+  if (fused) {
+    params[name] = rt->SgdUpdate(params[name], grad, scale);
+    return;
+  }
+  Tensor step = rt->ArithmeticConst(grad, scale, ArithmeticType::kMult, 0);
   params[name] = rt->Sub(params[name], step);
+}
+
+Tensor Net::ConvRelu(const Tensor& x, const Tensor& w, const Tensor& b, ConvInfo info) {
+  if (fused) return rt->ConvForwardRelu(x, w, b, info);
+  return rt->ReluForward(rt->ConvForward(x, w, b, info));
+}
+
+Tensor Net::ConvBackwardDataRelu(const Tensor& diff, const Tensor& bottom, const Tensor& w,
+                                 ConvInfo info) {
+  if (fused) return rt->ConvBackwardDataRelu(diff, bottom, w, info);
+  return rt->ReluBackward(rt->ConvBackwardData(diff, bottom, w, info), bottom, bottom);
+}
+
+Tensor Net::PoolBackwardRelu(const Tensor& diff, const Tensor& top, const Tensor& bottom,
+                             PoolingInfo info) {
+  if (fused) return rt->PoolingBackwardRelu(diff, top, bottom, info);
+  return rt->ReluBackward(rt->PoolingBackward(diff, top, bottom, info), bottom, bottom);
+}
+
+Tensor Net::Fc(const Tensor& w, const Tensor& x, const Tensor& b, bool relu) {
+  if (fused) return rt->MatMultBias(w, x, b, relu);
+  Tensor y = rt->NormArithmetic(rt->MatMult(w, x), b, ArithmeticType::kAdd);
+  return relu ? rt->ReluForward(y) : y;
+}
+
+Tensor Net::MatMultReluBackward(const Tensor& a, const Tensor& b, const Tensor& act) {
+  if (fused) return rt->MatMultReluBackward(a, b, act);
+  return rt->ReluBackward(rt->MatMult(a, b), act, act);
 }
 
 // ------------------------------------------------------------------------- MLP
@@ -27,15 +60,15 @@ void MlpNet::Step(const Tensor& data, const Tensor& label, float lr) {
   Tensor& w0 = params["w0"]; Tensor& b0 = params["b0"];
   Tensor& w1 = params["w1"]; Tensor& b1 = params["b1"];
   // FF
-  Tensor a1 = rt->ReluForward(rt->NormArithmetic(rt->MatMult(w0, data), b0, ArithmeticType::kAdd));
-  Tensor a2 = rt->NormArithmetic(rt->MatMult(w1, a1), b1, ArithmeticType::kAdd);
+  Tensor a1 = Fc(w0, data, b0, true);
+  Tensor a2 = Fc(w1, a1, b1, false);
   Tensor a3 = rt->Reshape(
       rt->SoftmaxForward(rt->Reshape(a2, Scale{out_, 1, 1, batch_}), SoftmaxAlgorithm::kInstance),
       Scale{out_, batch_});
   results["prob"] = a3;
   // BP
   Tensor s2 = rt->Sub(a3, label);
-  Tensor s1 = rt->ReluBackward(rt->MatMult(rt->Trans(w1), s2), a1, a1);
+  Tensor s1 = MatMultReluBackward(rt->Trans(w1), s2, a1);
   Tensor gw0 = rt->MatMult(s1, rt->Trans(data));
   Tensor gb0 = rt->Sum(s1, 1);
   Tensor gw1 = rt->MatMult(s2, rt->Trans(a1));
@@ -62,26 +95,46 @@ CnnNet::CnnNet(Runner* r, int batch, int pad2, int pool2) : Net(r, batch) {
 void CnnNet::Step(const Tensor& data, const Tensor& label, float lr) {
   const int b = batch_;
   Tensor a0 = data;
-  Tensor a1 = rt->ConvForward(a0, params["w0"], params["b0"], conv_info[0]);
-  Tensor a2 = rt->ActivationForward(a1, ActivationAlgorithm::kRelu);
+  // fused: the pre-activations a1 / a4 are never stored, and the ReLU gradients below test
+  // the activations a2 / a5 instead (x > 0 exactly when relu(x) > 0)
+  Tensor a1, a2, a4, a5;
+  if (fused) {
+    a2 = rt->ConvForwardRelu(a0, params["w0"], params["b0"], conv_info[0]);
+  } else {
+    a1 = rt->ConvForward(a0, params["w0"], params["b0"], conv_info[0]);
+    a2 = rt->ActivationForward(a1, ActivationAlgorithm::kRelu);
+  }
   Tensor a3 = rt->PoolingForward(a2, pool_info[0]);
-  Tensor a4 = rt->ConvForward(a3, params["w1"], params["b1"], conv_info[1]);
-  Tensor a5 = rt->ActivationForward(a4, ActivationAlgorithm::kRelu);
+  if (fused) {
+    a5 = rt->ConvForwardRelu(a3, params["w1"], params["b1"], conv_info[1]);
+  } else {
+    a4 = rt->ConvForward(a3, params["w1"], params["b1"], conv_info[1]);
+    a5 = rt->ActivationForward(a4, ActivationAlgorithm::kRelu);
+  }
   Tensor a6 = rt->PoolingForward(a5, pool_info[1]);
   Tensor re6 = rt->Reshape(a6, Scale{a6->size.Prod() / b, b});
   MNV_CHECK_EQ(re6->size[0], 512) << "the classifier expects 512 features";
-  Tensor a7 = rt->NormArithmetic(rt->MatMult(params["w2"], re6), params["b2"], ArithmeticType::kAdd);
+  Tensor a7 = Fc(params["w2"], re6, params["b2"], false);
   Tensor a8 = rt->SoftmaxForward(rt->Reshape(a7, Scale{10, 1, 1, b}), SoftmaxAlgorithm::kInstance);
   results["prob"] = a8;
   // BP
   Tensor s8 = rt->Sub(a8, label);
   Tensor s7 = rt->Reshape(s8, Scale{10, b});
   Tensor s6 = rt->Reshape(rt->MatMult(rt->Trans(params["w2"]), s7), a6->size);
-  Tensor s5 = rt->PoolingBackward(s6, a6, a5, pool_info[1]);
-  Tensor s4 = rt->ActivationBackward(s5, a5, a4, ActivationAlgorithm::kRelu);
+  Tensor s4, s1;
+  if (fused) {
+    s4 = rt->PoolingBackwardRelu(s6, a6, a5, pool_info[1]);
+  } else {
+    Tensor s5 = rt->PoolingBackward(s6, a6, a5, pool_info[1]);
+    s4 = rt->ActivationBackward(s5, a5, a4, ActivationAlgorithm::kRelu);
+  }
   Tensor s3 = rt->ConvBackwardData(s4, a3, params["w1"], conv_info[1]);
-  Tensor s2 = rt->PoolingBackward(s3, a3, a2, pool_info[0]);
-  Tensor s1 = rt->ActivationBackward(s2, a2, a1, ActivationAlgorithm::kRelu);
+  if (fused) {
+    s1 = rt->PoolingBackwardRelu(s3, a3, a2, pool_info[0]);
+  } else {
+    Tensor s2 = rt->PoolingBackward(s3, a3, a2, pool_info[0]);
+    s1 = rt->ActivationBackward(s2, a2, a1, ActivationAlgorithm::kRelu);
+  }
   Tensor gw0 = rt->ConvBackwardFilter(s1, a0, params["w0"], conv_info[0]);
   Tensor gb0 = rt->ConvBackwardBias(s1);
   Tensor gw1 = rt->ConvBackwardFilter(s4, a3, params["w1"], conv_info[1]);
@@ -122,34 +175,31 @@ void AlexNet::Step(const Tensor& data, const Tensor& label, float lr) {
   const int n = batch_;
   auto W = [&](int i) -> Tensor& { return params["w" + std::to_string(i)]; };
   auto B = [&](int i) -> Tensor& { return params["b" + std::to_string(i)]; };
-  auto fc = [&](int i, const Tensor& x) {
-    return rt->NormArithmetic(rt->MatMult(W(i), x), B(i), ArithmeticType::kAdd);
-  };
   Tensor acts[12], sens[12];
   // FF
   acts[0] = data;
-  acts[1] = rt->ReluForward(rt->ConvForward(acts[0], W(0), B(0), convs[0]));   // conv1
+  acts[1] = ConvRelu(acts[0], W(0), B(0), convs[0]);   // conv1
   acts[2] = rt->PoolingForward(acts[1], poolings[0]);                           // pool1
-  acts[3] = rt->ReluForward(rt->ConvForward(acts[2], W(1), B(1), convs[1]));   // conv2
+  acts[3] = ConvRelu(acts[2], W(1), B(1), convs[1]);   // conv2
   acts[4] = rt->PoolingForward(acts[3], poolings[1]);                           // pool2
-  acts[5] = rt->ReluForward(rt->ConvForward(acts[4], W(2), B(2), convs[2]));   // conv3
-  acts[6] = rt->ReluForward(rt->ConvForward(acts[5], W(3), B(3), convs[3]));   // conv4
-  acts[7] = rt->ReluForward(rt->ConvForward(acts[6], W(4), B(4), convs[4]));   // conv5
+  acts[5] = ConvRelu(acts[4], W(2), B(2), convs[2]);   // conv3
+  acts[6] = ConvRelu(acts[5], W(3), B(3), convs[3]);   // conv4
+  acts[7] = ConvRelu(acts[6], W(4), B(4), convs[4]);   // conv5
   acts[8] = rt->PoolingForward(acts[7], poolings[2]);                           // pool5
   Tensor re8 = rt->Reshape(acts[8], Scale{acts[8]->size.Prod() / n, n});
   const bool drop = dropout_rate_ > 0.f;
   Tensor mask6, mask7;
-  acts[9] = rt->ReluForward(fc(5, re8));                                        // fc6
+  acts[9] = Fc(W(5), re8, B(5), true);                                        // fc6
   if (drop) {
     mask6 = rt->RandBernoulli(acts[9]->size, dropout_rate_);
     acts[9] = rt->Mult(acts[9], mask6);                                         // drop6
   }
-  acts[10] = rt->ReluForward(fc(6, acts[9]));                                   // fc7
+  acts[10] = Fc(W(6), acts[9], B(6), true);                                   // fc7
   if (drop) {
     mask7 = rt->RandBernoulli(acts[10]->size, dropout_rate_);
     acts[10] = rt->Mult(acts[10], mask7);                                       // drop7
   }
-  acts[11] = fc(7, acts[10]);                                                   // fc8
+  acts[11] = Fc(W(7), acts[10], B(7), false);                                                   // fc8
   Tensor out = rt->Reshape(
       rt->SoftmaxForward(rt->Reshape(acts[11], Scale{classes_, 1, 1, n}), SoftmaxAlgorithm::kInstance),
       Scale{classes_, n});
@@ -158,20 +208,23 @@ void AlexNet::Step(const Tensor& data, const Tensor& label, float lr) {
     for (int i = 1; i <= 10; ++i) results["act" + std::to_string(i)] = acts[i];
   // BP
   sens[11] = rt->Sub(out, label);
-  sens[10] = rt->MatMult(rt->Trans(W(7)), sens[11]);                            // fc8
-  if (drop) sens[10] = rt->Mult(sens[10], mask7);                               // drop7
-  sens[10] = rt->ReluBackward(sens[10], acts[10], acts[10]);                    // relu7
-  sens[9] = rt->MatMult(rt->Trans(W(6)), sens[10]);
-  if (drop) sens[9] = rt->Mult(sens[9], mask6);                                 // drop6
-  sens[9] = rt->ReluBackward(sens[9], acts[9], acts[9]);                        // relu6
+  if (drop) {
+    sens[10] = rt->Mult(rt->MatMult(rt->Trans(W(7)), sens[11]), mask7);         // fc8, drop7
+    sens[10] = rt->ReluBackward(sens[10], acts[10], acts[10]);                  // relu7
+    sens[9] = rt->Mult(rt->MatMult(rt->Trans(W(6)), sens[10]), mask6);          // fc7, drop6
+    sens[9] = rt->ReluBackward(sens[9], acts[9], acts[9]);                      // relu6
+  } else {
+    sens[10] = MatMultReluBackward(rt->Trans(W(7)), sens[11], acts[10]);        // fc8, relu7
+    sens[9] = MatMultReluBackward(rt->Trans(W(6)), sens[10], acts[9]);          // fc7, relu6
+  }
   sens[8] = rt->Reshape(rt->MatMult(rt->Trans(W(5)), sens[9]), acts[8]->size);
-  sens[7] = rt->ReluBackward(rt->PoolingBackward(sens[8], acts[8], acts[7], poolings[2]), acts[7], acts[7]);
-  sens[6] = rt->ReluBackward(rt->ConvBackwardData(sens[7], acts[6], W(4), convs[4]), acts[6], acts[6]);
-  sens[5] = rt->ReluBackward(rt->ConvBackwardData(sens[6], acts[5], W(3), convs[3]), acts[5], acts[5]);
+  sens[7] = PoolBackwardRelu(sens[8], acts[8], acts[7], poolings[2]);
+  sens[6] = ConvBackwardDataRelu(sens[7], acts[6], W(4), convs[4]);
+  sens[5] = ConvBackwardDataRelu(sens[6], acts[5], W(3), convs[3]);
   sens[4] = rt->ConvBackwardData(sens[5], acts[4], W(2), convs[2]);
-  sens[3] = rt->ReluBackward(rt->PoolingBackward(sens[4], acts[4], acts[3], poolings[1]), acts[3], acts[3]);
+  sens[3] = PoolBackwardRelu(sens[4], acts[4], acts[3], poolings[1]);
   sens[2] = rt->ConvBackwardData(sens[3], acts[2], W(1), convs[1]);
-  sens[1] = rt->ReluBackward(rt->PoolingBackward(sens[2], acts[2], acts[1], poolings[0]), acts[1], acts[1]);
+  sens[1] = PoolBackwardRelu(sens[2], acts[2], acts[1], poolings[0]);
   Tensor gw[8], gb[8];
   gw[7] = rt->MatMult(sens[11], rt->Trans(acts[10]));
   gw[6] = rt->MatMult(sens[10], rt->Trans(acts[9]));

@@ -5,7 +5,9 @@
 //   AlexNet-shaped network  owl/apps/imagenet_alexnet/alexnet.py:7-133 (no dropout / LRN,
 //                           single group), plain SGD w -= lr/batch * grad
 // One Step = forward + backward + parameter update, one operator at a time; nothing is
-// fused across operator boundaries.
+// fused across operator boundaries unless `fused` is set, which swaps every
+// (producer, ReLU / ReLU gradient / bias add) pair and the two-operator SGD update for the
+// fused operator that returns the same bits (hip_fused_ops.h).
 #pragma once
 #include <map>
 
@@ -31,11 +33,19 @@ class Net {
   // Tests only: the step also leaves its activations in `results` ("act1", "act2", ...),
   // which keeps their device blocks alive until the next step.
   bool keep_activations = false;
+  // Opt-in fast path: fused epilogues instead of separate ReLU / bias / update operators.
+  bool fused = false;
 
  protected:
   // w <- w - (lr / batch) * g : ArithmeticConst(mult, const on the left) + Arithmetic(sub)
   void Sgd(const std::string& name, const Tensor& grad, float lr);
   void AddParam(const std::string& name, const Scale& size);
+  // The operator pairs of the graphs, separate or fused according to `fused`.
+  Tensor ConvRelu(const Tensor& x, const Tensor& w, const Tensor& b, ConvInfo info);
+  Tensor ConvBackwardDataRelu(const Tensor& diff, const Tensor& bottom, const Tensor& w, ConvInfo info);
+  Tensor PoolBackwardRelu(const Tensor& diff, const Tensor& top, const Tensor& bottom, PoolingInfo info);
+  Tensor Fc(const Tensor& w, const Tensor& x, const Tensor& b, bool relu);
+  Tensor MatMultReluBackward(const Tensor& a, const Tensor& b, const Tensor& act);
   Runner* rt;
   int batch_;
 };

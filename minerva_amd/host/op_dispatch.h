@@ -6,6 +6,7 @@
 #pragma once
 #include <typeinfo>
 
+#include "hip_fused_ops.h"
 #include "hip_ops.h"
 #include "minerva_types.h"
 
@@ -72,6 +73,13 @@ MNV_INSTALL_COMPUTE_FN(IndexClosure, hip::Index)
 MNV_INSTALL_COMPUTE_FN(ConcatClosure, hip::Concat)
 MNV_INSTALL_COMPUTE_FN(SliceClosure, hip::Slice)
 MNV_INSTALL_COMPUTE_FN(SelectClosure, hip::Select)
+// the opt-in fused operators (hip_fused_ops.h): no counterpart in the reference's table
+MNV_INSTALL_COMPUTE_FN(ConvForwardReluClosure, hip::ConvForwardRelu)
+MNV_INSTALL_COMPUTE_FN(ConvBackwardDataReluClosure, hip::ConvBackwardDataRelu)
+MNV_INSTALL_COMPUTE_FN(PoolingBackwardReluClosure, hip::PoolingBackwardRelu)
+MNV_INSTALL_COMPUTE_FN(MatMultBiasClosure, hip::MatMultBias)
+MNV_INSTALL_COMPUTE_FN(MatMultReluBackwardClosure, hip::MatMultReluBackward)
+MNV_INSTALL_COMPUTE_FN(SgdUpdateClosure, hip::SgdUpdate)
 MNV_INSTALL_DATAGEN_FN(ArrayLoaderClosure, hip::ArrayLoader)
 MNV_INSTALL_DATAGEN_FN(FillClosure, hip::Fill)
 MNV_INSTALL_DATAGEN_FN(RandnClosure, hip::Randn)
@@ -130,6 +138,15 @@ MNV_SIMPLE_OP(IndexOp, ComputeFnWithClosure, IndexClosure, "index")
 MNV_SIMPLE_OP(ConcatOp, ComputeFnWithClosure, ConcatClosure, "Concat")
 MNV_SIMPLE_OP(SliceOp, ComputeFnWithClosure, SliceClosure, "Slice")
 MNV_SIMPLE_OP(SelectOp, ComputeFnWithClosure, SelectClosure, "select")
+MNV_SIMPLE_OP(PoolingBackwardReluOp, ComputeFnWithClosure, PoolingBackwardReluClosure,
+              "max pooling bp + relu bp")
+MNV_SIMPLE_OP(MatMultReluBackwardOp, ComputeFnWithClosure, MatMultReluBackwardClosure, "* + relu bp")
+MNV_SIMPLE_OP(SgdUpdateOp, ComputeFnWithClosure, SgdUpdateClosure, "sgd update")
+
+class MatMultBiasOp : public ComputeFnWithClosure<MatMultBiasClosure> {
+ public:
+  std::string Name() const override { return closure.relu ? "* + bias + relu" : "* + bias"; }
+};
 
 class FillOp : public PhyDataGenFnWithClosure<FillClosure> {
  public:
@@ -185,13 +202,16 @@ template <class Base, int kind> class ConvNamed : public Base {
     std::ostringstream ss;
     ss << "pad:" << this->closure.pad_height << "*" << this->closure.pad_width
        << " stride:" << this->closure.stride_vertical << "*" << this->closure.stride_horizontal
-       << (kind == 0 ? " conv ff" : kind == 1 ? " conv bp data" : " conv bp filter");
+       << (kind == 0 ? " conv ff" : kind == 1 ? " conv bp data" : kind == 2 ? " conv bp filter"
+           : kind == 3 ? " conv ff + relu" : " conv bp data + relu bp");
     return ss.str();
   }
 };
 typedef ConvNamed<ComputeFnWithClosure<ConvForwardClosure>, 0> ConvForwardOp;
 typedef ConvNamed<ComputeFnWithClosure<ConvBackwardDataClosure>, 1> ConvBackwardDataOp;
 typedef ConvNamed<ComputeFnWithClosure<ConvBackwardFilterClosure>, 2> ConvBackwardFilterOp;
+typedef ConvNamed<ComputeFnWithClosure<ConvForwardReluClosure>, 3> ConvForwardReluOp;
+typedef ConvNamed<ComputeFnWithClosure<ConvBackwardDataReluClosure>, 4> ConvBackwardDataReluOp;
 
 template <class Base, bool fwd> class SoftmaxNamed : public Base {
  public:

@@ -379,4 +379,64 @@ Tensor Runner::LRNBackward(const Tensor& bottom, const Tensor& top, const Tensor
   return Compute({bottom, top, scale, top_diff}, bottom->size, op);
 }
 
+// ---------------------------------------------------------------- fused operators
+
+Tensor Runner::ConvForwardRelu(const Tensor& src, const Tensor& filter, const Tensor& bias,
+                               ConvInfo info) {
+  MNV_CHECK_EQ(src->size.NumDims(), 4u);
+  MNV_CHECK_EQ(filter->size.NumDims(), 4u);
+  MNV_CHECK_EQ(src->size[2], filter->size[2]) << "#input channels mismatch";
+  MNV_CHECK_EQ(bias->size.NumDims(), 1u) << "bias dimension mismatch";
+  MNV_CHECK_EQ(bias->size[0], filter->size[3]) << "bias size mismatch";
+  Scale out{(src->size[0] + 2 * info.pad_width - filter->size[0]) / info.stride_horizontal + 1,
+            (src->size[1] + 2 * info.pad_height - filter->size[1]) / info.stride_vertical + 1,
+            filter->size[3], src->size[3]};
+  auto op = std::make_shared<ConvForwardReluOp>();
+  op->closure = {info.pad_height, info.pad_width, info.stride_vertical, info.stride_horizontal};
+  return Compute({src, filter, bias}, out, op);
+}
+
+Tensor Runner::ConvBackwardDataRelu(const Tensor& diff, const Tensor& bottom, const Tensor& filter,
+                                    ConvInfo info) {
+  MNV_CHECK_EQ(diff->size[2], filter->size[3]) << "#output channels mismatch";
+  auto op = std::make_shared<ConvBackwardDataReluOp>();
+  op->closure = {info.pad_height, info.pad_width, info.stride_vertical, info.stride_horizontal};
+  return Compute({diff, filter, bottom}, bottom->size, op);
+}
+
+Tensor Runner::PoolingBackwardRelu(const Tensor& diff, const Tensor& top, const Tensor& bottom,
+                                   PoolingInfo info) {
+  CheckSame(diff, top);
+  MNV_CHECK(info.algorithm == PoolingInfo::Algorithm::kMax) << "fused only for max pooling";
+  auto op = std::make_shared<PoolingBackwardReluOp>();
+  op->closure = {info.height, info.width, info.stride_vertical, info.stride_horizontal,
+                 info.pad_height, info.pad_width};
+  return Compute({diff, top, bottom}, bottom->size, op);
+}
+
+Tensor Runner::MatMultBias(const Tensor& a, const Tensor& b, const Tensor& bias, bool relu) {
+  MNV_CHECK_EQ(a->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(b->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(a->size[1], b->size[0]) << "size must match";
+  MNV_CHECK(bias->size == (Scale{a->size[0], 1})) << "bias must be {m,1}";
+  auto op = std::make_shared<MatMultBiasOp>();
+  op->closure = {relu};
+  return Compute({a, b, bias}, Scale{a->size[0], b->size[1]}, op);
+}
+
+Tensor Runner::MatMultReluBackward(const Tensor& a, const Tensor& b, const Tensor& bottom) {
+  MNV_CHECK_EQ(a->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(b->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(a->size[1], b->size[0]) << "size must match";
+  MNV_CHECK(bottom->size == (Scale{a->size[0], b->size[1]})) << "gate extent must match the product";
+  return Compute({a, b, bottom}, bottom->size, std::make_shared<MatMultReluBackwardOp>());
+}
+
+Tensor Runner::SgdUpdate(const Tensor& w, const Tensor& g, float scale) {
+  MNV_CHECK_EQ(w->size.Prod(), g->size.Prod()) << "parameter and gradient differ in size";
+  auto op = std::make_shared<SgdUpdateOp>();
+  op->closure = {scale};
+  return Compute({w, g}, w->size, op);
+}
+
 }  // namespace minerva

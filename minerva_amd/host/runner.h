@@ -116,6 +116,23 @@ class Runner : public DeviceListener {
   Tensor LRNBackward(const Tensor& bottom, const Tensor& top, const Tensor& scale,
                      const Tensor& top_diff, int local_size, float alpha, float beta);
 
+  // The opt-in fused operators (hip_fused_ops.h).  Each returns the bits of the pair of calls
+  // named in its comment.
+  // ReluForward(ConvForward(src, filter, bias, info))
+  Tensor ConvForwardRelu(const Tensor& src, const Tensor& filter, const Tensor& bias, ConvInfo info);
+  // ReluBackward(ConvBackwardData(diff, bottom, filter, info), bottom, bottom)
+  Tensor ConvBackwardDataRelu(const Tensor& diff, const Tensor& bottom, const Tensor& filter,
+                              ConvInfo info);
+  // ReluBackward(PoolingBackward(diff, top, bottom, info), bottom, bottom); max pooling only
+  Tensor PoolingBackwardRelu(const Tensor& diff, const Tensor& top, const Tensor& bottom,
+                             PoolingInfo info);
+  // [ReluForward](NormArithmetic(MatMult(a, b), bias{m,1}, add))
+  Tensor MatMultBias(const Tensor& a, const Tensor& b, const Tensor& bias, bool relu);
+  // ReluBackward(MatMult(a, b), bottom, bottom)
+  Tensor MatMultReluBackward(const Tensor& a, const Tensor& b, const Tensor& bottom);
+  // Sub(w, ArithmeticConst(g, scale, mult))
+  Tensor SgdUpdate(const Tensor& w, const Tensor& g, float scale);
+
  private:
   friend struct TensorNode;
   std::unique_ptr<HipDevice> device_;

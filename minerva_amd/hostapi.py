@@ -224,6 +224,10 @@ class Net:
                                          l.ctypes.data_as(fp), ctypes.c_size_t(l.size)),
                "net_load_batch")
 
+    def set_fused(self, on=True):
+        """Opt-in fast path: fused epilogues instead of separate ReLU / bias / update operators."""
+        _check(lib().mnvh_net_set_fused(self.h, 1 if on else 0), "net_set_fused")
+
     def keep_activations(self, on=True):
         """The following steps also keep "act1" ... "act10" readable (AlexNet only)."""
         _check(lib().mnvh_net_keep_activations(self.h, 1 if on else 0), "net_keep_activations")

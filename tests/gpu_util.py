@@ -74,12 +74,15 @@ def net_state(net, label_floats):
     return s
 
 
-def run_steps(kind, batch, variant, lr, params, batches, **runtime_args):
-    """One step per batch, operator by operator; the state after every step."""
+def run_steps(kind, batch, variant, lr, params, batches, fused=False, **runtime_args):
+    """One step per batch, operator by operator (fused: with the fused operators); the state
+    after every step."""
     from minerva_amd import hostapi
     runtime_args.setdefault("sync_each_op", False)
     r = hostapi.Runtime(0, **runtime_args)
     net = hostapi.Net(r, kind, batch, variant)
+    if fused:
+        net.set_fused()
     for k, v in params.items():
         net.set_param(k, v)
     states = []
@@ -87,6 +90,7 @@ def run_steps(kind, batch, variant, lr, params, batches, **runtime_args):
         net.load_batch(d, l)
         net.step(lr)
         states.append(net_state(net, l.size))
+    run_steps.ops_issued = r.ops_issued()  # of the run that just ended
     net.close()
     r.close()
     return states
