@@ -397,6 +397,9 @@ int mnvh_concurrent_adds(void* runtime, const float* a, const float* b, size_t n
     }
     for (int i = 0; i < count; ++i) dev.PushTask(&tasks[i]);
     dev.WaitForAllFinished();
+    // the host threads are done; in dataflow mode their kernels may still be in flight on
+    // the four streams, and the copies below run on stream 0
+    dev.Barrier(0);
     std::string err = dev.TakeAsyncError();
     for (int i = 0; i < count; ++i) {
       if (err.empty()) dev.CopyToHost(out + (size_t)i * n, base_id + i, n);

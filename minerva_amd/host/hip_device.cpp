@@ -254,7 +254,7 @@ void HipDevice::WorkerLoop(int thrid) {
       ++busy_;
     }
     try {
-      Execute(task, thrid);
+      Execute(task, thrid, true);
     } catch (const std::exception& e) {
       std::lock_guard<std::mutex> lck(err_mutex_);
       if (async_error_.empty()) async_error_ = e.what();
@@ -295,7 +295,7 @@ void HipDevice::EnsureStaging(int thrid) {
   Ok(mnv_host_malloc(&staging_[thrid], kStagingBytes), "pinned staging");
 }
 
-void HipDevice::Execute(Task* task, int thrid) {
+void HipDevice::Execute(Task* task, int thrid, bool pooled) {
   Activate();  // every task re-selects the device on its thread (device.cpp:201-203)
   DataList input_shards;
   for (auto& i : task->inputs) {
@@ -337,8 +337,27 @@ void HipDevice::Execute(Task* task, int thrid) {
     output_shards.emplace_back(ptr, o.physical_data.size);
   }
   MNV_CHECK(task->op.compute_fn) << "task without an operator";
-  DoExecute(input_shards, output_shards, task->op, thrid);
+  DoExecute(input_shards, output_shards, task->op, thrid, pooled);
   if (dataflow_) {
+    // an operator that fills one of its inputs (LRNForward's scale) is that datum's producer
+    // from now on: later readers on other streams must wait for this operator, not for the
+    // one that created the block
+    const int mutated = task->op.compute_fn->MutatedInput();
+    if (mutated >= 0 && mutated < static_cast<int>(task->inputs.size())) {
+      void* e = nullptr;
+      Ok(mnv_event_create_ordering(&e), "event create");
+      Ok(mnv_event_record(e, streams_[thrid]), "event record");
+      void* old = nullptr;
+      {
+        std::lock_guard<std::mutex> lck(local_mutex_);
+        auto& p = produced_[task->inputs[mutated].physical_data.data_id];
+        old = p.event;
+        p.event = e;
+        p.stream = thrid;
+        p.users |= 1u << thrid;
+      }
+      if (old) mnv_event_destroy(old);
+    }
     for (auto& o : task->outputs) {
       void* e = nullptr;
       Ok(mnv_event_create_ordering(&e), "event create");
@@ -350,7 +369,8 @@ void HipDevice::Execute(Task* task, int thrid) {
   if (listener_) listener_->OnOperationComplete(task);
 }
 
-void HipDevice::DoExecute(const DataList& in, const DataList& out, PhysicalOp& op, int thrid) {
+void HipDevice::DoExecute(const DataList& in, const DataList& out, PhysicalOp& op, int thrid,
+                          bool pooled) {
   EnsureWorkspace(thrid, kWorkspaceBytes);
   Context ctx;
   ctx.impl_type = ImplType::kHip;
@@ -379,7 +399,10 @@ void HipDevice::DoExecute(const DataList& in, const DataList& out, PhysicalOp& o
     std::lock_guard<std::mutex> lck(prof_mutex_);
     timed_.push_back(t);
   }
-  if (sync_each_op_ && !capturing_) {
+  // A task of the thread pool runs on whichever worker took it: outside dataflow mode nothing
+  // orders the four worker streams among themselves, so such a task is complete only once
+  // its stream has drained (what the reference does for every task, device.cpp:221).
+  if ((sync_each_op_ || (pooled && !dataflow_)) && !capturing_) {
     int rc = mnv_stream_sync(streams_[thrid]);
     MNV_CHECK(rc == MNV_OK) << op.compute_fn->Name() << ": " << mnv_error_string(rc);
   }
@@ -499,6 +522,7 @@ void HipDevice::CopyFromHost(uint64_t data_id, const float* src, size_t floats) 
 }
 
 void HipDevice::CopyOnDevice(uint64_t dst_id, uint64_t src_id, size_t floats) {
+  MNV_CHECK(!dataflow_) << "the in-order device copy is for the one-stream order, not dataflow mode";
   Activate();
   Ok(mnv_copy(data_store_->GetData(src_id), data_store_->GetData(dst_id), floats, streams_[0]),
      "device copy");

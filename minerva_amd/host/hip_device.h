@@ -4,8 +4,9 @@
 // engine calls: PushTask / GetPtr / FreeDataIfExist and DeviceListener::OnOperationComplete.
 //
 //  - kParallelism (4) worker threads, each with its own HIP stream and its own
-//    grow-only scratch arena; a task runs on worker `thrid` and is synchronised before
-//    completion is reported, as the reference does after every operator.
+//    grow-only scratch arena; a task of the pool runs on worker `thrid` and, unless the
+//    device is in dataflow mode, is synchronised before completion is reported, as the
+//    reference does after every operator.
 //  - PooledDataStore: exact-size free lists over mnv_malloc / mnv_free; when the bytes
 //    held exceed the threshold every cached block is released.
 //  - Three ways to order operators: synchronise after every one (the reference);
@@ -171,8 +172,9 @@ class HipDevice {
   void LaunchGraph(void* graph_exec);
 
  private:
-  void Execute(Task* task, int thrid);
-  void DoExecute(const DataList& in, const DataList& out, PhysicalOp& op, int thrid);
+  // pooled: the task came through the thread pool (not issued inline by the caller)
+  void Execute(Task* task, int thrid, bool pooled = false);
+  void DoExecute(const DataList& in, const DataList& out, PhysicalOp& op, int thrid, bool pooled);
   void Activate() const;
   void EnsureWorkspace(int thrid, size_t bytes);
   void EnsureStaging(int thrid);

@@ -17,6 +17,10 @@ class ComputeFn {
   virtual ~ComputeFn() {}
   virtual void Execute(const DataList&, const DataList&, const Context&) = 0;
   virtual std::string Name() const = 0;
+  // Index of an input the operator writes (LRNForward fills its `scale` input, as the
+  // reference does, cuda.cpp:45-59), or -1: a device that orders operators by data
+  // dependencies must treat the operator as that datum's latest producer.
+  virtual int MutatedInput() const { return -1; }
 };
 
 template <typename C> struct FnBundle;
@@ -131,7 +135,11 @@ MNV_SIMPLE_OP(ReluBackwardOp, ComputeFnWithClosure, ReluBackwardClosure, "relu b
 MNV_SIMPLE_OP(TanhForwardOp, ComputeFnWithClosure, TanhForwardClosure, "tanh forward")
 MNV_SIMPLE_OP(TanhBackwardOp, ComputeFnWithClosure, TanhBackwardClosure, "tanh backward")
 MNV_SIMPLE_OP(ConvBackwardBiasOp, ComputeFnWithClosure, ConvBackwardBiasClosure, "conv bp bias")
-MNV_SIMPLE_OP(LRNForwardOp, ComputeFnWithClosure, LRNForwardClosure, "LRN Forward")
+class LRNForwardOp : public ComputeFnWithClosure<LRNForwardClosure> {
+ public:
+  std::string Name() const override { return "LRN Forward"; }
+  int MutatedInput() const override { return 1; }
+};
 MNV_SIMPLE_OP(LRNBackwardOp, ComputeFnWithClosure, LRNBackwardClosure, "LRN Backward")
 MNV_SIMPLE_OP(ThresholdNormOp, ComputeFnWithClosure, ThresholdNormClosure, "threshold norm")
 MNV_SIMPLE_OP(IndexOp, ComputeFnWithClosure, IndexClosure, "index")

@@ -273,6 +273,22 @@ def test_four_stream_thread_pool(rt):
         assert_bits_equal(out[i], a + b, "concurrent add %d" % i)
 
 
+@pytest.mark.parametrize("mode", ["stream_order", "dataflow"])
+def test_thread_pool_tasks_without_per_operator_sync(mode):
+    """Tasks of the thread pool run on whichever worker stream takes them.  With the
+    per-operator synchronisation switched off they must still be complete (stream order:
+    each worker drains its stream; dataflow: the reader waits for all streams) before the
+    results are copied back on stream 0."""
+    from minerva_amd import hostapi
+    r = hostapi.Runtime(0, sync_each_op=False, dataflow=(mode == "dataflow"))
+    a, b = _rand(3000003, 82), _rand(3000003, 83)
+    for _ in range(3):
+        out = r.concurrent_adds(a, b, 16)
+        for i in range(16):
+            assert_bits_equal(out[i], a + b, "concurrent add %d (%s)" % (i, mode))
+    r.close()
+
+
 def _run_net(kind, batch, steps, sync_each_op, variant=0, lr=0.01, keep_acts=False):
     from minerva_amd import hostapi
     from oracle import nets
