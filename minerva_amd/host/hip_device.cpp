@@ -19,114 +19,10 @@ constexpr size_t kWorkspaceBytes = (size_t)128 << 20;
 constexpr size_t kStagingBytes = (size_t)16 << 20;
 }  // namespace
 
-// ---------------------------------------------------------------- PooledDataStore
-
-PooledDataStore::PooledDataStore(size_t threshold, std::function<void*(size_t)> a,
-                                 std::function<void(void*)> d)
-    : allocator_(std::move(a)), deallocator_(std::move(d)), threshold_(threshold) {}
-
-PooledDataStore::~PooledDataStore() {
-  for (auto& kv : data_states_) deallocator_(kv.second.ptr);
-  for (auto& kv : free_space_)
-    for (auto& b : kv.second) deallocator_(b.ptr);
-}
-
-float* PooledDataStore::CreateData(uint64_t id, size_t length, int stream, unsigned* foreign) {
-  std::lock_guard<std::mutex> lck(access_mutex_);
-  auto it = data_states_.emplace(id, DataState{nullptr, length});
-  MNV_CHECK(it.second) << "data already existed";
-  DataState& ds = it.first->second;
-  if (foreign) *foreign = 0;
-  auto hit = free_space_.find(length);
-  if (hit != free_space_.end()) {  // reuse a block of exactly this size
-    auto& blocks = hit->second;
-    size_t pick = 0;
-    bool found = stream < 0;
-    if (stream >= 0) {
-      // a block no other stream still works on needs no wait: stream order protects it
-      const unsigned mine = 1u << stream;
-      for (size_t i = 0; i < blocks.size(); ++i)
-        if ((blocks[i].users & ~mine) == 0) {
-          pick = i;
-          found = true;
-          break;
-        }
-      // Otherwise a new block is better than making this stream wait for the others (it
-      // would wait for everything queued on them, which serialises the streams); the pool
-      // grows by at most what is allocated between two synchronisations, after which
-      // every cached block is free of users again.  Past half the threshold, recycle.
-      if (!found && total_ + length > threshold_ / 2) {
-        found = true;
-        if (foreign) *foreign = blocks[0].users & ~mine;
-      }
-    }
-    if (!found) {
-      ds.ptr = allocator_(length);
-      total_ += length;
-      return static_cast<float*>(ds.ptr);
-    }
-    ds.ptr = blocks[pick].ptr;
-    blocks.erase(blocks.begin() + pick);
-    if (blocks.empty()) free_space_.erase(hit);
-  } else {
-    ds.ptr = allocator_(length);
-    total_ += length;
-    if (threshold_ < total_) ReleaseFreeSpace();
-  }
-  return static_cast<float*>(ds.ptr);
-}
-
-float* PooledDataStore::GetData(uint64_t id) {
-  std::lock_guard<std::mutex> lck(access_mutex_);
-  auto it = data_states_.find(id);
-  MNV_CHECK(it != data_states_.end()) << "data #" << id << " does not exist";
-  return static_cast<float*>(it->second.ptr);
-}
-
-bool PooledDataStore::ExistData(uint64_t id) const {
-  std::lock_guard<std::mutex> lck(access_mutex_);
-  return data_states_.count(id) != 0;
-}
-
-void PooledDataStore::FreeData(uint64_t id, unsigned users) {
-  std::lock_guard<std::mutex> lck(access_mutex_);
-  auto it = data_states_.find(id);
-  MNV_CHECK(it != data_states_.end()) << "data #" << id << " does not exist";
-  free_space_[it->second.length].push_back(FreeBlock{it->second.ptr, users});
-  data_states_.erase(it);
-}
-
-void PooledDataStore::ClearUsers() {
-  std::lock_guard<std::mutex> lck(access_mutex_);
-  for (auto& kv : free_space_)
-    for (auto& b : kv.second) b.users = 0;
-}
-
-size_t PooledDataStore::GetTotalBytes() const {
-  std::lock_guard<std::mutex> lck(access_mutex_);
-  return total_;
-}
-
-size_t PooledDataStore::NumCachedBlocks() const {
-  std::lock_guard<std::mutex> lck(access_mutex_);
-  size_t n = 0;
-  for (auto& kv : free_space_) n += kv.second.size();
-  return n;
-}
-
-void PooledDataStore::ReleaseFreeSpace() {
-  for (auto& kv : free_space_)
-    for (auto& b : kv.second) {
-      deallocator_(b.ptr);
-      total_ -= kv.first;
-    }
-  free_space_.clear();
-}
-
 // ---------------------------------------------------------------------- HipDevice
 
 HipDevice::HipDevice(uint64_t device_id, DeviceListener* listener, int gpu_id, size_t pool_bytes)
-    : device_id_(device_id), listener_(listener), gpu_id_(gpu_id) {
+    : ThreadedDevice(device_id, listener, kParallelism), gpu_id_(gpu_id) {
   Activate();
   for (size_t i = 0; i < kParallelism; ++i) Ok(mnv_stream_create(&streams_[i]), "stream create");
   auto allocator = [this](size_t len) -> void* {
@@ -144,18 +40,10 @@ HipDevice::HipDevice(uint64_t device_id, DeviceListener* listener, int gpu_id, s
     mnv_free(p);
   };
   data_store_.reset(new PooledDataStore(pool_bytes, allocator, deallocator));
-  for (size_t i = 0; i < kParallelism; ++i)
-    workers_.emplace_back(&HipDevice::WorkerLoop, this, static_cast<int>(i));
 }
 
 HipDevice::~HipDevice() {
-  WaitForAllFinished();
-  {
-    std::lock_guard<std::mutex> lck(q_mutex_);
-    stop_ = true;
-  }
-  q_cv_.notify_all();
-  for (auto& t : workers_) t.join();
+  StopWorkers();  // before the streams they launch on go away
   Activate();
   for (size_t i = 0; i < kParallelism; ++i) mnv_stream_sync(streams_[i]);
   for (auto& kv : produced_) mnv_event_destroy(kv.second.event);
@@ -170,30 +58,27 @@ HipDevice::~HipDevice() {
 
 void HipDevice::Activate() const { Ok(mnv_device_set(gpu_id_), "set device"); }
 
+// every task re-selects the device on its thread (reference device.cpp:201-203)
+void HipDevice::PreExecute() { Activate(); }
+
+void HipDevice::DoCopyRemoteData(float* dst, float* src, size_t bytes, int thrid) {
+  Ok(mnv_memcpy_d2d(dst, src, bytes, streams_[thrid]), "remote copy");
+  Ok(mnv_stream_sync(streams_[thrid]), "remote copy sync");
+}
+
 std::string HipDevice::Name() const {
   char buf[64];
   snprintf(buf, sizeof(buf), "HIP device #%d", static_cast<int>(device_id_));
   return buf;
 }
 
-std::string HipDevice::GetMemUsage() const {
-  char buf[96];
-  snprintf(buf, sizeof(buf), "device #%d used %zuB", static_cast<int>(device_id_),
-           data_store_->GetTotalBytes());
-  return buf;
-}
-
-std::pair<HipDevice::MemType, float*> HipDevice::GetPtr(uint64_t data_id) {
-  return std::make_pair(MemType::kGpu, data_store_->GetData(data_id));
-}
-
 void HipDevice::FreeDataIfExist(uint64_t data_id) {
   size_t erased;
   unsigned users = 0;
   void* event = nullptr;
+  erased = local_data_.Erase(data_id);
   {
     std::lock_guard<std::mutex> lck(local_mutex_);
-    erased = local_data_.erase(data_id);
     auto it = produced_.find(data_id);
     if (it != produced_.end()) {
       // The host may be far ahead of the GPU: kernels that read or write this block can
@@ -235,49 +120,7 @@ void HipDevice::PushTask(Task* task) {
     Execute(task, task->stream);
     return;
   }
-  {
-    std::lock_guard<std::mutex> lck(q_mutex_);
-    queue_.push_back(task);
-  }
-  q_cv_.notify_one();
-}
-
-void HipDevice::WorkerLoop(int thrid) {
-  for (;;) {
-    Task* task = nullptr;
-    {
-      std::unique_lock<std::mutex> lck(q_mutex_);
-      q_cv_.wait(lck, [this] { return stop_ || !queue_.empty(); });
-      if (queue_.empty()) return;  // stop_ and drained
-      task = queue_.front();
-      queue_.pop_front();
-      ++busy_;
-    }
-    try {
-      Execute(task, thrid, true);
-    } catch (const std::exception& e) {
-      std::lock_guard<std::mutex> lck(err_mutex_);
-      if (async_error_.empty()) async_error_ = e.what();
-      if (listener_) listener_->OnOperationComplete(task);
-    }
-    {
-      std::lock_guard<std::mutex> lck(q_mutex_);
-      --busy_;
-    }
-    idle_cv_.notify_all();
-  }
-}
-
-void HipDevice::WaitForAllFinished() {
-  std::unique_lock<std::mutex> lck(q_mutex_);
-  idle_cv_.wait(lck, [this] { return queue_.empty() && busy_ == 0; });
-}
-
-std::string HipDevice::TakeAsyncError() {
-  std::lock_guard<std::mutex> lck(err_mutex_);
-  std::string e;
-  e.swap(async_error_);
-  return e;
+  ThreadedDevice::PushTask(task);
 }
 
 void HipDevice::EnsureWorkspace(int thrid, size_t bytes) {
@@ -295,8 +138,10 @@ void HipDevice::EnsureStaging(int thrid) {
   Ok(mnv_host_malloc(&staging_[thrid], kStagingBytes), "pinned staging");
 }
 
-void HipDevice::Execute(Task* task, int thrid, bool pooled) {
-  Activate();  // every task re-selects the device on its thread (device.cpp:201-203)
+// ThreadedDevice::Execute plus what dataflow mode needs: waits for producers on other
+// streams, stream-aware block recycling, and an event behind every output.
+void HipDevice::Execute(Task* task, int thrid) {
+  PreExecute();
   DataList input_shards;
   for (auto& i : task->inputs) {
     auto& d = i.physical_data;
@@ -304,9 +149,9 @@ void HipDevice::Execute(Task* task, int thrid, bool pooled) {
     // mnv_memcpy_d2d over xGMI, as DoCopyRemoteData does in the reference.
     MNV_CHECK_EQ(d.device_id, device_id_) << "remote inputs are not part of the one-GPU build";
     void* wait_for = nullptr;
+    MNV_CHECK_EQ(local_data_.Count(d.data_id), 1u) << "input data #" << d.data_id << " missing";
     {
       std::lock_guard<std::mutex> lck(local_mutex_);
-      MNV_CHECK_EQ(local_data_.count(d.data_id), 1u) << "input data #" << d.data_id << " missing";
       if (dataflow_) {
         auto it = produced_.find(d.data_id);
         if (it != produced_.end()) {
@@ -330,14 +175,11 @@ void HipDevice::Execute(Task* task, int thrid, bool pooled) {
                                          &foreign);
     // a recycled block that work queued on other streams may still touch
     if (foreign) WaitForStreams(thrid, foreign);
-    {
-      std::lock_guard<std::mutex> lck(local_mutex_);
-      MNV_CHECK(local_data_.insert(o.physical_data.data_id).second) << "duplicate data";
-    }
+    MNV_CHECK(local_data_.Insert(o.physical_data.data_id)) << "duplicate data";
     output_shards.emplace_back(ptr, o.physical_data.size);
   }
   MNV_CHECK(task->op.compute_fn) << "task without an operator";
-  DoExecute(input_shards, output_shards, task->op, thrid, pooled);
+  DoExecute(input_shards, output_shards, task->op, thrid);
   if (dataflow_) {
     // an operator that fills one of its inputs (LRNForward's scale) is that datum's producer
     // from now on: later readers on other streams must wait for this operator, not for the
@@ -369,8 +211,8 @@ void HipDevice::Execute(Task* task, int thrid, bool pooled) {
   if (listener_) listener_->OnOperationComplete(task);
 }
 
-void HipDevice::DoExecute(const DataList& in, const DataList& out, PhysicalOp& op, int thrid,
-                          bool pooled) {
+void HipDevice::DoExecute(const DataList& in, const DataList& out, PhysicalOp& op, int thrid) {
+  const bool pooled = OnPoolThread();
   EnsureWorkspace(thrid, kWorkspaceBytes);
   Context ctx;
   ctx.impl_type = ImplType::kHip;

@@ -6,22 +6,12 @@
 #pragma once
 #include <typeinfo>
 
+#include "device.h"
 #include "hip_fused_ops.h"
 #include "hip_ops.h"
 #include "minerva_types.h"
 
 namespace minerva {
-
-class ComputeFn {
- public:
-  virtual ~ComputeFn() {}
-  virtual void Execute(const DataList&, const DataList&, const Context&) = 0;
-  virtual std::string Name() const = 0;
-  // Index of an input the operator writes (LRNForward fills its `scale` input, as the
-  // reference does, cuda.cpp:45-59), or -1: a device that orders operators by data
-  // dependencies must treat the operator as that datum's latest producer.
-  virtual int MutatedInput() const { return -1; }
-};
 
 template <typename C> struct FnBundle;
 
