@@ -167,6 +167,38 @@ def owl_front_end_bench(steps, warmup):
             "ops_per_step": int(ops), "finite": finite}
 
 
+def owl_net_bench(steps, warmup):
+    """Caffe's reference AlexNet (norm1 / norm2 LRN, drop6 / drop7, momentum 0.9, weight decay
+    5e-4; every convolution in one group) trained through owl.net, the reference's Caffe-like
+    layer package, at batch 256 on one synthetic batch resident in HBM.  This is the network
+    behind the one number the reference publishes (189.63 images/s on a GTX Titan with
+    cuDNN): context only, it is neither the metric's configuration nor `value`."""
+    from minerva_amd import owl
+    from minerva_amd.owl import net as onet
+    from minerva_amd.owl.net import models
+    owl.set_device(owl.create_gpu_device(0))
+    tr = onet.NetTrainer(models.ALEXNET_SOLVER, models.alexnet_prototxt(BATCH), seed=1)
+    rng = np.random.default_rng(2)
+    tr.owl_net.get_data_unit().set_batch(rng.standard_normal(BATCH * 3 * 227 * 227, dtype=np.float32),
+                                         rng.integers(0, 1000, BATCH))
+    rt = owl._runtime()
+    tr.run(warmup)
+    ops0 = rt.ops_issued()
+    t0 = time.perf_counter()
+    tr.run(steps)
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    ops = (rt.ops_issued() - ops0) // steps
+    loss = tr.owl_net.get_loss_units()[0].getloss()
+    del tr
+    owl.close_devices()
+    log("caffe-style alexnet b=%d through owl.net: %.3f ms/step, %d ops/step" % (BATCH, ms, ops))
+    return {"network": "Caffe reference AlexNet, single group, LRN + dropout, momentum SGD",
+            "ms_per_step": round(ms, 3), "images_per_s": round(BATCH / (ms / 1e3), 1),
+            "ops_per_step": int(ops), "loss_finite": bool(np.isfinite(loss)),
+            "reference_published_images_per_s": 189.63,
+            "reference_published_on": "GTX Titan, cuDNN, full Caffe AlexNet (README.md:76-82)"}
+
+
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_gemm_kernels_hbm_traffic_pmc.txt")
 
 
@@ -595,6 +627,7 @@ def main():
         line["config"]["ops_per_step"] = main_run["ops_per_step"]
     if "owl" in want:
         line["owl_front_end"] = owl_front_end_bench(args.steps, args.warmup)
+        line["owl_net_caffe_alexnet"] = owl_net_bench(args.steps, args.warmup)
     if "sgemm" in want:
         line["sgemm"] = sgemm_bench()
     if "eltwise" in want:

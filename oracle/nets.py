@@ -264,3 +264,120 @@ def make_inputs(kind, batch, seed=1000, classes=None):
     label = np.zeros((batch, classes), np.float32)
     label[np.arange(batch), lab] = 1.0
     return params, data, label.ravel()
+
+
+# ---------------------------------------------------------------------------------------
+# Caffe-style networks as the reference's owl.net package runs them (owl/owl/net/net.py):
+# a chain of units, each a tuple; `acts[i]` is the output of unit i (acts[-1] of the data).
+#   ("conv", name, C, K, H, W, pad, stride, kernel)   ConvConnection  net.py:639-731
+#   ("relu",)                                          ReluUnit: gradient gated by the INPUT
+#   ("lrn", C, H, W, local_size, alpha, beta)          LRNUnit
+#   ("pool", C, H, W, kernel, stride, pad)             PoolingUnit (max)
+#   ("fc", name, n_in, n_out)                          FullyConnection
+#   ("dropout", n, ratio)                              DropoutUnit: x * mask * 1/(1-ratio)
+# followed by the softmax loss unit: sens = prob - onehot.
+def caffe_alexnet_units(classes=1000):
+    return [("conv", "conv1", 3, 96, 227, 227, 0, 4, 11), ("relu",), ("lrn", 96, 55, 55, 5, 1e-4, 0.75),
+            ("pool", 96, 55, 55, 3, 2, 0),
+            ("conv", "conv2", 96, 256, 27, 27, 2, 1, 5), ("relu",), ("lrn", 256, 27, 27, 5, 1e-4, 0.75),
+            ("pool", 256, 27, 27, 3, 2, 0),
+            ("conv", "conv3", 256, 384, 13, 13, 1, 1, 3), ("relu",),
+            ("conv", "conv4", 384, 384, 13, 13, 1, 1, 3), ("relu",),
+            ("conv", "conv5", 384, 256, 13, 13, 1, 1, 3), ("relu",), ("pool", 256, 13, 13, 3, 2, 0),
+            ("fc", "fc6", 9216, 4096), ("relu",), ("dropout", 4096, 0.5),
+            ("fc", "fc7", 4096, 4096), ("relu",), ("dropout", 4096, 0.5),
+            ("fc", "fc8", 4096, classes)]
+
+
+def caffe_param_shapes(units):
+    shapes = {}
+    for u in units:
+        if u[0] == "conv":
+            _, name, C, K, _, _, _, _, k = u
+            shapes[name] = ([k, k, C, K], [K])
+        elif u[0] == "fc":
+            shapes[u[1]] = ([u[3], u[2]], [u[3], 1])
+    return shapes
+
+
+def caffe_forward(units, params, data, batch, masks=()):
+    """params: name -> (weight, bias).  masks: one Bernoulli mask per dropout unit, in order
+    (empty: the TEST phase, dropout passes through).  Returns (acts, probabilities)."""
+    N = batch
+    acts, x, masks = [], data, list(masks)
+    for u in units:
+        if u[0] == "conv":
+            _, name, C, K, H, W, pad, stride, k = u
+            x = ora.conv_fwd(x, params[name][0], params[name][1], N, C, K, H, W, pad, pad, stride, stride, k, k)
+        elif u[0] == "relu":
+            x = _relu(x)
+        elif u[0] == "lrn":
+            _, C, H, W, size, alpha, beta = u
+            x = ora.lrn_fwd(x, size, alpha, beta, N, C, H, W)[0]
+        elif u[0] == "pool":
+            _, C, H, W, k, s, p = u
+            x = ora.pool_fwd(ora.POOL_MAX, x, N, C, H, W, s, s, k, k, p, p)
+        elif u[0] == "fc":
+            _, name, nin, nout = u
+            x = _fc(params[name][0], x, params[name][1], nout, nin, N)
+        elif u[0] == "dropout":
+            if masks:
+                scale = np.float32(1.0 / (1.0 - u[2]))
+                x = ora.arithmetic_const(ora.MUL, 1, scale, ora.arithmetic(ora.MUL, x, masks.pop(0)))
+        else:
+            raise ValueError(u[0])
+        acts.append(x)
+    classes = units[-1][3]
+    return acts, ora.softmax_instance_fwd(x, N, classes, 1, 1)
+
+
+def caffe_backward(units, params, data, acts, prob, labels, batch, masks=()):
+    """Gradients name -> (weight gradient, bias gradient) from given forward results (the
+    oracle's own or another implementation's: see alexnet_backward)."""
+    N = batch
+    classes = units[-1][3]
+    onehot = np.zeros((N, classes), np.float32)
+    onehot[np.arange(N), np.asarray(labels).astype(np.int64)] = 1
+    sen = ora.arithmetic(ora.SUB, prob, onehot.ravel())
+    masks = list(masks)
+    grads = {}
+    mm = lambda a, b, m, n, k: ora.matmult(a, b, m, n, k, fast=True)
+    for i in range(len(units) - 1, -1, -1):
+        u = units[i]
+        bottom = acts[i - 1] if i > 0 else data
+        if u[0] == "conv":
+            _, name, C, K, H, W, pad, stride, k = u
+            geo = (N, C, K, H, W, pad, pad, stride, stride, k, k)
+            Ho = (H + 2 * pad - k) // stride + 1
+            grads[name] = (ora.conv_bwd_filter(sen, bottom, *geo), ora.conv_bwd_bias(sen, N, K, Ho, Ho))
+            sen = ora.conv_bwd_data(sen, params[name][0], *geo) if i > 0 else None
+        elif u[0] == "relu":
+            sen = ora.activation_bwd(ora.RELU, sen, acts[i], bottom)
+        elif u[0] == "lrn":
+            _, C, H, W, size, alpha, beta = u
+            top, scale = ora.lrn_fwd(bottom, size, alpha, beta, N, C, H, W)
+            sen = ora.lrn_bwd(bottom, top, scale, sen, size, alpha, beta, N, C, H, W)
+        elif u[0] == "pool":
+            _, C, H, W, k, s, p = u
+            sen = ora.pool_bwd(ora.POOL_MAX, sen, acts[i], bottom, N, C, H, W, s, s, k, k, p, p)
+        elif u[0] == "fc":
+            _, name, nin, nout = u
+            grads[name] = (mm(sen, ora.transpose(bottom, N, nin), nout, nin, N),
+                           ora.reduction(ora.SUM, sen, [nout, N], [1]))
+            sen = mm(ora.transpose(params[name][0], nin, nout), sen, nin, N, nout)
+        elif u[0] == "dropout":
+            if masks:
+                scale = np.float32(1.0 / (1.0 - u[2]))
+                sen = ora.arithmetic_const(ora.MUL, 1, scale, ora.arithmetic(ora.MUL, sen, masks.pop()))
+    return grads
+
+
+def caffe_update(value, delta, grad, base_lr, lr_mult, weight_decay, decay_mult, momentum, batch):
+    """WeightedComputeUnit.weight_update (net.py:241-262), operation by operation in fp32:
+    delta' = momentum*delta - (lr*lr_mult/batch)*grad - (lr*lr_mult*wd*decay_mult)*value;
+    value' = value + delta'.  Returns (value', delta')."""
+    f = np.float32
+    t = ora.arithmetic_const(ora.MUL, 0, f(momentum), delta)
+    t = ora.arithmetic(ora.SUB, t, ora.arithmetic_const(ora.MUL, 0, f(base_lr * lr_mult / batch), grad))
+    t = ora.arithmetic(ora.SUB, t, ora.arithmetic_const(ora.MUL, 0, f(base_lr * lr_mult * weight_decay * decay_mult), value))
+    return ora.arithmetic(ora.ADD, value, t), t

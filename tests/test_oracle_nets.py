@@ -108,3 +108,43 @@ def test_alexnet_forward_is_the_forward_half_of_the_step():
     np.testing.assert_array_equal(out, res["prob"])
     assert all(np.array_equal(a, b) for a, b in zip(acts, res["acts"]))
     assert abs(float(out.sum()) - 1.0) < 1e-5
+
+
+def test_caffe_style_graph_gradient_is_the_loss_derivative():
+    """The owl.net-style unit chain (convolution, ReLU gated by its input, LRN, max pooling,
+    inner product, dropout with its 1/(1-ratio) scale, softmax loss): central differences of
+    the loss pin caffe_backward, including the LRN gradient and the dropout scale."""
+    units = [("conv", "c1", 2, 4, 8, 8, 1, 1, 3), ("relu",), ("lrn", 4, 8, 8, 3, 0.5, 0.75),
+             ("pool", 4, 8, 8, 3, 2, 0), ("fc", "f1", 64, 6), ("relu",), ("dropout", 6, 0.5),
+             ("fc", "f2", 6, 3)]
+    batch, classes = 3, 3
+    rng = np.random.default_rng(11)
+    shapes = nets.caffe_param_shapes(units)
+    flat = {}
+    for name, (ws, bs) in shapes.items():
+        flat[name + ".w"] = (rng.standard_normal(int(np.prod(ws))) * 0.4).astype(np.float32)
+        flat[name + ".b"] = (rng.standard_normal(int(np.prod(bs))) * 0.1).astype(np.float32)
+    data = rng.standard_normal(batch * 2 * 8 * 8).astype(np.float32)
+    labels = rng.integers(0, classes, batch)
+    onehot = np.zeros((batch, classes), np.float32)
+    onehot[np.arange(batch), labels] = 1
+    masks = [(rng.random(6 * batch) < 0.5).astype(np.float32)]
+
+    def step(p):
+        params = {n: (p[n + ".w"], p[n + ".b"]) for n in shapes}
+        acts, prob = nets.caffe_forward(units, params, data, batch, masks)
+        g = nets.caffe_backward(units, params, data, acts, prob, labels, batch, masks)
+        grads = {}
+        for n in shapes:
+            grads[n + ".w"], grads[n + ".b"] = g[n]
+        return grads, prob
+
+    _directional_check(step, flat, data, onehot, classes, batch, eps=1e-3, tol=1e-2, seed=12)
+
+
+def test_caffe_update_rule():
+    rng = np.random.default_rng(13)
+    w, d, g = (rng.standard_normal(50).astype(np.float32) for _ in range(3))
+    new_w, new_d = nets.caffe_update(w, d, g, 0.01, 2.0, 0.0005, 1.0, 0.9, 4)
+    want_d = 0.9 * d.astype(np.float64) - 0.01 * 2 / 4 * g - 0.01 * 2 * 0.0005 * w
+    assert np.max(np.abs(new_d - want_d)) < 1e-6 and np.max(np.abs(new_w - (w + want_d))) < 1e-6
