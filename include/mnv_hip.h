@@ -146,8 +146,11 @@ int mnv_maxindex_row(const float* in, float* out, int m, int n, mnv_stream_t str
 /* ---- SGEMM: CudaPerformMatMult (cuda_perform.h:17; cublasSgemm N,N, alpha 1,
  * beta 0, cuda_perform.cu:66-70).  C{m,n} = A{m,k} * B{k,n}, all column-major with
  * leading dimensions m, k, m.  The workspace (optional) lets skinny products split
- * the k range over more workgroups.  A and B are read through 32-bit byte offsets:
- * m*k and k*n must be below 2^29 elements (2 GiB each), else MNV_ERR_INVALID. ---- */
+ * the k range over more workgroups.  Each matrix may hold up to 2^31 - 1 elements (the
+ * reference's int counts).  One launch reads A and B through 32-bit byte offsets, i.e. up
+ * to 2^29 - 1 elements each; beyond that the product runs as several launches over column
+ * panels and k ranges (later k ranges accumulate into C): slower, and summed range by
+ * range. ---- */
 size_t mnv_sgemm_nn_workspace_bytes(int m, int n, int k);
 int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k,
                  void* workspace, size_t workspace_bytes, mnv_stream_t stream);
@@ -220,8 +223,10 @@ int mnv_softmax_channel_bwd(const float* top_diff, const float* top, float* bott
  * the filter for forward / backward_data (which then read the reduction dimension as
  * (tap, channel) and spend no address arithmetic per 16-channel slab) and the split
  * partial sums for backward_filter; without it a slower, equally exact path runs.
- * Each of bottom, top and filter must hold fewer than 2^29 elements (2 GiB; the tensors
- * are read through 32-bit byte offsets), else MNV_ERR_INVALID. ---- */
+ * One launch reads bottom, top and filter through 32-bit byte offsets (fewer than 2^29
+ * elements each).  A batch whose bottom or top is larger (up to 2^31 - 1 elements) runs as
+ * several launches over chunks of images, the filter gradient accumulating chunk by chunk;
+ * only a single image or a filter of 2^29 elements and more is refused (MNV_ERR_INVALID). ---- */
 size_t mnv_conv_fwd_workspace_bytes(int num_images, int bottom_num_channels,
                                    int top_num_channels, int bottom_height, int bottom_width,
                                    int pad_height, int pad_width, int stride_vertical,

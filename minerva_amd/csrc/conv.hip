@@ -343,6 +343,7 @@ struct ConvBwdFilter {
   float* __restrict__ filter_diff;
   ConvGeom g;
   int M, N, K, total_slabs, spp;  // C*R*S, Kout, N*Ho*Wo
+  int accumulate;                 // filter_diff += (a later chunk of images)
   struct Res {
     mnv_rsrc a, b;
   };
@@ -412,7 +413,10 @@ struct ConvBwdFilter {
                          float (&v)[4]) const {
     mnv_fetch_vec<4>(r.b, off, 0u, v);
   }
-  __device__ void c_store(int m, int n, float x) const { filter_diff[(size_t)n * M + m] = x; }
+  __device__ void c_store(int m, int n, float x) const {
+    float* p = filter_diff + (size_t)n * M + m;
+    *p = accumulate ? *p + x : x;
+  }
 };
 
 // Filter gradient, fast addressing.  The GEMM rows are ordered (tap, channel) instead of
@@ -439,6 +443,7 @@ struct ConvBwdFilterFast {
   int M, N, K, total_slabs, spp;  // C*R*S rows in (tap, c) order, Kout, N*Ho*Wo
   int PP, taps_per_block;         // padded positions per image, table rows per workgroup
   MnvFastDiv d_C;
+  int accumulate;                 // filter_diff += (a later chunk of images)
   struct Res {
     mnv_rsrc a, b;
     const unsigned* tab;  // LDS: [taps_per_block][PP]
@@ -530,13 +535,13 @@ struct ConvBwdFilterFast {
     }
   }
   __device__ void c_store(int m, int n, float x) const {
-    if (NP) {
-      filter_diff[(size_t)n * M + m] = x;
-      return;
+    int row = m;
+    if (!NP) {
+      int tap = mnv_fastdiv(m, d_C);
+      row = (m - tap * g.C) * g.RS + tap;
     }
-    int tap = mnv_fastdiv(m, d_C);
-    int c = m - tap * g.C;
-    filter_diff[(size_t)n * M + c * g.RS + tap] = x;
+    float* p = filter_diff + (size_t)n * M + row;
+    *p = accumulate ? *p + x : x;
   }
 };
 
@@ -624,6 +629,25 @@ int make_geom(ConvGeom* g, int N, int C, int K, int H, int W, int ph, int pw, in
   g->d_sv = mnv_fastdiv_make(sv);
   g->d_sh = mnv_fastdiv_make(sh);
   return MNV_OK;
+}
+
+// Images per launch: bottom, top and filter are read through 32-bit byte offsets, so one
+// launch takes at most 2^29 - 1 elements of each.  A larger batch (up to the reference's
+// limit of 2^31 - 1 elements per tensor) runs as several launches over chunks of images --
+// images are the slowest dimension, so a chunk is a contiguous slice of bottom and top --
+// with the filter gradient accumulated chunk by chunk.  0: a single image (or the filter)
+// is too large.
+int images_per_launch(int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S) {
+  if (N <= 0 || C <= 0 || K <= 0 || H <= 0 || W <= 0 || ph < 0 || pw < 0 || sv <= 0 || sh <= 0 ||
+      R <= 0 || S <= 0 || H + 2 * ph < R || W + 2 * pw < S)
+    return 0;
+  const long long lim = (1LL << 29) - 1;
+  const long long Ho = (H + 2 * ph - R) / sv + 1, Wo = (W + 2 * pw - S) / sh + 1;
+  const long long per_bottom = (long long)C * H * W, per_top = (long long)K * Ho * Wo;
+  if ((long long)K * C * R * S > lim || per_bottom > lim || per_top > lim) return 0;
+  if (per_bottom * N > 0x7fffffffLL || per_top * N > 0x7fffffffLL) return 0;
+  long long chunk = lim / (per_bottom > per_top ? per_bottom : per_top);
+  return (int)(chunk < N ? chunk : N);
 }
 
 int pick_tile(int m, int n) {
@@ -730,18 +754,38 @@ static int conv_fwd_impl(const float* bottom, const float* filter, const float* 
   return launch_tile(tile, p, splits, part, s);
 }
 
+static int conv_fwd_chunks(const float* bottom, const float* filter, const float* bias, float* top,
+                           int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R,
+                           int S, void* workspace, size_t workspace_bytes, mnv_stream_t stream,
+                           int relu) {
+  const int chunk = images_per_launch(N, C, K, H, W, ph, pw, sv, sh, R, S);
+  if (chunk <= 0 || chunk >= N)  // the usual case, and invalid geometry (refused inside)
+    return conv_fwd_impl(bottom, filter, bias, top, N, C, K, H, W, ph, pw, sv, sh, R, S, workspace,
+                         workspace_bytes, stream, relu);
+  if (!bottom || !top) return MNV_ERR_INVALID;
+  const size_t per_bottom = (size_t)C * H * W;
+  const size_t per_top = (size_t)K * ((H + 2 * ph - R) / sv + 1) * ((W + 2 * pw - S) / sh + 1);
+  for (int n0 = 0; n0 < N; n0 += chunk) {
+    const int nn = N - n0 < chunk ? N - n0 : chunk;
+    int rc = conv_fwd_impl(bottom + n0 * per_bottom, filter, bias, top + n0 * per_top, nn, C, K, H,
+                           W, ph, pw, sv, sh, R, S, workspace, workspace_bytes, stream, relu);
+    if (rc) return rc;
+  }
+  return MNV_OK;
+}
+
 int mnv_conv_fwd(const float* bottom, const float* filter, const float* bias, float* top, int N,
                  int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S,
                  void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
-  return conv_fwd_impl(bottom, filter, bias, top, N, C, K, H, W, ph, pw, sv, sh, R, S, workspace,
-                       workspace_bytes, stream, 0);
+  return conv_fwd_chunks(bottom, filter, bias, top, N, C, K, H, W, ph, pw, sv, sh, R, S, workspace,
+                         workspace_bytes, stream, 0);
 }
 
 int mnv_conv_fwd_relu(const float* bottom, const float* filter, const float* bias, float* top,
                       int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R,
                       int S, void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
-  return conv_fwd_impl(bottom, filter, bias, top, N, C, K, H, W, ph, pw, sv, sh, R, S, workspace,
-                       workspace_bytes, stream, 1);
+  return conv_fwd_chunks(bottom, filter, bias, top, N, C, K, H, W, ph, pw, sv, sh, R, S, workspace,
+                         workspace_bytes, stream, 1);
 }
 
 size_t mnv_conv_bwd_data_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw,
@@ -782,11 +826,32 @@ static int conv_bwd_data_impl(const float* top_diff, const float* filter, const 
   return launch_tile(tile, p, splits, part, s);
 }
 
+static int conv_bwd_data_chunks(const float* top_diff, const float* filter, const float* gate,
+                                float* bottom_diff, int N, int C, int K, int H, int W, int ph,
+                                int pw, int sv, int sh, int R, int S, void* workspace,
+                                size_t workspace_bytes, mnv_stream_t stream) {
+  const int chunk = images_per_launch(N, C, K, H, W, ph, pw, sv, sh, R, S);
+  if (chunk <= 0 || chunk >= N)
+    return conv_bwd_data_impl(top_diff, filter, gate, bottom_diff, N, C, K, H, W, ph, pw, sv, sh, R,
+                              S, workspace, workspace_bytes, stream);
+  if (!top_diff || !bottom_diff) return MNV_ERR_INVALID;
+  const size_t per_bottom = (size_t)C * H * W;
+  const size_t per_top = (size_t)K * ((H + 2 * ph - R) / sv + 1) * ((W + 2 * pw - S) / sh + 1);
+  for (int n0 = 0; n0 < N; n0 += chunk) {
+    const int nn = N - n0 < chunk ? N - n0 : chunk;
+    int rc = conv_bwd_data_impl(top_diff + n0 * per_top, filter, gate ? gate + n0 * per_bottom : nullptr,
+                                bottom_diff + n0 * per_bottom, nn, C, K, H, W, ph, pw, sv, sh, R, S,
+                                workspace, workspace_bytes, stream);
+    if (rc) return rc;
+  }
+  return MNV_OK;
+}
+
 int mnv_conv_bwd_data(const float* top_diff, const float* filter, float* bottom_diff, int N,
                       int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S,
                       void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
-  return conv_bwd_data_impl(top_diff, filter, nullptr, bottom_diff, N, C, K, H, W, ph, pw, sv, sh,
-                            R, S, workspace, workspace_bytes, stream);
+  return conv_bwd_data_chunks(top_diff, filter, nullptr, bottom_diff, N, C, K, H, W, ph, pw, sv, sh,
+                              R, S, workspace, workspace_bytes, stream);
 }
 
 int mnv_conv_bwd_data_relu(const float* top_diff, const float* filter, const float* bottom,
@@ -794,8 +859,8 @@ int mnv_conv_bwd_data_relu(const float* top_diff, const float* filter, const flo
                            int sv, int sh, int R, int S, void* workspace, size_t workspace_bytes,
                            mnv_stream_t stream) {
   if (!bottom) return MNV_ERR_INVALID;
-  return conv_bwd_data_impl(top_diff, filter, bottom, bottom_diff, N, C, K, H, W, ph, pw, sv, sh,
-                            R, S, workspace, workspace_bytes, stream);
+  return conv_bwd_data_chunks(top_diff, filter, bottom, bottom_diff, N, C, K, H, W, ph, pw, sv, sh,
+                              R, S, workspace, workspace_bytes, stream);
 }
 
 size_t mnv_conv_bwd_filter_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw,
@@ -806,9 +871,10 @@ size_t mnv_conv_bwd_filter_workspace_bytes(int N, int C, int K, int H, int W, in
   return splits > 1 ? (size_t)splits * g.CRS * K * sizeof(float) : 0;
 }
 
-int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filter_diff, int N,
-                        int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S,
-                        void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
+static int conv_bwd_filter_impl(const float* bottom, const float* top_diff, float* filter_diff,
+                                int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh,
+                                int R, int S, void* workspace, size_t workspace_bytes,
+                                mnv_stream_t stream, int accumulate) {
   ConvGeom g;
   if (!bottom || !top_diff || !filter_diff) return MNV_ERR_INVALID;
   int rc = make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S);
@@ -832,16 +898,36 @@ int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filte
   }
   if (tile != 0 && ph == 0 && pw == 0 && (size_t)PP * 4 <= 24 * 1024) {
     ConvBwdFilterFast<true> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
-                              PP / 16, PP, 1, mnv_fastdiv_make(C)};
+                              PP / 16, PP, 1, mnv_fastdiv_make(C), accumulate};
     return launch_tile(tile, p, splits, workspace, s);
   }
   if (tile != 0 && (size_t)taps_per_block * PP * 4 <= 24 * 1024) {
     ConvBwdFilterFast<false> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
-                               PP / 16, PP, taps_per_block, mnv_fastdiv_make(C)};
+                               PP / 16, PP, taps_per_block, mnv_fastdiv_make(C), accumulate};
     return launch_tile(tile, p, splits, workspace, s);
   }
-  ConvBwdFilter p{bottom, top_diff, filter_diff, g, gm, gn, gk, (gk + 15) / 16, 1};
+  ConvBwdFilter p{bottom, top_diff, filter_diff, g, gm, gn, gk, (gk + 15) / 16, 1, accumulate};
   return launch_tile(tile, p, splits, workspace, s);
+}
+
+int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filter_diff, int N,
+                        int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R, int S,
+                        void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
+  const int chunk = images_per_launch(N, C, K, H, W, ph, pw, sv, sh, R, S);
+  if (chunk <= 0 || chunk >= N)
+    return conv_bwd_filter_impl(bottom, top_diff, filter_diff, N, C, K, H, W, ph, pw, sv, sh, R, S,
+                                workspace, workspace_bytes, stream, 0);
+  if (!bottom || !top_diff) return MNV_ERR_INVALID;
+  const size_t per_bottom = (size_t)C * H * W;
+  const size_t per_top = (size_t)K * ((H + 2 * ph - R) / sv + 1) * ((W + 2 * pw - S) / sh + 1);
+  for (int n0 = 0; n0 < N; n0 += chunk) {
+    const int nn = N - n0 < chunk ? N - n0 : chunk;
+    int rc = conv_bwd_filter_impl(bottom + n0 * per_bottom, top_diff + n0 * per_top, filter_diff, nn,
+                                  C, K, H, W, ph, pw, sv, sh, R, S, workspace, workspace_bytes,
+                                  stream, n0 > 0);
+    if (rc) return rc;
+  }
+  return MNV_OK;
 }
 
 }  // extern "C"

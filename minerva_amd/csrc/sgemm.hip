@@ -27,6 +27,10 @@ struct SgemmNN {
   const float* __restrict__ B;
   float* __restrict__ C;
   int M, N, K, total_slabs, spp, bk;
+  // Leading dimensions (floats between consecutive columns): m, k, m for whole matrices;
+  // larger when the operands are panels of matrices too large for 32-bit byte offsets.
+  // accumulate: C += A*B (the k panels after the first).
+  int lda, ldb, ldc, accumulate;
   // Fused epilogues (all off for the plain product), applied in this order to the value
   // stored, each the single operation the separate operator performs:
   //   bias: + bias[m] (the broadcast add of an {m,1} vector); relu: max(., 0);
@@ -40,26 +44,26 @@ struct SgemmNN {
   struct AState {};
   struct BState {};
   __device__ void make_res(Res& r) const {
-    r.a = mnv_make_rsrc(A, (unsigned)M * (unsigned)K * 4u);
-    r.b = mnv_make_rsrc(B, (unsigned)K * (unsigned)N * 4u);
+    r.a = mnv_make_rsrc(A, ((unsigned)(K - 1) * (unsigned)lda + (unsigned)M) * 4u);
+    r.b = mnv_make_rsrc(B, ((unsigned)(N - 1) * (unsigned)ldb + (unsigned)K) * 4u);
   }
   __device__ void a_init(const Res&, AState&, int) const {}
   __device__ void b_init(const Res&, BState&, int) const {}
   // A[m..m+3, k]: x-fast
   __device__ void a_period(const AState&, unsigned (&off)[A_NOFF], int m, int kl, int period) const {
     const int k = period * spp * bk + kl;
-    const unsigned base = ((unsigned)k * (unsigned)M + (unsigned)m) * 4u;
+    const unsigned base = ((unsigned)k * (unsigned)lda + (unsigned)m) * 4u;
 #pragma unroll
     for (int q = 0; q < A_NOFF; ++q) off[q] = ((m + q < M) & (k < K)) ? base + 4u * q : MNV_OOB;
   }
   __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[A_NOFF], int, int s,
                          int, float (&v)[4]) const {
-    mnv_fetch_vec<A_NOFF>(r.a, off, (unsigned)s * (unsigned)bk * (unsigned)M * 4u, v);
+    mnv_fetch_vec<A_NOFF>(r.a, off, (unsigned)s * (unsigned)bk * (unsigned)lda * 4u, v);
   }
   // B[k..k+3, n]: k-fast
   __device__ void b_period(const BState&, unsigned (&off)[B_NOFF], int n, int kl, int period) const {
     const int k = period * spp * bk + kl;
-    const unsigned base = ((unsigned)n * (unsigned)K + (unsigned)k) * 4u;
+    const unsigned base = ((unsigned)n * (unsigned)ldb + (unsigned)k) * 4u;
 #pragma unroll
     for (int q = 0; q < B_NOFF; ++q) off[q] = ((n < N) & (k + q < K)) ? base + 4u * q : MNV_OOB;
   }
@@ -75,7 +79,8 @@ struct SgemmNN {
   }
   __device__ void block_init(Res&, float*, int, int) const {}
   __device__ void c_store(int m, int n, float x) const {
-    const size_t at = (size_t)n * M + m;
+    const size_t at = (size_t)n * ldc + m;
+    if (accumulate) x = C[at] + x;
     if (bias) x = x + bias[m];
     if (relu) x = x > 0.f ? x : 0.f;
     if (gate) x = gate[at] > 0.f ? x : 0.f;
@@ -87,6 +92,7 @@ struct SgemmEpilogue {
   const float* bias;
   const float* gate;
   int relu;
+  int lda = 0, ldb = 0, ldc = 0, accumulate = 0;  // 0: the matrices' own m, k, m
 };
 
 template <bool VEC>
@@ -95,6 +101,8 @@ SgemmNN<VEC> make_sgemm(const float* a, const float* b, float* c, int m, int n, 
   SgemmNN<VEC> p;
   p.A = a; p.B = b; p.C = c; p.M = m; p.N = n; p.K = k;
   p.bias = e.bias; p.gate = e.gate; p.relu = e.relu;
+  p.lda = e.lda ? e.lda : m; p.ldb = e.ldb ? e.ldb : k; p.ldc = e.ldc ? e.ldc : m;
+  p.accumulate = e.accumulate;
   p.set_bk(16);
   return p;
 }
@@ -163,7 +171,8 @@ int scratch_address(float** out) {
 int sgemm_nn_impl(const float* a, const float* b, float* c, int m, int n, int k, void* workspace,
                   size_t workspace_bytes, hipStream_t s,
                   const SgemmEpilogue& e = SgemmEpilogue{nullptr, nullptr, 0}) {
-  bool vec = (m % 4 == 0) && (k % 4 == 0) && mnv_aligned16(a) && mnv_aligned16(b);
+  bool vec = (m % 4 == 0) && (k % 4 == 0) && mnv_aligned16(a) && mnv_aligned16(b) &&
+             e.lda % 4 == 0 && e.ldb % 4 == 0;
   const SgemmPlan plan = plan_sgemm(m, n, k, workspace ? workspace_bytes / sizeof(float) : 0);
   const bool small = plan.small;
   const int splits = plan.splits;
@@ -175,6 +184,38 @@ int sgemm_nn_impl(const float* a, const float* b, float* c, int m, int n, int k,
   SgemmNN<false> p = make_sgemm<false>(a, b, c, m, n, k, e);
   return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
                : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
+}
+
+// Operands of 2^29 elements and more (up to the reference's limit, int element counts): the
+// product is cut into panels whose spans fit 32-bit byte offsets -- columns of B and C, rows
+// of A and C, and ranges of k, the later k ranges accumulating into C -- each panel one launch
+// with the whole matrices' leading dimensions.  Slower than one launch (C is re-read per k
+// range, no k ranges over workgroups), and the sum over k is taken range by range.
+const long long kOperandLimit = (1LL << 29) - 1;  // elements a launch can address per operand
+
+bool sgemm_is_large(int m, int n, int k) {
+  return (long long)m * k > kOperandLimit || (long long)k * n > kOperandLimit;
+}
+
+int sgemm_nn_large(const float* a, const float* b, float* c, int m, int n, int k, hipStream_t s) {
+  const long long mc = m < (1 << 28) ? m : (1 << 28);
+  long long kc = (kOperandLimit - mc) / m + 1;          // ((kc-1)*m + mc) <= limit
+  if (kc > k) kc = k;
+  if (kc >= 16) kc -= kc % 16;
+  long long nc = (kOperandLimit - kc) / k + 1;          // ((nc-1)*k + kc) <= limit
+  if (nc > n) nc = n;
+  if (kc < 1 || nc < 1) return MNV_ERR_INVALID;
+  for (long long n0 = 0; n0 < n; n0 += nc)
+    for (long long m0 = 0; m0 < m; m0 += mc)
+      for (long long k0 = 0; k0 < k; k0 += kc) {
+        const int mm = (int)(m - m0 < mc ? m - m0 : mc), nn = (int)(n - n0 < nc ? n - n0 : nc);
+        const int kk = (int)(k - k0 < kc ? k - k0 : kc);
+        SgemmEpilogue e{nullptr, nullptr, 0, m, k, m, k0 > 0};
+        int rc = sgemm_nn_impl(a + (size_t)k0 * m + m0, b + (size_t)n0 * k + k0,
+                               c + (size_t)n0 * m + m0, mm, nn, kk, nullptr, 0, s, e);
+        if (rc) return rc;
+      }
+  return MNV_OK;
 }
 
 }  // namespace
@@ -191,8 +232,11 @@ int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k, 
                  size_t workspace_bytes, mnv_stream_t stream) {
   if (m == 0 || n == 0) return MNV_OK;
   if (!a || !b || !c || m < 0 || n < 0 || k <= 0) return MNV_ERR_INVALID;
-  // operands are addressed through 32-bit buffer offsets: at most 2^31 - 1 bytes each
-  if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
+  // every operand is at most 2^31 - 1 elements (the reference's int element counts)
+  if ((long long)m * k > 0x7fffffffLL || (long long)k * n > 0x7fffffffLL ||
+      (long long)m * n > 0x7fffffffLL)
+    return MNV_ERR_INVALID;
+  if (sgemm_is_large(m, n, k)) return sgemm_nn_large(a, b, c, m, n, k, mnv_stream(stream));
   return sgemm_nn_impl(a, b, c, m, n, k, workspace, workspace_bytes, mnv_stream(stream));
 }
 
