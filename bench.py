@@ -400,33 +400,46 @@ def bandwidth_table(L, dev, rng, ne):
 
 def small_nets(steps=20, warmup=3):
     """BASELINE.json configs[0] (MLP) and configs[3] (CNN) at batch 256: latency-bound
-    graphs, reported as ms/step and operators/step without a roofline claim."""
+    graphs, reported as ms/step and operators/step without a roofline claim.  Beside the
+    one-stream order: the same step in dataflow mode (four streams ordered by events), with
+    the fused operators, and recorded into a HIP graph."""
     from minerva_amd import hostapi
     from minerva_amd import configs
     out = {}
     for name in ("mlp", "cnn"):
         params, data, label = configs.make_inputs(name, BATCH)
-        rt = hostapi.Runtime(0, sync_each_op=False)
-        net = hostapi.Net(rt, name, BATCH)
-        for k, v in params.items():
-            net.set_param(k, v)
-        net.load_batch(data, label)
-        for _ in range(warmup):
-            net.step(0.01)
-        rt.sync()
-        ops0 = rt.ops_issued()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            net.step(0.01)
+        row = {}
+        for mode in ("stream_order", "dataflow", "fused"):
+            rt = hostapi.Runtime(0, sync_each_op=False, dataflow=(mode == "dataflow"))
+            net = hostapi.Net(rt, name, BATCH)
+            if mode == "fused":
+                net.set_fused()
+            for k, v in params.items():
+                net.set_param(k, v)
+            net.load_batch(data, label)
+            for _ in range(warmup):
+                net.step(0.01)
             rt.sync()
-        ms = (time.perf_counter() - t0) * 1e3 / steps
-        out[name + "_b256"] = {"ms_per_step": round(ms, 4), "images_per_s": round(BATCH / ms * 1e3, 1),
-                               "ops_per_step": (rt.ops_issued() - ops0) // steps}
-        out[name + "_b256"]["graph_replay"] = g = graph_replay(rt, net, steps, warmup)
-        log("%s b=%d: %.3f ms/step, recorded step %.3f ms/replay (%d nodes)" %
-            (name, BATCH, ms, g["ms_per_step"], g["nodes"]))
-        net.close()
-        rt.close()
+            ops0 = rt.ops_issued()
+            ts = []
+            for _ in range(steps):
+                t0 = time.perf_counter()
+                net.step(0.01)
+                rt.sync()
+                ts.append((time.perf_counter() - t0) * 1e3)
+            ms = float(np.median(ts))
+            if mode == "stream_order":
+                row = {"ms_per_step": round(ms, 4), "images_per_s": round(BATCH / ms * 1e3, 1),
+                       "ops_per_step": (rt.ops_issued() - ops0) // steps}
+                row["graph_replay"] = g = graph_replay(rt, net, steps, warmup)
+            else:
+                row[mode + "_ms_per_step"] = round(ms, 4)
+            net.close()
+            rt.close()
+        out[name + "_b256"] = row
+        log("%s b=%d: %.3f ms/step (dataflow %.3f, fused %.3f), recorded step %.3f ms/replay (%d nodes)" %
+            (name, BATCH, row["ms_per_step"], row["dataflow_ms_per_step"], row["fused_ms_per_step"],
+             g["ms_per_step"], g["nodes"]))
     return out
 
 
