@@ -18,8 +18,9 @@
 // read twice, the loads of the next channels are issued before the current ones are
 // consumed, and a thread handles several neighbouring positions per access.  Other sizes
 // (and tensors of 2 GiB or more) take the generic kernels, which re-read the value that
-// leaves the window and the one needed for the output (cache hits).  All accesses are
-// ordinary: non-temporal 4-byte stores measured 35% slower here.
+// leaves the window and the one needed for the output (cache hits).  Planes of 512 positions
+// and more that do not lie on 64-byte boundaries take variants of the ring kernels whose
+// stores are re-cut on those boundaries (lrn_store_recut below).
 #include <math.h>
 
 #include <algorithm>
@@ -37,8 +38,13 @@ namespace {
 
 #define MNV_LRN_THREADS 256
 
-// s^e for s >= 1 through the hardware log2 / exp2: relative error ~1e-6
-__device__ __forceinline__ float pow_ge1(float s, float e) { return __expf(e * __logf(s)); }
+// s^e for s >= 1 through the hardware log2 / exp2 instructions themselves (v_log_f32,
+// v_exp_f32: 1 ulp each; relative error of the power ~1e-6).  The library wrappers add range
+// fix-ups for denormal arguments and results (five more instructions per value), which
+// cannot occur here: s >= 1, and s^e underflows only for |e| log2 s > 126.
+__device__ __forceinline__ float pow_ge1(float s, float e) {
+  return __builtin_amdgcn_exp2f(e * __builtin_amdgcn_logf(s));
+}
 
 __global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_fwd_kernel(
     const float* __restrict__ bottom, float* __restrict__ scale, float* __restrict__ top,
@@ -161,7 +167,74 @@ __device__ __forceinline__ void lrn_store(mnv_rsrc r, unsigned voff, unsigned so
   }
 }
 
-template <int SIZE, int G, int V, bool NT>
+// ---- stores re-cut on 64-byte boundaries ------------------------------------------------
+// An odd plane size (55 x 55) leaves every channel at a different offset from a 64-byte
+// boundary, and a wavefront's run of 64 * V floats then begins and ends inside a 64-byte
+// sector that a neighbouring wavefront completes later: both write that sector in part, and
+// the memory side pays a read-modify-write for each.  Re-cutting the run inside the
+// wavefront does not help by itself (the partial sectors at its two ends stay).  What helps
+// is ownership by sector: the runs of neighbouring wavefronts overlap by 16 positions
+// (a wavefront covers 64 * V positions and advances by 64 * V - 16; the 16 shared positions
+// are computed twice), and in every channel a wavefront writes exactly the sectors that
+// BEGIN inside the first 64 * V - 16 positions of its run, whole, wherever the sector grid
+// falls in that channel.  Measured on 256 x 96 x 55 x 55 with the arithmetic taken out:
+// 213 -> 178 us for one tensor read and two written.
+// The values travel through a strip of LDS that belongs to the wavefront (a wavefront's LDS
+// accesses are executed in order, so no workgroup barrier is needed).  Only the sector that
+// holds the first floats of a plane and the one that holds its last floats are written
+// element by element.
+#define MNV_LRN_STRIP (64 * 4 + 16)  // floats per wavefront and stream
+#define MNV_LRN_RECUT_MIN_PLANE 512   // positions per plane from which the re-cut kernels run
+template <int V>
+struct LrnRecut {
+  static constexpr int RUN = 64 * V;        // positions a wavefront covers
+  static constexpr int OWN = RUN - 16;      // positions it advances by
+  static constexpr int LANES = OWN / 4;     // lanes that store one 16-byte vector
+};
+// r: floats from the wavefront's first position to the first sector boundary at or after it in
+// this channel (wavefront-uniform); pw: first position of the wavefront in its plane;
+// voff: the lane's own byte offset (image, position pw + V * lane); soff: channel byte offset.
+template <int V, bool NT>
+__device__ __forceinline__ void lrn_store_recut(float* strip, int r, mnv_rsrc rs, unsigned voff,
+                                                unsigned soff, const float (&val)[V], int lane,
+                                                int pw, int hw) {
+#pragma unroll
+  for (int t = 0; t < V; ++t) strip[V * lane + t] = val[t];
+  __builtin_amdgcn_wave_barrier();
+  const unsigned vbase = voff - (unsigned)(4 * V * lane);  // byte offset of position pw
+  if (lane < LrnRecut<V>::LANES) {
+    const int e = r + 4 * lane, t = pw + e;
+    if (t < hw) {
+      float o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = strip[e + j];
+      if (t + 4 <= hw) {
+        mnv_f4 v = {o[0], o[1], o[2], o[3]};
+        __builtin_amdgcn_raw_buffer_store_b128(
+            __builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned, v), rs,
+            (int)(vbase + 4u * e), (int)soff, NT ? 2 : 0);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (t + j < hw)
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, o[j]), rs,
+                                                  (int)(vbase + 4u * (e + j)), (int)soff, 0);
+      }
+    }
+  } else if (pw == 0) {
+    // the floats of the plane in front of its first sector boundary
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = 4 * (lane - LrnRecut<V>::LANES) + j;
+      if (e < r && e < hw)
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, strip[e]), rs,
+                                              (int)(vbase + 4u * e), (int)soff, 0);
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
+template <int SIZE, int G, int V, bool NT, bool RECUT>
 __global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_fwd_ring_kernel(
     const float* __restrict__ bottom, float* __restrict__ scale, float* __restrict__ top,
     float alpha_over_size, float negative_beta, int channels, int hw, int groups_per_image,
@@ -171,43 +244,72 @@ __global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_fwd_ring_kernel(
   const mnv_rsrc rin = mnv_make_rsrc(bottom, bytes), rsc = mnv_make_rsrc(scale, bytes),
                  rtop = mnv_make_rsrc(top, bytes);
   const unsigned cstep = (unsigned)hw * 4u;  // bytes from one channel to the next
+  __shared__ float strips[RECUT ? 2 * (MNV_LRN_THREADS / 64) * MNV_LRN_STRIP : 1];
+  const int lane = threadIdx.x % 64;
+  float* const strip_s = strips + (RECUT ? (threadIdx.x / 64) * 2 * MNV_LRN_STRIP : 0);
+  float* const strip_t = strip_s + (RECUT ? MNV_LRN_STRIP : 0);
+  // floats from a 64-byte boundary to the first element of each output tensor
+  const int phase_s = (int)((reinterpret_cast<uintptr_t>(scale) >> 2) & 15u);
+  const int phase_t = (int)((reinterpret_cast<uintptr_t>(top) >> 2) & 15u);
   // A thread walks the channels [c0, c1) of one segment for V neighbouring positions: the
   // channel range is cut into nseg segments when the positions alone do not fill the chip
   // (13 x 13 planes with 256 channels); a segment starts its window sum afresh pre_pad
   // channels early.
-  for (size_t q = (size_t)blockIdx.x * MNV_LRN_THREADS + threadIdx.x; q < groups * nseg;
-       q += (size_t)gridDim.x * MNV_LRN_THREADS) {
-    const int seg = mnv_fastdiv((int)q, d_groups), qq = (int)q - seg * (int)groups;
-    const int n = mnv_fastdiv(qq, d_gpi), p0 = (qq - n * groups_per_image) * V;
+  // Workgroups never straddle channel segments (the thread columns of a segment are padded to
+  // whole workgroups), so the segment, and with it every channel offset, is a scalar: a
+  // channel offset that the compiler cannot prove uniform costs a readfirstlane loop around
+  // every buffer access.  RECUT: the workgroups of one run of positions (one per segment) are
+  // neighbours in launch order; otherwise segments are the slow index.  d_groups divides by
+  // nseg (RECUT) or by the workgroups of a segment.
+  const int bps = (int)((groups + MNV_LRN_THREADS - 1) / MNV_LRN_THREADS);
+  for (int vb = blockIdx.x; vb < bps * nseg; vb += gridDim.x) {
+    int seg, blk;
+    if (RECUT) {
+      blk = mnv_fastdiv(vb, d_groups);
+      seg = vb - blk * nseg;
+    } else {
+      seg = mnv_fastdiv(vb, d_groups);
+      blk = vb - seg * bps;
+    }
+    // RECUT: a "group" is a lane of a wavefront of its plane (groups_per_image = 64 x the
+    // wavefronts of a plane), wavefronts advance by OWN positions, image and wavefront are
+    // scalars
+    const int wave0 = blk * MNV_LRN_THREADS + __builtin_amdgcn_readfirstlane((int)threadIdx.x / 64) * 64;
+    const int qq = RECUT ? wave0 + lane : blk * MNV_LRN_THREADS + (int)threadIdx.x;
+    if (RECUT ? wave0 >= (int)groups : qq >= (int)groups) continue;
+    const int n = RECUT ? mnv_fastdiv(wave0, d_gpi) : mnv_fastdiv(qq, d_gpi);
+    const int gi = qq - n * groups_per_image;
+    const int pw = RECUT ? (wave0 - n * groups_per_image) / 64 * LrnRecut<V>::OWN : 0;
+    const int p0 = RECUT ? pw + V * lane : gi * V;
     const int valid = min(V, hw - p0);
     const unsigned voff = ((unsigned)n * (unsigned)channels * (unsigned)hw + (unsigned)p0) * 4u;
+    // float index of the wavefront's first position in channel 0 of its image
+    const int wave_first = RECUT ? n * channels * hw + pw : 0;
     const int c0 = seg * seg_len, c1 = min(channels, c0 + seg_len);
     const int h_start = c0 - pre_pad, h_end = min(channels, c1 + post_pad);
-    LrnVec<V> win[SIZE], nxt[G];
+    // Two register sets take turns as "current group" and "group being loaded" (the loop is
+    // unrolled by two), so that no value is copied from one to the other.
+    LrnVec<V> win[SIZE], set_a[G], set_b[G];
 #pragma unroll
     for (int u = 0; u < SIZE; ++u)
 #pragma unroll
       for (int t = 0; t < V; ++t) win[u].v[t] = 0.f;
-    auto fetch = [&](int h, int u) {
+    auto fetch = [&](LrnVec<V>(&dst)[G], int h, int u) {
       if (h >= 0 && h < h_end) {
-        nxt[u] = lrn_load<V>(rin, voff, (unsigned)h * cstep);
+        dst[u] = lrn_load<V>(rin, voff, (unsigned)h * cstep);
       } else {
 #pragma unroll
-        for (int t = 0; t < V; ++t) nxt[u].v[t] = 0.f;
+        for (int t = 0; t < V; ++t) dst[u].v[t] = 0.f;
       }
     };
 #pragma unroll
-    for (int u = 0; u < G; ++u) fetch(h_start + u, u);
+    for (int u = 0; u < G; ++u) fetch(set_a, h_start + u, u);
     float accum[V];
 #pragma unroll
     for (int t = 0; t < V; ++t) accum[t] = 0.f;
-    for (int h0 = h_start; h0 < c1 + post_pad; h0 += G) {
-      LrnVec<V> cur[G];
+    auto group = [&](LrnVec<V>(&cur)[G], LrnVec<V>(&nxt)[G], int h0) {
 #pragma unroll
-      for (int u = 0; u < G; ++u) {
-        cur[u] = nxt[u];
-        fetch(h0 + G + u, u);
-      }
+      for (int u = 0; u < G; ++u) fetch(nxt, h0 + G + u, u);
 #pragma unroll
       for (int u = 0; u < G; ++u) {
         const int c = h0 + u - post_pad;
@@ -224,16 +326,29 @@ __global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_fwd_ring_kernel(
             s[t] = 1.f + accum[t] * alpha_over_size;
             o[t] = win[(u - post_pad + SIZE) % SIZE].v[t] * pow_ge1(s[t], negative_beta);
           }
-          lrn_store<V, NT>(rsc, voff, (unsigned)c * cstep, s, valid);
-          lrn_store<V, NT>(rtop, voff, (unsigned)c * cstep, o, valid);
+          if (RECUT) {
+            const int first = wave_first + c * hw;
+            lrn_store_recut<V, NT>(strip_s, (16 - ((first + phase_s) & 15)) & 15, rsc, voff,
+                                   (unsigned)c * cstep, s, lane, pw, hw);
+            lrn_store_recut<V, NT>(strip_t, (16 - ((first + phase_t) & 15)) & 15, rtop, voff,
+                                   (unsigned)c * cstep, o, lane, pw, hw);
+          } else {
+            lrn_store<V, NT>(rsc, voff, (unsigned)c * cstep, s, valid);
+            lrn_store<V, NT>(rtop, voff, (unsigned)c * cstep, o, valid);
+          }
         }
       }
+    };
+    const int h_last = c1 + post_pad;
+    for (int h0 = h_start; h0 < h_last; h0 += 2 * G) {
+      group(set_a, set_b, h0);
+      if (h0 + G < h_last) group(set_b, set_a, h0 + G);
     }
   }
 }
 
-template <int SIZE, int G, int V>
-__global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_bwd_ring_kernel(
+template <int SIZE, int G, int V, bool NT, bool RECUT>
+__global__ __launch_bounds__(MNV_LRN_THREADS, (SIZE <= 5 && !RECUT) ? 4 : 1) void mnv_lrn_bwd_ring_kernel(
     const float* __restrict__ bottom, const float* __restrict__ top,
     const float* __restrict__ scale, const float* __restrict__ top_diff,
     float* __restrict__ bottom_diff, float negative_beta, float cache_ratio, int channels, int hw,
@@ -245,75 +360,112 @@ __global__ __launch_bounds__(MNV_LRN_THREADS) void mnv_lrn_bwd_ring_kernel(
                  rs = mnv_make_rsrc(scale, bytes), rdy = mnv_make_rsrc(top_diff, bytes),
                  rdx = mnv_make_rsrc(bottom_diff, bytes);
   const unsigned cstep = (unsigned)hw * 4u;
-  for (size_t q = (size_t)blockIdx.x * MNV_LRN_THREADS + threadIdx.x; q < groups * nseg;
-       q += (size_t)gridDim.x * MNV_LRN_THREADS) {
-    const int seg = mnv_fastdiv((int)q, d_groups), qq = (int)q - seg * (int)groups;
-    const int n = mnv_fastdiv(qq, d_gpi), p0 = (qq - n * groups_per_image) * V;
+  __shared__ float strips[RECUT ? (MNV_LRN_THREADS / 64) * MNV_LRN_STRIP : 1];
+  const int lane = threadIdx.x % 64;
+  float* const strip = strips + (RECUT ? (threadIdx.x / 64) * MNV_LRN_STRIP : 0);
+  const int phase = (int)((reinterpret_cast<uintptr_t>(bottom_diff) >> 2) & 15u);
+  // Workgroups never straddle channel segments (the thread columns of a segment are padded to
+  // whole workgroups), so the segment, and with it every channel offset, is a scalar: a
+  // channel offset that the compiler cannot prove uniform costs a readfirstlane loop around
+  // every buffer access.  RECUT: the workgroups of one run of positions (one per segment) are
+  // neighbours in launch order; otherwise segments are the slow index.  d_groups divides by
+  // nseg (RECUT) or by the workgroups of a segment.
+  const int bps = (int)((groups + MNV_LRN_THREADS - 1) / MNV_LRN_THREADS);
+  for (int vb = blockIdx.x; vb < bps * nseg; vb += gridDim.x) {
+    int seg, blk;
+    if (RECUT) {
+      blk = mnv_fastdiv(vb, d_groups);
+      seg = vb - blk * nseg;
+    } else {
+      seg = mnv_fastdiv(vb, d_groups);
+      blk = vb - seg * bps;
+    }
+    // RECUT: a "group" is a lane of a wavefront of its plane (groups_per_image = 64 x the
+    // wavefronts of a plane), wavefronts advance by OWN positions, image and wavefront are
+    // scalars
+    const int wave0 = blk * MNV_LRN_THREADS + __builtin_amdgcn_readfirstlane((int)threadIdx.x / 64) * 64;
+    const int qq = RECUT ? wave0 + lane : blk * MNV_LRN_THREADS + (int)threadIdx.x;
+    if (RECUT ? wave0 >= (int)groups : qq >= (int)groups) continue;
+    const int n = RECUT ? mnv_fastdiv(wave0, d_gpi) : mnv_fastdiv(qq, d_gpi);
+    const int gi = qq - n * groups_per_image;
+    const int pw = RECUT ? (wave0 - n * groups_per_image) / 64 * LrnRecut<V>::OWN : 0;
+    const int p0 = RECUT ? pw + V * lane : gi * V;
     const int valid = min(V, hw - p0);
     const unsigned voff = ((unsigned)n * (unsigned)channels * (unsigned)hw + (unsigned)p0) * 4u;
+    const int wave_first = RECUT ? n * channels * hw + pw : 0;
     const int c0 = seg * seg_len, c1 = min(channels, c0 + seg_len);  // this thread's outputs
     const int h_start = c0 - pre_pad, h_end = min(channels, c1 + post_pad);
     // rings: ratio = dy*y/scale (the summed quantity), and dy, scale for the output term
     LrnVec<V> rwin[SIZE], dwin[SIZE], swin[SIZE];
-    LrnVec<V> ndy[G], ny[G], nsc[G], nx[G];  // next group; nx is bottom at the output channel
+    // the next group of channels and the current one, in two register sets that take turns
+    // (loop unrolled by two); x is bottom at the output channel
+    struct Group {
+      LrnVec<V> dy[G], y[G], sc[G], x[G];
+    } set_a, set_b;
 #pragma unroll
     for (int u = 0; u < SIZE; ++u)
 #pragma unroll
       for (int t = 0; t < V; ++t) {
         rwin[u].v[t] = 0.f; dwin[u].v[t] = 0.f; swin[u].v[t] = 1.f;
       }
-    auto fetch = [&](int h, int u) {
+    auto fetch = [&](Group& g, int h, int u) {
       if (h >= 0 && h < h_end) {
-        ndy[u] = lrn_load<V>(rdy, voff, (unsigned)h * cstep);
-        ny[u] = lrn_load<V>(ry, voff, (unsigned)h * cstep);
-        nsc[u] = lrn_load<V>(rs, voff, (unsigned)h * cstep);
+        g.dy[u] = lrn_load<V>(rdy, voff, (unsigned)h * cstep);
+        g.y[u] = lrn_load<V>(ry, voff, (unsigned)h * cstep);
+        g.sc[u] = lrn_load<V>(rs, voff, (unsigned)h * cstep);
       } else {
 #pragma unroll
         for (int t = 0; t < V; ++t) {
-          ndy[u].v[t] = 0.f; ny[u].v[t] = 0.f; nsc[u].v[t] = 1.f;
+          g.dy[u].v[t] = 0.f; g.y[u].v[t] = 0.f; g.sc[u].v[t] = 1.f;
         }
       }
       const int c = h - post_pad;
       if (c >= c0 && c < c1) {
-        nx[u] = lrn_load<V>(rx, voff, (unsigned)c * cstep);
+        g.x[u] = lrn_load<V>(rx, voff, (unsigned)c * cstep);
       } else {
 #pragma unroll
-        for (int t = 0; t < V; ++t) nx[u].v[t] = 0.f;
+        for (int t = 0; t < V; ++t) g.x[u].v[t] = 0.f;
       }
     };
 #pragma unroll
-    for (int u = 0; u < G; ++u) fetch(h_start + u, u);
+    for (int u = 0; u < G; ++u) fetch(set_a, h_start + u, u);
     float accum[V];
 #pragma unroll
     for (int t = 0; t < V; ++t) accum[t] = 0.f;
-    for (int h0 = h_start; h0 < c1 + post_pad; h0 += G) {
-      LrnVec<V> cdy[G], cy[G], csc[G], cx[G];
+    auto group = [&](Group& cur, Group& nxt, int h0) {
 #pragma unroll
-      for (int u = 0; u < G; ++u) {
-        cdy[u] = ndy[u]; cy[u] = ny[u]; csc[u] = nsc[u]; cx[u] = nx[u];
-        fetch(h0 + G + u, u);
-      }
+      for (int u = 0; u < G; ++u) fetch(nxt, h0 + G + u, u);
 #pragma unroll
       for (int u = 0; u < G; ++u) {
         const int c = h0 + u - post_pad;
         LrnVec<V> r;
 #pragma unroll
         for (int t = 0; t < V; ++t) {
-          r.v[t] = cdy[u].v[t] * cy[u].v[t] / csc[u].v[t];  // 0 past the last channel
+          // 0 past the last channel; scale >= 1, and the hardware reciprocal is good to 1 ulp
+          r.v[t] = cur.dy[u].v[t] * cur.y[u].v[t] * __builtin_amdgcn_rcpf(cur.sc[u].v[t]);
           accum[t] += r.v[t];
           accum[t] -= rwin[u % SIZE].v[t];
         }
-        rwin[u % SIZE] = r; dwin[u % SIZE] = cdy[u]; swin[u % SIZE] = csc[u];
+        rwin[u % SIZE] = r; dwin[u % SIZE] = cur.dy[u]; swin[u % SIZE] = cur.sc[u];
         if (c >= c0 && c < c1) {
           const int slot = (u - post_pad + SIZE) % SIZE;
           float o[V];
 #pragma unroll
           for (int t = 0; t < V; ++t)
             o[t] = dwin[slot].v[t] * pow_ge1(swin[slot].v[t], negative_beta) -
-                   cache_ratio * cx[u].v[t] * accum[t];
-          lrn_store<V, false>(rdx, voff, (unsigned)c * cstep, o, valid);
+                   cache_ratio * cur.x[u].v[t] * accum[t];
+          if (RECUT)
+            lrn_store_recut<V, NT>(strip, (16 - ((wave_first + c * hw + phase) & 15)) & 15, rdx, voff,
+                                   (unsigned)c * cstep, o, lane, pw, hw);
+          else
+            lrn_store<V, false>(rdx, voff, (unsigned)c * cstep, o, valid);
         }
       }
+    };
+    const int h_last = c1 + post_pad;
+    for (int h0 = h_start; h0 < h_last; h0 += 2 * G) {
+      group(set_a, set_b, h0);
+      if (h0 + G < h_last) group(set_b, set_a, h0 + G);
     }
   }
 }
@@ -336,6 +488,19 @@ void lrn_segments(size_t groups, int channels, int size, int* seg_len, int* nseg
   const size_t max_n = (size_t)std::max(1, channels / (4 * size));
   if (n > max_n) n = max_n;
   *seg_len = (int)((channels + n - 1) / n);
+  *nseg = (channels + *seg_len - 1) / *seg_len;
+}
+
+// The re-cut kernels run best on short segments, whose workgroups are neighbours in launch
+// order: the workgroups in residence then stream through a compact part of the tensors
+// (a few dozen images), much as a plain copy does, and the halo channels a segment re-reads
+// were fetched by its neighbour a moment ago.  Measured on 256 x 96 x 55 x 55 (forward, 4 / 8 /
+// 16 / 24 segments: 191 / 175 / 157 / 166 us) and 256 x 256 x 27 x 27 (16 / 32 / 43: 125 / 111 /
+// 109 us); the backward pass re-reads three tensors per halo channel and pays for the ratio
+// of every halo value, so its segments stay longer (4 / 6 / 8 / 16 segments of the first
+// shape: 288 / 278 / 287 / 302 us).
+void lrn_short_segments(int channels, int len, int* seg_len, int* nseg) {
+  *seg_len = std::min(channels, len);
   *nseg = (channels + *seg_len - 1) / *seg_len;
 }
 
@@ -362,24 +527,34 @@ int mnv_lrn_fwd(const float* bottom, float* scale, float* top, int local_size, f
   const float aos = alpha / local_size;
   const size_t bytes = positions * channels * sizeof(float);
   constexpr int V = 4;
-  const int gpi = (hw + V - 1) / V;
+  // Planes of 512 positions and more have their stores re-cut on 64-byte boundaries (see
+  // lrn_store_recut) unless they lie on such boundaries already; on smaller planes the
+  // wavefronts that hang over the end of a plane would idle too many lanes.
+  const bool recut = hw >= MNV_LRN_RECUT_MIN_PLANE && (hw % 16 != 0 || ((reinterpret_cast<uintptr_t>(scale) |
+                                                     reinterpret_cast<uintptr_t>(top)) & 63u));
+  const int gpi = recut ? 64 * ((hw + LrnRecut<V>::OWN - 1) / LrnRecut<V>::OWN) : (hw + V - 1) / V;
   const size_t groups = (size_t)gpi * num_images;
-  const bool ring = bytes < 0x80000000ull && (local_size == 3 || local_size == 5 || local_size == 7);
+  const bool ring = bytes < 0x80000000ull && (local_size == 3 || local_size == 5 || local_size == 7) &&
+                    groups * (size_t)channels < 0x7fffffffull;
   if (ring) {
     int seg_len, nseg;
     lrn_segments(groups, channels, local_size, &seg_len, &nseg);
-    const dim3 grid(lrn_grid(groups * nseg));
-    const MnvFastDiv d = mnv_fastdiv_make(gpi), dg = mnv_fastdiv_make((int)groups);
+    if (recut) lrn_short_segments(channels, std::max(6, local_size + 1), &seg_len, &nseg);
+    const size_t bps = mnv_ceil_div(groups, MNV_LRN_THREADS);
+    const dim3 grid((unsigned)std::min<size_t>(bps * nseg, 4 * MNV_MAX_STREAM_BLOCKS));
+    const MnvFastDiv d = mnv_fastdiv_make(gpi), dg = mnv_fastdiv_make(recut ? nseg : (int)bps);
     const bool nt = 3 * bytes >= ((size_t)512 << 20);
+#define MNV_LRN_FWD_(SIZE, G, NT, RECUT)                                                           \
+  hipLaunchKernelGGL((mnv_lrn_fwd_ring_kernel<SIZE, G, V, NT, RECUT>), grid, block, 0, s, bottom,  \
+                     scale, top, aos, -beta, channels, hw, gpi, groups, (unsigned)bytes, d,        \
+                     seg_len, nseg, dg)
 #define MNV_LRN_FWD(SIZE, G)                                                                        \
-  if (nt)                                                                                           \
-    hipLaunchKernelGGL((mnv_lrn_fwd_ring_kernel<SIZE, G, V, true>), grid, block, 0, s, bottom,      \
-                       scale, top, aos, -beta, channels, hw, gpi, groups, (unsigned)bytes, d,       \
-                       seg_len, nseg, dg);                                                          \
+  if (recut) {                                                                                      \
+    if (nt) MNV_LRN_FWD_(SIZE, G, true, true); else MNV_LRN_FWD_(SIZE, G, false, true);             \
+  } else if (nt)                                                                                    \
+    MNV_LRN_FWD_(SIZE, G, true, false);                                                             \
   else                                                                                              \
-    hipLaunchKernelGGL((mnv_lrn_fwd_ring_kernel<SIZE, G, V, false>), grid, block, 0, s, bottom,     \
-                       scale, top, aos, -beta, channels, hw, gpi, groups, (unsigned)bytes, d,       \
-                       seg_len, nseg, dg)
+    MNV_LRN_FWD_(SIZE, G, false, false)
     if (local_size == 3) {
       MNV_LRN_FWD(3, 6);
     } else if (local_size == 5) {
@@ -388,6 +563,7 @@ int mnv_lrn_fwd(const float* bottom, float* scale, float* top, int local_size, f
       MNV_LRN_FWD(7, 7);
     }
 #undef MNV_LRN_FWD
+#undef MNV_LRN_FWD_
   } else {
     hipLaunchKernelGGL(mnv_lrn_fwd_kernel, dim3(lrn_grid(positions)), block, 0, s, bottom, scale, top,
                        local_size, aos, -beta, channels, hw, positions, mnv_fastdiv_make(hw));
@@ -408,22 +584,37 @@ int mnv_lrn_bwd(const float* bottom, const float* top, const float* scale, const
   const float ratio = (float)(2. * alpha * beta / local_size);
   const size_t bytes = positions * channels * sizeof(float);
   constexpr int V = 2;
-  const int gpi = (hw + V - 1) / V;
+  const bool recut = hw >= MNV_LRN_RECUT_MIN_PLANE && (hw % 16 != 0 || (reinterpret_cast<uintptr_t>(bottom_diff) & 63u));
+  const int gpi = recut ? 64 * ((hw + LrnRecut<V>::OWN - 1) / LrnRecut<V>::OWN) : (hw + V - 1) / V;
   const size_t groups = (size_t)gpi * num_images;
-  const bool ring = bytes < 0x80000000ull && (local_size == 3 || local_size == 5 || local_size == 7);
+  const bool ring = bytes < 0x80000000ull && (local_size == 3 || local_size == 5 || local_size == 7) &&
+                    groups * (size_t)channels < 0x7fffffffull;
   if (ring) {
     int seg_len, nseg;
     lrn_segments(groups, channels, local_size, &seg_len, &nseg);
-    const dim3 grid(lrn_grid(groups * nseg));
-    const MnvFastDiv d = mnv_fastdiv_make(gpi), dg = mnv_fastdiv_make((int)groups);
-#define MNV_LRN_BWD(SIZE, G)                                                                     \
-  hipLaunchKernelGGL((mnv_lrn_bwd_ring_kernel<SIZE, G, V>), grid, block, 0, s, bottom, top, scale, \
-                     top_diff, bottom_diff, -beta, ratio, channels, hw, gpi, groups,             \
+    if (recut) lrn_short_segments(channels, 16, &seg_len, &nseg);
+    const size_t bps = mnv_ceil_div(groups, MNV_LRN_THREADS);
+    const dim3 grid((unsigned)std::min<size_t>(bps * nseg, 4 * MNV_MAX_STREAM_BLOCKS));
+    const MnvFastDiv d = mnv_fastdiv_make(gpi), dg = mnv_fastdiv_make(recut ? nseg : (int)bps);
+    const bool nt = 5 * bytes >= ((size_t)512 << 20);
+#define MNV_LRN_BWD_(SIZE, G, NT, RECUT)                                                         \
+  hipLaunchKernelGGL((mnv_lrn_bwd_ring_kernel<SIZE, G, V, NT, RECUT>), grid, block, 0, s, bottom, \
+                     top, scale, top_diff, bottom_diff, -beta, ratio, channels, hw, gpi, groups, \
                      (unsigned)bytes, d, seg_len, nseg, dg)
-    if (local_size == 3) MNV_LRN_BWD(3, 6);
-    else if (local_size == 5) MNV_LRN_BWD(5, 5);
-    else MNV_LRN_BWD(7, 7);
+#define MNV_LRN_BWD(SIZE, G)                                                                     \
+  if (recut) {                                                                                   \
+    if (nt) MNV_LRN_BWD_(SIZE, G, true, true); else MNV_LRN_BWD_(SIZE, G, false, true);          \
+  } else                                                                                         \
+    MNV_LRN_BWD_(SIZE, G, false, false)
+    if (local_size == 3) {
+      MNV_LRN_BWD(3, 6);
+    } else if (local_size == 5) {
+      MNV_LRN_BWD(5, 5);
+    } else {
+      MNV_LRN_BWD(7, 7);
+    }
 #undef MNV_LRN_BWD
+#undef MNV_LRN_BWD_
   } else {
     hipLaunchKernelGGL(mnv_lrn_bwd_kernel, dim3(lrn_grid(positions)), block, 0, s, bottom, top, scale,
                        top_diff, bottom_diff, local_size, -beta, ratio, channels, hw, positions,

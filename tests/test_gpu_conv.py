@@ -322,6 +322,8 @@ LRN = [
     (3, 20, 55, 55, 5, 1e-4, 0.75),   # odd planes: whole wavefronts re-cut their runs, others straddle planes
     (2, 33, 31, 33, 3, 1e-2, 0.75),   # every channel starts at a different offset from a 64-byte boundary
     (2, 24, 28, 28, 7, 1e-2, 0.75),   # planes that start on 64-byte boundaries
+    (2, 24, 25, 23, 7, 1e-2, 0.75),   # window of 7 on odd planes: re-cut stores, segments of 8 / 16 channels
+    (3, 5, 41, 37, 5, 1e-2, 0.75),    # fewer channels than a segment, seven wavefronts per plane
 ]
 
 
