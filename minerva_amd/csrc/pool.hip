@@ -26,7 +26,9 @@
 
 namespace {
 
+#ifndef MNV_POOL_THREADS
 #define MNV_POOL_THREADS 256
+#endif
 #define MNV_POOL_XV 8  // 16-byte vectors of plane data a thread holds for the next group
 #define MNV_POOL_DV 4  // ... of top_diff
 #define MNV_POOL_X_FLOATS (MNV_POOL_THREADS * 4 * MNV_POOL_XV)

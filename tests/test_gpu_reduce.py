@@ -148,7 +148,10 @@ def test_softmax_channel(gpu, ora, n, c, h, w):
 
 @pytest.mark.parametrize("m,n", [(1, 1), (3, 4), (64, 64), (65, 63), (1000, 37), (256, 784),
                                  (4096, 9216), (10, 256), (2052, 1500), (1500, 2052),
-                                 (132, 16388)])
+                                 (132, 16388),
+                                 # rows of the result off the 64-byte grid (shifted runs): the last
+                                 # tile reaching past n, both tile sizes, the benchmark's ragged shape
+                                 (256, 8312), (64, 252), (68, 200), (8000, 8200)])
 def test_transpose_bit_exact(gpu, ora, m, n):
     x = _rand(m * n, 27)       # a is {m,n}
     dx, dout = gpu.up(x), gpu.empty(m * n)
@@ -160,6 +163,21 @@ def test_transpose_bit_exact(gpu, ora, m, n):
     dback = gpu.empty(m * n)
     gpu.call("mnv_transpose", dout.p, dback.p, n, m)
     assert_bits_equal(gpu.down(dback), x, "transpose twice")
+
+
+@pytest.mark.parametrize("off", [4, 8, 12])
+def test_transpose_into_a_result_off_the_64_byte_grid(gpu, off):
+    """n % 16 == 0 but c starts `off` floats past a 64-byte boundary: shifted runs again, and
+    nothing may be written in front of or behind the result."""
+    m, n = 260, 2048
+    x = _rand(m * n, 28)
+    dx = gpu.up(x)
+    dout = gpu.up(np.full(m * n + off + 20, np.nan, np.float32))
+    say("transpose into offset", off)
+    gpu.call("mnv_transpose", dx.p, dout.offset(off), m, n)
+    got = gpu.down(dout)
+    assert_bits_equal(got[off:off + m * n], np.ascontiguousarray(x.reshape(n, m).T).ravel(), "transpose")
+    assert np.isnan(got[:off]).all() and np.isnan(got[off + m * n:]).all(), "wrote outside the result"
 
 
 def test_large_operand_paths_8192x8192(gpu):
