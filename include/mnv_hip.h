@@ -343,7 +343,14 @@ int mnv_select(const float* src, float* dst, const int* indices_host, int num_in
  *                              (relu != 0) mnv_relu_fwd
  *   mnv_sgemm_nn_relu_bwd    = mnv_sgemm_nn, then mnv_relu_bwd gated by bottom{m,n}
  *   mnv_sgd_update           = mnv_const_mul(g, scale), then mnv_sub(w, .): w_out = w - scale*g
- * Workspaces are those of the unfused entry points (same *_workspace_bytes). ---- */
+ *   mnv_sgemm_tn             = mnv_transpose(at{k,m} -> a{m,k}), then mnv_sgemm_nn(a, b); with
+ *                              `gate` != NULL followed by mnv_relu_bwd gated by gate{m,n}
+ *                              (the inner-product data gradient W^T * sens of
+ *                              apps/mnist_common.h:258-262, owl/apps/imagenet_alexnet/alexnet.py:96-99)
+ *   mnv_sgemm_nt             = mnv_transpose(bt{n,k} -> b{k,n}), then mnv_sgemm_nn(a, b)
+ *                              (the weight gradient sens * act^T of the same lines)
+ * Workspaces are those of the unfused entry points (same *_workspace_bytes; for the
+ * transposed products mnv_sgemm_nn_workspace_bytes(m, n, k)). ---- */
 int mnv_conv_fwd_relu(const float* bottom, const float* filter, const float* bias, float* top,
                       int num_images, int bottom_num_channels, int top_num_channels,
                       int bottom_height, int bottom_width, int pad_height, int pad_width,
@@ -369,6 +376,10 @@ int mnv_sgemm_nn_relu_bwd(const float* a, const float* b, const float* bottom, f
                           mnv_stream_t stream);
 int mnv_sgd_update(const float* w, const float* g, float scale, float* w_out, size_t n,
                    mnv_stream_t stream);
+int mnv_sgemm_tn(const float* at, const float* b, const float* gate, float* c, int m, int n, int k,
+                 void* workspace, size_t workspace_bytes, mnv_stream_t stream);
+int mnv_sgemm_nt(const float* a, const float* bt, float* c, int m, int n, int k, void* workspace,
+                 size_t workspace_bytes, mnv_stream_t stream);
 
 /* ---- random tensors: CudaPerformRandn / CudaPerformRandBernoulli (cuda_perform.h:66-67).
  * The reference seeds cuRAND from the wall clock per call (cuda.cpp:601,606); here the seed

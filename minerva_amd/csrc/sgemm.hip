@@ -19,16 +19,21 @@ namespace {
 // Period 0 holds every full 16-deep slab: the per-thread byte offsets are fixed and only
 // the uniform slab offset moves.  A k extent that is not a multiple of 16 leaves one
 // partial slab, which is period 1 and gets its own masked offsets.
-template <bool VEC>
+// TA / TB: the operand is given transposed -- A as {k,m} (element (m,k) at k + m*lda), B as
+// {n,k} (element (k,n) at n + k*ldb) -- which only swaps its fetch direction: a transposed A
+// is k-fast, a transposed B x-fast.  The values multiplied and the order they are added in
+// are those of the product of the explicitly transposed matrices.
+template <bool VEC, bool TA = false, bool TB = false>
 struct SgemmNN {
-  static constexpr bool A_KFAST = false, B_KFAST = true;
+  static constexpr bool A_KFAST = TA, B_KFAST = !TB;
   static constexpr int A_NOFF = VEC ? 1 : 4, B_NOFF = VEC ? 1 : 4;
   const float* __restrict__ A;
   const float* __restrict__ B;
   float* __restrict__ C;
   int M, N, K, total_slabs, spp, bk;
-  // Leading dimensions (floats between consecutive columns): m, k, m for whole matrices;
-  // larger when the operands are panels of matrices too large for 32-bit byte offsets.
+  // Leading dimensions (floats between consecutive columns as stored): m, k, m for whole
+  // untransposed matrices (k for a transposed A, n for a transposed B); larger when the
+  // operands are panels of matrices too large for 32-bit byte offsets.
   // accumulate: C += A*B (the k panels after the first).
   int lda, ldb, ldc, accumulate;
   // Fused epilogues (all off for the plain product), applied in this order to the value
@@ -44,32 +49,46 @@ struct SgemmNN {
   struct AState {};
   struct BState {};
   __device__ void make_res(Res& r) const {
-    r.a = mnv_make_rsrc(A, ((unsigned)(K - 1) * (unsigned)lda + (unsigned)M) * 4u);
-    r.b = mnv_make_rsrc(B, ((unsigned)(N - 1) * (unsigned)ldb + (unsigned)K) * 4u);
+    r.a = mnv_make_rsrc(A, TA ? ((unsigned)(M - 1) * (unsigned)lda + (unsigned)K) * 4u
+                              : ((unsigned)(K - 1) * (unsigned)lda + (unsigned)M) * 4u);
+    r.b = mnv_make_rsrc(B, TB ? ((unsigned)(K - 1) * (unsigned)ldb + (unsigned)N) * 4u
+                              : ((unsigned)(N - 1) * (unsigned)ldb + (unsigned)K) * 4u);
   }
   __device__ void a_init(const Res&, AState&, int) const {}
   __device__ void b_init(const Res&, BState&, int) const {}
-  // A[m..m+3, k]: x-fast
+  // A[m..m+3, k] (x-fast) or, transposed, A[m, k..k+3] (k-fast)
   __device__ void a_period(const AState&, unsigned (&off)[A_NOFF], int m, int kl, int period) const {
     const int k = period * spp * bk + kl;
-    const unsigned base = ((unsigned)k * (unsigned)lda + (unsigned)m) * 4u;
+    if (TA) {
+      const unsigned base = ((unsigned)m * (unsigned)lda + (unsigned)k) * 4u;
 #pragma unroll
-    for (int q = 0; q < A_NOFF; ++q) off[q] = ((m + q < M) & (k < K)) ? base + 4u * q : MNV_OOB;
+      for (int q = 0; q < A_NOFF; ++q) off[q] = ((m < M) & (k + q < K)) ? base + 4u * q : MNV_OOB;
+    } else {
+      const unsigned base = ((unsigned)k * (unsigned)lda + (unsigned)m) * 4u;
+#pragma unroll
+      for (int q = 0; q < A_NOFF; ++q) off[q] = ((m + q < M) & (k < K)) ? base + 4u * q : MNV_OOB;
+    }
   }
   __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[A_NOFF], int, int s,
                          int, float (&v)[4]) const {
-    mnv_fetch_vec<A_NOFF>(r.a, off, (unsigned)s * (unsigned)bk * (unsigned)lda * 4u, v);
+    mnv_fetch_vec<A_NOFF>(r.a, off, (unsigned)s * (unsigned)bk * (TA ? 1u : (unsigned)lda) * 4u, v);
   }
-  // B[k..k+3, n]: k-fast
+  // B[k..k+3, n] (k-fast) or, transposed, B[k, n..n+3] (x-fast)
   __device__ void b_period(const BState&, unsigned (&off)[B_NOFF], int n, int kl, int period) const {
     const int k = period * spp * bk + kl;
-    const unsigned base = ((unsigned)n * (unsigned)ldb + (unsigned)k) * 4u;
+    if (TB) {
+      const unsigned base = ((unsigned)k * (unsigned)ldb + (unsigned)n) * 4u;
 #pragma unroll
-    for (int q = 0; q < B_NOFF; ++q) off[q] = ((n < N) & (k + q < K)) ? base + 4u * q : MNV_OOB;
+      for (int q = 0; q < B_NOFF; ++q) off[q] = ((n + q < N) & (k < K)) ? base + 4u * q : MNV_OOB;
+    } else {
+      const unsigned base = ((unsigned)n * (unsigned)ldb + (unsigned)k) * 4u;
+#pragma unroll
+      for (int q = 0; q < B_NOFF; ++q) off[q] = ((n < N) & (k + q < K)) ? base + 4u * q : MNV_OOB;
+    }
   }
   __device__ void b_load(const Res& r, const BState&, const unsigned (&off)[B_NOFF], int, int s,
                          int, float (&v)[4]) const {
-    mnv_fetch_vec<B_NOFF>(r.b, off, (unsigned)s * (unsigned)bk * 4u, v);
+    mnv_fetch_vec<B_NOFF>(r.b, off, (unsigned)s * (unsigned)bk * (TB ? (unsigned)ldb : 1u) * 4u, v);
   }
   size_t extra_lds_bytes() const { return 0; }
   void set_bk(int b) {
@@ -95,13 +114,13 @@ struct SgemmEpilogue {
   int lda = 0, ldb = 0, ldc = 0, accumulate = 0;  // 0: the matrices' own m, k, m
 };
 
-template <bool VEC>
-SgemmNN<VEC> make_sgemm(const float* a, const float* b, float* c, int m, int n, int k,
-                        const SgemmEpilogue& e) {
-  SgemmNN<VEC> p;
+template <bool VEC, bool TA = false, bool TB = false>
+SgemmNN<VEC, TA, TB> make_sgemm(const float* a, const float* b, float* c, int m, int n, int k,
+                                const SgemmEpilogue& e) {
+  SgemmNN<VEC, TA, TB> p;
   p.A = a; p.B = b; p.C = c; p.M = m; p.N = n; p.K = k;
   p.bias = e.bias; p.gate = e.gate; p.relu = e.relu;
-  p.lda = e.lda ? e.lda : m; p.ldb = e.ldb ? e.ldb : k; p.ldc = e.ldc ? e.ldc : m;
+  p.lda = e.lda ? e.lda : (TA ? k : m); p.ldb = e.ldb ? e.ldb : (TB ? n : k); p.ldc = e.ldc ? e.ldc : m;
   p.accumulate = e.accumulate;
   p.set_bk(16);
   return p;
@@ -186,6 +205,24 @@ int sgemm_nn_impl(const float* a, const float* b, float* c, int m, int n, int k,
                : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
 }
 
+// Products with one operand given transposed: same plan (tile shape, k ranges) as the plain
+// product of the same extents, so that the result has the bits of transposing first.
+template <bool TA, bool TB>
+int sgemm_t_impl(const float* a, const float* b, float* c, int m, int n, int k, void* workspace,
+                 size_t workspace_bytes, hipStream_t s, const SgemmEpilogue& e) {
+  const bool vec = mnv_aligned16(a) && mnv_aligned16(b) && (TA ? k % 4 == 0 : m % 4 == 0) &&
+                   (TB ? n % 4 == 0 : k % 4 == 0);
+  const SgemmPlan plan = plan_sgemm(m, n, k, workspace ? workspace_bytes / sizeof(float) : 0);
+  if (vec) {
+    auto p = make_sgemm<true, TA, TB>(a, b, c, m, n, k, e);
+    return plan.small ? mnv_gemm_launch<TileSmall>(p, plan.splits, workspace, s)
+                      : mnv_gemm_launch<TileBig>(p, plan.splits, workspace, s);
+  }
+  auto p = make_sgemm<false, TA, TB>(a, b, c, m, n, k, e);
+  return plan.small ? mnv_gemm_launch<TileSmall>(p, plan.splits, workspace, s)
+                    : mnv_gemm_launch<TileBig>(p, plan.splits, workspace, s);
+}
+
 // Operands of 2^29 elements and more (up to the reference's limit, int element counts): the
 // product is cut into panels whose spans fit 32-bit byte offsets -- columns of B and C, rows
 // of A and C, and ranges of k, the later k ranges accumulating into C -- each panel one launch
@@ -258,6 +295,24 @@ int mnv_sgemm_nn_relu_bwd(const float* a, const float* b, const float* bottom, f
   if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
   return sgemm_nn_impl(a, b, c, m, n, k, workspace, workspace_bytes, mnv_stream(stream),
                        SgemmEpilogue{nullptr, bottom, 0});
+}
+
+int mnv_sgemm_tn(const float* at, const float* b, const float* gate, float* c, int m, int n, int k,
+                 void* workspace, size_t workspace_bytes, mnv_stream_t stream) {
+  if (m == 0 || n == 0) return MNV_OK;
+  if (!at || !b || !c || m < 0 || n < 0 || k <= 0) return MNV_ERR_INVALID;
+  if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
+  return sgemm_t_impl<true, false>(at, b, c, m, n, k, workspace, workspace_bytes, mnv_stream(stream),
+                                   SgemmEpilogue{nullptr, gate, 0});
+}
+
+int mnv_sgemm_nt(const float* a, const float* bt, float* c, int m, int n, int k, void* workspace,
+                 size_t workspace_bytes, mnv_stream_t stream) {
+  if (m == 0 || n == 0) return MNV_OK;
+  if (!a || !bt || !c || m < 0 || n < 0 || k <= 0) return MNV_ERR_INVALID;
+  if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
+  return sgemm_t_impl<false, true>(a, bt, c, m, n, k, workspace, workspace_bytes, mnv_stream(stream),
+                                   SgemmEpilogue{nullptr, nullptr, 0});
 }
 
 int mnv_sgemm_nn_static(const float* a, const float* b, float* c, int m, int n, int k,

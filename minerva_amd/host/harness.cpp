@@ -173,6 +173,12 @@ Tensor RunNamedOp(Runner* rt, const std::string& op, const std::vector<Tensor>& 
   } else if (op == "matmult_relu_backward") {  // inputs: a, b, bottom
     need(3);
     r = rt->MatMultReluBackward(in[0], in[1], in[2]);
+  } else if (op == "matmult_trans_a") {  // inputs: at {k,m}, b {k,n} [, bottom {m,n}]
+    MNV_CHECK(n_inputs == 2 || n_inputs == 3) << "matmult_trans_a takes 2 or 3 inputs";
+    r = n_inputs == 3 ? rt->MatMultTransA(in[0], in[1], in[2]) : rt->MatMultTransA(in[0], in[1]);
+  } else if (op == "matmult_trans_b") {  // inputs: a {m,k}, bt {n,k}
+    need(2);
+    r = rt->MatMultTransB(in[0], in[1]);
   } else if (op == "sgd_update") {  // params: scale; inputs: w, g
     need(2);
     MNV_CHECK(n_params >= 1) << "sgd_update takes the scale";

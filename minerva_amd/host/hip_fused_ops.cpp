@@ -86,6 +86,37 @@ void MatMultReluBackward(const DataList& inputs, const DataList& outputs,
      "sgemm + relu backward");
 }
 
+void MatMultTransA(const DataList& inputs, const DataList& outputs, MatMultTransAClosure&,
+                   const Context& ctx) {
+  MNV_CHECK(inputs.size() == 2u || inputs.size() == 3u) << "(transposed matmult) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(transposed matmult) #outputs is wrong!";
+  int k = inputs[0].size_[0];
+  int m = inputs[0].size_[1];
+  int n = outputs[0].size_[1];
+  MNV_CHECK_EQ(inputs[1].size_[0], k) << "(transposed matmult) inner dimensions differ";
+  const float* gate = nullptr;
+  if (inputs.size() == 3u) {
+    MNV_CHECK(inputs[2].size_ == outputs[0].size_) << "gate and product extents differ";
+    gate = inputs[2].data_;
+  }
+  Ok(mnv_sgemm_tn(inputs[0].data_, inputs[1].data_, gate, outputs[0].data_, m, n, k, ctx.workspace,
+                  ctx.workspace_bytes, ctx.stream),
+     "sgemm, left operand transposed");
+}
+
+void MatMultTransB(const DataList& inputs, const DataList& outputs, MatMultTransBClosure&,
+                   const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 2u) << "(matmult transposed) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(matmult transposed) #outputs is wrong!";
+  int m = inputs[0].size_[0];
+  int k = inputs[0].size_[1];
+  int n = inputs[1].size_[0];
+  MNV_CHECK_EQ(inputs[1].size_[1], k) << "(matmult transposed) inner dimensions differ";
+  Ok(mnv_sgemm_nt(inputs[0].data_, inputs[1].data_, outputs[0].data_, m, n, k, ctx.workspace,
+                  ctx.workspace_bytes, ctx.stream),
+     "sgemm, right operand transposed");
+}
+
 void SgdUpdate(const DataList& inputs, const DataList& outputs, SgdUpdateClosure& c,
                const Context& ctx) {
   MNV_CHECK_EQ(inputs.size(), 2u) << "(sgd update) #inputs is wrong!";

@@ -32,6 +32,12 @@ struct MatMultBiasClosure {
 };
 // out = relu_backward(a * b, bottom); inputs {a, b, bottom}
 struct MatMultReluBackwardClosure {};
+// out = a^T * b, a given as {k,m}; with three inputs {a, b, bottom} the product is gated like
+// MatMultReluBackward: the pair Transpose(a), MatMult[ReluBackward] of an inner product's
+// data gradient
+struct MatMultTransAClosure {};
+// out = a * b^T, b given as {n,k}: Transpose(b), MatMult -- an inner product's weight gradient
+struct MatMultTransBClosure {};
 // out = w - scale * g; inputs {w, g}
 struct SgdUpdateClosure {
   float scale;
@@ -47,6 +53,8 @@ void PoolingBackwardRelu(const DataList&, const DataList&, PoolingBackwardReluCl
 void MatMultBias(const DataList&, const DataList&, MatMultBiasClosure&, const Context&);
 void MatMultReluBackward(const DataList&, const DataList&, MatMultReluBackwardClosure&,
                          const Context&);
+void MatMultTransA(const DataList&, const DataList&, MatMultTransAClosure&, const Context&);
+void MatMultTransB(const DataList&, const DataList&, MatMultTransBClosure&, const Context&);
 void SgdUpdate(const DataList&, const DataList&, SgdUpdateClosure&, const Context&);
 
 }  // namespace hip

@@ -46,6 +46,24 @@ Tensor Net::MatMultReluBackward(const Tensor& a, const Tensor& b, const Tensor& 
   return rt->ReluBackward(rt->MatMult(a, b), act, act);
 }
 
+// The products of an inner product's backward pass, which the reference's applications write
+// as Transpose + MatMult (apps/mnist_common.h:258-262): fused, the transposed operand is read
+// in place.
+Tensor Net::TransMatMult(const Tensor& at, const Tensor& b) {
+  if (fused) return rt->MatMultTransA(at, b);
+  return rt->MatMult(rt->Trans(at), b);
+}
+
+Tensor Net::TransMatMultReluBackward(const Tensor& at, const Tensor& b, const Tensor& act) {
+  if (fused) return rt->MatMultTransA(at, b, act);
+  return rt->ReluBackward(rt->MatMult(rt->Trans(at), b), act, act);
+}
+
+Tensor Net::MatMultTrans(const Tensor& a, const Tensor& bt) {
+  if (fused) return rt->MatMultTransB(a, bt);
+  return rt->MatMult(a, rt->Trans(bt));
+}
+
 // ------------------------------------------------------------------------- MLP
 
 MlpNet::MlpNet(Runner* r, int batch, int in, int hidden, int out)
@@ -68,10 +86,10 @@ void MlpNet::Step(const Tensor& data, const Tensor& label, float lr) {
   results["prob"] = a3;
   // BP
   Tensor s2 = rt->Sub(a3, label);
-  Tensor s1 = MatMultReluBackward(rt->Trans(w1), s2, a1);
-  Tensor gw0 = rt->MatMult(s1, rt->Trans(data));
+  Tensor s1 = TransMatMultReluBackward(w1, s2, a1);
+  Tensor gw0 = MatMultTrans(s1, data);
   Tensor gb0 = rt->Sum(s1, 1);
-  Tensor gw1 = rt->MatMult(s2, rt->Trans(a1));
+  Tensor gw1 = MatMultTrans(s2, a1);
   Tensor gb1 = rt->Sum(s2, 1);
   // update
   Sgd("w0", gw0, lr); Sgd("b0", gb0, lr); Sgd("w1", gw1, lr); Sgd("b1", gb1, lr);
@@ -120,7 +138,7 @@ void CnnNet::Step(const Tensor& data, const Tensor& label, float lr) {
   // BP
   Tensor s8 = rt->Sub(a8, label);
   Tensor s7 = rt->Reshape(s8, Scale{10, b});
-  Tensor s6 = rt->Reshape(rt->MatMult(rt->Trans(params["w2"]), s7), a6->size);
+  Tensor s6 = rt->Reshape(TransMatMult(params["w2"], s7), a6->size);
   Tensor s4, s1;
   if (fused) {
     s4 = rt->PoolingBackwardRelu(s6, a6, a5, pool_info[1]);
@@ -139,7 +157,7 @@ void CnnNet::Step(const Tensor& data, const Tensor& label, float lr) {
   Tensor gb0 = rt->ConvBackwardBias(s1);
   Tensor gw1 = rt->ConvBackwardFilter(s4, a3, params["w1"], conv_info[1]);
   Tensor gb1 = rt->ConvBackwardBias(s4);
-  Tensor gw2 = rt->MatMult(s7, rt->Trans(re6));
+  Tensor gw2 = MatMultTrans(s7, re6);
   Tensor gb2 = rt->Sum(s7, 1);
   Sgd("w0", gw0, lr); Sgd("b0", gb0, lr); Sgd("w1", gw1, lr); Sgd("b1", gb1, lr);
   Sgd("w2", gw2, lr); Sgd("b2", gb2, lr);
@@ -209,15 +227,15 @@ void AlexNet::Step(const Tensor& data, const Tensor& label, float lr) {
   // BP
   sens[11] = rt->Sub(out, label);
   if (drop) {
-    sens[10] = rt->Mult(rt->MatMult(rt->Trans(W(7)), sens[11]), mask7);         // fc8, drop7
+    sens[10] = rt->Mult(TransMatMult(W(7), sens[11]), mask7);         // fc8, drop7
     sens[10] = rt->ReluBackward(sens[10], acts[10], acts[10]);                  // relu7
-    sens[9] = rt->Mult(rt->MatMult(rt->Trans(W(6)), sens[10]), mask6);          // fc7, drop6
+    sens[9] = rt->Mult(TransMatMult(W(6), sens[10]), mask6);          // fc7, drop6
     sens[9] = rt->ReluBackward(sens[9], acts[9], acts[9]);                      // relu6
   } else {
-    sens[10] = MatMultReluBackward(rt->Trans(W(7)), sens[11], acts[10]);        // fc8, relu7
-    sens[9] = MatMultReluBackward(rt->Trans(W(6)), sens[10], acts[9]);          // fc7, relu6
+    sens[10] = TransMatMultReluBackward(W(7), sens[11], acts[10]);        // fc8, relu7
+    sens[9] = TransMatMultReluBackward(W(6), sens[10], acts[9]);          // fc7, relu6
   }
-  sens[8] = rt->Reshape(rt->MatMult(rt->Trans(W(5)), sens[9]), acts[8]->size);
+  sens[8] = rt->Reshape(TransMatMult(W(5), sens[9]), acts[8]->size);
   sens[7] = PoolBackwardRelu(sens[8], acts[8], acts[7], poolings[2]);
   sens[6] = ConvBackwardDataRelu(sens[7], acts[6], W(4), convs[4]);
   sens[5] = ConvBackwardDataRelu(sens[6], acts[5], W(3), convs[3]);
@@ -226,9 +244,9 @@ void AlexNet::Step(const Tensor& data, const Tensor& label, float lr) {
   sens[2] = rt->ConvBackwardData(sens[3], acts[2], W(1), convs[1]);
   sens[1] = PoolBackwardRelu(sens[2], acts[2], acts[1], poolings[0]);
   Tensor gw[8], gb[8];
-  gw[7] = rt->MatMult(sens[11], rt->Trans(acts[10]));
-  gw[6] = rt->MatMult(sens[10], rt->Trans(acts[9]));
-  gw[5] = rt->MatMult(sens[9], rt->Trans(re8));
+  gw[7] = MatMultTrans(sens[11], acts[10]);
+  gw[6] = MatMultTrans(sens[10], acts[9]);
+  gw[5] = MatMultTrans(sens[9], re8);
   gw[4] = rt->ConvBackwardFilter(sens[7], acts[6], W(4), convs[4]);
   gw[3] = rt->ConvBackwardFilter(sens[6], acts[5], W(3), convs[3]);
   gw[2] = rt->ConvBackwardFilter(sens[5], acts[4], W(2), convs[2]);

@@ -46,6 +46,9 @@ class Net {
   Tensor PoolBackwardRelu(const Tensor& diff, const Tensor& top, const Tensor& bottom, PoolingInfo info);
   Tensor Fc(const Tensor& w, const Tensor& x, const Tensor& b, bool relu);
   Tensor MatMultReluBackward(const Tensor& a, const Tensor& b, const Tensor& act);
+  Tensor TransMatMult(const Tensor& at, const Tensor& b);
+  Tensor TransMatMultReluBackward(const Tensor& at, const Tensor& b, const Tensor& act);
+  Tensor MatMultTrans(const Tensor& a, const Tensor& bt);
   Runner* rt;
   int batch_;
 };

@@ -73,6 +73,8 @@ MNV_INSTALL_COMPUTE_FN(ConvBackwardDataReluClosure, hip::ConvBackwardDataRelu)
 MNV_INSTALL_COMPUTE_FN(PoolingBackwardReluClosure, hip::PoolingBackwardRelu)
 MNV_INSTALL_COMPUTE_FN(MatMultBiasClosure, hip::MatMultBias)
 MNV_INSTALL_COMPUTE_FN(MatMultReluBackwardClosure, hip::MatMultReluBackward)
+MNV_INSTALL_COMPUTE_FN(MatMultTransAClosure, hip::MatMultTransA)
+MNV_INSTALL_COMPUTE_FN(MatMultTransBClosure, hip::MatMultTransB)
 MNV_INSTALL_COMPUTE_FN(SgdUpdateClosure, hip::SgdUpdate)
 MNV_INSTALL_DATAGEN_FN(ArrayLoaderClosure, hip::ArrayLoader)
 MNV_INSTALL_DATAGEN_FN(FillClosure, hip::Fill)
@@ -139,6 +141,8 @@ MNV_SIMPLE_OP(SelectOp, ComputeFnWithClosure, SelectClosure, "select")
 MNV_SIMPLE_OP(PoolingBackwardReluOp, ComputeFnWithClosure, PoolingBackwardReluClosure,
               "max pooling bp + relu bp")
 MNV_SIMPLE_OP(MatMultReluBackwardOp, ComputeFnWithClosure, MatMultReluBackwardClosure, "* + relu bp")
+MNV_SIMPLE_OP(MatMultTransAOp, ComputeFnWithClosure, MatMultTransAClosure, "trans * [+ relu bp]")
+MNV_SIMPLE_OP(MatMultTransBOp, ComputeFnWithClosure, MatMultTransBClosure, "* trans")
 MNV_SIMPLE_OP(SgdUpdateOp, ComputeFnWithClosure, SgdUpdateClosure, "sgd update")
 
 class MatMultBiasOp : public ComputeFnWithClosure<MatMultBiasClosure> {

@@ -432,6 +432,23 @@ Tensor Runner::MatMultReluBackward(const Tensor& a, const Tensor& b, const Tenso
   return Compute({a, b, bottom}, bottom->size, std::make_shared<MatMultReluBackwardOp>());
 }
 
+Tensor Runner::MatMultTransA(const Tensor& at, const Tensor& b, const Tensor& bottom) {
+  MNV_CHECK_EQ(at->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(b->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(at->size[0], b->size[0]) << "size must match";
+  const Scale out{at->size[1], b->size[1]};
+  if (!bottom) return Compute({at, b}, out, std::make_shared<MatMultTransAOp>());
+  MNV_CHECK(bottom->size == out) << "gate extent must match the product";
+  return Compute({at, b, bottom}, out, std::make_shared<MatMultTransAOp>());
+}
+
+Tensor Runner::MatMultTransB(const Tensor& a, const Tensor& bt) {
+  MNV_CHECK_EQ(a->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(bt->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(a->size[1], bt->size[1]) << "size must match";
+  return Compute({a, bt}, Scale{a->size[0], bt->size[0]}, std::make_shared<MatMultTransBOp>());
+}
+
 Tensor Runner::SgdUpdate(const Tensor& w, const Tensor& g, float scale) {
   MNV_CHECK_EQ(w->size.Prod(), g->size.Prod()) << "parameter and gradient differ in size";
   auto op = std::make_shared<SgdUpdateOp>();

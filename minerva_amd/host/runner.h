@@ -130,6 +130,10 @@ class Runner : public DeviceListener {
   Tensor MatMultBias(const Tensor& a, const Tensor& b, const Tensor& bias, bool relu);
   // ReluBackward(MatMult(a, b), bottom, bottom)
   Tensor MatMultReluBackward(const Tensor& a, const Tensor& b, const Tensor& bottom);
+  // MatMult(Trans(at), b), or with a gate ReluBackward(MatMult(Trans(at), b), bottom, bottom)
+  Tensor MatMultTransA(const Tensor& at, const Tensor& b, const Tensor& bottom = Tensor());
+  // MatMult(a, Trans(bt))
+  Tensor MatMultTransB(const Tensor& a, const Tensor& bt);
   // Sub(w, ArithmeticConst(g, scale, mult))
   Tensor SgdUpdate(const Tensor& w, const Tensor& g, float scale);
 

@@ -112,6 +112,37 @@ def test_sgemm_fused_epilogues_equal_the_operator_chain(gpu, m, n, k, workspace)
     assert_bits_equal(gpu.down(fused), gpu.down(t1), "sgemm + relu gradient")
 
 
+@pytest.mark.parametrize("m,n,k", [(7, 5, 3), (64, 64, 64), (130, 70, 33), (256, 784, 256), (784, 256, 10),
+                                   (4096, 256, 1000), (1000, 256, 4096), (4096, 9216, 256),
+                                   (9216, 256, 4096), (100, 36, 5000), (132, 260, 68)])
+@pytest.mark.parametrize("workspace", [True, False])
+def test_sgemm_with_a_transposed_operand_equals_transpose_then_sgemm(gpu, m, n, k, workspace):
+    """mnv_sgemm_tn / mnv_sgemm_nt against mnv_transpose followed by mnv_sgemm_nn (and
+    mnv_relu_bwd for the gated form), bit for bit, and against the fp64 product."""
+    a, b = _rand(m * k, 154, 0.1), _rand(k * n, 155)
+    gate = np.maximum(_rand(m * n, 156), 0).astype(np.float32)
+    da, db, dgate = gpu.up(a), gpu.up(b), gpu.up(gate)      # a{m,k}, b{k,n}
+    at, bt = gpu.empty(m * k), gpu.empty(k * n)
+    gpu.call("mnv_transpose", da.p, at.p, m, k)              # at{k,m}
+    gpu.call("mnv_transpose", db.p, bt.p, k, n)              # bt{n,k}
+    prod, gated = gpu.empty(m * n), gpu.empty(m * n)
+    fused = gpu.up(np.full(m * n, np.nan, np.float32))
+    wp, wb, keep = _ws(gpu, "mnv_sgemm_nn_workspace_bytes", (m, n, k), workspace)
+    say("sgemm with transposed operands", m, n, k, workspace)
+    gpu.call("mnv_sgemm_nn", da.p, db.p, prod.p, m, n, k, wp, wb)
+    want = gpu.down(prod)
+    gpu.call("mnv_sgemm_tn", at.p, db.p, None, fused.p, m, n, k, wp, wb)
+    assert_bits_equal(gpu.down(fused), want, "A given transposed")
+    gpu.call("mnv_sgemm_nt", da.p, bt.p, fused.p, m, n, k, wp, wb)
+    assert_bits_equal(gpu.down(fused), want, "B given transposed")
+    gpu.call("mnv_relu_bwd", dgate.p, dgate.p, prod.p, gated.p, ctypes.c_size_t(m * n))
+    gpu.call("mnv_sgemm_tn", at.p, db.p, dgate.p, fused.p, m, n, k, wp, wb)
+    assert_bits_equal(gpu.down(fused), gpu.down(gated), "A given transposed + relu gradient")
+    A = a.reshape(k, m).T.astype(np.float64)
+    B = b.reshape(n, k).T.astype(np.float64)
+    assert normwise(want.reshape(n, m).T, A @ B) <= TOL
+
+
 POOL = [
     # N, C, H, W, sv, sh, kh, kw, ph, pw
     (2, 96, 55, 55, 2, 2, 3, 3, 0, 0),    # AlexNet pool1: ordered scatter, large planes
