@@ -350,6 +350,13 @@ def bandwidth_table(L, dev, rng, ne):
         table.append({"op": name, "ms": round(ms, 4), "gbs": round(gbs, 1),
                       "frac": round(gbs / PEAK_HBM_GBS, 4),
                       "gbs_one_set": round(bpe * ne / (ms_one * 1e-3) / 1e9, 1)})
+    # a ragged transpose in the same operands (8000 x 8200 floats fit an 8192^2 buffer): rows of
+    # the result off the 64-byte grid, partial tiles on both edges
+    rm, rn = 8000, 8200
+    ms = rotating(dev, lambda x, y, z: lambda: L.mnv_transpose(x.p, z.p, rm, rn, S), sets)
+    gbs = 8 * rm * rn / (ms * 1e-3) / 1e9
+    table.append({"op": "transpose 8000x8200", "ms": round(ms, 4), "gbs": round(gbs, 1),
+                  "frac": round(gbs / PEAK_HBM_GBS, 4)})
     add = table[0]
     elt = {"op": "add 8192x8192", "ms": add["ms"], "gbs": add["gbs"],
            "roofline": {"bound": "hbm", "achieved": add["gbs"], "peak": PEAK_HBM_GBS,
