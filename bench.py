@@ -115,10 +115,10 @@ def alexnet_bench(steps, warmup, dataflow=True):
             all_ops = rt.profile_read()
             rt.profile(False)
         graph = None
-        if plain:
+        if plain or mode == "fused":
             graph = graph_replay(rt, net, steps, warmup)
-            log("alexnet b=%d recorded step: %d nodes, %.3f ms/replay" %
-                (BATCH, graph["nodes"], graph["ms_per_step"]))
+            log("alexnet b=%d %s recorded step: %d nodes, %.3f ms/replay" %
+                (BATCH, mode, graph["nodes"], graph["ms_per_step"]))
         out[mode] = {"graph_replay": graph, "ms_per_step": ms, "images_per_s": BATCH / (ms / 1e3),
                      "median_ms_per_step": float(np.median(per_step)),
                      "ops_per_step": ops_per_step,
@@ -634,6 +634,7 @@ def main():
             "fused_epilogues": {"images_per_s": round(res["fused"]["images_per_s"], 1),
                                 "ms_per_step": round(res["fused"]["ms_per_step"], 3),
                                 "ops_per_step": res["fused"]["ops_per_step"],
+                                "graph_replay": res["fused"]["graph_replay"],
                                 "note": "opt-in fused operators, results bit-identical to the "
                                         "operator-by-operator step"},
             "dataflow_4_streams": ({"images_per_s": round(res["dataflow"]["images_per_s"], 1),
