@@ -389,3 +389,47 @@ def test_lrn_batch_256_properties(gpu):
         s = 1.0 + alpha / size * np.sum(X[n, lo:hi + 1, p] ** 2)
         worst = max(worst, abs(top[n, c, p] - X[n, c, p] * s ** (-beta)))
     assert worst <= TOL * np.max(np.abs(top))
+
+
+def test_lrn_benchmark_shape_properties(gpu):
+    """The shape the bandwidth table times (Caffe-style norm1 on conv1's output, batch 256: the
+    re-cut, non-temporal kernels with short channel segments): forward and backward against
+    the closed forms in fp64 on sampled positions, and every element written."""
+    N, C, H, W, size, alpha, beta = 256, 96, 55, 55, 5, 1e-4, 0.75
+    hw, n = H * W, N * C * H * W
+    rng = np.random.default_rng(66)
+    x = (rng.standard_normal(n, dtype=np.float32) * 10).astype(np.float32)
+    dy = rng.standard_normal(n, dtype=np.float32)
+    say("lrn at the benchmark shape")
+    dx_, ds, dt = gpu.up(x), gpu.up(np.full(n, np.nan, np.float32)), gpu.up(np.full(n, np.nan, np.float32))
+    f = ctypes.c_float
+    gpu.call("mnv_lrn_fwd", dx_.p, ds.p, dt.p, size, f(alpha), f(beta), N, C, H, W)
+    top, scale = gpu.down(dt), gpu.down(ds)
+    assert np.isfinite(top).all() and np.isfinite(scale).all(), "an element was not written"
+    ddy, dbd = gpu.up(dy), gpu.up(np.full(n, np.nan, np.float32))
+    gpu.call("mnv_lrn_bwd", dx_.p, dt.p, ds.p, ddy.p, dbd.p, size, f(alpha), f(beta), N, C, H, W)
+    bd = gpu.down(dbd)
+    assert np.isfinite(bd).all(), "an element of the gradient was not written"
+    X = x.reshape(N, C, hw).astype(np.float64)
+    DY = dy.reshape(N, C, hw).astype(np.float64)
+    T, S, B = top.reshape(N, C, hw), scale.reshape(N, C, hw), bd.reshape(N, C, hw)
+    worst_t = worst_s = worst_b = 0.0
+    picks = [(0, 0, 0), (N - 1, C - 1, hw - 1), (1, 0, hw - 1), (0, C - 1, 0), (7, 5, 239), (7, 5, 240),
+             (7, 6, 241), (3, 95, 3024), (200, 47, 1008)]
+    picks += [(int(rng.integers(N)), int(rng.integers(C)), int(rng.integers(hw))) for _ in range(600)]
+    for nn, c, p in picks:
+        lo, hi = max(c - 2, 0), min(c + 2, C - 1)
+        col = X[nn, :, p]
+        sc = 1.0 + alpha / size * np.array([np.sum(col[max(k - 2, 0):min(k + 2, C - 1) + 1] ** 2)
+                                             for k in range(lo, hi + 1)])
+        s_c = sc[c - lo]
+        worst_s = max(worst_s, abs(S[nn, c, p] - s_c) / s_c)
+        worst_t = max(worst_t, abs(T[nn, c, p] - col[c] * s_c ** (-beta)))
+        # bottom_diff = dy * s^-beta - 2 alpha beta / size * x * sum_k dy_k * y_k / s_k over the window
+        yk = col[lo:hi + 1] * sc ** (-beta)
+        acc = np.sum(DY[nn, lo:hi + 1, p] * yk / sc)
+        want = DY[nn, c, p] * s_c ** (-beta) - 2.0 * alpha * beta / size * col[c] * acc
+        worst_b = max(worst_b, abs(B[nn, c, p] - want))
+    assert worst_s <= 1e-6
+    assert worst_t <= TOL * np.max(np.abs(top))
+    assert worst_b <= TOL * np.max(np.abs(bd))
