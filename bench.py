@@ -70,14 +70,16 @@ def alexnet_bench(steps, warmup, dataflow=True):
     out = {}
     # "fused": the same step with the opt-in fused operators (bit-identical results, fewer
     # launches): reported beside `value`, which stays the operator-by-operator step
-    modes = [("per_step_sync", False), ("per_op_sync", True), ("fused", False)]
+    # "fused_updates": the fused step with the weight updates applied in the stores of the
+    # kernels that produce the weight gradients (same parameters, no gradient tensors)
+    modes = [("per_step_sync", False), ("per_op_sync", True), ("fused", False), ("fused_updates", False)]
     if dataflow:  # kernels of different streams overlap: a kernel trace that wants undisturbed
         modes.append(("dataflow", False))  # durations runs with --no-dataflow
     for mode, sync_each in modes:
         rt = hostapi.Runtime(0, sync_each_op=sync_each, dataflow=(mode == "dataflow"))
         net = hostapi.Net(rt, "alexnet", BATCH)
-        if mode == "fused":
-            net.set_fused()
+        if mode in ("fused", "fused_updates"):
+            net.set_fused(updates=(mode == "fused_updates"))
         for k, v in params.items():
             net.set_param(k, v)
         t_h2d = time.perf_counter()
@@ -416,11 +418,11 @@ def small_nets(steps=20, warmup=3):
     for name in ("mlp", "cnn"):
         params, data, label = configs.make_inputs(name, BATCH)
         row = {}
-        for mode in ("stream_order", "dataflow", "fused"):
+        for mode in ("stream_order", "dataflow", "fused", "fused_updates"):
             rt = hostapi.Runtime(0, sync_each_op=False, dataflow=(mode == "dataflow"))
             net = hostapi.Net(rt, name, BATCH)
-            if mode == "fused":
-                net.set_fused()
+            if mode in ("fused", "fused_updates"):
+                net.set_fused(updates=(mode == "fused_updates"))
             for k, v in params.items():
                 net.set_param(k, v)
             net.load_batch(data, label)
@@ -444,9 +446,10 @@ def small_nets(steps=20, warmup=3):
             net.close()
             rt.close()
         out[name + "_b256"] = row
-        log("%s b=%d: %.3f ms/step (dataflow %.3f, fused %.3f), recorded step %.3f ms/replay (%d nodes)" %
+        log("%s b=%d: %.3f ms/step (dataflow %.3f, fused %.3f, with fused updates %.3f), recorded step "
+            "%.3f ms/replay (%d nodes)" %
             (name, BATCH, row["ms_per_step"], row["dataflow_ms_per_step"], row["fused_ms_per_step"],
-             g["ms_per_step"], g["nodes"]))
+             row["fused_updates_ms_per_step"], g["ms_per_step"], g["nodes"]))
     return out
 
 
@@ -635,6 +638,11 @@ def main():
                                 "ms_per_step": round(res["fused"]["ms_per_step"], 3),
                                 "ops_per_step": res["fused"]["ops_per_step"],
                                 "graph_replay": res["fused"]["graph_replay"],
+                                "weight_updates_in_gradient_kernels": {
+                                    "images_per_s": round(res["fused_updates"]["images_per_s"], 1),
+                                    "ms_per_step": round(res["fused_updates"]["ms_per_step"], 3),
+                                    "ops_per_step": res["fused_updates"]["ops_per_step"],
+                                    "note": "same parameters bit for bit; weight gradients are not stored"},
                                 "note": "opt-in fused operators, results bit-identical to the "
                                         "operator-by-operator step"},
             "dataflow_4_streams": ({"images_per_s": round(res["dataflow"]["images_per_s"], 1),

@@ -349,6 +349,14 @@ int mnv_select(const float* src, float* dst, const int* indices_host, int num_in
  *                              apps/mnist_common.h:258-262, owl/apps/imagenet_alexnet/alexnet.py:96-99)
  *   mnv_sgemm_nt             = mnv_transpose(bt{n,k} -> b{k,n}), then mnv_sgemm_nn(a, b)
  *                              (the weight gradient sens * act^T of the same lines)
+ *   mnv_sgemm_nt_sgd         = mnv_sgemm_nt into a gradient g{m,n}, then mnv_sgd_update(w, g):
+ *                              w_out = w - scale * (a * bt^T); the gradient is never stored.
+ *                              w_out may be w (each element is read, then written, once)
+ *   mnv_conv_bwd_filter_sgd  = mnv_conv_bwd_filter into a gradient, then mnv_sgd_update:
+ *                              filter_out = filter - scale * gradient; filter_out may be filter.
+ *                              Refused (-1) for problems that mnv_conv_bwd_filter cuts into
+ *                              several launches (operands of 2^29 elements and more)
+ *                              (gradient and update of apps/mnist_common.h:185-197)
  * Workspaces are those of the unfused entry points (same *_workspace_bytes; for the
  * transposed products mnv_sgemm_nn_workspace_bytes(m, n, k)). ---- */
 int mnv_conv_fwd_relu(const float* bottom, const float* filter, const float* bias, float* top,
@@ -380,6 +388,15 @@ int mnv_sgemm_tn(const float* at, const float* b, const float* gate, float* c, i
                  void* workspace, size_t workspace_bytes, mnv_stream_t stream);
 int mnv_sgemm_nt(const float* a, const float* bt, float* c, int m, int n, int k, void* workspace,
                  size_t workspace_bytes, mnv_stream_t stream);
+int mnv_sgemm_nt_sgd(const float* a, const float* bt, const float* w, float scale, float* w_out,
+                     int m, int n, int k, void* workspace, size_t workspace_bytes,
+                     mnv_stream_t stream);
+int mnv_conv_bwd_filter_sgd(const float* bottom, const float* top_diff, const float* filter,
+                            float scale, float* filter_out, int num_images,
+                            int bottom_num_channels, int top_num_channels, int bottom_height,
+                            int bottom_width, int pad_height, int pad_width, int stride_vertical,
+                            int stride_horizontal, int filter_height, int filter_width,
+                            void* workspace, size_t workspace_bytes, mnv_stream_t stream);
 
 /* ---- random tensors: CudaPerformRandn / CudaPerformRandBernoulli (cuda_perform.h:66-67).
  * The reference seeds cuRAND from the wall clock per call (cuda.cpp:601,606); here the seed

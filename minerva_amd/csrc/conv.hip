@@ -344,6 +344,10 @@ struct ConvBwdFilter {
   ConvGeom g;
   int M, N, K, total_slabs, spp;  // C*R*S, Kout, N*Ho*Wo
   int accumulate;                 // filter_diff += (a later chunk of images)
+  // Parameter update in the store: filter_diff receives sgd_w - sgd_scale * gradient
+  // (sgd_w may be filter_diff itself)
+  const float* sgd_w;
+  float sgd_scale;
   struct Res {
     mnv_rsrc a, b;
   };
@@ -414,8 +418,10 @@ struct ConvBwdFilter {
     mnv_fetch_vec<4>(r.b, off, 0u, v);
   }
   __device__ void c_store(int m, int n, float x) const {
-    float* p = filter_diff + (size_t)n * M + m;
-    *p = accumulate ? *p + x : x;
+    const size_t at = (size_t)n * M + m;
+    if (sgd_w) x = sgd_w[at] - sgd_scale * x;
+    else if (accumulate) x = filter_diff[at] + x;
+    filter_diff[at] = x;
   }
 };
 
@@ -444,6 +450,8 @@ struct ConvBwdFilterFast {
   int PP, taps_per_block;         // padded positions per image, table rows per workgroup
   MnvFastDiv d_C;
   int accumulate;                 // filter_diff += (a later chunk of images)
+  const float* sgd_w;             // update in the store, as in ConvBwdFilter
+  float sgd_scale;
   struct Res {
     mnv_rsrc a, b;
     const unsigned* tab;  // LDS: [taps_per_block][PP]
@@ -540,8 +548,10 @@ struct ConvBwdFilterFast {
       int tap = mnv_fastdiv(m, d_C);
       row = (m - tap * g.C) * g.RS + tap;
     }
-    float* p = filter_diff + (size_t)n * M + row;
-    *p = accumulate ? *p + x : x;
+    const size_t at = (size_t)n * M + row;
+    if (sgd_w) x = sgd_w[at] - sgd_scale * x;
+    else if (accumulate) x = filter_diff[at] + x;
+    filter_diff[at] = x;
   }
 };
 
@@ -874,7 +884,8 @@ size_t mnv_conv_bwd_filter_workspace_bytes(int N, int C, int K, int H, int W, in
 static int conv_bwd_filter_impl(const float* bottom, const float* top_diff, float* filter_diff,
                                 int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh,
                                 int R, int S, void* workspace, size_t workspace_bytes,
-                                mnv_stream_t stream, int accumulate) {
+                                mnv_stream_t stream, int accumulate,
+                                const float* sgd_w = nullptr, float sgd_scale = 0.f) {
   ConvGeom g;
   if (!bottom || !top_diff || !filter_diff) return MNV_ERR_INVALID;
   int rc = make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S);
@@ -898,15 +909,15 @@ static int conv_bwd_filter_impl(const float* bottom, const float* top_diff, floa
   }
   if (tile != 0 && ph == 0 && pw == 0 && (size_t)PP * 4 <= 24 * 1024) {
     ConvBwdFilterFast<true> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
-                              PP / 16, PP, 1, mnv_fastdiv_make(C), accumulate};
+                              PP / 16, PP, 1, mnv_fastdiv_make(C), accumulate, sgd_w, sgd_scale};
     return launch_tile(tile, p, splits, workspace, s);
   }
   if (tile != 0 && (size_t)taps_per_block * PP * 4 <= 24 * 1024) {
     ConvBwdFilterFast<false> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
-                               PP / 16, PP, taps_per_block, mnv_fastdiv_make(C), accumulate};
+                               PP / 16, PP, taps_per_block, mnv_fastdiv_make(C), accumulate, sgd_w, sgd_scale};
     return launch_tile(tile, p, splits, workspace, s);
   }
-  ConvBwdFilter p{bottom, top_diff, filter_diff, g, gm, gn, gk, (gk + 15) / 16, 1, accumulate};
+  ConvBwdFilter p{bottom, top_diff, filter_diff, g, gm, gn, gk, (gk + 15) / 16, 1, accumulate, sgd_w, sgd_scale};
   return launch_tile(tile, p, splits, workspace, s);
 }
 
@@ -928,6 +939,18 @@ int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filte
     if (rc) return rc;
   }
   return MNV_OK;
+}
+
+int mnv_conv_bwd_filter_sgd(const float* bottom, const float* top_diff, const float* filter,
+                            float scale, float* filter_out, int N, int C, int K, int H, int W,
+                            int ph, int pw, int sv, int sh, int R, int S, void* workspace,
+                            size_t workspace_bytes, mnv_stream_t stream) {
+  if (!filter || !filter_out) return MNV_ERR_INVALID;
+  // a gradient summed over several launches cannot be folded into the store of one
+  const int chunk = images_per_launch(N, C, K, H, W, ph, pw, sv, sh, R, S);
+  if (chunk > 0 && chunk < N) return MNV_ERR_INVALID;
+  return conv_bwd_filter_impl(bottom, top_diff, filter_out, N, C, K, H, W, ph, pw, sv, sh, R, S,
+                              workspace, workspace_bytes, stream, 0, filter, scale);
 }
 
 }  // extern "C"

@@ -101,6 +101,21 @@ struct MnvFetchMap {
 //   void block_init(Res&, float* extra_lds, int m0, int n0) const;   once per workgroup,
 //        before the first load; a barrier follows it
 //   void c_store(int m, int n, float v) const;   only called for m < M, n < N
+//   optional, for a store that combines the product with a value read from memory:
+//   static constexpr bool C_PRELOAD = true;
+//   bool c_preload_on() const;                   uniform: whether this launch reads
+//   float c_preload(int m, int n) const;         the value that goes with element (m,n)
+//   void c_store_with(int m, int n, float v, float pre) const;
+//        the kernel then reads the 16 values of a 32x32 block before it stores the block,
+//        so the reads are in flight together instead of one ahead of each store
+template <class P, class = void>
+struct MnvCPreload {
+  static constexpr bool value = false;
+};
+template <class P>
+struct MnvCPreload<P, std::enable_if_t<P::C_PRELOAD>> {
+  static constexpr bool value = true;
+};
 template <int NOFF>
 __device__ __forceinline__ void mnv_fetch_vec(mnv_rsrc r, const unsigned (&off)[NOFF],
                                               unsigned soff, float (&v)[4]) {
@@ -278,6 +293,30 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
   // of its 32x32 block.
   const bool split = gridDim.z > 1;
   float* part = split ? partial + (size_t)blockIdx.z * prob.M * prob.N : nullptr;
+  if constexpr (MnvCPreload<P>::value) {
+    if (!split && prob.c_preload_on()) {
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i) {
+        const int m = m0 + wm + i * 32 + lm;
+        if (m >= prob.M) continue;
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) {
+          float pre[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int n = n0 + wn + j * 32 + lk * 4 + (r & 3) + 8 * (r >> 2);
+            pre[r] = n < prob.N ? prob.c_preload(m, n) : 0.f;
+          }
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int n = n0 + wn + j * 32 + lk * 4 + (r & 3) + 8 * (r >> 2);
+            if (n < prob.N) prob.c_store_with(m, n, acc[i][j][r], pre[r]);
+          }
+        }
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < T::TM; ++i) {
     const int m = m0 + wm + i * 32 + lm;

@@ -40,9 +40,13 @@ struct SgemmNN {
   // stored, each the single operation the separate operator performs:
   //   bias: + bias[m] (the broadcast add of an {m,1} vector); relu: max(., 0);
   //   gate: gate[m,n] > 0 ? . : 0 (the ReLU gradient's selection)
+  //   sgd_w (B transposed only, the weight gradient of an inner product): the value stored
+  //   is sgd_w[m,n] - sgd_scale * ., the parameter update; C may be sgd_w itself
   const float* __restrict__ bias;
   const float* __restrict__ gate;
   int relu;
+  const float* sgd_w;
+  float sgd_scale;
   struct Res {
     mnv_rsrc a, b;
   };
@@ -103,7 +107,17 @@ struct SgemmNN {
     if (bias) x = x + bias[m];
     if (relu) x = x > 0.f ? x : 0.f;
     if (gate) x = gate[at] > 0.f ? x : 0.f;
+    if (TB) {
+      if (sgd_w) x = sgd_w[at] - sgd_scale * x;
+    }
     C[at] = x;
+  }
+  // the update read ahead of the block's stores (only bias / relu / gate / accumulate off)
+  static constexpr bool C_PRELOAD = TB;
+  __device__ bool c_preload_on() const { return sgd_w != nullptr; }
+  __device__ float c_preload(int m, int n) const { return sgd_w[(size_t)n * ldc + m]; }
+  __device__ void c_store_with(int m, int n, float x, float w) const {
+    C[(size_t)n * ldc + m] = w - sgd_scale * x;
   }
 };
 
@@ -112,6 +126,8 @@ struct SgemmEpilogue {
   const float* gate;
   int relu;
   int lda = 0, ldb = 0, ldc = 0, accumulate = 0;  // 0: the matrices' own m, k, m
+  const float* sgd_w = nullptr;
+  float sgd_scale = 0.f;
 };
 
 template <bool VEC, bool TA = false, bool TB = false>
@@ -122,6 +138,7 @@ SgemmNN<VEC, TA, TB> make_sgemm(const float* a, const float* b, float* c, int m,
   p.bias = e.bias; p.gate = e.gate; p.relu = e.relu;
   p.lda = e.lda ? e.lda : (TA ? k : m); p.ldb = e.ldb ? e.ldb : (TB ? n : k); p.ldc = e.ldc ? e.ldc : m;
   p.accumulate = e.accumulate;
+  p.sgd_w = e.sgd_w; p.sgd_scale = e.sgd_scale;
   p.set_bk(16);
   return p;
 }
@@ -313,6 +330,19 @@ int mnv_sgemm_nt(const float* a, const float* bt, float* c, int m, int n, int k,
   if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
   return sgemm_t_impl<false, true>(a, bt, c, m, n, k, workspace, workspace_bytes, mnv_stream(stream),
                                    SgemmEpilogue{nullptr, nullptr, 0});
+}
+
+int mnv_sgemm_nt_sgd(const float* a, const float* bt, const float* w, float scale, float* w_out,
+                     int m, int n, int k, void* workspace, size_t workspace_bytes,
+                     mnv_stream_t stream) {
+  if (m == 0 || n == 0) return MNV_OK;
+  if (!a || !bt || !w || !w_out || m < 0 || n < 0 || k <= 0) return MNV_ERR_INVALID;
+  if ((long long)m * k >= (1LL << 29) || (long long)k * n >= (1LL << 29)) return MNV_ERR_INVALID;
+  SgemmEpilogue e{nullptr, nullptr, 0};
+  e.sgd_w = w;
+  e.sgd_scale = scale;
+  return sgemm_t_impl<false, true>(a, bt, w_out, m, n, k, workspace, workspace_bytes,
+                                   mnv_stream(stream), e);
 }
 
 int mnv_sgemm_nn_static(const float* a, const float* b, float* c, int m, int n, int k,

@@ -183,6 +183,15 @@ Tensor RunNamedOp(Runner* rt, const std::string& op, const std::vector<Tensor>& 
     need(2);
     MNV_CHECK(n_params >= 1) << "sgd_update takes the scale";
     r = rt->SgdUpdate(in[0], in[1], static_cast<float>(params[0]));
+  } else if (op == "matmult_trans_b_sgd") {  // params: scale; inputs: a {m,k}, bt {n,k}, w {m,n}
+    need(3);
+    MNV_CHECK(n_params >= 1) << "matmult_trans_b_sgd takes the scale";
+    r = rt->MatMultTransBSgd(in[0], in[1], in[2], static_cast<float>(params[0]));
+  } else if (op == "conv_backward_filter_sgd") {  // params: conv info, scale; inputs: diff, bottom, filter
+    need(3);
+    MNV_CHECK(n_params >= 5) << "conv_backward_filter_sgd takes the convolution and the scale";
+    r = rt->ConvBackwardFilterSgd(in[0], in[1], in[2], conv_info(),
+                                  static_cast<float>(params[4]));
   } else if (op == "threshold_norm") {  // params: threshold
     need(1);
     MNV_CHECK(n_params >= 1) << "threshold_norm takes the threshold";
@@ -484,6 +493,7 @@ int mnvh_net_set_fused(void* net, int on) {
     NetHandle* h = static_cast<NetHandle*>(net);
     MNV_CHECK(!h->graph) << "release the recorded step before switching operator sets";
     h->net->fused = on != 0;
+    h->net->fuse_update = on == 2;
   });
 }
 

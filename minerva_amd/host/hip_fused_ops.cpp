@@ -127,5 +127,35 @@ void SgdUpdate(const DataList& inputs, const DataList& outputs, SgdUpdateClosure
      "sgd update");
 }
 
+void MatMultTransBSgd(const DataList& inputs, const DataList& outputs, MatMultTransBSgdClosure& c,
+                      const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 3u) << "(matmult transposed + sgd) #inputs is wrong!";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(matmult transposed + sgd) #outputs is wrong!";
+  int m = inputs[0].size_[0];
+  int k = inputs[0].size_[1];
+  int n = inputs[1].size_[0];
+  MNV_CHECK_EQ(inputs[1].size_[1], k) << "(matmult transposed + sgd) inner dimensions differ";
+  MNV_CHECK(inputs[2].size_ == (Scale{m, n})) << "parameter and gradient differ";
+  Ok(mnv_sgemm_nt_sgd(inputs[0].data_, inputs[1].data_, inputs[2].data_, c.scale, outputs[0].data_,
+                      m, n, k, ctx.workspace, ctx.workspace_bytes, ctx.stream),
+     "sgemm, right operand transposed, + sgd update");
+}
+
+void ConvBackwardFilterSgd(const DataList& inputs, const DataList& outputs,
+                           ConvBackwardFilterSgdClosure& c, const Context& ctx) {
+  MNV_CHECK_EQ(inputs.size(), 3u) << "(conv backward filter + sgd) #inputs wrong";
+  MNV_CHECK_EQ(outputs.size(), 1u) << "(conv backward filter + sgd) #outputs wrong";
+  auto& top_diff = inputs[0];
+  auto& bottom = inputs[1];
+  auto& filter = inputs[2];
+  MNV_CHECK(filter.size_ == outputs[0].size_) << "parameter and result differ";
+  Ok(mnv_conv_bwd_filter_sgd(bottom.data_, top_diff.data_, filter.data_, c.scale, outputs[0].data_,
+                             top_diff.size_[3], bottom.size_[2], top_diff.size_[2],
+                             bottom.size_[1], bottom.size_[0], c.pad_height, c.pad_width,
+                             c.stride_vertical, c.stride_horizontal, filter.size_[1],
+                             filter.size_[0], ctx.workspace, ctx.workspace_bytes, ctx.stream),
+     "conv backward filter + sgd update");
+}
+
 }  // namespace hip
 }  // namespace minerva

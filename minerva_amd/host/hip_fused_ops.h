@@ -42,6 +42,16 @@ struct MatMultTransBClosure {};
 struct SgdUpdateClosure {
   float scale;
 };
+// out = w - scale * (a * b^T), b given as {n,k}; inputs {a, b, w}: MatMultTransB, then SgdUpdate,
+// with the gradient never stored
+struct MatMultTransBSgdClosure {
+  float scale;
+};
+// out = filter - scale * conv_backward_filter(top_diff, bottom); inputs {top_diff, bottom, filter}
+struct ConvBackwardFilterSgdClosure {
+  int pad_height, pad_width, stride_vertical, stride_horizontal;
+  float scale;
+};
 
 namespace hip {
 
@@ -56,6 +66,9 @@ void MatMultReluBackward(const DataList&, const DataList&, MatMultReluBackwardCl
 void MatMultTransA(const DataList&, const DataList&, MatMultTransAClosure&, const Context&);
 void MatMultTransB(const DataList&, const DataList&, MatMultTransBClosure&, const Context&);
 void SgdUpdate(const DataList&, const DataList&, SgdUpdateClosure&, const Context&);
+void MatMultTransBSgd(const DataList&, const DataList&, MatMultTransBSgdClosure&, const Context&);
+void ConvBackwardFilterSgd(const DataList&, const DataList&, ConvBackwardFilterSgdClosure&,
+                           const Context&);
 
 }  // namespace hip
 }  // namespace minerva

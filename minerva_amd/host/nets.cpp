@@ -64,6 +64,26 @@ Tensor Net::MatMultTrans(const Tensor& a, const Tensor& bt) {
   return rt->MatMult(a, rt->Trans(bt));
 }
 
+void Net::SgdFc(const std::string& name, const Tensor& sens, const Tensor& act, float lr) {
+  if (fused && fuse_update) {
+    results.erase("g_" + name);
+    params[name] = rt->MatMultTransBSgd(sens, act, params[name], lr / static_cast<float>(batch_));
+    return;
+  }
+  Sgd(name, MatMultTrans(sens, act), lr);
+}
+
+void Net::SgdConv(const std::string& name, const Tensor& diff, const Tensor& bottom, ConvInfo info,
+                  float lr) {
+  if (fused && fuse_update) {
+    results.erase("g_" + name);
+    params[name] = rt->ConvBackwardFilterSgd(diff, bottom, params[name], info,
+                                             lr / static_cast<float>(batch_));
+    return;
+  }
+  Sgd(name, rt->ConvBackwardFilter(diff, bottom, params[name], info), lr);
+}
+
 // ------------------------------------------------------------------------- MLP
 
 MlpNet::MlpNet(Runner* r, int batch, int in, int hidden, int out)
@@ -87,12 +107,10 @@ void MlpNet::Step(const Tensor& data, const Tensor& label, float lr) {
   // BP
   Tensor s2 = rt->Sub(a3, label);
   Tensor s1 = TransMatMultReluBackward(w1, s2, a1);
-  Tensor gw0 = MatMultTrans(s1, data);
   Tensor gb0 = rt->Sum(s1, 1);
-  Tensor gw1 = MatMultTrans(s2, a1);
   Tensor gb1 = rt->Sum(s2, 1);
-  // update
-  Sgd("w0", gw0, lr); Sgd("b0", gb0, lr); Sgd("w1", gw1, lr); Sgd("b1", gb1, lr);
+  // weight gradients and update
+  SgdFc("w0", s1, data, lr); Sgd("b0", gb0, lr); SgdFc("w1", s2, a1, lr); Sgd("b1", gb1, lr);
 }
 
 // ------------------------------------------------------------------------- CNN
@@ -153,14 +171,12 @@ void CnnNet::Step(const Tensor& data, const Tensor& label, float lr) {
     Tensor s2 = rt->PoolingBackward(s3, a3, a2, pool_info[0]);
     s1 = rt->ActivationBackward(s2, a2, a1, ActivationAlgorithm::kRelu);
   }
-  Tensor gw0 = rt->ConvBackwardFilter(s1, a0, params["w0"], conv_info[0]);
   Tensor gb0 = rt->ConvBackwardBias(s1);
-  Tensor gw1 = rt->ConvBackwardFilter(s4, a3, params["w1"], conv_info[1]);
   Tensor gb1 = rt->ConvBackwardBias(s4);
-  Tensor gw2 = MatMultTrans(s7, re6);
   Tensor gb2 = rt->Sum(s7, 1);
-  Sgd("w0", gw0, lr); Sgd("b0", gb0, lr); Sgd("w1", gw1, lr); Sgd("b1", gb1, lr);
-  Sgd("w2", gw2, lr); Sgd("b2", gb2, lr);
+  SgdConv("w0", s1, a0, conv_info[0], lr); Sgd("b0", gb0, lr);
+  SgdConv("w1", s4, a3, conv_info[1], lr); Sgd("b1", gb1, lr);
+  SgdFc("w2", s7, re6, lr); Sgd("b2", gb2, lr);
 }
 
 // --------------------------------------------------------------------- AlexNet
@@ -243,15 +259,7 @@ void AlexNet::Step(const Tensor& data, const Tensor& label, float lr) {
   sens[3] = PoolBackwardRelu(sens[4], acts[4], acts[3], poolings[1]);
   sens[2] = rt->ConvBackwardData(sens[3], acts[2], W(1), convs[1]);
   sens[1] = PoolBackwardRelu(sens[2], acts[2], acts[1], poolings[0]);
-  Tensor gw[8], gb[8];
-  gw[7] = MatMultTrans(sens[11], acts[10]);
-  gw[6] = MatMultTrans(sens[10], acts[9]);
-  gw[5] = MatMultTrans(sens[9], re8);
-  gw[4] = rt->ConvBackwardFilter(sens[7], acts[6], W(4), convs[4]);
-  gw[3] = rt->ConvBackwardFilter(sens[6], acts[5], W(3), convs[3]);
-  gw[2] = rt->ConvBackwardFilter(sens[5], acts[4], W(2), convs[2]);
-  gw[1] = rt->ConvBackwardFilter(sens[3], acts[2], W(1), convs[1]);
-  gw[0] = rt->ConvBackwardFilter(sens[1], acts[0], W(0), convs[0]);
+  Tensor gb[8];
   gb[7] = rt->Sum(sens[11], 1);
   gb[6] = rt->Sum(sens[10], 1);
   gb[5] = rt->Sum(sens[9], 1);
@@ -260,10 +268,16 @@ void AlexNet::Step(const Tensor& data, const Tensor& label, float lr) {
   gb[2] = rt->ConvBackwardBias(sens[5]);
   gb[1] = rt->ConvBackwardBias(sens[3]);
   gb[0] = rt->ConvBackwardBias(sens[1]);
-  for (int i = 0; i < 8; ++i) {
-    Sgd("w" + std::to_string(i), gw[i], lr);
-    Sgd("b" + std::to_string(i), gb[i], lr);
-  }
+  // weight gradients and updates
+  SgdFc("w7", sens[11], acts[10], lr);
+  SgdFc("w6", sens[10], acts[9], lr);
+  SgdFc("w5", sens[9], re8, lr);
+  SgdConv("w4", sens[7], acts[6], convs[4], lr);
+  SgdConv("w3", sens[6], acts[5], convs[3], lr);
+  SgdConv("w2", sens[5], acts[4], convs[2], lr);
+  SgdConv("w1", sens[3], acts[2], convs[1], lr);
+  SgdConv("w0", sens[1], acts[0], convs[0], lr);
+  for (int i = 0; i < 8; ++i) Sgd("b" + std::to_string(i), gb[i], lr);
 }
 
 }  // namespace minerva

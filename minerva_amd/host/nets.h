@@ -35,6 +35,10 @@ class Net {
   bool keep_activations = false;
   // Opt-in fast path: fused epilogues instead of separate ReLU / bias / update operators.
   bool fused = false;
+  // With `fused`: the weight updates of convolutions and inner products are applied in the
+  // store of the kernel that produces the gradient.  Same parameters bit for bit, but the
+  // weight gradients are never stored, so `results` holds no "g_w<i>".
+  bool fuse_update = false;
 
  protected:
   // w <- w - (lr / batch) * g : ArithmeticConst(mult, const on the left) + Arithmetic(sub)
@@ -49,6 +53,9 @@ class Net {
   Tensor TransMatMult(const Tensor& at, const Tensor& b);
   Tensor TransMatMultReluBackward(const Tensor& at, const Tensor& b, const Tensor& act);
   Tensor MatMultTrans(const Tensor& a, const Tensor& bt);
+  // gradient + update of an inner product's weights (sens * act^T) and of a filter
+  void SgdFc(const std::string& name, const Tensor& sens, const Tensor& act, float lr);
+  void SgdConv(const std::string& name, const Tensor& diff, const Tensor& bottom, ConvInfo info, float lr);
   Runner* rt;
   int batch_;
 };

@@ -76,6 +76,8 @@ MNV_INSTALL_COMPUTE_FN(MatMultReluBackwardClosure, hip::MatMultReluBackward)
 MNV_INSTALL_COMPUTE_FN(MatMultTransAClosure, hip::MatMultTransA)
 MNV_INSTALL_COMPUTE_FN(MatMultTransBClosure, hip::MatMultTransB)
 MNV_INSTALL_COMPUTE_FN(SgdUpdateClosure, hip::SgdUpdate)
+MNV_INSTALL_COMPUTE_FN(MatMultTransBSgdClosure, hip::MatMultTransBSgd)
+MNV_INSTALL_COMPUTE_FN(ConvBackwardFilterSgdClosure, hip::ConvBackwardFilterSgd)
 MNV_INSTALL_DATAGEN_FN(ArrayLoaderClosure, hip::ArrayLoader)
 MNV_INSTALL_DATAGEN_FN(FillClosure, hip::Fill)
 MNV_INSTALL_DATAGEN_FN(RandnClosure, hip::Randn)
@@ -144,6 +146,7 @@ MNV_SIMPLE_OP(MatMultReluBackwardOp, ComputeFnWithClosure, MatMultReluBackwardCl
 MNV_SIMPLE_OP(MatMultTransAOp, ComputeFnWithClosure, MatMultTransAClosure, "trans * [+ relu bp]")
 MNV_SIMPLE_OP(MatMultTransBOp, ComputeFnWithClosure, MatMultTransBClosure, "* trans")
 MNV_SIMPLE_OP(SgdUpdateOp, ComputeFnWithClosure, SgdUpdateClosure, "sgd update")
+MNV_SIMPLE_OP(MatMultTransBSgdOp, ComputeFnWithClosure, MatMultTransBSgdClosure, "* trans + sgd update")
 
 class MatMultBiasOp : public ComputeFnWithClosure<MatMultBiasClosure> {
  public:
@@ -205,7 +208,8 @@ template <class Base, int kind> class ConvNamed : public Base {
     ss << "pad:" << this->closure.pad_height << "*" << this->closure.pad_width
        << " stride:" << this->closure.stride_vertical << "*" << this->closure.stride_horizontal
        << (kind == 0 ? " conv ff" : kind == 1 ? " conv bp data" : kind == 2 ? " conv bp filter"
-           : kind == 3 ? " conv ff + relu" : " conv bp data + relu bp");
+           : kind == 3 ? " conv ff + relu" : kind == 4 ? " conv bp data + relu bp"
+                                           : " conv bp filter + sgd update");
     return ss.str();
   }
 };
@@ -214,6 +218,7 @@ typedef ConvNamed<ComputeFnWithClosure<ConvBackwardDataClosure>, 1> ConvBackward
 typedef ConvNamed<ComputeFnWithClosure<ConvBackwardFilterClosure>, 2> ConvBackwardFilterOp;
 typedef ConvNamed<ComputeFnWithClosure<ConvForwardReluClosure>, 3> ConvForwardReluOp;
 typedef ConvNamed<ComputeFnWithClosure<ConvBackwardDataReluClosure>, 4> ConvBackwardDataReluOp;
+typedef ConvNamed<ComputeFnWithClosure<ConvBackwardFilterSgdClosure>, 5> ConvBackwardFilterSgdOp;
 
 template <class Base, bool fwd> class SoftmaxNamed : public Base {
  public:

@@ -456,4 +456,22 @@ Tensor Runner::SgdUpdate(const Tensor& w, const Tensor& g, float scale) {
   return Compute({w, g}, w->size, op);
 }
 
+Tensor Runner::MatMultTransBSgd(const Tensor& a, const Tensor& bt, const Tensor& w, float scale) {
+  MNV_CHECK_EQ(a->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(bt->size.NumDims(), 2u) << "eligible only for 2D";
+  MNV_CHECK_EQ(a->size[1], bt->size[1]) << "size must match";
+  MNV_CHECK(w->size == (Scale{a->size[0], bt->size[0]})) << "parameter extent must match the product";
+  auto op = std::make_shared<MatMultTransBSgdOp>();
+  op->closure = {scale};
+  return Compute({a, bt, w}, w->size, op);
+}
+
+Tensor Runner::ConvBackwardFilterSgd(const Tensor& diff, const Tensor& bottom, const Tensor& filter,
+                                     ConvInfo info, float scale) {
+  MNV_CHECK_EQ(diff->size[3], bottom->size[3]) << "#images mismatch";
+  auto op = std::make_shared<ConvBackwardFilterSgdOp>();
+  op->closure = {info.pad_height, info.pad_width, info.stride_vertical, info.stride_horizontal, scale};
+  return Compute({diff, bottom, filter}, filter->size, op);
+}
+
 }  // namespace minerva

@@ -136,6 +136,11 @@ class Runner : public DeviceListener {
   Tensor MatMultTransB(const Tensor& a, const Tensor& bt);
   // Sub(w, ArithmeticConst(g, scale, mult))
   Tensor SgdUpdate(const Tensor& w, const Tensor& g, float scale);
+  // w - scale * (a * bt^T) and filter - scale * ConvBackwardFilter(diff, bottom): the update
+  // applied where the gradient is produced
+  Tensor MatMultTransBSgd(const Tensor& a, const Tensor& bt, const Tensor& w, float scale);
+  Tensor ConvBackwardFilterSgd(const Tensor& diff, const Tensor& bottom, const Tensor& filter,
+                               ConvInfo info, float scale);
 
  private:
   friend struct TensorNode;

@@ -224,9 +224,11 @@ class Net:
                                          l.ctypes.data_as(fp), ctypes.c_size_t(l.size)),
                "net_load_batch")
 
-    def set_fused(self, on=True):
-        """Opt-in fast path: fused epilogues instead of separate ReLU / bias / update operators."""
-        _check(lib().mnvh_net_set_fused(self.h, 1 if on else 0), "net_set_fused")
+    def set_fused(self, on=True, updates=False):
+        """Opt-in fast path: fused epilogues instead of separate ReLU / bias / update operators.
+        `updates`: the weight updates are also applied where the weight gradients are produced;
+        the parameters keep their bits, but no "g_w<i>" can be read after a step."""
+        _check(lib().mnvh_net_set_fused(self.h, (2 if updates else 1) if on else 0), "net_set_fused")
 
     def keep_activations(self, on=True):
         """The following steps also keep "act1" ... "act10" readable (AlexNet only)."""

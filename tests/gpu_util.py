@@ -67,29 +67,32 @@ def net_batches(kind, batch, count):
     return params, out
 
 
-def net_state(net, label_floats):
+def net_state(net, label_floats, weight_gradients=True):
     s = {k: net.read(k, n) for k, n in net.params.items()}
-    s.update({"g_" + k: net.read("g_" + k, n) for k, n in net.params.items()})
+    s.update({"g_" + k: net.read("g_" + k, n) for k, n in net.params.items()
+              if weight_gradients or not k.startswith("w")})
     s["prob"] = net.read("prob", label_floats)
     return s
 
 
-def run_steps(kind, batch, variant, lr, params, batches, fused=False, **runtime_args):
-    """One step per batch, operator by operator (fused: with the fused operators); the state
-    after every step."""
+def run_steps(kind, batch, variant, lr, params, batches, fused=False, fused_updates=False,
+              **runtime_args):
+    """One step per batch, operator by operator (fused: with the fused operators;
+    fused_updates: weight updates in the gradient kernels' stores as well, which leaves no
+    weight gradients to read); the state after every step."""
     from minerva_amd import hostapi
     runtime_args.setdefault("sync_each_op", False)
     r = hostapi.Runtime(0, **runtime_args)
     net = hostapi.Net(r, kind, batch, variant)
-    if fused:
-        net.set_fused()
+    if fused or fused_updates:
+        net.set_fused(updates=fused_updates)
     for k, v in params.items():
         net.set_param(k, v)
     states = []
     for d, l in batches:
         net.load_batch(d, l)
         net.step(lr)
-        states.append(net_state(net, l.size))
+        states.append(net_state(net, l.size, weight_gradients=not fused_updates))
     run_steps.ops_issued = r.ops_issued()  # of the run that just ended
     net.close()
     r.close()

@@ -80,6 +80,39 @@ def test_conv_fused_epilogues_equal_the_operator_chain(gpu, ora, p, workspace):
     assert gpu.L.mnv_conv_bwd_data_relu(ddy.p, dw.p, None, fused.p, *p, wp, wb, gpu.dev.stream) == -1
 
 
+@pytest.mark.parametrize("p", CONV, ids=lambda p: "x".join(map(str, p)))
+@pytest.mark.parametrize("workspace", [True, False])
+def test_filter_gradient_with_the_update_in_its_store(gpu, ora, p, workspace):
+    """mnv_conv_bwd_filter_sgd against mnv_conv_bwd_filter followed by mnv_sgd_update, bit for
+    bit, into a fresh filter and in place; against the oracle's three operators at 1e-4."""
+    N, C, K, H, W, ph, pw, sv, sh, R, S = p
+    Ho, Wo = (H + 2 * ph - R) // sv + 1, (W + 2 * pw - S) // sh + 1
+    x, dy = _rand(N * C * H * W, 145), _rand(N * K * Ho * Wo, 146)
+    w = _rand(K * C * R * S, 147, 0.1)
+    scale = float(np.float32(0.01) / np.float32(N))
+    dx, ddy, dw = gpu.up(x), gpu.up(dy), gpu.up(w)
+    nf = w.size
+    grad, chain = gpu.empty(nf), gpu.empty(nf)
+    fused = gpu.up(np.full(nf, np.nan, np.float32))
+    wp, wb, keep = _ws(gpu, "mnv_conv_bwd_filter_workspace_bytes", p, workspace)
+    say("conv bwd filter + sgd update", p, workspace)
+    gpu.call("mnv_conv_bwd_filter", dx.p, ddy.p, grad.p, *p, wp, wb)
+    gpu.call("mnv_sgd_update", dw.p, grad.p, ctypes.c_float(scale), chain.p, ctypes.c_size_t(nf))
+    gpu.call("mnv_conv_bwd_filter_sgd", dx.p, ddy.p, dw.p, ctypes.c_float(scale), fused.p, *p, wp, wb)
+    want = gpu.down(chain)
+    assert_bits_equal(gpu.down(fused), want, "conv_bwd_filter_sgd vs conv_bwd_filter + sgd_update")
+    gpu.call("mnv_conv_bwd_filter_sgd", dx.p, ddy.p, dw.p, ctypes.c_float(scale), dw.p, *p, wp, wb)
+    assert_bits_equal(gpu.down(dw), want, "conv_bwd_filter_sgd in place")
+    if N * K * Ho * Wo * C * R * S < 3e8:
+        g = ora.conv_bwd_filter(dy, x, *p)
+        ref = ora.arithmetic(ora.SUB, w, ora.arithmetic_const(ora.MUL, 0, scale, g))
+        # the update is small against the weights: compare the step taken, not the sum
+        assert normwise(want - w, ref - w) <= 1e-3
+        assert normwise(want, ref) <= TOL
+    assert gpu.L.mnv_conv_bwd_filter_sgd(dx.p, ddy.p, None, ctypes.c_float(scale), fused.p, *p, wp, wb,
+                                         gpu.dev.stream) == -1
+
+
 GEMM = [(3, 5, 2), (37, 29, 53), (130, 70, 19), (256, 256, 784), (10, 256, 256), (1000, 256, 512),
         (4096, 256, 4096), (4096, 2, 9216), (1000, 2, 4096), (512, 384, 100)]
 
@@ -141,6 +174,16 @@ def test_sgemm_with_a_transposed_operand_equals_transpose_then_sgemm(gpu, m, n, 
     A = a.reshape(k, m).T.astype(np.float64)
     B = b.reshape(n, k).T.astype(np.float64)
     assert normwise(want.reshape(n, m).T, A @ B) <= TOL
+    # the weight gradient with the update in its store: w - scale * (a * bt^T)
+    w = _rand(m * n, 157, 0.05)
+    scale = float(np.float32(0.01) / np.float32(256))
+    dw, chain = gpu.up(w), gpu.empty(m * n)
+    gpu.call("mnv_sgd_update", dw.p, prod.p, ctypes.c_float(scale), chain.p, ctypes.c_size_t(m * n))
+    gpu.call("mnv_sgemm_nt_sgd", da.p, bt.p, dw.p, ctypes.c_float(scale), fused.p, m, n, k, wp, wb)
+    stepped = gpu.down(chain)
+    assert_bits_equal(gpu.down(fused), stepped, "B given transposed + sgd update")
+    gpu.call("mnv_sgemm_nt_sgd", da.p, bt.p, dw.p, ctypes.c_float(scale), dw.p, m, n, k, wp, wb)
+    assert_bits_equal(gpu.down(dw), stepped, "B given transposed + sgd update, in place")
 
 
 POOL = [
@@ -215,11 +258,18 @@ def test_fused_training_steps_bit_identical_to_operator_by_operator(kind, batch,
     ops_plain = run_steps.ops_issued
     fused = run_steps(kind, batch, variant, 0.01, params, batches, fused=True)
     ops_fused = run_steps.ops_issued
-    for step, (a, b) in enumerate(zip(plain, fused)):
+    updates = run_steps(kind, batch, variant, 0.01, params, batches, fused_updates=True)
+    ops_updates = run_steps.ops_issued
+    for step, (a, b, c) in enumerate(zip(plain, fused, updates)):
         for k in a:
             assert_bits_equal(b[k], a[k], "%s after step %d" % (k, step))
-    assert ops_fused < ops_plain
-    say("  operators issued: %d fused, %d separate" % (ops_fused, ops_plain))
+        # with the weight updates folded into the gradient kernels there are no weight
+        # gradients to read; everything else, the updated weights first of all, keeps its bits
+        assert sorted(set(a) - set(c)) == sorted("g_" + k for k in params if k.startswith("w"))
+        for k in c:
+            assert_bits_equal(c[k], a[k], "%s after step %d, updates in the gradient kernels" % (k, step))
+    assert ops_updates < ops_fused < ops_plain
+    say("  operators issued: %d with fused updates, %d fused, %d separate" % (ops_updates, ops_fused, ops_plain))
 
 
 def test_fused_host_operators_by_name():
