@@ -150,8 +150,16 @@ int mnv_maxindex_row(const float* in, float* out, int m, int n, mnv_stream_t str
  * reference's int counts).  One launch reads A and B through 32-bit byte offsets, i.e. up
  * to 2^29 - 1 elements each; beyond that the product runs as several launches over column
  * panels and k ranges (later k ranges accumulate into C): slower, and summed range by
- * range. ---- */
+ * range.
+ * mnv_sgemm_nn_plan reports how a product of these extents is launched with a workspace of
+ * that size (no counterpart in the reference, where the plan is cuBLAS's own): tile_rows is
+ * 128 or 64 (square tiles), k_ranges the number of partial results reduced by a second
+ * kernel (1: none), groups 4 when four wavefront groups of a workgroup share a tile and add
+ * their quarters of the k range through LDS.  The plan depends on (m, n, k, workspace_bytes)
+ * only, never on the operands. ---- */
 size_t mnv_sgemm_nn_workspace_bytes(int m, int n, int k);
+int mnv_sgemm_nn_plan(int m, int n, int k, size_t workspace_bytes, int* tile_rows, int* k_ranges,
+                      int* groups);
 int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k,
                  void* workspace, size_t workspace_bytes, mnv_stream_t stream);
 

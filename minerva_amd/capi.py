@@ -94,6 +94,7 @@ PROTOTYPES["mnv_sgemm_nn_bias"] = [_P, _P, _P, _P, _I, _I, _I, _I, _P, c_sz, _S]
 PROTOTYPES["mnv_sgemm_nn_relu_bwd"] = [_P, _P, _P, _P, _I, _I, _I, _P, c_sz, _S]
 PROTOTYPES["mnv_sgd_update"] = [_P, _P, c_f, _P, c_sz, _S]
 PROTOTYPES["mnv_sgemm_tn"] = [_P, _P, _P, _P, _I, _I, _I, _P, c_sz, _S]
+PROTOTYPES["mnv_sgemm_nn_plan"] = [_I, _I, _I, c_sz, _P, _P, _P]
 PROTOTYPES["mnv_sgemm_nt"] = [_P, _P, _P, _I, _I, _I, _P, c_sz, _S]
 PROTOTYPES["mnv_sgemm_nt_sgd"] = [_P, _P, _P, c_f, _P, _I, _I, _I, _P, c_sz, _S]
 PROTOTYPES["mnv_conv_bwd_filter_sgd"] = [_P, _P, _P, c_f, _P] + [_I] * 11 + [_P, c_sz, _S]

@@ -131,17 +131,26 @@ __device__ __forceinline__ void mnv_fetch_vec(mnv_rsrc r, const unsigned (&off)[
   }
 }
 
-template <class T, class P>
-__global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
+// G > 1: the workgroup is G groups of T::NT threads that work on the same output tile.
+// Each group has its own pair of LDS buffers and multiplies its own quarter of the
+// workgroup's k range; at the end the groups' accumulators are added through LDS in a fixed
+// order ((g0 + g2) + (g1 + g3)) and group 0 stores.  For a product with few output tiles and
+// a long k this keeps 16 wavefronts per CU busy with a quarter of the partial results (and of
+// the reduction kernel's reads) that as many separate workgroups would write to memory.
+template <class T, class P, int G = 1>
+__global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
     P prob, int tiles_m, int tiles_n, int slabs_per_split, float* __restrict__ partial) {
   extern __shared__ float mnv_gemm_lds[];
   constexpr int ATILE = T::a_tile(P::A_KFAST), BTILE = T::b_tile(P::B_KFAST);
-  float* As = mnv_gemm_lds;              // two buffers of ATILE floats
-  float* Bs = mnv_gemm_lds + 2 * ATILE;  // two buffers of BTILE floats
+  constexpr int GROUP_FLOATS = 2 * (ATILE + BTILE);
+  static_assert(G == 1 || G == 4, "one group, or four that are added pairwise");
+  const int tid = G > 1 ? (int)(threadIdx.x % T::NT) : (int)threadIdx.x;
+  const int grp = G > 1 ? __builtin_amdgcn_readfirstlane((int)(threadIdx.x / T::NT)) : 0;
+  float* As = mnv_gemm_lds + grp * GROUP_FLOATS;  // two buffers of ATILE floats
+  float* Bs = As + 2 * ATILE;                     // two buffers of BTILE floats
   typedef MnvFetchMap<T::BM, T::BK, T::NT, P::A_KFAST> MapA;
   typedef MnvFetchMap<T::BN, T::BK, T::NT, P::B_KFAST> MapB;
 
-  const int tid = threadIdx.x;
   // Workgroups are dealt round-robin to the 8 XCDs; remap so that each XCD (one L2)
   // works on a contiguous run of tiles that share B panels.
   int b = blockIdx.x;
@@ -151,13 +160,22 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
   const int tile_m = b % tiles_m, tile_n = b / tiles_m;
   const int m0 = tile_m * T::BM, n0 = tile_n * T::BNU;
 
-  const int slab_begin = blockIdx.z * slabs_per_split;
+  int slab_begin = blockIdx.z * slabs_per_split;
   int slab_end = slab_begin + slabs_per_split;
   if (slab_end > prob.total_slabs) slab_end = prob.total_slabs;
+  // slabs every group steps through (the same count in all of them: the steps hold
+  // workgroup barriers); a group whose quarter is shorter multiplies only its own slabs
+  int trips = slab_end - slab_begin;
+  if (G > 1) {
+    trips = (trips + G - 1) / G;
+    slab_begin += grp * trips;
+    if (slab_begin > slab_end) slab_begin = slab_end;
+    if (slab_end > slab_begin + trips) slab_end = slab_begin + trips;
+  }
 
   typename P::Res res;
   prob.make_res(res);
-  prob.block_init(res, mnv_gemm_lds + 2 * (ATILE + BTILE), m0, n0);
+  prob.block_init(res, mnv_gemm_lds + G * GROUP_FLOATS, m0, n0);
   typename P::AState ast[T::AV];
   typename P::BState bst[T::BV];
   unsigned aoff[T::AV][P::A_NOFF], boff[T::BV][P::B_NOFF];
@@ -227,7 +245,7 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
   // is unrolled by two) so that the LDS addresses of both buffers are one register plus an
   // immediate: selecting the buffer at run time cost seven address instructions per slab,
   // and every vector instruction in this loop is time the matrix pipe stands still.
-  auto step = [&](auto BUF) {
+  auto step = [&](auto BUF, bool active) {
     constexpr int buf = decltype(BUF)::value;
     // Loads of the next slab are in flight while this one is multiplied.  Past the end of
     // the k range the loads run past the tensors and read as 0 (or fetch a slab of the
@@ -245,6 +263,7 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
     // k = 8h + 4 + t (lanes 32..63), so a lane's four steps use four consecutive k.
     const float* a = As + buf * ATILE;
     const float* bb = Bs + buf * BTILE;
+    if (G == 1 || active) {
 #pragma unroll
     for (int h = 0; h < T::BK / 8; ++h) {
       float av[T::TM][4], bv[T::TN][4];
@@ -279,15 +298,52 @@ __global__ __launch_bounds__(T::NT, T::MIN_WAVES) void mnv_gemm_kernel(
           for (int j = 0; j < T::TN; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j][t], av[i][t], acc[i][j], 0, 0, 0);
     }
+    }
     stash(buf ^ 1);
     __syncthreads();
   };
   int slab = slab_begin;
-  for (; slab + 1 < slab_end; slab += 2) {
-    step(std::integral_constant<int, 0>{});
-    step(std::integral_constant<int, 1>{});
+  const int loop_end = slab_begin + trips;
+  for (; slab + 1 < loop_end; slab += 2) {
+    step(std::integral_constant<int, 0>{}, slab < slab_end);
+    step(std::integral_constant<int, 1>{}, slab + 1 < slab_end);
   }
-  if (slab < slab_end) step(std::integral_constant<int, 0>{});
+  if (slab < loop_end) step(std::integral_constant<int, 0>{}, slab < slab_end);
+
+  if constexpr (G > 1) {
+    // Every wavefront has passed the last step's barrier: the tile buffers are free and
+    // hold two groups' accumulators at a time, register by register (consecutive lanes at
+    // consecutive addresses).
+    constexpr int PART = T::NT * T::TM * T::TN * 16;
+    static_assert(2 * PART <= G * GROUP_FLOATS, "two partial tiles must fit the tile buffers");
+    float* red = mnv_gemm_lds;
+    auto put = [&](int region) {
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            red[region * PART + ((i * T::TN + j) * 16 + r) * T::NT + tid] = acc[i][j][r];
+    };
+    auto add = [&](int region) {
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            acc[i][j][r] += red[region * PART + ((i * T::TN + j) * 16 + r) * T::NT + tid];
+    };
+    if (grp >= 2) put(grp - 2);
+    __syncthreads();
+    if (grp < 2) add(grp);
+    __syncthreads();
+    if (grp == 1) put(0);
+    __syncthreads();
+    if (grp != 0) return;
+    add(0);
+  }
 
   // Accumulator register r of lane (lm, lk) holds C[m = lm, n = lk*4 + r%4 + 8*(r/4)]
   // of its 32x32 block.
@@ -419,7 +475,7 @@ static inline int mnv_pick_splits(long long tiles, int slabs, int max_splits, do
 
 // Host-side launch of one tile configuration.  `splits` > 1 needs
 // splits*M*N*sizeof(float) bytes at `workspace`.
-template <class T, class P>
+template <class T, int G = 1, class P>
 static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream_t s) {
   const int tiles_m = (prob.M + T::BM - 1) / T::BM, tiles_n = (prob.N + T::BNU - 1) / T::BNU;
   const int total_slabs = prob.total_slabs;
@@ -430,16 +486,18 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
   splits = total_slabs > 0 ? (total_slabs + per - 1) / per : 1;
   if ((long long)tiles_m * tiles_n > 0x7fffffffLL || splits > 65535) return MNV_ERR_INVALID;
   static bool attr_set = false;  // idempotent; a race only repeats the same call
-  const size_t tile_bytes = T::lds_bytes(P::A_KFAST, P::B_KFAST);
+  const size_t tile_bytes = G * T::lds_bytes(P::A_KFAST, P::B_KFAST);
+  const size_t lds_limit = (G > 1 ? 160 : 64) * 1024;
+  if (G > 1 && prob.extra_lds_bytes()) return MNV_ERR_INVALID;  // groups use every tile buffer
   if (!attr_set && tile_bytes + prob.extra_lds_bytes() > 48 * 1024) {
-    MNV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&mnv_gemm_kernel<T, P>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+    MNV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&mnv_gemm_kernel<T, P, G>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_limit));
     attr_set = true;
   }
   const size_t lds_bytes = tile_bytes + prob.extra_lds_bytes();
-  if (lds_bytes > 64 * 1024) return MNV_ERR_INVALID;
-  hipLaunchKernelGGL((mnv_gemm_kernel<T, P>), dim3(tiles_m * tiles_n, 1, splits), dim3(T::NT),
-                     lds_bytes, s, prob, tiles_m, tiles_n, per,
+  if (lds_bytes > lds_limit) return MNV_ERR_INVALID;
+  hipLaunchKernelGGL((mnv_gemm_kernel<T, P, G>), dim3(tiles_m * tiles_n, 1, splits),
+                     dim3(T::NT * G), lds_bytes, s, prob, tiles_m, tiles_n, per,
                      reinterpret_cast<float*>(workspace));
   int rc = MNV_LAUNCH_STATUS();
   if (rc) return rc;

@@ -155,6 +155,7 @@ typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
 struct SgemmPlan {
   bool small;
   int splits;
+  int groups = 1;  // 4: workgroups of four wavefront groups that share a tile's k range
 };
 
 SgemmPlan plan_sgemm(int m, int n, int k, size_t ws_floats) {
@@ -181,7 +182,51 @@ SgemmPlan plan_sgemm(int m, int n, int k, size_t ws_floats) {
       best_cost = cost;
     }
   }
+  // Workgroups of four wavefront groups (one per CU for the large tile, two for the small
+  // one): a step multiplies four slabs, one per group, and ends in about five slab times
+  // for the prologue and the addition through LDS.  Measured on the inner products of the
+  // AlexNet shape, back to back at sustained clocks: 4096x256x9216 0.190 -> 0.180 ms,
+  // 4096x256x4096 0.100 -> 0.092 ms (64x64 tiles, no k ranges in memory at all),
+  // 1000x256x4096 0.0304 -> 0.0278 ms, 4096x256x1000 0.031 -> 0.025 ms; 9216x256x4096, whose
+  // 144 large tiles do not divide the 256 CUs, stays with single groups.
+  // The launch of the reduction kernel itself (about six slab times) only matters in this
+  // comparison, where a plan without k ranges in memory competes.
+  const double reduce_launch = 6.0;
+  if (best.splits > 1) best_cost += reduce_launch;
+  for (int small = 0; small < 2; ++small) {
+    if (!small && (m <= 64 || n <= 64)) continue;
+    const int bm = small ? 64 : 128;
+    const long long tiles = (long long)((m + bm - 1) / bm) * ((n + bm - 1) / bm);
+    const double unit = small ? 0.27 : 1.0, overhead = small ? 4.0 : 5.0;
+    const size_t fit = mn ? ws_floats / mn : 0;
+    for (int z = 1; z <= MNV_SGEMM_MAX_SPLITS; ++z) {
+      if (z > 1 && (size_t)z > fit) break;
+      const int len4 = ((slabs + z - 1) / z + 3) / 4;
+      if (len4 < 8) break;  // shorter loops do not repay the prologue and the addition
+      // The sixteen wavefronts of such a workgroup share every barrier, so each step waits
+      // out a trip to memory that separate workgroups would overlap: worth it only when the
+      // workgroups cover most of the chip (MLP 784-256-10 at batch 256, 16 tiles: 0.111 ms
+      // per step with single groups, 0.158 ms with grouped ones).
+      if (tiles * z < 192) continue;
+      const long long per_cu = (tiles * z + 255) / 256;
+      const double cost = (double)per_cu * (4.0 * len4 * unit + overhead) +
+                          (z > 1 ? per_split * z + reduce_launch : 0.0);
+      if (cost < best_cost * 0.95) {
+        best = SgemmPlan{small != 0, z, 4};
+        best_cost = cost;
+      }
+    }
+  }
   return best;
+}
+
+template <class P>
+int launch_plan(const SgemmPlan& plan, const P& p, void* workspace, hipStream_t s) {
+  if (plan.groups == 4)
+    return plan.small ? mnv_gemm_launch<TileSmall, 4>(p, plan.splits, workspace, s)
+                      : mnv_gemm_launch<TileBig, 4>(p, plan.splits, workspace, s);
+  return plan.small ? mnv_gemm_launch<TileSmall>(p, plan.splits, workspace, s)
+                    : mnv_gemm_launch<TileBig>(p, plan.splits, workspace, s);
 }
 
 #define MNV_MAX_DEVICES 64
@@ -210,16 +255,8 @@ int sgemm_nn_impl(const float* a, const float* b, float* c, int m, int n, int k,
   bool vec = (m % 4 == 0) && (k % 4 == 0) && mnv_aligned16(a) && mnv_aligned16(b) &&
              e.lda % 4 == 0 && e.ldb % 4 == 0;
   const SgemmPlan plan = plan_sgemm(m, n, k, workspace ? workspace_bytes / sizeof(float) : 0);
-  const bool small = plan.small;
-  const int splits = plan.splits;
-  if (vec) {
-    SgemmNN<true> p = make_sgemm<true>(a, b, c, m, n, k, e);
-    return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
-                 : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
-  }
-  SgemmNN<false> p = make_sgemm<false>(a, b, c, m, n, k, e);
-  return small ? mnv_gemm_launch<TileSmall>(p, splits, workspace, s)
-               : mnv_gemm_launch<TileBig>(p, splits, workspace, s);
+  if (vec) return launch_plan(plan, make_sgemm<true>(a, b, c, m, n, k, e), workspace, s);
+  return launch_plan(plan, make_sgemm<false>(a, b, c, m, n, k, e), workspace, s);
 }
 
 // Products with one operand given transposed: same plan (tile shape, k ranges) as the plain
@@ -230,14 +267,8 @@ int sgemm_t_impl(const float* a, const float* b, float* c, int m, int n, int k, 
   const bool vec = mnv_aligned16(a) && mnv_aligned16(b) && (TA ? k % 4 == 0 : m % 4 == 0) &&
                    (TB ? n % 4 == 0 : k % 4 == 0);
   const SgemmPlan plan = plan_sgemm(m, n, k, workspace ? workspace_bytes / sizeof(float) : 0);
-  if (vec) {
-    auto p = make_sgemm<true, TA, TB>(a, b, c, m, n, k, e);
-    return plan.small ? mnv_gemm_launch<TileSmall>(p, plan.splits, workspace, s)
-                      : mnv_gemm_launch<TileBig>(p, plan.splits, workspace, s);
-  }
-  auto p = make_sgemm<false, TA, TB>(a, b, c, m, n, k, e);
-  return plan.small ? mnv_gemm_launch<TileSmall>(p, plan.splits, workspace, s)
-                    : mnv_gemm_launch<TileBig>(p, plan.splits, workspace, s);
+  if (vec) return launch_plan(plan, make_sgemm<true, TA, TB>(a, b, c, m, n, k, e), workspace, s);
+  return launch_plan(plan, make_sgemm<false, TA, TB>(a, b, c, m, n, k, e), workspace, s);
 }
 
 // Operands of 2^29 elements and more (up to the reference's limit, int element counts): the
@@ -280,6 +311,17 @@ size_t mnv_sgemm_nn_workspace_bytes(int m, int n, int k) {
   if (m <= 0 || n <= 0 || k <= 0) return 0;
   const SgemmPlan plan = plan_sgemm(m, n, k, (size_t)-1);
   return plan.splits > 1 ? (size_t)plan.splits * m * n * sizeof(float) : 0;
+}
+
+int mnv_sgemm_nn_plan(int m, int n, int k, size_t workspace_bytes, int* tile_rows, int* k_ranges,
+                      int* groups) {
+  if (m <= 0 || n <= 0 || k <= 0 || !tile_rows || !k_ranges || !groups) return MNV_ERR_INVALID;
+  const SgemmPlan plan = plan_sgemm(m, n, k, workspace_bytes / sizeof(float));
+  *tile_rows = plan.small ? 64 : 128;
+  const int slabs = (k + 15) / 16, per = (slabs + plan.splits - 1) / plan.splits;
+  *k_ranges = (slabs + per - 1) / per;  // as the launch rounds it: ranges of equal length
+  *groups = plan.groups;
+  return MNV_OK;
 }
 
 int mnv_sgemm_nn(const float* a, const float* b, float* c, int m, int n, int k, void* workspace,

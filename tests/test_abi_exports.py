@@ -55,6 +55,37 @@ def test_pure_host_entry_points():
     assert L.mnv_conv_bwd_filter_workspace_bytes(256, 256, 384, 13, 13, 1, 1, 1, 1, 3, 3) > 0
 
 
+def _plan(m, n, k, workspace=True):
+    import ctypes
+    from minerva_amd import capi
+    L = capi.lib()
+    ws = L.mnv_sgemm_nn_workspace_bytes(m, n, k) if workspace else 0
+    tile, ranges, groups = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    assert L.mnv_sgemm_nn_plan(m, n, k, ctypes.c_size_t(ws), ctypes.byref(tile), ctypes.byref(ranges),
+                               ctypes.byref(groups)) == 0
+    return tile.value, ranges.value, groups.value, ws
+
+
+def test_sgemm_plans_of_the_benchmark_shapes():
+    """The launch plan is host arithmetic on the extents alone.  Square and short-k products
+    run one tile per workgroup without k ranges; the skinny inner products of the AlexNet
+    shape run as workgroups of four wavefront groups; the workspace the query asks for is
+    exactly what the plan's partial results need; without a workspace nothing is split in
+    memory."""
+    assert _plan(4096, 4096, 4096)[:3] == (128, 1, 1)
+    assert _plan(4096, 9216, 256)[:3] == (128, 1, 1)
+    assert _plan(4096, 256, 9216)[:3] == (128, 4, 4)
+    assert _plan(4096, 256, 4096)[:3] == (64, 1, 4)
+    assert _plan(1000, 256, 4096)[:3] == (64, 4, 4)
+    assert _plan(9216, 256, 4096)[2] == 1
+    for (m, n, k) in [(4096, 256, 9216), (1000, 256, 4096), (9216, 256, 4096), (256, 256, 784),
+                      (10, 256, 256), (4, 4, 4096), (130, 70, 1000)]:
+        tile, ranges, groups, ws = _plan(m, n, k)
+        assert tile in (64, 128) and groups in (1, 4) and 1 <= ranges <= 16
+        assert ws == (ranges * m * n * 4 if ranges > 1 else 0)
+        assert _plan(m, n, k, workspace=False)[1] == 1
+
+
 def test_host_library_exports_every_declared_symbol():
     """include/mnv_host.h against libmnv_host.so (loading it needs no GPU either)."""
     from minerva_amd import capi, hostapi

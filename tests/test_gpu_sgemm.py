@@ -47,6 +47,47 @@ def test_sgemm_against_oracle(gpu, ora, m, n, k, workspace):
     assert normwise(got.reshape(n, m).T, A @ B) <= TOL
 
 
+def _plan(gpu, m, n, k, ws_bytes):
+    tile, ranges, groups = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    assert gpu.L.mnv_sgemm_nn_plan(m, n, k, ctypes.c_size_t(ws_bytes), ctypes.byref(tile),
+                                   ctypes.byref(ranges), ctypes.byref(groups)) == 0
+    return tile.value, ranges.value, groups.value
+
+
+GROUPED = [  # m, n, k, workspace: plans with four wavefront groups per workgroup
+    (1000, 1000, 2049, False),  # ragged in every extent, the last slab holds one k
+    (777, 1030, 777, False),    # 49 slabs: the last group multiplies one slab, a partial one
+    (500, 500, 3000, True),     # with k ranges in memory as well
+    (200, 1000, 4099, True),
+    (36, 4096, 5000, True),     # a single partial tile in m
+    (1000, 130, 8200, True),    # five ranges of four quarters, 513 slabs
+    (1024, 1024, 1024, True),   # no k ranges at all: one workgroup per tile and CU
+    (4096, 256, 9216, True),   # 128x128 tiles, four ranges
+]
+
+
+@pytest.mark.parametrize("m,n,k,workspace", GROUPED)
+def test_sgemm_with_grouped_workgroups(gpu, m, n, k, workspace):
+    """Products whose plan runs four wavefront groups per workgroup (each group a quarter of
+    the workgroup's k range, added through LDS) against the fp64 product."""
+    ws_bytes = gpu.L.mnv_sgemm_nn_workspace_bytes(m, n, k) if workspace else 0
+    tile, ranges, groups = _plan(gpu, m, n, k, ws_bytes)
+    assert groups == 4, "the case is meant to take the grouped kernel"
+    a, b = _rand(m * k, 40), _rand(k * n, 41)
+    say("sgemm, grouped workgroups", m, n, k, "tile", tile, "k ranges", ranges)
+    got = _gemm(gpu, a, b, m, n, k, workspace).reshape(n, m)
+    A = a.reshape(k, m).astype(np.float64)   # A[l, i]
+    B = b.reshape(n, k).astype(np.float64)   # B[j, l]
+    if m * n * k <= 2e9:
+        assert normwise(got, B @ A) <= TOL
+    else:
+        rng = np.random.default_rng(42)
+        rows, cols = rng.integers(0, m, 64), rng.integers(0, n, 64)
+        assert normwise(got[np.ix_(cols, rows)], B[cols] @ A[:, rows]) <= TOL
+    # identical calls give identical bits (the groups are added in a fixed order)
+    assert_bits_equal(_gemm(gpu, a, b, m, n, k, workspace).reshape(n, m), got, "second call")
+
+
 def test_sgemm_reference_unit_test_shape(gpu):
     # tests/unittest_sgemm.cpp:7-28: {3,2} x {2,5} against the triple loop
     a = np.arange(6, dtype=np.float32)
