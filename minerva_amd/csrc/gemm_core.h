@@ -485,14 +485,21 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
   if (per < 1) per = 1;
   splits = total_slabs > 0 ? (total_slabs + per - 1) / per : 1;
   if ((long long)tiles_m * tiles_n > 0x7fffffffLL || splits > 65535) return MNV_ERR_INVALID;
-  static bool attr_set = false;  // idempotent; a race only repeats the same call
+  // The LDS limit of a kernel is an attribute per device; set once on each (idempotent: a
+  // race only repeats the same call).
+  static bool attr_set[64] = {};
   const size_t tile_bytes = G * T::lds_bytes(P::A_KFAST, P::B_KFAST);
   const size_t lds_limit = (G > 1 ? 160 : 64) * 1024;
   if (G > 1 && prob.extra_lds_bytes()) return MNV_ERR_INVALID;  // groups use every tile buffer
-  if (!attr_set && tile_bytes + prob.extra_lds_bytes() > 48 * 1024) {
-    MNV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&mnv_gemm_kernel<T, P, G>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_limit));
-    attr_set = true;
+  if (tile_bytes + prob.extra_lds_bytes() > 48 * 1024) {
+    int dev = 0;
+    MNV_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return MNV_ERR_INVALID;
+    if (!attr_set[dev]) {
+      MNV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&mnv_gemm_kernel<T, P, G>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_limit));
+      attr_set[dev] = true;
+    }
   }
   const size_t lds_bytes = tile_bytes + prob.extra_lds_bytes();
   if (lds_bytes > lds_limit) return MNV_ERR_INVALID;

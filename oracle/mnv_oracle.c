@@ -205,8 +205,9 @@ int ora_reduction(int type, const float* in, const int* dims, int nd, const int*
 
 /* MaxIndex: basic.cpp:369-398.  Index (stored as float) of the first maximum
  * along `dim`; strict '<' so the lowest index wins ties.
- * pinned by: closed form (pure selection); compiled-reference value 4,4,4 on
- * the {5,3} iota of tests/unittest_reduction.cpp recorded in the survey. */
+ * pinned by: closed form (pure selection): on the {5,3} iota of the reference's
+ * reduction test (tests/unittest_reduction.cpp) the index is 4,4,4 along dim 0
+ * and 2,2,2,2,2 along dim 1; ties, NaN and signed zeros by exhaustive small cases. */
 int ora_maxindex(const float* in, const int* dims, int nd, int dim, float* out) {
   if (nd > ORA_MAX_DIMS || dim < 0 || dim >= nd) return 1;
   int odims[ORA_MAX_DIMS], it[ORA_MAX_DIMS];
@@ -267,7 +268,7 @@ int ora_norm_arithmetic(int type, const float* in0, const int* dims, int nd, con
 /* Softmax forward over dim 0: basic.cpp:219-261.                              */
 /* m = max, e_i = expf(x_i - m), s = sequential sum of e_i from 0, y = e_i / s */
 /* `len` = dims[0], `cols` = product of the remaining dims.                    */
-/* pinned by: fp64 closed form; rows sum to 1 (survey check on compiled ref).  */
+/* pinned by: fp64 closed form; rows sum to 1.                                  */
 /* ------------------------------------------------------------------------- */
 int ora_softmax_dim0(const float* in, float* out, int len, size_t cols) {
   for (size_t c = 0; c < cols; ++c) {
