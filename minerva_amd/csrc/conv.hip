@@ -596,15 +596,24 @@ typedef MnvGemmTile<128, 64, 16, 4, 1, 0, 32> TileThin;
 
 // tile 0: 64x64 output tiles, tile 1: 128x128, tile 2: 128x96, tile 3: 128x32
 template <class P>
-int launch_tile(int tile, const P& p, int splits, void* ws, hipStream_t s) {
+int launch_tile(int tile, const P& p, int splits, void* ws, hipStream_t s, size_t tail_bytes = 0) {
   switch (tile) {
     case 0: return mnv_gemm_launch<TileSmall>(p, splits, ws, s);
-    case 2: return mnv_gemm_launch<Tile96>(p, splits, ws, s);
+    case 2: return mnv_gemm_launch<Tile96>(p, splits, ws, s, tail_bytes);
     case 3: return mnv_gemm_launch<TileThin>(p, splits, ws, s);
-    default: return mnv_gemm_launch<TileBig>(p, splits, ws, s);
+    default: return mnv_gemm_launch<TileBig>(p, splits, ws, s, tail_bytes);
   }
 }
 const int kTileM[4] = {64, 128, 128, 128}, kTileN[4] = {64, 128, 96, 32};
+
+// Bytes the large tiles' launches want for the partial tiles of a cut tail (0: no tail).
+size_t tail_workspace_bytes(int tile, int m, int n, int slabs) {
+  if (tile != 1 && tile != 2) return 0;
+  const long long tiles = (long long)((m + kTileM[tile] - 1) / kTileM[tile]) * ((n + kTileN[tile] - 1) / kTileN[tile]);
+  const size_t tile_floats = (size_t)kTileM[tile] * kTileN[tile];
+  const MnvTailPlan t = mnv_tail_plan(tiles, slabs, tile_floats, (size_t)-1 / sizeof(float));
+  return t.z > 1 ? (size_t)(tiles - t.begin) * t.z * tile_floats * sizeof(float) : 0;
+}
 
 // 128-row tiles: 96 columns wide when that leaves clearly fewer idle columns than 128
 // (an output 96 or 192 wide), since the narrower tile does a little less work per byte
@@ -724,6 +733,8 @@ size_t mnv_conv_fwd_workspace_bytes(int N, int C, int K, int H, int W, int ph, i
   const size_t permuted = C % 16 == 0 ? (size_t)K * g.CRS * sizeof(float) : 0;
   const int gm = N * g.HoWo, gn = K;
   const int splits = small_tile_splits(pick_tile(gm, gn), gm, gn, (g.CRS + 15) / 16, (size_t)-1);
+  const size_t tail = tail_workspace_bytes(pick_tile(gm, gn), gm, gn, (g.CRS + 15) / 16);
+  if (tail) return align256(permuted) + tail;
   return splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
 }
 
@@ -754,14 +765,14 @@ static int conv_fwd_impl(const float* bottom, const float* filter, const float* 
     rc = permute_filter(filter, wp, K, C, g.RS, false, s);
     if (rc) return rc;
     ConvFwd<true> p{bottom, wp, bias, top, g, gm, gn, gk, g.RS * (C / 16), C / 16, relu};
-    return launch_tile(tile, p, splits, part, s);
+    return launch_tile(tile, p, splits, part, s, part ? workspace_bytes - used : 0);
   }
   if (np) {
     ConvFwdNP p{bottom, filter, bias, top, g, gm, gn, gk, (gk + 15) / 16, gk >= 16 ? gk / 16 : 1, relu};
-    return launch_tile(tile, p, splits, part, s);
+    return launch_tile(tile, p, splits, part, s, part ? workspace_bytes - used : 0);
   }
   ConvFwd<false> p{bottom, filter, bias, top, g, gm, gn, gk, (gk + 15) / 16, 1, relu};
-  return launch_tile(tile, p, splits, part, s);
+  return launch_tile(tile, p, splits, part, s, part ? workspace_bytes - used : 0);
 }
 
 static int conv_fwd_chunks(const float* bottom, const float* filter, const float* bias, float* top,
@@ -805,6 +816,8 @@ size_t mnv_conv_bwd_data_workspace_bytes(int N, int C, int K, int H, int W, int 
   const size_t permuted = (sv == 1 && sh == 1 && K % 16 == 0) ? (size_t)K * g.CRS * sizeof(float) : 0;
   const int gm = N * g.HW, gn = C;
   const int splits = small_tile_splits(pick_tile(gm, gn), gm, gn, (K * g.RS + 15) / 16, (size_t)-1);
+  const size_t tail = tail_workspace_bytes(pick_tile(gm, gn), gm, gn, (K * g.RS + 15) / 16);
+  if (tail) return align256(permuted) + tail;
   return splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
 }
 
@@ -830,10 +843,10 @@ static int conv_bwd_data_impl(const float* top_diff, const float* filter, const 
     rc = permute_filter(filter, wq, K, C, g.RS, true, s);
     if (rc) return rc;
     ConvBwdData<true> p{top_diff, wq, bottom_diff, g, gm, gn, gk, g.RS * (K / 16), K / 16, gate};
-    return launch_tile(tile, p, splits, part, s);
+    return launch_tile(tile, p, splits, part, s, part ? workspace_bytes - used : 0);
   }
   ConvBwdData<false> p{top_diff, filter, bottom_diff, g, gm, gn, gk, (gk + 15) / 16, 1, gate};
-  return launch_tile(tile, p, splits, part, s);
+  return launch_tile(tile, p, splits, part, s, part ? workspace_bytes - used : 0);
 }
 
 static int conv_bwd_data_chunks(const float* top_diff, const float* filter, const float* gate,

@@ -131,6 +131,20 @@ __device__ __forceinline__ void mnv_fetch_vec(mnv_rsrc r, const unsigned (&off)[
   }
 }
 
+// Workgroups are dealt round-robin to the 8 XCDs; the tile index is remapped so that each XCD
+// (one L2) works on a contiguous run of tiles that share B panels.
+__device__ __forceinline__ int mnv_tile_remap(int t, int total) {
+  const int per_xcd = total / 8;
+  return t < per_xcd * 8 ? (t % 8) * per_xcd + t / 8 : t;
+}
+
+// Tail: tiles are whole units of work, so when their number is not a multiple of the 256
+// CUs the CUs that receive one tile more than the others set the duration (676 tiles: three
+// on some CUs, 2.64 on average).  The tiles past the last multiple of 256 (`tail_begin`
+// on, in dispatch order) are therefore cut into `tail_z` k ranges, one workgroup each: small
+// units that are dispatched last and fill the CUs evenly.  Their partial tiles go to the
+// workspace, tile by tile, and mnv_gemm_tail_reduce_kernel adds them in range order.
+//
 // G > 1: the workgroup is G groups of T::NT threads that work on the same output tile.
 // Each group has its own pair of LDS buffers and multiplies its own quarter of the
 // workgroup's k range; at the end the groups' accumulators are added through LDS in a fixed
@@ -139,7 +153,8 @@ __device__ __forceinline__ void mnv_fetch_vec(mnv_rsrc r, const unsigned (&off)[
 // the reduction kernel's reads) that as many separate workgroups would write to memory.
 template <class T, class P, int G = 1>
 __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
-    P prob, int tiles_m, int tiles_n, int slabs_per_split, float* __restrict__ partial) {
+    P prob, int tiles_m, int tiles_n, int slabs_per_split, float* __restrict__ partial,
+    int tail_begin, int tail_z) {
   extern __shared__ float mnv_gemm_lds[];
   constexpr int ATILE = T::a_tile(P::A_KFAST), BTILE = T::b_tile(P::B_KFAST);
   constexpr int GROUP_FLOATS = 2 * (ATILE + BTILE);
@@ -151,12 +166,13 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
   typedef MnvFetchMap<T::BM, T::BK, T::NT, P::A_KFAST> MapA;
   typedef MnvFetchMap<T::BN, T::BK, T::NT, P::B_KFAST> MapB;
 
-  // Workgroups are dealt round-robin to the 8 XCDs; remap so that each XCD (one L2)
-  // works on a contiguous run of tiles that share B panels.
-  int b = blockIdx.x;
-  const int total = tiles_m * tiles_n;
-  const int per_xcd = total / 8;
-  if (b < per_xcd * 8) b = (b % 8) * per_xcd + b / 8;
+  int vb = blockIdx.x, tail_part = -1;
+  if (G == 1 && tail_z > 1 && vb >= tail_begin) {
+    const int i = vb - tail_begin, tl = i / tail_z;
+    tail_part = i - tl * tail_z;
+    vb = tail_begin + tl;
+  }
+  const int b = mnv_tile_remap(vb, tiles_m * tiles_n);
   const int tile_m = b % tiles_m, tile_n = b / tiles_m;
   const int m0 = tile_m * T::BM, n0 = tile_n * T::BNU;
 
@@ -165,6 +181,12 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
   if (slab_end > prob.total_slabs) slab_end = prob.total_slabs;
   // slabs every group steps through (the same count in all of them: the steps hold
   // workgroup barriers); a group whose quarter is shorter multiplies only its own slabs
+  if (G == 1 && tail_part >= 0) {
+    const int per = (prob.total_slabs + tail_z - 1) / tail_z;
+    slab_begin = tail_part * per;
+    slab_end = slab_begin + per < prob.total_slabs ? slab_begin + per : prob.total_slabs;
+    if (slab_begin > slab_end) slab_begin = slab_end;
+  }
   int trips = slab_end - slab_begin;
   if (G > 1) {
     trips = (trips + G - 1) / G;
@@ -347,6 +369,17 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
 
   // Accumulator register r of lane (lm, lk) holds C[m = lm, n = lk*4 + r%4 + 8*(r/4)]
   // of its 32x32 block.
+  if (G == 1 && tail_part >= 0) {  // a k range of a tail tile: the whole tile, in tile order
+    float* pt = partial + ((size_t)(vb - tail_begin) * tail_z + tail_part) * (T::BM * T::BNU);
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          pt[(wn + j * 32 + lk * 4 + (r & 3) + 8 * (r >> 2)) * T::BM + wm + i * 32 + lm] = acc[i][j][r];
+    return;
+  }
   const bool split = gridDim.z > 1;
   float* part = split ? partial + (size_t)blockIdx.z * prob.M * prob.N : nullptr;
   if constexpr (MnvCPreload<P>::value) {
@@ -445,6 +478,59 @@ static int mnv_gemm_splitk_reduce_launch(const P& prob, const float* partial, in
   return MNV_LAUNCH_STATUS();
 }
 
+// Adds the k ranges of the tail tiles (see mnv_gemm_kernel) in range order and hands every
+// element to the policy's store.  One thread per four consecutive rows of a tile column.
+template <class T, class P>
+__global__ __launch_bounds__(256) void mnv_gemm_tail_reduce_kernel(P prob,
+                                                                   const float* __restrict__ partial,
+                                                                   int tiles_m, int tiles_n,
+                                                                   int tail_begin, int tail_z) {
+  constexpr int TILE = T::BM * T::BNU;
+  const int b = mnv_tile_remap(tail_begin + (int)blockIdx.y, tiles_m * tiles_n);
+  const int m0 = (b % tiles_m) * T::BM, n0 = (b / tiles_m) * T::BNU;
+  const float* p = partial + (size_t)blockIdx.y * tail_z * TILE;
+  for (int e = (blockIdx.x * 256 + threadIdx.x) * 4; e < TILE; e += gridDim.x * 256 * 4) {
+    mnv_f4 s = *reinterpret_cast<const mnv_f4*>(p + e);
+    for (int z = 1; z < tail_z; ++z) {
+      const mnv_f4 v = *reinterpret_cast<const mnv_f4*>(p + (size_t)z * TILE + e);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    const int m = m0 + e % T::BM, n = n0 + e / T::BM;
+    if (n < prob.N) {
+      if (m + 0 < prob.M) prob.c_store(m + 0, n, s.x);
+      if (m + 1 < prob.M) prob.c_store(m + 1, n, s.y);
+      if (m + 2 < prob.M) prob.c_store(m + 2, n, s.z);
+      if (m + 3 < prob.M) prob.c_store(m + 3, n, s.w);
+    }
+  }
+}
+
+// Which tiles form the tail and into how many k ranges each is cut (z <= 1: none).  Only
+// for launches of at least 256 large tiles without k ranges of their own; taken when the
+// uneven last tile per CU costs at least 3% (tiles / 256 = 2.64: 12%; 11.39: 5%; 3.96: 1%),
+// with about three small workgroups per CU (two to four measured alike: conv2 data gradient
+// 1.77 -> 1.74 / 1.71 / 1.70 ms, conv5 forward 0.71 -> 0.66 ms with any of them), at least
+// eight slabs each, and only as far as the workspace holds the partial tiles.
+struct MnvTailPlan {
+  int begin, z;
+};
+static inline MnvTailPlan mnv_tail_plan(long long tiles, int slabs, size_t tile_floats,
+                                        size_t ws_floats) {
+  const MnvTailPlan none{(int)(tiles < 0x7fffffff ? tiles : 0x7fffffff), 1};
+  if (tiles < 256 || tiles > 0x3fffffff) return none;
+  const int rem = (int)(tiles % 256);
+  if (rem == 0) return none;
+  const double per_cu = (double)tiles / 256.0, most = (double)((tiles + 255) / 256);
+  if ((most - per_cu) / most < 0.03) return none;
+  int z = 768 / rem;
+  if (z > 16) z = 16;
+  if (z > slabs / 8) z = slabs / 8;
+  const size_t fit = ws_floats / ((size_t)rem * tile_floats);
+  if ((size_t)z > fit) z = (int)fit;
+  if (z < 2) return none;
+  return MnvTailPlan{(int)(tiles - rem), z};
+}
+
 // Number of k ranges for `tiles` output tiles of `slabs` k-slabs each.  Workgroups are
 // dealt evenly to 256 CUs that hold four of them at a time, and the kernel ends when the
 // fullest CU does: a split count that puts a few workgroups past a multiple of 1024 costs a
@@ -475,8 +561,11 @@ static inline int mnv_pick_splits(long long tiles, int slabs, int max_splits, do
 
 // Host-side launch of one tile configuration.  `splits` > 1 needs
 // splits*M*N*sizeof(float) bytes at `workspace`.
+// `tail_bytes`: bytes at `workspace` that a launch without k ranges may use for the partial
+// tiles of its tail (0: never cut the tail).
 template <class T, int G = 1, class P>
-static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream_t s) {
+static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream_t s,
+                           size_t tail_bytes = 0) {
   const int tiles_m = (prob.M + T::BM - 1) / T::BM, tiles_n = (prob.N + T::BNU - 1) / T::BNU;
   const int total_slabs = prob.total_slabs;
   if (splits < 1) splits = 1;
@@ -503,11 +592,23 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
   }
   const size_t lds_bytes = tile_bytes + prob.extra_lds_bytes();
   if (lds_bytes > lds_limit) return MNV_ERR_INVALID;
-  hipLaunchKernelGGL((mnv_gemm_kernel<T, P, G>), dim3(tiles_m * tiles_n, 1, splits),
-                     dim3(T::NT * G), lds_bytes, s, prob, tiles_m, tiles_n, per,
-                     reinterpret_cast<float*>(workspace));
+  MnvTailPlan tail{tiles_m * tiles_n, 1};
+  if (G == 1 && splits == 1 && T::MIN_WAVES == 4 && workspace && tail_bytes)
+    tail = mnv_tail_plan((long long)tiles_m * tiles_n, total_slabs, (size_t)T::BM * T::BNU,
+                         tail_bytes / sizeof(float));
+  const int tail_tiles = tiles_m * tiles_n - tail.begin;
+  hipLaunchKernelGGL((mnv_gemm_kernel<T, P, G>),
+                     dim3(tail.begin + tail_tiles * tail.z, 1, splits), dim3(T::NT * G), lds_bytes,
+                     s, prob, tiles_m, tiles_n, per, reinterpret_cast<float*>(workspace),
+                     tail.begin, tail.z);
   int rc = MNV_LAUNCH_STATUS();
   if (rc) return rc;
+  if (tail.z > 1) {
+    hipLaunchKernelGGL((mnv_gemm_tail_reduce_kernel<T, P>), dim3(T::BM * T::BNU / 1024, tail_tiles),
+                       dim3(256), 0, s, prob, reinterpret_cast<const float*>(workspace), tiles_m,
+                       tiles_n, tail.begin, tail.z);
+    return MNV_LAUNCH_STATUS();
+  }
   if (splits > 1) {
     // enough threads to cover the chip: one per element for a large output, up to 64 per
     // element (never more than half the ranges) for a small one

@@ -145,6 +145,32 @@ def test_conv_all_passes_against_oracle(gpu, ora, p):
         assert normwise(cv.bwd_bias(dy, ws), ref) <= TOL
 
 
+def test_conv_with_a_cut_tail_against_oracle(gpu, ora):
+    """Launches of a few more large tiles than a multiple of the 256 CUs cut the tiles past
+    that multiple into k ranges (partial tiles in the workspace, added by a second kernel):
+    264 tiles forward, 526 tiles in the data gradient.  With and without a workspace (no
+    workspace: no cut), against the oracle; the workspace query must ask for the partial
+    tiles on top of the permuted filter."""
+    p = (10, 32, 256, 41, 41, 1, 1, 1, 1, 3, 3)
+    N, C, K, H, W = p[:5]
+    cv = Conv(gpu, *p)
+    assert gpu.L.mnv_conv_fwd_workspace_bytes(*p) >= K * C * 9 * 4 + 8 * 2 * 128 * 128 * 4
+    x, w, b = _rand(N * C * H * W, 50), _rand(K * C * 9, 51, 0.1), _rand(K, 52)
+    ref = ora.conv_fwd(x, w, b, *p)
+    for ws in (True, False):
+        say("conv fwd, cut tail", p, ws)
+        assert normwise(cv.fwd(x, w, b, ws), ref) <= TOL
+    p = (20, 256, 32, 41, 41, 1, 1, 1, 1, 3, 3)
+    N, C, K, H, W = p[:5]
+    cv = Conv(gpu, *p)
+    assert gpu.L.mnv_conv_bwd_data_workspace_bytes(*p) >= K * C * 9 * 4 + 14 * 2 * 128 * 128 * 4
+    dy, w = _rand(N * K * H * W, 53), _rand(K * C * 9, 54, 0.1)
+    ref = ora.conv_bwd_data(dy, w, *p)
+    for ws in (True, False):
+        say("conv bwd data, cut tail", p, ws)
+        assert normwise(cv.bwd_data(dy, w, ws), ref) <= TOL
+
+
 ALEXNET = [
     # name, N, C, K, H, W, ph, pw, sv, sh, R, S   (owl/apps/imagenet_alexnet/alexnet.py:9-32)
     ("conv1", 1, 3, 96, 227, 227, 0, 0, 4, 4, 11, 11),
