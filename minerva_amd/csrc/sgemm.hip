@@ -220,13 +220,25 @@ SgemmPlan plan_sgemm(int m, int n, int k, size_t ws_floats) {
   return best;
 }
 
+// A launch without k ranges may use the workspace for the partial tiles of a cut tail.
 template <class P>
-int launch_plan(const SgemmPlan& plan, const P& p, void* workspace, hipStream_t s) {
+int launch_plan(const SgemmPlan& plan, const P& p, void* workspace, size_t workspace_bytes,
+                hipStream_t s) {
   if (plan.groups == 4)
     return plan.small ? mnv_gemm_launch<TileSmall, 4>(p, plan.splits, workspace, s)
                       : mnv_gemm_launch<TileBig, 4>(p, plan.splits, workspace, s);
-  return plan.small ? mnv_gemm_launch<TileSmall>(p, plan.splits, workspace, s)
-                    : mnv_gemm_launch<TileBig>(p, plan.splits, workspace, s);
+  const size_t tail_bytes = plan.splits == 1 && workspace ? workspace_bytes : 0;
+  return plan.small ? mnv_gemm_launch<TileSmall>(p, plan.splits, workspace, s, tail_bytes)
+                    : mnv_gemm_launch<TileBig>(p, plan.splits, workspace, s, tail_bytes);
+}
+
+// Bytes a product without k ranges wants for the partial tiles of its cut tail.
+size_t sgemm_tail_bytes(const SgemmPlan& plan, int m, int n, int k) {
+  if (plan.splits != 1 || plan.groups != 1) return 0;
+  const int bm = plan.small ? 64 : 128;
+  const long long tiles = (long long)((m + bm - 1) / bm) * ((n + bm - 1) / bm);
+  const MnvTailPlan t = mnv_tail_plan(tiles, (k + 15) / 16, (size_t)bm * bm, (size_t)-1 / sizeof(float));
+  return t.z > 1 ? (size_t)(tiles - t.begin) * t.z * bm * bm * sizeof(float) : 0;
 }
 
 #define MNV_MAX_DEVICES 64
@@ -255,8 +267,8 @@ int sgemm_nn_impl(const float* a, const float* b, float* c, int m, int n, int k,
   bool vec = (m % 4 == 0) && (k % 4 == 0) && mnv_aligned16(a) && mnv_aligned16(b) &&
              e.lda % 4 == 0 && e.ldb % 4 == 0;
   const SgemmPlan plan = plan_sgemm(m, n, k, workspace ? workspace_bytes / sizeof(float) : 0);
-  if (vec) return launch_plan(plan, make_sgemm<true>(a, b, c, m, n, k, e), workspace, s);
-  return launch_plan(plan, make_sgemm<false>(a, b, c, m, n, k, e), workspace, s);
+  if (vec) return launch_plan(plan, make_sgemm<true>(a, b, c, m, n, k, e), workspace, workspace_bytes, s);
+  return launch_plan(plan, make_sgemm<false>(a, b, c, m, n, k, e), workspace, workspace_bytes, s);
 }
 
 // Products with one operand given transposed: same plan (tile shape, k ranges) as the plain
@@ -267,8 +279,8 @@ int sgemm_t_impl(const float* a, const float* b, float* c, int m, int n, int k, 
   const bool vec = mnv_aligned16(a) && mnv_aligned16(b) && (TA ? k % 4 == 0 : m % 4 == 0) &&
                    (TB ? n % 4 == 0 : k % 4 == 0);
   const SgemmPlan plan = plan_sgemm(m, n, k, workspace ? workspace_bytes / sizeof(float) : 0);
-  if (vec) return launch_plan(plan, make_sgemm<true, TA, TB>(a, b, c, m, n, k, e), workspace, s);
-  return launch_plan(plan, make_sgemm<false, TA, TB>(a, b, c, m, n, k, e), workspace, s);
+  if (vec) return launch_plan(plan, make_sgemm<true, TA, TB>(a, b, c, m, n, k, e), workspace, workspace_bytes, s);
+  return launch_plan(plan, make_sgemm<false, TA, TB>(a, b, c, m, n, k, e), workspace, workspace_bytes, s);
 }
 
 // Operands of 2^29 elements and more (up to the reference's limit, int element counts): the
@@ -310,7 +322,7 @@ extern "C" {
 size_t mnv_sgemm_nn_workspace_bytes(int m, int n, int k) {
   if (m <= 0 || n <= 0 || k <= 0) return 0;
   const SgemmPlan plan = plan_sgemm(m, n, k, (size_t)-1);
-  return plan.splits > 1 ? (size_t)plan.splits * m * n * sizeof(float) : 0;
+  return plan.splits > 1 ? (size_t)plan.splits * m * n * sizeof(float) : sgemm_tail_bytes(plan, m, n, k);
 }
 
 int mnv_sgemm_nn_plan(int m, int n, int k, size_t workspace_bytes, int* tile_rows, int* k_ranges,

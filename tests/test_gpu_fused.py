@@ -147,7 +147,8 @@ def test_sgemm_fused_epilogues_equal_the_operator_chain(gpu, m, n, k, workspace)
 
 @pytest.mark.parametrize("m,n,k", [(7, 5, 3), (64, 64, 64), (130, 70, 33), (256, 784, 256), (784, 256, 10),
                                    (4096, 256, 1000), (1000, 256, 4096), (4096, 9216, 256),
-                                   (9216, 256, 4096), (100, 36, 5000), (132, 260, 68)])
+                                   (9216, 256, 4096), (100, 36, 5000), (132, 260, 68),
+                                   (2100, 2052, 260)])
 @pytest.mark.parametrize("workspace", [True, False])
 def test_sgemm_with_a_transposed_operand_equals_transpose_then_sgemm(gpu, m, n, k, workspace):
     """mnv_sgemm_tn / mnv_sgemm_nt against mnv_transpose followed by mnv_sgemm_nn (and

@@ -88,6 +88,27 @@ def test_sgemm_with_grouped_workgroups(gpu, m, n, k, workspace):
     assert_bits_equal(_gemm(gpu, a, b, m, n, k, workspace).reshape(n, m), got, "second call")
 
 
+@pytest.mark.parametrize("m,n,k", [(2100, 2100, 700), (2052, 2300, 261), (4224, 4100, 300)])
+def test_sgemm_with_a_cut_tail(gpu, m, n, k):
+    """Tile counts a little over a multiple of 256 (1089 and 1188 small tiles, 1089 large ones): with a
+    workspace the tiles past the multiple are cut into k ranges and added by a second
+    kernel; against the fp64 product, and against the same call without a workspace
+    (no cut) to the tolerance of two fp32 summation orders."""
+    assert gpu.L.mnv_sgemm_nn_workspace_bytes(m, n, k) > 0
+    assert _plan(gpu, m, n, k, gpu.L.mnv_sgemm_nn_workspace_bytes(m, n, k))[1:] == (1, 1)
+    a, b = _rand(m * k, 44), _rand(k * n, 45)
+    say("sgemm, cut tail", m, n, k)
+    got = _gemm(gpu, a, b, m, n, k, True).reshape(n, m)
+    plain = _gemm(gpu, a, b, m, n, k, False).reshape(n, m)
+    A = a.reshape(k, m).astype(np.float64)
+    B = b.reshape(n, k).astype(np.float64)
+    want = B @ A
+    assert normwise(got, want) <= TOL
+    assert normwise(plain, want) <= TOL
+    assert normwise(got, plain) <= 1e-5
+    assert_bits_equal(_gemm(gpu, a, b, m, n, k, True).reshape(n, m), got, "second call")
+
+
 def test_sgemm_reference_unit_test_shape(gpu):
     # tests/unittest_sgemm.cpp:7-28: {3,2} x {2,5} against the triple loop
     a = np.arange(6, dtype=np.float32)
