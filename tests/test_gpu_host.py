@@ -478,6 +478,47 @@ def test_alexnet_forward_batch_256_prefix_matches_oracle(ora):
     assert_bits_equal(w7, params["w7"] - step, "SGD update of w7 at b=256")
 
 
+def test_alexnet_gradients_batch_256_against_oracle_on_a_replicated_batch(ora):
+    """The backward pass at the benchmark's batch size, which the oracle cannot walk in
+    reasonable time: a batch of 64 copies of four images.  Weight and bias gradients are sums
+    over the images, so they must be 64 times the oracle's gradients for the four images
+    (the oracle's backward pass evaluated at the GPU's activations of the first copy: same
+    ReLU gates and pooling routes).  This runs every batch-256 kernel plan of the backward
+    pass (k ranges of the filter gradients, cut tails of the data gradients, grouped
+    workgroups of the inner products) against the oracle."""
+    from minerva_amd import hostapi
+    from oracle import nets
+    B, nb = 256, 4
+    params, data4, label4 = nets.make_inputs("alexnet", nb)
+    data = np.tile(data4, B // nb)
+    label = np.tile(label4, B // nb)
+    say("alexnet GPU step b=256 on 64 copies of 4 images")
+    r = hostapi.Runtime(0, sync_each_op=False)
+    net = hostapi.Net(r, "alexnet", B)
+    for k, v in params.items():
+        net.set_param(k, v)
+    net.load_batch(data, label)
+    net.keep_activations()
+    net.step(0.01)
+    r.sync()
+    prob = net.read("prob", 1000 * B)
+    acts = {i: net.read("act%d" % i, n * B) for i, n in ALEX_ACT_ELEMS.items()}
+    got = {k: net.read("g_" + k, n) for k, n in net.params.items()}
+    net.close()
+    r.close()
+    # every copy of an image must give the same probabilities (to rounding: copies that fall
+    # into differently cut tiles are summed in a different order)
+    P = prob.reshape(B // nb, nb * 1000)
+    assert normwise(P, np.broadcast_to(P[0], P.shape)) <= 1e-5
+    acts4 = [data4] + [acts[i][:n * nb] for i, n in sorted(ALEX_ACT_ELEMS.items())] + [None]
+    say("alexnet oracle backward b=4 at the GPU's activations (CPU)")
+    g4, _, _ = nets.alexnet_backward(params, acts4, np.ascontiguousarray(prob[:nb * 1000]), label4, nb)
+    worst = {k: normwise(got[k], np.float32(B // nb) * g4[k].astype(np.float64)) for k in sorted(params)}
+    say("  worst normwise error %.2e (%s)" % (max(worst.values()), max(worst, key=worst.get)))
+    bad = {k: v for k, v in worst.items() if not v <= TOL}
+    assert not bad, bad
+
+
 def test_alexnet_step_with_dropout_matches_oracle(ora):
     """The reference application's graph including drop6 / drop7: the masks come from the
     library's generator, which the oracle reproduces bit for bit from the seed sequence."""
