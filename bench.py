@@ -234,7 +234,7 @@ def dominant_kernel_roofline(prof, steps):
     avg_ms = total_ms / launches
     achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
     return {"bound": "mfma",
-            "kernel": "mnv_gemm_kernel<128x128x16,ConvBwdFilterFast<false>> (conv2-5 filter gradient)",
+            "kernel": "mnv_gemm_kernel<128x128x16,ConvBwdFilterFast<false,1|2>> (conv2-5 filter gradient)",
             "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
             "traffic": dominant_kernel_traffic(),

@@ -438,9 +438,20 @@ struct ConvBwdFilter {
 // NP ("no padding", any channel count): with ph == pw == 0 every tap of every output
 // position is a real pixel, so the pixel offset splits into a row part (channel, tap) and a
 // position part: one position table serves all rows, which stay in (channel, tap) order.
-template <bool NP>
+//
+// LK (padded convolutions whose channel count is a multiple of 16, so that every 16 rows of
+// a tile are 16 consecutive channels of one tap): the gathered operand is fetched with the
+// slab's 16 positions on 16 consecutive lanes.  A load instruction then reads 64 contiguous
+// bytes of each of four channel planes instead of 16 bytes of each of sixteen; a thread's
+// eight rows are 16 rows apart, so what distinguishes them (tap, first channel) is uniform
+// and lives in the workgroup's Res; and nothing else changes: same tile in LDS, same
+// products, same order.  LK = 1: all rows of a tile share one tap (channel counts that are
+// multiples of 128: one table entry and one add per thread and slab); LK = 2: a table entry
+// per row group.
+template <bool NP, int LK = 0>
 struct ConvBwdFilterFast {
   static constexpr bool A_KFAST = true, B_KFAST = true;
+  static constexpr bool A_LANE_K = LK != 0;
   static constexpr int A_NOFF = 1, B_NOFF = 1;
   const float* __restrict__ bottom;
   const float* __restrict__ top_diff;
@@ -456,6 +467,11 @@ struct ConvBwdFilterFast {
     mnv_rsrc a, b;
     const unsigned* tab;  // LDS: [taps_per_block][PP]
     int tap0;             // first tap of the workgroup's rows
+    // LK: row group j (rows m0 + 16 j ...) starts at channel c0: c0 * H * W * 4, its table
+    // row (tap - tap0) * PP, and whether it lies inside M
+    unsigned group_off[LK ? 8 : 1];
+    int group_trow[LK ? 8 : 1];
+    bool group_ok[LK ? 8 : 1];
   };
   struct AState {
     unsigned cbase;  // c*H*W*4, or MNV_OOB for rows past M
@@ -474,6 +490,15 @@ struct ConvBwdFilterFast {
     r.tab = tab;
     const int tap0 = mnv_fastdiv(m0, d_C);
     r.tap0 = tap0;
+    if (LK) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int row = m0 + 16 * j, tap = mnv_fastdiv(row, d_C);
+        r.group_off[j] = (unsigned)((row - tap * g.C) * g.HW) * 4u;
+        r.group_trow[j] = (tap - tap0 < taps_per_block ? tap - tap0 : 0) * PP;
+        r.group_ok[j] = row < M;
+      }
+    }
     for (int e = threadIdx.x; e < taps_per_block * PP; e += blockDim.x) {
       int t = e / PP, pos = e - t * PP;
       int tap = tap0 + t;
@@ -495,6 +520,11 @@ struct ConvBwdFilterFast {
       st.trow = 0;
       return;
     }
+    if (LK) {  // the thread's row inside its groups of 16: a channel offset
+      st.cbase = (unsigned)((m & 15) * g.HW) * 4u;
+      st.trow = 0;
+      return;
+    }
     int tap = mnv_fastdiv(m, d_C);
     int c = m - tap * g.C;
     st.cbase = m < M ? (unsigned)(c * g.HW) * 4u : MNV_OOB;
@@ -506,6 +536,24 @@ struct ConvBwdFilterFast {
   // come from the table every slab); a slab then adds s * 64 to it, one instruction
   __device__ void a_period(const AState& st, unsigned (&off)[1], int, int kl, int) const {
     off[0] = (unsigned)(st.trow + kl) * 4u;
+  }
+  template <int AV>
+  __device__ void a_load_lanek(const Res& r, const AState& st, int period, int s, int kl,
+                               float (&v)[AV][4]) const {
+    static_assert(AV * 4 <= 8, "row groups of a tile");
+    const unsigned img = (unsigned)period * (unsigned)(g.C * g.HW) * 4u;
+    const int pos = s * 16 + kl;
+    const unsigned one = st.cbase + r.tab[pos];
+#pragma unroll
+    for (int j = 0; j < AV * 4; ++j) {
+      unsigned voff = one;
+      if (LK == 2) {
+        voff = st.cbase + r.tab[r.group_trow[j] + pos];
+        voff = r.group_ok[j] ? voff : MNV_OOB;
+      }
+      v[j / 4][j % 4] = __builtin_bit_cast(
+          float, __builtin_amdgcn_raw_buffer_load_b32(r.a, (int)voff, (int)(img + r.group_off[j]), 0));
+    }
   }
   __device__ void a_load(const Res& r, const AState& st, const unsigned (&off)[1], int period, int s,
                          int, float (&v)[4]) const {
@@ -923,6 +971,17 @@ static int conv_bwd_filter_impl(const float* bottom, const float* top_diff, floa
   if (tile != 0 && ph == 0 && pw == 0 && (size_t)PP * 4 <= 24 * 1024) {
     ConvBwdFilterFast<true> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
                               PP / 16, PP, 1, mnv_fastdiv_make(C), accumulate, sgd_w, sgd_scale};
+    return launch_tile(tile, p, splits, workspace, s);
+  }
+  if (tile != 0 && C % 128 == 0 && (size_t)PP * 4 <= 24 * 1024) {
+    ConvBwdFilterFast<false, 1> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
+                                  PP / 16, PP, 1, mnv_fastdiv_make(C), accumulate, sgd_w, sgd_scale};
+    return launch_tile(tile, p, splits, workspace, s);
+  }
+  if (tile != 0 && C % 16 == 0 && (size_t)taps_per_block * PP * 4 <= 24 * 1024) {
+    ConvBwdFilterFast<false, 2> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
+                                  PP / 16, PP, taps_per_block, mnv_fastdiv_make(C), accumulate,
+                                  sgd_w, sgd_scale};
     return launch_tile(tile, p, splits, workspace, s);
   }
   if (tile != 0 && (size_t)taps_per_block * PP * 4 <= 24 * 1024) {

@@ -101,6 +101,13 @@ struct MnvFetchMap {
 //   void block_init(Res&, float* extra_lds, int m0, int n0) const;   once per workgroup,
 //        before the first load; a barrier follows it
 //   void c_store(int m, int n, float v) const;   only called for m < M, n < N
+//   optional, for a k-fast A whose k direction is contiguous in memory but whose rows are not
+//   (the gathered operand of the filter gradient): static constexpr bool A_LANE_K = true;
+//        The 16 k values of a slab then go to 16 consecutive lanes (a load instruction reads
+//        64 contiguous bytes of each of four rows) and a thread holds one k of the rows
+//        tid / 16 + 16 j.  a_init is called once, for row tid / 16, and
+//   void a_load_lanek(const Res&, const AState&, int period, int s, int kl, float (&v)[AV][4]) const;
+//        loads element j (row tid / 16 + 16 j, k = kl) into v[j / 4][j % 4]; a_period is unused
 //   optional, for a store that combines the product with a value read from memory:
 //   static constexpr bool C_PRELOAD = true;
 //   bool c_preload_on() const;                   uniform: whether this launch reads
@@ -108,6 +115,14 @@ struct MnvFetchMap {
 //   void c_store_with(int m, int n, float v, float pre) const;
 //        the kernel then reads the 16 values of a 32x32 block before it stores the block,
 //        so the reads are in flight together instead of one ahead of each store
+template <class P, class = void>
+struct MnvALaneK {
+  static constexpr bool value = false;
+};
+template <class P>
+struct MnvALaneK<P, std::enable_if_t<P::A_LANE_K>> {
+  static constexpr bool value = true;
+};
 template <class P, class = void>
 struct MnvCPreload {
   static constexpr bool value = false;
@@ -201,25 +216,37 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
   typename P::AState ast[T::AV];
   typename P::BState bst[T::BV];
   unsigned aoff[T::AV][P::A_NOFF], boff[T::BV][P::B_NOFF];
+  constexpr bool LK = MnvALaneK<P>::value;
+  static_assert(!LK || (P::A_KFAST && T::BK == 16 && T::NT == 256), "lane-per-k fetch: 16 x 16 threads");
+  if constexpr (LK) {
+    prob.a_init(res, ast[0], m0 + tid / 16);
+  } else {
 #pragma unroll
-  for (int p = 0; p < T::AV; ++p) prob.a_init(res, ast[p], m0 + MapA::x(tid, p));
+    for (int p = 0; p < T::AV; ++p) prob.a_init(res, ast[p], m0 + MapA::x(tid, p));
+  }
 #pragma unroll
   for (int p = 0; p < T::BV; ++p) prob.b_init(res, bst[p], n0 + MapB::x(tid, p));
 
   float ra[T::AV][4], rb[T::BV][4];
 
   auto new_period = [&](int period) {
+    if constexpr (!LK) {
 #pragma unroll
-    for (int p = 0; p < T::AV; ++p)
-      prob.a_period(ast[p], aoff[p], m0 + MapA::x(tid, p), MapA::k(tid, p), period);
+      for (int p = 0; p < T::AV; ++p)
+        prob.a_period(ast[p], aoff[p], m0 + MapA::x(tid, p), MapA::k(tid, p), period);
+    }
 #pragma unroll
     for (int p = 0; p < T::BV; ++p)
       prob.b_period(bst[p], boff[p], n0 + MapB::x(tid, p), MapB::k(tid, p), period);
   };
   auto fetch = [&](int period, int s) {
+    if constexpr (LK) {
+      prob.a_load_lanek(res, ast[0], period, s, tid % 16, ra);
+    } else {
 #pragma unroll
-    for (int p = 0; p < T::AV; ++p)
-      prob.a_load(res, ast[p], aoff[p], period, s, MapA::k(tid, p), ra[p]);
+      for (int p = 0; p < T::AV; ++p)
+        prob.a_load(res, ast[p], aoff[p], period, s, MapA::k(tid, p), ra[p]);
+    }
 #pragma unroll
     for (int p = 0; p < T::BV; ++p)
       prob.b_load(res, bst[p], boff[p], period, s, MapB::k(tid, p), rb[p]);
@@ -227,11 +254,17 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
   auto stash = [&](int buf) {
     float* a = As + buf * ATILE;
     float* bb = Bs + buf * BTILE;
+    if constexpr (LK) {  // element j: row tid / 16 + 16 j, k = tid % 16
 #pragma unroll
-    for (int p = 0; p < T::AV; ++p) {
-      const int x = MapA::x(tid, p), k = MapA::k(tid, p);
-      mnv_f4 v = {ra[p][0], ra[p][1], ra[p][2], ra[p][3]};
-      *reinterpret_cast<mnv_f4*>(a + (P::A_KFAST ? T::kaddr(x, k >> 2) : k * T::LDA + x)) = v;
+      for (int j = 0; j < T::AV * 4; ++j)
+        a[T::kaddr(tid / 16 + 16 * j, (tid % 16) >> 2) + (tid & 3)] = ra[j / 4][j % 4];
+    } else {
+#pragma unroll
+      for (int p = 0; p < T::AV; ++p) {
+        const int x = MapA::x(tid, p), k = MapA::k(tid, p);
+        mnv_f4 v = {ra[p][0], ra[p][1], ra[p][2], ra[p][3]};
+        *reinterpret_cast<mnv_f4*>(a + (P::A_KFAST ? T::kaddr(x, k >> 2) : k * T::LDA + x)) = v;
+      }
     }
 #pragma unroll
     for (int p = 0; p < T::BV; ++p) {
