@@ -167,14 +167,14 @@ def test_reader_of_lrn_scale_waits_for_the_forward_pass(ora):
     tx = r.tensor(x, dims)
     big = r.tensor(_rand(2048 * 2048, 6) / np.float32(45), [2048, 2048])
     for rep in range(3):
-        say("lrn scale reader, round", rep)
+        say("lrn scale reader, repetition", rep)
         busy = r.top("matmult", [big, big])          # keeps the producer's stream busy first
         busy = r.top("matmult", [busy, big])
         scale = r.top("fill", [], [0.0] + dims)
         top = r.top("lrn_forward", [tx, scale], [5, 1e-4, 0.75])
         twice = r.top("arithmetic_const", [scale], [2, 2.0, 0])   # reads `scale` alone
         if twice.stream == top.stream:
-            continue  # placement put both on one stream this round: stream order covers it
+            continue  # placement put both on one stream this time: stream order covers it
         got = twice.read()
         assert float(np.max(np.abs(got - 2 * want_scale))) <= 1e-4 * float(np.max(np.abs(want_scale)))
         assert float(np.max(np.abs(top.read() - want_top))) <= 1e-4 * float(np.max(np.abs(want_top)))
