@@ -46,7 +46,8 @@ HipDevice::~HipDevice() {
   StopWorkers();  // before the streams they launch on go away
   Activate();
   for (size_t i = 0; i < kParallelism; ++i) mnv_stream_sync(streams_[i]);
-  for (auto& kv : produced_) mnv_event_destroy(kv.second.event);
+  for (auto& e : latest_event_)
+    if (e) mnv_event_destroy(e);
   produced_.clear();
   data_store_.reset();  // before the streams: the deallocator uses the device
   for (size_t i = 0; i < kParallelism; ++i) {
@@ -75,7 +76,6 @@ std::string HipDevice::Name() const {
 void HipDevice::FreeDataIfExist(uint64_t data_id) {
   size_t erased;
   unsigned users = 0;
-  void* event = nullptr;
   erased = local_data_.Erase(data_id);
   {
     std::lock_guard<std::mutex> lck(local_mutex_);
@@ -84,11 +84,9 @@ void HipDevice::FreeDataIfExist(uint64_t data_id) {
       // The host may be far ahead of the GPU: kernels that read or write this block can
       // still be queued on these streams when the block goes back to the pool.
       users = it->second.users;
-      event = it->second.event;
       produced_.erase(it);
     }
   }
-  if (event) mnv_event_destroy(event);  // waits already queued on it keep their meaning
   if (erased == 1) data_store_->FreeData(data_id, users);
 }
 
@@ -98,6 +96,19 @@ void HipDevice::set_dataflow(bool v) {
   for (size_t i = 0; i < kParallelism; ++i) Ok(mnv_stream_sync(streams_[i]), "mode change sync");
   dataflow_ = v;
   if (v) sync_each_op_ = false;
+}
+
+// An event on `stream` that was recorded after operator number `seq` of that stream was
+// queued.  A replaced event is destroyed; waits already queued on it keep their meaning.
+void* HipDevice::EventCovering(int stream, uint64_t seq) {
+  if (latest_event_[stream] && latest_event_seq_[stream] >= seq) return latest_event_[stream];
+  void* e = nullptr;
+  Ok(mnv_event_create_ordering(&e), "event create");
+  Ok(mnv_event_record(e, streams_[stream]), "event record");
+  if (latest_event_[stream]) mnv_event_destroy(latest_event_[stream]);
+  latest_event_[stream] = e;
+  latest_event_seq_[stream] = queued_ops_[stream];
+  return e;
 }
 
 // Makes stream `thrid` wait for everything queued so far on each of `streams`.
@@ -148,22 +159,19 @@ void HipDevice::Execute(Task* task, int thrid) {
     // One GPU: every input is local.  A remote input would be copied here with
     // mnv_memcpy_d2d over xGMI, as DoCopyRemoteData does in the reference.
     MNV_CHECK_EQ(d.device_id, device_id_) << "remote inputs are not part of the one-GPU build";
-    void* wait_for = nullptr;
     MNV_CHECK_EQ(local_data_.Count(d.data_id), 1u) << "input data #" << d.data_id << " missing";
-    {
+    if (dataflow_) {
       std::lock_guard<std::mutex> lck(local_mutex_);
-      if (dataflow_) {
-        auto it = produced_.find(d.data_id);
-        if (it != produced_.end()) {
-          if (it->second.stream != thrid) wait_for = it->second.event;
-          it->second.users |= 1u << thrid;
+      auto it = produced_.find(d.data_id);
+      if (it != produced_.end()) {
+        // produced on another stream: this stream waits for the producer on the GPU
+        if (it->second.stream != thrid) {
+          Ok(mnv_stream_wait_event(streams_[thrid], EventCovering(it->second.stream, it->second.seq)),
+             "stream wait");
+          ++producer_waits_;
         }
+        it->second.users |= 1u << thrid;
       }
-    }
-    // produced on another stream: this stream waits for the producer on the GPU
-    if (wait_for) {
-      Ok(mnv_stream_wait_event(streams_[thrid], wait_for), "stream wait");
-      ++producer_waits_;
     }
     input_shards.emplace_back(data_store_->GetData(d.data_id), d.size);
   }
@@ -184,29 +192,18 @@ void HipDevice::Execute(Task* task, int thrid) {
     // an operator that fills one of its inputs (LRNForward's scale) is that datum's producer
     // from now on: later readers on other streams must wait for this operator, not for the
     // one that created the block
+    // The operator's kernels are queued: count it now, so that an event said to cover
+    // this number was recorded behind them.
+    std::lock_guard<std::mutex> lck(local_mutex_);
+    const uint64_t seq = ++queued_ops_[thrid];
     const int mutated = task->op.compute_fn->MutatedInput();
     if (mutated >= 0 && mutated < static_cast<int>(task->inputs.size())) {
-      void* e = nullptr;
-      Ok(mnv_event_create_ordering(&e), "event create");
-      Ok(mnv_event_record(e, streams_[thrid]), "event record");
-      void* old = nullptr;
-      {
-        std::lock_guard<std::mutex> lck(local_mutex_);
-        auto& p = produced_[task->inputs[mutated].physical_data.data_id];
-        old = p.event;
-        p.event = e;
-        p.stream = thrid;
-        p.users |= 1u << thrid;
-      }
-      if (old) mnv_event_destroy(old);
+      auto& p = produced_[task->inputs[mutated].physical_data.data_id];
+      p.seq = seq;
+      p.stream = thrid;
+      p.users |= 1u << thrid;
     }
-    for (auto& o : task->outputs) {
-      void* e = nullptr;
-      Ok(mnv_event_create_ordering(&e), "event create");
-      Ok(mnv_event_record(e, streams_[thrid]), "event record");
-      std::lock_guard<std::mutex> lck(local_mutex_);
-      produced_[o.physical_data.data_id] = Produced{e, thrid, 1u << thrid};
-    }
+    for (auto& o : task->outputs) produced_[o.physical_data.data_id] = Produced{seq, thrid, 1u << thrid};
   }
   if (listener_) listener_->OnOperationComplete(task);
 }

@@ -99,14 +99,23 @@ class HipDevice : public ThreadedDevice {
   bool sync_each_op_ = true;
   bool capturing_ = false;
   bool dataflow_ = false;
-  // dataflow mode, guarded by local_mutex_: where each datum was produced (stream, event
-  // recorded behind the producer) and which streams have work queued that touches it
+  // dataflow mode, guarded by local_mutex_: where each datum was produced (stream and the
+  // stream's operator count once the producer was queued) and which streams have work
+  // queued that touches it.  No event is recorded behind an operator: most consumers run
+  // on the producer's stream, and every event costs the GPU a few microseconds between two
+  // kernels.  A consumer on another stream asks for an event that covers the producer
+  // (EventCovering): the stream's latest event if it was recorded after the producer,
+  // otherwise a new one recorded now, behind everything the stream has been given so far.
   struct Produced {
-    void* event;
+    uint64_t seq;
     int stream;
     unsigned users;
   };
   std::unordered_map<uint64_t, Produced> produced_;
+  std::array<uint64_t, kParallelism> queued_ops_{};      // operators queued per stream
+  std::array<void*, kParallelism> latest_event_{};       // last event recorded per stream
+  std::array<uint64_t, kParallelism> latest_event_seq_{};  // queued_ops_ when it was recorded
+  void* EventCovering(int stream, uint64_t seq);  // call with local_mutex_ held
   void WaitForStreams(int thrid, unsigned streams);
   std::atomic<uint64_t> producer_waits_{0}, recycle_waits_{0};
   std::array<void*, kParallelism> streams_{};
