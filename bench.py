@@ -266,6 +266,16 @@ def sgemm_bench():
              "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
                           "unit": "TFLOP/s", "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}}
     log("sgemm 4096^3: %.3f ms, %.1f TFLOP/s" % (ms, tf))
+    # the same product with one operand given transposed (the operand is read in place: what
+    # the reference writes as Trans + MatMult); the values differ, the timing does not care
+    t_tn = dev.time_ms(lambda: L.mnv_sgemm_tn(a.p, b.p, None, c.p, m, n, k, None, 0, dev.stream),
+                       iters=10, warmup=5, reps=5)
+    t_nt = dev.time_ms(lambda: L.mnv_sgemm_nt(a.p, b.p, c.p, m, n, k, None, 0, dev.stream),
+                       iters=10, warmup=5, reps=5)
+    sgemm["transposed_operands"] = {
+        "A^T*B": {"ms": round(t_tn, 4), "tflops": round(2.0 * m * n * k / (t_tn * 1e-3) / 1e12, 2)},
+        "A*B^T": {"ms": round(t_nt, 4), "tflops": round(2.0 * m * n * k / (t_nt * 1e-3) / 1e12, 2)}}
+    log("sgemm 4096^3 with A / B transposed: %.3f / %.3f ms" % (t_tn, t_nt))
     # the other shapes of BASELINE.json configs[2], with the split-k workspace the host layer lends
     shapes = []
     for (mm, kk, nn) in ((256, 9216, 4096), (4096, 4096, 256), (1000, 4096, 256)):

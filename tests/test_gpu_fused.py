@@ -200,6 +200,25 @@ POOL = [
 ]
 
 
+def test_sgemm_transposed_operands_at_4096_cubed(gpu):
+    """The benchmark's square product with either operand given transposed: the bits of
+    transposing first (mnv_sgemm_nn at this size is checked against fp64 samples elsewhere)."""
+    n = 4096
+    a, b = _rand(n * n, 160, 0.1), _rand(n * n, 161)
+    da, db = gpu.up(a), gpu.up(b)
+    at, bt, prod = gpu.empty(n * n), gpu.empty(n * n), gpu.empty(n * n)
+    fused = gpu.up(np.full(n * n, np.nan, np.float32))
+    say("sgemm 4096^3 with transposed operands")
+    gpu.call("mnv_transpose", da.p, at.p, n, n)
+    gpu.call("mnv_transpose", db.p, bt.p, n, n)
+    gpu.call("mnv_sgemm_nn", da.p, db.p, prod.p, n, n, n, None, ctypes.c_size_t(0))
+    want = gpu.down(prod)
+    gpu.call("mnv_sgemm_tn", at.p, db.p, None, fused.p, n, n, n, None, ctypes.c_size_t(0))
+    assert_bits_equal(gpu.down(fused), want, "A given transposed, 4096^3")
+    gpu.call("mnv_sgemm_nt", da.p, bt.p, fused.p, n, n, n, None, ctypes.c_size_t(0))
+    assert_bits_equal(gpu.down(fused), want, "B given transposed, 4096^3")
+
+
 @pytest.mark.parametrize("p", POOL)
 def test_maxpool_bwd_relu_equals_the_operator_chain(gpu, ora, p):
     N, C, H, W, sv, sh, kh, kw, ph, pw = p
