@@ -267,6 +267,18 @@ int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filte
                         int stride_vertical, int stride_horizontal, int filter_height,
                         int filter_width, void* workspace, size_t workspace_bytes,
                         mnv_stream_t stream);
+/* How mnv_conv_bwd_filter launches a problem with a workspace of `workspace_bytes` on the
+ * current device (no reference counterpart: cuDNN chooses its algorithm out of sight,
+ * cuda_perform.cu:293-318): rows of the output tile (64 or 128); the k ranges the reduction
+ * over images and positions is cut into, each with a partial result in the workspace (1: none);
+ * and, when the launch is dealt to the chip in equal shares of tiles x k-slabs instead
+ * ("stream-k": k_ranges is then 1), the number of workgroups, else 0.  For a batch that runs
+ * as several launches, the plan of the first.  Launches nothing. */
+int mnv_conv_bwd_filter_plan(int num_images, int bottom_num_channels, int top_num_channels,
+                             int bottom_height, int bottom_width, int pad_height, int pad_width,
+                             int stride_vertical, int stride_horizontal, int filter_height,
+                             int filter_width, size_t workspace_bytes, int* tile_rows,
+                             int* k_ranges, int* streamk_workgroups);
 /* workspace (optional; 0 bytes = one workgroup per channel) lets each channel's sum be split
  * over image groups whose partial sums are added in a fixed order. */
 size_t mnv_conv_bwd_bias_workspace_bytes(int num_images, int top_num_channels);

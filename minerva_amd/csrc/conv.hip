@@ -447,7 +447,10 @@ struct ConvBwdFilter {
 // and lives in the workgroup's Res; and nothing else changes: same tile in LDS, same
 // products, same order.  LK = 1: all rows of a tile share one tap (channel counts that are
 // multiples of 128: one table entry and one add per thread and slab); LK = 2: a table entry
-// per row group.
+// per row group; LK = 3: the rows of a tile lie in at most two taps (96 channels: conv2 of the
+// AlexNet shape), so a thread reads two table entries per slab and every row group picks one
+// of the two by a uniform flag.  Row groups past M fetch whatever their offsets point at: their
+// accumulators are never stored.
 template <bool NP, int LK = 0>
 struct ConvBwdFilterFast {
   static constexpr bool A_KFAST = true, B_KFAST = true;
@@ -472,6 +475,7 @@ struct ConvBwdFilterFast {
     unsigned group_off[LK ? 8 : 1];
     int group_trow[LK ? 8 : 1];
     bool group_ok[LK ? 8 : 1];
+    bool group_second[LK ? 8 : 1];  // LK = 3: the group's rows lie in the tile's second tap
   };
   struct AState {
     unsigned cbase;  // c*H*W*4, or MNV_OOB for rows past M
@@ -497,6 +501,7 @@ struct ConvBwdFilterFast {
         r.group_off[j] = (unsigned)((row - tap * g.C) * g.HW) * 4u;
         r.group_trow[j] = (tap - tap0 < taps_per_block ? tap - tap0 : 0) * PP;
         r.group_ok[j] = row < M;
+        r.group_second[j] = tap - tap0 == 1;
       }
     }
     for (int e = threadIdx.x; e < taps_per_block * PP; e += blockDim.x) {
@@ -544,9 +549,11 @@ struct ConvBwdFilterFast {
     const unsigned img = (unsigned)period * (unsigned)(g.C * g.HW) * 4u;
     const int pos = s * 16 + kl;
     const unsigned one = st.cbase + r.tab[pos];
+    const unsigned two = LK == 3 ? st.cbase + r.tab[PP + pos] : 0u;
 #pragma unroll
     for (int j = 0; j < AV * 4; ++j) {
       unsigned voff = one;
+      if (LK == 3) voff = r.group_second[j] ? two : one;
       if (LK == 2) {
         voff = st.cbase + r.tab[r.group_trow[j] + pos];
         voff = r.group_ok[j] ? voff : MNV_OOB;
@@ -571,23 +578,22 @@ struct ConvBwdFilterFast {
   __device__ void b_period(const BState&, unsigned (&off)[1], int n, int kl, int) const {
     off[0] = n < N ? (unsigned)(n * g.HoWo + kl) * 4u : MNV_OOB;
   }
+  // Every slab is one 16-byte load per vector.  In the last slab of an image the positions
+  // past the image read whatever follows in memory (the next plane, or 0 past the tensor);
+  // b_stash_fix zeroes them on their way to LDS, when the values have arrived anyway.  (A
+  // branch to per-element loads at this point made the wavefront wait for every load in
+  // flight, the gathered operand's just-issued ones included, once per image.)
+  static constexpr bool B_STASH_FIX = true;
   __device__ void b_load(const Res& r, const BState&, const unsigned (&off)[1], int period, int s,
-                         int kl, float (&v)[4]) const {
+                         int, float (&v)[4]) const {
     const unsigned soff = ((unsigned)period * (unsigned)(g.K * g.HoWo) + (unsigned)s * 16u) * 4u;
-    if (s * 16 + 16 <= g.HoWo) {  // uniform: every position of the slab is inside the image
-      mnv_fetch_vec<1>(r.b, off, soff, v);
-    } else {
-      // the last slab of an image; the empty asm keeps its index arithmetic in this branch
-      // (hoisted above the test it would run in every slab: five vector instructions)
-      int first = s * 16 + kl;
-      asm volatile("" : "+v"(first));
+    mnv_fetch_vec<1>(r.b, off, soff, v);
+  }
+  __device__ void b_stash_fix(int s, int kl, float (&v)[4]) const {
+    if (s * 16 + 16 > g.HoWo) {  // uniform
+      const int first = s * 16 + kl;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        bool ok = first + q < g.HoWo;
-        v[q] = __builtin_bit_cast(
-            float, __builtin_amdgcn_raw_buffer_load_b32(r.b, (int)(ok ? off[0] + 4u * q : MNV_OOB),
-                                                        (int)soff, 0));
-      }
+      for (int q = 0; q < 4; ++q) v[q] = first + q < g.HoWo ? v[q] : 0.f;
     }
   }
   __device__ void c_store(int m, int n, float x) const {
@@ -653,6 +659,38 @@ int launch_tile(int tile, const P& p, int splits, void* ws, hipStream_t s, size_
   }
 }
 const int kTileM[4] = {64, 128, 128, 128}, kTileN[4] = {64, 128, 96, 32};
+
+// The filter gradient: few output tiles and a very long k.  On the large tiles it is dealt
+// to the chip in equal shares of tiles x k-slabs (stream-k) when the workspace holds the
+// shares' partial tiles; otherwise, and on the small tiles, in `splits` whole k ranges.
+// Slabs the filter gradient's loads run ahead (see mnv_gemm_kernel): two, which costs a
+// fourth workgroup per CU; measured on the four padded convolutions of the AlexNet shape, four
+// resident workgroups per CU with equal shares ran 16% slower than three (1.18 against
+// 1.03 ms per launch): the chip is then waiting for the L2 and fabric, not for the matrix pipe.
+#define MNV_SK_PF 2
+// `plan` (optional): nothing is launched; plan[0] = rows of the tile, plan[1] = k ranges,
+// plan[2] = workgroups of the stream-k launch (0: k ranges).
+template <class P>
+int launch_filter_gradient(int tile, const P& p, int splits, void* ws, size_t ws_bytes, hipStream_t s,
+                           int* plan = nullptr) {
+  if (plan) {
+    plan[0] = kTileM[tile];
+    plan[1] = splits;
+    plan[2] = 0;
+  }
+  if (tile == 1 || tile == 2) {
+    bool done = false;
+    int* wgs = plan ? plan + 2 : nullptr;
+    const int rc = tile == 1 ? mnv_gemm_streamk_launch<TileBig, MNV_SK_PF>(p, ws, ws_bytes, s, &done, wgs)
+                             : mnv_gemm_streamk_launch<Tile96, MNV_SK_PF>(p, ws, ws_bytes, s, &done, wgs);
+    if (rc || done) {
+      if (plan && done) plan[1] = 1;
+      return rc;
+    }
+  }
+  if (plan) return MNV_OK;
+  return launch_tile(tile, p, splits, ws, s);
+}
 
 // Bytes the large tiles' launches want for the partial tiles of a cut tail (0: no tail).
 size_t tail_workspace_bytes(int tile, int m, int n, int slabs) {
@@ -939,16 +977,27 @@ size_t mnv_conv_bwd_filter_workspace_bytes(int N, int C, int K, int H, int W, in
   ConvGeom g;
   if (make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S)) return 0;
   int splits = bwd_filter_splits(g.CRS, K, N * g.HoWo, (size_t)-1);
-  return splits > 1 ? (size_t)splits * g.CRS * K * sizeof(float) : 0;
+  size_t bytes = splits > 1 ? (size_t)splits * g.CRS * K * sizeof(float) : 0;
+  // the stream-k plan of the large tiles: at most four workgroups per CU, a partial tile each
+  // and one more per output tile
+  const int tile = bwd_filter_tile(g.CRS, K);
+  if (tile == 1 || tile == 2) {
+    const long long tiles = (long long)((g.CRS + kTileM[tile] - 1) / kTileM[tile]) *
+                            ((K + kTileN[tile] - 1) / kTileN[tile]);
+    const size_t sk = (size_t)(4 * mnv_cu_count() + tiles) * kTileM[tile] * kTileN[tile] * sizeof(float);
+    if (tiles <= 4LL * mnv_cu_count() && sk > bytes) bytes = sk;
+  }
+  return bytes;
 }
 
 static int conv_bwd_filter_impl(const float* bottom, const float* top_diff, float* filter_diff,
                                 int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh,
                                 int R, int S, void* workspace, size_t workspace_bytes,
                                 mnv_stream_t stream, int accumulate,
-                                const float* sgd_w = nullptr, float sgd_scale = 0.f) {
+                                const float* sgd_w = nullptr, float sgd_scale = 0.f,
+                                int* plan = nullptr) {
   ConvGeom g;
-  if (!bottom || !top_diff || !filter_diff) return MNV_ERR_INVALID;
+  if (!plan && (!bottom || !top_diff || !filter_diff)) return MNV_ERR_INVALID;
   int rc = make_geom(&g, N, C, K, H, W, ph, pw, sv, sh, R, S);
   if (rc) return rc;
   int gm = g.CRS, gn = K, gk = N * g.HoWo;
@@ -971,26 +1020,32 @@ static int conv_bwd_filter_impl(const float* bottom, const float* top_diff, floa
   if (tile != 0 && ph == 0 && pw == 0 && (size_t)PP * 4 <= 24 * 1024) {
     ConvBwdFilterFast<true> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
                               PP / 16, PP, 1, mnv_fastdiv_make(C), accumulate, sgd_w, sgd_scale};
-    return launch_tile(tile, p, splits, workspace, s);
+    return launch_filter_gradient(tile, p, splits, workspace, workspace_bytes, s, plan);
   }
   if (tile != 0 && C % 128 == 0 && (size_t)PP * 4 <= 24 * 1024) {
     ConvBwdFilterFast<false, 1> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
                                   PP / 16, PP, 1, mnv_fastdiv_make(C), accumulate, sgd_w, sgd_scale};
-    return launch_tile(tile, p, splits, workspace, s);
+    return launch_filter_gradient(tile, p, splits, workspace, workspace_bytes, s, plan);
+  }
+  if (tile != 0 && C % 16 == 0 && taps_per_block == 2 && (size_t)taps_per_block * PP * 4 <= 24 * 1024) {
+    ConvBwdFilterFast<false, 3> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
+                                  PP / 16, PP, taps_per_block, mnv_fastdiv_make(C), accumulate,
+                                  sgd_w, sgd_scale};
+    return launch_filter_gradient(tile, p, splits, workspace, workspace_bytes, s, plan);
   }
   if (tile != 0 && C % 16 == 0 && (size_t)taps_per_block * PP * 4 <= 24 * 1024) {
     ConvBwdFilterFast<false, 2> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
                                   PP / 16, PP, taps_per_block, mnv_fastdiv_make(C), accumulate,
                                   sgd_w, sgd_scale};
-    return launch_tile(tile, p, splits, workspace, s);
+    return launch_filter_gradient(tile, p, splits, workspace, workspace_bytes, s, plan);
   }
   if (tile != 0 && (size_t)taps_per_block * PP * 4 <= 24 * 1024) {
     ConvBwdFilterFast<false> p{bottom, top_diff, filter_diff, g, gm, gn, gk, N * (PP / 16),
                                PP / 16, PP, taps_per_block, mnv_fastdiv_make(C), accumulate, sgd_w, sgd_scale};
-    return launch_tile(tile, p, splits, workspace, s);
+    return launch_filter_gradient(tile, p, splits, workspace, workspace_bytes, s, plan);
   }
   ConvBwdFilter p{bottom, top_diff, filter_diff, g, gm, gn, gk, (gk + 15) / 16, 1, accumulate, sgd_w, sgd_scale};
-  return launch_tile(tile, p, splits, workspace, s);
+  return launch_filter_gradient(tile, p, splits, workspace, workspace_bytes, s, plan);
 }
 
 int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filter_diff, int N,
@@ -1010,6 +1065,23 @@ int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filte
                                   stream, n0 > 0);
     if (rc) return rc;
   }
+  return MNV_OK;
+}
+
+int mnv_conv_bwd_filter_plan(int N, int C, int K, int H, int W, int ph, int pw, int sv, int sh, int R,
+                             int S, size_t workspace_bytes, int* tile_rows, int* k_ranges,
+                             int* streamk_workgroups) {
+  int plan[3] = {0, 0, 0};
+  const int chunk = images_per_launch(N, C, K, H, W, ph, pw, sv, sh, R, S);
+  if (chunk <= 0) return MNV_ERR_INVALID;
+  // the workspace is only compared with sizes here, never dereferenced
+  void* some = workspace_bytes ? reinterpret_cast<void*>(&plan) : nullptr;
+  int rc = conv_bwd_filter_impl(nullptr, nullptr, nullptr, chunk < N ? chunk : N, C, K, H, W, ph, pw, sv,
+                                sh, R, S, some, workspace_bytes, nullptr, 0, nullptr, 0.f, plan);
+  if (rc) return rc;
+  if (tile_rows) *tile_rows = plan[0];
+  if (k_ranges) *k_ranges = plan[1];
+  if (streamk_workgroups) *streamk_workgroups = plan[2];
   return MNV_OK;
 }
 

@@ -3,7 +3,26 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "mnv_common.h"
+
+int mnv_cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  cached[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
 
 extern "C" {
 

@@ -18,6 +18,7 @@
 //
 // Roofline: fp32 MFMA, 2*M*N*K algorithmic flops; 256 flop/clk/CU.
 #pragma once
+#include <atomic>
 #include <type_traits>
 
 #include "mnv_common.h"
@@ -108,6 +109,10 @@ struct MnvFetchMap {
 //        tid / 16 + 16 j.  a_init is called once, for row tid / 16, and
 //   void a_load_lanek(const Res&, const AState&, int period, int s, int kl, float (&v)[AV][4]) const;
 //        loads element j (row tid / 16 + 16 j, k = kl) into v[j / 4][j % 4]; a_period is unused
+//   optional, for a right operand whose loads may fetch values that must read as 0 and that are
+//   cheaper to clear once they have arrived: static constexpr bool B_STASH_FIX = true;
+//   void b_stash_fix(int s, int kl, float (&v)[4]) const;   called on every vector of slab s of
+//        its period right before the vector is written to LDS
 //   optional, for a store that combines the product with a value read from memory:
 //   static constexpr bool C_PRELOAD = true;
 //   bool c_preload_on() const;                   uniform: whether this launch reads
@@ -121,6 +126,14 @@ struct MnvALaneK {
 };
 template <class P>
 struct MnvALaneK<P, std::enable_if_t<P::A_LANE_K>> {
+  static constexpr bool value = true;
+};
+template <class P, class = void>
+struct MnvBStashFix {
+  static constexpr bool value = false;
+};
+template <class P>
+struct MnvBStashFix<P, std::enable_if_t<P::B_STASH_FIX>> {
   static constexpr bool value = true;
 };
 template <class P, class = void>
@@ -166,10 +179,30 @@ __device__ __forceinline__ int mnv_tile_remap(int t, int total) {
 // order ((g0 + g2) + (g1 + g3)) and group 0 stores.  For a product with few output tiles and
 // a long k this keeps 16 wavefronts per CU busy with a quarter of the partial results (and of
 // the reduction kernel's reads) that as many separate workgroups would write to memory.
-template <class T, class P, int G = 1>
-__global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
+//
+// SK ("stream-k"): the launch has exactly as many workgroups as the chip holds at once and
+// the tiles x k-slabs of the whole product, laid end to end (tile-major), are dealt to them in
+// equal contiguous shares: workgroup w multiplies the units [U w / W, U (w + 1) / W).  A share
+// that crosses a tile boundary is worked off segment by segment; every segment leaves its
+// partial tile in slot w + tile of the workspace (w and tile never decrease from one segment
+// to the next and one of them grows, so the slots are distinct and W + tiles - 1 in number)
+// and mnv_gemm_streamk_reduce_kernel adds a tile's segments in workgroup order, which is
+// k order: deterministic.  With whole k ranges per workgroup (blockIdx.z) the chip works in
+// rounds of equal workgroups, and a count of workgroups that is not a multiple of what the
+// chip holds leaves part of it idle for a whole round (54 tiles x 28 ranges = 1512 workgroups
+// on 1024 slots: the second round runs half empty).
+//
+// PF: slabs the loads run ahead of the multiplies.  1: the loads of slab i + 1 are issued at
+// the head of slab i and written to LDS at its end, through one set of staging registers
+// (the kernel then fits 128 registers: four workgroups per CU).  2: a second set of staging
+// registers lets the loads of slab i + 2 start at the head of slab i, so that a trip to
+// memory may take two slab times instead of one; 24 more registers, three workgroups per CU.
+template <class T, class P, int G = 1, bool SK = false, int PF = 1>
+__global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MIN_WAVES) void mnv_gemm_kernel(
     P prob, int tiles_m, int tiles_n, int slabs_per_split, float* __restrict__ partial,
     int tail_begin, int tail_z) {
+  static_assert(!SK || G == 1, "stream-k shares are per workgroup");
+  static_assert(PF == 1 || (PF == 2 && G == 1), "one or two slabs ahead");
   extern __shared__ float mnv_gemm_lds[];
   constexpr int ATILE = T::a_tile(P::A_KFAST), BTILE = T::b_tile(P::B_KFAST);
   constexpr int GROUP_FLOATS = 2 * (ATILE + BTILE);
@@ -181,19 +214,34 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
   typedef MnvFetchMap<T::BM, T::BK, T::NT, P::A_KFAST> MapA;
   typedef MnvFetchMap<T::BN, T::BK, T::NT, P::B_KFAST> MapB;
 
+  // SK: the units of this workgroup that are still to do
+  long long sk_u = 0, sk_end = 0;
+  if constexpr (SK) {
+    const long long units = (long long)tiles_m * tiles_n * prob.total_slabs;
+    sk_u = units * blockIdx.x / gridDim.x;
+    sk_end = units * (blockIdx.x + 1) / gridDim.x;
+    if (sk_u >= sk_end) return;
+  }
+  for (;;) {  // SK: one pass per segment; otherwise a single pass that ends in a return
   int vb = blockIdx.x, tail_part = -1;
-  if (G == 1 && tail_z > 1 && vb >= tail_begin) {
+  if (!SK && G == 1 && tail_z > 1 && vb >= tail_begin) {
     const int i = vb - tail_begin, tl = i / tail_z;
     tail_part = i - tl * tail_z;
     vb = tail_begin + tl;
   }
-  const int b = mnv_tile_remap(vb, tiles_m * tiles_n);
+  if constexpr (SK) vb = (int)(sk_u / prob.total_slabs);
+  const int b = SK ? vb : mnv_tile_remap(vb, tiles_m * tiles_n);
   const int tile_m = b % tiles_m, tile_n = b / tiles_m;
   const int m0 = tile_m * T::BM, n0 = tile_n * T::BNU;
 
   int slab_begin = blockIdx.z * slabs_per_split;
   int slab_end = slab_begin + slabs_per_split;
   if (slab_end > prob.total_slabs) slab_end = prob.total_slabs;
+  if constexpr (SK) {
+    slab_begin = (int)(sk_u - (long long)vb * prob.total_slabs);
+    const long long left = sk_end - sk_u;
+    slab_end = left < prob.total_slabs - slab_begin ? slab_begin + (int)left : prob.total_slabs;
+  }
   // slabs every group steps through (the same count in all of them: the steps hold
   // workgroup barriers); a group whose quarter is shorter multiplies only its own slabs
   if (G == 1 && tail_part >= 0) {
@@ -227,7 +275,7 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
 #pragma unroll
   for (int p = 0; p < T::BV; ++p) prob.b_init(res, bst[p], n0 + MapB::x(tid, p));
 
-  float ra[T::AV][4], rb[T::BV][4];
+  float ra[PF][T::AV][4], rb[PF][T::BV][4];  // staging set of slab j: j % PF
 
   auto new_period = [&](int period) {
     if constexpr (!LK) {
@@ -239,37 +287,45 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
     for (int p = 0; p < T::BV; ++p)
       prob.b_period(bst[p], boff[p], n0 + MapB::x(tid, p), MapB::k(tid, p), period);
   };
-  auto fetch = [&](int period, int s) {
+  int s_of_set[PF] = {};  // slab (inside its period) that each staging set holds
+  auto fetch = [&](int period, int s, auto SET) {
+    constexpr int set = decltype(SET)::value;
+    s_of_set[set] = s;
     if constexpr (LK) {
-      prob.a_load_lanek(res, ast[0], period, s, tid % 16, ra);
+      prob.a_load_lanek(res, ast[0], period, s, tid % 16, ra[set]);
     } else {
 #pragma unroll
       for (int p = 0; p < T::AV; ++p)
-        prob.a_load(res, ast[p], aoff[p], period, s, MapA::k(tid, p), ra[p]);
+        prob.a_load(res, ast[p], aoff[p], period, s, MapA::k(tid, p), ra[set][p]);
     }
 #pragma unroll
     for (int p = 0; p < T::BV; ++p)
-      prob.b_load(res, bst[p], boff[p], period, s, MapB::k(tid, p), rb[p]);
+      prob.b_load(res, bst[p], boff[p], period, s, MapB::k(tid, p), rb[set][p]);
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int buf, auto SET) {
+    constexpr int set = decltype(SET)::value;
     float* a = As + buf * ATILE;
     float* bb = Bs + buf * BTILE;
+    if constexpr (MnvBStashFix<P>::value) {
+#pragma unroll
+      for (int p = 0; p < T::BV; ++p) prob.b_stash_fix(s_of_set[set], MapB::k(tid, p), rb[set][p]);
+    }
     if constexpr (LK) {  // element j: row tid / 16 + 16 j, k = tid % 16
 #pragma unroll
       for (int j = 0; j < T::AV * 4; ++j)
-        a[T::kaddr(tid / 16 + 16 * j, (tid % 16) >> 2) + (tid & 3)] = ra[j / 4][j % 4];
+        a[T::kaddr(tid / 16 + 16 * j, (tid % 16) >> 2) + (tid & 3)] = ra[set][j / 4][j % 4];
     } else {
 #pragma unroll
       for (int p = 0; p < T::AV; ++p) {
         const int x = MapA::x(tid, p), k = MapA::k(tid, p);
-        mnv_f4 v = {ra[p][0], ra[p][1], ra[p][2], ra[p][3]};
+        mnv_f4 v = {ra[set][p][0], ra[set][p][1], ra[set][p][2], ra[set][p][3]};
         *reinterpret_cast<mnv_f4*>(a + (P::A_KFAST ? T::kaddr(x, k >> 2) : k * T::LDA + x)) = v;
       }
     }
 #pragma unroll
     for (int p = 0; p < T::BV; ++p) {
       const int x = MapB::x(tid, p), k = MapB::k(tid, p);
-      mnv_f4 v = {rb[p][0], rb[p][1], rb[p][2], rb[p][3]};
+      mnv_f4 v = {rb[set][p][0], rb[set][p][1], rb[set][p][2], rb[set][p][3]};
       *reinterpret_cast<mnv_f4*>(bb + (P::B_KFAST ? T::kaddr(x, k >> 2) : k * T::LDB + x)) = v;
     }
   };
@@ -289,10 +345,19 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
   // (period, s) of the slab whose loads are issued next
   int period = slab_begin / prob.spp, s = slab_begin - period * prob.spp;
   __syncthreads();  // block_init may have written LDS
+  typedef std::integral_constant<int, 0> Set0;
+  typedef std::integral_constant<int, PF - 1> Set1;
   if (slab_begin < slab_end) {
     new_period(period);
-    fetch(period, s);
-    stash(0);
+    fetch(period, s, Set0{});
+    if constexpr (PF == 2) {
+      if (++s == prob.spp) {
+        s = 0;
+        new_period(++period);
+      }
+      fetch(period, s, Set1{});
+    }
+    stash(0, Set0{});
   }
   __syncthreads();
 
@@ -309,11 +374,14 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
       s = 0;
       new_period(++period);
     }
-    fetch(period, s);
-    // Keep the loads up here: left alone, the scheduler sinks them below most of the
-    // multiplies to shorten register lifetimes, and each wavefront then waits out the
-    // full memory latency once per slab.
-    __builtin_amdgcn_sched_barrier(0);
+    fetch(period, s, std::integral_constant<int, PF == 2 ? buf : 0>{});
+    // One slab ahead, keep the loads up here: left alone, the scheduler sinks them below most
+    // of the multiplies to shorten register lifetimes, and each wavefront then waits out the
+    // full memory latency once per slab.  Two slabs ahead that is exactly what is wanted: the
+    // loads have a whole slab of slack, and issued in the shadow of the multiplies they cost
+    // the wavefront no issue slots at the head of the slab, where its four operand reads and
+    // the first multiply wait (filter gradients of the AlexNet shape: 1.014 -> 0.987 ms).
+    if (PF == 1) __builtin_amdgcn_sched_barrier(0);
     // A round multiplies 8 k values: MFMA step t pairs k = 8h + t (lanes 0..31) with
     // k = 8h + 4 + t (lanes 32..63), so a lane's four steps use four consecutive k.
     const float* a = As + buf * ATILE;
@@ -354,7 +422,7 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv[j][t], av[i][t], acc[i][j], 0, 0, 0);
     }
     }
-    stash(buf ^ 1);
+    stash(buf ^ 1, std::integral_constant<int, PF == 2 ? (buf ^ 1) : 0>{});
     __syncthreads();
   };
   int slab = slab_begin;
@@ -402,6 +470,26 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
 
   // Accumulator register r of lane (lm, lk) holds C[m = lm, n = lk*4 + r%4 + 8*(r/4)]
   // of its 32x32 block.
+  if constexpr (SK) {  // a segment: the whole tile, in tile order, into slot w + tile
+    // The empty asm keeps the store addresses from being computed once before the segment
+    // loop (they do not change from segment to segment): 64 registers held across the main
+    // loop would spill.
+    int at = (wn + lk * 4) * T::BM + wm + lm;
+    asm volatile("" : "+v"(at));
+    float* pt = partial + (size_t)(blockIdx.x + vb) * (T::BM * T::BNU) + at;
+#pragma unroll
+    for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < T::TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          pt[(j * 32 + (r & 3) + 8 * (r >> 2)) * T::BM + i * 32] = acc[i][j][r];
+    sk_u += slab_end - slab_begin;
+    if (sk_u >= sk_end) return;
+    // every wavefront is past the last slab's barrier: the tile buffers and the policy's
+    // LDS are free for the next segment
+    continue;
+  }
   if (G == 1 && tail_part >= 0) {  // a k range of a tail tile: the whole tile, in tile order
     float* pt = partial + ((size_t)(vb - tail_begin) * tail_z + tail_part) * (T::BM * T::BNU);
 #pragma unroll
@@ -454,6 +542,8 @@ __global__ __launch_bounds__(T::NT * G, T::MIN_WAVES) void mnv_gemm_kernel(
         }
       }
   }
+  return;
+  }  // for (;;)
 }
 
 // Sums the per-split partial results in a fixed order (deterministic) and hands each
@@ -538,6 +628,53 @@ __global__ __launch_bounds__(256) void mnv_gemm_tail_reduce_kernel(P prob,
   }
 }
 
+// Adds the segments of every tile of a stream-k launch (see mnv_gemm_kernel) in workgroup
+// order and hands each element to the policy's store.  Workgroup w of the launch covered the
+// units [U w / W, U (w + 1) / W); tile t is the units [t S, (t + 1) S).  One thread per four
+// consecutive rows of a tile column; four segments' loads in flight.
+template <class T, class P>
+__global__ __launch_bounds__(256) void mnv_gemm_streamk_reduce_kernel(P prob,
+                                                                      const float* __restrict__ partial,
+                                                                      int tiles_m, int tiles_n,
+                                                                      int workgroups) {
+  constexpr int TILE = T::BM * T::BNU;
+  const int t = blockIdx.y;
+  const long long S = prob.total_slabs, U = S * tiles_m * tiles_n, W = workgroups;
+  const long long first = t * S, last = first + S;
+  long long w0 = first * W / U;                  // U w0 / W <= first
+  while (U * (w0 + 1) / W <= first) ++w0;        // the share that holds the tile's first unit
+  long long w1 = w0 + 1;
+  while (w1 < W && U * w1 / W < last) ++w1;      // one past the share that holds its last unit
+  const int m0 = (t % tiles_m) * T::BM, n0 = (t / tiles_m) * T::BNU;
+  const int count = (int)(w1 - w0);
+  const float* p = partial + (size_t)(w0 + t) * TILE;
+  for (int e = (blockIdx.x * 256 + threadIdx.x) * 4; e < TILE; e += gridDim.x * 256 * 4) {
+    mnv_f4 s = *reinterpret_cast<const mnv_f4*>(p + e);
+    int z = 1;
+    for (; z + 3 < count; z += 4) {
+      const mnv_f4 v0 = *reinterpret_cast<const mnv_f4*>(p + (size_t)z * TILE + e);
+      const mnv_f4 v1 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + 1) * TILE + e);
+      const mnv_f4 v2 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + 2) * TILE + e);
+      const mnv_f4 v3 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + 3) * TILE + e);
+      s.x += v0.x; s.y += v0.y; s.z += v0.z; s.w += v0.w;
+      s.x += v1.x; s.y += v1.y; s.z += v1.z; s.w += v1.w;
+      s.x += v2.x; s.y += v2.y; s.z += v2.z; s.w += v2.w;
+      s.x += v3.x; s.y += v3.y; s.z += v3.z; s.w += v3.w;
+    }
+    for (; z < count; ++z) {
+      const mnv_f4 v = *reinterpret_cast<const mnv_f4*>(p + (size_t)z * TILE + e);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    const int m = m0 + e % T::BM, n = n0 + e / T::BM;
+    if (n < prob.N) {
+      if (m + 0 < prob.M) prob.c_store(m + 0, n, s.x);
+      if (m + 1 < prob.M) prob.c_store(m + 1, n, s.y);
+      if (m + 2 < prob.M) prob.c_store(m + 2, n, s.z);
+      if (m + 3 < prob.M) prob.c_store(m + 3, n, s.w);
+    }
+  }
+}
+
 // Which tiles form the tail and into how many k ranges each is cut (z <= 1: none).  Only
 // for launches of at least 256 large tiles without k ranges of their own; taken when the
 // uneven last tile per CU costs at least 3% (tiles / 256 = 2.64: 12%; 11.39: 5%; 3.96: 1%),
@@ -609,7 +746,7 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
   if ((long long)tiles_m * tiles_n > 0x7fffffffLL || splits > 65535) return MNV_ERR_INVALID;
   // The LDS limit of a kernel is an attribute per device; set once on each (idempotent: a
   // race only repeats the same call).
-  static bool attr_set[64] = {};
+  static std::atomic<bool> attr_set[64];
   const size_t tile_bytes = G * T::lds_bytes(P::A_KFAST, P::B_KFAST);
   const size_t lds_limit = (G > 1 ? 160 : 64) * 1024;
   if (G > 1 && prob.extra_lds_bytes()) return MNV_ERR_INVALID;  // groups use every tile buffer
@@ -617,10 +754,10 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
     int dev = 0;
     MNV_HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= 64) return MNV_ERR_INVALID;
-    if (!attr_set[dev]) {
+    if (!attr_set[dev].load(std::memory_order_acquire)) {
       MNV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&mnv_gemm_kernel<T, P, G>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_limit));
-      attr_set[dev] = true;
+      attr_set[dev].store(true, std::memory_order_release);
     }
   }
   const size_t lds_bytes = tile_bytes + prob.extra_lds_bytes();
@@ -653,5 +790,69 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
     else rc = mnv_gemm_splitk_reduce_launch<P, 64>(prob, part, splits, s);
   }
   return rc;
+}
+
+// Stream-k launch of one tile configuration (see mnv_gemm_kernel): as many workgroups as the
+// current device holds at once, equal shares of the tiles x k-slabs, then the reduction.
+// `*done` is false, and nothing was launched, when the plan does not apply: fewer than eight
+// slabs per workgroup, more tiles than workgroups, or a workspace under
+// mnv_gemm_streamk_bytes.  The plan depends on the extents, the device (its CU count and how
+// many of the kernel's workgroups a CU holds) and nothing else.
+template <class T>
+static inline size_t mnv_gemm_streamk_bytes(long long tiles, int workgroups) {
+  return (size_t)(workgroups + tiles - 1) * T::BM * T::BNU * sizeof(float);
+}
+
+// `plan_workgroups` (optional): receives the number of workgroups of the plan, 0 when it
+// does not apply, and nothing is launched.
+template <class T, int PF = 1, class P>
+static int mnv_gemm_streamk_launch(const P& prob, void* workspace, size_t ws_bytes, hipStream_t s,
+                                   bool* done, int* plan_workgroups = nullptr) {
+  *done = false;
+  if (plan_workgroups) *plan_workgroups = 0;
+  const int tiles_m = (prob.M + T::BM - 1) / T::BM, tiles_n = (prob.N + T::BNU - 1) / T::BNU;
+  const long long tiles = (long long)tiles_m * tiles_n;
+  const size_t lds_bytes = T::lds_bytes(P::A_KFAST, P::B_KFAST) + prob.extra_lds_bytes();
+  if (!workspace || prob.total_slabs <= 0 || tiles > 0x7fffffffLL / prob.total_slabs ||
+      lds_bytes > 64 * 1024)
+    return MNV_OK;
+  int dev = 0;
+  MNV_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) return MNV_ERR_INVALID;
+  const void* fn = reinterpret_cast<const void*>(&mnv_gemm_kernel<T, P, 1, true, PF>);
+  // (LDS bytes << 8 | workgroups per CU) of the last query on each device
+  static std::atomic<unsigned long long> cached[64];
+  static std::atomic<bool> attr_set[64];
+  if (lds_bytes > 48 * 1024 && !attr_set[dev].load(std::memory_order_acquire)) {
+    MNV_HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+    attr_set[dev].store(true, std::memory_order_release);
+  }
+  unsigned long long c = cached[dev].load(std::memory_order_relaxed);
+  if ((c >> 8) != lds_bytes || (c & 255) == 0) {
+    int per_cu = 0;
+    MNV_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, T::NT, lds_bytes));
+    if (per_cu < 1) return MNV_OK;
+    if (per_cu > 255) per_cu = 255;
+    c = ((unsigned long long)lds_bytes << 8) | (unsigned)per_cu;
+    cached[dev].store(c, std::memory_order_relaxed);
+  }
+  const int workgroups = (int)(c & 255) * mnv_cu_count();
+  if (tiles > workgroups || tiles * prob.total_slabs < 8LL * workgroups ||
+      ws_bytes < mnv_gemm_streamk_bytes<T>(tiles, workgroups))
+    return MNV_OK;
+  if (plan_workgroups) {
+    *plan_workgroups = workgroups;
+    *done = true;
+    return MNV_OK;
+  }
+  hipLaunchKernelGGL((mnv_gemm_kernel<T, P, 1, true, PF>), dim3(workgroups), dim3(T::NT), lds_bytes, s,
+                     prob, tiles_m, tiles_n, 0, reinterpret_cast<float*>(workspace), 0, 1);
+  int rc = MNV_LAUNCH_STATUS();
+  if (rc) return rc;
+  hipLaunchKernelGGL((mnv_gemm_streamk_reduce_kernel<T, P>),
+                     dim3(T::BM * T::BNU / 1024, (unsigned)tiles), dim3(256), 0, s, prob,
+                     reinterpret_cast<const float*>(workspace), tiles_m, tiles_n, workgroups);
+  *done = true;
+  return MNV_LAUNCH_STATUS();
 }
 #endif  // __HIPCC__

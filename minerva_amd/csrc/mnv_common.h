@@ -24,6 +24,10 @@ static inline bool mnv_aligned16(const void* p) { return (reinterpret_cast<uintp
 
 static inline size_t mnv_ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
 
+// Compute units of the current device (cached per device; 256, the MI355X's count, when no
+// device can be asked, so that size queries work on a machine without a GPU).
+int mnv_cu_count();
+
 // Upper bound on grid.x for grid-stride kernels: enough resident work for
 // 256 CUs without paying launch cost for millions of tiny blocks.
 #define MNV_MAX_STREAM_BLOCKS 16384u

@@ -234,12 +234,100 @@ def test_conv_batch_256_properties(gpu, case):
     say(name, "b256 bwd filter")
     dw = cv.bwd_filter(dy, x)
     assert abs(float(np.dot(dw.astype(np.float64), w.astype(np.float64))) - lhs) <= 1e-5 * scale
+    # sampled filter-gradient entries against fp64 sums over the 256 distinct images, written
+    # from the definition (cuda_perform.cu:293-318 hands the same sum to cuDNN): corners of
+    # the (k, c, tap) index space first, where tile edges, channel groups and padded taps
+    # live, then random entries.  One scalar identity cannot see a wrong tap or an image
+    # counted twice; one entry out of place fails here by its whole size.
+    DY = dy.reshape(N, K, cv.Ho, cv.Wo)
+    DW = dw.reshape(K, C, R, S)
+    picks = [(k, c, r, s_) for k in (0, K - 1) for c in (0, C - 1) for r in (0, R - 1)
+             for s_ in (0, S - 1)]
+    picks += [(K // 2, C // 2, R // 2, S // 2), (127 % K, 15 % C, 0, S - 1), (128 % K, 16 % C, R - 1, 0)]
+    while len(picks) < 72:
+        picks.append((int(rng.integers(K)), int(rng.integers(C)), int(rng.integers(R)),
+                      int(rng.integers(S))))
+    worst, top = 0.0, float(np.max(np.abs(dw)))
+    for (k, c, r, s_) in picks:
+        rf, sf = R - 1 - r, S - 1 - s_          # the tap of the flipped filter
+        i = np.arange(cv.Ho)
+        j = np.arange(cv.Wo)
+        i = i[(i * sv - ph + rf >= 0) & (i * sv - ph + rf < H)]
+        j = j[(j * sh - pw + sf >= 0) & (j * sh - pw + sf < W)]
+        xs = X[:, c][:, i * sv - ph + rf][:, :, j * sh - pw + sf].astype(np.float64)
+        want = float(np.sum(xs * DY[:, k][:, i][:, :, j]))
+        worst = max(worst, abs(float(DW[k, c, r, s_]) - want))
+    assert worst <= TOL * top, "filter gradient entry off by %.3e of %.3e" % (worst, top)
     if name != "conv1":  # the network never asks for conv1's data gradient
         say(name, "b256 bwd data")
         dx = cv.bwd_data(dy, w)
         assert abs(float(np.dot(dx.astype(np.float64), x.astype(np.float64))) - lhs) <= 1e-5 * scale
+        # sampled data-gradient entries (cuda_perform.cu:266-291), borders and corners included
+        DX = dx.reshape(N, C, H, W)
+        picks = [(n, c, y, x_) for n in (0, N - 1) for c in (0, C - 1) for y in (0, H - 1)
+                 for x_ in (0, W - 1)]
+        picks += [(N // 2, C // 2, H // 2, W // 2), (1, 1, 0, W // 2), (N - 2, C - 2, H - 1, 1)]
+        while len(picks) < 72:
+            picks.append((int(rng.integers(N)), int(rng.integers(C)), int(rng.integers(H)),
+                          int(rng.integers(W))))
+        worst, top = 0.0, float(np.max(np.abs(dx)))
+        for (n, c, y, x_) in picks:
+            want = 0.0
+            for r in range(R):
+                if (y + ph - r) % sv or not 0 <= (y + ph - r) // sv < cv.Ho:
+                    continue
+                for s_ in range(S):
+                    if (x_ + pw - s_) % sh or not 0 <= (x_ + pw - s_) // sh < cv.Wo:
+                        continue
+                    want += float(np.dot(DY[n, :, (y + ph - r) // sv, (x_ + pw - s_) // sh].astype(np.float64),
+                                         Wt[:, c, r, s_]))
+            worst = max(worst, abs(float(DX[n, c, y, x_]) - want))
+        assert worst <= TOL * top, "data gradient entry off by %.3e of %.3e" % (worst, top)
     db = cv.bwd_bias(dy)
     assert normwise(db, dy.reshape(N, K, -1).astype(np.float64).sum(axis=(0, 2))) <= TOL
+
+
+def _filter_plan(gpu, p, nbytes):
+    tile, ranges, wgs = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    rc = gpu.L.mnv_conv_bwd_filter_plan(*p, ctypes.c_size_t(nbytes), ctypes.byref(tile),
+                                        ctypes.byref(ranges), ctypes.byref(wgs))
+    assert rc == 0
+    return tile.value, ranges.value, wgs.value
+
+
+# Filter gradients whose launch is dealt to the chip in equal shares of tiles x k-slabs: few
+# output tiles, a long reduction.  One case per way of fetching the gathered operand.
+STREAMK = [
+    ("one tap per tile", 84, 128, 128, 13, 13, 1, 1, 1, 1, 3, 3),
+    ("two taps per tile", 40, 96, 128, 13, 13, 2, 2, 1, 1, 5, 5),
+    ("a table row per row group", 76, 48, 128, 13, 13, 2, 2, 1, 1, 5, 5),
+    ("no padding", 150, 22, 128, 17, 17, 0, 0, 1, 1, 5, 5),
+    ("channels not in sixteens", 150, 24, 128, 13, 13, 2, 2, 1, 1, 5, 5),
+    ("96-column tile", 96, 128, 96, 13, 13, 1, 1, 1, 1, 3, 3),
+    ("strided, ragged tile edges", 60, 120, 200, 23, 21, 1, 2, 2, 2, 3, 5),
+]
+
+
+@pytest.mark.parametrize("case", STREAMK, ids=lambda c: c[0])
+def test_conv_bwd_filter_in_equal_shares_against_oracle(gpu, ora, case):
+    p = case[1:]
+    N, C, K, H, W, ph, pw, sv, sh, R, S = p
+    cv = Conv(gpu, *p)
+    nbytes = gpu.L.mnv_conv_bwd_filter_workspace_bytes(*p)
+    tile, ranges, wgs = _filter_plan(gpu, p, nbytes)
+    say("filter gradient,", case[0], "tile", tile, "workgroups", wgs)
+    assert tile == 128 and ranges == 1 and wgs >= 256, "the case is meant to take the stream-k plan"
+    # the shares cross tile boundaries: more shares than tiles, and not a multiple
+    tiles = ((C * R * S + 127) // 128) * ((K + (95 if K in (96, 192) else 127)) // (96 if K in (96, 192) else 128))
+    assert tiles < wgs and wgs % tiles != 0
+    x, dy = _rand(N * C * H * W, 61), _rand(N * K * cv.Ho * cv.Wo, 62)
+    got = cv.bwd_filter(dy, x)
+    assert normwise(got, ora.conv_bwd_filter(dy, x, *p)) <= TOL
+    # equal shares are added in a fixed order: identical bits on a second call
+    assert_bits_equal(cv.bwd_filter(dy, x), got, "second call")
+    # without a workspace the same problem runs in one k range per tile
+    assert _filter_plan(gpu, p, 0)[1:] == (1, 0)
+    assert normwise(cv.bwd_filter(dy, x, workspace=False), got.astype(np.float64)) <= 1e-5
 
 
 # ------------------------------------------------------------------- pooling

@@ -123,22 +123,35 @@ BIG = [(4096, 4096, 4096), (4096, 256, 9216), (4096, 256, 4096), (1000, 256, 409
 
 
 @pytest.mark.parametrize("m,n,k", BIG)
-def test_sgemm_config_shapes_sampled_fp64(gpu, m, n, k):
+def test_sgemm_config_shapes_full_fp64(gpu, m, n, k):
+    """The products of the benchmark configuration against the fp64 product, every element
+    (tests/unittest_sgemm.cpp:19-27 compares every element of its small product the same
+    way).  A sampled sub-product and the four corners go first: they fail fast and name a
+    place; the full comparison then reaches every output tile, so an error confined to one
+    tile (tile order, a partial tile at an edge, one k range) cannot pass."""
     a, b = _rand(m * k, 32), _rand(k * n, 33)
     say("sgemm big", m, n, k)
     got = _gemm(gpu, a, b, m, n, k).reshape(n, m)
-    A = a.reshape(k, m)   # A[l, i]
-    B = b.reshape(n, k)   # B[j, l]
+    A = a.reshape(k, m).astype(np.float64)   # A[l, i]
+    B = b.reshape(n, k).astype(np.float64)   # B[j, l]
     rng = np.random.default_rng(34)
     rows = rng.integers(0, m, 48)
     cols = rng.integers(0, n, 48)
-    want = (B[cols].astype(np.float64) @ A[:, rows].astype(np.float64))  # [cols, rows]
-    sub = got[np.ix_(cols, rows)]
-    assert normwise(sub, want) <= TOL
-    # the corners and edges of the tile grid are where indexing slips show
+    assert normwise(got[np.ix_(cols, rows)], B[cols] @ A[:, rows]) <= TOL
     for (i, j) in ((0, 0), (m - 1, 0), (0, n - 1), (m - 1, n - 1)):
-        w = float(B[j].astype(np.float64) @ A[:, i].astype(np.float64))
-        assert abs(got[j, i] - w) <= TOL * np.sqrt(k) * 4
+        assert abs(got[j, i] - float(B[j] @ A[:, i])) <= TOL * np.sqrt(k) * 4
+    want = B @ A
+    scale = float(np.max(np.abs(want)))
+    err = np.abs(got - want)
+    worst = np.unravel_index(int(np.argmax(err)), err.shape)
+    assert err[worst] <= TOL * scale, "largest error at column %d, row %d" % worst
+    # per 128 x 128 output tile: no tile may stand out (an error that is small against the
+    # largest element of the whole product but systematic inside one tile)
+    tn, tm = (n + 127) // 128, (m + 127) // 128
+    pad = np.zeros((tn * 128, tm * 128))
+    pad[:n, :m] = err
+    per_tile = pad.reshape(tn, 128, tm, 128).max(axis=(1, 3))
+    assert float(per_tile.max()) <= 8 * max(float(np.median(per_tile)), 1e-7 * scale)
 
 
 def test_sgemm_permutation_is_exact(gpu):
