@@ -5,6 +5,8 @@
                   linked against libmnv_hip.so              <- minerva_amd/host/*.cpp
 
 hipcc cross-compiles for gfx950 without a GPU, so this runs anywhere ROCm is installed.
+build() drives hipcc and g++ directly; build_with_cmake() runs the top-level CMakeLists.txt
+(the build a Minerva tree consumes) with the libraries written to the same place.
 """
 import concurrent.futures
 import glob
@@ -73,6 +75,20 @@ def build(verbose=True, jobs=8):
     return LIB_HIP
 
 
+def build_with_cmake(build_dir=None, jobs=8, verbose=True):
+    """Configures and builds the top-level CMake project; libraries go to minerva_amd/lib."""
+    build_dir = build_dir or os.path.join(ROOT, "build")
+    _run(["cmake", "-S", ROOT, "-B", build_dir, "-DCMAKE_BUILD_TYPE=Release",
+          "-DMNV_OUTPUT_DIR=" + LIBDIR])
+    _run(["cmake", "--build", build_dir, "-j%d" % jobs])
+    if verbose:
+        print("built", LIB_HIP, "and", LIB_HOST, "with cmake in", build_dir)
+    return LIB_HIP
+
+
 if __name__ == "__main__":
-    build()
+    if "--cmake" in sys.argv[1:]:
+        build_with_cmake()
+    else:
+        build()
     sys.exit(0)

@@ -435,8 +435,11 @@ void Concat(const DataList& inputs, const DataList& outputs, ConcatClosure& c, c
   size_t offset = 0;
   for (auto& in : inputs) {
     MNV_CHECK_EQ(in.size_.NumDims(), os.NumDims()) << "(Concat) rank mismatch";
-    for (size_t i = 0; i < os.NumDims(); ++i)
-      if (i != d) MNV_CHECK_EQ(in.size_[i], os[i]) << "(Concat) extent mismatch in dimension " << i;
+    for (size_t i = 0; i < os.NumDims(); ++i) {
+      if (i != d) {
+        MNV_CHECK_EQ(in.size_[i], os[i]) << "(Concat) extent mismatch in dimension " << i;
+      }
+    }
     const size_t e = static_cast<size_t>(in.size_[d]);
     MNV_CHECK_LE(offset + e, static_cast<size_t>(os[d])) << "(Concat) inputs exceed the output";
     Ok(mnv_copy_2d(in.data_, outputs[0].data_ + offset * inner, e * inner, outer, e * inner,
