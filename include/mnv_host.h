@@ -57,6 +57,10 @@ int mnvh_runtime_pool_stats(void* runtime, size_t* total_bytes, size_t* cached_b
  * streams before it reused a recycled block. */
 int mnvh_runtime_dataflow_stats(void* runtime, unsigned long long* producer_waits,
                                 unsigned long long* recycle_waits);
+/* Switches a live runtime between the one-stream order (enable = 0: mode 0 above) and dataflow
+ * placement.  Drains the device first; every tensor stays valid, and tensors created before
+ * the switch are tracked from their first use in the new mode. */
+int mnvh_runtime_set_dataflow(void* runtime, int enable);
 
 /* Per-operator device timing (two events per operator on its own stream).  The read
  * synchronises, writes one "name<TAB>launches<TAB>total_ms" line per operator name and

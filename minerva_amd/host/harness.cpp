@@ -293,6 +293,10 @@ int mnvh_runtime_dataflow_stats(void* runtime, unsigned long long* producer_wait
   });
 }
 
+int mnvh_runtime_set_dataflow(void* runtime, int enable) {
+  return Guard([&] { static_cast<Runner*>(runtime)->SetDataflow(enable != 0); });
+}
+
 int mnvh_runtime_profile(void* runtime, int enable) {
   return Guard([&] { static_cast<Runner*>(runtime)->device().set_profile(enable != 0); });
 }

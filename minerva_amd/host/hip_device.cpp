@@ -171,6 +171,12 @@ void HipDevice::Execute(Task* task, int thrid) {
           ++producer_waits_;
         }
         it->second.users |= 1u << thrid;
+      } else {
+        // Created before dataflow mode was switched on (the switch drained every stream, so
+        // the contents are complete): no producer to wait for, but this reader must be on
+        // record, or the block could go back to the pool and on to another stream while
+        // this stream's kernels still read it.
+        produced_[d.data_id] = Produced{0, thrid, 1u << thrid};
       }
     }
     input_shards.emplace_back(data_store_->GetData(d.data_id), d.size);

@@ -5,12 +5,14 @@
 namespace minerva {
 
 TensorNode::~TensorNode() {
-  if (runner && runner->device_) runner->device_->FreeDataIfExist(id);
+  if (runner && runner->manager_) runner->manager_->FreeData(id);
 }
 
 Runner::Runner(int gpu_id, bool sync_each_op, bool dataflow, size_t pool_bytes)
     : dataflow_(dataflow) {
-  device_.reset(new HipDevice(0, this, gpu_id, pool_bytes));
+  manager_.reset(new DeviceManager(pool_bytes));
+  manager_->RegisterListener(this);
+  device_ = static_cast<HipDevice*>(manager_->GetDevice(manager_->CreateGpuDevice(gpu_id)));
   device_->set_sync_each_op(sync_each_op);
   if (dataflow) device_->set_dataflow(true);
 }
@@ -18,21 +20,24 @@ Runner::Runner(int gpu_id, bool sync_each_op, bool dataflow, size_t pool_bytes)
 void Runner::Sync() {
   device_->Barrier(0);
   for (auto& q : queued_) q = 0;
+  ++epoch_;
+}
+
+void Runner::SetDataflow(bool on) {
+  Sync();
+  device_->set_dataflow(on);
+  if (!on) device_->set_sync_each_op(false);
+  dataflow_ = on;
 }
 
 int Runner::PickStream(const std::vector<Tensor>& inputs) {
-  int pick = -1;
-  uint64_t newest = 0;
+  const TensorNode* newest = nullptr;
   for (auto& t : inputs)
-    if (tail_[t->stream] == t->id && t->id >= newest) {
-      pick = t->stream;
-      newest = t->id;
-    }
-  if (pick < 0) {
-    pick = 0;
-    for (int s = 1; s < static_cast<int>(HipDevice::kParallelism); ++s)
-      if (queued_[s] < queued_[pick]) pick = s;
-  }
+    if (t->epoch == epoch_ && (!newest || t->id > newest->id)) newest = t.get();
+  if (newest && issued_[newest->stream] - newest->seq <= kStayBehind) return newest->stream;
+  int pick = 0;
+  for (int s = 1; s < static_cast<int>(HipDevice::kParallelism); ++s)
+    if (queued_[s] < queued_[pick]) pick = s;
   return pick;
 }
 
@@ -55,7 +60,8 @@ Tensor Runner::Compute(const std::vector<Tensor>& inputs, const Scale& out_size,
   task.light = true;  // issued in program order from the caller's thread
   if (dataflow_) {
     task.stream = out->stream = PickStream(inputs);
-    tail_[task.stream] = out->id;
+    out->seq = ++issued_[task.stream];
+    out->epoch = epoch_;
     ++queued_[task.stream];
   }
   device_->PushTask(&task);

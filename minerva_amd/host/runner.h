@@ -11,6 +11,7 @@
 #pragma once
 #include <atomic>
 
+#include "device_manager.h"
 #include "hip_device.h"
 
 namespace minerva {
@@ -23,7 +24,9 @@ struct TensorNode {
   Runner* runner;
   uint64_t id;
   Scale size;
-  int stream = 0;  // the worker stream its producer ran on
+  int stream = 0;      // the worker stream its producer ran on
+  uint64_t seq = 0;    // how many operators that stream had been given when the producer was queued
+  uint64_t epoch = 0;  // Sync count at that time: a tensor of an earlier epoch is complete
 };
 using Tensor = std::shared_ptr<TensorNode>;
 
@@ -39,6 +42,8 @@ class Runner : public DeviceListener {
   HipDevice& device() { return *device_; }
   uint64_t ops_issued() const { return ops_issued_; }
   void Sync();
+  // Switches between the one-stream order and dataflow placement; tensors stay valid.
+  void SetDataflow(bool on);
 
   Tensor Compute(const std::vector<Tensor>& inputs, const Scale& out_size,
                  std::shared_ptr<ComputeFn> fn);
@@ -144,20 +149,26 @@ class Runner : public DeviceListener {
 
  private:
   friend struct TensorNode;
-  std::unique_ptr<HipDevice> device_;
+  // the devices live in a manager, as in the reference's MinervaSystem (system/minerva_system.cpp:84);
+  // this runner drives the one GPU device it created there
+  std::unique_ptr<DeviceManager> manager_;
+  HipDevice* device_ = nullptr;
   std::atomic<uint64_t> next_id_{1};
   std::atomic<uint64_t> ops_issued_{0}, ops_completed_{0};
   bool retain_ = false;
   std::vector<Tensor> retained_;
-  // Dataflow placement.  An operator whose newest input is the last thing queued on some
-  // stream continues that stream (a chain stays together and needs no event wait);
-  // any other operator starts a new chain on the stream with the least work queued since
-  // the last Sync.  Independent chains -- the weight-gradient branches of a backward pass
-  // against its data-gradient spine -- so end up on different streams and overlap.
+  // Dataflow placement.  An operator follows its newest input that is still in flight onto
+  // that input's stream (a chain and its short side branches stay together: stream order
+  // does the waiting, no event), unless more than kStayBehind operators have been queued on
+  // that stream behind the input: then the operator does not depend on that work and starts a
+  // chain of its own on the stream with the least queued since the last Sync.  So does an
+  // operator with no input in flight (a load of the next batch, a fill).
+  static constexpr uint64_t kStayBehind = 3;
   int PickStream(const std::vector<Tensor>& inputs);
   bool dataflow_ = false;
-  uint64_t tail_[HipDevice::kParallelism] = {};    // id of the last output queued per stream
+  uint64_t issued_[HipDevice::kParallelism] = {};  // operators ever queued per stream
   uint64_t queued_[HipDevice::kParallelism] = {};  // operators queued per stream since Sync
+  uint64_t epoch_ = 1;                             // Syncs so far + 1
 };
 
 }  // namespace minerva

@@ -122,6 +122,10 @@ class Runtime:
         _check(lib().mnvh_runtime_pool_stats(self.h, ctypes.byref(t), ctypes.byref(c)), "pool_stats")
         return t.value, c.value
 
+    def set_dataflow(self, on):
+        """Switches a live runtime between the one-stream order and dataflow placement."""
+        _check(lib().mnvh_runtime_set_dataflow(self.h, 1 if on else 0), "set_dataflow")
+
     def dataflow_stats(self):
         """(waits for a producer on another stream, waits before reusing a recycled block)"""
         a, b = ctypes.c_ulonglong(), ctypes.c_ulonglong()

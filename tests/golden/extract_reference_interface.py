@@ -5,6 +5,7 @@ Reads the reference's headers as text only (nothing is compiled, imported or run
   minerva/op/impl/cuda.h:10-48      GPU operator functions: names and parameter lists
   minerva/op/closure.h:8-176        enums, closure structs and their fields
   minerva/device/device.h:18-78     Device / ThreadedDevice / GpuDevice member functions
+  minerva/device/device_manager.h:9-26   DeviceManager member functions
 
 Usage (in the build container, where /root/reference is mounted):
   python tests/golden/extract_reference_interface.py [/root/reference]
@@ -23,13 +24,16 @@ def main():
     read = lambda rel: open(os.path.join(ref, rel)).read()
     closure_h = read("minerva/op/closure.h")
     device_h = read("minerva/device/device.h")
+    manager_h = read("minerva/device/device_manager.h")
     out = {
         "source": {"operators": "minerva/op/impl/cuda.h", "closures": "minerva/op/closure.h",
-                   "device": "minerva/device/device.h"},
+                   "device": "minerva/device/device.h",
+                   "device_manager": "minerva/device/device_manager.h"},
         "operators": ip.free_functions(read("minerva/op/impl/cuda.h"), "cuda"),
         "closures": ip.structs(closure_h),
         "enums": ip.enums(closure_h),
-        "classes": {c: ip.class_methods(device_h, c) for c in ("Device", "ThreadedDevice", "GpuDevice")},
+        "classes": dict({c: ip.class_methods(device_h, c) for c in ("Device", "ThreadedDevice", "GpuDevice")},
+                        DeviceManager=ip.class_methods(manager_h, "DeviceManager")),
     }
     path = os.path.join(HERE, "interface.json")
     with open(path, "w") as f:

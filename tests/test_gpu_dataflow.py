@@ -166,16 +166,65 @@ def test_reader_of_lrn_scale_waits_for_the_forward_pass(ora):
     dims = [W, H, C, N]
     tx = r.tensor(x, dims)
     big = r.tensor(_rand(2048 * 2048, 6) / np.float32(45), [2048, 2048])
+    crossed = 0
     for rep in range(3):
         say("lrn scale reader, repetition", rep)
         busy = r.top("matmult", [big, big])          # keeps the producer's stream busy first
         busy = r.top("matmult", [busy, big])
         scale = r.top("fill", [], [0.0] + dims)
         top = r.top("lrn_forward", [tx, scale], [5, 1e-4, 0.75])
+        # four more operators behind the forward pass on its stream: the reader of `scale`
+        # then starts a chain of its own on another stream
+        for _ in range(4):
+            busy = r.top("matmult", [busy, big]) if busy.stream == top.stream else \
+                r.top("arithmetic_const", [top], [2, 1.0, 0])
+        waits_before = r.dataflow_stats()[0]
         twice = r.top("arithmetic_const", [scale], [2, 2.0, 0])   # reads `scale` alone
         if twice.stream == top.stream:
             continue  # placement put both on one stream this time: stream order covers it
+        crossed += 1
+        assert r.dataflow_stats()[0] > waits_before, "the reader must wait for the forward pass"
         got = twice.read()
         assert float(np.max(np.abs(got - 2 * want_scale))) <= 1e-4 * float(np.max(np.abs(want_scale)))
         assert float(np.max(np.abs(top.read() - want_top))) <= 1e-4 * float(np.max(np.abs(want_top)))
+    assert crossed >= 1, "no repetition placed the reader on another stream than the forward pass"
     r.close()
+
+
+def test_mode_switched_on_live_data_tracks_readers_of_older_tensors():
+    """Tensors created in the one-stream order have no producer on record.  After the switch
+    to dataflow mode a long reader of such a tensor must still be known when the tensor's block
+    is freed and taken by another stream: that stream has to wait for the reader."""
+    from minerva_amd import hostapi
+    n = 4096
+    x = _rand(n * n, 8) / np.float32(64)
+    results = {}
+    for mode in ("order", "switched"):
+        r = hostapi.Runtime(0, sync_each_op=False, pool_bytes=512 << 20)
+        tx = r.tensor(x, [n, n])
+        y = r.top("arithmetic_const", [tx], [2, 1.0, 0])      # created before the switch
+        r.sync()
+        if mode == "switched":
+            r.set_dataflow(True)
+        say("reader of a tensor older than the mode", mode)
+        prod = r.top("matmult", [y, y])                         # ~1 ms, reads y throughout
+        prod2 = r.top("matmult", [prod, tx])
+        for _ in range(4):                                      # the fill below must not follow `prod`
+            prod2 = r.top("arithmetic_const", [prod2], [2, 1.0, 0])
+        waits_before = r.dataflow_stats()[1]
+        total_before, _ = r.pool_stats()
+        y.free()
+        z = r.top("fill", [], [7.0, n, n])                      # takes y's block
+        assert r.pool_stats()[0] == total_before, "the fill must recycle the freed block"
+        if mode == "switched":
+            assert z.stream != prod.stream, "the fill must sit on another stream than the reader"
+            assert r.dataflow_stats()[1] > waits_before, "the fill's stream must wait for the reader"
+        results[mode] = prod.read()
+        assert_bits_equal(z.read(), np.full(n * n, 7.0, np.float32), "fill")
+        if mode == "switched":   # and back: everything on one stream again
+            r.set_dataflow(False)
+            again = r.top("matmult", [tx, tx])
+            assert again.stream == 0
+            again.read()
+        r.close()
+    assert_bits_equal(results["switched"], results["order"], "product that read the freed block")

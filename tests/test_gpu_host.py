@@ -255,6 +255,19 @@ def test_error_convention(rt):
     assert_bits_equal(got, a + a, "after error")
 
 
+def test_device_manager_creates_the_device_and_refuses_a_missing_gpu():
+    # device_manager.cpp:33-47: devices are made by GPU index and live in the manager; the
+    # runtime's device comes from there
+    from minerva_amd import hostapi
+    with pytest.raises(hostapi.HostError, match="no GPU #99"):
+        hostapi.Runtime(99)
+    r = hostapi.Runtime(0)
+    a = _rand(12, 79)
+    got, _ = r.op("arithmetic", [(a, [3, 4]), (a, [3, 4])], [2])
+    assert_bits_equal(got, a * a, "product on the managed device")
+    r.close()
+
+
 def test_pooled_allocator_reuses_exact_sizes(rt):
     a = _rand(5000, 79)
     rt.op("arithmetic", [(a, [5000]), (a, [5000])], [0])

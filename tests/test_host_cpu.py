@@ -93,6 +93,18 @@ def test_device_classes_have_the_reference_member_functions(ref):
         assert got["params"] == m["params"] and got["ret"] == m["ret"] and got["const"] == m["const"], name
 
 
+def test_device_manager_has_the_reference_member_functions(ref):
+    # minerva/device/device_manager.h:9-26
+    want = ref["classes"]["DeviceManager"]
+    mine = ip.class_methods(_read("device_manager.h"), "DeviceManager")
+    assert mine is not None and mine["base"] == want["base"]
+    assert set(mine["methods"]) == set(want["methods"])
+    for name, m in want["methods"].items():
+        got = mine["methods"][name]
+        for key in ("ret", "params", "const", "access", "virtual"):
+            assert got[key] == m[key], "DeviceManager::%s %s: %r vs %r" % (name, key, got[key], m[key])
+
+
 def test_interface_fixture_is_what_the_extractor_writes():
     """Where the reference tree is present (the build container), the committed fixture must be
     what the extractor produces from it today."""
@@ -103,3 +115,5 @@ def test_interface_fixture_is_what_the_extractor_writes():
     want = json.load(open(os.path.join(GOLD, "interface.json")))
     assert ip.free_functions(read("minerva/op/impl/cuda.h"), "cuda") == want["operators"]
     assert ip.structs(read("minerva/op/closure.h")) == want["closures"]
+    assert ip.class_methods(read("minerva/device/device_manager.h"), "DeviceManager") == \
+        want["classes"]["DeviceManager"]
