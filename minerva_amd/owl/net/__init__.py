@@ -5,4 +5,4 @@ window data providers and Caffe's protobuf classes -- networks are described in 
 prototxt TEXT, which a small parser here reads (no protobuf), and batches come from memory."""
 from .net import *  # noqa: F401,F403
 from .net_helper import NetBuilder, parse_prototxt, save_net_to_file, init_net_from_file  # noqa: F401
-from .trainer import NetTrainer  # noqa: F401
+from .trainer import NetTrainer, NetTester  # noqa: F401

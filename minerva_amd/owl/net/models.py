@@ -62,3 +62,33 @@ ALEXNET_SOLVER = '''
 base_lr: 0.01 lr_policy: "step" gamma: 0.1 stepsize: 100000
 momentum: 0.9 weight_decay: 0.0005 max_iter: 450000
 '''
+
+
+def mnist_cnn_prototxt(batch_size, test_batch_size=None, top_k=1):
+    """The MNIST CNN of the reference's applications (owl/apps/mnist/mnist_cnn.py:17-47: conv 5x5
+    16 - ReLU - max-pool 2x2/2 - conv 5x5 32 - ReLU - max-pool 2x2/2 - fully connected 10 -
+    softmax, weights N(0, 0.1)) as a network description with a TRAIN-phase and a TEST-phase data
+    unit and an accuracy unit in the TEST phase, the shape of the reference's prototxt networks."""
+    test_batch_size = test_batch_size or batch_size
+    data = ('layer { name: "mnist" type: "MemoryData" top: "data" top: "label" include { phase: %s }\n'
+            '  memory_data_param { batch_size: %d channels: 1 height: 28 width: 28 } }\n')
+    conv = ('layer { name: "%s" type: "Convolution" bottom: "%s" top: "%s"\n'
+            '  convolution_param { num_output: %d kernel_size: 5 weight_filler { type: "gaussian" std: 0.1 } } }\n'
+            'layer { name: "relu_%s" type: "ReLU" bottom: "%s" top: "%s" }\n')
+    pool = ('layer { name: "%s" type: "Pooling" bottom: "%s" top: "%s"'
+            ' pooling_param { pool: MAX kernel_size: 2 stride: 2 } }\n')
+    return ('name: "MnistCnn"\n' + data % ("TRAIN", batch_size) + data % ("TEST", test_batch_size)
+            + conv % ("conv1", "data", "conv1", 16, "conv1", "conv1", "conv1")
+            + pool % ("pool1", "conv1", "pool1")
+            + conv % ("conv2", "pool1", "conv2", 32, "conv2", "conv2", "conv2")
+            + pool % ("pool2", "conv2", "pool2")
+            + 'layer { name: "ip" type: "InnerProduct" bottom: "pool2" top: "ip"\n'
+              '  inner_product_param { num_output: 10 weight_filler { type: "gaussian" std: 0.1 } } }\n'
+              'layer { name: "loss" type: "SoftmaxWithLoss" bottom: "ip" bottom: "label" top: "loss" }\n'
+              'layer { name: "accuracy" type: "Accuracy" bottom: "ip" bottom: "label" top: "accuracy"\n'
+              '  accuracy_param { top_k: %d } include { phase: TEST } }\n' % top_k)
+
+
+MNIST_CNN_SOLVER = (
+    'base_lr: 0.05 lr_policy: "step" gamma: 0.5 stepsize: 1000 momentum: 0.9 weight_decay: 0.0001\n'
+    'max_iter: 1000 test_iter: 3 test_interval: 10\n')

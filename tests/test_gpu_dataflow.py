@@ -175,9 +175,10 @@ def test_reader_of_lrn_scale_waits_for_the_forward_pass(ora):
         top = r.top("lrn_forward", [tx, scale], [5, 1e-4, 0.75])
         # four more operators behind the forward pass on its stream: the reader of `scale`
         # then starts a chain of its own on another stream
+        tail = top
         for _ in range(4):
-            busy = r.top("matmult", [busy, big]) if busy.stream == top.stream else \
-                r.top("arithmetic_const", [top], [2, 1.0, 0])
+            tail = r.top("arithmetic_const", [tail], [2, 1.0, 0])
+            assert tail.stream == top.stream, "a chain stays on its stream"
         waits_before = r.dataflow_stats()[0]
         twice = r.top("arithmetic_const", [scale], [2, 2.0, 0])   # reads `scale` alone
         if twice.stream == top.stream:

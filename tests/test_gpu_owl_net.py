@@ -166,3 +166,73 @@ def test_caffe_alexnet_step_matches_oracle(owl):
         assert_bits_equal(u.weightdelta.to_numpy().ravel(), dw, "momentum of " + u.name)
         assert_bits_equal(u.bias.to_numpy().ravel(), b, "updated bias of " + u.name)
         assert_bits_equal(u.biasdelta.to_numpy().ravel(), db, "bias momentum of " + u.name)
+
+
+def _pattern_batches(count, batch, seed):
+    """Synthetic digits a small CNN can learn in a few steps: class k lights a 6x6 patch whose
+    position depends on k, on a noisy background."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        y = rng.integers(0, 10, batch)
+        x = (rng.standard_normal((batch, 1, 28, 28)) * 0.3).astype(np.float32)
+        for i, k in enumerate(y):
+            r, c = 2 + 5 * (k // 5) * 2, 1 + 5 * (k % 5)
+            x[i, 0, r:r + 6, c:c + 6] += 2.0
+        out.append((x, y))
+    return out
+
+
+def test_mnist_cnn_test_phase_and_tester(owl, tmp_path):
+    """trainer.py:156-169 (the TEST-phase pass every test_interval minibatches) and NetTester
+    (trainer.py:247-329) on the MNIST CNN description: the accuracies they report are the
+    share of arg-max predictions that hit the label, recomputed here from the probabilities."""
+    from minerva_amd.owl import net as onet
+    from minerva_amd.owl.net import models
+    batch, test_batch = 32, 16
+    solver = models.MNIST_CNN_SOLVER + 'snapshot_prefix: "%s" snapshot: 20\n' % tmp_path
+    text = models.mnist_cnn_prototxt(batch, test_batch)
+    train = _pattern_batches(20, batch, 1)
+    test = _pattern_batches(3, test_batch, 2)
+    tr = onet.NetTrainer(solver, text, seed=7)
+    net = tr.owl_net
+    assert net.get_data_unit("TRAIN") is not net.get_data_unit("TEST")
+    assert net.get_data_unit("TEST").batch_size == test_batch
+    say("owl.net: MNIST CNN, accuracy before training")
+    before = tr.test(lambda i: test[i])
+    logged = []
+    say("owl.net: MNIST CNN, 20 minibatches with a TEST pass every 10")
+    tr.run(20, lambda i: train[i], sync_freq=5, log=logged.append, next_test_batch=lambda i: test[i])
+    assert [it for it, _ in tr.accuracies] == [10, 20]
+    after = tr.accuracies[-1][1]
+    assert after >= 0.9 and after > before + 0.3, (before, tr.accuracies)
+    assert any(l.startswith("Testing Accuracy") for l in logged)
+    # the reported accuracy is what the probabilities say, batch by batch
+    hits = total = 0
+    loss = net.get_units_by_name("loss")[0]
+    for x, y in test:
+        net.get_data_unit("TEST").set_batch(x, y)
+        net.forward("TEST")
+        prob = loss.ff_y.to_numpy().reshape(test_batch, 10)
+        hits += int(np.sum(np.argmax(prob, axis=1) == y))
+        total += test_batch
+        assert abs(net.get_accuracy_units()[-1].acc - np.mean(np.argmax(prob, axis=1) == y)) < 1e-12
+    assert abs(after - hits / total) < 1e-12
+    # the tester on the snapshot written after 20 minibatches reports the same number
+    tester = onet.NetTester(solver, "loss", "accuracy", 1, net_text=text)
+    tester.build_net()
+    lines = []
+    assert abs(tester.run(lambda i: test[i], log=lines.append) - after) < 1e-12
+    assert len(lines) == 4 and lines[-1].startswith("Testing Accuracy")
+    # top-5 through the accuracy unit's top_k against a numpy ranking
+    top5 = onet.NetTester(solver, "loss", "accuracy", 1,
+                          net_text=models.mnist_cnn_prototxt(batch, test_batch, top_k=5))
+    top5.build_net()
+    got = top5.run(lambda i: test[i])
+    want = 0
+    for x, y in test:
+        top5.owl_net.get_data_unit("TEST").set_batch(x, y)
+        top5.owl_net.forward("TEST")
+        prob = top5.owl_net.get_units_by_name("loss")[0].ff_y.to_numpy().reshape(test_batch, 10)
+        want += sum(int(y[i] in np.argsort(prob[i])[::-1][:5]) for i in range(test_batch))
+    assert abs(got - want / (3.0 * test_batch)) < 1e-12 and got >= after
