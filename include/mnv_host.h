@@ -149,7 +149,15 @@ int mnvh_net_keep_activations(void* net, int on);
 /* Uploads one batch; it stays resident in HBM for the following steps. */
 int mnvh_net_load_batch(void* net, const float* data, size_t data_floats, const float* label,
                         size_t label_floats);
-/* One forward + backward + SGD step on the resident batch. */
+/* Loads the NEXT batch while the step in flight keeps the GPU busy: the copy runs on a second
+ * worker stream through pinned staging memory into a second pair of tensors (what the
+ * reference's trainer gets from its data provider thread and the engine's ArrayLoader operator,
+ * owl/owl/net/trainer.py:118-145, op/impl/cuda.cpp:592-598).  The next mnvh_net_step trains on
+ * it.  Returns when the copy is complete; the caller's buffers may then be reused. */
+int mnvh_net_prefetch_batch(void* net, const float* data, size_t data_floats, const float* label,
+                            size_t label_floats);
+/* One forward + backward + SGD step on the resident batch (on the prefetched one, if one was
+ * loaded since the last step). */
 int mnvh_net_step(void* net, float lr);
 /* Records one step on the resident batch into a HIP graph (nothing of it is applied:
  * parameters are unchanged afterwards), for networks whose step is launch-bound.  The

@@ -16,6 +16,11 @@ struct NetHandle {
   Runner* rt;
   std::unique_ptr<Net> net;
   Tensor data, label;
+  // the batch being loaded while a step runs (mnvh_net_prefetch_batch): a second pair of
+  // tensors, and a marker behind the last step that read them
+  Tensor next_data, next_label;
+  bool next_ready = false;
+  void* spare_last_use = nullptr;
   // a recorded Step: the instantiated graph and every tensor its kernels read or write
   void* graph = nullptr;
   std::vector<Tensor> graph_tensors;
@@ -522,11 +527,44 @@ int mnvh_net_load_batch(void* net, const float* data, size_t data_floats, const 
   });
 }
 
+int mnvh_net_prefetch_batch(void* net, const float* data, size_t data_floats, const float* label,
+                            size_t label_floats) {
+  return Guard([&] {
+    NetHandle* h = static_cast<NetHandle*>(net);
+    Scale ds = h->net->DataSize(), ls = h->net->LabelSize();
+    MNV_CHECK_EQ(static_cast<size_t>(ds.Prod()), data_floats) << "data size";
+    MNV_CHECK_EQ(static_cast<size_t>(ls.Prod()), label_floats) << "label size";
+    MNV_CHECK(!h->graph) << "a recorded step reads one pair of tensors: use mnvh_net_load_batch";
+    MNV_CHECK(!h->rt->device().dataflow()) << "in dataflow mode mnvh_net_load_batch is placed on a "
+                                           << "stream of its own already";
+    HipDevice& dev = h->rt->device();
+    if (!h->next_data) {  // first use: the second pair, created in stream order
+      h->next_data = h->rt->Constant(ds, 0.f);
+      h->next_label = h->rt->Constant(ls, 0.f);
+      h->spare_last_use = dev.StreamMarker(0);
+    }
+    // the step that last read the spare pair must have left the GPU
+    dev.WaitMarker(h->spare_last_use);
+    h->spare_last_use = nullptr;
+    // worker stream 1 carries the copy; stream 0 keeps computing the step in flight
+    h->rt->UploadOn(1, h->next_data, data);
+    h->rt->UploadOn(1, h->next_label, label);
+    h->next_ready = true;
+  });
+}
+
 int mnvh_net_step(void* net, float lr) {
   return Guard([&] {
     NetHandle* h = static_cast<NetHandle*>(net);
-    MNV_CHECK(h->data && h->label) << "load a batch first";
     MNV_CHECK(!h->graph) << "the step is recorded: replay it or release the recording first";
+    if (h->next_ready) {  // the prefetched batch becomes the current one
+      std::swap(h->data, h->next_data);
+      std::swap(h->label, h->next_label);
+      h->next_ready = false;
+      // the pair that just became spare was read by the previous step, which may still run
+      if (h->next_data) h->spare_last_use = h->rt->device().StreamMarker(0);
+    }
+    MNV_CHECK(h->data && h->label) << "load a batch first";
     h->net->Step(h->data, h->label, lr);
   });
 }

@@ -1,4 +1,5 @@
 #include "hip_device.h"
+#include "staged_copy.h"
 
 #include <cstdio>
 #include <cstring>
@@ -364,6 +365,30 @@ void HipDevice::CopyFromHost(uint64_t data_id, const float* src, size_t floats) 
   Ok(mnv_memcpy_h2d(data_store_->GetData(data_id), src, floats * sizeof(float), streams_[0]),
      "copy from host");
   Ok(mnv_stream_sync(streams_[0]), "copy from host sync");
+}
+
+void HipDevice::CopyFromHostOn(int thrid, uint64_t data_id, const float* src, size_t floats) {
+  MNV_CHECK(!capturing_) << "no host copies while a graph is recorded";
+  MNV_CHECK(thrid >= 0 && thrid < static_cast<int>(kParallelism)) << "bad stream";
+  Activate();
+  EnsureStaging(thrid);
+  Ok(StagedHostToDevice(data_store_->GetData(data_id), src, floats * sizeof(float), streams_[thrid],
+                        staging_[thrid], kStagingBytes),
+     "copy from host");
+}
+
+void* HipDevice::StreamMarker(int thrid) {
+  Activate();
+  void* e = nullptr;
+  Ok(mnv_event_create_ordering(&e), "event create");
+  Ok(mnv_event_record(e, streams_[thrid]), "event record");
+  return e;
+}
+
+void HipDevice::WaitMarker(void* marker) {
+  if (!marker) return;
+  Ok(mnv_event_sync(marker), "event sync");
+  mnv_event_destroy(marker);
 }
 
 void HipDevice::CopyOnDevice(uint64_t dst_id, uint64_t src_id, size_t floats) {

@@ -58,6 +58,15 @@ class HipDevice : public ThreadedDevice {
   void CopyToHost(float* dst, uint64_t data_id, size_t floats);
   // Overwrites existing data in place (its address does not change).
   void CopyFromHost(uint64_t data_id, const float* src, size_t floats);
+  // The same on worker stream `thrid`, through that stream's pinned staging area, and
+  // synchronised with that stream only: work queued on the other streams keeps running while
+  // the caller's thread feeds the copy.  The caller vouches that nothing queued still touches
+  // the data (see StreamMarker).  This is how the next batch is loaded under a running step.
+  void CopyFromHostOn(int thrid, uint64_t data_id, const float* src, size_t floats);
+  // A marker behind everything queued on worker stream `thrid` so far; WaitMarker blocks the
+  // caller until the GPU has passed it and releases it.
+  void* StreamMarker(int thrid);
+  void WaitMarker(void* marker);
   // dst <- src on worker stream 0, left in flight (a kernel, so it can be recorded).
   void CopyOnDevice(uint64_t dst_id, uint64_t src_id, size_t floats);
   // Per-operator timing, the counterpart of the reference's ExecutionProfiler

@@ -1,4 +1,5 @@
 #include "hip_ops.h"
+#include "staged_copy.h"
 
 #include <cstring>
 
@@ -483,39 +484,13 @@ void Select(const DataList& inputs, const DataList& outputs, SelectClosure& c, c
 void ArrayLoader(const DataList& outputs, ArrayLoaderClosure& closure, const Context& ctx) {
   MNV_CHECK_EQ(outputs.size(), 1u) << "(array loader) #outputs wrong";
   MNV_CHECK(closure.data) << "probably already executed";
-  // on the operator's own stream (the reference uses the default stream, cuda.cpp:595)
+  // on the operator's own stream (the reference uses the default stream, cuda.cpp:595); large
+  // pageable buffers go through the stream's pinned staging area; synchronised, because the
+  // host buffer must outlive the copy
   const size_t bytes = outputs[0].size_.Prod() * sizeof(float);
-  const char* src = reinterpret_cast<const char*>(closure.data.get());
-  char* dst = reinterpret_cast<char*>(outputs[0].data_);
-  const size_t half = ctx.staging_bytes / 2;
-  if (!ctx.staging || half == 0 || bytes <= half) {
-    Ok(mnv_memcpy_h2d(dst, src, bytes, ctx.stream), "array loader");
-  } else {
-    // A large copy out of pageable memory goes through the stream's pinned staging area in
-    // two alternating halves: the CPU fills one while the DMA engine drains the other
-    // (left to the runtime, such a copy runs at a fraction of the link's rate).
-    char* stage = static_cast<char*>(ctx.staging);
-    void* drained[2] = {nullptr, nullptr};
-    Ok(mnv_event_create_ordering(&drained[0]), "event create");
-    Ok(mnv_event_create_ordering(&drained[1]), "event create");
-    int rc = MNV_OK;
-    size_t off = 0;
-    for (int i = 0; off < bytes && rc == MNV_OK; ++i, off += half) {
-      const int b = i & 1;
-      const size_t n = bytes - off < half ? bytes - off : half;
-      if (i >= 2) rc = mnv_event_sync(drained[b]);  // this half has left for the device
-      if (rc != MNV_OK) break;
-      std::memcpy(stage + b * half, src + off, n);
-      rc = mnv_memcpy_h2d(dst + off, stage + b * half, n, ctx.stream);
-      if (rc == MNV_OK) rc = mnv_event_record(drained[b], ctx.stream);
-    }
-    mnv_stream_sync(ctx.stream);
-    mnv_event_destroy(drained[0]);
-    mnv_event_destroy(drained[1]);
-    Ok(rc, "array loader");
-  }
-  // the host buffer must outlive the asynchronous copy
-  Ok(mnv_stream_sync(ctx.stream), "array loader sync");
+  Ok(StagedHostToDevice(outputs[0].data_, closure.data.get(), bytes, ctx.stream, ctx.staging,
+                        ctx.staging_bytes),
+     "array loader");
   closure.data.reset();
 }
 

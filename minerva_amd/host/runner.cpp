@@ -30,11 +30,20 @@ void Runner::SetDataflow(bool on) {
   dataflow_ = on;
 }
 
-int Runner::PickStream(const std::vector<Tensor>& inputs) {
+int Runner::PickStream(const std::vector<Tensor>& inputs, const Scale& out_size) {
   const TensorNode* newest = nullptr;
-  for (auto& t : inputs)
+  size_t bytes = static_cast<size_t>(out_size.Prod()) * sizeof(float);
+  for (auto& t : inputs) {
+    bytes += static_cast<size_t>(t->size.Prod()) * sizeof(float);
     if (t->epoch == epoch_ && (!newest || t->id > newest->id)) newest = t.get();
-  if (newest && issued_[newest->stream] - newest->seq <= kStayBehind) return newest->stream;
+  }
+  // small operators never leave the chain: an event and a wait cost more than they take
+  const bool may_fork = bytes >= kForkBytes;
+  if (newest && (!may_fork || issued_[newest->stream] - newest->seq <= kStayBehind))
+    return newest->stream;
+  // inputs, but none in flight (weights of the last step, a resident batch): what this
+  // operator makes is most likely for the chain that is being queued right now
+  if (!newest && (!inputs.empty() || !may_fork)) return last_stream_;
   int pick = 0;
   for (int s = 1; s < static_cast<int>(HipDevice::kParallelism); ++s)
     if (queued_[s] < queued_[pick]) pick = s;
@@ -59,7 +68,8 @@ Tensor Runner::Compute(const std::vector<Tensor>& inputs, const Scale& out_size,
   task.id = ops_issued_++;
   task.light = true;  // issued in program order from the caller's thread
   if (dataflow_) {
-    task.stream = out->stream = PickStream(inputs);
+    task.stream = out->stream = PickStream(inputs, out_size);
+    last_stream_ = task.stream;
     out->seq = ++issued_[task.stream];
     out->epoch = epoch_;
     ++queued_[task.stream];
@@ -73,6 +83,11 @@ void Runner::Upload(const Tensor& t, const float* host) {
   MNV_CHECK(t && host) << "null argument";
   device_->Barrier(0);
   device_->CopyFromHost(t->id, host, t->size.Prod());
+}
+
+void Runner::UploadOn(int stream, const Tensor& t, const float* host) {
+  MNV_CHECK(t && host) << "null argument";
+  device_->CopyFromHostOn(stream, t->id, host, t->size.Prod());
 }
 
 void Runner::CopyInto(const Tensor& dst, const Tensor& src) {

@@ -42,6 +42,9 @@ class Runner : public DeviceListener {
   HipDevice& device() { return *device_; }
   uint64_t ops_issued() const { return ops_issued_; }
   void Sync();
+  // Overwrites `t` from host memory on worker stream `stream` while the other streams keep
+  // running (HipDevice::CopyFromHostOn); the caller vouches that no queued work touches `t`.
+  void UploadOn(int stream, const Tensor& t, const float* host);
   // Switches between the one-stream order and dataflow placement; tensors stay valid.
   void SetDataflow(bool on);
 
@@ -162,13 +165,20 @@ class Runner : public DeviceListener {
   // does the waiting, no event), unless more than kStayBehind operators have been queued on
   // that stream behind the input: then the operator does not depend on that work and starts a
   // chain of its own on the stream with the least queued since the last Sync.  So does an
-  // operator with no input in flight (a load of the next batch, a fill).
+  // operator without inputs (a load of the next batch, a fill).  An operator whose inputs are
+  // all complete (weights of the last step, a resident batch) joins the stream that was given
+  // the operator before it: its result is most likely meant for the chain being queued.
+  // Only operators that move at least kForkBytes (inputs + output) ever leave their chain: a
+  // cross-stream edge costs an event and a wait, about what a 32 MiB elementwise pass takes,
+  // and the launch-bound training graphs (MLP, MNIST CNN) must not pay it on every branch.
   static constexpr uint64_t kStayBehind = 3;
-  int PickStream(const std::vector<Tensor>& inputs);
+  static constexpr size_t kForkBytes = (size_t)32 << 20;
+  int PickStream(const std::vector<Tensor>& inputs, const Scale& out_size);
   bool dataflow_ = false;
   uint64_t issued_[HipDevice::kParallelism] = {};  // operators ever queued per stream
   uint64_t queued_[HipDevice::kParallelism] = {};  // operators queued per stream since Sync
   uint64_t epoch_ = 1;                             // Syncs so far + 1
+  int last_stream_ = 0;                            // stream of the operator queued last
 };
 
 }  // namespace minerva

@@ -228,6 +228,16 @@ class Net:
                                          l.ctypes.data_as(fp), ctypes.c_size_t(l.size)),
                "net_load_batch")
 
+    def prefetch_batch(self, data, label):
+        """Loads the batch of the NEXT step while the step in flight keeps the GPU busy (a second
+        worker stream, pinned staging); the next `step` trains on it."""
+        d = np.ascontiguousarray(data, np.float32).ravel()
+        l = np.ascontiguousarray(label, np.float32).ravel()
+        fp = ctypes.POINTER(ctypes.c_float)
+        _check(lib().mnvh_net_prefetch_batch(self.h, d.ctypes.data_as(fp), ctypes.c_size_t(d.size),
+                                             l.ctypes.data_as(fp), ctypes.c_size_t(l.size)),
+               "net_prefetch_batch")
+
     def set_fused(self, on=True, updates=False):
         """Opt-in fast path: fused epilogues instead of separate ReLU / bias / update operators.
         `updates`: the weight updates are also applied where the weight gradients are produced;

@@ -76,10 +76,11 @@ def net_state(net, label_floats, weight_gradients=True):
 
 
 def run_steps(kind, batch, variant, lr, params, batches, fused=False, fused_updates=False,
-              **runtime_args):
+              prefetch=False, **runtime_args):
     """One step per batch, operator by operator (fused: with the fused operators;
     fused_updates: weight updates in the gradient kernels' stores as well, which leaves no
-    weight gradients to read); the state after every step."""
+    weight gradients to read; prefetch: every batch but the first is loaded on a second
+    stream while the step before it is in flight); the state after every step."""
     from minerva_amd import hostapi
     runtime_args.setdefault("sync_each_op", False)
     r = hostapi.Runtime(0, **runtime_args)
@@ -89,9 +90,12 @@ def run_steps(kind, batch, variant, lr, params, batches, fused=False, fused_upda
     for k, v in params.items():
         net.set_param(k, v)
     states = []
-    for d, l in batches:
-        net.load_batch(d, l)
+    for i, (d, l) in enumerate(batches):
+        if not prefetch or i == 0:
+            net.load_batch(d, l)
         net.step(lr)
+        if prefetch and i + 1 < len(batches):
+            net.prefetch_batch(*batches[i + 1])   # under the step that was just queued
         states.append(net_state(net, l.size, weight_gradients=not fused_updates))
     run_steps.ops_issued = r.ops_issued()  # of the run that just ended
     net.close()

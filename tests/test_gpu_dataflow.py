@@ -92,11 +92,11 @@ def test_random_operator_graph_with_frees():
     """A few hundred operators over a changing set of live tensors, tensors freed while
     their consumers are queued: dataflow placement against the one-stream order."""
     from minerva_amd import hostapi
-    m = 192
+    m = 2048   # 16 MiB tensors: large enough for an operator to start a chain of its own
     rng_ops = np.random.default_rng(11)
     plan = []
     live = 4
-    for _ in range(300):
+    for _ in range(120):
         kind = int(rng_ops.integers(0, 5))
         i, j = int(rng_ops.integers(0, live)), int(rng_ops.integers(0, live))
         drop = int(rng_ops.integers(0, live + 1)) if live > 6 else -1
@@ -229,3 +229,21 @@ def test_mode_switched_on_live_data_tracks_readers_of_older_tensors():
             again.read()
         r.close()
     assert_bits_equal(results["switched"], results["order"], "product that read the freed block")
+
+
+@pytest.mark.parametrize("kind,batch", [("mlp", 256), ("cnn", 64), ("alexnet", 2)])
+def test_batches_prefetched_under_the_running_step_train_the_same(kind, batch):
+    """The next batch loaded on a second stream while a step is in flight (what the
+    reference's trainer gets from its data provider, owl/owl/net/trainer.py:118-145): five
+    different batches, every parameter, gradient and probability bit-identical to loading each
+    batch in stream order before its step."""
+    params, batches = net_batches(kind, batch, 5)
+    say("batches loaded in stream order", kind, batch)
+    want = run_steps(kind, batch, 0, 0.05, params, batches)
+    say("batches prefetched under the step before", kind, batch)
+    got = run_steps(kind, batch, 0, 0.05, params, batches, prefetch=True)
+    for i, (g, w) in enumerate(zip(got, want)):
+        for k in w:
+            assert_bits_equal(g[k], w[k], "%s after step %d" % (k, i))
+    # the batches differ, so a step that trained on a stale batch would show
+    assert not np.array_equal(want[1]["prob"], want[2]["prob"])
