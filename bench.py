@@ -284,6 +284,16 @@ def sgemm_bench():
              "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
                           "unit": "TFLOP/s", "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}}
     log("sgemm 4096^3: %.3f ms, %.1f TFLOP/s" % (ms, tf))
+    # the same product back to back for more than a second: the clock the chip sustains under
+    # this load, beside the burst figure above (50 calls spread over five batches)
+    calls = 1200
+    t_sus = dev.time_ms(lambda: L.mnv_sgemm_nn(a.p, b.p, c.p, m, n, k, None, 0, dev.stream),
+                        iters=calls, warmup=20, reps=1)
+    tf_sus = 2.0 * m * n * k / (t_sus * 1e-3) / 1e12
+    sgemm["sustained"] = {"calls_back_to_back": calls, "seconds": round(calls * t_sus * 1e-3, 2),
+                          "ms": round(t_sus, 4), "tflops": round(tf_sus, 2),
+                          "frac": round(tf_sus / PEAK_FP32_MFMA_TFLOPS, 4)}
+    log("sgemm 4096^3 sustained over %d calls: %.3f ms, %.1f TFLOP/s" % (calls, t_sus, tf_sus))
     # the same product with one operand given transposed (the operand is read in place: what
     # the reference writes as Trans + MatMult); the values differ, the timing does not care
     t_tn = dev.time_ms(lambda: L.mnv_sgemm_tn(a.p, b.p, None, c.p, m, n, k, None, 0, dev.stream),
@@ -368,8 +378,12 @@ def bandwidth_table(L, dev, rng, ne):
         ("max dim 0", 4, lambda x, y, z: lambda: L.mnv_reduce_max_col(x.p, small.p, m, n, S)),
         ("max dim 1", 4, lambda x, y, z: lambda: L.mnv_reduce_max_row(x.p, small.p, m, n, S)),
         ("maxindex dim 0", 4, lambda x, y, z: lambda: L.mnv_maxindex_col(x.p, small.p, m, n, S)),
+        ("maxindex dim 1", 4, lambda x, y, z: lambda: L.mnv_maxindex_row(x.p, small.p, m, n, S)),
         ("softmax rows", 8, lambda x, y, z: lambda: L.mnv_softmax_instance_fwd(x.p, z.p, n, m, 1, 1, S)),
         ("softmax rows bwd", 12, lambda x, y, z: lambda: L.mnv_softmax_instance_bwd(x.p, y.p, z.p, n, m, 1, 1, S)),
+        # channel mode (cuda_perform.cu:355-369): 1024 channels over 256 x 256 positions
+        ("softmax over channels", 8, lambda x, y, z: lambda: L.mnv_softmax_channel_fwd(x.p, z.p, 1, 1024, 256, 256, S)),
+        ("softmax over channels bwd", 12, lambda x, y, z: lambda: L.mnv_softmax_channel_bwd(x.p, y.p, z.p, 1, 1024, 256, 256, S)),
         ("transpose", 8, lambda x, y, z: lambda: L.mnv_transpose(x.p, z.p, m, n, S)),
     ]
     table = []
@@ -416,6 +430,10 @@ def bandwidth_table(L, dev, rng, ne):
          lambda px, py, pdy, o1, o2, o3, o4: lambda: L.mnv_maxpool_fwd(px.p, py.p, *geo, S)),
         ("maxpool 3x3/2 bwd (pool1)", 4 * (2 * nin + nout),
          lambda px, py, pdy, o1, o2, o3, o4: lambda: L.mnv_maxpool_bwd(px.p, py.p, pdy.p, o3.p, *geo, S)),
+        ("avgpool 3x3/2 fwd (pool1 shape)", 4 * (nin + nout),
+         lambda px, py, pdy, o1, o2, o3, o4: lambda: L.mnv_avgpool_fwd(px.p, py.p, *geo, S)),
+        ("avgpool 3x3/2 bwd (pool1 shape)", 4 * (nin + nout),
+         lambda px, py, pdy, o1, o2, o3, o4: lambda: L.mnv_avgpool_bwd(px.p, py.p, pdy.p, o3.p, *geo, S)),
         ("conv bias gradient (conv1)", 4 * nin,
          lambda px, py, pdy, o1, o2, o3, o4: lambda: L.mnv_conv_bwd_bias(
              px.p, small.p, 256, 96, 55, 55, bias_ws.p, ctypes.c_size_t(1 << 20), S)),
@@ -609,6 +627,127 @@ def cpu_baseline(batch=4, full=False):
     return out
 
 
+def parity_report():
+    """Part of the CPU leg: every operator family once on the GPU (through the C ABI) and once
+    through the CPU oracle on the same seeded inputs at a reduced size; "bit_exact" where the
+    operator is one IEEE operation or a selection per element, else the normwise error
+    max|gpu - cpu| / max|cpu| against the 1e-4 bound.  The tests hold the same comparisons at
+    more sizes; this puts the figures of THIS run into the line."""
+    from minerva_amd import capi
+    from oracle import mnv_oracle as ora
+    L = capi.lib()
+    dev = capi.Device(0)
+    S = dev.stream
+    rng = np.random.default_rng(21)
+    f = ctypes.c_float
+    m, n = 1024, 768
+    x, y = rng.standard_normal(m * n, dtype=np.float32), rng.standard_normal(m * n, dtype=np.float32)
+    dx, dy = dev.upload(x), dev.upload(y)
+    out = []
+
+    def run(fn, count):
+        o = dev.empty(count)
+        capi.check(fn(o), "parity call")
+        dev.sync()
+        return dev.download(o)
+
+    def exact(name, got, want):
+        same = bool(np.array_equal(np.asarray(got, np.float32).view(np.uint32),
+                                   np.asarray(want, np.float32).view(np.uint32)))
+        out.append({"op": name, "bit_exact": same})
+
+    def close(name, got, want):
+        want = np.asarray(want, np.float64)
+        err = float(np.max(np.abs(np.asarray(got, np.float64) - want)) / max(np.max(np.abs(want)), 1e-30))
+        out.append({"op": name, "normwise_error": float("%.3g" % err), "within_1e-4": err <= 1e-4})
+
+    for name, typ, fn in (("add", ora.ADD, L.mnv_add), ("sub", ora.SUB, L.mnv_sub),
+                          ("mul", ora.MUL, L.mnv_mul), ("div", ora.DIV, L.mnv_div)):
+        exact(name, run(lambda o: fn(dx.p, dy.p, o.p, m * n, S), m * n), ora.arithmetic(typ, x, y))
+    exact("scalar mul", run(lambda o: L.mnv_const_mul(dx.p, o.p, f(3.291), m * n, S), m * n),
+          ora.arithmetic_const(ora.MUL, 1, 3.291, x))
+    col, row = rng.standard_normal(n, dtype=np.float32), rng.standard_normal(m, dtype=np.float32)
+    dcol, drow = dev.upload(col), dev.upload(row)
+    exact("broadcast add {1,n}", run(lambda o: L.mnv_norm_add_col(dx.p, dcol.p, o.p, m, n, S), m * n),
+          ora.norm_arithmetic(ora.ADD, x, [m, n], col, [0]))
+    exact("broadcast add {m,1}", run(lambda o: L.mnv_norm_add_row(dx.p, drow.p, o.p, m, n, S), m * n),
+          ora.norm_arithmetic(ora.ADD, x, [m, n], row, [1]))
+    close("exp", run(lambda o: L.mnv_exp(dx.p, o.p, m * n, S), m * n), ora.elewise(ora.EXP, x))
+    for name, alg, fw, bw in (("sigmoid", ora.SIGMOID, L.mnv_sigmoid_fwd, L.mnv_sigmoid_bwd),
+                              ("relu", ora.RELU, L.mnv_relu_fwd, L.mnv_relu_bwd),
+                              ("tanh", ora.TANH, L.mnv_tanh_fwd, L.mnv_tanh_bwd)):
+        top = ora.activation_fwd(alg, x)
+        dtop = dev.upload(top)
+        (exact if alg == ora.RELU else close)(name + " fwd", run(lambda o: fw(dx.p, o.p, m * n, S), m * n), top)
+        (exact if alg == ora.RELU else close)(
+            name + " bwd", run(lambda o: bw(dx.p, dtop.p, dy.p, o.p, m * n, S), m * n),
+            ora.activation_bwd(alg, y, top, x))
+    close("sum dim 0", run(lambda o: L.mnv_reduce_sum_col(dx.p, o.p, m, n, S), n), ora.reduction(ora.SUM, x, [m, n], [0]))
+    close("sum dim 1", run(lambda o: L.mnv_reduce_sum_row(dx.p, o.p, m, n, S), m), ora.reduction(ora.SUM, x, [m, n], [1]))
+    exact("max dim 0", run(lambda o: L.mnv_reduce_max_col(dx.p, o.p, m, n, S), n), ora.reduction(ora.MAX, x, [m, n], [0]))
+    exact("max dim 1", run(lambda o: L.mnv_reduce_max_row(dx.p, o.p, m, n, S), m), ora.reduction(ora.MAX, x, [m, n], [1]))
+    exact("maxindex dim 0", run(lambda o: L.mnv_maxindex_col(dx.p, o.p, m, n, S), n), ora.maxindex(x, [m, n], 0))
+    exact("maxindex dim 1", run(lambda o: L.mnv_maxindex_row(dx.p, o.p, m, n, S), m), ora.maxindex(x, [m, n], 1))
+    sm = ora.softmax_instance_fwd(x, n, m, 1, 1)
+    dsm = dev.upload(sm)
+    close("softmax rows", run(lambda o: L.mnv_softmax_instance_fwd(dx.p, o.p, n, m, 1, 1, S), m * n), sm)
+    close("softmax rows bwd", run(lambda o: L.mnv_softmax_instance_bwd(dy.p, dsm.p, o.p, n, m, 1, 1, S), m * n),
+          ora.softmax_instance_bwd(y, sm, n, m, 1, 1))
+    exact("transpose", run(lambda o: L.mnv_transpose(dx.p, o.p, m, n, S), m * n), ora.transpose(x, m, n))
+    gm, gn, gk = 384, 200, 1000
+    a, b = rng.standard_normal(gm * gk, dtype=np.float32), rng.standard_normal(gk * gn, dtype=np.float32)
+    da, db = dev.upload(a), dev.upload(b)
+    close("sgemm 384x1000x200", run(lambda o: L.mnv_sgemm_nn(da.p, db.p, o.p, gm, gn, gk, None, 0, S), gm * gn),
+          ora.matmult(a, b, gm, gn, gk))
+    # conv3 of the AlexNet shape at batch 4, pool1's window on a 27x27 plane
+    p = (4, 256, 384, 13, 13, 1, 1, 1, 1, 3, 3)
+    N, C, K, H, W = p[:5]
+    cx, cw = rng.standard_normal(N * C * H * W, dtype=np.float32), rng.standard_normal(K * C * 9, dtype=np.float32) * np.float32(0.05)
+    cb, cdy = rng.standard_normal(K, dtype=np.float32), rng.standard_normal(N * K * H * W, dtype=np.float32)
+    dcx, dcw, dcb, dcdy = dev.upload(cx), dev.upload(cw), dev.upload(cb), dev.upload(cdy)
+    wsb = 64 << 20
+    ws = dev.empty(wsb // 4)
+    z = ctypes.c_size_t(wsb)
+    close("conv forward", run(lambda o: L.mnv_conv_fwd(dcx.p, dcw.p, dcb.p, o.p, *p, ws.p, z, S), N * K * H * W),
+          ora.conv_fwd(cx, cw, cb, *p))
+    close("conv backward data", run(lambda o: L.mnv_conv_bwd_data(dcdy.p, dcw.p, o.p, *p, ws.p, z, S), N * C * H * W),
+          ora.conv_bwd_data(cdy, cw, *p))
+    close("conv backward filter", run(lambda o: L.mnv_conv_bwd_filter(dcx.p, dcdy.p, o.p, *p, ws.p, z, S), K * C * 9),
+          ora.conv_bwd_filter(cdy, cx, *p))
+    close("conv backward bias", run(lambda o: L.mnv_conv_bwd_bias(dcdy.p, o.p, N, K, H, W, ws.p, z, S), K),
+          ora.conv_bwd_bias(cdy, N, K, H, W))
+    g = (8, 16, 27, 27, 2, 2, 3, 3, 0, 0)
+    px = np.round(rng.standard_normal(8 * 16 * 27 * 27) * 2).astype(np.float32)  # many ties
+    pt = ora.pool_fwd(ora.POOL_MAX, px, *g)
+    pdy = rng.standard_normal(pt.size, dtype=np.float32)
+    dpx, dpt, dpdy = dev.upload(px), dev.upload(pt), dev.upload(pdy)
+    exact("max pooling forward", run(lambda o: L.mnv_maxpool_fwd(dpx.p, o.p, *g, S), pt.size), pt)
+    exact("max pooling backward (ties)", run(lambda o: L.mnv_maxpool_bwd(dpx.p, dpt.p, dpdy.p, o.p, *g, S), px.size),
+          ora.pool_bwd(ora.POOL_MAX, pdy, pt, px, *g))
+    del dev
+    # the benchmark's own step: batch 256 on the GPU, and the probabilities of its first four
+    # images against the oracle's forward pass at batch 4 on the same parameters and images
+    # (the forward pass treats images independently)
+    from minerva_amd import hostapi
+    from oracle import nets
+    params, data, label = nets.make_inputs("alexnet", BATCH)
+    _, want = nets.alexnet_forward(params, np.ascontiguousarray(data[:4 * 3 * 227 * 227]), 4)
+    rt = hostapi.Runtime(0, sync_each_op=False)
+    net = hostapi.Net(rt, "alexnet", BATCH)
+    for k, v in params.items():
+        net.set_param(k, v)
+    net.load_batch(data, label)
+    net.step(0.01)
+    rt.sync()
+    prob = net.read("prob", 1000 * BATCH)
+    net.close()
+    rt.close()
+    close("alexnet step at batch 256: probabilities of the first 4 images", prob[:4000], want)
+    bad = [r["op"] for r in out if not (r.get("bit_exact") or r.get("within_1e-4"))]
+    return {"against": "the CPU oracle (oracle/mnv_oracle.c), same seeded inputs, reduced sizes",
+            "all_within_bounds": not bad, "failed": bad, "ops": out}
+
+
 SECTIONS = ("alexnet", "sgemm", "eltwise", "small", "owl", "cpu")
 
 
@@ -700,6 +839,10 @@ def main():
     line["device"] = dev_info
     if "cpu" in want:
         line["cpu_baseline"] = cpu_baseline(full=args.cpu_full)
+        line["cpu_baseline"]["parity"] = parity_report()
+        log("parity against the CPU oracle: %s" % ("all operators within their bounds"
+            if line["cpu_baseline"]["parity"]["all_within_bounds"]
+            else "FAILED: " + ", ".join(line["cpu_baseline"]["parity"]["failed"])))
     print(json.dumps(line))
 
 

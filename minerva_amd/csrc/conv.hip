@@ -765,14 +765,15 @@ int pick_tile(int m, int n) {
 // A 64x64 or 128x32 tile does little arithmetic per k-slab, so a slab costs one trip to
 // memory and back; its kernels need about 64 registers and at most 24 KB of LDS, which
 // lets a CU hold six to eight workgroups whose trips overlap.  When the output has fewer tiles than that, the
-// reduction is cut into k ranges (at least six slabs each) until about 2048 workgroups
-// are in flight.  `ws_floats`: workspace left for the partial results.
+// reduction is cut into k ranges (at least six slabs each) until about eight workgroups per
+// CU are in flight.  `ws_floats`: workspace left for the partial results.
 int small_tile_splits(int tile, int m, int n, int slabs, size_t ws_floats) {
   if (tile != 0 && tile != 3) return 1;
   const int bm = kTileM[tile], bn = kTileN[tile];
   long long tiles = (long long)((m + bm - 1) / bm) * ((n + bn - 1) / bn);
-  if (tiles >= 1536) return 1;
-  long long want = (2048 + tiles - 1) / tiles;
+  const long long cus = mnv_cu_count();
+  if (tiles >= 6 * cus) return 1;
+  long long want = (8 * cus + tiles - 1) / tiles;
   if (want > slabs / 6) want = slabs / 6;
   size_t fit = ws_floats / ((size_t)m * n);
   if ((size_t)want > fit) want = (long long)fit;

@@ -166,9 +166,9 @@ __device__ __forceinline__ int mnv_tile_remap(int t, int total) {
   return t < per_xcd * 8 ? (t % 8) * per_xcd + t / 8 : t;
 }
 
-// Tail: tiles are whole units of work, so when their number is not a multiple of the 256
-// CUs the CUs that receive one tile more than the others set the duration (676 tiles: three
-// on some CUs, 2.64 on average).  The tiles past the last multiple of 256 (`tail_begin`
+// Tail: tiles are whole units of work, so when their number is not a multiple of the CU
+// count the CUs that receive one tile more than the others set the duration (676 tiles on 256
+// CUs: three on some, 2.64 on average).  The tiles past the last multiple (`tail_begin`
 // on, in dispatch order) are therefore cut into `tail_z` k ranges, one workgroup each: small
 // units that are dispatched last and fill the CUs evenly.  Their partial tiles go to the
 // workspace, tile by tile, and mnv_gemm_tail_reduce_kernel adds them in range order.
@@ -676,8 +676,9 @@ __global__ __launch_bounds__(256) void mnv_gemm_streamk_reduce_kernel(P prob,
 }
 
 // Which tiles form the tail and into how many k ranges each is cut (z <= 1: none).  Only
-// for launches of at least 256 large tiles without k ranges of their own; taken when the
-// uneven last tile per CU costs at least 3% (tiles / 256 = 2.64: 12%; 11.39: 5%; 3.96: 1%),
+// for launches of at least one large tile per CU (the device's count, mnv_cu_count) without k
+// ranges of their own; taken when the uneven last tile per CU costs at least 3% (on 256 CUs:
+// tiles / 256 = 2.64: 12%; 11.39: 5%; 3.96: 1%),
 // with about three small workgroups per CU (two to four measured alike: conv2 data gradient
 // 1.77 -> 1.74 / 1.71 / 1.70 ms, conv5 forward 0.71 -> 0.66 ms with any of them), at least
 // eight slabs each, and only as far as the workspace holds the partial tiles.
@@ -686,13 +687,14 @@ struct MnvTailPlan {
 };
 static inline MnvTailPlan mnv_tail_plan(long long tiles, int slabs, size_t tile_floats,
                                         size_t ws_floats) {
+  const int cus = mnv_cu_count();
   const MnvTailPlan none{(int)(tiles < 0x7fffffff ? tiles : 0x7fffffff), 1};
-  if (tiles < 256 || tiles > 0x3fffffff) return none;
-  const int rem = (int)(tiles % 256);
+  if (tiles < cus || tiles > 0x3fffffff) return none;
+  const int rem = (int)(tiles % cus);
   if (rem == 0) return none;
-  const double per_cu = (double)tiles / 256.0, most = (double)((tiles + 255) / 256);
+  const double per_cu = (double)tiles / cus, most = (double)((tiles + cus - 1) / cus);
   if ((most - per_cu) / most < 0.03) return none;
-  int z = 768 / rem;
+  int z = 3 * cus / rem;
   if (z > 16) z = 16;
   if (z > slabs / 8) z = slabs / 8;
   const size_t fit = ws_floats / ((size_t)rem * tile_floats);
@@ -702,7 +704,7 @@ static inline MnvTailPlan mnv_tail_plan(long long tiles, int slabs, size_t tile_
 }
 
 // Number of k ranges for `tiles` output tiles of `slabs` k-slabs each.  Workgroups are
-// dealt evenly to 256 CUs that hold four of them at a time, and the kernel ends when the
+// dealt evenly to the device's CUs, which hold four of them at a time, and the kernel ends when the
 // fullest CU does: a split count that puts a few workgroups past a multiple of 1024 costs a
 // whole extra round, so the estimate below (workgroups on the fullest CU x slabs each,
 // corrected for the matrix pipe running below its rate with fewer than four workgroups in
@@ -713,11 +715,12 @@ static inline MnvTailPlan mnv_tail_plan(long long tiles, int slabs, size_t tile_
 static inline int mnv_pick_splits(long long tiles, int slabs, int max_splits, double per_split = 0.0,
                                   double* cost_out = nullptr) {
   static const double rate[5] = {1.0, 0.45, 0.75, 0.92, 1.0};
+  const int cus = mnv_cu_count();
   if (max_splits < 1) max_splits = 1;
   int best = 1;
   double best_cost = 0;
   for (int s = 1; s <= max_splits; ++s) {
-    long long per_cu = (tiles * s + 255) / 256;
+    long long per_cu = (tiles * s + cus - 1) / cus;
     int len = (slabs + s - 1) / s;
     double cost = (double)per_cu * (len + 4) / rate[per_cu < 4 ? per_cu : 4] + (s > 1 ? per_split * s : 0.0);
     if (s == 1 || cost < best_cost * 0.98) {  // prefer fewer partial results on a near tie

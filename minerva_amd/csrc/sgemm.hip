@@ -171,7 +171,7 @@ SgemmPlan plan_sgemm(int m, int n, int k, size_t ws_floats) {
     if (max_splits > slabs / 4) max_splits = slabs / 4;
     const size_t fit = mn ? ws_floats / mn : 0;
     if ((size_t)max_splits > fit) max_splits = (int)fit;
-    if (tiles >= 1024 || slabs < 8) max_splits = 1;
+    if (tiles >= 4LL * mnv_cu_count() || slabs < 8) max_splits = 1;  // one per resident workgroup
     const double unit = small ? 0.31 : 1.0;
     double cost;
     const int splits = mnv_pick_splits(tiles, slabs, max_splits, per_split / unit, &cost);
