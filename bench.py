@@ -693,7 +693,7 @@ def parity_report():
     close("softmax rows", run(lambda o: L.mnv_softmax_instance_fwd(dx.p, o.p, n, m, 1, 1, S), m * n), sm)
     close("softmax rows bwd", run(lambda o: L.mnv_softmax_instance_bwd(dy.p, dsm.p, o.p, n, m, 1, 1, S), m * n),
           ora.softmax_instance_bwd(y, sm, n, m, 1, 1))
-    exact("transpose", run(lambda o: L.mnv_transpose(dx.p, o.p, m, n, S), m * n), ora.transpose(x, m, n))
+    exact("transpose", run(lambda o: L.mnv_transpose(dx.p, o.p, m, n, S), m * n), ora.transpose(x, n, m))
     gm, gn, gk = 384, 200, 1000
     a, b = rng.standard_normal(gm * gk, dtype=np.float32), rng.standard_normal(gk * gn, dtype=np.float32)
     da, db = dev.upload(a), dev.upload(b)

@@ -61,6 +61,10 @@ int mnvh_runtime_dataflow_stats(void* runtime, unsigned long long* producer_wait
  * placement.  Drains the device first; every tensor stays valid, and tensors created before
  * the switch are tracked from their first use in the new mode. */
 int mnvh_runtime_set_dataflow(void* runtime, int enable);
+/* Dataflow mode: places the following operators on worker stream `stream` (0..3), -1 returns to
+ * automatic placement (an operator follows its newest input that is still in flight).  What
+ * owl.set_device is between devices in the reference, between the streams of one device. */
+int mnvh_runtime_set_stream(void* runtime, int stream);
 
 /* Per-operator device timing (two events per operator on its own stream).  The read
  * synchronises, writes one "name<TAB>launches<TAB>total_ms" line per operator name and

@@ -298,6 +298,10 @@ int mnvh_runtime_dataflow_stats(void* runtime, unsigned long long* producer_wait
   });
 }
 
+int mnvh_runtime_set_stream(void* runtime, int stream) {
+  return Guard([&] { static_cast<Runner*>(runtime)->SetStream(stream); });
+}
+
 int mnvh_runtime_set_dataflow(void* runtime, int enable) {
   return Guard([&] { static_cast<Runner*>(runtime)->SetDataflow(enable != 0); });
 }

@@ -27,27 +27,32 @@ void Runner::SetDataflow(bool on) {
   Sync();
   device_->set_dataflow(on);
   if (!on) device_->set_sync_each_op(false);
+  if (!on) forced_stream_ = -1;
   dataflow_ = on;
 }
 
 int Runner::PickStream(const std::vector<Tensor>& inputs, const Scale& out_size) {
+  if (forced_stream_ >= 0) return forced_stream_;
   const TensorNode* newest = nullptr;
-  size_t bytes = static_cast<size_t>(out_size.Prod()) * sizeof(float);
-  for (auto& t : inputs) {
-    bytes += static_cast<size_t>(t->size.Prod()) * sizeof(float);
+  for (auto& t : inputs)
     if (t->epoch == epoch_ && (!newest || t->id > newest->id)) newest = t.get();
-  }
-  // small operators never leave the chain: an event and a wait cost more than they take
-  const bool may_fork = bytes >= kForkBytes;
-  if (newest && (!may_fork || issued_[newest->stream] - newest->seq <= kStayBehind))
-    return newest->stream;
+  if (newest) return newest->stream;
   // inputs, but none in flight (weights of the last step, a resident batch): what this
   // operator makes is most likely for the chain that is being queued right now
-  if (!newest && (!inputs.empty() || !may_fork)) return last_stream_;
+  if (!inputs.empty()) return last_stream_;
+  // no inputs: a load or a fill.  A large one depends on nothing that is queued and goes
+  // where the least is queued; a small one is not worth an event and a wait later on
+  if (static_cast<size_t>(out_size.Prod()) * sizeof(float) < kForkBytes) return last_stream_;
   int pick = 0;
   for (int s = 1; s < static_cast<int>(HipDevice::kParallelism); ++s)
     if (queued_[s] < queued_[pick]) pick = s;
   return pick;
+}
+
+void Runner::SetStream(int stream) {
+  MNV_CHECK(stream >= -1 && stream < static_cast<int>(HipDevice::kParallelism)) << "bad stream";
+  MNV_CHECK(stream < 0 || dataflow_) << "operators are placed on streams in dataflow mode only";
+  forced_stream_ = stream;
 }
 
 Runner::~Runner() {

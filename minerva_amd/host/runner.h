@@ -45,6 +45,9 @@ class Runner : public DeviceListener {
   // Overwrites `t` from host memory on worker stream `stream` while the other streams keep
   // running (HipDevice::CopyFromHostOn); the caller vouches that no queued work touches `t`.
   void UploadOn(int stream, const Tensor& t, const float* host);
+  // Dataflow mode: the following operators go to worker stream `stream` (-1: placed
+  // automatically again).  Dependencies on tensors of other streams are kept by events.
+  void SetStream(int stream);
   // Switches between the one-stream order and dataflow placement; tensors stay valid.
   void SetDataflow(bool on);
 
@@ -161,17 +164,14 @@ class Runner : public DeviceListener {
   bool retain_ = false;
   std::vector<Tensor> retained_;
   // Dataflow placement.  An operator follows its newest input that is still in flight onto
-  // that input's stream (a chain and its short side branches stay together: stream order
-  // does the waiting, no event), unless more than kStayBehind operators have been queued on
-  // that stream behind the input: then the operator does not depend on that work and starts a
-  // chain of its own on the stream with the least queued since the last Sync.  So does an
-  // operator without inputs (a load of the next batch, a fill).  An operator whose inputs are
-  // all complete (weights of the last step, a resident batch) joins the stream that was given
-  // the operator before it: its result is most likely meant for the chain being queued.
-  // Only operators that move at least kForkBytes (inputs + output) ever leave their chain: a
-  // cross-stream edge costs an event and a wait, about what a 32 MiB elementwise pass takes,
-  // and the launch-bound training graphs (MLP, MNIST CNN) must not pay it on every branch.
-  static constexpr uint64_t kStayBehind = 3;
+  // that input's stream, so a chain and its side branches stay together and stream order does
+  // the waiting (on one GPU the branches of a training graph compete for the same CUs: spread
+  // over streams they gained nothing and every cross-stream edge cost an event and a wait).
+  // An operator whose inputs are all complete (weights of the last step, a resident batch)
+  // joins the stream that was given the operator before it.  Only a large operator without
+  // inputs (the load of the next batch) goes to the stream with the least queued since the last
+  // Sync.  A caller that knows two chains to be independent says so with SetStream, the
+  // counterpart on one device of the reference's owl.set_device (owl/owl/__init__.py).
   static constexpr size_t kForkBytes = (size_t)32 << 20;
   int PickStream(const std::vector<Tensor>& inputs, const Scale& out_size);
   bool dataflow_ = false;
@@ -179,6 +179,7 @@ class Runner : public DeviceListener {
   uint64_t queued_[HipDevice::kParallelism] = {};  // operators queued per stream since Sync
   uint64_t epoch_ = 1;                             // Syncs so far + 1
   int last_stream_ = 0;                            // stream of the operator queued last
+  int forced_stream_ = -1;                         // SetStream: where the caller wants the next operators
 };
 
 }  // namespace minerva

@@ -122,6 +122,10 @@ class Runtime:
         _check(lib().mnvh_runtime_pool_stats(self.h, ctypes.byref(t), ctypes.byref(c)), "pool_stats")
         return t.value, c.value
 
+    def set_stream(self, stream):
+        """Dataflow mode: the following operators go to worker stream `stream` (-1: automatic)."""
+        _check(lib().mnvh_runtime_set_stream(self.h, int(stream)), "set_stream")
+
     def set_dataflow(self, on):
         """Switches a live runtime between the one-stream order and dataflow placement."""
         _check(lib().mnvh_runtime_set_dataflow(self.h, 1 if on else 0), "set_dataflow")

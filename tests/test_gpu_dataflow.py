@@ -40,9 +40,14 @@ def test_consumer_on_another_stream_waits_for_its_producer():
         for _ in range(7):  # ~0.15 ms each: the host is several products ahead of the GPU
             chain.append(r.top("matmult", [chain[-1], tb]))
         mid = chain[3]
-        # `mid` is not the last thing queued on its stream, so this starts a new chain
+        # a side branch off the middle of the chain, declared independent of what follows `mid`:
+        # placed on another stream, it must wait for `mid` on the GPU
+        if mode == "dataflow":
+            r.set_stream((chain[0].stream + 1) % 4)
         side = r.top("arithmetic", [mid, mid], [0])
-        side2 = r.top("arithmetic_const", [side], [2, 0.5, 0])
+        if mode == "dataflow":
+            r.set_stream(-1)
+        side2 = r.top("arithmetic_const", [side], [2, 0.5, 0])   # follows `side` by itself
         if mode == "dataflow":
             assert all(c.stream == chain[0].stream for c in chain), "a chain shares one stream"
             assert side.stream != mid.stream, "the side branch must sit on another stream"
@@ -72,8 +77,8 @@ def test_block_recycled_on_another_stream_waits_for_its_last_reader():
         prod2 = r.top("matmult", [prod, tx])
         total_before, _ = r.pool_stats()
         y.free()                                              # y's block goes back to the pool
-        z = r.top("fill", [], [7.0, n, n])                    # same size: takes y's block
-        total_after, _ = r.pool_stats()
+        z = r.top("fill", [], [7.0, n, n])                    # 64 MiB, no inputs: a stream of its own;
+        total_after, _ = r.pool_stats()                       # same size: takes y's block
         assert total_after == total_before, "the fill must recycle the freed block"
         if mode == "dataflow":
             assert z.stream != prod.stream, "the fill must sit on another stream than the reader"
@@ -100,7 +105,7 @@ def test_random_operator_graph_with_frees():
         kind = int(rng_ops.integers(0, 5))
         i, j = int(rng_ops.integers(0, live)), int(rng_ops.integers(0, live))
         drop = int(rng_ops.integers(0, live + 1)) if live > 6 else -1
-        plan.append((kind, i, j, drop))
+        plan.append((kind, i, j, drop, int(rng_ops.integers(-1, 4))))
         live += 1
         if 0 <= drop < live - 1:
             live -= 1
@@ -110,7 +115,9 @@ def test_random_operator_graph_with_frees():
         ts = [r.tensor(_rand(m * m, 20 + k) / np.float32(16), [m, m]) for k in range(4)]
         streams = set()
         say("random graph", mode)
-        for kind, i, j, drop in plan:
+        for kind, i, j, drop, where in plan:
+            if mode == "dataflow":
+                r.set_stream(where)     # -1: automatic (follows the newest input in flight)
             if kind == 0:
                 t = r.top("matmult", [ts[i], ts[j]])
                 t2 = r.top("arithmetic_const", [t], [2, 1.0 / 16, 0])  # keep magnitudes bounded
@@ -180,7 +187,9 @@ def test_reader_of_lrn_scale_waits_for_the_forward_pass(ora):
             tail = r.top("arithmetic_const", [tail], [2, 1.0, 0])
             assert tail.stream == top.stream, "a chain stays on its stream"
         waits_before = r.dataflow_stats()[0]
+        r.set_stream((top.stream + 1 + rep) % 4 if (top.stream + 1 + rep) % 4 != top.stream else (top.stream + 1) % 4)
         twice = r.top("arithmetic_const", [scale], [2, 2.0, 0])   # reads `scale` alone
+        r.set_stream(-1)
         if twice.stream == top.stream:
             continue  # placement put both on one stream this time: stream order covers it
         crossed += 1
@@ -210,8 +219,6 @@ def test_mode_switched_on_live_data_tracks_readers_of_older_tensors():
         say("reader of a tensor older than the mode", mode)
         prod = r.top("matmult", [y, y])                         # ~1 ms, reads y throughout
         prod2 = r.top("matmult", [prod, tx])
-        for _ in range(4):                                      # the fill below must not follow `prod`
-            prod2 = r.top("arithmetic_const", [prod2], [2, 1.0, 0])
         waits_before = r.dataflow_stats()[1]
         total_before, _ = r.pool_stats()
         y.free()
