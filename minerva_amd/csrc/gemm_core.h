@@ -736,7 +736,7 @@ static inline int mnv_pick_splits(long long tiles, int slabs, int max_splits, do
 // splits*M*N*sizeof(float) bytes at `workspace`.
 // `tail_bytes`: bytes at `workspace` that a launch without k ranges may use for the partial
 // tiles of its tail (0: never cut the tail).
-template <class T, int G = 1, class P>
+template <class T, int G = 1, int PF = 1, class P>
 static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream_t s,
                            size_t tail_bytes = 0) {
   const int tiles_m = (prob.M + T::BM - 1) / T::BM, tiles_n = (prob.N + T::BNU - 1) / T::BNU;
@@ -758,7 +758,7 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
     MNV_HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= 64) return MNV_ERR_INVALID;
     if (!attr_set[dev].load(std::memory_order_acquire)) {
-      MNV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&mnv_gemm_kernel<T, P, G>),
+      MNV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&mnv_gemm_kernel<T, P, G, false, PF>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_limit));
       attr_set[dev].store(true, std::memory_order_release);
     }
@@ -770,7 +770,7 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
     tail = mnv_tail_plan((long long)tiles_m * tiles_n, total_slabs, (size_t)T::BM * T::BNU,
                          tail_bytes / sizeof(float));
   const int tail_tiles = tiles_m * tiles_n - tail.begin;
-  hipLaunchKernelGGL((mnv_gemm_kernel<T, P, G>),
+  hipLaunchKernelGGL((mnv_gemm_kernel<T, P, G, false, PF>),
                      dim3(tail.begin + tail_tiles * tail.z, 1, splits), dim3(T::NT * G), lds_bytes,
                      s, prob, tiles_m, tiles_n, per, reinterpret_cast<float*>(workspace),
                      tail.begin, tail.z);
