@@ -6,7 +6,7 @@ shapes under one name and only the grid tells them apart.
       per-kernel durations of a `rocprofv3 --kernel-trace --stats` run (microseconds)
 
   python -m minerva_amd.rocprof_summary counters <dir-or-db> [<dir-or-db> ...] [--only SUBSTR]
-                                        [--trace <dir-or-db>]
+                                        [--trace <dir-or-db>] [--show COUNTER,COUNTER,...]
       per-kernel averages of every counter of one or more `rocprofv3 --pmc` runs (one counter set
       per run), plus, where their counters are present, the derived columns
         cycles     = GRBM_GUI_ACTIVE / 8                        (the counter sums the eight XCDs)
@@ -91,7 +91,8 @@ def counter_rows(cons, only=""):
     return {key: {c: sum(v) / len(v) for c, v in d.items()} for key, d in vals.items()}
 
 
-def counter_table(rows, trace=None, min_cycles=20000):
+def counter_table(rows, trace=None, min_cycles=20000, show=None):
+    """`show`: the raw counters to print beside the derived columns (None: all of them)."""
     counters = sorted({c for d in rows.values() for c in d})
     derived = []
     have = lambda *names: all(n in counters for n in names)
@@ -107,7 +108,7 @@ def counter_table(rows, trace=None, min_cycles=20000):
         derived.append("waiting")
     if trace is not None and have("GRBM_GUI_ACTIVE"):
         derived += ["avg_us", "clock GHz"]
-    raw = [c for c in counters if c != "GRBM_GUI_ACTIVE"]
+    raw = [c for c in counters if c != "GRBM_GUI_ACTIVE" and (show is None or c in show)]
     head = "%-70s %9s %4s" % ("kernel", "grid.x", "z") + "".join(" %12s" % d for d in derived)
     head += "".join(" %26s" % c for c in raw)
     lines = [head]
@@ -151,12 +152,15 @@ def main(argv=None):
     c.add_argument("db", nargs="+")
     c.add_argument("--only", default="", help="kernel name substring")
     c.add_argument("--trace", default=None, help="kernel-trace run of the same command, for durations")
+    c.add_argument("--show", default=None, help="comma-separated raw counters to print (default: all)")
     args = ap.parse_args(argv)
     if args.what == "trace":
         sys.stdout.write(trace_table(trace_rows(open_db(args.db), args.by_grid), args.min_share))
     else:
         trace = trace_rows(open_db(args.trace), "*") if args.trace else None
-        sys.stdout.write(counter_table(counter_rows([open_db(p) for p in args.db], args.only), trace))
+        show = None if args.show is None else set(filter(None, args.show.split(",")))
+        sys.stdout.write(counter_table(counter_rows([open_db(p) for p in args.db], args.only), trace,
+                                       show=show))
 
 
 if __name__ == "__main__":

@@ -133,7 +133,16 @@ def test_softmax_instance(gpu, ora, length, lines):
     assert normwise(gpu.down(dout), ora.softmax_instance_bwd(dy, ref, lines, length, 1, 1)) <= TOL
 
 
-@pytest.mark.parametrize("n,c,h,w", [(2, 5, 3, 4), (3, 10, 1, 7), (4, 21, 13, 13), (1, 2, 1, 2)])
+@pytest.mark.parametrize("n,c,h,w", [
+    (2, 5, 3, 4), (3, 10, 1, 7), (4, 21, 13, 13), (1, 2, 1, 2),
+    (2, 64, 9, 15),      # the last channel count of the 64-position x 4-group kernel, ragged positions
+    (3, 65, 7, 11),      # the first of the 32 x 32 kernel
+    (2, 512, 5, 13),     # all channels in registers, forward and backward
+    (1, 1000, 6, 7),     # in registers forward, re-read backward
+    (1, 1024, 3, 33),
+    (2, 1500, 2, 17),    # re-read in both passes
+    (1, 1024, 256, 256),  # the 8192 x 8192-element case of the bandwidth table
+])
 def test_softmax_channel(gpu, ora, n, c, h, w):
     x = _rand(n * c * h * w, 25) * 3
     dy = _rand(x.size, 26)
