@@ -628,42 +628,65 @@ __global__ __launch_bounds__(256) void mnv_gemm_tail_reduce_kernel(P prob,
   }
 }
 
-// Adds the segments of every tile of a stream-k launch (see mnv_gemm_kernel) in workgroup
-// order and hands each element to the policy's store.  Workgroup w of the launch covered the
-// units [U w / W, U (w + 1) / W); tile t is the units [t S, (t + 1) S).  One thread per four
-// consecutive rows of a tile column; four segments' loads in flight.
-template <class T, class P>
+// Adds the segments of every tile of a stream-k launch (see mnv_gemm_kernel) in a fixed order
+// and hands each element to the policy's store.  Workgroup w of the launch covered the units
+// [U w / W, U (w + 1) / W); tile t is the units [t S, (t + 1) S).  A thread owns four
+// consecutive rows of a tile column; ZL threads share them: thread z adds the segments z,
+// z + ZL, ... in order, and the ZL sums are added in order through LDS.  An output of few
+// tiles has hundreds of segments per tile (three tiles on 768 workgroups: 256 each), which
+// one thread per element walked in 52 us; sixteen walk them in a quarter of that.
+template <class T, class P, int ZL>
 __global__ __launch_bounds__(256) void mnv_gemm_streamk_reduce_kernel(P prob,
                                                                       const float* __restrict__ partial,
                                                                       int tiles_m, int tiles_n,
                                                                       int workgroups) {
   constexpr int TILE = T::BM * T::BNU;
+  constexpr int QL = 256 / ZL;  // 4-vectors of a tile per workgroup
+  __shared__ mnv_f4 red[ZL > 1 ? 256 : 1];
   const int t = blockIdx.y;
   const long long S = prob.total_slabs, U = S * tiles_m * tiles_n, W = workgroups;
   const long long first = t * S, last = first + S;
   long long w0 = first * W / U;                  // U w0 / W <= first
   while (U * (w0 + 1) / W <= first) ++w0;        // the share that holds the tile's first unit
-  long long w1 = w0 + 1;
-  while (w1 < W && U * w1 / W < last) ++w1;      // one past the share that holds its last unit
+  long long w1 = (last * W + U - 1) / U;         // the first share that begins at or past the
+  while (w1 > w0 + 1 && U * (w1 - 1) / W >= last) --w1;  // tile's end (a step or two of rounding,
+  while (w1 < W && U * w1 / W < last) ++w1;              // not a walk over the shares)
   const int m0 = (t % tiles_m) * T::BM, n0 = (t / tiles_m) * T::BNU;
   const int count = (int)(w1 - w0);
   const float* p = partial + (size_t)(w0 + t) * TILE;
-  for (int e = (blockIdx.x * 256 + threadIdx.x) * 4; e < TILE; e += gridDim.x * 256 * 4) {
-    mnv_f4 s = *reinterpret_cast<const mnv_f4*>(p + e);
-    int z = 1;
-    for (; z + 3 < count; z += 4) {
+  const int tq = threadIdx.x % QL, tz = threadIdx.x / QL;
+  static_assert(TILE % (4 * QL) == 0, "whole passes");
+  for (int e = (blockIdx.x * QL + tq) * 4; e < TILE; e += gridDim.x * QL * 4) {
+    mnv_f4 s = {0.f, 0.f, 0.f, 0.f};
+    int z = tz;
+    if (z < count) {
+      s = *reinterpret_cast<const mnv_f4*>(p + (size_t)z * TILE + e);
+      z += ZL;
+    }
+    for (; z + 3 * ZL < count; z += 4 * ZL) {
       const mnv_f4 v0 = *reinterpret_cast<const mnv_f4*>(p + (size_t)z * TILE + e);
-      const mnv_f4 v1 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + 1) * TILE + e);
-      const mnv_f4 v2 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + 2) * TILE + e);
-      const mnv_f4 v3 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + 3) * TILE + e);
+      const mnv_f4 v1 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + ZL) * TILE + e);
+      const mnv_f4 v2 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + 2 * ZL) * TILE + e);
+      const mnv_f4 v3 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + 3 * ZL) * TILE + e);
       s.x += v0.x; s.y += v0.y; s.z += v0.z; s.w += v0.w;
       s.x += v1.x; s.y += v1.y; s.z += v1.z; s.w += v1.w;
       s.x += v2.x; s.y += v2.y; s.z += v2.z; s.w += v2.w;
       s.x += v3.x; s.y += v3.y; s.z += v3.z; s.w += v3.w;
     }
-    for (; z < count; ++z) {
+    for (; z < count; z += ZL) {
       const mnv_f4 v = *reinterpret_cast<const mnv_f4*>(p + (size_t)z * TILE + e);
       s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    if (ZL > 1) {
+      __syncthreads();  // the previous pass has read its sums
+      red[threadIdx.x] = s;
+      __syncthreads();
+      if (tz != 0) continue;
+#pragma unroll
+      for (int q = 1; q < ZL; ++q) {
+        const mnv_f4 v = red[q * QL + tq];
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+      }
     }
     const int m = m0 + e % T::BM, n = n0 + e / T::BM;
     if (n < prob.N) {
@@ -852,9 +875,22 @@ static int mnv_gemm_streamk_launch(const P& prob, void* workspace, size_t ws_byt
                      prob, tiles_m, tiles_n, 0, reinterpret_cast<float*>(workspace), 0, 1);
   int rc = MNV_LAUNCH_STATUS();
   if (rc) return rc;
-  hipLaunchKernelGGL((mnv_gemm_streamk_reduce_kernel<T, P>),
-                     dim3(T::BM * T::BNU / 1024, (unsigned)tiles), dim3(256), 0, s, prob,
-                     reinterpret_cast<const float*>(workspace), tiles_m, tiles_n, workgroups);
+  // segments per tile: workgroups / tiles, one more where a share straddles
+  const long long per_tile = workgroups / tiles + 1;
+  const float* part = reinterpret_cast<const float*>(workspace);
+  const dim3 block(256);
+  if (per_tile >= 64)
+    hipLaunchKernelGGL((mnv_gemm_streamk_reduce_kernel<T, P, 16>),
+                       dim3(T::BM * T::BNU / 64, (unsigned)tiles), block, 0, s, prob, part, tiles_m,
+                       tiles_n, workgroups);
+  else if (per_tile >= 32)
+    hipLaunchKernelGGL((mnv_gemm_streamk_reduce_kernel<T, P, 4>),
+                       dim3(T::BM * T::BNU / 256, (unsigned)tiles), block, 0, s, prob, part, tiles_m,
+                       tiles_n, workgroups);
+  else
+    hipLaunchKernelGGL((mnv_gemm_streamk_reduce_kernel<T, P, 1>),
+                       dim3(T::BM * T::BNU / 1024, (unsigned)tiles), block, 0, s, prob, part, tiles_m,
+                       tiles_n, workgroups);
   *done = true;
   return MNV_LAUNCH_STATUS();
 }
