@@ -240,8 +240,8 @@ def dominant_kernel_traffic():
 
 def dominant_kernel_roofline(prof, steps):
     """The filter-gradient operators of conv2..conv5 run the 128x128 MFMA kernel
-    (mnv_gemm_kernel<128x128x16, ConvBwdFilterFast>) followed by its split-k reduction; the
-    event pair brackets both, so the figure is slightly conservative."""
+    (mnv_gemm_kernel<128x128x16, ConvBwdFilterFast, stream-k>) followed by the reduction of its
+    shares' partial tiles; the event pair brackets both, so the figure is slightly conservative."""
     names = [n for n in prof if n.endswith("conv bp filter") and "stride:1*1" in n]
     launches = sum(prof[n][0] for n in names)
     total_ms = sum(prof[n][1] for n in names)
@@ -252,7 +252,8 @@ def dominant_kernel_roofline(prof, steps):
     avg_ms = total_ms / launches
     achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
     return {"bound": "mfma",
-            "kernel": "mnv_gemm_kernel<128x128x16,ConvBwdFilterFast<false,1|2>> (conv2-5 filter gradient)",
+            "kernel": "mnv_gemm_kernel<128x128x16,ConvBwdFilterFast<false,1|3>,stream-k,2 slabs ahead> "
+                      "(conv2-5 filter gradient) + its reduction",
             "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
             "traffic": dominant_kernel_traffic(),
