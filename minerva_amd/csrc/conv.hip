@@ -667,7 +667,9 @@ const int kTileM[4] = {64, 128, 128, 128}, kTileN[4] = {64, 128, 96, 32};
 // fourth workgroup per CU; measured on the four padded convolutions of the AlexNet shape, four
 // resident workgroups per CU with equal shares ran 16% slower than three (1.18 against
 // 1.03 ms per launch): the chip is then waiting for the L2 and fabric, not for the matrix pipe.
+#ifndef MNV_SK_PF
 #define MNV_SK_PF 2
+#endif
 // `plan` (optional): nothing is launched; plan[0] = rows of the tile, plan[1] = k ranges,
 // plan[2] = workgroups of the stream-k launch (0: k ranges).
 template <class P>

@@ -180,17 +180,28 @@ __device__ __forceinline__ int mnv_tile_remap(int t, int total) {
 // a long k this keeps 16 wavefronts per CU busy with a quarter of the partial results (and of
 // the reduction kernel's reads) that as many separate workgroups would write to memory.
 //
-// SK ("stream-k"): the launch has exactly as many workgroups as the chip holds at once and
-// the tiles x k-slabs of the whole product, laid end to end (tile-major), are dealt to them in
-// equal contiguous shares: workgroup w multiplies the units [U w / W, U (w + 1) / W).  A share
-// that crosses a tile boundary is worked off segment by segment; every segment leaves its
-// partial tile in slot w + tile of the workspace (w and tile never decrease from one segment
-// to the next and one of them grows, so the slots are distinct and W + tiles - 1 in number)
-// and mnv_gemm_streamk_reduce_kernel adds a tile's segments in workgroup order, which is
-// k order: deterministic.  With whole k ranges per workgroup (blockIdx.z) the chip works in
+// SK ("stream-k"): the launch has exactly as many workgroups as the chip holds at once (W) and
+// every one of them multiplies the same number of k-slabs, U / W of the U = tiles x slabs units
+// of the whole product.  With T tiles, Z = W / T of every tile's k ranges are "aligned": range
+// z of every tile covers the same slabs [z CH, (z + 1) CH), CH = U / W, one workgroup each,
+// and the workgroups of one range sit side by side on one XCD (the launch index is remapped
+// as for the tiles of a plain launch) -- they start together, run at the same pace and so
+// read the same operand panels at the same time, out of that XCD's L2.  What the aligned
+// ranges leave of every tile, the slabs from Z CH on, is laid end to end (tile-major) and
+// dealt in equal contiguous shares to the R = W - T Z workgroups that remain (none when T
+// divides W: the Z ranges then cut the tile evenly); such a share crosses tile boundaries and
+// is worked off segment by segment.  Every aligned range leaves its partial tile in slot
+// z T + tile of the workspace, every segment of remaining workgroup r in slot T Z + r + tile (r
+// and tile never decrease from one segment to the next and one of them grows, so the slots
+// are distinct, W + T at most), and mnv_gemm_streamk_reduce_kernel adds a tile's partial tiles
+// in k order: deterministic.  With whole k ranges per workgroup (blockIdx.z) the chip works in
 // rounds of equal workgroups, and a count of workgroups that is not a multiple of what the
 // chip holds leaves part of it idle for a whole round (54 tiles x 28 ranges = 1512 workgroups
-// on 1024 slots: the second round runs half empty).
+// on 1024 slots: the second round runs half empty).  Equal contiguous shares of the units
+// laid end to end without aligned ranges balance as well but no two workgroups ever read the
+// same panel at the same time: measured on the padded convolutions' filter gradients of the
+// AlexNet shape, 5.3 GB of L2 fills per launch for 3.9 GB of operand reads, and 3% slower
+// than whole ranges of 729 to 760 workgroups on 768 slots.
 //
 // PF: slabs the loads run ahead of the multiplies.  1: the loads of slab i + 1 are issued at
 // the head of slab i and written to LDS at its end, through one set of staging registers
@@ -214,13 +225,23 @@ __global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MI
   typedef MnvFetchMap<T::BM, T::BK, T::NT, P::A_KFAST> MapA;
   typedef MnvFetchMap<T::BN, T::BK, T::NT, P::B_KFAST> MapB;
 
-  // SK: the units of this workgroup that are still to do
+  // SK: slabs_per_split = CH, tail_begin = Z.  sk_p: this workgroup's place in the plan (an
+  // aligned range below T Z, else a remaining workgroup); sk_u, sk_end: the remaining
+  // workgroup's units, counted over the slabs the aligned ranges leave, that are still to do.
   long long sk_u = 0, sk_end = 0;
+  int sk_p = 0, sk_aligned = 0, sk_rest = 0;  // sk_rest: slabs per tile past the aligned ranges
   if constexpr (SK) {
-    const long long units = (long long)tiles_m * tiles_n * prob.total_slabs;
-    sk_u = units * blockIdx.x / gridDim.x;
-    sk_end = units * (blockIdx.x + 1) / gridDim.x;
-    if (sk_u >= sk_end) return;
+    const int tiles = tiles_m * tiles_n, aligned = tiles * tail_begin;
+    const int rem = (int)gridDim.x - aligned;
+    sk_p = mnv_tile_remap((int)blockIdx.x, (int)gridDim.x);
+    sk_aligned = sk_p < aligned;
+    sk_rest = prob.total_slabs - tail_begin * slabs_per_split;
+    if (!sk_aligned) {
+      const long long units = (long long)sk_rest * tiles;
+      sk_u = units * (sk_p - aligned) / rem;
+      sk_end = units * (sk_p - aligned + 1) / rem;
+      if (sk_u >= sk_end) return;
+    }
   }
   for (;;) {  // SK: one pass per segment; otherwise a single pass that ends in a return
   int vb = blockIdx.x, tail_part = -1;
@@ -229,7 +250,15 @@ __global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MI
     tail_part = i - tl * tail_z;
     vb = tail_begin + tl;
   }
-  if constexpr (SK) vb = (int)(sk_u / prob.total_slabs);
+  int sk_z = 0;
+  if constexpr (SK) {
+    if (sk_aligned) {
+      sk_z = sk_p / (tiles_m * tiles_n);
+      vb = sk_p - sk_z * (tiles_m * tiles_n);
+    } else {
+      vb = (int)(sk_u / sk_rest);
+    }
+  }
   const int b = SK ? vb : mnv_tile_remap(vb, tiles_m * tiles_n);
   const int tile_m = b % tiles_m, tile_n = b / tiles_m;
   const int m0 = tile_m * T::BM, n0 = tile_n * T::BNU;
@@ -238,9 +267,19 @@ __global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MI
   int slab_end = slab_begin + slabs_per_split;
   if (slab_end > prob.total_slabs) slab_end = prob.total_slabs;
   if constexpr (SK) {
-    slab_begin = (int)(sk_u - (long long)vb * prob.total_slabs);
-    const long long left = sk_end - sk_u;
-    slab_end = left < prob.total_slabs - slab_begin ? slab_begin + (int)left : prob.total_slabs;
+    if (sk_aligned) {
+      if ((int)gridDim.x == tiles_m * tiles_n * tail_begin) {  // no remaining workgroups: even cuts
+        slab_begin = (int)((long long)prob.total_slabs * sk_z / tail_begin);
+        slab_end = (int)((long long)prob.total_slabs * (sk_z + 1) / tail_begin);
+      } else {
+        slab_begin = sk_z * slabs_per_split;
+        slab_end = slab_begin + slabs_per_split;
+      }
+    } else {
+      slab_begin = prob.total_slabs - sk_rest + (int)(sk_u - (long long)vb * sk_rest);
+      const long long left = sk_end - sk_u;
+      slab_end = left < prob.total_slabs - slab_begin ? slab_begin + (int)left : prob.total_slabs;
+    }
   }
   // slabs every group steps through (the same count in all of them: the steps hold
   // workgroup barriers); a group whose quarter is shorter multiplies only its own slabs
@@ -470,13 +509,13 @@ __global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MI
 
   // Accumulator register r of lane (lm, lk) holds C[m = lm, n = lk*4 + r%4 + 8*(r/4)]
   // of its 32x32 block.
-  if constexpr (SK) {  // a segment: the whole tile, in tile order, into slot w + tile
+  if constexpr (SK) {  // a range or a segment: the whole tile, in tile order, into its slot
     // The empty asm keeps the store addresses from being computed once before the segment
     // loop (they do not change from segment to segment): 64 registers held across the main
     // loop would spill.
     int at = (wn + lk * 4) * T::BM + wm + lm;
     asm volatile("" : "+v"(at));
-    float* pt = partial + (size_t)(blockIdx.x + vb) * (T::BM * T::BNU) + at;
+    float* pt = partial + (size_t)(sk_aligned ? sk_p : sk_p + vb) * (T::BM * T::BNU) + at;
 #pragma unroll
     for (int i = 0; i < T::TM; ++i)
 #pragma unroll
@@ -484,6 +523,7 @@ __global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MI
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           pt[(j * 32 + (r & 3) + 8 * (r >> 2)) * T::BM + i * 32] = acc[i][j][r];
+    if (sk_aligned) return;
     sk_u += slab_end - slab_begin;
     if (sk_u >= sk_end) return;
     // every wavefront is past the last slab's barrier: the tile buffers and the policy's
@@ -628,53 +668,68 @@ __global__ __launch_bounds__(256) void mnv_gemm_tail_reduce_kernel(P prob,
   }
 }
 
-// Adds the segments of every tile of a stream-k launch (see mnv_gemm_kernel) in a fixed order
-// and hands each element to the policy's store.  Workgroup w of the launch covered the units
-// [U w / W, U (w + 1) / W); tile t is the units [t S, (t + 1) S).  A thread owns four
-// consecutive rows of a tile column; ZL threads share them: thread z adds the segments z,
+// Adds the partial tiles of every tile of a stream-k launch (see mnv_gemm_kernel) in k order and
+// hands each element to the policy's store.  Tile t has the `aligned` ranges' partial tiles in
+// the slots z T + t and, when the launch had R = W - T aligned remaining workgroups, the
+// segments of those that met the tile: remaining workgroup r covered the units [U r / R,
+// U (r + 1) / R) of the U = T `rest` slabs the aligned ranges left, tile t is the units [t rest,
+// (t + 1) rest), and the segment sits in slot T aligned + r + t.  A thread owns four
+// consecutive rows of a tile column; ZL threads share them: thread z adds the partial tiles z,
 // z + ZL, ... in order, and the ZL sums are added in order through LDS.  An output of few
-// tiles has hundreds of segments per tile (three tiles on 768 workgroups: 256 each), which
-// one thread per element walked in 52 us; sixteen walk them in a quarter of that.
+// tiles has hundreds of partial tiles per tile (three tiles on 768 workgroups: 256 each),
+// which one thread per element walked in 52 us; sixteen walk them in a quarter of that.
 template <class T, class P, int ZL>
 __global__ __launch_bounds__(256) void mnv_gemm_streamk_reduce_kernel(P prob,
                                                                       const float* __restrict__ partial,
                                                                       int tiles_m, int tiles_n,
-                                                                      int workgroups) {
+                                                                      int workgroups, int aligned,
+                                                                      int rest) {
   constexpr int TILE = T::BM * T::BNU;
   constexpr int QL = 256 / ZL;  // 4-vectors of a tile per workgroup
   __shared__ mnv_f4 red[ZL > 1 ? 256 : 1];
-  const int t = blockIdx.y;
-  const long long S = prob.total_slabs, U = S * tiles_m * tiles_n, W = workgroups;
-  const long long first = t * S, last = first + S;
-  long long w0 = first * W / U;                  // U w0 / W <= first
-  while (U * (w0 + 1) / W <= first) ++w0;        // the share that holds the tile's first unit
-  long long w1 = (last * W + U - 1) / U;         // the first share that begins at or past the
-  while (w1 > w0 + 1 && U * (w1 - 1) / W >= last) --w1;  // tile's end (a step or two of rounding,
-  while (w1 < W && U * w1 / W < last) ++w1;              // not a walk over the shares)
+  const int t = blockIdx.y, tiles = tiles_m * tiles_n;
+  const long long R = workgroups - (long long)tiles * aligned;
+  int seg_first = 0, segs = 0;  // remaining workgroups that met the tile
+  if (R > 0) {
+    const long long S = rest, U = S * tiles;
+    const long long first = t * S, last = first + S;
+    long long w0 = first * R / U;                  // U w0 / R <= first
+    while (U * (w0 + 1) / R <= first) ++w0;        // the share that holds the tile's first unit
+    long long w1 = (last * R + U - 1) / U;         // the first share that begins at or past the
+    while (w1 > w0 + 1 && U * (w1 - 1) / R >= last) --w1;  // tile's end (a step or two of rounding,
+    while (w1 < R && U * w1 / R < last) ++w1;              // not a walk over the shares)
+    seg_first = (int)w0;
+    segs = (int)(w1 - w0);
+  }
   const int m0 = (t % tiles_m) * T::BM, n0 = (t / tiles_m) * T::BNU;
-  const int count = (int)(w1 - w0);
-  const float* p = partial + (size_t)(w0 + t) * TILE;
+  const int count = aligned + segs;
+  // partial tile i of the tile, in k order
+  const float* p = partial + (size_t)t * TILE;
+  const float* pseg = partial + ((size_t)tiles * aligned + seg_first + t) * TILE;
+  auto part = [&](int i) -> const float* {
+    return i < aligned ? p + (size_t)i * tiles * TILE : pseg + (size_t)(i - aligned) * TILE;
+  };
   const int tq = threadIdx.x % QL, tz = threadIdx.x / QL;
   static_assert(TILE % (4 * QL) == 0, "whole passes");
   for (int e = (blockIdx.x * QL + tq) * 4; e < TILE; e += gridDim.x * QL * 4) {
     mnv_f4 s = {0.f, 0.f, 0.f, 0.f};
     int z = tz;
     if (z < count) {
-      s = *reinterpret_cast<const mnv_f4*>(p + (size_t)z * TILE + e);
+      s = *reinterpret_cast<const mnv_f4*>(part(z) + e);
       z += ZL;
     }
     for (; z + 3 * ZL < count; z += 4 * ZL) {
-      const mnv_f4 v0 = *reinterpret_cast<const mnv_f4*>(p + (size_t)z * TILE + e);
-      const mnv_f4 v1 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + ZL) * TILE + e);
-      const mnv_f4 v2 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + 2 * ZL) * TILE + e);
-      const mnv_f4 v3 = *reinterpret_cast<const mnv_f4*>(p + (size_t)(z + 3 * ZL) * TILE + e);
+      const mnv_f4 v0 = *reinterpret_cast<const mnv_f4*>(part(z) + e);
+      const mnv_f4 v1 = *reinterpret_cast<const mnv_f4*>(part(z + ZL) + e);
+      const mnv_f4 v2 = *reinterpret_cast<const mnv_f4*>(part(z + 2 * ZL) + e);
+      const mnv_f4 v3 = *reinterpret_cast<const mnv_f4*>(part(z + 3 * ZL) + e);
       s.x += v0.x; s.y += v0.y; s.z += v0.z; s.w += v0.w;
       s.x += v1.x; s.y += v1.y; s.z += v1.z; s.w += v1.w;
       s.x += v2.x; s.y += v2.y; s.z += v2.z; s.w += v2.w;
       s.x += v3.x; s.y += v3.y; s.z += v3.z; s.w += v3.w;
     }
     for (; z < count; z += ZL) {
-      const mnv_f4 v = *reinterpret_cast<const mnv_f4*>(p + (size_t)z * TILE + e);
+      const mnv_f4 v = *reinterpret_cast<const mnv_f4*>(part(z) + e);
       s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
     if (ZL > 1) {
@@ -826,7 +881,7 @@ static int mnv_gemm_launch(const P& prob, int splits, void* workspace, hipStream
 // many of the kernel's workgroups a CU holds) and nothing else.
 template <class T>
 static inline size_t mnv_gemm_streamk_bytes(long long tiles, int workgroups) {
-  return (size_t)(workgroups + tiles - 1) * T::BM * T::BNU * sizeof(float);
+  return (size_t)(workgroups + tiles) * T::BM * T::BNU * sizeof(float);
 }
 
 // `plan_workgroups` (optional): receives the number of workgroups of the plan, 0 when it
@@ -866,31 +921,49 @@ static int mnv_gemm_streamk_launch(const P& prob, void* workspace, size_t ws_byt
   if (tiles > workgroups || tiles * prob.total_slabs < 8LL * workgroups ||
       ws_bytes < mnv_gemm_streamk_bytes<T>(tiles, workgroups))
     return MNV_OK;
+  // Aligned ranges per tile and the slabs of each (see mnv_gemm_kernel).  A range or a segment
+  // costs about six slab times beside its slabs (first loads, the partial tile's store), and a
+  // remaining workgroup works off tiles / left + 1 segments: the ranges are made that much
+  // longer than an equal share, so that the remaining workgroups end with the others and not
+  // after them.  When that leaves them nothing, they are not launched.
+  const int aligned = (int)(workgroups / tiles);
+  long long left = workgroups - tiles * aligned;
+  int chunk = 0, rest = 0;
+  if (left > 0) {
+    chunk = (int)((tiles * (prob.total_slabs + 6LL) + workgroups - 1) / workgroups);
+    rest = prob.total_slabs - aligned * chunk;
+    if (rest <= 0) left = 0;
+  }
+  if (left == 0) {
+    chunk = (prob.total_slabs + aligned - 1) / aligned;
+    rest = 0;
+  }
+  const int launched = (int)(tiles * aligned + left);
   if (plan_workgroups) {
-    *plan_workgroups = workgroups;
+    *plan_workgroups = launched;
     *done = true;
     return MNV_OK;
   }
-  hipLaunchKernelGGL((mnv_gemm_kernel<T, P, 1, true, PF>), dim3(workgroups), dim3(T::NT), lds_bytes, s,
-                     prob, tiles_m, tiles_n, 0, reinterpret_cast<float*>(workspace), 0, 1);
+  hipLaunchKernelGGL((mnv_gemm_kernel<T, P, 1, true, PF>), dim3(launched), dim3(T::NT), lds_bytes, s,
+                     prob, tiles_m, tiles_n, chunk, reinterpret_cast<float*>(workspace), aligned, 1);
   int rc = MNV_LAUNCH_STATUS();
   if (rc) return rc;
-  // segments per tile: workgroups / tiles, one more where a share straddles
-  const long long per_tile = workgroups / tiles + 1;
+  // partial tiles per tile: the aligned ranges, and the remaining workgroups that met the tile
+  const long long per_tile = aligned + (left ? left / tiles + 2 : 0);
   const float* part = reinterpret_cast<const float*>(workspace);
   const dim3 block(256);
   if (per_tile >= 64)
     hipLaunchKernelGGL((mnv_gemm_streamk_reduce_kernel<T, P, 16>),
                        dim3(T::BM * T::BNU / 64, (unsigned)tiles), block, 0, s, prob, part, tiles_m,
-                       tiles_n, workgroups);
+                       tiles_n, launched, aligned, rest);
   else if (per_tile >= 32)
     hipLaunchKernelGGL((mnv_gemm_streamk_reduce_kernel<T, P, 4>),
                        dim3(T::BM * T::BNU / 256, (unsigned)tiles), block, 0, s, prob, part, tiles_m,
-                       tiles_n, workgroups);
+                       tiles_n, launched, aligned, rest);
   else
     hipLaunchKernelGGL((mnv_gemm_streamk_reduce_kernel<T, P, 1>),
                        dim3(T::BM * T::BNU / 1024, (unsigned)tiles), block, 0, s, prob, part, tiles_m,
-                       tiles_n, workgroups);
+                       tiles_n, launched, aligned, rest);
   *done = true;
   return MNV_LAUNCH_STATUS();
 }

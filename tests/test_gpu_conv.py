@@ -295,31 +295,38 @@ def _filter_plan(gpu, p, nbytes):
     return tile.value, ranges.value, wgs.value
 
 
-# Filter gradients whose launch is dealt to the chip in equal shares of tiles x k-slabs: few
-# output tiles, a long reduction.  One case per way of fetching the gathered operand.
+# Filter gradients whose launch is dealt to the chip in equal amounts of k-slabs per workgroup
+# (few output tiles, a long reduction): every tile is cut into the same aligned k ranges, and
+# what those leave goes to the workgroups that remain, in shares that cross tile boundaries.
+# One case per way of fetching the gathered operand with remaining workgroups (True), and
+# three whose tiles divide the workgroups' number or whose shares are too short to leave a
+# rest (False): every tile is then cut evenly.
 STREAMK = [
-    ("one tap per tile", 84, 128, 128, 13, 13, 1, 1, 1, 1, 3, 3),
-    ("two taps per tile", 40, 96, 128, 13, 13, 2, 2, 1, 1, 5, 5),
-    ("a table row per row group", 76, 48, 128, 13, 13, 2, 2, 1, 1, 5, 5),
-    ("no padding", 150, 22, 128, 17, 17, 0, 0, 1, 1, 5, 5),
-    ("channels not in sixteens", 150, 24, 128, 13, 13, 2, 2, 1, 1, 5, 5),
-    ("96-column tile", 96, 128, 96, 13, 13, 1, 1, 1, 1, 3, 3),
-    ("strided, ragged tile edges", 60, 120, 200, 23, 21, 1, 2, 2, 2, 3, 5),
+    ("one tap per tile", True, 4, 256, 1408, 13, 13, 1, 1, 1, 1, 3, 3),
+    ("two taps per tile", True, 3, 96, 1792, 13, 13, 2, 2, 1, 1, 5, 5),
+    ("a table row per row group", True, 7, 48, 1408, 13, 13, 2, 2, 1, 1, 5, 5),
+    ("no padding", True, 17, 22, 1408, 17, 17, 0, 0, 1, 1, 5, 5),
+    ("channels not in sixteens", True, 7, 24, 2816, 13, 13, 2, 2, 1, 1, 5, 5),
+    ("96-column tile", True, 32, 1088, 192, 7, 7, 1, 1, 1, 1, 3, 3),
+    ("strided, ragged tile edges", True, 5, 120, 1608, 23, 21, 1, 2, 2, 2, 3, 5),
+    ("one tap per tile, even cuts", False, 84, 128, 128, 13, 13, 1, 1, 1, 1, 3, 3),
+    ("no padding, even cuts", False, 150, 22, 128, 17, 17, 0, 0, 1, 1, 5, 5),
+    ("96-column tile, even cuts", False, 96, 128, 96, 13, 13, 1, 1, 1, 1, 3, 3),
 ]
 
 
 @pytest.mark.parametrize("case", STREAMK, ids=lambda c: c[0])
 def test_conv_bwd_filter_in_equal_shares_against_oracle(gpu, ora, case):
-    p = case[1:]
+    remaining, p = case[1], case[2:]
     N, C, K, H, W, ph, pw, sv, sh, R, S = p
     cv = Conv(gpu, *p)
     nbytes = gpu.L.mnv_conv_bwd_filter_workspace_bytes(*p)
     tile, ranges, wgs = _filter_plan(gpu, p, nbytes)
-    say("filter gradient,", case[0], "tile", tile, "workgroups", wgs)
-    assert tile == 128 and ranges == 1 and wgs >= 256, "the case is meant to take the stream-k plan"
-    # the shares cross tile boundaries: more shares than tiles, and not a multiple
     tiles = ((C * R * S + 127) // 128) * ((K + (95 if K in (96, 192) else 127)) // (96 if K in (96, 192) else 128))
-    assert tiles < wgs and wgs % tiles != 0
+    say("filter gradient,", case[0], "tile", tile, "workgroups", wgs, "tiles", tiles)
+    assert tile == 128 and ranges == 1 and wgs >= 256, "the case is meant to take the stream-k plan"
+    # workgroups = tiles x aligned ranges + the remaining ones (fewer than the tiles)
+    assert tiles < wgs and (wgs % tiles != 0) == remaining
     x, dy = _rand(N * C * H * W, 61), _rand(N * K * cv.Ho * cv.Wo, 62)
     got = cv.bwd_filter(dy, x)
     assert normwise(got, ora.conv_bwd_filter(dy, x, *p)) <= TOL
