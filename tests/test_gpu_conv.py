@@ -302,7 +302,7 @@ def _filter_plan(gpu, p, nbytes):
 # three whose tiles divide the workgroups' number or whose shares are too short to leave a
 # rest (False): every tile is then cut evenly.
 STREAMK = [
-    ("one tap per tile", True, 4, 256, 1408, 13, 13, 1, 1, 1, 1, 3, 3),
+    ("one tap per tile", True, 5, 256, 1408, 13, 13, 1, 1, 1, 1, 3, 3),
     ("two taps per tile", True, 3, 96, 1792, 13, 13, 2, 2, 1, 1, 5, 5),
     ("a table row per row group", True, 7, 48, 1408, 13, 13, 2, 2, 1, 1, 5, 5),
     ("no padding", True, 17, 22, 1408, 17, 17, 0, 0, 1, 1, 5, 5),
