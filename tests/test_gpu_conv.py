@@ -299,7 +299,7 @@ def _filter_plan(gpu, p, nbytes):
 # (few output tiles, a long reduction): every tile is cut into the same aligned k ranges, and
 # what those leave goes to the workgroups that remain, in shares that cross tile boundaries.
 # One case per way of fetching the gathered operand with remaining workgroups (True), and
-# three whose tiles divide the workgroups' number or whose shares are too short to leave a
+# four whose tiles divide the workgroups' number or whose shares are too short to leave a
 # rest (False): every tile is then cut evenly.
 STREAMK = [
     ("one tap per tile", True, 5, 256, 1408, 13, 13, 1, 1, 1, 1, 3, 3),
@@ -310,6 +310,7 @@ STREAMK = [
     ("96-column tile", True, 32, 1088, 192, 7, 7, 1, 1, 1, 1, 3, 3),
     ("strided, ragged tile edges", True, 5, 120, 1608, 23, 21, 1, 2, 2, 2, 3, 5),
     ("one tap per tile, even cuts", False, 84, 128, 128, 13, 13, 1, 1, 1, 1, 3, 3),
+    ("two taps per tile, even cuts", False, 40, 96, 128, 13, 13, 2, 2, 1, 1, 5, 5),
     ("no padding, even cuts", False, 150, 22, 128, 17, 17, 0, 0, 1, 1, 5, 5),
     ("96-column tile, even cuts", False, 96, 128, 96, 13, 13, 1, 1, 1, 1, 3, 3),
 ]
