@@ -145,6 +145,42 @@ def test_conv_all_passes_against_oracle(gpu, ora, p):
         assert normwise(cv.bwd_bias(dy, ws), ref) <= TOL
 
 
+def _random_geometries(count, seed):
+    """Seeded geometries that mix what the launch plans branch on: channel counts below, at and
+    off multiples of 16 / 96 / 128, unit and larger strides, padding up to the filter's reach,
+    planes whose rows are not multiples of four."""
+    rng = np.random.default_rng(seed)
+    menu = [1, 2, 3, 5, 8, 16, 17, 24, 32, 33, 48, 64, 96, 100, 128, 130, 192]
+    out = []
+    while len(out) < count:
+        N = int(rng.integers(1, 7))
+        C, K = int(rng.choice(menu)), int(rng.choice(menu))
+        H, W = int(rng.integers(4, 23)), int(rng.integers(4, 23))
+        R, S = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        ph, pw = int(rng.integers(0, R)), int(rng.integers(0, S))
+        sv, sh = int(rng.choice([1, 1, 2, 3])), int(rng.choice([1, 1, 2, 3]))
+        if H + 2 * ph < R or W + 2 * pw < S:
+            continue
+        Ho, Wo = (H + 2 * ph - R) // sv + 1, (W + 2 * pw - S) // sh + 1
+        if N * C * K * Ho * Wo * R * S > 150e6:
+            continue
+        out.append((N, C, K, H, W, ph, pw, sv, sh, R, S))
+    return out
+
+
+@pytest.mark.parametrize("p", _random_geometries(96, 2024), ids=lambda p: "x".join(map(str, p)))
+def test_conv_random_geometries_against_oracle(gpu, ora, p):
+    N, C, K, H, W, ph, pw, sv, sh, R, S = p
+    cv = Conv(gpu, *p)
+    x, w, b = _rand(N * C * H * W, 50), _rand(K * C * R * S, 51), _rand(K, 52)
+    dy = _rand(N * K * cv.Ho * cv.Wo, 53)
+    say("conv, random geometry", p)
+    assert normwise(cv.fwd(x, w, b), ora.conv_fwd(x, w, b, *p)) <= TOL
+    assert normwise(cv.bwd_data(dy, w), ora.conv_bwd_data(dy, w, *p)) <= TOL
+    assert normwise(cv.bwd_filter(dy, x), ora.conv_bwd_filter(dy, x, *p)) <= TOL
+    assert normwise(cv.bwd_bias(dy), ora.conv_bwd_bias(dy, N, K, cv.Ho, cv.Wo)) <= TOL
+
+
 def test_conv_with_a_cut_tail_against_oracle(gpu, ora):
     """Launches of a few more large tiles than a multiple of the 256 CUs cut the tiles past
     that multiple into k ranges (partial tiles in the workspace, added by a second kernel):
