@@ -47,6 +47,42 @@ def test_sgemm_against_oracle(gpu, ora, m, n, k, workspace):
     assert normwise(got.reshape(n, m).T, A @ B) <= TOL
 
 
+def _random_shapes(count, seed):
+    """Seeded extents around what the plans branch on: tile edges (63 / 64 / 65, 127 / 128 / 129),
+    multiples of four and not, a k of one slab and of many."""
+    rng = np.random.default_rng(seed)
+    edge = [1, 2, 3, 4, 15, 16, 17, 63, 64, 65, 96, 127, 128, 129, 191, 192, 255, 256, 257]
+    out = []
+    while len(out) < count:
+        pick = lambda hi: int(rng.choice(edge)) if rng.random() < 0.5 else int(rng.integers(1, hi))
+        m, n, k = pick(700), pick(700), pick(3000)
+        if m * n * k <= 80e6:
+            out.append((m, n, k))
+    return out
+
+
+@pytest.mark.parametrize("m,n,k", _random_shapes(60, 7))
+def test_sgemm_random_shapes_against_fp64(gpu, m, n, k):
+    """mnv_sgemm_nn with and without a workspace, and the same product with either operand
+    given transposed (mnv_sgemm_tn / mnv_sgemm_nt), against the fp64 product."""
+    a, b = _rand(m * k, 60), _rand(k * n, 61)
+    A = a.reshape(k, m).T.astype(np.float64)   # column-major m x k
+    B = b.reshape(n, k).T.astype(np.float64)   # column-major k x n
+    want = (A @ B).T.reshape(-1)               # column-major m x n, flattened
+    say("sgemm, random shape", m, n, k)
+    for workspace in (True, False):
+        assert normwise(_gemm(gpu, a, b, m, n, k, workspace), want) <= TOL
+    ws_bytes = gpu.L.mnv_sgemm_nn_workspace_bytes(m, n, k)
+    ws = gpu.empty(ws_bytes // 4 + 1)
+    dc = gpu.empty(m * n)
+    at = gpu.up(np.ascontiguousarray(a.reshape(k, m).T).reshape(-1))   # A^T: column-major k x m
+    gpu.call("mnv_sgemm_tn", at.p, gpu.up(b).p, None, dc.p, m, n, k, ws.p, ctypes.c_size_t(ws_bytes))
+    assert normwise(gpu.down(dc), want) <= TOL
+    bt = gpu.up(np.ascontiguousarray(b.reshape(n, k).T).reshape(-1))   # B^T: column-major n x k
+    gpu.call("mnv_sgemm_nt", gpu.up(a).p, bt.p, dc.p, m, n, k, ws.p, ctypes.c_size_t(ws_bytes))
+    assert normwise(gpu.down(dc), want) <= TOL
+
+
 def _plan(gpu, m, n, k, ws_bytes):
     tile, ranges, groups = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     assert gpu.L.mnv_sgemm_nn_plan(m, n, k, ctypes.c_size_t(ws_bytes), ctypes.byref(tile),
