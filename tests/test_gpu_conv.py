@@ -444,6 +444,33 @@ def test_pooling_against_oracle(gpu, ora, p, ties):
     assert normwise(gpu.down(dbd), ora.pool_bwd(ora.POOL_AVG, dy, avg, x, *p)) <= TOL
 
 
+def _random_pools(count, seed):
+    """Seeded pooling geometries: windows of 1..4 with strides up to the window, padding below
+    the window, planes from one row to 30, a few and many planes."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        N, C = int(rng.integers(1, 5)), int(rng.choice([1, 2, 3, 16, 33, 96]))
+        H, W = int(rng.integers(1, 31)), int(rng.integers(1, 31))
+        kh, kw = int(rng.integers(1, 5)), int(rng.integers(1, 5))
+        if rng.random() < 0.5:   # the square windows the fast kernels take
+            kw = kh = int(rng.choice([2, 3]))
+        sv, sh = int(rng.integers(1, kh + 1)), int(rng.integers(1, kw + 1))
+        if rng.random() < 0.5:
+            sv = sh = 2
+        ph, pw = int(rng.integers(0, kh)), int(rng.integers(0, kw))
+        if H + 2 * ph < kh or W + 2 * pw < kw:
+            continue
+        out.append((N, C, H, W, sv, sh, kh, kw, ph, pw))
+    return out
+
+
+@pytest.mark.parametrize("p", _random_pools(48, 11), ids=lambda p: "x".join(map(str, p)))
+def test_pooling_random_geometries_against_oracle(gpu, ora, p):
+    test_pooling_against_oracle(gpu, ora, p, True)
+    test_pooling_against_oracle(gpu, ora, p, False)
+
+
 def test_pooling_batch_256_properties(gpu):
     p = (256, 96, 55, 55, 2, 2, 3, 3, 0, 0)
     N, C, H, W = p[:4]
