@@ -271,8 +271,9 @@ int mnv_conv_bwd_filter(const float* bottom, const float* top_diff, float* filte
  * current device (no reference counterpart: cuDNN chooses its algorithm out of sight,
  * cuda_perform.cu:293-318): rows of the output tile (64 or 128); the k ranges the reduction
  * over images and positions is cut into, each with a partial result in the workspace (1: none);
- * and, when the launch is dealt to the chip in equal shares of tiles x k-slabs instead
- * ("stream-k": k_ranges is then 1), the number of workgroups, else 0.  For a batch that runs
+ * and, when the launch instead has as many workgroups as the chip holds at once, each with the
+ * same number of k-slabs ("stream-k": aligned k ranges of every tile, the rest in shares;
+ * k_ranges is then 1), the number of workgroups, else 0.  For a batch that runs
  * as several launches, the plan of the first.  Launches nothing. */
 int mnv_conv_bwd_filter_plan(int num_images, int bottom_num_channels, int top_num_channels,
                              int bottom_height, int bottom_width, int pad_height, int pad_width,

@@ -660,13 +660,15 @@ int launch_tile(int tile, const P& p, int splits, void* ws, hipStream_t s, size_
 }
 const int kTileM[4] = {64, 128, 128, 128}, kTileN[4] = {64, 128, 96, 32};
 
-// The filter gradient: few output tiles and a very long k.  On the large tiles it is dealt
-// to the chip in equal shares of tiles x k-slabs (stream-k) when the workspace holds the
-// shares' partial tiles; otherwise, and on the small tiles, in `splits` whole k ranges.
+// The filter gradient: few output tiles and a very long k.  On the large tiles it runs as
+// one launch of as many workgroups as the chip holds, every one with the same number of
+// k-slabs (stream-k: aligned k ranges of every tile, the rest in shares; see mnv_gemm_kernel),
+// when the workspace holds the partial tiles; otherwise, and on the small tiles, in `splits`
+// whole k ranges.
 // Slabs the filter gradient's loads run ahead (see mnv_gemm_kernel): two, which costs a
-// fourth workgroup per CU; measured on the four padded convolutions of the AlexNet shape, four
-// resident workgroups per CU with equal shares ran 16% slower than three (1.18 against
-// 1.03 ms per launch): the chip is then waiting for the L2 and fabric, not for the matrix pipe.
+// fourth workgroup per CU.  Measured on the four padded convolutions of the AlexNet shape
+// with the aligned plan: one slab ahead and four workgroups per CU 3.88 ms over the four
+// launches, two ahead and three per CU 3.84 ms.
 #ifndef MNV_SK_PF
 #define MNV_SK_PF 2
 #endif
