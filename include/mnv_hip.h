@@ -153,7 +153,7 @@ int mnv_maxindex_row(const float* in, float* out, int m, int n, mnv_stream_t str
  * range.
  * mnv_sgemm_nn_plan reports how a product of these extents is launched with a workspace of
  * that size (no counterpart in the reference, where the plan is cuBLAS's own): tile_rows is
- * 128 or 64 (square tiles), k_ranges the number of partial results reduced by a second
+ * 128 or 64 (square tiles) or 256 (256 x 128), k_ranges the number of partial results reduced by a second
  * kernel (1: none), groups 4 when four wavefront groups of a workgroup share a tile and add
  * their quarters of the k range through LDS.  The plan depends on (m, n, k, workspace_bytes)
  * only, never on the operands. ---- */

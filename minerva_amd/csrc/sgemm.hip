@@ -145,6 +145,9 @@ SgemmNN<VEC, TA, TB> make_sgemm(const float* a, const float* b, float* c, int m,
 
 typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 typedef MnvGemmTile<64, 64, 16, 2, 2> TileSmall;
+// Eight wavefronts of 64 x 64 (512 threads, two workgroups per CU): a quarter fewer bytes
+// fetched and staged per multiply than TileBig, the same reads from LDS.
+typedef MnvGemmTile<256, 128, 16, 4, 2> TileTall;
 #define MNV_SGEMM_MAX_SPLITS 16
 
 // Tile shape and number of k ranges for an (m,n,k) product given `ws_floats` floats of
@@ -156,6 +159,7 @@ struct SgemmPlan {
   bool small;
   int splits;
   int groups = 1;  // 4: workgroups of four wavefront groups that share a tile's k range
+  bool tall = false;  // 256 x 128 tiles (no k ranges, one wavefront group)
 };
 
 SgemmPlan plan_sgemm(int m, int n, int k, size_t ws_floats) {
@@ -217,6 +221,15 @@ SgemmPlan plan_sgemm(int m, int n, int k, size_t ws_floats) {
       }
     }
   }
+  // Large products whose 256 x 128 tiles fill the chip's two-per-CU slots in whole rounds
+  // (at least 95% of the multiplies of all rounds are the product's own): measured back to
+  // back, 4096^3 0.956 -> 0.940 ms, 8192 x 4096 x 8192 3.85 -> 3.74 ms.  Every element is summed
+  // over k in the same order as on the 128 x 128 tile: the same bits.
+  if (!best.small && best.splits == 1 && best.groups == 1 && m >= 256 && slabs >= 32) {
+    const long long tiles = (long long)((m + 255) / 256) * ((n + 127) / 128);
+    const long long slots = 2LL * mnv_cu_count(), rounds = (tiles + slots - 1) / slots;
+    if ((double)m * n >= 0.95 * (double)(rounds * slots) * 256.0 * 128.0) best.tall = true;
+  }
   return best;
 }
 
@@ -224,6 +237,7 @@ SgemmPlan plan_sgemm(int m, int n, int k, size_t ws_floats) {
 template <class P>
 int launch_plan(const SgemmPlan& plan, const P& p, void* workspace, size_t workspace_bytes,
                 hipStream_t s) {
+  if (plan.tall) return mnv_gemm_launch<TileTall>(p, 1, workspace, s);
   if (plan.groups == 4)
     return plan.small ? mnv_gemm_launch<TileSmall, 4>(p, plan.splits, workspace, s)
                       : mnv_gemm_launch<TileBig, 4>(p, plan.splits, workspace, s);
@@ -234,7 +248,7 @@ int launch_plan(const SgemmPlan& plan, const P& p, void* workspace, size_t works
 
 // Bytes a product without k ranges wants for the partial tiles of its cut tail.
 size_t sgemm_tail_bytes(const SgemmPlan& plan, int m, int n, int k) {
-  if (plan.splits != 1 || plan.groups != 1) return 0;
+  if (plan.splits != 1 || plan.groups != 1 || plan.tall) return 0;
   const int bm = plan.small ? 64 : 128;
   const long long tiles = (long long)((m + bm - 1) / bm) * ((n + bm - 1) / bm);
   const MnvTailPlan t = mnv_tail_plan(tiles, (k + 15) / 16, (size_t)bm * bm, (size_t)-1 / sizeof(float));
@@ -329,7 +343,7 @@ int mnv_sgemm_nn_plan(int m, int n, int k, size_t workspace_bytes, int* tile_row
                       int* groups) {
   if (m <= 0 || n <= 0 || k <= 0 || !tile_rows || !k_ranges || !groups) return MNV_ERR_INVALID;
   const SgemmPlan plan = plan_sgemm(m, n, k, workspace_bytes / sizeof(float));
-  *tile_rows = plan.small ? 64 : 128;
+  *tile_rows = plan.tall ? 256 : plan.small ? 64 : 128;
   const int slabs = (k + 15) / 16, per = (slabs + plan.splits - 1) / plan.splits;
   *k_ranges = (slabs + per - 1) / per;  // as the launch rounds it: ranges of equal length
   *groups = plan.groups;

@@ -145,6 +145,32 @@ def test_sgemm_with_a_cut_tail(gpu, m, n, k):
     assert_bits_equal(_gemm(gpu, a, b, m, n, k, True).reshape(n, m), got, "second call")
 
 
+@pytest.mark.parametrize("m,n,k", [(4092, 4092, 520), (4095, 4093, 515), (8192, 2048, 512)])
+def test_sgemm_on_256_row_tiles(gpu, m, n, k):
+    """Large products whose 256 x 128 tiles fill the chip in whole rounds take that tile (eight
+    wavefronts per workgroup): ragged edges in both extents, vector and scalar fetches, against
+    the fp64 product element by element, and the same bits with either operand transposed."""
+    ws_bytes = gpu.L.mnv_sgemm_nn_workspace_bytes(m, n, k)
+    assert _plan(gpu, m, n, k, ws_bytes) == (256, 1, 1), "the case is meant to take the 256-row tile"
+    a, b = _rand(m * k, 46), _rand(k * n, 47)
+    say("sgemm, 256 x 128 tiles", m, n, k)
+    got = _gemm(gpu, a, b, m, n, k)
+    A = a.reshape(k, m).astype(np.float64)
+    B = b.reshape(n, k).astype(np.float64)
+    want = B @ A
+    err = np.abs(got.reshape(n, m) - want)
+    worst = np.unravel_index(int(np.argmax(err)), err.shape)
+    assert err[worst] <= TOL * float(np.max(np.abs(want))), "largest error at column %d, row %d" % worst
+    ws = gpu.empty(ws_bytes // 4 + 1)
+    dc = gpu.empty(m * n)
+    at = gpu.up(np.ascontiguousarray(a.reshape(k, m).T).reshape(-1))
+    gpu.call("mnv_sgemm_tn", at.p, gpu.up(b).p, None, dc.p, m, n, k, ws.p, ctypes.c_size_t(ws_bytes))
+    assert_bits_equal(gpu.down(dc), got, "A given transposed")
+    bt = gpu.up(np.ascontiguousarray(b.reshape(n, k).T).reshape(-1))
+    gpu.call("mnv_sgemm_nt", gpu.up(a).p, bt.p, dc.p, m, n, k, ws.p, ctypes.c_size_t(ws_bytes))
+    assert_bits_equal(gpu.down(dc), got, "B given transposed")
+
+
 def test_sgemm_reference_unit_test_shape(gpu):
     # tests/unittest_sgemm.cpp:7-28: {3,2} x {2,5} against the triple loop
     a = np.arange(6, dtype=np.float32)
