@@ -649,8 +649,24 @@ typedef MnvGemmTile<128, 128, 16, 4, 1, 0, 96> Tile96;  // four wavefronts of 32
 typedef MnvGemmTile<128, 64, 16, 4, 1, 0, 32> TileThin;
 
 // tile 0: 64x64 output tiles, tile 1: 128x128, tile 2: 128x96, tile 3: 128x32
+// Eight wavefronts of 64 x 64 (512 threads, two workgroups per CU): a quarter fewer bytes
+// fetched and staged per multiply than TileBig, and every element summed in the same order.
+// For the (tap, channel) forward and data-gradient policies, when the 256 x 128 tiles fill
+// the chip's two-per-CU slots in whole rounds to 97% (conv3 / conv4 forward and conv4 / conv5
+// data gradient of the AlexNet shape at batch 256: 507 tiles on 512 slots, 2-3% faster; conv2
+// forward, 1458 tiles in three rounds of 512 at 95%, is 3% SLOWER than on 128 x 128 tiles with
+// their cut tail).
+typedef MnvGemmTile<256, 128, 16, 4, 2> TileTall;
 template <class P>
 int launch_tile(int tile, const P& p, int splits, void* ws, hipStream_t s, size_t tail_bytes = 0) {
+  if constexpr (P::A_KFAST == false && P::B_NOFF == 1) {
+    if (tile == 1 && splits == 1) {
+      const long long tiles = (long long)((p.M + 255) / 256) * ((p.N + 127) / 128);
+      const long long slots = 2LL * mnv_cu_count(), rounds = (tiles + slots - 1) / slots;
+      if ((double)p.M * p.N >= 0.97 * (double)(rounds * slots) * 256.0 * 128.0)
+        return mnv_gemm_launch<TileTall>(p, 1, ws, s);
+    }
+  }
   switch (tile) {
     case 0: return mnv_gemm_launch<TileSmall>(p, splits, ws, s);
     case 2: return mnv_gemm_launch<Tile96>(p, splits, ws, s, tail_bytes);

@@ -56,8 +56,10 @@ struct MnvGemmTile {
   }
   // Wavefronts per SIMD the register allocation must allow: four 4-wavefront workgroups
   // per CU make 1024 resident tiles, which lets tile counts just under a multiple of
-  // 1024 finish in whole rounds.
-  static constexpr int MIN_WAVES = (NT == 256 && BM * BN <= 128 * 128 && BK <= 16) ? 4 : 1;
+  // 1024 finish in whole rounds; two 8-wavefront workgroups are the same four wavefronts
+  // per SIMD.
+  static constexpr int MIN_WAVES = (NT == 256 && BM * BN <= 128 * 128 && BK <= 16) ? 4
+                                   : (NT == 512 && BM * BN <= 256 * 128 && BK <= 16) ? 4 : 1;
   static_assert(WM % 32 == 0 && WN % 32 == 0 && BNU <= BN, "wave tile must be a multiple of 32x32");
   static_assert((BK == 8 || BK == 16 || BK == 32) && (BM * BK) % (4 * NT) == 0 &&
                     (BN * BK) % (4 * NT) == 0,

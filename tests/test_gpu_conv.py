@@ -181,6 +181,25 @@ def test_conv_random_geometries_against_oracle(gpu, ora, p):
     assert normwise(cv.bwd_bias(dy), ora.conv_bwd_bias(dy, N, K, cv.Ho, cv.Wo)) <= TOL
 
 
+@pytest.mark.parametrize("p", [(8, 16, 128, 127, 127, 1, 1, 1, 1, 3, 3),    # forward: 505 tiles of 256 x 128
+                               (8, 128, 16, 127, 127, 1, 1, 1, 1, 3, 3)],   # the same for the data gradient
+                         ids=["forward", "data gradient"])
+def test_conv_on_256_row_tiles_against_oracle(gpu, ora, p):
+    """Outputs of about 2^24 elements whose 256 x 128 tiles fill two workgroup slots per CU:
+    the (tap, channel) forward / data-gradient kernels then run eight wavefronts per
+    workgroup.  Ragged last tile (8 x 127 x 127 positions)."""
+    N, C, K, H, W, ph, pw, sv, sh, R, S = p
+    cv = Conv(gpu, *p)
+    x, w, b = _rand(N * C * H * W, 70), _rand(K * C * R * S, 71), _rand(K, 72)
+    dy = _rand(N * K * cv.Ho * cv.Wo, 73)
+    say("conv on 256-row tiles", p)
+    assert normwise(cv.fwd(x, w, b), ora.conv_fwd(x, w, b, *p)) <= TOL
+    assert normwise(cv.bwd_data(dy, w), ora.conv_bwd_data(dy, w, *p)) <= TOL
+    # the same geometry without a workspace runs the generic kernels on 128 x 128 tiles
+    assert normwise(cv.fwd(x, w, b, False), cv.fwd(x, w, b).astype(np.float64)) <= 1e-5
+    assert normwise(cv.bwd_data(dy, w, False), cv.bwd_data(dy, w).astype(np.float64)) <= 1e-5
+
+
 def test_conv_with_a_cut_tail_against_oracle(gpu, ora):
     """Launches of a few more large tiles than a multiple of the 256 CUs cut the tiles past
     that multiple into k ranges (partial tiles in the workspace, added by a second kernel):
