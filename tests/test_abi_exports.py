@@ -68,11 +68,13 @@ def _plan(m, n, k, workspace=True):
 
 def test_sgemm_plans_of_the_benchmark_shapes():
     """The launch plan is host arithmetic on the extents alone.  Square and short-k products
-    run one tile per workgroup without k ranges; the skinny inner products of the AlexNet
+    run one tile per workgroup without k ranges (the large square one on 256 x 128 tiles, which
+    fill the chip's two-per-CU slots exactly); the skinny inner products of the AlexNet
     shape run as workgroups of four wavefront groups; the workspace the query asks for is
     exactly what the plan's partial results need; without a workspace nothing is split in
     memory."""
-    assert _plan(4096, 4096, 4096)[:3] == (128, 1, 1)
+    assert _plan(4096, 4096, 4096)[:3] == (256, 1, 1)
+    assert _plan(4096, 4096, 256)[:3] == (128, 1, 1)
     assert _plan(4096, 9216, 256)[:3] == (128, 1, 1)
     assert _plan(4096, 256, 9216)[:3] == (128, 4, 4)
     assert _plan(4096, 256, 4096)[:3] == (64, 1, 4)
