@@ -393,6 +393,54 @@ def test_conv_bwd_filter_in_equal_shares_against_oracle(gpu, ora, case):
     assert normwise(cv.bwd_filter(dy, x, workspace=False), got.astype(np.float64)) <= 1e-5
 
 
+def _random_streamk_geometries(count, seed):
+    """Seeded mid-size geometries whose filter gradient takes the stream-k plan: hundreds of
+    k-slabs per tile, a few to a few hundred tiles, every way of fetching the gathered operand."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        N = int(rng.integers(24, 100))
+        C, K = int(rng.choice([48, 64, 96, 100, 128, 160, 256])), int(rng.choice([128, 192, 200, 256, 384]))
+        H, W = int(rng.integers(8, 21)), int(rng.integers(8, 21))
+        R = S = int(rng.choice([3, 5]))
+        ph = pw = int(rng.choice([0, R // 2]))
+        Ho, Wo = H + 2 * ph - R + 1, W + 2 * pw - S + 1
+        bn = 96 if K in (96, 192) else 128
+        tiles = ((C * R * S + 127) // 128) * ((K + bn - 1) // bn)
+        if tiles * N * ((Ho * Wo + 15) // 16) < 8 * 1024:   # eight slabs for each of at most 1024 workgroups
+            continue
+        out.append((N, C, K, H, W, ph, pw, 1, 1, R, S))
+    return out
+
+
+@pytest.mark.parametrize("p", _random_streamk_geometries(40, 99), ids=lambda p: "x".join(map(str, p)))
+def test_conv_bwd_filter_streamk_random_geometries_sampled_fp64(gpu, p):
+    """Beyond what the oracle reaches in seconds: 64 filter-gradient entries per geometry (the
+    corners of the index space first) against fp64 sums written from the definition."""
+    N, C, K, H, W, ph, pw, sv, sh, R, S = p
+    cv = Conv(gpu, *p)
+    tile, ranges, wgs = _filter_plan(gpu, p, gpu.L.mnv_conv_bwd_filter_workspace_bytes(*p))
+    say("filter gradient, random stream-k geometry", p, "tile", tile, "k ranges", ranges, "workgroups", wgs)
+    assert wgs > 0, "the geometry is meant to take the stream-k plan"
+    x, dy = _rand(N * C * H * W, 80), _rand(N * K * cv.Ho * cv.Wo, 81)
+    dw = cv.bwd_filter(dy, x)
+    X, DY, DW = x.reshape(N, C, H, W), dy.reshape(N, K, cv.Ho, cv.Wo), dw.reshape(K, C, R, S)
+    rng = np.random.default_rng(82)
+    picks = [(k, c, r, s_) for k in (0, K - 1) for c in (0, C - 1) for r in (0, R - 1) for s_ in (0, S - 1)]
+    while len(picks) < 64:
+        picks.append((int(rng.integers(K)), int(rng.integers(C)), int(rng.integers(R)), int(rng.integers(S))))
+    worst, top = 0.0, float(np.max(np.abs(dw)))
+    for (k, c, r, s_) in picks:
+        rf, sf = R - 1 - r, S - 1 - s_
+        i, j = np.arange(cv.Ho), np.arange(cv.Wo)
+        i = i[(i - ph + rf >= 0) & (i - ph + rf < H)]
+        j = j[(j - pw + sf >= 0) & (j - pw + sf < W)]
+        xs = X[:, c][:, i - ph + rf][:, :, j - pw + sf].astype(np.float64)
+        worst = max(worst, abs(float(DW[k, c, r, s_]) - float(np.sum(xs * DY[:, k][:, i][:, :, j]))))
+    assert worst <= TOL * top, "filter gradient entry off by %.3e of %.3e" % (worst, top)
+    assert_bits_equal(cv.bwd_filter(dy, x), dw, "second call")
+
+
 # ------------------------------------------------------------------- pooling
 
 @pytest.mark.parametrize("case", json.load(open(os.path.join(GOLD, "pooling_forward.json"))),
