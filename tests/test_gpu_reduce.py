@@ -189,6 +189,36 @@ def test_transpose_into_a_result_off_the_64_byte_grid(gpu, off):
     assert np.isnan(got[:off]).all() and np.isnan(got[off + m * n:]).all(), "wrote outside the result"
 
 
+def _random_extents(count, seed, hi_m, hi_n, limit):
+    """Seeded (m, n) pairs: half of the extents from the values the kernels branch on (vector
+    width, wavefront, workgroup and tile sizes and their neighbours), half anywhere below hi."""
+    rng = np.random.default_rng(seed)
+    edge = [1, 2, 3, 4, 5, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513,
+            1023, 1024, 1025, 2047, 2048, 2052, 4095, 4096, 4100]
+    out = []
+    while len(out) < count:
+        m = int(rng.choice(edge)) if rng.random() < 0.5 else int(rng.integers(1, hi_m))
+        n = int(rng.choice(edge)) if rng.random() < 0.5 else int(rng.integers(1, hi_n))
+        if m * n <= limit:
+            out.append((m, n))
+    return out
+
+
+@pytest.mark.parametrize("m,n", _random_extents(40, 5, 5000, 5000, 3_000_000))
+def test_reductions_random_extents(gpu, ora, m, n):
+    test_reductions(gpu, ora, m, n)
+
+
+@pytest.mark.parametrize("length,lines", _random_extents(40, 6, 9000, 600, 2_000_000))
+def test_softmax_instance_random_extents(gpu, ora, length, lines):
+    test_softmax_instance(gpu, ora, length, lines)
+
+
+@pytest.mark.parametrize("m,n", _random_extents(40, 7, 5000, 5000, 3_000_000))
+def test_transpose_random_extents(gpu, ora, m, n):
+    test_transpose_bit_exact(gpu, ora, m, n)
+
+
 def test_large_operand_paths_8192x8192(gpu):
     """Inputs of 256 MB and more take the variants that read past the caches: softmax,
     transpose and the broadcast add at the size of the bandwidth benchmark."""
