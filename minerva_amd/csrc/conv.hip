@@ -132,6 +132,26 @@ struct ConvFwd {
     if (relu) v = v > 0.f ? v : 0.f;
     top[((size_t)img * N + n) * g.HoWo + pos] = v;
   }
+  // four consecutive positions of one channel: one 16-byte store (4-byte aligned) unless the
+  // four straddle two images or the end of the batch
+  static constexpr bool C_STORE4 = true;
+  __device__ void c_store4(int m, int n, const float (&x)[4]) const {
+    int img = mnv_fastdiv(m, g.d_HoWo);
+    int pos = m - img * g.HoWo;
+    if (m + 3 < M && pos + 3 < g.HoWo) {
+      const float b = bias[n];
+      mnv_f4u v = {x[0] + b, x[1] + b, x[2] + b, x[3] + b};
+      if (relu) {
+        v.x = v.x > 0.f ? v.x : 0.f; v.y = v.y > 0.f ? v.y : 0.f;
+        v.z = v.z > 0.f ? v.z : 0.f; v.w = v.w > 0.f ? v.w : 0.f;
+      }
+      *reinterpret_cast<mnv_f4u*>(top + ((size_t)img * N + n) * g.HoWo + pos) = v;
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (m + q < M) c_store(m + q, n, x[q]);
+    }
+  }
 };
 
 // Forward without padding (ph == pw == 0, any channel count and stride).  Every tap of
@@ -223,6 +243,26 @@ struct ConvFwdNP {
     float v = x + bias[n];
     if (relu) v = v > 0.f ? v : 0.f;
     top[((size_t)img * N + n) * g.HoWo + pos] = v;
+  }
+  // four consecutive positions of one channel: one 16-byte store (4-byte aligned) unless the
+  // four straddle two images or the end of the batch
+  static constexpr bool C_STORE4 = true;
+  __device__ void c_store4(int m, int n, const float (&x)[4]) const {
+    int img = mnv_fastdiv(m, g.d_HoWo);
+    int pos = m - img * g.HoWo;
+    if (m + 3 < M && pos + 3 < g.HoWo) {
+      const float b = bias[n];
+      mnv_f4u v = {x[0] + b, x[1] + b, x[2] + b, x[3] + b};
+      if (relu) {
+        v.x = v.x > 0.f ? v.x : 0.f; v.y = v.y > 0.f ? v.y : 0.f;
+        v.z = v.z > 0.f ? v.z : 0.f; v.w = v.w > 0.f ? v.w : 0.f;
+      }
+      *reinterpret_cast<mnv_f4u*>(top + ((size_t)img * N + n) * g.HoWo + pos) = v;
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (m + q < M) c_store(m + q, n, x[q]);
+    }
   }
 };
 
@@ -331,6 +371,25 @@ struct ConvBwdData {
     const size_t at = ((size_t)img * N + n) * g.HW + pos;
     if (gate) x = gate[at] > 0.f ? x : 0.f;
     bottom_diff[at] = x;
+  }
+  static constexpr bool C_STORE4 = true;
+  __device__ void c_store4(int m, int n, const float (&x)[4]) const {
+    int img = mnv_fastdiv(m, g.d_HW);
+    int pos = m - img * g.HW;
+    if (m + 3 < M && pos + 3 < g.HW) {
+      const size_t at = ((size_t)img * N + n) * g.HW + pos;
+      mnv_f4u v = {x[0], x[1], x[2], x[3]};
+      if (gate) {
+        const mnv_f4u t = *reinterpret_cast<const mnv_f4u*>(gate + at);
+        v.x = t.x > 0.f ? v.x : 0.f; v.y = t.y > 0.f ? v.y : 0.f;
+        v.z = t.z > 0.f ? v.z : 0.f; v.w = t.w > 0.f ? v.w : 0.f;
+      }
+      *reinterpret_cast<mnv_f4u*>(bottom_diff + at) = v;
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (m + q < M) c_store(m + q, n, x[q]);
+    }
   }
 };
 

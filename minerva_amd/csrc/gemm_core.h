@@ -115,6 +115,15 @@ struct MnvFetchMap {
 //   cheaper to clear once they have arrived: static constexpr bool B_STASH_FIX = true;
 //   void b_stash_fix(int s, int kl, float (&v)[4]) const;   called on every vector of slab s of
 //        its period right before the vector is written to LDS
+//   optional, for an output whose m direction is contiguous in memory:
+//   static constexpr bool C_STORE4 = true;
+//   void c_store4(int m, int n, const float (&v)[4]) const;   the elements (m .. m + 3, n); m is a
+//        multiple of 4 below M, the elements from M on are not to be stored
+//        A launch without k ranges then passes every 32 x 32 block of accumulators through LDS
+//        (a lane holds 4 consecutive n of one m, the store wants 4 consecutive m of one n) and
+//        stores 16 bytes per lane, 512 contiguous bytes per column and instruction, instead of
+//        4 bytes per lane: a quarter of the store instructions.  Taken for products of at most
+//        MNV_STORE4_MAX_SLABS k-slabs.
 //   optional, for a store that combines the product with a value read from memory:
 //   static constexpr bool C_PRELOAD = true;
 //   bool c_preload_on() const;                   uniform: whether this launch reads
@@ -136,6 +145,15 @@ struct MnvBStashFix {
 };
 template <class P>
 struct MnvBStashFix<P, std::enable_if_t<P::B_STASH_FIX>> {
+  static constexpr bool value = true;
+};
+#define MNV_STORE4_MAX_SLABS 64
+template <class P, class = void>
+struct MnvCStore4 {
+  static constexpr bool value = false;
+};
+template <class P>
+struct MnvCStore4<P, std::enable_if_t<P::C_STORE4>> {
   static constexpr bool value = true;
 };
 template <class P, class = void>
@@ -545,6 +563,46 @@ __global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MI
   }
   const bool split = gridDim.z > 1;
   float* part = split ? partial + (size_t)blockIdx.z * prob.M * prob.N : nullptr;
+  // rows x columns of one pass through LDS: one 32 x 32 block of every wavefront
+  constexpr int SROWS = T::WGM * 32, SCOLS = T::WGN * 32, SPITCH = SROWS + 4;
+  if constexpr (MnvCStore4<P>::value && G == 1 && SCOLS * SPITCH <= GROUP_FLOATS &&
+                (SCOLS * (SROWS / 4)) % T::NT == 0) {
+    // Worth it where the stores are a large part of a tile's time, i.e. for a short k
+    // (measured: conv1 forward of the AlexNet shape, 23 slabs, 0.526 -> 0.482 ms; 4096 x 9216
+    // x 256, 16 slabs, 0.177 -> 0.161 ms; with 144-216 slabs the two extra barriers per block
+    // cost the data gradients 2% and gain the forward kernels nothing)
+    bool direct = !split && prob.total_slabs <= MNV_STORE4_MAX_SLABS;
+    if constexpr (MnvCPreload<P>::value) direct = direct && !prob.c_preload_on();
+    if (direct) {
+      // every wavefront is past the last slab's barrier: the tile buffers are free
+      float* stage = mnv_gemm_lds;
+      const int srow = (wave % T::WGM) * 32 + lm, scol = (wave / T::WGM) * 32 + lk * 4;
+      constexpr int QPC = SROWS / 4;                    // 16-byte groups per column
+      constexpr int PER = SCOLS * QPC / T::NT;          // groups per thread and pass
+#pragma unroll
+      for (int i = 0; i < T::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < T::TN; ++j) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            stage[(scol + (r & 3) + 8 * (r >> 2)) * SPITCH + srow] = acc[i][j][r];
+          __syncthreads();
+#pragma unroll
+          for (int q = 0; q < PER; ++q) {
+            const int idx = q * T::NT + tid, col = idx / QPC, row = (idx - col * QPC) * 4;
+            const mnv_f4 v = *reinterpret_cast<const mnv_f4*>(stage + col * SPITCH + row);
+            const int m = m0 + (row / 32) * T::WM + i * 32 + row % 32;
+            const int n = n0 + (col / 32) * T::WN + j * 32 + col % 32;
+            if (m < prob.M && n < prob.N) {
+              const float x[4] = {v.x, v.y, v.z, v.w};
+              prob.c_store4(m, n, x);
+            }
+          }
+          __syncthreads();
+        }
+      return;
+    }
+  }
   if constexpr (MnvCPreload<P>::value) {
     if (!split && prob.c_preload_on()) {
 #pragma unroll

@@ -54,6 +54,8 @@ __device__ __forceinline__ int mnv_fastdiv(int n, const MnvFastDiv& f) {
 }
 
 typedef float mnv_f4 __attribute__((ext_vector_type(4)));
+// the same four floats where only their 4-byte alignment is known
+typedef float mnv_f4u __attribute__((ext_vector_type(4), aligned(4)));
 #ifdef __HIPCC__
 // A 16-byte load of data that is read once.  NT: non-temporal, for tensors of 256 MB and
 // more, which cannot stay in the last-level cache anyway (measured with operands cycled so

@@ -112,6 +112,19 @@ struct SgemmNN {
     }
     C[at] = x;
   }
+  // four consecutive rows of one column: one 16-byte store for the plain product, element by
+  // element when an epilogue is on
+  static constexpr bool C_STORE4 = true;
+  __device__ void c_store4(int m, int n, const float (&x)[4]) const {
+    if (m + 3 < M && !accumulate && !bias && !relu && !gate && !sgd_w) {
+      const mnv_f4u v = {x[0], x[1], x[2], x[3]};
+      *reinterpret_cast<mnv_f4u*>(C + (size_t)n * ldc + m) = v;
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (m + q < M) c_store(m + q, n, x[q]);
+    }
+  }
   // the update read ahead of the block's stores (only bias / relu / gate / accumulate off)
   static constexpr bool C_PRELOAD = TB;
   __device__ bool c_preload_on() const { return sgd_w != nullptr; }
