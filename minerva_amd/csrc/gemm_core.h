@@ -228,6 +228,20 @@ __device__ __forceinline__ int mnv_tile_remap(int t, int total) {
 // (the kernel then fits 128 registers: four workgroups per CU).  2: a second set of staging
 // registers lets the loads of slab i + 2 start at the head of slab i, so that a trip to
 // memory may take two slab times instead of one; 24 more registers, three workgroups per CU.
+// Partial tiles (the k ranges of a cut tail, the ranges and segments of a stream-k launch) are
+// private to this file, so they are kept in the order the accumulators have in registers:
+// 16-byte group q of thread t, i.e. the accumulators 4 g .. 4 g + 3 of the thread's block (i, j)
+// with q = (i TN + j) 4 + g, sits at float (q NT + t) 4.  A thread then writes its tile in
+// TM x TN x 4 fully coalesced 16-byte stores instead of 16 times as many 4-byte ones.  The
+// four floats of a group are four consecutive n of one m:
+template <class T>
+__device__ __forceinline__ void mnv_partial_group_mn(int group, int& m, int& n) {
+  const int q = group / T::NT, t = group - q * T::NT;
+  const int wave = t / MNV_WAVE, lane = t % MNV_WAVE;
+  const int i = q / (T::TN * 4), j = (q / 4) % T::TN, g = q % 4;
+  m = (wave % T::WGM) * T::WM + i * 32 + lane % 32;
+  n = (wave / T::WGM) * T::WN + j * 32 + (lane / 32) * 4 + 8 * g;
+}
 template <class T, class P, int G = 1, bool SK = false, int PF = 1>
 __global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MIN_WAVES) void mnv_gemm_kernel(
     P prob, int tiles_m, int tiles_n, int slabs_per_split, float* __restrict__ partial,
@@ -529,11 +543,11 @@ __global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MI
 
   // Accumulator register r of lane (lm, lk) holds C[m = lm, n = lk*4 + r%4 + 8*(r/4)]
   // of its 32x32 block.
-  if constexpr (SK) {  // a range or a segment: the whole tile, in tile order, into its slot
+  if constexpr (SK) {  // a range or a segment: the whole tile, in register order, into its slot
     // The empty asm keeps the store addresses from being computed once before the segment
     // loop (they do not change from segment to segment): 64 registers held across the main
     // loop would spill.
-    int at = (wn + lk * 4) * T::BM + wm + lm;
+    int at = tid * 4;
     asm volatile("" : "+v"(at));
     float* pt = partial + (size_t)(sk_aligned ? sk_p : sk_p + vb) * (T::BM * T::BNU) + at;
 #pragma unroll
@@ -541,8 +555,10 @@ __global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MI
 #pragma unroll
       for (int j = 0; j < T::TN; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          pt[(j * 32 + (r & 3) + 8 * (r >> 2)) * T::BM + i * 32] = acc[i][j][r];
+        for (int g = 0; g < 4; ++g) {
+          const mnv_f4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+          *reinterpret_cast<mnv_f4*>(pt + ((i * T::TN + j) * 4 + g) * (T::NT * 4)) = v;
+        }
     if (sk_aligned) return;
     sk_u += slab_end - slab_begin;
     if (sk_u >= sk_end) return;
@@ -550,15 +566,17 @@ __global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MI
     // LDS are free for the next segment
     continue;
   }
-  if (G == 1 && tail_part >= 0) {  // a k range of a tail tile: the whole tile, in tile order
-    float* pt = partial + ((size_t)(vb - tail_begin) * tail_z + tail_part) * (T::BM * T::BNU);
+  if (G == 1 && tail_part >= 0) {  // a k range of a tail tile: the whole tile, in register order
+    float* pt = partial + ((size_t)(vb - tail_begin) * tail_z + tail_part) * (T::BM * T::BNU) + tid * 4;
 #pragma unroll
     for (int i = 0; i < T::TM; ++i)
 #pragma unroll
       for (int j = 0; j < T::TN; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          pt[(wn + j * 32 + lk * 4 + (r & 3) + 8 * (r >> 2)) * T::BM + wm + i * 32 + lm] = acc[i][j][r];
+        for (int g = 0; g < 4; ++g) {
+          const mnv_f4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+          *reinterpret_cast<mnv_f4*>(pt + ((i * T::TN + j) * 4 + g) * (T::NT * 4)) = v;
+        }
     return;
   }
   const bool split = gridDim.z > 1;
@@ -702,7 +720,8 @@ static int mnv_gemm_splitk_reduce_launch(const P& prob, const float* partial, in
 }
 
 // Adds the k ranges of the tail tiles (see mnv_gemm_kernel) in range order and hands every
-// element to the policy's store.  One thread per four consecutive rows of a tile column.
+// element to the policy's store.  One thread per 16-byte group of the partial tiles (register
+// order, see mnv_partial_group_mn): four consecutive columns of one row.
 template <class T, class P>
 __global__ __launch_bounds__(256) void mnv_gemm_tail_reduce_kernel(P prob,
                                                                    const float* __restrict__ partial,
@@ -718,12 +737,15 @@ __global__ __launch_bounds__(256) void mnv_gemm_tail_reduce_kernel(P prob,
       const mnv_f4 v = *reinterpret_cast<const mnv_f4*>(p + (size_t)z * TILE + e);
       s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
-    const int m = m0 + e % T::BM, n = n0 + e / T::BM;
-    if (n < prob.N) {
-      if (m + 0 < prob.M) prob.c_store(m + 0, n, s.x);
-      if (m + 1 < prob.M) prob.c_store(m + 1, n, s.y);
-      if (m + 2 < prob.M) prob.c_store(m + 2, n, s.z);
-      if (m + 3 < prob.M) prob.c_store(m + 3, n, s.w);
+    int m, n;
+    mnv_partial_group_mn<T>(e / 4, m, n);
+    m += m0;
+    n += n0;
+    if (m < prob.M) {
+      if (n + 0 < prob.N) prob.c_store(m, n + 0, s.x);
+      if (n + 1 < prob.N) prob.c_store(m, n + 1, s.y);
+      if (n + 2 < prob.N) prob.c_store(m, n + 2, s.z);
+      if (n + 3 < prob.N) prob.c_store(m, n + 3, s.w);
     }
   }
 }
@@ -733,8 +755,8 @@ __global__ __launch_bounds__(256) void mnv_gemm_tail_reduce_kernel(P prob,
 // the slots z T + t and, when the launch had R = W - T aligned remaining workgroups, the
 // segments of those that met the tile: remaining workgroup r covered the units [U r / R,
 // U (r + 1) / R) of the U = T `rest` slabs the aligned ranges left, tile t is the units [t rest,
-// (t + 1) rest), and the segment sits in slot T aligned + r + t.  A thread owns four
-// consecutive rows of a tile column; ZL threads share them: thread z adds the partial tiles z,
+// (t + 1) rest), and the segment sits in slot T aligned + r + t.  A thread owns one 16-byte
+// group of the tile (register order, see mnv_partial_group_mn); ZL threads share it: thread z adds the partial tiles z,
 // z + ZL, ... in order, and the ZL sums are added in order through LDS.  An output of few
 // tiles has hundreds of partial tiles per tile (three tiles on 768 workgroups: 256 each),
 // which one thread per element walked in 52 us; sixteen walk them in a quarter of that.
@@ -803,12 +825,15 @@ __global__ __launch_bounds__(256) void mnv_gemm_streamk_reduce_kernel(P prob,
         s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
       }
     }
-    const int m = m0 + e % T::BM, n = n0 + e / T::BM;
-    if (n < prob.N) {
-      if (m + 0 < prob.M) prob.c_store(m + 0, n, s.x);
-      if (m + 1 < prob.M) prob.c_store(m + 1, n, s.y);
-      if (m + 2 < prob.M) prob.c_store(m + 2, n, s.z);
-      if (m + 3 < prob.M) prob.c_store(m + 3, n, s.w);
+    int m, n;
+    mnv_partial_group_mn<T>(e / 4, m, n);
+    m += m0;
+    n += n0;
+    if (m < prob.M) {
+      if (n + 0 < prob.N) prob.c_store(m, n + 0, s.x);
+      if (n + 1 < prob.N) prob.c_store(m, n + 1, s.y);
+      if (n + 2 < prob.N) prob.c_store(m, n + 2, s.z);
+      if (n + 3 < prob.N) prob.c_store(m, n + 3, s.w);
     }
   }
 }
