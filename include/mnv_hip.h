@@ -234,7 +234,22 @@ int mnv_softmax_channel_bwd(const float* top_diff, const float* top, float* bott
  * One launch reads bottom, top and filter through 32-bit byte offsets (fewer than 2^29
  * elements each).  A batch whose bottom or top is larger (up to 2^31 - 1 elements) runs as
  * several launches over chunks of images, the filter gradient accumulating chunk by chunk;
- * only a single image or a filter of 2^29 elements and more is refused (MNV_ERR_INVALID). ---- */
+ * only a single image or a filter of 2^29 elements and more is refused (MNV_ERR_INVALID).
+ * 3 x 3 filters at unit stride with a bottom (forward) / top (backward_data) channel count
+ * that is a multiple of 16 may run by minimal filtering F(2 x 2, 3 x 3): 16 multiplies per
+ * 2 x 2 outputs of a channel pair instead of 36, as 16 matrix products between transforms
+ * of 4 x 4 tiles, summed in fp32; results differ from the direct sum by a few 1e-7 of the
+ * output's norm.  It wants the workspace the size queries report (16 transformed values
+ * per tile and channel of both tensors); with less it runs in groups of images, with less
+ * than one image needs the direct kernels run. ---- */
+/* Selects when forward / backward_data take the minimal-filtering path.  0: never;
+ * 1 (initial): where the geometry makes it faster (at least 32 input channels, output
+ * channels that fill 128-wide tiles to three quarters, at least 1024 tiles per launch,
+ * output extents whose rounding up to even wastes at most 40%); 2: wherever it applies.
+ * Process-wide; returns the previous mode; any other value only queries.  No reference
+ * counterpart: cuDNN picks its algorithm out of sight (CUDNN_CONVOLUTION_FWD_PREFER_FASTEST,
+ * cuda_perform.cu:227-264). */
+int mnv_conv_winograd_mode(int mode);
 size_t mnv_conv_fwd_workspace_bytes(int num_images, int bottom_num_channels,
                                    int top_num_channels, int bottom_height, int bottom_width,
                                    int pad_height, int pad_width, int stride_vertical,

@@ -14,6 +14,7 @@
 // Roofline: fp32 MFMA, 2*N*Ho*Wo*K*C*R*S algorithmic flops per pass.
 
 #include "gemm_core.h"
+#include "winograd.h"
 
 namespace {
 
@@ -900,8 +901,13 @@ size_t mnv_conv_fwd_workspace_bytes(int N, int C, int K, int H, int W, int ph, i
   const int gm = N * g.HoWo, gn = K;
   const int splits = small_tile_splits(pick_tile(gm, gn), gm, gn, (g.CRS + 15) / 16, (size_t)-1);
   const size_t tail = tail_workspace_bytes(pick_tile(gm, gn), gm, gn, (g.CRS + 15) / 16);
-  if (tail) return align256(permuted) + tail;
-  return splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
+  size_t need = tail ? align256(permuted) + tail
+                     : splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
+  if (mnv_wino_images(N, C, K, H, W, ph, pw, R, S, sv, sh, (size_t)-1)) {
+    const size_t w = mnv_wino_workspace_bytes(N, C, K, H, W, ph, pw);
+    if (w > need) need = w;
+  }
+  return need;
 }
 
 static int conv_fwd_impl(const float* bottom, const float* filter, const float* bias, float* top,
@@ -914,6 +920,10 @@ static int conv_fwd_impl(const float* bottom, const float* filter, const float* 
   if (rc) return rc;
   int gm = N * g.HoWo, gn = K, gk = g.CRS;
   hipStream_t s = mnv_stream(stream);
+  // 3 x 3 unit-stride layers with enough channels and tiles: F(2 x 2, 3 x 3), see winograd.hip
+  if (const int images = mnv_wino_images(N, C, K, H, W, ph, pw, R, S, sv, sh, workspace ? workspace_bytes : 0))
+    return mnv_wino_conv(bottom, filter, bias, nullptr, top, N, C, K, H, W, ph, pw, 0, relu, images,
+                         workspace, workspace_bytes, s);
   const int tile = pick_tile(gm, gn);
   const size_t permuted_bytes = (size_t)K * g.CRS * sizeof(float);
   // the no-padding policy reads the filter where it is; for a small problem the extra
@@ -983,8 +993,13 @@ size_t mnv_conv_bwd_data_workspace_bytes(int N, int C, int K, int H, int W, int 
   const int gm = N * g.HW, gn = C;
   const int splits = small_tile_splits(pick_tile(gm, gn), gm, gn, (K * g.RS + 15) / 16, (size_t)-1);
   const size_t tail = tail_workspace_bytes(pick_tile(gm, gn), gm, gn, (K * g.RS + 15) / 16);
-  if (tail) return align256(permuted) + tail;
-  return splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
+  size_t need = tail ? align256(permuted) + tail
+                     : splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
+  if (mnv_wino_images(N, K, C, g.Ho, g.Wo, 2 - ph, 2 - pw, R, S, sv, sh, (size_t)-1)) {
+    const size_t w = mnv_wino_workspace_bytes(N, K, C, g.Ho, g.Wo, 2 - ph, 2 - pw);
+    if (w > need) need = w;
+  }
+  return need;
 }
 
 static int conv_bwd_data_impl(const float* top_diff, const float* filter, const float* gate,
@@ -997,6 +1012,11 @@ static int conv_bwd_data_impl(const float* top_diff, const float* filter, const 
   if (rc) return rc;
   int gm = N * g.HW, gn = C, gk = K * g.RS;
   hipStream_t s = mnv_stream(stream);
+  // the same correlation, of top_diff with the unflipped filters, under a padding of 2 - pad
+  if (const int images = mnv_wino_images(N, K, C, g.Ho, g.Wo, 2 - ph, 2 - pw, R, S, sv, sh,
+                                         workspace ? workspace_bytes : 0))
+    return mnv_wino_conv(top_diff, filter, nullptr, gate, bottom_diff, N, K, C, g.Ho, g.Wo, 2 - ph,
+                         2 - pw, 1, 0, images, workspace, workspace_bytes, s);
   const int tile = pick_tile(gm, gn);
   const size_t permuted_bytes = (size_t)K * g.CRS * sizeof(float);
   const bool fast = sv == 1 && sh == 1 && K % 16 == 0 && workspace && workspace_bytes >= permuted_bytes;

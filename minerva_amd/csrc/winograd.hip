@@ -1,0 +1,331 @@
+// 3 x 3, unit-stride convolutions by the minimal-filtering algorithm F(2 x 2, 3 x 3)
+// (Winograd): every 2 x 2 block of outputs of one channel pair costs 16 multiplies instead
+// of 36.  The work becomes 16 independent matrix products, one per point (xi, nu) of the
+// transformed 4 x 4 tile,
+//     M[xi,nu][co][p] = sum_ci U[xi,nu][co][ci] * V[xi,nu][ci][p],      p = (image, tile row, tile col)
+// with U = G g G^T (filters), V = B^T d B (4 x 4 input tiles, stride 2) and the outputs
+// Y = A^T M A.  The 16 products run as ONE launch of the fp32 MFMA core (gemm_core.h): the
+// transform point is folded into the column index, n = point * Coutp + co, and a workgroup
+// picks the V panel of its point once, in block_init.  Semantics are those of conv.hip: the
+// forward pass correlates with the flipped filter (cuDNN's CUDNN_CONVOLUTION as selected at
+// minerva/op/impl/cuda/cuda_perform.cu:227-264), the data gradient (cuda_perform.cu:266-291)
+// is the same correlation of top_diff with the unflipped filter, channels exchanged, under a
+// padding of 2 - pad.
+//
+//   B^T = | 1  0 -1  0 |   G = | 1    0    0  |   A^T = | 1  1  1  0 |
+//         | 0  1  1  0 |       | 1/2  1/2  1/2|         | 0  1 -1 -1 |
+//         | 0 -1  1  0 |       | 1/2 -1/2  1/2|
+//         | 0  1  0 -1 |       | 0    0    1  |
+//
+// Rounding: the transforms add and halve, the products are summed in fp32 over Cin; the
+// result differs from the direct sum by a few 1e-7 of the output's norm.
+// Roofline: the matrix products are MFMA-bound (2 * 16 * Cout * Cin * tiles flops, 4 / 9 of
+// the direct flops when the output extents are even); the three transform kernels stream
+// 16 * 4 bytes per (channel, tile) and are HBM-bound.
+
+#include "gemm_core.h"
+#include "winograd.h"
+
+namespace {
+
+struct WinoGeom {
+  int N, Cin, Cout, Coutp;  // Coutp: Cout rounded up to the tile width of the product
+  int Hs, Ws, Hd, Wd;       // source and destination planes
+  int pad_h, pad_w;         // of the correlation: d[a][b] = src[2 th - pad_h + a][2 tw - pad_w + b]
+  int TH, TW, P, Pp;        // tiles per plane, tiles in all, P rounded up to 4
+  MnvFastDiv d_T, d_TW, d_Cin;
+};
+
+// U[point][co][ci] from filter[k][c][3][3].  Forward: co = k, ci = c, g[r][s] = f[2-r][2-s];
+// data gradient (`transposed`): co = c, ci = k, g = f.  Rows co >= Cout are zero.
+__global__ __launch_bounds__(256) void mnv_wino_filter_kernel(const float* __restrict__ filter,
+                                                              float* __restrict__ U, WinoGeom g,
+                                                              int K, int C, bool transposed) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= g.Coutp * g.Cin) return;
+  const int co = mnv_fastdiv(t, g.d_Cin), ci = t - co * g.Cin;
+  float f[3][3];
+  if (co < g.Cout) {
+    const float* src = transposed ? filter + ((size_t)ci * C + co) * 9 : filter + ((size_t)co * C + ci) * 9;
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+      for (int s = 0; s < 3; ++s) f[r][s] = transposed ? src[r * 3 + s] : src[(2 - r) * 3 + (2 - s)];
+  } else {
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+      for (int s = 0; s < 3; ++s) f[r][s] = 0.f;
+  }
+  float h[4][3];
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+    h[0][s] = f[0][s];
+    h[1][s] = 0.5f * (f[0][s] + f[1][s] + f[2][s]);
+    h[2][s] = 0.5f * (f[0][s] - f[1][s] + f[2][s]);
+    h[3][s] = f[2][s];
+  }
+  const size_t plane = (size_t)g.Coutp * g.Cin;
+  float* out = U + (size_t)co * g.Cin + ci;
+#pragma unroll
+  for (int xi = 0; xi < 4; ++xi) {
+    out[(xi * 4 + 0) * plane] = h[xi][0];
+    out[(xi * 4 + 1) * plane] = 0.5f * (h[xi][0] + h[xi][1] + h[xi][2]);
+    out[(xi * 4 + 2) * plane] = 0.5f * (h[xi][0] - h[xi][1] + h[xi][2]);
+    out[(xi * 4 + 3) * plane] = h[xi][2];
+  }
+}
+
+// V[point][ci][p] = (B^T d B)[point] of the 4 x 4 tile p of channel ci; p >= P writes zeros.
+__global__ __launch_bounds__(256) void mnv_wino_input_kernel(const float* __restrict__ src,
+                                                             float* __restrict__ V, WinoGeom g) {
+  const int p = blockIdx.x * 256 + threadIdx.x;
+  const int ci = blockIdx.y;
+  if (p >= g.Pp) return;
+  float d[4][4];
+  if (p < g.P) {
+    const int img = mnv_fastdiv(p, g.d_T);
+    const int t = p - img * (g.TH * g.TW);
+    const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
+    const int y0 = 2 * th - g.pad_h, x0 = 2 * tw - g.pad_w;
+    const float* plane = src + ((size_t)img * g.Cin + ci) * (g.Hs * g.Ws);
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int y = y0 + a, x = x0 + b;
+        d[a][b] = ((unsigned)y < (unsigned)g.Hs && (unsigned)x < (unsigned)g.Ws) ? plane[y * g.Ws + x] : 0.f;
+      }
+  } else {
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) d[a][b] = 0.f;
+  }
+  float h[4][4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    h[0][b] = d[0][b] - d[2][b];
+    h[1][b] = d[1][b] + d[2][b];
+    h[2][b] = d[2][b] - d[1][b];
+    h[3][b] = d[1][b] - d[3][b];
+  }
+  const size_t plane = (size_t)g.Cin * g.Pp;
+  float* out = V + (size_t)ci * g.Pp + p;
+#pragma unroll
+  for (int xi = 0; xi < 4; ++xi) {
+    out[(xi * 4 + 0) * plane] = h[xi][0] - h[xi][2];
+    out[(xi * 4 + 1) * plane] = h[xi][1] + h[xi][2];
+    out[(xi * 4 + 2) * plane] = h[xi][2] - h[xi][1];
+    out[(xi * 4 + 3) * plane] = h[xi][1] - h[xi][3];
+  }
+}
+
+// dst[img][co][2 th + a][2 tw + b] = (A^T M A)[a][b] (+ bias[co]) (then max(., 0)) (then kept
+// only where gate > 0): the epilogues of the direct kernels, each the single operation of the
+// separate operator.
+__global__ __launch_bounds__(256) void mnv_wino_output_kernel(const float* __restrict__ Mx,
+                                                              const float* __restrict__ bias,
+                                                              const float* __restrict__ gate,
+                                                              float* __restrict__ dst, WinoGeom g,
+                                                              int relu) {
+  const int p = blockIdx.x * 256 + threadIdx.x;
+  const int co = blockIdx.y;
+  if (p >= g.P) return;
+  const size_t plane = (size_t)g.Coutp * g.Pp;
+  const float* in = Mx + (size_t)co * g.Pp + p;
+  float m[4][4];
+#pragma unroll
+  for (int xi = 0; xi < 4; ++xi)
+#pragma unroll
+    for (int nu = 0; nu < 4; ++nu) m[xi][nu] = in[(xi * 4 + nu) * plane];
+  float h[2][4];
+#pragma unroll
+  for (int nu = 0; nu < 4; ++nu) {
+    h[0][nu] = m[0][nu] + m[1][nu] + m[2][nu];
+    h[1][nu] = m[1][nu] - m[2][nu] - m[3][nu];
+  }
+  float y[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+    y[a][0] = h[a][0] + h[a][1] + h[a][2];
+    y[a][1] = h[a][1] - h[a][2] - h[a][3];
+  }
+  const int img = mnv_fastdiv(p, g.d_T);
+  const int t = p - img * (g.TH * g.TW);
+  const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
+  const float b = bias ? bias[co] : 0.f;
+  const size_t base = ((size_t)img * g.Cout + co) * (g.Hd * g.Wd);
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int yy = 2 * th + a, xx = 2 * tw + c;
+      if (yy < g.Hd && xx < g.Wd) {
+        float v = y[a][c];
+        if (bias) v = v + b;
+        if (relu) v = v > 0.f ? v : 0.f;
+        const size_t at = base + yy * g.Wd + xx;
+        if (gate) v = gate[at] > 0.f ? v : 0.f;
+        dst[at] = v;
+      }
+    }
+}
+
+// The 16 products as one: C{Pp, 16 Coutp} = A{Pp, Cin} B{Cin, 16 Coutp}, column-major, where the
+// A of a column tile is the V panel of the tile's transform point.
+struct WinoGemm {
+  static constexpr bool A_KFAST = false, B_KFAST = true;
+  static constexpr int A_NOFF = 1, B_NOFF = 1;
+  const float* __restrict__ V;
+  const float* __restrict__ U;
+  float* __restrict__ Mx;
+  int M, N, K, total_slabs, spp;  // Pp, 16 Coutp, Cin
+  int coutp;
+  struct Res {
+    mnv_rsrc a, b;
+  };
+  struct AState {};
+  struct BState {};
+  __device__ void make_res(Res& r) const {
+    r.a = mnv_make_rsrc(V, (unsigned)K * (unsigned)M * 4u);
+    r.b = mnv_make_rsrc(U, (unsigned)N * (unsigned)K * 4u);
+  }
+  __device__ void block_init(Res& r, float*, int, int n0) const {
+    r.a = mnv_make_rsrc(V + (size_t)(n0 / coutp) * K * M, (unsigned)K * (unsigned)M * 4u);
+  }
+  __device__ void a_init(const Res&, AState&, int) const {}
+  __device__ void b_init(const Res&, BState&, int) const {}
+  __device__ void a_period(const AState&, unsigned (&off)[1], int m, int kl, int period) const {
+    const int k = period * spp * 16 + kl;
+    off[0] = ((m < M) & (k < K)) ? ((unsigned)k * (unsigned)M + (unsigned)m) * 4u : MNV_OOB;
+  }
+  __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[1], int, int s, int,
+                         float (&v)[4]) const {
+    mnv_fetch_vec<1>(r.a, off, (unsigned)s * 16u * (unsigned)M * 4u, v);
+  }
+  __device__ void b_period(const BState&, unsigned (&off)[1], int n, int kl, int period) const {
+    const int k = period * spp * 16 + kl;
+    off[0] = ((n < N) & (k < K)) ? ((unsigned)n * (unsigned)K + (unsigned)k) * 4u : MNV_OOB;
+  }
+  __device__ void b_load(const Res& r, const BState&, const unsigned (&off)[1], int, int s, int,
+                         float (&v)[4]) const {
+    mnv_fetch_vec<1>(r.b, off, (unsigned)s * 64u, v);
+  }
+  size_t extra_lds_bytes() const { return 0; }
+  __device__ void c_store(int m, int n, float x) const { Mx[(size_t)n * M + m] = x; }
+  static constexpr bool C_STORE4 = true;
+  __device__ void c_store4(int m, int n, const float (&x)[4]) const {
+    const mnv_f4 v = {x[0], x[1], x[2], x[3]};  // M is a multiple of 4: whole and aligned
+    *reinterpret_cast<mnv_f4*>(Mx + (size_t)n * M + m) = v;
+  }
+};
+
+typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
+
+inline size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+int make_wino_geom(WinoGeom* g, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w) {
+  if (N <= 0 || Cin <= 0 || Cout <= 0 || Hs <= 0 || Ws <= 0 || pad_h < 0 || pad_w < 0 || pad_h > 2 ||
+      pad_w > 2 || Hs + 2 * pad_h < 3 || Ws + 2 * pad_w < 3)
+    return MNV_ERR_INVALID;
+  g->N = N; g->Cin = Cin; g->Cout = Cout; g->Coutp = (Cout + 127) / 128 * 128;
+  g->Hs = Hs; g->Ws = Ws; g->Hd = Hs + 2 * pad_h - 2; g->Wd = Ws + 2 * pad_w - 2;
+  g->pad_h = pad_h; g->pad_w = pad_w;
+  g->TH = (g->Hd + 1) / 2; g->TW = (g->Wd + 1) / 2;
+  const long long P = (long long)N * g->TH * g->TW;
+  if (P > (1LL << 28)) return MNV_ERR_INVALID;
+  g->P = (int)P; g->Pp = (int)((P + 3) / 4 * 4);
+  // a V panel and U are read through 32-bit byte offsets
+  if ((long long)Cin * g->Pp > (1LL << 29) - 1 || 16LL * g->Coutp * Cin > (1LL << 29) - 1)
+    return MNV_ERR_INVALID;
+  g->d_T = mnv_fastdiv_make(g->TH * g->TW);
+  g->d_TW = mnv_fastdiv_make(g->TW);
+  g->d_Cin = mnv_fastdiv_make(Cin);
+  return MNV_OK;
+}
+
+size_t u_bytes(const WinoGeom& g) { return align256((size_t)16 * g.Coutp * g.Cin * sizeof(float)); }
+// V and M of `images` images
+size_t vm_bytes(const WinoGeom& g, int images) {
+  const size_t pp = ((size_t)images * g.TH * g.TW + 3) / 4 * 4;
+  return align256(16 * pp * g.Cin * sizeof(float)) + align256(16 * pp * g.Coutp * sizeof(float));
+}
+
+std::atomic<int> g_mode{1};
+
+}  // namespace
+
+extern "C" int mnv_conv_winograd_mode(int mode) {
+  if (mode < 0 || mode > 2) return g_mode.load(std::memory_order_relaxed);
+  return g_mode.exchange(mode, std::memory_order_relaxed);
+}
+
+size_t mnv_wino_workspace_bytes(int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w) {
+  WinoGeom g;
+  if (make_wino_geom(&g, N, Cin, Cout, Hs, Ws, pad_h, pad_w)) return 0;
+  return u_bytes(g) + vm_bytes(g, N);
+}
+
+int mnv_wino_images(int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w, int R, int S,
+                    int sv, int sh, size_t workspace_bytes) {
+  const int mode = g_mode.load(std::memory_order_relaxed);
+  WinoGeom g;
+  if (mode == 0 || R != 3 || S != 3 || sv != 1 || sh != 1 || Cin % 16 != 0 ||
+      make_wino_geom(&g, N, Cin, Cout, Hs, Ws, pad_h, pad_w))
+    return 0;
+  if (workspace_bytes < u_bytes(g) + vm_bytes(g, 1)) return 0;
+  int images = N;
+  if (workspace_bytes < u_bytes(g) + vm_bytes(g, N)) {
+    // the largest chunk that fits, then chunks of equal size
+    int lo = 1, hi = N;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) / 2;
+      if (u_bytes(g) + vm_bytes(g, mid) <= workspace_bytes) lo = mid;
+      else hi = mid - 1;
+    }
+    const int chunks = (N + lo - 1) / lo;
+    images = (N + chunks - 1) / chunks;
+  }
+  if (mode == 2) return images;
+  const long long tiles = (long long)images * g.TH * g.TW;
+  const bool pays = Cin >= 32 && Cout * 4 >= g.Coutp * 3 && tiles >= 1024 &&
+                    4LL * g.TH * g.TW * 5 <= 7LL * g.Hd * g.Wd;
+  return pays ? images : 0;
+}
+
+int mnv_wino_conv(const float* src, const float* filter, const float* bias, const float* gate,
+                  float* dst, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w,
+                  int transposed, int relu, int images, void* workspace, size_t workspace_bytes,
+                  hipStream_t s) {
+  WinoGeom g;
+  if (!src || !filter || !dst || images <= 0 || Cin % 16 != 0) return MNV_ERR_INVALID;
+  if (images > N) images = N;
+  int rc = make_wino_geom(&g, images, Cin, Cout, Hs, Ws, pad_h, pad_w);
+  if (rc) return rc;
+  if (!workspace || workspace_bytes < u_bytes(g) + vm_bytes(g, images)) return MNV_ERR_INVALID;
+  char* w = static_cast<char*>(workspace);
+  float* U = reinterpret_cast<float*>(w);
+  w += u_bytes(g);
+  float* V = reinterpret_cast<float*>(w);
+  w += align256((size_t)16 * g.Pp * Cin * sizeof(float));
+  float* Mx = reinterpret_cast<float*>(w);
+  const int K = transposed ? Cin : Cout, C = transposed ? Cout : Cin;
+  hipLaunchKernelGGL(mnv_wino_filter_kernel, dim3((g.Coutp * Cin + 255) / 256), dim3(256), 0, s,
+                     filter, U, g, K, C, transposed != 0);
+  if ((rc = MNV_LAUNCH_STATUS())) return rc;
+  const size_t per_src = (size_t)Cin * Hs * Ws, per_dst = (size_t)Cout * g.Hd * g.Wd;
+  for (int n0 = 0; n0 < N; n0 += images) {
+    const int nn = N - n0 < images ? N - n0 : images;
+    if (nn != g.N && (rc = make_wino_geom(&g, nn, Cin, Cout, Hs, Ws, pad_h, pad_w))) return rc;
+    hipLaunchKernelGGL(mnv_wino_input_kernel, dim3((g.Pp + 255) / 256, Cin), dim3(256), 0, s,
+                       src + n0 * per_src, V, g);
+    if ((rc = MNV_LAUNCH_STATUS())) return rc;
+    WinoGemm p{V, U, Mx, g.Pp, 16 * g.Coutp, Cin, Cin / 16, Cin / 16, g.Coutp};
+    if ((rc = mnv_gemm_launch<TileBig>(p, 1, nullptr, s))) return rc;
+    hipLaunchKernelGGL(mnv_wino_output_kernel, dim3((g.P + 255) / 256, Cout), dim3(256), 0, s, Mx,
+                       bias, gate ? gate + n0 * per_dst : nullptr, dst + n0 * per_dst, g, relu);
+    if ((rc = MNV_LAUNCH_STATUS())) return rc;
+  }
+  return MNV_OK;
+}

@@ -55,6 +55,33 @@ def test_pure_host_entry_points():
     assert L.mnv_conv_bwd_filter_workspace_bytes(256, 256, 384, 13, 13, 1, 1, 1, 1, 3, 3) > 0
 
 
+def test_winograd_switch_and_size_queries():
+    """The path switch is process-wide host state and the size queries follow it (pure
+    arithmetic): the 384 -> 384 channel layer on 13 x 13 planes at batch 256 asks for its
+    transformed tensors (16 values per 4 x 4 tile and channel: 597 MB) only while the path
+    is on; a 5 x 5 layer never does."""
+    from minerva_amd import capi
+    L = capi.lib()
+    conv4 = (256, 384, 384, 13, 13, 1, 1, 1, 1, 3, 3)
+    conv2 = (256, 96, 256, 27, 27, 2, 2, 1, 1, 5, 5)
+    assert L.mnv_conv_winograd_mode(-1) == 1
+    try:
+        on = L.mnv_conv_fwd_workspace_bytes(*conv4)
+        tiles = 256 * 7 * 7
+        assert on == 16 * 384 * 384 * 4 + 2 * 16 * tiles * 384 * 4
+        assert L.mnv_conv_bwd_data_workspace_bytes(*conv4) == on
+        five = L.mnv_conv_fwd_workspace_bytes(*conv2)
+        assert L.mnv_conv_winograd_mode(0) == 1
+        assert L.mnv_conv_fwd_workspace_bytes(*conv4) < on // 4
+        assert L.mnv_conv_fwd_workspace_bytes(*conv2) == five
+        assert L.mnv_conv_winograd_mode(2) == 0
+        assert L.mnv_conv_fwd_workspace_bytes(*conv4) == on
+        assert L.mnv_conv_fwd_workspace_bytes(*conv2) == five
+        assert L.mnv_conv_winograd_mode(7) == 2      # out of range: a query
+    finally:
+        L.mnv_conv_winograd_mode(1)
+
+
 def _plan(m, n, k, workspace=True):
     import ctypes
     from minerva_amd import capi

@@ -20,6 +20,15 @@ def gpu():
     return Gpu()
 
 
+@pytest.fixture
+def direct(gpu):
+    """The direct implicit-GEMM kernels for 3 x 3 layers too (tests that aim at one of their
+    launch plans); the minimal-filtering path has tests of its own."""
+    prev = gpu.L.mnv_conv_winograd_mode(0)
+    yield
+    gpu.L.mnv_conv_winograd_mode(prev)
+
+
 def _rand(n, seed, scale=1.0):
     return (np.random.default_rng(seed).standard_normal(n) * scale).astype(np.float32)
 
@@ -184,7 +193,7 @@ def test_conv_random_geometries_against_oracle(gpu, ora, p):
 @pytest.mark.parametrize("p", [(8, 16, 128, 127, 127, 1, 1, 1, 1, 3, 3),    # forward: 505 tiles of 256 x 128
                                (8, 128, 16, 127, 127, 1, 1, 1, 1, 3, 3)],   # the same for the data gradient
                          ids=["forward", "data gradient"])
-def test_conv_on_256_row_tiles_against_oracle(gpu, ora, p):
+def test_conv_on_256_row_tiles_against_oracle(gpu, ora, direct, p):
     """Outputs of about 2^24 elements whose 256 x 128 tiles fill two workgroup slots per CU:
     the (tap, channel) forward / data-gradient kernels then run eight wavefronts per
     workgroup.  Ragged last tile (8 x 127 x 127 positions)."""
@@ -200,7 +209,7 @@ def test_conv_on_256_row_tiles_against_oracle(gpu, ora, p):
     assert normwise(cv.bwd_data(dy, w, False), cv.bwd_data(dy, w).astype(np.float64)) <= 1e-5
 
 
-def test_conv_with_a_cut_tail_against_oracle(gpu, ora):
+def test_conv_with_a_cut_tail_against_oracle(gpu, ora, direct):
     """Launches of a few more large tiles than a multiple of the 256 CUs cut the tiles past
     that multiple into k ranges (partial tiles in the workspace, added by a second kernel):
     264 tiles forward, 526 tiles in the data gradient.  With and without a workspace (no

@@ -1,0 +1,198 @@
+"""GPU parity of the minimal-filtering path F(2 x 2, 3 x 3) of the 3 x 3 unit-stride
+convolutions (forward and data gradient), through the C ABI: against the CPU oracle's direct
+sums on geometries that exercise odd and even extents, every padding, ragged tile counts and
+channel counts off the tile width; in groups of images under a small workspace (same bits as
+in one group); with the fused epilogues (same bits as the operator chain); and the switch
+that selects the path."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from gpu_util import Gpu, assert_bits_equal, normwise, say
+from test_gpu_conv import Conv, _rand
+
+pytestmark = pytest.mark.gpu
+# F(2 x 2, 3 x 3) adds and halves in its transforms: a few 1e-7 of the output's norm in fp32;
+# the bound of the convolutions is 1e-4
+TIGHT = 2e-5
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    return Gpu()
+
+
+class mode:
+    """The path switch set for a block, the previous mode restored after it."""
+
+    def __init__(self, gpu, m):
+        self.L, self.m = gpu.L, m
+
+    def __enter__(self):
+        self.prev = self.L.mnv_conv_winograd_mode(self.m)
+
+    def __exit__(self, *exc):
+        self.L.mnv_conv_winograd_mode(self.prev)
+
+
+GEOMS = [
+    # N, C, K, H, W, ph, pw
+    (2, 16, 16, 6, 6, 1, 1),        # even outputs, one tile row of the product
+    (3, 32, 48, 13, 13, 1, 1),      # odd outputs: the last tile row and column are half empty
+    (2, 16, 128, 8, 8, 0, 0),       # no padding
+    (2, 16, 16, 5, 6, 2, 2),        # full padding (the data gradient then has none)
+    (1, 16, 32, 3, 3, 0, 0),        # a single output per plane
+    (2, 48, 20, 9, 11, 1, 0),       # unequal paddings; 20 output channels (data gradient: direct)
+    (5, 64, 144, 7, 7, 1, 1),       # 144 output channels in two 128-wide column tiles per point
+    (1, 16, 16, 4, 3, 0, 1),        # tiles in all: 1, rounded up to 4
+    (7, 32, 32, 10, 9, 2, 1),
+    (4, 144, 160, 13, 13, 1, 1),    # 9 and 10 k-slabs
+    (3, 16, 16, 21, 2, 1, 1),       # two-pixel-wide planes
+]
+
+
+@pytest.mark.parametrize("p7", GEOMS, ids=lambda p: "x".join(map(str, p)))
+def test_winograd_passes_against_oracle(gpu, ora, p7):
+    N, C, K, H, W, ph, pw = p7
+    p = (N, C, K, H, W, ph, pw, 1, 1, 3, 3)
+    cv = Conv(gpu, *p)
+    x, w, b = _rand(N * C * H * W, 80), _rand(K * C * 9, 81, 0.2), _rand(K, 82)
+    dy = _rand(N * K * cv.Ho * cv.Wo, 83)
+    want_y, want_dx = ora.conv_fwd(x, w, b, *p), ora.conv_bwd_data(dy, w, *p)
+    with mode(gpu, 0):
+        direct_y, direct_dx = cv.fwd(x, w, b), cv.bwd_data(dy, w)
+        direct_bare = cv.fwd(x, w, b, False)
+        direct_bytes = gpu.L.mnv_conv_fwd_workspace_bytes(*p)
+    with mode(gpu, 2):
+        say("winograd fwd", p)
+        # the size query covers the transformed tensors, and the path really ran: its bits
+        # are not those of the direct kernels
+        assert gpu.L.mnv_conv_fwd_workspace_bytes(*p) > direct_bytes
+        y = cv.fwd(x, w, b)
+        assert normwise(y, want_y) <= TIGHT
+        assert np.any(y.view(np.uint32) != direct_y.view(np.uint32))
+        say("winograd bwd data", p)
+        dx = cv.bwd_data(dy, w)
+        assert normwise(dx, want_dx) <= TIGHT
+        if K % 16 == 0:
+            assert np.any(dx.view(np.uint32) != direct_dx.view(np.uint32))
+        else:
+            assert_bits_equal(dx, direct_dx, "top channel count off 16: the direct kernels")
+        # without a workspace the direct kernels run
+        assert_bits_equal(cv.fwd(x, w, b, False), direct_bare, "no workspace")
+
+
+def _wino_bytes(images, C, K, Ho, Wo):
+    """The workspace the path wants for `images` images at once (U, V, M from 256-byte
+    boundaries; tiles rounded up to 4, output channels to 128)."""
+    a256 = lambda v: (v + 255) // 256 * 256
+    kp = (K + 127) // 128 * 128
+    pp = (images * ((Ho + 1) // 2) * ((Wo + 1) // 2) + 3) // 4 * 4
+    return a256(16 * kp * C * 4) + a256(16 * pp * C * 4) + a256(16 * pp * kp * 4)
+
+
+@pytest.mark.parametrize("N", [12, 13])
+def test_winograd_in_groups_of_images_has_the_same_bits(gpu, N):
+    """A workspace that holds five images: 12 images run as three groups of four, 13 as five,
+    five and three.  Every output element is the same sum in the same order."""
+    C, K, H, W = 32, 64, 13, 13
+    p = (N, C, K, H, W, 1, 1, 1, 1, 3, 3)
+    cv = Conv(gpu, *p)
+    x, w, b = _rand(N * C * H * W, 84), _rand(K * C * 9, 85, 0.2), _rand(K, 86)
+    dy = _rand(N * K * H * W, 87)
+    with mode(gpu, 2):
+        assert gpu.L.mnv_conv_fwd_workspace_bytes(*p) == _wino_bytes(N, C, K, H, W)
+        whole_y, whole_dx = cv.fwd(x, w, b), cv.bwd_data(dy, w)
+        small = _wino_bytes(5, C, K, H, W) + 1024
+        assert small < _wino_bytes(N, C, K, H, W)
+        ws = gpu.empty(small // 4 + 64)
+        dxb, dwb, dbb, dyb = gpu.up(x), gpu.up(w), gpu.up(b), gpu.up(dy)
+        top, bd = gpu.empty(whole_y.size), gpu.empty(whole_dx.size)
+        say("winograd in groups, fwd", p)
+        gpu.call("mnv_conv_fwd", dxb.p, dwb.p, dbb.p, top.p, *p, ws.p, ctypes.c_size_t(small))
+        assert_bits_equal(gpu.down(top), whole_y, "forward in groups")
+        say("winograd in groups, bwd data", p)
+        small = _wino_bytes(5, K, C, H, W) + 1024
+        gpu.call("mnv_conv_bwd_data", dyb.p, dwb.p, bd.p, *p, ws.p, ctypes.c_size_t(small))
+        assert_bits_equal(gpu.down(bd), whole_dx, "data gradient in groups")
+
+
+def test_winograd_fused_epilogues_have_the_bits_of_the_chain(gpu):
+    """conv + ReLU and data gradient + ReLU gradient in one call against the separate
+    operators, both on the minimal-filtering path."""
+    p = (6, 32, 48, 11, 12, 1, 1, 1, 1, 3, 3)
+    N, C, K, H, W = p[:5]
+    cv = Conv(gpu, *p)
+    x, w, b = _rand(N * C * H * W, 88), _rand(K * C * 9, 89, 0.2), _rand(K, 90)
+    dy = _rand(N * K * cv.Ho * cv.Wo, 91)
+    with mode(gpu, 2):
+        nbytes = gpu.L.mnv_conv_fwd_workspace_bytes(*p)
+        nbytes = max(nbytes, gpu.L.mnv_conv_bwd_data_workspace_bytes(*p))
+        ws = gpu.empty(nbytes // 4 + 64)
+        dxb, dwb, dbb, dyb = gpu.up(x), gpu.up(w), gpu.up(b), gpu.up(dy)
+        top, bd = gpu.empty(N * K * cv.Ho * cv.Wo), gpu.empty(x.size)
+        say("winograd conv + relu", p)
+        gpu.call("mnv_conv_fwd_relu", dxb.p, dwb.p, dbb.p, top.p, *p, ws.p, ctypes.c_size_t(nbytes))
+        assert_bits_equal(gpu.down(top), np.maximum(cv.fwd(x, w, b), np.float32(0)), "conv + relu")
+        say("winograd data gradient + relu gradient", p)
+        gpu.call("mnv_conv_bwd_data_relu", dyb.p, dwb.p, dxb.p, bd.p, *p, ws.p, ctypes.c_size_t(nbytes))
+        assert_bits_equal(gpu.down(bd), np.where(x > 0, cv.bwd_data(dy, w), np.float32(0)),
+                          "data gradient + relu gradient")
+
+
+def test_winograd_is_taken_by_itself_where_it_pays(gpu, ora):
+    """In the initial mode a 3 x 3 layer with enough channels and tiles takes the path without
+    being asked (96 output channels on 1176 tiles); the same layer with 16 input channels, or
+    at stride 2, or with 5 x 5 filters, does not."""
+    assert gpu.L.mnv_conv_winograd_mode(-1) == 1
+    p = (24, 32, 96, 13, 13, 1, 1, 1, 1, 3, 3)
+    N, C, K, H, W = p[:5]
+    cv = Conv(gpu, *p)
+    x, w, b = _rand(N * C * H * W, 92), _rand(K * C * 9, 93, 0.2), _rand(K, 94)
+    assert gpu.L.mnv_conv_fwd_workspace_bytes(*p) == _wino_bytes(N, C, K, H, W)
+    say("winograd in the initial mode", p)
+    y = cv.fwd(x, w, b)
+    assert normwise(y, ora.conv_fwd(x, w, b, *p)) <= TIGHT
+    with mode(gpu, 0):
+        assert gpu.L.mnv_conv_fwd_workspace_bytes(*p) < _wino_bytes(N, C, K, H, W)
+        direct = cv.fwd(x, w, b)
+    assert np.any(y.view(np.uint32) != direct.view(np.uint32))
+    assert normwise(y, direct) <= TIGHT
+    for q in [(24, 16, 96, 13, 13, 1, 1, 1, 1, 3, 3), (24, 32, 96, 13, 13, 1, 1, 2, 2, 3, 3),
+              (24, 32, 96, 13, 13, 2, 2, 1, 1, 5, 5), (4, 32, 96, 13, 13, 1, 1, 1, 1, 3, 3)]:
+        with mode(gpu, 0):
+            want = gpu.L.mnv_conv_fwd_workspace_bytes(*q)
+        assert gpu.L.mnv_conv_fwd_workspace_bytes(*q) == want, q
+
+
+ALEX3 = [("conv3", 256, 384), ("conv4", 384, 384), ("conv5", 384, 256)]
+
+
+@pytest.mark.parametrize("case", ALEX3, ids=lambda c: c[0])
+def test_direct_and_winograd_agree_at_batch_256(gpu, case):
+    """The 13 x 13 layers of the AlexNet shape at batch 256 on both paths (two independent
+    algorithms over the same 256 distinct images), as the host layer runs them: with the
+    whole-batch workspace and in groups under 128 MB."""
+    name, C, K = case
+    p = (256, C, K, 13, 13, 1, 1, 1, 1, 3, 3)
+    N, H, W = 256, 13, 13
+    cv = Conv(gpu, *p)
+    x, w, b = np.maximum(_rand(N * C * H * W, 95), 0), _rand(K * C * 9, 96, 0.05), _rand(K, 97)
+    dy = _rand(N * K * H * W, 98)
+    say(name, "b256 both paths")
+    with mode(gpu, 0):
+        direct_y, direct_dx = cv.fwd(x, w, b), cv.bwd_data(dy, w)
+    with mode(gpu, 1):
+        assert gpu.L.mnv_conv_fwd_workspace_bytes(*p) == _wino_bytes(N, C, K, H, W)
+        y, dx = cv.fwd(x, w, b), cv.bwd_data(dy, w)
+        assert np.any(y.view(np.uint32) != direct_y.view(np.uint32))
+        assert normwise(y, direct_y) <= TIGHT and normwise(dx, direct_dx) <= TIGHT
+        small = 128 << 20
+        ws = gpu.empty(small // 4)
+        dxb, dwb, dbb, dyb = gpu.up(x), gpu.up(w), gpu.up(b), gpu.up(dy)
+        top, bd = gpu.empty(y.size), gpu.empty(dx.size)
+        gpu.call("mnv_conv_fwd", dxb.p, dwb.p, dbb.p, top.p, *p, ws.p, ctypes.c_size_t(small))
+        assert_bits_equal(gpu.down(top), y, "forward in groups")
+        gpu.call("mnv_conv_bwd_data", dyb.p, dwb.p, bd.p, *p, ws.p, ctypes.c_size_t(small))
+        assert_bits_equal(gpu.down(bd), dx, "data gradient in groups")
