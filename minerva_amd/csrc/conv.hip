@@ -1087,6 +1087,10 @@ size_t mnv_conv_bwd_filter_workspace_bytes(int N, int C, int K, int H, int W, in
     const size_t sk = (size_t)(4 * mnv_cu_count() + tiles) * kTileM[tile] * kTileN[tile] * sizeof(float);
     if (tiles <= 4LL * mnv_cu_count() && sk > bytes) bytes = sk;
   }
+  if (mnv_wino_grad_images(N, C, K, H, W, ph, pw, R, S, sv, sh, (size_t)-1)) {
+    const size_t w = mnv_wino_grad_workspace_bytes(N, C, K, H, W, ph, pw);
+    if (w > bytes) bytes = w;
+  }
   return bytes;
 }
 
@@ -1102,6 +1106,11 @@ static int conv_bwd_filter_impl(const float* bottom, const float* top_diff, floa
   if (rc) return rc;
   int gm = g.CRS, gn = K, gk = N * g.HoWo;
   hipStream_t s = mnv_stream(stream);
+  // 3 x 3 unit-stride layers with enough channels and tiles: F(3 x 3, 2 x 2), see winograd.hip
+  if (const int images = mnv_wino_grad_images(N, C, K, H, W, ph, pw, R, S, sv, sh,
+                                              workspace ? workspace_bytes : 0))
+    return mnv_wino_filter_grad(bottom, top_diff, filter_diff, N, C, K, H, W, ph, pw, images,
+                                accumulate, sgd_w, sgd_scale, workspace, workspace_bytes, s, plan);
   int splits = bwd_filter_splits(gm, gn, gk, workspace ? workspace_bytes / sizeof(float) : 0);
   const int tile = bwd_filter_tile(gm, gn);
   // Fast addressing: rows in (tap, channel) order with per-tap offset tables in LDS.  The

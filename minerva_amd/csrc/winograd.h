@@ -24,3 +24,20 @@ int mnv_wino_conv(const float* src, const float* filter, const float* bias, cons
                   float* dst, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w,
                   int transposed, int relu, int images, void* workspace, size_t workspace_bytes,
                   hipStream_t s);
+
+// The filter gradient of the same layers by F(3 x 3, 2 x 2): the sum over images and tiles is the
+// reduction dimension of the 16 products, which run as one equal-shares launch of the MFMA
+// core.  (C, H, W): bottom; K: channels of top_diff; (ph, pw): the layer's padding.
+// mnv_wino_grad_images as mnv_wino_images (no condition on the channel counts' divisors);
+// with more than one group the products accumulate group by group.
+int mnv_wino_grad_images(int N, int C, int K, int H, int W, int ph, int pw, int R, int S, int sv,
+                         int sh, size_t workspace_bytes);
+size_t mnv_wino_grad_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw);
+// filter_diff {K, C, 3, 3} = the gradient; `accumulate`: added to what is there; `sgd_w`: the value
+// stored is sgd_w - sgd_scale * gradient.  `plan` (optional): nothing is launched, plan[0] =
+// rows of the tile, plan[1] = 1, plan[2] = workgroups of the equal-shares launch (0: the product
+// is too small for it and runs one workgroup per tile).
+int mnv_wino_filter_grad(const float* bottom, const float* top_diff, float* filter_diff, int N, int C,
+                         int K, int H, int W, int ph, int pw, int images, int accumulate,
+                         const float* sgd_w, float sgd_scale, void* workspace,
+                         size_t workspace_bytes, hipStream_t s, int* plan);

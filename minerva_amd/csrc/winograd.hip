@@ -221,6 +221,142 @@ struct WinoGemm {
   }
 };
 
+// ---- filter gradient: F(3 x 3, 2 x 2), the same four points
+//   dg[k][c] = sum_p A'^T [ (G' dy_p G'^T) (.) (B^T d_p B) ] A'      dy_p: the 2 x 2 tile p of top_diff
+//   A'^T = | 1  1  1  0 |   G' = | 1    0  |
+//          | 0  1 -1  0 |        | 1/2  1/2|
+//          | 0  1  1 -1 |        | 1/2 -1/2|
+//                                | 0    1  |
+// The sum over the tiles is the k dimension of the 16 products Q[point][k][c] =
+// sum_p Yt[point][k][p] V[point][c][p].
+
+// Yt[point][k][p] = (G' dy G'^T)[point] of the 2 x 2 tile p of channel k of top_diff; zeros
+// for p >= P and for the rows k >= Cout.
+__global__ __launch_bounds__(256) void mnv_wino_grad_kernel(const float* __restrict__ top_diff,
+                                                            float* __restrict__ Yt, WinoGeom g) {
+  const int p = blockIdx.x * 256 + threadIdx.x;
+  const int k = blockIdx.y;
+  if (p >= g.Pp) return;
+  float d[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+  if (p < g.P && k < g.Cout) {
+    const int img = mnv_fastdiv(p, g.d_T);
+    const int t = p - img * (g.TH * g.TW);
+    const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
+    const float* plane = top_diff + ((size_t)img * g.Cout + k) * (g.Hd * g.Wd);
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int y = 2 * th + a, x = 2 * tw + b;
+        if (y < g.Hd && x < g.Wd) d[a][b] = plane[y * g.Wd + x];
+      }
+  }
+  float h[4][2];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    h[0][b] = d[0][b];
+    h[1][b] = 0.5f * (d[0][b] + d[1][b]);
+    h[2][b] = 0.5f * (d[0][b] - d[1][b]);
+    h[3][b] = d[1][b];
+  }
+  const size_t plane = (size_t)g.Coutp * g.Pp;
+  float* out = Yt + (size_t)k * g.Pp + p;
+#pragma unroll
+  for (int xi = 0; xi < 4; ++xi) {
+    out[(xi * 4 + 0) * plane] = h[xi][0];
+    out[(xi * 4 + 1) * plane] = 0.5f * (h[xi][0] + h[xi][1]);
+    out[(xi * 4 + 2) * plane] = 0.5f * (h[xi][0] - h[xi][1]);
+    out[(xi * 4 + 3) * plane] = h[xi][1];
+  }
+}
+
+// filter_diff[k][c][2-r][2-s] = (A'^T Q A')[r][s] with the epilogues of the direct kernel's
+// store: the parameter update sgd_w - sgd_scale * ., or the sum with what is there.
+// (filter_diff may be sgd_w itself: a thread reads the nine parameters it then writes.)
+__global__ __launch_bounds__(256) void mnv_wino_grad_output_kernel(const float* __restrict__ Q,
+                                                                   float* filter_diff, WinoGeom g,
+                                                                   int accumulate, const float* sgd_w,
+                                                                   float sgd_scale) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= g.Cout * g.Cin) return;
+  const int k = mnv_fastdiv(t, g.d_Cin), c = t - k * g.Cin;
+  const size_t plane = (size_t)g.Coutp * g.Cin;
+  const float* in = Q + (size_t)k * g.Cin + c;
+  float q[4][4];
+#pragma unroll
+  for (int xi = 0; xi < 4; ++xi)
+#pragma unroll
+    for (int nu = 0; nu < 4; ++nu) q[xi][nu] = in[(xi * 4 + nu) * plane];
+  float h[3][4];
+#pragma unroll
+  for (int nu = 0; nu < 4; ++nu) {
+    h[0][nu] = q[0][nu] + q[1][nu] + q[2][nu];
+    h[1][nu] = q[1][nu] - q[2][nu];
+    h[2][nu] = q[1][nu] + q[2][nu] - q[3][nu];
+  }
+  float* out = filter_diff + (size_t)t * 9;
+#pragma unroll
+  for (int r = 0; r < 3; ++r) {
+    const float dg[3] = {h[r][0] + h[r][1] + h[r][2], h[r][1] - h[r][2], h[r][1] + h[r][2] - h[r][3]};
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+      const int at = (2 - r) * 3 + (2 - s);
+      float x = dg[s];
+      if (sgd_w) x = sgd_w[(size_t)t * 9 + at] - sgd_scale * x;
+      else if (accumulate) x = out[at] + x;
+      out[at] = x;
+    }
+  }
+}
+
+// The 16 products of the filter gradient as one: C{Cin, 16 Coutp} = A{Cin, Pp} B{Pp, 16 Coutp},
+// both operands with the reduction index p contiguous; the A of a column tile is the V panel
+// of the tile's transform point.
+struct WinoGradGemm {
+  static constexpr bool A_KFAST = true, B_KFAST = true;
+  static constexpr int A_NOFF = 1, B_NOFF = 1;
+  const float* __restrict__ V;
+  const float* __restrict__ Yt;
+  float* __restrict__ Q;
+  int M, N, K, total_slabs, spp;  // Cin, 16 Coutp, Pp
+  int coutp, accumulate;
+  struct Res {
+    mnv_rsrc a, b;
+  };
+  struct AState {};
+  struct BState {};
+  __device__ void make_res(Res& r) const {
+    r.a = mnv_make_rsrc(V, (unsigned)M * (unsigned)K * 4u);
+    r.b = mnv_make_rsrc(Yt, (unsigned)N * (unsigned)K * 4u);
+  }
+  __device__ void block_init(Res& r, float*, int, int n0) const {
+    r.a = mnv_make_rsrc(V + (size_t)(n0 / coutp) * M * K, (unsigned)M * (unsigned)K * 4u);
+  }
+  __device__ void a_init(const Res&, AState&, int) const {}
+  __device__ void b_init(const Res&, BState&, int) const {}
+  __device__ void a_period(const AState&, unsigned (&off)[1], int m, int kl, int period) const {
+    const int k = period * spp * 16 + kl;  // K is a multiple of 4: a vector is whole or absent
+    off[0] = ((m < M) & (k < K)) ? ((unsigned)m * (unsigned)K + (unsigned)k) * 4u : MNV_OOB;
+  }
+  __device__ void a_load(const Res& r, const AState&, const unsigned (&off)[1], int, int s, int,
+                         float (&v)[4]) const {
+    mnv_fetch_vec<1>(r.a, off, (unsigned)s * 64u, v);
+  }
+  __device__ void b_period(const BState&, unsigned (&off)[1], int n, int kl, int period) const {
+    const int k = period * spp * 16 + kl;
+    off[0] = ((n < N) & (k < K)) ? ((unsigned)n * (unsigned)K + (unsigned)k) * 4u : MNV_OOB;
+  }
+  __device__ void b_load(const Res& r, const BState&, const unsigned (&off)[1], int, int s, int,
+                         float (&v)[4]) const {
+    mnv_fetch_vec<1>(r.b, off, (unsigned)s * 64u, v);
+  }
+  size_t extra_lds_bytes() const { return 0; }
+  __device__ void c_store(int m, int n, float x) const {
+    const size_t at = (size_t)n * M + m;
+    Q[at] = accumulate ? Q[at] + x : x;
+  }
+};
+
 typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 
 inline size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
@@ -252,7 +388,29 @@ size_t vm_bytes(const WinoGeom& g, int images) {
   return align256(16 * pp * g.Cin * sizeof(float)) + align256(16 * pp * g.Coutp * sizeof(float));
 }
 
+// partial tiles of the filter gradient's equal-shares launch: at most four workgroups per CU,
+// a partial tile each and one more per output tile
+size_t grad_sk_bytes(const WinoGeom& g) {
+  const long long tiles = (long long)((g.Cin + 127) / 128) * (16 * g.Coutp / 128);
+  return (size_t)(4 * mnv_cu_count() + tiles) * 128 * 128 * sizeof(float);
+}
+
 std::atomic<int> g_mode{1};
+
+// the largest group of images whose transformed tensors fit `avail` bytes, then groups of
+// equal size; 0 when not even one image fits
+int images_that_fit(const WinoGeom& g, int N, size_t avail) {
+  if (avail < vm_bytes(g, 1)) return 0;
+  if (avail >= vm_bytes(g, N)) return N;
+  int lo = 1, hi = N;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) / 2;
+    if (vm_bytes(g, mid) <= avail) lo = mid;
+    else hi = mid - 1;
+  }
+  const int groups = (N + lo - 1) / lo;
+  return (N + groups - 1) / groups;
+}
 
 }  // namespace
 
@@ -274,20 +432,9 @@ int mnv_wino_images(int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad
   if (mode == 0 || R != 3 || S != 3 || sv != 1 || sh != 1 || Cin % 16 != 0 ||
       make_wino_geom(&g, N, Cin, Cout, Hs, Ws, pad_h, pad_w))
     return 0;
-  if (workspace_bytes < u_bytes(g) + vm_bytes(g, 1)) return 0;
-  int images = N;
-  if (workspace_bytes < u_bytes(g) + vm_bytes(g, N)) {
-    // the largest chunk that fits, then chunks of equal size
-    int lo = 1, hi = N;
-    while (lo < hi) {
-      const int mid = (lo + hi + 1) / 2;
-      if (u_bytes(g) + vm_bytes(g, mid) <= workspace_bytes) lo = mid;
-      else hi = mid - 1;
-    }
-    const int chunks = (N + lo - 1) / lo;
-    images = (N + chunks - 1) / chunks;
-  }
-  if (mode == 2) return images;
+  if (workspace_bytes < u_bytes(g)) return 0;
+  const int images = images_that_fit(g, N, workspace_bytes - u_bytes(g));
+  if (mode == 2 || images == 0) return images;
   const long long tiles = (long long)images * g.TH * g.TW;
   const bool pays = Cin >= 32 && Cout * 4 >= g.Coutp * 3 && tiles >= 1024 &&
                     4LL * g.TH * g.TW * 5 <= 7LL * g.Hd * g.Wd;
@@ -328,4 +475,80 @@ int mnv_wino_conv(const float* src, const float* filter, const float* bias, cons
     if ((rc = MNV_LAUNCH_STATUS())) return rc;
   }
   return MNV_OK;
+}
+
+size_t mnv_wino_grad_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw) {
+  WinoGeom g;
+  if (make_wino_geom(&g, N, C, K, H, W, ph, pw)) return 0;
+  return u_bytes(g) + vm_bytes(g, N) + grad_sk_bytes(g);
+}
+
+int mnv_wino_grad_images(int N, int C, int K, int H, int W, int ph, int pw, int R, int S, int sv,
+                         int sh, size_t workspace_bytes) {
+  const int mode = g_mode.load(std::memory_order_relaxed);
+  WinoGeom g;
+  if (mode == 0 || R != 3 || S != 3 || sv != 1 || sh != 1 || make_wino_geom(&g, N, C, K, H, W, ph, pw))
+    return 0;
+  if (workspace_bytes < u_bytes(g) + grad_sk_bytes(g)) return 0;
+  int images = images_that_fit(g, N, workspace_bytes - u_bytes(g) - grad_sk_bytes(g));
+  // Yt of a group is read through 32-bit byte offsets
+  const long long per_image = (long long)g.TH * g.TW;
+  const long long most = ((1LL << 29) - 1) / (16LL * g.Coutp) / per_image;
+  if (images > most) images = (int)most;
+  if (mode == 2 || images == 0) return images;
+  const long long tiles = (long long)images * per_image;
+  const bool pays = C >= 32 && C * 4 >= (C + 127) / 128 * 128 * 3 && K * 4 >= g.Coutp * 3 &&
+                    tiles >= 1024 && 4LL * g.TH * g.TW * 5 <= 7LL * g.Hd * g.Wd;
+  return pays ? images : 0;
+}
+
+#ifndef MNV_WINO_SK_PF
+#define MNV_WINO_SK_PF 1
+#endif
+int mnv_wino_filter_grad(const float* bottom, const float* top_diff, float* filter_diff, int N, int C,
+                         int K, int H, int W, int ph, int pw, int images, int accumulate,
+                         const float* sgd_w, float sgd_scale, void* workspace,
+                         size_t workspace_bytes, hipStream_t s, int* plan) {
+  WinoGeom g;
+  if (images <= 0) return MNV_ERR_INVALID;
+  if (images > N) images = N;
+  int rc = make_wino_geom(&g, images, C, K, H, W, ph, pw);
+  if (rc) return rc;
+  const size_t sk_bytes = grad_sk_bytes(g);
+  if (!workspace || workspace_bytes < u_bytes(g) + vm_bytes(g, images) + sk_bytes) return MNV_ERR_INVALID;
+  char* w = static_cast<char*>(workspace);
+  float* Q = reinterpret_cast<float*>(w);
+  w += u_bytes(g);
+  float* V = reinterpret_cast<float*>(w);
+  w += align256((size_t)16 * g.Pp * C * sizeof(float));
+  float* Yt = reinterpret_cast<float*>(w);
+  w += align256((size_t)16 * g.Pp * g.Coutp * sizeof(float));
+  if (plan) {
+    WinoGradGemm p{V, Yt, Q, C, 16 * g.Coutp, g.Pp, (g.Pp + 15) / 16, g.Pp >= 16 ? g.Pp / 16 : 1, g.Coutp, 0};
+    bool done = false;
+    plan[0] = 128;
+    plan[1] = 1;
+    plan[2] = 0;
+    return mnv_gemm_streamk_launch<TileBig, MNV_WINO_SK_PF>(p, w, sk_bytes, s, &done, plan + 2);
+  }
+  if (!bottom || !top_diff || !filter_diff) return MNV_ERR_INVALID;
+  const size_t per_bottom = (size_t)C * H * W, per_top = (size_t)K * g.Hd * g.Wd;
+  for (int n0 = 0; n0 < N; n0 += images) {
+    const int nn = N - n0 < images ? N - n0 : images;
+    if (nn != g.N && (rc = make_wino_geom(&g, nn, C, K, H, W, ph, pw))) return rc;
+    hipLaunchKernelGGL(mnv_wino_input_kernel, dim3((g.Pp + 255) / 256, C), dim3(256), 0, s,
+                       bottom + n0 * per_bottom, V, g);
+    if ((rc = MNV_LAUNCH_STATUS())) return rc;
+    hipLaunchKernelGGL(mnv_wino_grad_kernel, dim3((g.Pp + 255) / 256, g.Coutp), dim3(256), 0, s,
+                       top_diff + n0 * per_top, Yt, g);
+    if ((rc = MNV_LAUNCH_STATUS())) return rc;
+    WinoGradGemm p{V, Yt, Q, C, 16 * g.Coutp, g.Pp, (g.Pp + 15) / 16, g.Pp >= 16 ? g.Pp / 16 : 1,
+                   g.Coutp, n0 > 0};
+    bool done = false;
+    if ((rc = mnv_gemm_streamk_launch<TileBig, MNV_WINO_SK_PF>(p, w, sk_bytes, s, &done))) return rc;
+    if (!done && (rc = mnv_gemm_launch<TileBig>(p, 1, nullptr, s))) return rc;
+  }
+  hipLaunchKernelGGL(mnv_wino_grad_output_kernel, dim3((K * C + 255) / 256), dim3(256), 0, s, Q,
+                     filter_diff, g, accumulate, sgd_w, sgd_scale);
+  return MNV_LAUNCH_STATUS();
 }

@@ -381,7 +381,7 @@ STREAMK = [
 
 
 @pytest.mark.parametrize("case", STREAMK, ids=lambda c: c[0])
-def test_conv_bwd_filter_in_equal_shares_against_oracle(gpu, ora, case):
+def test_conv_bwd_filter_in_equal_shares_against_oracle(gpu, ora, direct, case):
     remaining, p = case[1], case[2:]
     N, C, K, H, W, ph, pw, sv, sh, R, S = p
     cv = Conv(gpu, *p)
@@ -423,7 +423,7 @@ def _random_streamk_geometries(count, seed):
 
 
 @pytest.mark.parametrize("p", _random_streamk_geometries(40, 99), ids=lambda p: "x".join(map(str, p)))
-def test_conv_bwd_filter_streamk_random_geometries_sampled_fp64(gpu, p):
+def test_conv_bwd_filter_streamk_random_geometries_sampled_fp64(gpu, direct, p):
     """Beyond what the oracle reaches in seconds: 64 filter-gradient entries per geometry (the
     corners of the index space first) against fp64 sums written from the definition."""
     N, C, K, H, W, ph, pw, sv, sh, R, S = p

@@ -1,5 +1,5 @@
-"""GPU parity of the minimal-filtering path F(2 x 2, 3 x 3) of the 3 x 3 unit-stride
-convolutions (forward and data gradient), through the C ABI: against the CPU oracle's direct
+"""GPU parity of the minimal-filtering paths of the 3 x 3 unit-stride convolutions (forward
+and data gradient by F(2 x 2, 3 x 3), filter gradient by F(3 x 3, 2 x 2)), through the C ABI: against the CPU oracle's direct
 sums on geometries that exercise odd and even extents, every padding, ragged tile counts and
 channel counts off the tile width; in groups of images under a small workspace (same bits as
 in one group); with the fused epilogues (same bits as the operator chain); and the switch
@@ -49,6 +49,8 @@ GEOMS = [
     (7, 32, 32, 10, 9, 2, 1),
     (4, 144, 160, 13, 13, 1, 1),    # 9 and 10 k-slabs
     (3, 16, 16, 21, 2, 1, 1),       # two-pixel-wide planes
+    (2, 20, 24, 5, 6, 2, 2),        # channel counts off 16: only the filter gradient takes the path
+    (9, 130, 40, 9, 9, 1, 1),       # 130 input channels: two row tiles in the filter gradient
 ]
 
 
@@ -60,11 +62,22 @@ def test_winograd_passes_against_oracle(gpu, ora, p7):
     x, w, b = _rand(N * C * H * W, 80), _rand(K * C * 9, 81, 0.2), _rand(K, 82)
     dy = _rand(N * K * cv.Ho * cv.Wo, 83)
     want_y, want_dx = ora.conv_fwd(x, w, b, *p), ora.conv_bwd_data(dy, w, *p)
+    want_dw = ora.conv_bwd_filter(dy, x, *p)
     with mode(gpu, 0):
-        direct_y, direct_dx = cv.fwd(x, w, b), cv.bwd_data(dy, w)
-        direct_bare = cv.fwd(x, w, b, False)
+        direct_y, direct_dx, direct_dw = cv.fwd(x, w, b), cv.bwd_data(dy, w), cv.bwd_filter(dy, x)
+        direct_bare, direct_bare_dw = cv.fwd(x, w, b, False), cv.bwd_filter(dy, x, False)
         direct_bytes = gpu.L.mnv_conv_fwd_workspace_bytes(*p)
     with mode(gpu, 2):
+        say("winograd bwd filter", p)
+        dw = cv.bwd_filter(dy, x)
+        assert normwise(dw, want_dw) <= TIGHT
+        assert np.any(dw.view(np.uint32) != direct_dw.view(np.uint32))
+        assert_bits_equal(cv.bwd_filter(dy, x), dw, "second call")
+        assert_bits_equal(cv.bwd_filter(dy, x, False), direct_bare_dw, "no workspace: the direct kernels")
+        if C % 16:
+            assert_bits_equal(cv.fwd(x, w, b), direct_y, "bottom channel count off 16: the direct kernels")
+            assert_bits_equal(cv.bwd_data(dy, w), direct_dx, "top channel count off 16")
+            return
         say("winograd fwd", p)
         # the size query covers the transformed tensors, and the path really ran: its bits
         # are not those of the direct kernels
@@ -116,6 +129,18 @@ def test_winograd_in_groups_of_images_has_the_same_bits(gpu, N):
         small = _wino_bytes(5, K, C, H, W) + 1024
         gpu.call("mnv_conv_bwd_data", dyb.p, dwb.p, bd.p, *p, ws.p, ctypes.c_size_t(small))
         assert_bits_equal(gpu.down(bd), whole_dx, "data gradient in groups")
+        # the filter gradient sums over the images: in groups the 16 products accumulate group
+        # by group, the same sum in another order
+        say("winograd in groups, bwd filter", p)
+        whole_dw = cv.bwd_filter(dy, x)
+        full = gpu.L.mnv_conv_bwd_filter_workspace_bytes(*p)
+        small = full - (_wino_bytes(N, C, K, H, W) - _wino_bytes(5, C, K, H, W)) + 1024
+        big = gpu.empty(small // 4 + 64)
+        fd = gpu.up(np.full(K * C * 9, np.nan, np.float32))
+        gpu.call("mnv_conv_bwd_filter", dxb.p, dyb.p, fd.p, *p, big.p, ctypes.c_size_t(small))
+        got = gpu.down(fd)
+        assert normwise(got, whole_dw.astype(np.float64)) <= 1e-5
+        assert np.any(got.view(np.uint32) != whole_dw.view(np.uint32))
 
 
 def test_winograd_fused_epilogues_have_the_bits_of_the_chain(gpu):
@@ -139,6 +164,18 @@ def test_winograd_fused_epilogues_have_the_bits_of_the_chain(gpu):
         gpu.call("mnv_conv_bwd_data_relu", dyb.p, dwb.p, dxb.p, bd.p, *p, ws.p, ctypes.c_size_t(nbytes))
         assert_bits_equal(gpu.down(bd), np.where(x > 0, cv.bwd_data(dy, w), np.float32(0)),
                           "data gradient + relu gradient")
+        say("winograd filter gradient + update", p)
+        nbytes = gpu.L.mnv_conv_bwd_filter_workspace_bytes(*p)
+        ws = gpu.empty(nbytes // 4 + 64)
+        scale = np.float32(0.0123)
+        want = w - scale * cv.bwd_filter(dy, x)
+        out = gpu.empty(w.size)
+        gpu.call("mnv_conv_bwd_filter_sgd", dxb.p, dyb.p, dwb.p, ctypes.c_float(scale), out.p, *p, ws.p,
+                 ctypes.c_size_t(nbytes))
+        assert_bits_equal(gpu.down(out), want, "filter gradient + update")
+        gpu.call("mnv_conv_bwd_filter_sgd", dxb.p, dyb.p, dwb.p, ctypes.c_float(scale), dwb.p, *p, ws.p,
+                 ctypes.c_size_t(nbytes))
+        assert_bits_equal(gpu.down(dwb), want, "filter gradient + update in place")
 
 
 def test_winograd_is_taken_by_itself_where_it_pays(gpu, ora):
@@ -182,9 +219,20 @@ def test_direct_and_winograd_agree_at_batch_256(gpu, case):
     dy = _rand(N * K * H * W, 98)
     say(name, "b256 both paths")
     with mode(gpu, 0):
-        direct_y, direct_dx = cv.fwd(x, w, b), cv.bwd_data(dy, w)
+        direct_y, direct_dx, direct_dw = cv.fwd(x, w, b), cv.bwd_data(dy, w), cv.bwd_filter(dy, x)
     with mode(gpu, 1):
         assert gpu.L.mnv_conv_fwd_workspace_bytes(*p) == _wino_bytes(N, C, K, H, W)
+        # the filter gradient's 16 products as one equal-shares launch: as many workgroups as
+        # the chip holds
+        nbytes = gpu.L.mnv_conv_bwd_filter_workspace_bytes(*p)
+        assert nbytes > _wino_bytes(N, C, K, H, W)
+        tile, ranges, wgs = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        assert gpu.L.mnv_conv_bwd_filter_plan(*p, ctypes.c_size_t(nbytes), ctypes.byref(tile),
+                                              ctypes.byref(ranges), ctypes.byref(wgs)) == 0
+        assert (tile.value, ranges.value) == (128, 1) and wgs.value >= 512
+        dw = cv.bwd_filter(dy, x)
+        assert np.any(dw.view(np.uint32) != direct_dw.view(np.uint32))
+        assert normwise(dw, direct_dw) <= TIGHT
         y, dx = cv.fwd(x, w, b), cv.bwd_data(dy, w)
         assert np.any(y.view(np.uint32) != direct_y.view(np.uint32))
         assert normwise(y, direct_y) <= TIGHT and normwise(dx, direct_dx) <= TIGHT
