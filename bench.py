@@ -7,9 +7,9 @@ One step = one forward + backward + SGD pass of the AlexNet-shaped network
 through the C++ host layer (Task -> HipDevice -> hip::<Op> -> C ABI -> HIP kernel),
 synthetic seeded inputs already resident in HBM.  `value` is images/s with one stream
 synchronisation per step; the same step with the reference device's per-operator
-synchronisation is reported beside it.  The dominant kernel (the MFMA implicit-GEMM
-filter-gradient kernel) is timed with HIP events on its own stream inside the timed
-steps and priced against the fp32 MFMA peak.  SGEMM 4096^3 and the 8192^2 elementwise add
+synchronisation is reported beside it.  The dominant kernels (the MFMA implicit-GEMM
+kernels of conv2's three passes) are timed with HIP events on their own stream inside the
+timed steps and priced against the fp32 MFMA peak; `roofline` is the slowest of the three.  SGEMM 4096^3 and the 8192^2 elementwise add
 are measured the same way and reported in the same JSON line, and the CPU oracle is
 timed on a bounded sample of the same workload on the host cores.
 
@@ -65,11 +65,20 @@ def graph_replay(rt, net, steps, warmup):
     return {"nodes": nodes, "ms_per_step": round(ms, 4), "images_per_s": round(BATCH / ms * 1e3, 1)}
 
 
-# The longest kernel of the step: conv2's filter gradient (5 x 5 filters, 229 GFLOP; conv2's
-# forward and data-gradient kernels do the same flops in about the same time, and the 3 x 3
-# layers run as shorter launches of the minimal-filtering products).  Operator names:
-# "pad:2*2 stride:1*1 conv bp filter" ...
-DOMINANT_OP = "pad:2*2 stride:1*1 conv bp filter"
+# The longest kernels of the step are conv2's three (5 x 5 filters, 229 GFLOP each, within a
+# few percent of one another; the 3 x 3 layers run as shorter launches of the minimal-filtering
+# products): all three operators carry event pairs inside the timed steps and the roofline
+# object is that of the slowest.  Operator names: "pad:2*2 stride:1*1 conv bp filter" ...
+DOMINANT_OP = "pad:2*2 stride:1*1 conv"
+DOMINANT_KERNELS = {
+    "conv ff": ("conv2 forward", "mnv_gemm_kernel<128x128x16,ConvFwd<true>> (conv2 forward) + the "
+                                 "reduction of its cut tail"),
+    "conv bp filter": ("conv2 filter gradient", "mnv_gemm_kernel<128x128x16,ConvBwdFilterFast<false,3>,"
+                                                "stream-k,2 slabs ahead> (conv2 filter gradient) + its "
+                                                "reduction"),
+    "conv bp data": ("conv2 data gradient", "mnv_gemm_kernel<128x96x16,ConvBwdData<true>> (conv2 data "
+                                            "gradient) + the reduction of its cut tail"),
+}
 
 
 def alexnet_bench(steps, warmup, dataflow=True):
@@ -231,42 +240,45 @@ def owl_net_bench(steps, warmup):
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_gemm_kernels_hbm_traffic_pmc.txt")
 
 
-def dominant_kernel_traffic():
-    """HBM bytes per launch of the dominant kernel (conv2's filter gradient), from two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB
-    per dispatch, each scaled by what the same counter reads for the 8192^2 copy kernel).
-    The figure is the one recorded in the committed summary of those runs (its line
-    "dominant kernel traffic bytes per launch: X"), so that the two cannot drift apart; None
-    when the summary is absent."""
+def dominant_kernel_traffic(tag):
+    """HBM bytes per launch of one of conv2's kernels, from two rocprofv3 --pmc runs of this
+    script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, each scaled by what the same counter
+    reads for the 8192^2 add kernel).  The figure is the one recorded in the committed summary
+    of those runs (its line "traffic bytes per launch, <tag>: X"), so that the two cannot drift
+    apart; None when the summary is absent."""
     try:
         for line in open(TRAFFIC_PROFILE):
-            if "dominant kernel traffic bytes per launch:" in line:
+            if "traffic bytes per launch, %s:" % tag in line:
                 return float(line.split(":")[1].split()[0])
-    except OSError:
+    except (OSError, ValueError, IndexError):
         pass
     return None
 
 
 def dominant_kernel_roofline(prof, steps):
-    """The filter-gradient operator of conv2 runs the 128x128 MFMA kernel
-    (mnv_gemm_kernel<128x128x16, ConvBwdFilterFast, stream-k>) followed by the reduction of its
-    shares' partial tiles; the event pair brackets both, so the figure is slightly conservative."""
-    names = [n for n in prof if n.endswith(DOMINANT_OP)]
-    launches = sum(prof[n][0] for n in names)
-    total_ms = sum(prof[n][1] for n in names)
-    if not launches:
+    """conv2's operators each run one MFMA kernel followed by the small kernel that adds the
+    partial tiles of its shares or of its cut tail; the event pair brackets both, so the
+    figures are slightly conservative.  Every one of them does conv2's 229 GFLOP."""
+    rows = []
+    for name, (launches, total_ms) in prof.items():
+        if DOMINANT_OP not in name or not launches:
+            continue
+        tag, kernel = next(v for k, v in DOMINANT_KERNELS.items() if name.endswith(k))
+        avg_ms = total_ms / launches
+        achieved = CONV_GFLOP[1] * 1e9 / (avg_ms * 1e-3) / 1e12
+        rows.append({"bound": "mfma", "kernel": kernel,
+                     "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                     "traffic": dominant_kernel_traffic(tag),
+                     "avg_launch_ms": round(avg_ms, 4), "launches": launches,
+                     "algorithmic_gflop_per_launch": CONV_GFLOP[1]})
+    if not rows:
         return None
-    gflop_per_step = CONV_GFLOP[1]
-    flops_per_launch = gflop_per_step * 1e9 * steps / launches
-    avg_ms = total_ms / launches
-    achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
-    return {"bound": "mfma",
-            "kernel": "mnv_gemm_kernel<128x128x16,ConvBwdFilterFast<false,3>,stream-k,2 slabs ahead> "
-                      "(conv2 filter gradient) + its reduction",
-            "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-            "traffic": dominant_kernel_traffic(),
-            "avg_launch_ms": round(avg_ms, 4), "launches": launches,
-            "algorithmic_gflop_per_launch": round(flops_per_launch / 1e9, 2)}
+    rows.sort(key=lambda r: -r["avg_launch_ms"])
+    top = rows[0]
+    top["conv2_other_kernels"] = [{k: r[k] for k in ("kernel", "achieved", "frac", "traffic", "avg_launch_ms")}
+                                  for r in rows[1:]]
+    return top
 
 
 def op_table(prof, steps):
@@ -714,7 +726,7 @@ def parity_report():
     cx, cw = rng.standard_normal(N * C * H * W, dtype=np.float32), rng.standard_normal(K * C * 9, dtype=np.float32) * np.float32(0.05)
     cb, cdy = rng.standard_normal(K, dtype=np.float32), rng.standard_normal(N * K * H * W, dtype=np.float32)
     dcx, dcw, dcb, dcdy = dev.upload(cx), dev.upload(cw), dev.upload(cb), dev.upload(cdy)
-    wsb = 64 << 20
+    wsb = 128 << 20
     ws = dev.empty(wsb // 4)
     z = ctypes.c_size_t(wsb)
     close("conv forward", run(lambda o: L.mnv_conv_fwd(dcx.p, dcw.p, dcb.p, o.p, *p, ws.p, z, S), N * K * H * W),
@@ -725,6 +737,18 @@ def parity_report():
           ora.conv_bwd_filter(cdy, cx, *p))
     close("conv backward bias", run(lambda o: L.mnv_conv_bwd_bias(dcdy.p, o.p, N, K, H, W, ws.p, z, S), K),
           ora.conv_bwd_bias(cdy, N, K, H, W))
+    # the same layer by minimal filtering, the way the batch-256 step runs it (at batch 4 the
+    # library would not choose it by itself)
+    L.mnv_conv_winograd_mode(2)
+    try:
+        close("conv forward, F(2x2,3x3)", run(lambda o: L.mnv_conv_fwd(dcx.p, dcw.p, dcb.p, o.p, *p, ws.p, z, S), N * K * H * W),
+              ora.conv_fwd(cx, cw, cb, *p))
+        close("conv backward data, F(2x2,3x3)", run(lambda o: L.mnv_conv_bwd_data(dcdy.p, dcw.p, o.p, *p, ws.p, z, S), N * C * H * W),
+              ora.conv_bwd_data(cdy, cw, *p))
+        close("conv backward filter, F(3x3,2x2)", run(lambda o: L.mnv_conv_bwd_filter(dcx.p, dcdy.p, o.p, *p, ws.p, z, S), K * C * 9),
+              ora.conv_bwd_filter(cdy, cx, *p))
+    finally:
+        L.mnv_conv_winograd_mode(1)
     g = (8, 16, 27, 27, 2, 2, 3, 3, 0, 0)
     px = np.round(rng.standard_normal(8 * 16 * 27 * 27) * 2).astype(np.float32)  # many ties
     pt = ora.pool_fwd(ora.POOL_MAX, px, *g)

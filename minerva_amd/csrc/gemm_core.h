@@ -124,6 +124,12 @@ struct MnvFetchMap {
 //        stores 16 bytes per lane, 512 contiguous bytes per column and instruction, instead of
 //        4 bytes per lane: a quarter of the store instructions.  Taken for products of at most
 //        MNV_STORE4_MAX_SLABS k-slabs.
+//   optional, for a product whose left operand depends on the column tile (batched products
+//   folded into the column index): static constexpr bool N_GROUPED = true;  int n_group;
+//        Tiles are then dealt m-tile by m-tile within groups of n_group consecutive column
+//        tiles (tiles_n is a multiple of n_group), so that the column tiles that read the
+//        same A panel run next to each other; without it all m-tiles of one column tile come
+//        first (the B panel is shared).  Not for stream-k launches.
 //   optional, for a store that combines the product with a value read from memory:
 //   static constexpr bool C_PRELOAD = true;
 //   bool c_preload_on() const;                   uniform: whether this launch reads
@@ -157,6 +163,14 @@ struct MnvCStore4<P, std::enable_if_t<P::C_STORE4>> {
   static constexpr bool value = true;
 };
 template <class P, class = void>
+struct MnvNGrouped {
+  static constexpr bool value = false;
+};
+template <class P>
+struct MnvNGrouped<P, std::enable_if_t<P::N_GROUPED>> {
+  static constexpr bool value = true;
+};
+template <class P, class = void>
 struct MnvCPreload {
   static constexpr bool value = false;
 };
@@ -184,6 +198,21 @@ __device__ __forceinline__ void mnv_fetch_vec(mnv_rsrc r, const unsigned (&off)[
 __device__ __forceinline__ int mnv_tile_remap(int t, int total) {
   const int per_xcd = total / 8;
   return t < per_xcd * 8 ? (t % 8) * per_xcd + t / 8 : t;
+}
+
+// Tile coordinates of the (remapped) tile index b.
+template <class P>
+__device__ __forceinline__ void mnv_tile_coords(const P& prob, int b, int tiles_m, int& tile_m,
+                                                int& tile_n) {
+  if constexpr (MnvNGrouped<P>::value) {
+    const int per = tiles_m * prob.n_group;
+    const int grp = b / per, r = b - grp * per;
+    tile_m = r / prob.n_group;
+    tile_n = grp * prob.n_group + (r - tile_m * prob.n_group);
+  } else {
+    tile_m = b % tiles_m;
+    tile_n = b / tiles_m;
+  }
 }
 
 // Tail: tiles are whole units of work, so when their number is not a multiple of the CU
@@ -294,7 +323,13 @@ __global__ __launch_bounds__(T::NT * G, PF == 2 && T::MIN_WAVES == 4 ? 3 : T::MI
     }
   }
   const int b = SK ? vb : mnv_tile_remap(vb, tiles_m * tiles_n);
-  const int tile_m = b % tiles_m, tile_n = b / tiles_m;
+  int tile_m, tile_n;
+  if constexpr (SK) {
+    tile_m = b % tiles_m;
+    tile_n = b / tiles_m;
+  } else {
+    mnv_tile_coords(prob, b, tiles_m, tile_m, tile_n);
+  }
   const int m0 = tile_m * T::BM, n0 = tile_n * T::BNU;
 
   int slab_begin = blockIdx.z * slabs_per_split;
@@ -729,7 +764,9 @@ __global__ __launch_bounds__(256) void mnv_gemm_tail_reduce_kernel(P prob,
                                                                    int tail_begin, int tail_z) {
   constexpr int TILE = T::BM * T::BNU;
   const int b = mnv_tile_remap(tail_begin + (int)blockIdx.y, tiles_m * tiles_n);
-  const int m0 = (b % tiles_m) * T::BM, n0 = (b / tiles_m) * T::BNU;
+  int tile_m, tile_n;
+  mnv_tile_coords(prob, b, tiles_m, tile_m, tile_n);
+  const int m0 = tile_m * T::BM, n0 = tile_n * T::BNU;
   const float* p = partial + (size_t)blockIdx.y * tail_z * TILE;
   for (int e = (blockIdx.x * 256 + threadIdx.x) * 4; e < TILE; e += gridDim.x * 256 * 4) {
     mnv_f4 s = *reinterpret_cast<const mnv_f4*>(p + e);

@@ -5,7 +5,7 @@ shapes under one name and only the grid tells them apart.
   python -m minerva_amd.rocprof_summary trace <dir-or-db> [--by-grid SUBSTR] [--min-share 0.0005]
       per-kernel durations of a `rocprofv3 --kernel-trace --stats` run (microseconds)
 
-  python -m minerva_amd.rocprof_summary counters <dir-or-db> [<dir-or-db> ...] [--only SUBSTR]
+  python -m minerva_amd.rocprof_summary counters <dir-or-db> [<dir-or-db> ...] [--only SUBSTR[,SUBSTR...]]
                                         [--trace <dir-or-db>] [--show COUNTER,COUNTER,...]
       per-kernel averages of every counter of one or more `rocprofv3 --pmc` runs (one counter set
       per run), plus, where their counters are present, the derived columns
@@ -85,7 +85,7 @@ def counter_rows(cons, only=""):
         q = "select kernel_name, counter_name, value, grid_size_x, grid_size_z from counters_collection"
         for name, ctr, v, x, z in con.execute(q):
             k = short(name)
-            if only and only not in k:
+            if only and not any(o in k for o in only.split(",")):
                 continue
             vals[(k, x, z)][ctr].append(v)
     return {key: {c: sum(v) / len(v) for c, v in d.items()} for key, d in vals.items()}
@@ -150,7 +150,7 @@ def main(argv=None):
     t.add_argument("--min-share", type=float, default=0.0005)
     c = sub.add_parser("counters")
     c.add_argument("db", nargs="+")
-    c.add_argument("--only", default="", help="kernel name substring")
+    c.add_argument("--only", default="", help="kernel name substring (several, separated by commas: any of them)")
     c.add_argument("--trace", default=None, help="kernel-trace run of the same command, for durations")
     c.add_argument("--show", default=None, help="comma-separated raw counters to print (default: all)")
     args = ap.parse_args(argv)
