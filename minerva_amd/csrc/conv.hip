@@ -921,7 +921,9 @@ static int conv_fwd_impl(const float* bottom, const float* filter, const float* 
   int gm = N * g.HoWo, gn = K, gk = g.CRS;
   hipStream_t s = mnv_stream(stream);
   // 3 x 3 unit-stride layers with enough channels and tiles: F(2 x 2, 3 x 3), see winograd.hip
-  if (const int images = mnv_wino_images(N, C, K, H, W, ph, pw, R, S, sv, sh, workspace ? workspace_bytes : 0))
+  // (its transformed tensors are read and written in 16-byte vectors)
+  if (const int images = mnv_wino_images(N, C, K, H, W, ph, pw, R, S, sv, sh,
+                                         workspace && mnv_aligned16(workspace) ? workspace_bytes : 0))
     return mnv_wino_conv(bottom, filter, bias, nullptr, top, N, C, K, H, W, ph, pw, 0, relu, images,
                          workspace, workspace_bytes, s);
   const int tile = pick_tile(gm, gn);
@@ -1014,7 +1016,7 @@ static int conv_bwd_data_impl(const float* top_diff, const float* filter, const 
   hipStream_t s = mnv_stream(stream);
   // the same correlation, of top_diff with the unflipped filters, under a padding of 2 - pad
   if (const int images = mnv_wino_images(N, K, C, g.Ho, g.Wo, 2 - ph, 2 - pw, R, S, sv, sh,
-                                         workspace ? workspace_bytes : 0))
+                                         workspace && mnv_aligned16(workspace) ? workspace_bytes : 0))
     return mnv_wino_conv(top_diff, filter, nullptr, gate, bottom_diff, N, K, C, g.Ho, g.Wo, 2 - ph,
                          2 - pw, 1, 0, images, workspace, workspace_bytes, s);
   const int tile = pick_tile(gm, gn);
@@ -1108,7 +1110,7 @@ static int conv_bwd_filter_impl(const float* bottom, const float* top_diff, floa
   hipStream_t s = mnv_stream(stream);
   // 3 x 3 unit-stride layers with enough channels and tiles: F(3 x 3, 2 x 2), see winograd.hip
   if (const int images = mnv_wino_grad_images(N, C, K, H, W, ph, pw, R, S, sv, sh,
-                                              workspace ? workspace_bytes : 0))
+                                              workspace && (plan || mnv_aligned16(workspace)) ? workspace_bytes : 0))
     return mnv_wino_filter_grad(bottom, top_diff, filter_diff, N, C, K, H, W, ph, pw, images,
                                 accumulate, sgd_w, sgd_scale, workspace, workspace_bytes, s, plan);
   int splits = bwd_filter_splits(gm, gn, gk, workspace ? workspace_bytes / sizeof(float) : 0);

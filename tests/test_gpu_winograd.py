@@ -96,6 +96,27 @@ def test_winograd_passes_against_oracle(gpu, ora, p7):
         assert_bits_equal(cv.fwd(x, w, b, False), direct_bare, "no workspace")
 
 
+def test_winograd_needs_a_16_byte_aligned_workspace(gpu, ora):
+    """The transformed tensors are moved in 16-byte vectors: a workspace that starts 4 bytes
+    off runs the direct kernels (same bits as with the path switched off)."""
+    p = (3, 32, 48, 9, 9, 1, 1, 1, 1, 3, 3)
+    N, C, K, H, W = p[:5]
+    cv = Conv(gpu, *p)
+    x, w, b = _rand(N * C * H * W, 70), _rand(K * C * 9, 71, 0.2), _rand(K, 72)
+    with mode(gpu, 0):
+        direct = cv.fwd(x, w, b)
+    with mode(gpu, 2):
+        nbytes = gpu.L.mnv_conv_fwd_workspace_bytes(*p)
+        ws = gpu.empty(nbytes // 4 + 64)
+        dxb, dwb, dbb, top = gpu.up(x), gpu.up(w), gpu.up(b), gpu.empty(direct.size)
+        say("winograd, workspace off the 16-byte grid", p)
+        gpu.call("mnv_conv_fwd", dxb.p, dwb.p, dbb.p, top.p, *p, ws.offset(1),
+                 ctypes.c_size_t(nbytes))
+        assert_bits_equal(gpu.down(top), direct, "unaligned workspace")
+        gpu.call("mnv_conv_fwd", dxb.p, dwb.p, dbb.p, top.p, *p, ws.p, ctypes.c_size_t(nbytes))
+        assert np.any(gpu.down(top).view(np.uint32) != direct.view(np.uint32))
+
+
 def _wino_bytes(images, C, K, Ho, Wo):
     """The workspace the path wants for `images` images at once (U, V, M from 256-byte
     boundaries; tiles rounded up to 4, output channels to 128)."""
