@@ -235,17 +235,22 @@ int mnv_softmax_channel_bwd(const float* top_diff, const float* top, float* bott
  * elements each).  A batch whose bottom or top is larger (up to 2^31 - 1 elements) runs as
  * several launches over chunks of images, the filter gradient accumulating chunk by chunk;
  * only a single image or a filter of 2^29 elements and more is refused (MNV_ERR_INVALID).
- * 3 x 3 filters at unit stride with a bottom (forward) / top (backward_data) channel count
- * that is a multiple of 16 may run by minimal filtering F(2 x 2, 3 x 3): 16 multiplies per
- * 2 x 2 outputs of a channel pair instead of 36, as 16 matrix products between transforms
- * of 4 x 4 tiles, summed in fp32; results differ from the direct sum by a few 1e-7 of the
- * output's norm.  It wants the workspace the size queries report (16 transformed values
- * per tile and channel of both tensors); with less it runs in groups of images, with less
- * than one image needs the direct kernels run. ---- */
-/* Selects when forward / backward_data take the minimal-filtering path.  0: never;
- * 1 (initial): where the geometry makes it faster (at least 32 input channels, output
- * channels that fill 128-wide tiles to three quarters, at least 1024 tiles per launch,
- * output extents whose rounding up to even wastes at most 40%); 2: wherever it applies.
+ * 3 x 3 filters at unit stride may run by minimal filtering (Winograd): F(2 x 2, 3 x 3), 16
+ * multiplies per 2 x 2 outputs of a channel pair instead of 36, or F(4 x 4, 3 x 3), 36 per 4 x 4
+ * outputs instead of 144 -- whichever needs fewer products for the plane at hand, the smaller
+ * tile on a near tie -- as 16 / 36 matrix products between transforms of 4 x 4 / 6 x 6 tiles,
+ * summed in fp32; backward_filter by F(3 x 3, 2 x 2) / F(3 x 3, 4 x 4) with the sum over the tiles
+ * as the products' reduction.  Results differ from the direct sum by a few 1e-6 of the output's
+ * norm (up to about 6e-6 with the larger tile).  forward / backward_data need a bottom / top
+ * channel count that is a multiple of 16.  The path wants the workspace the size queries
+ * report (16 / 36 transformed values per tile and channel of both tensors), 16-byte aligned;
+ * with less it runs in groups of images, with less than one image needs the direct kernels
+ * run. ---- */
+/* Selects when the three passes take the minimal-filtering path.  0: never; 1 (initial):
+ * where the geometry makes it faster (at least 32 input channels, channel counts that fill
+ * 128-wide tiles to three quarters, at least 1024 tiles of 2 x 2 or 512 of 4 x 4 outputs per
+ * launch, output extents whose rounding up to whole 2 x 2 tiles wastes at most 40%); 2:
+ * wherever it applies; 3 / 4: as 2 with the tile pinned to 2 x 2 / 4 x 4 outputs.
  * Process-wide; returns the previous mode; any other value only queries.  No reference
  * counterpart: cuDNN picks its algorithm out of sight (CUDNN_CONVOLUTION_FWD_PREFER_FASTEST,
  * cuda_perform.cu:227-264). */

@@ -1,5 +1,5 @@
-// 3 x 3 unit-stride convolutions by F(2 x 2, 3 x 3) minimal filtering (winograd.hip), as the
-// convolution entry points of conv.hip call it.
+// 3 x 3 unit-stride convolutions by minimal filtering, F(2 x 2, 3 x 3) or F(4 x 4, 3 x 3)
+// (winograd.hip), as the convolution entry points of conv.hip call it.
 #pragma once
 #include "mnv_common.h"
 
@@ -25,8 +25,8 @@ int mnv_wino_conv(const float* src, const float* filter, const float* bias, cons
                   int transposed, int relu, int images, void* workspace, size_t workspace_bytes,
                   hipStream_t s);
 
-// The filter gradient of the same layers by F(3 x 3, 2 x 2): the sum over images and tiles is the
-// reduction dimension of the 16 products, which run as one equal-shares launch of the MFMA
+// The filter gradient of the same layers by F(3 x 3, 2 x 2) / F(3 x 3, 4 x 4): the sum over images and tiles is the
+// reduction dimension of the products, which run as one equal-shares launch of the MFMA
 // core.  (C, H, W): bottom; K: channels of top_diff; (ph, pw): the layer's padding.
 // mnv_wino_grad_images as mnv_wino_images (no condition on the channel counts' divisors);
 // with more than one group the products accumulate group by group.

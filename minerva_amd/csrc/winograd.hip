@@ -1,51 +1,160 @@
-// 3 x 3, unit-stride convolutions by the minimal-filtering algorithm F(2 x 2, 3 x 3)
-// (Winograd): every 2 x 2 block of outputs of one channel pair costs 16 multiplies instead
-// of 36.  The work becomes 16 independent matrix products, one per point (xi, nu) of the
-// transformed 4 x 4 tile,
+// 3 x 3, unit-stride convolutions by minimal filtering (Winograd): an m x m block of outputs
+// of one channel pair costs (m + 2)^2 multiplies instead of 9 m^2.  Two tile sizes:
+//   F(2 x 2, 3 x 3): 4 x 4 input tiles at stride 2, 16 points, 16 multiplies per 4 outputs;
+//   F(4 x 4, 3 x 3): 6 x 6 input tiles at stride 4, 36 points, 36 multiplies per 16 outputs,
+// the second taken when it needs clearly fewer products for the plane at hand (13 x 13 outputs:
+// 4 x 4 tiles x 36 = 576 against 7 x 7 x 16 = 784).  The work becomes al^2 independent matrix
+// products, one per point (xi, nu) of the transformed al x al tile (al = m + 2),
 //     M[xi,nu][co][p] = sum_ci U[xi,nu][co][ci] * V[xi,nu][ci][p],      p = (image, tile row, tile col)
-// with U = G g G^T (filters), V = B^T d B (4 x 4 input tiles, stride 2) and the outputs
-// Y = A^T M A.  The 16 products run as ONE launch of the fp32 MFMA core (gemm_core.h): the
-// transform point is folded into the column index, n = point * Coutp + co, and a workgroup
-// picks the V panel of its point once, in block_init.  Semantics are those of conv.hip: the
-// forward pass correlates with the flipped filter (cuDNN's CUDNN_CONVOLUTION as selected at
-// minerva/op/impl/cuda/cuda_perform.cu:227-264), the data gradient (cuda_perform.cu:266-291)
-// is the same correlation of top_diff with the unflipped filter, channels exchanged, under a
-// padding of 2 - pad.
+// with U = G g G^T (filters), V = B^T d B (input tiles) and the outputs Y = A^T M A.  The
+// products run as ONE launch of the fp32 MFMA core (gemm_core.h): the point is folded into the
+// column index, n = point * Coutp + co, and a workgroup picks the V panel of its point once, in
+// block_init.  Semantics are those of conv.hip: the forward pass correlates with the flipped
+// filter (cuDNN's CUDNN_CONVOLUTION as selected at minerva/op/impl/cuda/cuda_perform.cu:227-264),
+// the data gradient (cuda_perform.cu:266-291) is the same correlation of top_diff with the
+// unflipped filter, channels exchanged, under a padding of 2 - pad.  The filter gradient
+// (cuda_perform.cu:293-318) is F(3 x 3, m x m) on the same points: the m x m tiles of top_diff
+// take the filter's place, Yt = G' dy G'^T, the sum over images and tiles is the reduction
+// dimension of the products Q[xi,nu][k][c] = sum_p Yt[xi,nu][k][p] V[xi,nu][c][p], and the
+// gradient is A'^T Q A'.
 //
-//   B^T = | 1  0 -1  0 |   G = | 1    0    0  |   A^T = | 1  1  1  0 |
-//         | 0  1  1  0 |       | 1/2  1/2  1/2|         | 0  1 -1 -1 |
-//         | 0 -1  1  0 |       | 1/2 -1/2  1/2|
-//         | 0  1  0 -1 |       | 0    0    1  |
+// The matrices are those of the Toom-Cook construction on the points {0, 1, -1, inf} (al = 4)
+// and {0, 1, -1, 2, -1/2, inf} (al = 6): B^T depends on the points alone and serves all three
+// passes.  al = 4 (G and G' carry the halves):
+//   B^T = | 1  0 -1  0 |   G = | 1    0    0  |   A^T = | 1  1  1  0 |   G' = | 1    0  |   A'^T = | 1  1  1  0 |
+//         | 0  1  1  0 |       | 1/2  1/2  1/2|         | 0  1 -1 -1 |        | 1/2  1/2|          | 0  1 -1  0 |
+//         | 0 -1  1  0 |       | 1/2 -1/2  1/2|                              | 1/2 -1/2|          | 0  1  1 -1 |
+//         | 0  1  0 -1 |       | 0    0    1  |                              | 0    1  |
+// al = 6: see WinoF<6> below (G, G', A^T, A'^T are powers of the points, exact in fp32; B^T
+// carries the fractions).
 //
-// Rounding: the transforms add and halve, the products are summed in fp32 over Cin; the
-// result differs from the direct sum by a few 1e-7 of the output's norm.
-// Roofline: the matrix products are MFMA-bound (2 * 16 * Cout * Cin * tiles flops, 4 / 9 of
-// the direct flops when the output extents are even); the three transform kernels stream
-// 16 * 4 bytes per (channel, tile) and are HBM-bound.
+// Rounding: the transforms are short sums with small constants, the products are summed in
+// fp32 in k order; against the direct sum the results differ by a few 1e-6 of the output's
+// norm (al = 4) and up to about 1e-5 (al = 6); the bound of the convolutions is 1e-4.
+// Roofline: the matrix products are MFMA-bound (2 * al^2 * Cout * Cin * tiles flops); the
+// transform kernels stream al^2 * 4 bytes per (channel, tile) and are HBM-bound.
 
 #include "gemm_core.h"
 #include "winograd.h"
 
 namespace {
 
-// Channels per workgroup of the LDS-staged input transform.  Four channels per workgroup (the
-// tile arithmetic done once for four) measured no faster than one: 84.7 against 79.6 us for
-// 384 channels of 256 x 13 x 13.
-#define WINO_CH 1
-
 struct WinoGeom {
   int N, Cin, Cout, Coutp;  // Coutp: Cout rounded up to the tile width of the product
   int Hs, Ws, Hd, Wd;       // source and destination planes
-  int pad_h, pad_w;         // of the correlation: d[a][b] = src[2 th - pad_h + a][2 tw - pad_w + b]
+  int pad_h, pad_w;         // of the correlation: d[a][b] = src[m th - pad_h + a][m tw - pad_w + b]
+  int al, m;                // points per dimension (4 or 6), outputs per tile and dimension (al - 2)
   int TH, TW, P, Pp;        // tiles per plane, tiles in all, P rounded up to 4
   MnvFastDiv d_T, d_TW, d_Cin;
 };
 
+// The matrices of one tile size as compile-time functions, so that the unrolled transforms
+// below fold every coefficient (zeros cost nothing, +-1 no multiply).
+template <int AL>
+struct WinoF;
+template <>
+struct WinoF<4> {
+  struct BT { static constexpr int R = 4, C = 4;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[4][4] = {{1, 0, -1, 0}, {0, 1, 1, 0}, {0, -1, 1, 0}, {0, 1, 0, -1}};
+      return t[i][j]; } };
+  struct G { static constexpr int R = 4, C = 3;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[4][3] = {{1, 0, 0}, {.5f, .5f, .5f}, {.5f, -.5f, .5f}, {0, 0, 1}};
+      return t[i][j]; } };
+  struct AT { static constexpr int R = 2, C = 4;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[2][4] = {{1, 1, 1, 0}, {0, 1, -1, -1}};
+      return t[i][j]; } };
+  struct GG { static constexpr int R = 4, C = 2;  // G'
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[4][2] = {{1, 0}, {.5f, .5f}, {.5f, -.5f}, {0, 1}};
+      return t[i][j]; } };
+  struct AAT { static constexpr int R = 3, C = 4;  // A'^T
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[3][4] = {{1, 1, 1, 0}, {0, 1, -1, 0}, {0, 1, 1, -1}};
+      return t[i][j]; } };
+};
+template <>
+struct WinoF<6> {
+  struct BT { static constexpr int R = 6, C = 6;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[6][6] = {{1, 1.5f, -2, -1.5f, 1, 0},
+                                 {0, 1.f / 3, 5.f / 6, 1.f / 6, -1.f / 3, 0},
+                                 {0, 1.f / 3, 1.f / 6, -5.f / 6, 1.f / 3, 0},
+                                 {0, -1.f / 30, -1.f / 15, 1.f / 30, 1.f / 15, 0},
+                                 {0, -32.f / 15, 16.f / 15, 32.f / 15, -16.f / 15, 0},
+                                 {0, 1, 1.5f, -2, -1.5f, 1}};
+      return t[i][j]; } };
+  struct G { static constexpr int R = 6, C = 3;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[6][3] = {{1, 0, 0}, {1, 1, 1}, {1, -1, 1}, {1, 2, 4}, {1, -.5f, .25f}, {0, 0, 1}};
+      return t[i][j]; } };
+  struct AT { static constexpr int R = 4, C = 6;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[4][6] = {{1, 1, 1, 1, 1, 0}, {0, 1, -1, 2, -.5f, 0}, {0, 1, 1, 4, .25f, 0},
+                                 {0, 1, -1, 8, -.125f, 1}};
+      return t[i][j]; } };
+  struct GG { static constexpr int R = 6, C = 4;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[6][4] = {{1, 0, 0, 0}, {1, 1, 1, 1}, {1, -1, 1, -1}, {1, 2, 4, 8},
+                                 {1, -.5f, .25f, -.125f}, {0, 0, 0, 1}};
+      return t[i][j]; } };
+  struct AAT { static constexpr int R = 3, C = 6;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[3][6] = {{1, 1, 1, 1, 1, 0}, {0, 1, -1, 2, -.5f, 0}, {0, 1, 1, 4, .25f, 1}};
+      return t[i][j]; } };
+};
+
+// out = L in (rows) and out = in L^T (columns), fully unrolled with the coefficients folded.
+template <class L, int K>
+__device__ __forceinline__ void wino_rows(const float (&in)[L::C][K], float (&out)[L::R][K]) {
+#pragma unroll
+  for (int i = 0; i < L::R; ++i)
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      float acc = 0.f;
+      bool any = false;
+#pragma unroll
+      for (int j = 0; j < L::C; ++j) {
+        const float c = L::at(i, j);
+        if (c != 0.f) {
+          const float t = c == 1.f ? in[j][k] : c == -1.f ? -in[j][k] : c * in[j][k];
+          acc = any ? acc + t : t;
+          any = true;
+        }
+      }
+      out[i][k] = acc;
+    }
+}
+template <class L, int K>
+__device__ __forceinline__ void wino_cols(const float (&in)[K][L::C], float (&out)[K][L::R]) {
+#pragma unroll
+  for (int k = 0; k < K; ++k)
+#pragma unroll
+    for (int i = 0; i < L::R; ++i) {
+      float acc = 0.f;
+      bool any = false;
+#pragma unroll
+      for (int j = 0; j < L::C; ++j) {
+        const float c = L::at(i, j);
+        if (c != 0.f) {
+          const float t = c == 1.f ? in[k][j] : c == -1.f ? -in[k][j] : c * in[k][j];
+          acc = any ? acc + t : t;
+          any = true;
+        }
+      }
+      out[k][i] = acc;
+    }
+}
+
 // U[point][co][ci] from filter[k][c][3][3].  Forward: co = k, ci = c, g[r][s] = f[2-r][2-s];
 // data gradient (`transposed`): co = c, ci = k, g = f.  Rows co >= Cout are zero.
+template <int AL>
 __global__ __launch_bounds__(256) void mnv_wino_filter_kernel(const float* __restrict__ filter,
                                                               float* __restrict__ U, WinoGeom g,
                                                               int K, int C, bool transposed) {
+  typedef WinoF<AL> F;
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= g.Coutp * g.Cin) return;
   const int co = mnv_fastdiv(t, g.d_Cin), ci = t - co * g.Cin;
@@ -62,178 +171,137 @@ __global__ __launch_bounds__(256) void mnv_wino_filter_kernel(const float* __res
 #pragma unroll
       for (int s = 0; s < 3; ++s) f[r][s] = 0.f;
   }
-  float h[4][3];
-#pragma unroll
-  for (int s = 0; s < 3; ++s) {
-    h[0][s] = f[0][s];
-    h[1][s] = 0.5f * (f[0][s] + f[1][s] + f[2][s]);
-    h[2][s] = 0.5f * (f[0][s] - f[1][s] + f[2][s]);
-    h[3][s] = f[2][s];
-  }
+  float h[AL][3], u[AL][AL];
+  wino_rows<typename F::G, 3>(f, h);
+  wino_cols<typename F::G, AL>(h, u);
   const size_t plane = (size_t)g.Coutp * g.Cin;
   float* out = U + (size_t)co * g.Cin + ci;
 #pragma unroll
-  for (int xi = 0; xi < 4; ++xi) {
-    out[(xi * 4 + 0) * plane] = h[xi][0];
-    out[(xi * 4 + 1) * plane] = 0.5f * (h[xi][0] + h[xi][1] + h[xi][2]);
-    out[(xi * 4 + 2) * plane] = 0.5f * (h[xi][0] - h[xi][1] + h[xi][2]);
-    out[(xi * 4 + 3) * plane] = h[xi][2];
-  }
+  for (int xi = 0; xi < AL; ++xi)
+#pragma unroll
+    for (int nu = 0; nu < AL; ++nu) out[(xi * AL + nu) * plane] = u[xi][nu];
 }
 
-// V[point][ci][p] = (B^T d B)[point] of the 4 x 4 tile p of channel ci; p >= P writes zeros.
+// V[point][ci][p] = (B^T d B)[point] of the al x al tile p of channel ci; p >= P writes zeros.
+template <int AL>
+__device__ __forceinline__ void wino_store_v(float (&d)[AL][AL], float* __restrict__ out, size_t plane) {
+  typedef WinoF<AL> F;
+  float h[AL][AL], v[AL][AL];
+  wino_rows<typename F::BT, AL>(d, h);
+  wino_cols<typename F::BT, AL>(h, v);
+#pragma unroll
+  for (int xi = 0; xi < AL; ++xi)
+#pragma unroll
+    for (int nu = 0; nu < AL; ++nu) out[(xi * AL + nu) * plane] = v[xi][nu];
+}
+
+template <int AL>
 __global__ __launch_bounds__(256) void mnv_wino_input_kernel(const float* __restrict__ src,
                                                              float* __restrict__ V, WinoGeom g) {
   const int p = blockIdx.x * 256 + threadIdx.x;
   const int ci = blockIdx.y;
   if (p >= g.Pp) return;
-  float d[4][4];
+  float d[AL][AL];
+#pragma unroll
+  for (int a = 0; a < AL; ++a)
+#pragma unroll
+    for (int b = 0; b < AL; ++b) d[a][b] = 0.f;
   if (p < g.P) {
     const int img = mnv_fastdiv(p, g.d_T);
     const int t = p - img * (g.TH * g.TW);
     const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
-    const int y0 = 2 * th - g.pad_h, x0 = 2 * tw - g.pad_w;
+    const int y0 = (AL - 2) * th - g.pad_h, x0 = (AL - 2) * tw - g.pad_w;
     const float* plane = src + ((size_t)img * g.Cin + ci) * (g.Hs * g.Ws);
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < AL; ++a)
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
+      for (int b = 0; b < AL; ++b) {
         const int y = y0 + a, x = x0 + b;
-        d[a][b] = ((unsigned)y < (unsigned)g.Hs && (unsigned)x < (unsigned)g.Ws) ? plane[y * g.Ws + x] : 0.f;
+        if ((unsigned)y < (unsigned)g.Hs && (unsigned)x < (unsigned)g.Ws) d[a][b] = plane[y * g.Ws + x];
       }
-  } else {
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-#pragma unroll
-      for (int b = 0; b < 4; ++b) d[a][b] = 0.f;
   }
-  float h[4][4];
-#pragma unroll
-  for (int b = 0; b < 4; ++b) {
-    h[0][b] = d[0][b] - d[2][b];
-    h[1][b] = d[1][b] + d[2][b];
-    h[2][b] = d[2][b] - d[1][b];
-    h[3][b] = d[1][b] - d[3][b];
-  }
-  const size_t plane = (size_t)g.Cin * g.Pp;
-  float* out = V + (size_t)ci * g.Pp + p;
-#pragma unroll
-  for (int xi = 0; xi < 4; ++xi) {
-    out[(xi * 4 + 0) * plane] = h[xi][0] - h[xi][2];
-    out[(xi * 4 + 1) * plane] = h[xi][1] + h[xi][2];
-    out[(xi * 4 + 2) * plane] = h[xi][2] - h[xi][1];
-    out[(xi * 4 + 3) * plane] = h[xi][1] - h[xi][3];
-  }
+  wino_store_v<AL>(d, V + (size_t)ci * g.Pp + p, (size_t)g.Cin * g.Pp);
 }
 
 // The same through LDS, for planes small enough that the planes of the images a workgroup's
 // 256 tiles belong to fit there: they are fetched whole, in runs of contiguous floats (a
-// plane of 13 x 13 is 676 contiguous bytes), where the kernel above gathers 16 values per
-// thread at a stride of 8 bytes between neighbouring tiles.
+// plane of 13 x 13 is 676 contiguous bytes), where the kernel above gathers al^2 values per
+// thread at a stride of a few bytes between neighbouring tiles (F(2 x 2) on 384 channels of
+// 256 x 13 x 13: 107 -> 80 us).  One channel per workgroup: four (the tile arithmetic done once
+// for four) measured 84.7 against 79.6 us.
+template <int AL>
 __global__ __launch_bounds__(256) void mnv_wino_input_lds_kernel(const float* __restrict__ src,
                                                                  float* __restrict__ V, WinoGeom g,
                                                                  MnvFastDiv d_HW) {
   extern __shared__ float planes[];
   const int p0 = blockIdx.x * 256, p = p0 + threadIdx.x;
-  const int c0 = blockIdx.y * WINO_CH;
-  const int nch = g.Cin - c0 < WINO_CH ? g.Cin - c0 : WINO_CH;
+  const int ci = blockIdx.y;
   const int HW = g.Hs * g.Ws;
   const int img0 = mnv_fastdiv(p0, g.d_T);
   const int last = p0 + 255 < g.P ? p0 + 255 : g.P - 1;
-  const int count = (last >= p0 ? mnv_fastdiv(last, g.d_T) - img0 + 1 : 0) * HW;  // per channel
+  const int count = (last >= p0 ? mnv_fastdiv(last, g.d_T) - img0 + 1 : 0) * HW;
   for (int i = threadIdx.x; i < count; i += 256) {
     const int pl = mnv_fastdiv(i, d_HW);
-    const float* at = src + ((size_t)(img0 + pl) * g.Cin + c0) * HW + (i - pl * HW);
-#pragma unroll
-    for (int cc = 0; cc < WINO_CH; ++cc)
-      if (cc < nch) planes[cc * count + i] = at[(size_t)cc * HW];
+    planes[i] = src[((size_t)(img0 + pl) * g.Cin + ci) * HW + (i - pl * HW)];
   }
   __syncthreads();
   if (p >= g.Pp) return;
-  int at[4][4];  // LDS index of every tile element of this thread's tile, -1: reads as zero
+  float d[AL][AL];
 #pragma unroll
-  for (int a = 0; a < 4; ++a)
+  for (int a = 0; a < AL; ++a)
 #pragma unroll
-    for (int b = 0; b < 4; ++b) at[a][b] = -1;
+    for (int b = 0; b < AL; ++b) d[a][b] = 0.f;
   if (p < g.P) {
     const int img = mnv_fastdiv(p, g.d_T);
     const int t = p - img * (g.TH * g.TW);
     const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
-    const int y0 = 2 * th - g.pad_h, x0 = 2 * tw - g.pad_w;
+    const int y0 = (AL - 2) * th - g.pad_h, x0 = (AL - 2) * tw - g.pad_w;
+    const float* plane = planes + (img - img0) * HW;
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < AL; ++a)
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
+      for (int b = 0; b < AL; ++b) {
         const int y = y0 + a, x = x0 + b;
-        if ((unsigned)y < (unsigned)g.Hs && (unsigned)x < (unsigned)g.Ws)
-          at[a][b] = (img - img0) * HW + y * g.Ws + x;
+        if ((unsigned)y < (unsigned)g.Hs && (unsigned)x < (unsigned)g.Ws) d[a][b] = plane[y * g.Ws + x];
       }
   }
-  const size_t plane = (size_t)g.Cin * g.Pp;
-  for (int cc = 0; cc < nch; ++cc) {
-    const float* pl = planes + cc * count;
-    float h[4][4];
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      float d[4];
-#pragma unroll
-      for (int a = 0; a < 4; ++a) d[a] = at[a][b] >= 0 ? pl[at[a][b]] : 0.f;
-      h[0][b] = d[0] - d[2];
-      h[1][b] = d[1] + d[2];
-      h[2][b] = d[2] - d[1];
-      h[3][b] = d[1] - d[3];
-    }
-    float* out = V + (size_t)(c0 + cc) * g.Pp + p;
-#pragma unroll
-    for (int xi = 0; xi < 4; ++xi) {
-      out[(xi * 4 + 0) * plane] = h[xi][0] - h[xi][2];
-      out[(xi * 4 + 1) * plane] = h[xi][1] + h[xi][2];
-      out[(xi * 4 + 2) * plane] = h[xi][2] - h[xi][1];
-      out[(xi * 4 + 3) * plane] = h[xi][1] - h[xi][3];
-    }
-  }
+  wino_store_v<AL>(d, V + (size_t)ci * g.Pp + p, (size_t)g.Cin * g.Pp);
 }
 
-// dst[img][co][2 th + a][2 tw + b] = (A^T M A)[a][b] (+ bias[co]) (then max(., 0)) (then kept
+// dst[img][co][m th + a][m tw + b] = (A^T M A)[a][b] (+ bias[co]) (then max(., 0)) (then kept
 // only where gate > 0): the epilogues of the direct kernels, each the single operation of the
 // separate operator.
+template <int AL>
 __global__ __launch_bounds__(256) void mnv_wino_output_kernel(const float* __restrict__ Mx,
                                                               const float* __restrict__ bias,
                                                               const float* __restrict__ gate,
                                                               float* __restrict__ dst, WinoGeom g,
                                                               int relu) {
+  typedef WinoF<AL> F;
+  constexpr int MO = AL - 2;
   const int p = blockIdx.x * 256 + threadIdx.x;
   const int co = blockIdx.y;
   if (p >= g.P) return;
   const size_t plane = (size_t)g.Coutp * g.Pp;
   const float* in = Mx + (size_t)co * g.Pp + p;
-  float m[4][4];
+  float mm[AL][AL];
 #pragma unroll
-  for (int xi = 0; xi < 4; ++xi)
+  for (int xi = 0; xi < AL; ++xi)
 #pragma unroll
-    for (int nu = 0; nu < 4; ++nu) m[xi][nu] = in[(xi * 4 + nu) * plane];
-  float h[2][4];
-#pragma unroll
-  for (int nu = 0; nu < 4; ++nu) {
-    h[0][nu] = m[0][nu] + m[1][nu] + m[2][nu];
-    h[1][nu] = m[1][nu] - m[2][nu] - m[3][nu];
-  }
-  float y[2][2];
-#pragma unroll
-  for (int a = 0; a < 2; ++a) {
-    y[a][0] = h[a][0] + h[a][1] + h[a][2];
-    y[a][1] = h[a][1] - h[a][2] - h[a][3];
-  }
+    for (int nu = 0; nu < AL; ++nu) mm[xi][nu] = in[(xi * AL + nu) * plane];
+  float h[MO][AL], y[MO][MO];
+  wino_rows<typename F::AT, AL>(mm, h);
+  wino_cols<typename F::AT, MO>(h, y);
   const int img = mnv_fastdiv(p, g.d_T);
   const int t = p - img * (g.TH * g.TW);
   const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
   const float b = bias ? bias[co] : 0.f;
   const size_t base = ((size_t)img * g.Cout + co) * (g.Hd * g.Wd);
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < MO; ++a)
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-      const int yy = 2 * th + a, xx = 2 * tw + c;
+    for (int c = 0; c < MO; ++c) {
+      const int yy = MO * th + a, xx = MO * tw + c;
       if (yy < g.Hd && xx < g.Wd) {
         float v = y[a][c];
         if (bias) v = v + b;
@@ -245,7 +313,7 @@ __global__ __launch_bounds__(256) void mnv_wino_output_kernel(const float* __res
     }
 }
 
-// The 16 products as one: C{Pp, 16 Coutp} = A{Pp, Cin} B{Cin, 16 Coutp}, column-major, where the
+// The products of all points as one: C{Pp, points Coutp} = A{Pp, Cin} B{Cin, points Coutp}, column-major, where the
 // A of a column tile is the V panel of the tile's transform point.
 struct WinoGemm {
   static constexpr bool A_KFAST = false, B_KFAST = true;
@@ -253,7 +321,7 @@ struct WinoGemm {
   const float* __restrict__ V;
   const float* __restrict__ U;
   float* __restrict__ Mx;
-  int M, N, K, total_slabs, spp;  // Pp, 16 Coutp, Cin
+  int M, N, K, total_slabs, spp;  // Pp, points * Coutp, Cin
   int coutp;
   int n_group;  // column tiles per transform point: they read the same V panel
   static constexpr bool N_GROUPED = true;
@@ -296,95 +364,82 @@ struct WinoGemm {
   }
 };
 
-// ---- filter gradient: F(3 x 3, 2 x 2), the same four points
-//   dg[k][c] = sum_p A'^T [ (G' dy_p G'^T) (.) (B^T d_p B) ] A'      dy_p: the 2 x 2 tile p of top_diff
-//   A'^T = | 1  1  1  0 |   G' = | 1    0  |
-//          | 0  1 -1  0 |        | 1/2  1/2|
-//          | 0  1  1 -1 |        | 1/2 -1/2|
-//                                | 0    1  |
-// The sum over the tiles is the k dimension of the 16 products Q[point][k][c] =
-// sum_p Yt[point][k][p] V[point][c][p].
-
-// Yt[point][k][p] = (G' dy G'^T)[point] of the 2 x 2 tile p of channel k of top_diff; zeros
+// ---- filter gradient
+// Yt[point][k][p] = (G' dy G'^T)[point] of the m x m tile p of channel k of top_diff; zeros
 // for p >= P and for the rows k >= Cout.
+template <int AL>
 __global__ __launch_bounds__(256) void mnv_wino_grad_kernel(const float* __restrict__ top_diff,
                                                             float* __restrict__ Yt, WinoGeom g) {
+  typedef WinoF<AL> F;
+  constexpr int MO = AL - 2;
   const int p = blockIdx.x * 256 + threadIdx.x;
   const int k = blockIdx.y;
   if (p >= g.Pp) return;
-  float d[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+  float d[MO][MO];
+#pragma unroll
+  for (int a = 0; a < MO; ++a)
+#pragma unroll
+    for (int b = 0; b < MO; ++b) d[a][b] = 0.f;
   if (p < g.P && k < g.Cout) {
     const int img = mnv_fastdiv(p, g.d_T);
     const int t = p - img * (g.TH * g.TW);
     const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
     const float* plane = top_diff + ((size_t)img * g.Cout + k) * (g.Hd * g.Wd);
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < MO; ++a)
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const int y = 2 * th + a, x = 2 * tw + b;
+      for (int b = 0; b < MO; ++b) {
+        const int y = MO * th + a, x = MO * tw + b;
         if (y < g.Hd && x < g.Wd) d[a][b] = plane[y * g.Wd + x];
       }
   }
-  float h[4][2];
-#pragma unroll
-  for (int b = 0; b < 2; ++b) {
-    h[0][b] = d[0][b];
-    h[1][b] = 0.5f * (d[0][b] + d[1][b]);
-    h[2][b] = 0.5f * (d[0][b] - d[1][b]);
-    h[3][b] = d[1][b];
-  }
+  float h[AL][MO], v[AL][AL];
+  wino_rows<typename F::GG, MO>(d, h);
+  wino_cols<typename F::GG, AL>(h, v);
   const size_t plane = (size_t)g.Coutp * g.Pp;
   float* out = Yt + (size_t)k * g.Pp + p;
 #pragma unroll
-  for (int xi = 0; xi < 4; ++xi) {
-    out[(xi * 4 + 0) * plane] = h[xi][0];
-    out[(xi * 4 + 1) * plane] = 0.5f * (h[xi][0] + h[xi][1]);
-    out[(xi * 4 + 2) * plane] = 0.5f * (h[xi][0] - h[xi][1]);
-    out[(xi * 4 + 3) * plane] = h[xi][1];
-  }
+  for (int xi = 0; xi < AL; ++xi)
+#pragma unroll
+    for (int nu = 0; nu < AL; ++nu) out[(xi * AL + nu) * plane] = v[xi][nu];
 }
 
 // filter_diff[k][c][2-r][2-s] = (A'^T Q A')[r][s] with the epilogues of the direct kernel's
 // store: the parameter update sgd_w - sgd_scale * ., or the sum with what is there.
 // (filter_diff may be sgd_w itself: a thread reads the nine parameters it then writes.)
+template <int AL>
 __global__ __launch_bounds__(256) void mnv_wino_grad_output_kernel(const float* __restrict__ Q,
                                                                    float* filter_diff, WinoGeom g,
                                                                    int accumulate, const float* sgd_w,
                                                                    float sgd_scale) {
+  typedef WinoF<AL> F;
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= g.Cout * g.Cin) return;
   const int k = mnv_fastdiv(t, g.d_Cin), c = t - k * g.Cin;
   const size_t plane = (size_t)g.Coutp * g.Cin;
   const float* in = Q + (size_t)k * g.Cin + c;
-  float q[4][4];
+  float q[AL][AL];
 #pragma unroll
-  for (int xi = 0; xi < 4; ++xi)
+  for (int xi = 0; xi < AL; ++xi)
 #pragma unroll
-    for (int nu = 0; nu < 4; ++nu) q[xi][nu] = in[(xi * 4 + nu) * plane];
-  float h[3][4];
-#pragma unroll
-  for (int nu = 0; nu < 4; ++nu) {
-    h[0][nu] = q[0][nu] + q[1][nu] + q[2][nu];
-    h[1][nu] = q[1][nu] - q[2][nu];
-    h[2][nu] = q[1][nu] + q[2][nu] - q[3][nu];
-  }
+    for (int nu = 0; nu < AL; ++nu) q[xi][nu] = in[(xi * AL + nu) * plane];
+  float h[3][AL], dg[3][3];
+  wino_rows<typename F::AAT, AL>(q, h);
+  wino_cols<typename F::AAT, 3>(h, dg);
   float* out = filter_diff + (size_t)t * 9;
 #pragma unroll
-  for (int r = 0; r < 3; ++r) {
-    const float dg[3] = {h[r][0] + h[r][1] + h[r][2], h[r][1] - h[r][2], h[r][1] + h[r][2] - h[r][3]};
+  for (int r = 0; r < 3; ++r)
 #pragma unroll
     for (int s = 0; s < 3; ++s) {
       const int at = (2 - r) * 3 + (2 - s);
-      float x = dg[s];
+      float x = dg[r][s];
       if (sgd_w) x = sgd_w[(size_t)t * 9 + at] - sgd_scale * x;
       else if (accumulate) x = out[at] + x;
       out[at] = x;
     }
-  }
 }
 
-// The 16 products of the filter gradient as one: C{Cin, 16 Coutp} = A{Cin, Pp} B{Pp, 16 Coutp},
+// The products of the filter gradient as one: C{Cin, points Coutp} = A{Cin, Pp} B{Pp, points Coutp},
 // both operands with the reduction index p contiguous; the A of a column tile is the V panel
 // of the tile's transform point.
 struct WinoGradGemm {
@@ -393,7 +448,7 @@ struct WinoGradGemm {
   const float* __restrict__ V;
   const float* __restrict__ Yt;
   float* __restrict__ Q;
-  int M, N, K, total_slabs, spp;  // Cin, 16 Coutp, Pp
+  int M, N, K, total_slabs, spp;  // Cin, points * Coutp, Pp
   int coutp, accumulate;
   struct Res {
     mnv_rsrc a, b;
@@ -436,19 +491,36 @@ typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 
 inline size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
 
-int make_wino_geom(WinoGeom* g, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w) {
+// Mode of mnv_conv_winograd_mode: 0 never, 1 where it pays, 2 wherever it applies, 3 / 4 as 2
+// with the tile size pinned to F(2 x 2) / F(4 x 4).
+std::atomic<int> g_mode{1};
+
+// Points per dimension for an Hd x Wd output plane: 6 (4 x 4 outputs per tile) when that needs
+// at most 85% of the products of 4 (2 x 2 outputs per tile); its results are a few times
+// further from the direct sum, so a near tie goes to the smaller tile.
+int pick_points(int Hd, int Wd, int mode) {
+  if (mode == 3) return 4;
+  if (mode == 4) return 6;
+  const long long small = 16LL * ((Hd + 1) / 2) * ((Wd + 1) / 2);
+  const long long large = 36LL * ((Hd + 3) / 4) * ((Wd + 3) / 4);
+  return large * 100 <= small * 85 ? 6 : 4;
+}
+
+int make_wino_geom(WinoGeom* g, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w,
+                   int al) {
   if (N <= 0 || Cin <= 0 || Cout <= 0 || Hs <= 0 || Ws <= 0 || pad_h < 0 || pad_w < 0 || pad_h > 2 ||
-      pad_w > 2 || Hs + 2 * pad_h < 3 || Ws + 2 * pad_w < 3)
+      pad_w > 2 || Hs + 2 * pad_h < 3 || Ws + 2 * pad_w < 3 || (al != 4 && al != 6))
     return MNV_ERR_INVALID;
   g->N = N; g->Cin = Cin; g->Cout = Cout; g->Coutp = (Cout + 127) / 128 * 128;
   g->Hs = Hs; g->Ws = Ws; g->Hd = Hs + 2 * pad_h - 2; g->Wd = Ws + 2 * pad_w - 2;
   g->pad_h = pad_h; g->pad_w = pad_w;
-  g->TH = (g->Hd + 1) / 2; g->TW = (g->Wd + 1) / 2;
+  g->al = al; g->m = al - 2;
+  g->TH = (g->Hd + g->m - 1) / g->m; g->TW = (g->Wd + g->m - 1) / g->m;
   const long long P = (long long)N * g->TH * g->TW;
   if (P > (1LL << 28)) return MNV_ERR_INVALID;
   g->P = (int)P; g->Pp = (int)((P + 3) / 4 * 4);
   // a V panel and U are read through 32-bit byte offsets
-  if ((long long)Cin * g->Pp > (1LL << 29) - 1 || 16LL * g->Coutp * Cin > (1LL << 29) - 1)
+  if ((long long)Cin * g->Pp > (1LL << 29) - 1 || (long long)al * al * g->Coutp * Cin > (1LL << 29) - 1)
     return MNV_ERR_INVALID;
   g->d_T = mnv_fastdiv_make(g->TH * g->TW);
   g->d_TW = mnv_fastdiv_make(g->TW);
@@ -457,33 +529,34 @@ int make_wino_geom(WinoGeom* g, int N, int Cin, int Cout, int Hs, int Ws, int pa
 }
 
 // V of the group of images that `g` describes
+template <int AL>
 int launch_input_transform(const float* src, float* V, const WinoGeom& g, hipStream_t s) {
   const int T = g.TH * g.TW, HW = g.Hs * g.Ws;
   // planes a workgroup's 256 consecutive tiles can touch
-  const size_t lds = (size_t)WINO_CH * (255 / T + 2) * HW * sizeof(float);
+  const size_t lds = (size_t)(255 / T + 2) * HW * sizeof(float);
   if (lds <= 32 * 1024)
-    hipLaunchKernelGGL(mnv_wino_input_lds_kernel, dim3((g.Pp + 255) / 256, (g.Cin + WINO_CH - 1) / WINO_CH),
-                       dim3(256), lds, s, src, V, g, mnv_fastdiv_make(HW));
+    hipLaunchKernelGGL(mnv_wino_input_lds_kernel<AL>, dim3((g.Pp + 255) / 256, g.Cin), dim3(256), lds,
+                       s, src, V, g, mnv_fastdiv_make(HW));
   else
-    hipLaunchKernelGGL(mnv_wino_input_kernel, dim3((g.Pp + 255) / 256, g.Cin), dim3(256), 0, s, src, V, g);
+    hipLaunchKernelGGL(mnv_wino_input_kernel<AL>, dim3((g.Pp + 255) / 256, g.Cin), dim3(256), 0, s, src,
+                       V, g);
   return MNV_LAUNCH_STATUS();
 }
 
-size_t u_bytes(const WinoGeom& g) { return align256((size_t)16 * g.Coutp * g.Cin * sizeof(float)); }
+size_t u_bytes(const WinoGeom& g) {
+  return align256((size_t)g.al * g.al * g.Coutp * g.Cin * sizeof(float));
+}
 // V and M of `images` images
 size_t vm_bytes(const WinoGeom& g, int images) {
-  const size_t pp = ((size_t)images * g.TH * g.TW + 3) / 4 * 4;
-  return align256(16 * pp * g.Cin * sizeof(float)) + align256(16 * pp * g.Coutp * sizeof(float));
+  const size_t pp = ((size_t)images * g.TH * g.TW + 3) / 4 * 4, points = (size_t)g.al * g.al;
+  return align256(points * pp * g.Cin * sizeof(float)) + align256(points * pp * g.Coutp * sizeof(float));
 }
-
 // partial tiles of the filter gradient's equal-shares launch: at most four workgroups per CU,
 // a partial tile each and one more per output tile
 size_t grad_sk_bytes(const WinoGeom& g) {
-  const long long tiles = (long long)((g.Cin + 127) / 128) * (16 * g.Coutp / 128);
+  const long long tiles = (long long)((g.Cin + 127) / 128) * (g.al * g.al * g.Coutp / 128);
   return (size_t)(4 * mnv_cu_count() + tiles) * 128 * 128 * sizeof(float);
 }
-
-std::atomic<int> g_mode{1};
 
 // the largest group of images whose transformed tensors fit `avail` bytes, then groups of
 // equal size; 0 when not even one image fits
@@ -500,33 +573,128 @@ int images_that_fit(const WinoGeom& g, int N, size_t avail) {
   return (N + groups - 1) / groups;
 }
 
+// the geometry of a pass under the current mode; false: the pass does not run this way
+bool plan_geom(WinoGeom* g, int* mode_out, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w,
+               int R, int S, int sv, int sh) {
+  const int mode = g_mode.load(std::memory_order_relaxed);
+  *mode_out = mode;
+  if (mode == 0 || R != 3 || S != 3 || sv != 1 || sh != 1 || pad_h < 0 || pad_w < 0 || pad_h > 2 ||
+      pad_w > 2 || Hs + 2 * pad_h < 3 || Ws + 2 * pad_w < 3)
+    return false;
+  const int al = pick_points(Hs + 2 * pad_h - 2, Ws + 2 * pad_w - 2, mode);
+  return make_wino_geom(g, N, Cin, Cout, Hs, Ws, pad_h, pad_w, al) == MNV_OK;
+}
+
+// mode 1: enough channels to fill the tiles of the products, enough tiles, and output extents
+// whose rounding up to whole tiles wastes at most 40% (al = 4) -- with al = 6 the choice of
+// the tile size has already weighed the waste
+bool pays(const WinoGeom& g, int images, int m_extent) {
+  const long long tiles = (long long)images * g.TH * g.TW;
+  const bool fills = m_extent < 0 || m_extent * 4 >= (m_extent + 127) / 128 * 128 * 3;
+  return g.Cin >= 32 && fills && g.Cout * 4 >= g.Coutp * 3 && tiles * (g.al * g.al / 16) >= 1024 &&
+         (g.al == 6 || 4LL * g.TH * g.TW * 5 <= 7LL * g.Hd * g.Wd);
+}
+
+template <int AL>
+int wino_conv(const WinoGeom& g0, const float* src, const float* filter, const float* bias,
+              const float* gate, float* dst, int N, int transposed, int relu, int images,
+              void* workspace, hipStream_t s) {
+  WinoGeom g = g0;
+  const int Cin = g.Cin, Cout = g.Cout;
+  char* w = static_cast<char*>(workspace);
+  float* U = reinterpret_cast<float*>(w);
+  w += u_bytes(g);
+  float* V = reinterpret_cast<float*>(w);
+  w += align256((size_t)AL * AL * g.Pp * Cin * sizeof(float));
+  float* Mx = reinterpret_cast<float*>(w);
+  const int K = transposed ? Cin : Cout, C = transposed ? Cout : Cin;
+  hipLaunchKernelGGL(mnv_wino_filter_kernel<AL>, dim3((g.Coutp * Cin + 255) / 256), dim3(256), 0, s,
+                     filter, U, g, K, C, transposed != 0);
+  int rc = MNV_LAUNCH_STATUS();
+  if (rc) return rc;
+  const size_t per_src = (size_t)Cin * g.Hs * g.Ws, per_dst = (size_t)Cout * g.Hd * g.Wd;
+  for (int n0 = 0; n0 < N; n0 += images) {
+    const int nn = N - n0 < images ? N - n0 : images;
+    if (nn != g.N && (rc = make_wino_geom(&g, nn, Cin, Cout, g.Hs, g.Ws, g.pad_h, g.pad_w, AL))) return rc;
+    if ((rc = launch_input_transform<AL>(src + n0 * per_src, V, g, s))) return rc;
+    WinoGemm p{V, U, Mx, g.Pp, AL * AL * g.Coutp, Cin, Cin / 16, Cin / 16, g.Coutp, g.Coutp / 128};
+    if ((rc = mnv_gemm_launch<TileBig>(p, 1, nullptr, s))) return rc;
+    hipLaunchKernelGGL(mnv_wino_output_kernel<AL>, dim3((g.P + 255) / 256, Cout), dim3(256), 0, s, Mx,
+                       bias, gate ? gate + n0 * per_dst : nullptr, dst + n0 * per_dst, g, relu);
+    if ((rc = MNV_LAUNCH_STATUS())) return rc;
+  }
+  return MNV_OK;
+}
+
+#ifndef MNV_WINO_SK_PF
+#define MNV_WINO_SK_PF 1
+#endif
+template <int AL>
+int wino_filter_grad(const WinoGeom& g0, const float* bottom, const float* top_diff, float* filter_diff,
+                     int N, int images, int accumulate, const float* sgd_w, float sgd_scale,
+                     void* workspace, hipStream_t s, int* plan) {
+  WinoGeom g = g0;
+  const int C = g.Cin, K = g.Cout;
+  const size_t sk_bytes = grad_sk_bytes(g);
+  char* w = static_cast<char*>(workspace);
+  float* Q = reinterpret_cast<float*>(w);
+  w += u_bytes(g);
+  float* V = reinterpret_cast<float*>(w);
+  w += align256((size_t)AL * AL * g.Pp * C * sizeof(float));
+  float* Yt = reinterpret_cast<float*>(w);
+  w += align256((size_t)AL * AL * g.Pp * g.Coutp * sizeof(float));
+  if (plan) {
+    WinoGradGemm p{V, Yt, Q, C, AL * AL * g.Coutp, g.Pp, (g.Pp + 15) / 16, g.Pp >= 16 ? g.Pp / 16 : 1,
+                   g.Coutp, 0};
+    bool done = false;
+    plan[0] = 128;
+    plan[1] = 1;
+    plan[2] = 0;
+    return mnv_gemm_streamk_launch<TileBig, MNV_WINO_SK_PF>(p, w, sk_bytes, s, &done, plan + 2);
+  }
+  int rc;
+  const size_t per_bottom = (size_t)C * g.Hs * g.Ws, per_top = (size_t)K * g.Hd * g.Wd;
+  for (int n0 = 0; n0 < N; n0 += images) {
+    const int nn = N - n0 < images ? N - n0 : images;
+    if (nn != g.N && (rc = make_wino_geom(&g, nn, C, K, g.Hs, g.Ws, g.pad_h, g.pad_w, AL))) return rc;
+    if ((rc = launch_input_transform<AL>(bottom + n0 * per_bottom, V, g, s))) return rc;
+    hipLaunchKernelGGL(mnv_wino_grad_kernel<AL>, dim3((g.Pp + 255) / 256, g.Coutp), dim3(256), 0, s,
+                       top_diff + n0 * per_top, Yt, g);
+    if ((rc = MNV_LAUNCH_STATUS())) return rc;
+    WinoGradGemm p{V, Yt, Q, C, AL * AL * g.Coutp, g.Pp, (g.Pp + 15) / 16, g.Pp >= 16 ? g.Pp / 16 : 1,
+                   g.Coutp, n0 > 0};
+    bool done = false;
+    if ((rc = mnv_gemm_streamk_launch<TileBig, MNV_WINO_SK_PF>(p, w, sk_bytes, s, &done))) return rc;
+    if (!done && (rc = mnv_gemm_launch<TileBig>(p, 1, nullptr, s))) return rc;
+  }
+  hipLaunchKernelGGL(mnv_wino_grad_output_kernel<AL>, dim3((K * C + 255) / 256), dim3(256), 0, s, Q,
+                     filter_diff, g, accumulate, sgd_w, sgd_scale);
+  return MNV_LAUNCH_STATUS();
+}
+
 }  // namespace
 
 extern "C" int mnv_conv_winograd_mode(int mode) {
-  if (mode < 0 || mode > 2) return g_mode.load(std::memory_order_relaxed);
+  if (mode < 0 || mode > 4) return g_mode.load(std::memory_order_relaxed);
   return g_mode.exchange(mode, std::memory_order_relaxed);
 }
 
 size_t mnv_wino_workspace_bytes(int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w) {
   WinoGeom g;
-  if (make_wino_geom(&g, N, Cin, Cout, Hs, Ws, pad_h, pad_w)) return 0;
+  int mode;
+  if (!plan_geom(&g, &mode, N, Cin, Cout, Hs, Ws, pad_h, pad_w, 3, 3, 1, 1)) return 0;
   return u_bytes(g) + vm_bytes(g, N);
 }
 
 int mnv_wino_images(int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w, int R, int S,
                     int sv, int sh, size_t workspace_bytes) {
-  const int mode = g_mode.load(std::memory_order_relaxed);
   WinoGeom g;
-  if (mode == 0 || R != 3 || S != 3 || sv != 1 || sh != 1 || Cin % 16 != 0 ||
-      make_wino_geom(&g, N, Cin, Cout, Hs, Ws, pad_h, pad_w))
-    return 0;
+  int mode;
+  if (Cin % 16 != 0 || !plan_geom(&g, &mode, N, Cin, Cout, Hs, Ws, pad_h, pad_w, R, S, sv, sh)) return 0;
   if (workspace_bytes < u_bytes(g)) return 0;
   const int images = images_that_fit(g, N, workspace_bytes - u_bytes(g));
-  if (mode == 2 || images == 0) return images;
-  const long long tiles = (long long)images * g.TH * g.TW;
-  const bool pays = Cin >= 32 && Cout * 4 >= g.Coutp * 3 && tiles >= 1024 &&
-                    4LL * g.TH * g.TW * 5 <= 7LL * g.Hd * g.Wd;
-  return pays ? images : 0;
+  if (mode != 1 || images == 0) return images;
+  return pays(g, images, -1) ? images : 0;
 }
 
 int mnv_wino_conv(const float* src, const float* filter, const float* bias, const float* gate,
@@ -534,105 +702,51 @@ int mnv_wino_conv(const float* src, const float* filter, const float* bias, cons
                   int transposed, int relu, int images, void* workspace, size_t workspace_bytes,
                   hipStream_t s) {
   WinoGeom g;
+  int mode;
   if (!src || !filter || !dst || images <= 0 || Cin % 16 != 0) return MNV_ERR_INVALID;
   if (images > N) images = N;
-  int rc = make_wino_geom(&g, images, Cin, Cout, Hs, Ws, pad_h, pad_w);
-  if (rc) return rc;
+  if (!plan_geom(&g, &mode, images, Cin, Cout, Hs, Ws, pad_h, pad_w, 3, 3, 1, 1)) return MNV_ERR_INVALID;
   if (!workspace || workspace_bytes < u_bytes(g) + vm_bytes(g, images)) return MNV_ERR_INVALID;
-  char* w = static_cast<char*>(workspace);
-  float* U = reinterpret_cast<float*>(w);
-  w += u_bytes(g);
-  float* V = reinterpret_cast<float*>(w);
-  w += align256((size_t)16 * g.Pp * Cin * sizeof(float));
-  float* Mx = reinterpret_cast<float*>(w);
-  const int K = transposed ? Cin : Cout, C = transposed ? Cout : Cin;
-  hipLaunchKernelGGL(mnv_wino_filter_kernel, dim3((g.Coutp * Cin + 255) / 256), dim3(256), 0, s,
-                     filter, U, g, K, C, transposed != 0);
-  if ((rc = MNV_LAUNCH_STATUS())) return rc;
-  const size_t per_src = (size_t)Cin * Hs * Ws, per_dst = (size_t)Cout * g.Hd * g.Wd;
-  for (int n0 = 0; n0 < N; n0 += images) {
-    const int nn = N - n0 < images ? N - n0 : images;
-    if (nn != g.N && (rc = make_wino_geom(&g, nn, Cin, Cout, Hs, Ws, pad_h, pad_w))) return rc;
-    if ((rc = launch_input_transform(src + n0 * per_src, V, g, s))) return rc;
-    WinoGemm p{V, U, Mx, g.Pp, 16 * g.Coutp, Cin, Cin / 16, Cin / 16, g.Coutp, g.Coutp / 128};
-    if ((rc = mnv_gemm_launch<TileBig>(p, 1, nullptr, s))) return rc;
-    hipLaunchKernelGGL(mnv_wino_output_kernel, dim3((g.P + 255) / 256, Cout), dim3(256), 0, s, Mx,
-                       bias, gate ? gate + n0 * per_dst : nullptr, dst + n0 * per_dst, g, relu);
-    if ((rc = MNV_LAUNCH_STATUS())) return rc;
-  }
-  return MNV_OK;
+  return g.al == 6 ? wino_conv<6>(g, src, filter, bias, gate, dst, N, transposed, relu, images, workspace, s)
+                   : wino_conv<4>(g, src, filter, bias, gate, dst, N, transposed, relu, images, workspace, s);
 }
 
 size_t mnv_wino_grad_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw) {
   WinoGeom g;
-  if (make_wino_geom(&g, N, C, K, H, W, ph, pw)) return 0;
+  int mode;
+  if (!plan_geom(&g, &mode, N, C, K, H, W, ph, pw, 3, 3, 1, 1)) return 0;
   return u_bytes(g) + vm_bytes(g, N) + grad_sk_bytes(g);
 }
 
 int mnv_wino_grad_images(int N, int C, int K, int H, int W, int ph, int pw, int R, int S, int sv,
                          int sh, size_t workspace_bytes) {
-  const int mode = g_mode.load(std::memory_order_relaxed);
   WinoGeom g;
-  if (mode == 0 || R != 3 || S != 3 || sv != 1 || sh != 1 || make_wino_geom(&g, N, C, K, H, W, ph, pw))
-    return 0;
+  int mode;
+  if (!plan_geom(&g, &mode, N, C, K, H, W, ph, pw, R, S, sv, sh)) return 0;
   if (workspace_bytes < u_bytes(g) + grad_sk_bytes(g)) return 0;
   int images = images_that_fit(g, N, workspace_bytes - u_bytes(g) - grad_sk_bytes(g));
   // Yt of a group is read through 32-bit byte offsets
   const long long per_image = (long long)g.TH * g.TW;
-  const long long most = ((1LL << 29) - 1) / (16LL * g.Coutp) / per_image;
+  const long long most = ((1LL << 29) - 1) / ((long long)g.al * g.al * g.Coutp) / per_image;
   if (images > most) images = (int)most;
-  if (mode == 2 || images == 0) return images;
-  const long long tiles = (long long)images * per_image;
-  const bool pays = C >= 32 && C * 4 >= (C + 127) / 128 * 128 * 3 && K * 4 >= g.Coutp * 3 &&
-                    tiles >= 1024 && 4LL * g.TH * g.TW * 5 <= 7LL * g.Hd * g.Wd;
-  return pays ? images : 0;
+  if (mode != 1 || images == 0) return images;
+  return pays(g, images, C) ? images : 0;
 }
 
-#ifndef MNV_WINO_SK_PF
-#define MNV_WINO_SK_PF 1
-#endif
 int mnv_wino_filter_grad(const float* bottom, const float* top_diff, float* filter_diff, int N, int C,
                          int K, int H, int W, int ph, int pw, int images, int accumulate,
                          const float* sgd_w, float sgd_scale, void* workspace,
                          size_t workspace_bytes, hipStream_t s, int* plan) {
   WinoGeom g;
+  int mode;
   if (images <= 0) return MNV_ERR_INVALID;
   if (images > N) images = N;
-  int rc = make_wino_geom(&g, images, C, K, H, W, ph, pw);
-  if (rc) return rc;
-  const size_t sk_bytes = grad_sk_bytes(g);
-  if (!workspace || workspace_bytes < u_bytes(g) + vm_bytes(g, images) + sk_bytes) return MNV_ERR_INVALID;
-  char* w = static_cast<char*>(workspace);
-  float* Q = reinterpret_cast<float*>(w);
-  w += u_bytes(g);
-  float* V = reinterpret_cast<float*>(w);
-  w += align256((size_t)16 * g.Pp * C * sizeof(float));
-  float* Yt = reinterpret_cast<float*>(w);
-  w += align256((size_t)16 * g.Pp * g.Coutp * sizeof(float));
-  if (plan) {
-    WinoGradGemm p{V, Yt, Q, C, 16 * g.Coutp, g.Pp, (g.Pp + 15) / 16, g.Pp >= 16 ? g.Pp / 16 : 1, g.Coutp, 0};
-    bool done = false;
-    plan[0] = 128;
-    plan[1] = 1;
-    plan[2] = 0;
-    return mnv_gemm_streamk_launch<TileBig, MNV_WINO_SK_PF>(p, w, sk_bytes, s, &done, plan + 2);
-  }
-  if (!bottom || !top_diff || !filter_diff) return MNV_ERR_INVALID;
-  const size_t per_bottom = (size_t)C * H * W, per_top = (size_t)K * g.Hd * g.Wd;
-  for (int n0 = 0; n0 < N; n0 += images) {
-    const int nn = N - n0 < images ? N - n0 : images;
-    if (nn != g.N && (rc = make_wino_geom(&g, nn, C, K, H, W, ph, pw))) return rc;
-    if ((rc = launch_input_transform(bottom + n0 * per_bottom, V, g, s))) return rc;
-    hipLaunchKernelGGL(mnv_wino_grad_kernel, dim3((g.Pp + 255) / 256, g.Coutp), dim3(256), 0, s,
-                       top_diff + n0 * per_top, Yt, g);
-    if ((rc = MNV_LAUNCH_STATUS())) return rc;
-    WinoGradGemm p{V, Yt, Q, C, 16 * g.Coutp, g.Pp, (g.Pp + 15) / 16, g.Pp >= 16 ? g.Pp / 16 : 1,
-                   g.Coutp, n0 > 0};
-    bool done = false;
-    if ((rc = mnv_gemm_streamk_launch<TileBig, MNV_WINO_SK_PF>(p, w, sk_bytes, s, &done))) return rc;
-    if (!done && (rc = mnv_gemm_launch<TileBig>(p, 1, nullptr, s))) return rc;
-  }
-  hipLaunchKernelGGL(mnv_wino_grad_output_kernel, dim3((K * C + 255) / 256), dim3(256), 0, s, Q,
-                     filter_diff, g, accumulate, sgd_w, sgd_scale);
-  return MNV_LAUNCH_STATUS();
+  if (!plan_geom(&g, &mode, images, C, K, H, W, ph, pw, 3, 3, 1, 1)) return MNV_ERR_INVALID;
+  if (!workspace || workspace_bytes < u_bytes(g) + vm_bytes(g, images) + grad_sk_bytes(g))
+    return MNV_ERR_INVALID;
+  if (!plan && (!bottom || !top_diff || !filter_diff)) return MNV_ERR_INVALID;
+  return g.al == 6 ? wino_filter_grad<6>(g, bottom, top_diff, filter_diff, N, images, accumulate, sgd_w,
+                                         sgd_scale, workspace, s, plan)
+                   : wino_filter_grad<4>(g, bottom, top_diff, filter_diff, N, images, accumulate, sgd_w,
+                                         sgd_scale, workspace, s, plan);
 }

@@ -58,8 +58,9 @@ def test_pure_host_entry_points():
 def test_winograd_switch_and_size_queries():
     """The path switch is process-wide host state and the size queries follow it (pure
     arithmetic): the 384 -> 384 channel layer on 13 x 13 planes at batch 256 asks for its
-    transformed tensors (16 values per 4 x 4 tile and channel: 597 MB) only while the path
-    is on; a 5 x 5 layer never does."""
+    transformed tensors only while the path is on (36 values per 6 x 6 tile and channel on
+    4 x 4 tiles per plane, 474 MB; 16 per 4 x 4 tile on 7 x 7 tiles, 597 MB, with the tile
+    size pinned); a 5 x 5 layer never does."""
     from minerva_amd import capi
     L = capi.lib()
     conv4 = (256, 384, 384, 13, 13, 1, 1, 1, 1, 3, 3)
@@ -67,8 +68,8 @@ def test_winograd_switch_and_size_queries():
     assert L.mnv_conv_winograd_mode(-1) == 1
     try:
         on = L.mnv_conv_fwd_workspace_bytes(*conv4)
-        tiles = 256 * 7 * 7
-        assert on == 16 * 384 * 384 * 4 + 2 * 16 * tiles * 384 * 4
+        tiles = 256 * 4 * 4
+        assert on == 36 * 384 * 384 * 4 + 2 * 36 * tiles * 384 * 4
         assert L.mnv_conv_bwd_data_workspace_bytes(*conv4) == on
         five = L.mnv_conv_fwd_workspace_bytes(*conv2)
         assert L.mnv_conv_winograd_mode(0) == 1
@@ -77,7 +78,11 @@ def test_winograd_switch_and_size_queries():
         assert L.mnv_conv_winograd_mode(2) == 0
         assert L.mnv_conv_fwd_workspace_bytes(*conv4) == on
         assert L.mnv_conv_fwd_workspace_bytes(*conv2) == five
-        assert L.mnv_conv_winograd_mode(7) == 2      # out of range: a query
+        assert L.mnv_conv_winograd_mode(3) == 2      # 2 x 2 output tiles only
+        assert L.mnv_conv_fwd_workspace_bytes(*conv4) == 16 * 384 * 384 * 4 + 2 * 16 * 256 * 49 * 384 * 4
+        assert L.mnv_conv_winograd_mode(4) == 3      # 4 x 4 output tiles only
+        assert L.mnv_conv_fwd_workspace_bytes(*conv4) == on
+        assert L.mnv_conv_winograd_mode(7) == 4      # out of range: a query
     finally:
         L.mnv_conv_winograd_mode(1)
 

@@ -1,5 +1,6 @@
 """GPU parity of the minimal-filtering paths of the 3 x 3 unit-stride convolutions (forward
-and data gradient by F(2 x 2, 3 x 3), filter gradient by F(3 x 3, 2 x 2)), through the C ABI: against the CPU oracle's direct
+and data gradient by F(m x m, 3 x 3), filter gradient by F(3 x 3, m x m), m = 2 and 4), through
+the C ABI: against the CPU oracle's direct
 sums on geometries that exercise odd and even extents, every padding, ragged tile counts and
 channel counts off the tile width; in groups of images under a small workspace (same bits as
 in one group); with the fused epilogues (same bits as the operator chain); and the switch
@@ -13,9 +14,11 @@ from gpu_util import Gpu, assert_bits_equal, normwise, say
 from test_gpu_conv import Conv, _rand
 
 pytestmark = pytest.mark.gpu
-# F(2 x 2, 3 x 3) adds and halves in its transforms: a few 1e-7 of the output's norm in fp32;
-# the bound of the convolutions is 1e-4
+# The transforms are short sums with small constants: against the direct sum a few 1e-6 of the
+# output's norm in fp32 with 2 x 2 tiles, up to about 6e-6 with 4 x 4 tiles (measured on the
+# batch-256 layers); the bound of the convolutions is 1e-4
 TIGHT = 2e-5
+F2, F4 = 3, 4   # modes that pin the tile size (2: the library picks it)
 
 
 @pytest.fixture(scope="module")
@@ -54,8 +57,9 @@ GEOMS = [
 ]
 
 
+@pytest.mark.parametrize("tile", [F2, F4], ids=["2x2", "4x4"])
 @pytest.mark.parametrize("p7", GEOMS, ids=lambda p: "x".join(map(str, p)))
-def test_winograd_passes_against_oracle(gpu, ora, p7):
+def test_winograd_passes_against_oracle(gpu, ora, p7, tile):
     N, C, K, H, W, ph, pw = p7
     p = (N, C, K, H, W, ph, pw, 1, 1, 3, 3)
     cv = Conv(gpu, *p)
@@ -67,7 +71,7 @@ def test_winograd_passes_against_oracle(gpu, ora, p7):
         direct_y, direct_dx, direct_dw = cv.fwd(x, w, b), cv.bwd_data(dy, w), cv.bwd_filter(dy, x)
         direct_bare, direct_bare_dw = cv.fwd(x, w, b, False), cv.bwd_filter(dy, x, False)
         direct_bytes = gpu.L.mnv_conv_fwd_workspace_bytes(*p)
-    with mode(gpu, 2):
+    with mode(gpu, tile):
         say("winograd bwd filter", p)
         dw = cv.bwd_filter(dy, x)
         assert normwise(dw, want_dw) <= TIGHT
@@ -117,17 +121,28 @@ def test_winograd_needs_a_16_byte_aligned_workspace(gpu, ora):
         assert np.any(gpu.down(top).view(np.uint32) != direct.view(np.uint32))
 
 
-def _wino_bytes(images, C, K, Ho, Wo):
+def _points(Ho, Wo):
+    """Points per dimension the library picks by itself: 6 (4 x 4 outputs per tile) when that
+    takes at most 85% of the products of 4 (2 x 2 outputs per tile)."""
+    small = 16 * ((Ho + 1) // 2) * ((Wo + 1) // 2)
+    large = 36 * ((Ho + 3) // 4) * ((Wo + 3) // 4)
+    return 6 if large * 100 <= small * 85 else 4
+
+
+def _wino_bytes(images, C, K, Ho, Wo, al=None):
     """The workspace the path wants for `images` images at once (U, V, M from 256-byte
     boundaries; tiles rounded up to 4, output channels to 128)."""
+    al = al or _points(Ho, Wo)
+    m = al - 2
     a256 = lambda v: (v + 255) // 256 * 256
     kp = (K + 127) // 128 * 128
-    pp = (images * ((Ho + 1) // 2) * ((Wo + 1) // 2) + 3) // 4 * 4
-    return a256(16 * kp * C * 4) + a256(16 * pp * C * 4) + a256(16 * pp * kp * 4)
+    pp = (images * ((Ho + m - 1) // m) * ((Wo + m - 1) // m) + 3) // 4 * 4
+    return a256(al * al * kp * C * 4) + a256(al * al * pp * C * 4) + a256(al * al * pp * kp * 4)
 
 
+@pytest.mark.parametrize("tile", [F2, F4], ids=["2x2", "4x4"])
 @pytest.mark.parametrize("N", [12, 13])
-def test_winograd_in_groups_of_images_has_the_same_bits(gpu, N):
+def test_winograd_in_groups_of_images_has_the_same_bits(gpu, N, tile):
     """A workspace that holds five images: 12 images run as three groups of four, 13 as five,
     five and three.  Every output element is the same sum in the same order."""
     C, K, H, W = 32, 64, 13, 13
@@ -135,11 +150,12 @@ def test_winograd_in_groups_of_images_has_the_same_bits(gpu, N):
     cv = Conv(gpu, *p)
     x, w, b = _rand(N * C * H * W, 84), _rand(K * C * 9, 85, 0.2), _rand(K, 86)
     dy = _rand(N * K * H * W, 87)
-    with mode(gpu, 2):
-        assert gpu.L.mnv_conv_fwd_workspace_bytes(*p) == _wino_bytes(N, C, K, H, W)
+    al = 4 if tile == F2 else 6
+    with mode(gpu, tile):
+        assert gpu.L.mnv_conv_fwd_workspace_bytes(*p) == _wino_bytes(N, C, K, H, W, al)
         whole_y, whole_dx = cv.fwd(x, w, b), cv.bwd_data(dy, w)
-        small = _wino_bytes(5, C, K, H, W) + 1024
-        assert small < _wino_bytes(N, C, K, H, W)
+        small = _wino_bytes(5, C, K, H, W, al) + 1024
+        assert small < _wino_bytes(N, C, K, H, W, al)
         ws = gpu.empty(small // 4 + 64)
         dxb, dwb, dbb, dyb = gpu.up(x), gpu.up(w), gpu.up(b), gpu.up(dy)
         top, bd = gpu.empty(whole_y.size), gpu.empty(whole_dx.size)
@@ -147,7 +163,7 @@ def test_winograd_in_groups_of_images_has_the_same_bits(gpu, N):
         gpu.call("mnv_conv_fwd", dxb.p, dwb.p, dbb.p, top.p, *p, ws.p, ctypes.c_size_t(small))
         assert_bits_equal(gpu.down(top), whole_y, "forward in groups")
         say("winograd in groups, bwd data", p)
-        small = _wino_bytes(5, K, C, H, W) + 1024
+        small = _wino_bytes(5, K, C, H, W, al) + 1024
         gpu.call("mnv_conv_bwd_data", dyb.p, dwb.p, bd.p, *p, ws.p, ctypes.c_size_t(small))
         assert_bits_equal(gpu.down(bd), whole_dx, "data gradient in groups")
         # the filter gradient sums over the images: in groups the 16 products accumulate group
@@ -155,7 +171,7 @@ def test_winograd_in_groups_of_images_has_the_same_bits(gpu, N):
         say("winograd in groups, bwd filter", p)
         whole_dw = cv.bwd_filter(dy, x)
         full = gpu.L.mnv_conv_bwd_filter_workspace_bytes(*p)
-        small = full - (_wino_bytes(N, C, K, H, W) - _wino_bytes(5, C, K, H, W)) + 1024
+        small = full - (_wino_bytes(N, C, K, H, W, al) - _wino_bytes(5, C, K, H, W, al)) + 1024
         big = gpu.empty(small // 4 + 64)
         fd = gpu.up(np.full(K * C * 9, np.nan, np.float32))
         gpu.call("mnv_conv_bwd_filter", dxb.p, dyb.p, fd.p, *p, big.p, ctypes.c_size_t(small))
@@ -164,7 +180,8 @@ def test_winograd_in_groups_of_images_has_the_same_bits(gpu, N):
         assert np.any(got.view(np.uint32) != whole_dw.view(np.uint32))
 
 
-def test_winograd_fused_epilogues_have_the_bits_of_the_chain(gpu):
+@pytest.mark.parametrize("tile", [F2, F4], ids=["2x2", "4x4"])
+def test_winograd_fused_epilogues_have_the_bits_of_the_chain(gpu, tile):
     """conv + ReLU and data gradient + ReLU gradient in one call against the separate
     operators, both on the minimal-filtering path."""
     p = (6, 32, 48, 11, 12, 1, 1, 1, 1, 3, 3)
@@ -172,7 +189,7 @@ def test_winograd_fused_epilogues_have_the_bits_of_the_chain(gpu):
     cv = Conv(gpu, *p)
     x, w, b = _rand(N * C * H * W, 88), _rand(K * C * 9, 89, 0.2), _rand(K, 90)
     dy = _rand(N * K * cv.Ho * cv.Wo, 91)
-    with mode(gpu, 2):
+    with mode(gpu, tile):
         nbytes = gpu.L.mnv_conv_fwd_workspace_bytes(*p)
         nbytes = max(nbytes, gpu.L.mnv_conv_bwd_data_workspace_bytes(*p))
         ws = gpu.empty(nbytes // 4 + 64)
@@ -201,10 +218,10 @@ def test_winograd_fused_epilogues_have_the_bits_of_the_chain(gpu):
 
 def test_winograd_is_taken_by_itself_where_it_pays(gpu, ora):
     """In the initial mode a 3 x 3 layer with enough channels and tiles takes the path without
-    being asked (96 output channels on 1176 tiles); the same layer with 16 input channels, or
-    at stride 2, or with 5 x 5 filters, does not."""
+    being asked (96 output channels on 40 x 16 tiles of 4 x 4 outputs); the same layer with 16
+    input channels, or at stride 2, or with 5 x 5 filters, or on 4 images, does not."""
     assert gpu.L.mnv_conv_winograd_mode(-1) == 1
-    p = (24, 32, 96, 13, 13, 1, 1, 1, 1, 3, 3)
+    p = (40, 32, 96, 13, 13, 1, 1, 1, 1, 3, 3)
     N, C, K, H, W = p[:5]
     cv = Conv(gpu, *p)
     x, w, b = _rand(N * C * H * W, 92), _rand(K * C * 9, 93, 0.2), _rand(K, 94)
@@ -217,8 +234,8 @@ def test_winograd_is_taken_by_itself_where_it_pays(gpu, ora):
         direct = cv.fwd(x, w, b)
     assert np.any(y.view(np.uint32) != direct.view(np.uint32))
     assert normwise(y, direct) <= TIGHT
-    for q in [(24, 16, 96, 13, 13, 1, 1, 1, 1, 3, 3), (24, 32, 96, 13, 13, 1, 1, 2, 2, 3, 3),
-              (24, 32, 96, 13, 13, 2, 2, 1, 1, 5, 5), (4, 32, 96, 13, 13, 1, 1, 1, 1, 3, 3)]:
+    for q in [(40, 16, 96, 13, 13, 1, 1, 1, 1, 3, 3), (40, 32, 96, 13, 13, 1, 1, 2, 2, 3, 3),
+              (40, 32, 96, 13, 13, 2, 2, 1, 1, 5, 5), (4, 32, 96, 13, 13, 1, 1, 1, 1, 3, 3)]:
         with mode(gpu, 0):
             want = gpu.L.mnv_conv_fwd_workspace_bytes(*q)
         assert gpu.L.mnv_conv_fwd_workspace_bytes(*q) == want, q
@@ -230,8 +247,9 @@ ALEX3 = [("conv3", 256, 384), ("conv4", 384, 384), ("conv5", 384, 256)]
 @pytest.mark.parametrize("case", ALEX3, ids=lambda c: c[0])
 def test_direct_and_winograd_agree_at_batch_256(gpu, case):
     """The 13 x 13 layers of the AlexNet shape at batch 256 on both paths (two independent
-    algorithms over the same 256 distinct images), as the host layer runs them: with the
-    whole-batch workspace and in groups under 128 MB."""
+    algorithms over the same 256 distinct images), as the host layer runs them (4 x 4 output
+    tiles, the library's choice for 13 x 13 planes): with the whole-batch workspace and in
+    groups under 128 MB; and the 2 x 2 tiles beside them."""
     name, C, K = case
     p = (256, C, K, 13, 13, 1, 1, 1, 1, 3, 3)
     N, H, W = 256, 13, 13
@@ -265,3 +283,10 @@ def test_direct_and_winograd_agree_at_batch_256(gpu, case):
         assert_bits_equal(gpu.down(top), y, "forward in groups")
         gpu.call("mnv_conv_bwd_data", dyb.p, dwb.p, bd.p, *p, ws.p, ctypes.c_size_t(small))
         assert_bits_equal(gpu.down(bd), dx, "data gradient in groups")
+    assert _points(13, 13) == 6
+    with mode(gpu, F2):
+        assert gpu.L.mnv_conv_fwd_workspace_bytes(*p) == _wino_bytes(N, C, K, H, W, 4)
+        y2, dx2, dw2 = cv.fwd(x, w, b), cv.bwd_data(dy, w), cv.bwd_filter(dy, x)
+        assert np.any(y2.view(np.uint32) != y.view(np.uint32))
+        assert normwise(y2, direct_y) <= TIGHT and normwise(dx2, direct_dx) <= TIGHT
+        assert normwise(dw2, direct_dw) <= TIGHT
