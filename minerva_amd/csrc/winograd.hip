@@ -313,6 +313,70 @@ __global__ __launch_bounds__(256) void mnv_wino_output_kernel(const float* __res
     }
 }
 
+// The same through LDS, for planes small enough that the output planes a workgroup's 256
+// tiles belong to fit there: a thread leaves its m x m outputs in LDS and the workgroup then
+// stores every plane in runs of contiguous floats, where the kernel above stores m floats per
+// row and thread, neighbouring threads m floats apart (4 x 4 tiles on 384 channels of
+// 256 x 13 x 13: 95 us).  A pixel is stored by the workgroup that holds its tile.
+template <int AL>
+__global__ __launch_bounds__(256) void mnv_wino_output_lds_kernel(const float* __restrict__ Mx,
+                                                                  const float* __restrict__ bias,
+                                                                  const float* __restrict__ gate,
+                                                                  float* __restrict__ dst, WinoGeom g,
+                                                                  int relu, MnvFastDiv d_HW, MnvFastDiv d_W) {
+  typedef WinoF<AL> F;
+  constexpr int MO = AL - 2;
+  extern __shared__ float planes[];
+  const int p0 = blockIdx.x * 256, p = p0 + threadIdx.x;
+  const int co = blockIdx.y;
+  const int HW = g.Hd * g.Wd, T = g.TH * g.TW;
+  const int img0 = mnv_fastdiv(p0, g.d_T);
+  const int last = p0 + 255 < g.P ? p0 + 255 : g.P - 1;  // p0 < P: the grid covers P
+  const int count = (mnv_fastdiv(last, g.d_T) - img0 + 1) * HW;
+  if (p < g.P) {
+    const size_t plane = (size_t)g.Coutp * g.Pp;
+    const float* in = Mx + (size_t)co * g.Pp + p;
+    float mm[AL][AL];
+#pragma unroll
+    for (int xi = 0; xi < AL; ++xi)
+#pragma unroll
+      for (int nu = 0; nu < AL; ++nu) mm[xi][nu] = in[(xi * AL + nu) * plane];
+    float h[MO][AL], y[MO][MO];
+    wino_rows<typename F::AT, AL>(mm, h);
+    wino_cols<typename F::AT, MO>(h, y);
+    const int img = mnv_fastdiv(p, g.d_T);
+    const int t = p - img * T;
+    const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
+    const float b = bias ? bias[co] : 0.f;
+    float* out = planes + (img - img0) * HW;
+#pragma unroll
+    for (int a = 0; a < MO; ++a)
+#pragma unroll
+      for (int c = 0; c < MO; ++c) {
+        const int yy = MO * th + a, xx = MO * tw + c;
+        if (yy < g.Hd && xx < g.Wd) {
+          float v = y[a][c];
+          if (bias) v = v + b;
+          if (relu) v = v > 0.f ? v : 0.f;
+          out[yy * g.Wd + xx] = v;
+        }
+      }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < count; i += 256) {
+    const int pl = mnv_fastdiv(i, d_HW);
+    const int r = i - pl * HW;
+    const int yy = mnv_fastdiv(r, d_W), xx = r - yy * g.Wd;
+    const int owner = (img0 + pl) * T + (yy / MO) * g.TW + xx / MO;
+    if (owner >= p0 && owner <= last) {
+      const size_t at = ((size_t)(img0 + pl) * g.Cout + co) * HW + r;
+      float v = planes[i];
+      if (gate) v = gate[at] > 0.f ? v : 0.f;
+      dst[at] = v;
+    }
+  }
+}
+
 // The products of all points as one: C{Pp, points Coutp} = A{Pp, Cin} B{Cin, points Coutp}, column-major, where the
 // A of a column tile is the V panel of the tile's transform point.
 struct WinoGemm {
@@ -385,6 +449,55 @@ __global__ __launch_bounds__(256) void mnv_wino_grad_kernel(const float* __restr
     const int t = p - img * (g.TH * g.TW);
     const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
     const float* plane = top_diff + ((size_t)img * g.Cout + k) * (g.Hd * g.Wd);
+#pragma unroll
+    for (int a = 0; a < MO; ++a)
+#pragma unroll
+      for (int b = 0; b < MO; ++b) {
+        const int y = MO * th + a, x = MO * tw + b;
+        if (y < g.Hd && x < g.Wd) d[a][b] = plane[y * g.Wd + x];
+      }
+  }
+  float h[AL][MO], v[AL][AL];
+  wino_rows<typename F::GG, MO>(d, h);
+  wino_cols<typename F::GG, AL>(h, v);
+  const size_t plane = (size_t)g.Coutp * g.Pp;
+  float* out = Yt + (size_t)k * g.Pp + p;
+#pragma unroll
+  for (int xi = 0; xi < AL; ++xi)
+#pragma unroll
+    for (int nu = 0; nu < AL; ++nu) out[(xi * AL + nu) * plane] = v[xi][nu];
+}
+
+// The same with the planes of top_diff fetched whole into LDS (see mnv_wino_input_lds_kernel).
+template <int AL>
+__global__ __launch_bounds__(256) void mnv_wino_grad_lds_kernel(const float* __restrict__ top_diff,
+                                                                float* __restrict__ Yt, WinoGeom g,
+                                                                MnvFastDiv d_HW) {
+  typedef WinoF<AL> F;
+  constexpr int MO = AL - 2;
+  extern __shared__ float planes[];
+  const int p0 = blockIdx.x * 256, p = p0 + threadIdx.x;
+  const int k = blockIdx.y;
+  const int HW = g.Hd * g.Wd;
+  const int img0 = mnv_fastdiv(p0, g.d_T);
+  const int last = p0 + 255 < g.P ? p0 + 255 : g.P - 1;
+  const int count = (last >= p0 && k < g.Cout ? mnv_fastdiv(last, g.d_T) - img0 + 1 : 0) * HW;
+  for (int i = threadIdx.x; i < count; i += 256) {
+    const int pl = mnv_fastdiv(i, d_HW);
+    planes[i] = top_diff[((size_t)(img0 + pl) * g.Cout + k) * HW + (i - pl * HW)];
+  }
+  __syncthreads();
+  if (p >= g.Pp) return;
+  float d[MO][MO];
+#pragma unroll
+  for (int a = 0; a < MO; ++a)
+#pragma unroll
+    for (int b = 0; b < MO; ++b) d[a][b] = 0.f;
+  if (p < g.P && k < g.Cout) {
+    const int img = mnv_fastdiv(p, g.d_T);
+    const int t = p - img * (g.TH * g.TW);
+    const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
+    const float* plane = planes + (img - img0) * HW;
 #pragma unroll
     for (int a = 0; a < MO; ++a)
 #pragma unroll
@@ -619,8 +732,14 @@ int wino_conv(const WinoGeom& g0, const float* src, const float* filter, const f
     if ((rc = launch_input_transform<AL>(src + n0 * per_src, V, g, s))) return rc;
     WinoGemm p{V, U, Mx, g.Pp, AL * AL * g.Coutp, Cin, Cin / 16, Cin / 16, g.Coutp, g.Coutp / 128};
     if ((rc = mnv_gemm_launch<TileBig>(p, 1, nullptr, s))) return rc;
-    hipLaunchKernelGGL(mnv_wino_output_kernel<AL>, dim3((g.P + 255) / 256, Cout), dim3(256), 0, s, Mx,
-                       bias, gate ? gate + n0 * per_dst : nullptr, dst + n0 * per_dst, g, relu);
+    const size_t lds = (size_t)(255 / (g.TH * g.TW) + 2) * g.Hd * g.Wd * sizeof(float);
+    if (lds <= 32 * 1024)
+      hipLaunchKernelGGL(mnv_wino_output_lds_kernel<AL>, dim3((g.P + 255) / 256, Cout), dim3(256), lds, s,
+                         Mx, bias, gate ? gate + n0 * per_dst : nullptr, dst + n0 * per_dst, g, relu,
+                         mnv_fastdiv_make(g.Hd * g.Wd), mnv_fastdiv_make(g.Wd));
+    else
+      hipLaunchKernelGGL(mnv_wino_output_kernel<AL>, dim3((g.P + 255) / 256, Cout), dim3(256), 0, s, Mx,
+                         bias, gate ? gate + n0 * per_dst : nullptr, dst + n0 * per_dst, g, relu);
     if ((rc = MNV_LAUNCH_STATUS())) return rc;
   }
   return MNV_OK;
@@ -658,8 +777,13 @@ int wino_filter_grad(const WinoGeom& g0, const float* bottom, const float* top_d
     const int nn = N - n0 < images ? N - n0 : images;
     if (nn != g.N && (rc = make_wino_geom(&g, nn, C, K, g.Hs, g.Ws, g.pad_h, g.pad_w, AL))) return rc;
     if ((rc = launch_input_transform<AL>(bottom + n0 * per_bottom, V, g, s))) return rc;
-    hipLaunchKernelGGL(mnv_wino_grad_kernel<AL>, dim3((g.Pp + 255) / 256, g.Coutp), dim3(256), 0, s,
-                       top_diff + n0 * per_top, Yt, g);
+    const size_t lds = (size_t)(255 / (g.TH * g.TW) + 2) * g.Hd * g.Wd * sizeof(float);
+    if (lds <= 32 * 1024)
+      hipLaunchKernelGGL(mnv_wino_grad_lds_kernel<AL>, dim3((g.Pp + 255) / 256, g.Coutp), dim3(256), lds, s,
+                         top_diff + n0 * per_top, Yt, g, mnv_fastdiv_make(g.Hd * g.Wd));
+    else
+      hipLaunchKernelGGL(mnv_wino_grad_kernel<AL>, dim3((g.Pp + 255) / 256, g.Coutp), dim3(256), 0, s,
+                         top_diff + n0 * per_top, Yt, g);
     if ((rc = MNV_LAUNCH_STATUS())) return rc;
     WinoGradGemm p{V, Yt, Q, C, AL * AL * g.Coutp, g.Pp, (g.Pp + 15) / 16, g.Pp >= 16 ? g.Pp / 16 : 1,
                    g.Coutp, n0 > 0};
