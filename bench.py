@@ -7,9 +7,9 @@ One step = one forward + backward + SGD pass of the AlexNet-shaped network
 through the C++ host layer (Task -> HipDevice -> hip::<Op> -> C ABI -> HIP kernel),
 synthetic seeded inputs already resident in HBM.  `value` is images/s with one stream
 synchronisation per step; the same step with the reference device's per-operator
-synchronisation is reported beside it.  The dominant kernels (the MFMA implicit-GEMM
-kernels of conv2's three passes) are timed with HIP events on their own stream inside the
-timed steps and priced against the fp32 MFMA peak; `roofline` is the slowest of the three.  SGEMM 4096^3 and the 8192^2 elementwise add
+synchronisation is reported beside it.  The dominant kernel (the MFMA matrix products of the
+minimal-filtering convolution passes) is timed with HIP events on its own stream inside the
+timed steps and priced against the fp32 MFMA peak.  SGEMM 4096^3 and the 8192^2 elementwise add
 are measured the same way and reported in the same JSON line, and the CPU oracle is
 timed on a bounded sample of the same workload on the host cores.
 
@@ -34,12 +34,13 @@ BATCH = 256
 # 2*N*Ho*Wo*K*C*R*S per convolution pass at batch 256, in GFLOP (conv1..conv5)
 CONV_GFLOP = [53.97, 229.32, 76.55, 114.83, 76.55]
 STEP_GFLOP = 1689.8  # convolutions (fwd, bwd-filter, bwd-data except conv1) + three FC layers
-# What the matrix pipe executes: the three passes of conv3..conv5 run by minimal filtering,
-# 36 multiplies per 4 x 4 outputs (or per 3 x 3 filter taps and 4 x 4 tile of top_diff) of a
-# channel pair on 4 x 4 tiles per 13 x 13 plane: 2 * 36 * K * C * 256 * 16 flops per pass
-# instead of 2 * 9 * K * C * 256 * 169.
-WINOGRAD_GFLOP = [2 * 36 * k * c * 256 * 16 / 1e9 for (c, k) in ((256, 384), (384, 384), (384, 256))]
-STEP_EXECUTED_GFLOP = round(STEP_GFLOP - 3 * sum(CONV_GFLOP[2:]) + 3 * sum(WINOGRAD_GFLOP), 1)
+# What the matrix pipe executes: the three passes of conv2..conv5 run by minimal filtering.
+# conv2 (5 x 5): 64 multiplies per 4 x 4 outputs of a channel pair on 7 x 7 tiles per 27 x 27
+# plane; conv3..5 (3 x 3): 36 per 4 x 4 outputs on 4 x 4 tiles per 13 x 13 plane; the filter
+# gradients the same counts with the tiles of top_diff in the filter's place.
+WINOGRAD_GFLOP = [2 * 64 * 256 * 96 * 256 * 49 / 1e9] + \
+                 [2 * 36 * k * c * 256 * 16 / 1e9 for (c, k) in ((256, 384), (384, 384), (384, 256))]
+STEP_EXECUTED_GFLOP = round(STEP_GFLOP - 3 * sum(CONV_GFLOP[1:]) + 3 * sum(WINOGRAD_GFLOP), 1)
 
 
 def capi_check(rc):
@@ -66,23 +67,16 @@ def graph_replay(rt, net, steps, warmup):
     return {"nodes": nodes, "ms_per_step": round(ms, 4), "images_per_s": round(BATCH / ms * 1e3, 1)}
 
 
-# The longest kernels of the step are conv2's three (5 x 5 filters, 229 GFLOP each, within a
-# few percent of one another; the 3 x 3 layers run as shorter launches of the minimal-filtering
-# products): all three operators carry event pairs inside the timed steps and the roofline
-# object is that of the slowest.  Operator names: "pad:2*2 stride:1*1 conv bp filter" ...
-DOMINANT_OP = "pad:2*2 stride:1*1 conv"
-DOMINANT_KERNELS = {
-    "conv ff": ("conv2 forward", "mnv_gemm_kernel<128x128x16,ConvFwd<true>> (conv2 forward) + the "
-                                 "reduction of its cut tail"),
-    "conv bp filter": ("conv2 filter gradient", "mnv_gemm_kernel<128x128x16,ConvBwdFilterFast<false,3>,"
-                                                "stream-k,2 slabs ahead> (conv2 filter gradient) + its "
-                                                "reduction"),
-    "conv bp data": ("conv2 data gradient", "mnv_gemm_kernel<128x96x16,ConvBwdData<true>> (conv2 data "
-                                            "gradient) + the reduction of its cut tail"),
-}
+# The kernel with the largest share of the step is the matrix product of the minimal-filtering
+# passes (mnv_gemm_kernel<128x128x16, WinoGemm>: forward and data gradient of conv2..conv5, eight
+# launches per step); the filter gradients' products (WinoGradGemm, a stream-k launch each) come
+# second.  The library brackets every such launch with an event pair on its stream while
+# mnv_conv_winograd_profile is on, which is how the timed steps measure them apart from the
+# transform kernels of the same operator.
 
 
 def alexnet_bench(steps, warmup, dataflow=True):
+    from minerva_amd import capi
     from minerva_amd import hostapi
     from minerva_amd import configs
     params, data, label = configs.make_inputs("alexnet", BATCH)
@@ -108,11 +102,12 @@ def alexnet_bench(steps, warmup, dataflow=True):
             net.step(0.01)
         rt.sync()
         ops0 = rt.ops_issued()
-        # Inside the timed steps only the dominant kernel's operators carry event pairs (on
-        # their own stream): timing all ~100 operators costs ~5% of the step in idle gaps.
+        # Inside the timed steps only the launches of the dominant kernels carry event pairs
+        # (twelve per step, on their own stream): timing all ~100 operators costs ~5% of the
+        # step in idle gaps.
         plain = mode == "per_step_sync"
         if plain:
-            rt.profile(True, only=DOMINANT_OP)
+            capi.lib().mnv_conv_winograd_profile(1)
         rt.sync()
         per_step = []
         t0 = time.perf_counter()
@@ -122,8 +117,7 @@ def alexnet_bench(steps, warmup, dataflow=True):
             rt.sync()
             per_step.append((time.perf_counter() - ts) * 1e3)
         t1 = time.perf_counter()
-        prof = rt.profile_read() if plain else {}
-        rt.profile(False)
+        prof = product_profile() if plain else {}
         prob = net.read("prob", 1000 * BATCH)
         ms = (t1 - t0) * 1e3 / steps
         ops_per_step = (rt.ops_issued() - ops0) // steps
@@ -242,10 +236,10 @@ TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_gemm_kernels_hbm_traffic
 
 
 def dominant_kernel_traffic(tag):
-    """HBM bytes per launch of one of conv2's kernels, from two rocprofv3 --pmc runs of this
-    script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, each scaled by what the same counter
-    reads for the 8192^2 add kernel).  The figure is the one recorded in the committed summary
-    of those runs (its line "traffic bytes per launch, <tag>: X"), so that the two cannot drift
+    """HBM-side bytes per launch of a kernel, from two rocprofv3 --pmc runs of this script
+    (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, each scaled by what the same counter reads
+    for the 8192^2 add kernel).  The figure is the one recorded in the committed summary of
+    those runs (its line "traffic bytes per launch, <tag>: X"), so that the two cannot drift
     apart; None when the summary is absent."""
     try:
         for line in open(TRAFFIC_PROFILE):
@@ -256,29 +250,50 @@ def dominant_kernel_traffic(tag):
     return None
 
 
+def product_profile():
+    """{kind: (launches, device ms, GFLOP)} of the minimal-filtering products since the profile
+    was switched on; switches it off."""
+    from minerva_amd import capi
+    L = capi.lib()
+    out = {}
+    for kind in (0, 1):
+        n, ms, gf = ctypes.c_int(), ctypes.c_double(), ctypes.c_double()
+        capi.check(L.mnv_conv_winograd_profile_read(kind, ctypes.byref(n), ctypes.byref(ms), ctypes.byref(gf)),
+                   "mnv_conv_winograd_profile_read")
+        out[kind] = (n.value, ms.value, gf.value)
+    L.mnv_conv_winograd_profile(0)
+    return out
+
+
+PRODUCT_KERNELS = {
+    0: ("minimal-filtering products", "mnv_gemm_kernel<128x128x16,WinoGemm> (the 16 / 36 / 64 matrix products of "
+        "the forward and data-gradient passes of conv2..conv5, one launch per pass)"),
+    1: ("minimal-filtering filter-gradient products", "mnv_gemm_kernel<128x128x16,WinoGradGemm,stream-k> (the "
+        "products of the filter gradients of conv2..conv5, one launch per pass) + the reduction of its shares"),
+}
+
+
 def dominant_kernel_roofline(prof, steps):
-    """conv2's operators each run one MFMA kernel followed by the small kernel that adds the
-    partial tiles of its shares or of its cut tail; the event pair brackets both, so the
-    figures are slightly conservative.  Every one of them does conv2's 229 GFLOP."""
+    """The products' flops are those of the transformed problem (2 x points x channels x channels
+    x tiles), i.e. what the kernel itself multiplies, not the direct sum's."""
     rows = []
-    for name, (launches, total_ms) in prof.items():
-        if DOMINANT_OP not in name or not launches:
+    for kind, (launches, ms, gflop) in prof.items():
+        if not launches:
             continue
-        tag, kernel = next(v for k, v in DOMINANT_KERNELS.items() if name.endswith(k))
-        avg_ms = total_ms / launches
-        achieved = CONV_GFLOP[1] * 1e9 / (avg_ms * 1e-3) / 1e12
-        rows.append({"bound": "mfma", "kernel": kernel,
-                     "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+        tag, kernel = PRODUCT_KERNELS[kind]
+        achieved = gflop / ms
+        rows.append({"bound": "mfma", "kernel": kernel, "achieved": round(achieved, 2),
+                     "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
                      "traffic": dominant_kernel_traffic(tag),
-                     "avg_launch_ms": round(avg_ms, 4), "launches": launches,
-                     "algorithmic_gflop_per_launch": CONV_GFLOP[1]})
+                     "avg_launch_ms": round(ms / launches, 4), "launches": launches,
+                     "ms_per_step": round(ms / steps, 4),
+                     "algorithmic_gflop_per_launch": round(gflop / launches, 2)})
     if not rows:
         return None
-    rows.sort(key=lambda r: -r["avg_launch_ms"])
+    rows.sort(key=lambda r: -r["ms_per_step"])
     top = rows[0]
-    top["conv2_other_kernels"] = [{k: r[k] for k in ("kernel", "achieved", "frac", "traffic", "avg_launch_ms")}
-                                  for r in rows[1:]]
+    top["other_kernels"] = rows[1:]
     return top
 
 
@@ -840,7 +855,7 @@ def main():
             "median_ms_per_step": round(main_run["median_ms_per_step"], 3),
             "step_mfma_frac": round(STEP_GFLOP / main_run["ms_per_step"] / PEAK_FP32_MFMA_TFLOPS, 4),
             "step_mfma_frac_note": "algorithmic (direct-sum) flops of the step / time / fp32 MFMA peak; "
-                                   "the 3 x 3 layers execute 1/4 x (16/13)^2 of theirs",
+                                   "conv2 executes 4/25 x (28/27)^2 of its, the 3 x 3 layers 1/4 x (16/13)^2 of theirs",
             "step_executed_gflop": STEP_EXECUTED_GFLOP,
             "step_executed_mfma_frac": round(STEP_EXECUTED_GFLOP / main_run["ms_per_step"] /
                                              PEAK_FP32_MFMA_TFLOPS, 4),

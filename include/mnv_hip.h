@@ -235,26 +235,38 @@ int mnv_softmax_channel_bwd(const float* top_diff, const float* top, float* bott
  * elements each).  A batch whose bottom or top is larger (up to 2^31 - 1 elements) runs as
  * several launches over chunks of images, the filter gradient accumulating chunk by chunk;
  * only a single image or a filter of 2^29 elements and more is refused (MNV_ERR_INVALID).
- * 3 x 3 filters at unit stride may run by minimal filtering (Winograd): F(2 x 2, 3 x 3), 16
- * multiplies per 2 x 2 outputs of a channel pair instead of 36, or F(4 x 4, 3 x 3), 36 per 4 x 4
- * outputs instead of 144 -- whichever needs fewer products for the plane at hand, the smaller
- * tile on a near tie -- as 16 / 36 matrix products between transforms of 4 x 4 / 6 x 6 tiles,
- * summed in fp32; backward_filter by F(3 x 3, 2 x 2) / F(3 x 3, 4 x 4) with the sum over the tiles
- * as the products' reduction.  Results differ from the direct sum by a few 1e-6 of the output's
- * norm (up to about 6e-6 with the larger tile).  forward / backward_data need a bottom / top
+ * 3 x 3 and 5 x 5 filters at unit stride may run by minimal filtering (Winograd): F(2 x 2, 3 x 3),
+ * 16 multiplies per 2 x 2 outputs of a channel pair instead of 36, or F(4 x 4, 3 x 3), 36 per
+ * 4 x 4 outputs instead of 144 -- whichever needs fewer products for the plane at hand, the
+ * smaller tile on a near tie --, F(4 x 4, 5 x 5), 64 per 4 x 4 outputs instead of 400: as 16 / 36 /
+ * 64 matrix products between transforms of 4 x 4 / 6 x 6 / 8 x 8 tiles, summed in fp32;
+ * backward_filter by F(3 x 3, m x m) / F(5 x 5, 4 x 4) with the sum over the tiles as the products'
+ * reduction.  Results differ from the direct sum by a few 1e-6 of the output's norm (up to
+ * about 6e-6 with 6 x 6 tiles, up to about 2.5e-5 with 8 x 8 tiles; the bound of the
+ * convolutions is 1e-4).  forward / backward_data need a bottom / top
  * channel count that is a multiple of 16.  The path wants the workspace the size queries
- * report (16 / 36 transformed values per tile and channel of both tensors), 16-byte aligned;
+ * report (16 / 36 / 64 transformed values per tile and channel of both tensors), 16-byte aligned;
  * with less it runs in groups of images, with less than one image needs the direct kernels
  * run. ---- */
 /* Selects when the three passes take the minimal-filtering path.  0: never; 1 (initial):
- * where the geometry makes it faster (at least 32 input channels, channel counts that fill
- * 128-wide tiles to three quarters, at least 1024 tiles of 2 x 2 or 512 of 4 x 4 outputs per
- * launch, output extents whose rounding up to whole 2 x 2 tiles wastes at most 40%); 2:
- * wherever it applies; 3 / 4: as 2 with the tile pinned to 2 x 2 / 4 x 4 outputs.
+ * where a cost estimate from the extents (multiplies saved against transformed values moved;
+ * in practice layers of about 200 channels and more whose direct pass takes over 100 us)
+ * puts it at 80% of the direct kernels' time or less; 2: wherever it applies; 3 / 4: as 2
+ * with the tile pinned to 2 x 2 / 4 x 4 outputs (3: 5 x 5 filters stay direct).
  * Process-wide; returns the previous mode; any other value only queries.  No reference
  * counterpart: cuDNN picks its algorithm out of sight (CUDNN_CONVOLUTION_FWD_PREFER_FASTEST,
  * cuda_perform.cu:227-264). */
 int mnv_conv_winograd_mode(int mode);
+/* Measurement aid (no reference counterpart; a benchmark's way to time the MFMA kernel of a
+ * minimal-filtering pass apart from the transform kernels around it).  While enabled, every
+ * launch of the matrix products of such a pass is bracketed by an event pair on its stream
+ * (about 4 us of idle GPU per launch); enabling drops earlier records.  _read waits for the
+ * recorded launches of one kind (0: forward / backward_data products, 1: backward_filter
+ * products with the reduction of their shares) and reports their number, their summed device
+ * milliseconds and the flops of the products (2 x points x channels x channels x tiles).
+ * Not for use while a stream is being captured into a graph. */
+int mnv_conv_winograd_profile(int enable);
+int mnv_conv_winograd_profile_read(int kind, int* launches, double* milliseconds, double* gflop);
 size_t mnv_conv_fwd_workspace_bytes(int num_images, int bottom_num_channels,
                                    int top_num_channels, int bottom_height, int bottom_width,
                                    int pad_height, int pad_width, int stride_vertical,

@@ -99,6 +99,8 @@ PROTOTYPES["mnv_sgemm_nt"] = [_P, _P, _P, _I, _I, _I, _P, c_sz, _S]
 PROTOTYPES["mnv_sgemm_nt_sgd"] = [_P, _P, _P, c_f, _P, _I, _I, _I, _P, c_sz, _S]
 PROTOTYPES["mnv_conv_bwd_filter_plan"] = [_I] * 11 + [c_sz, _P, _P, _P]
 PROTOTYPES["mnv_conv_winograd_mode"] = [_I]
+PROTOTYPES["mnv_conv_winograd_profile"] = [_I]
+PROTOTYPES["mnv_conv_winograd_profile_read"] = [_I, _P, _P, _P]
 PROTOTYPES["mnv_conv_bwd_filter_sgd"] = [_P, _P, _P, c_f, _P] + [_I] * 11 + [_P, c_sz, _S]
 PROTOTYPES["mnv_copy_2d"] = [_P, _P, c_sz, c_sz, c_sz, c_sz, _S]
 PROTOTYPES["mnv_select_workspace_bytes"] = [_I]

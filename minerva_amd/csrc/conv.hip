@@ -904,7 +904,7 @@ size_t mnv_conv_fwd_workspace_bytes(int N, int C, int K, int H, int W, int ph, i
   size_t need = tail ? align256(permuted) + tail
                      : splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
   if (mnv_wino_images(N, C, K, H, W, ph, pw, R, S, sv, sh, (size_t)-1)) {
-    const size_t w = mnv_wino_workspace_bytes(N, C, K, H, W, ph, pw);
+    const size_t w = mnv_wino_workspace_bytes(N, C, K, H, W, ph, pw, R);
     if (w > need) need = w;
   }
   return need;
@@ -924,7 +924,7 @@ static int conv_fwd_impl(const float* bottom, const float* filter, const float* 
   // (its transformed tensors are read and written in 16-byte vectors)
   if (const int images = mnv_wino_images(N, C, K, H, W, ph, pw, R, S, sv, sh,
                                          workspace && mnv_aligned16(workspace) ? workspace_bytes : 0))
-    return mnv_wino_conv(bottom, filter, bias, nullptr, top, N, C, K, H, W, ph, pw, 0, relu, images,
+    return mnv_wino_conv(bottom, filter, bias, nullptr, top, N, C, K, H, W, ph, pw, R, 0, relu, images,
                          workspace, workspace_bytes, s);
   const int tile = pick_tile(gm, gn);
   const size_t permuted_bytes = (size_t)K * g.CRS * sizeof(float);
@@ -997,8 +997,8 @@ size_t mnv_conv_bwd_data_workspace_bytes(int N, int C, int K, int H, int W, int 
   const size_t tail = tail_workspace_bytes(pick_tile(gm, gn), gm, gn, (K * g.RS + 15) / 16);
   size_t need = tail ? align256(permuted) + tail
                      : splits > 1 ? align256(permuted) + (size_t)splits * gm * gn * sizeof(float) : permuted;
-  if (mnv_wino_images(N, K, C, g.Ho, g.Wo, 2 - ph, 2 - pw, R, S, sv, sh, (size_t)-1)) {
-    const size_t w = mnv_wino_workspace_bytes(N, K, C, g.Ho, g.Wo, 2 - ph, 2 - pw);
+  if (mnv_wino_images(N, K, C, g.Ho, g.Wo, R - 1 - ph, S - 1 - pw, R, S, sv, sh, (size_t)-1)) {
+    const size_t w = mnv_wino_workspace_bytes(N, K, C, g.Ho, g.Wo, R - 1 - ph, S - 1 - pw, R);
     if (w > need) need = w;
   }
   return need;
@@ -1014,11 +1014,11 @@ static int conv_bwd_data_impl(const float* top_diff, const float* filter, const 
   if (rc) return rc;
   int gm = N * g.HW, gn = C, gk = K * g.RS;
   hipStream_t s = mnv_stream(stream);
-  // the same correlation, of top_diff with the unflipped filters, under a padding of 2 - pad
-  if (const int images = mnv_wino_images(N, K, C, g.Ho, g.Wo, 2 - ph, 2 - pw, R, S, sv, sh,
+  // the same correlation, of top_diff with the unflipped filters, under a padding of R - 1 - pad
+  if (const int images = mnv_wino_images(N, K, C, g.Ho, g.Wo, R - 1 - ph, S - 1 - pw, R, S, sv, sh,
                                          workspace && mnv_aligned16(workspace) ? workspace_bytes : 0))
-    return mnv_wino_conv(top_diff, filter, nullptr, gate, bottom_diff, N, K, C, g.Ho, g.Wo, 2 - ph,
-                         2 - pw, 1, 0, images, workspace, workspace_bytes, s);
+    return mnv_wino_conv(top_diff, filter, nullptr, gate, bottom_diff, N, K, C, g.Ho, g.Wo, R - 1 - ph,
+                         S - 1 - pw, R, 1, 0, images, workspace, workspace_bytes, s);
   const int tile = pick_tile(gm, gn);
   const size_t permuted_bytes = (size_t)K * g.CRS * sizeof(float);
   const bool fast = sv == 1 && sh == 1 && K % 16 == 0 && workspace && workspace_bytes >= permuted_bytes;
@@ -1090,7 +1090,7 @@ size_t mnv_conv_bwd_filter_workspace_bytes(int N, int C, int K, int H, int W, in
     if (tiles <= 4LL * mnv_cu_count() && sk > bytes) bytes = sk;
   }
   if (mnv_wino_grad_images(N, C, K, H, W, ph, pw, R, S, sv, sh, (size_t)-1)) {
-    const size_t w = mnv_wino_grad_workspace_bytes(N, C, K, H, W, ph, pw);
+    const size_t w = mnv_wino_grad_workspace_bytes(N, C, K, H, W, ph, pw, R);
     if (w > bytes) bytes = w;
   }
   return bytes;
@@ -1111,7 +1111,7 @@ static int conv_bwd_filter_impl(const float* bottom, const float* top_diff, floa
   // 3 x 3 unit-stride layers with enough channels and tiles: F(3 x 3, 2 x 2), see winograd.hip
   if (const int images = mnv_wino_grad_images(N, C, K, H, W, ph, pw, R, S, sv, sh,
                                               workspace && (plan || mnv_aligned16(workspace)) ? workspace_bytes : 0))
-    return mnv_wino_filter_grad(bottom, top_diff, filter_diff, N, C, K, H, W, ph, pw, images,
+    return mnv_wino_filter_grad(bottom, top_diff, filter_diff, N, C, K, H, W, ph, pw, R, images,
                                 accumulate, sgd_w, sgd_scale, workspace, workspace_bytes, s, plan);
   int splits = bwd_filter_splits(gm, gn, gk, workspace ? workspace_bytes / sizeof(float) : 0);
   const int tile = bwd_filter_tile(gm, gn);

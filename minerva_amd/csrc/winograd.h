@@ -13,7 +13,7 @@ int mnv_wino_images(int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad
                     int sv, int sh, size_t workspace_bytes);
 
 // Bytes the pass wants to run all N images as one group.
-size_t mnv_wino_workspace_bytes(int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w);
+size_t mnv_wino_workspace_bytes(int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w, int R);
 
 // dst {N, Cout, Hs + 2 pad_h - 2, Ws + 2 pad_w - 2} = correlation of src {N, Cin, Hs, Ws} with
 // the 3 x 3 filters.  `filter` is the caller's {K, C, 3, 3} tensor: forward (transposed = 0)
@@ -21,7 +21,7 @@ size_t mnv_wino_workspace_bytes(int N, int Cin, int Cout, int Hs, int Ws, int pa
 // stored.  Epilogue in this order, each optional: + bias[co]; max(., 0); kept where gate > 0.
 // `images`: what mnv_wino_images returned for this workspace.
 int mnv_wino_conv(const float* src, const float* filter, const float* bias, const float* gate,
-                  float* dst, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w,
+                  float* dst, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w, int R,
                   int transposed, int relu, int images, void* workspace, size_t workspace_bytes,
                   hipStream_t s);
 
@@ -32,12 +32,12 @@ int mnv_wino_conv(const float* src, const float* filter, const float* bias, cons
 // with more than one group the products accumulate group by group.
 int mnv_wino_grad_images(int N, int C, int K, int H, int W, int ph, int pw, int R, int S, int sv,
                          int sh, size_t workspace_bytes);
-size_t mnv_wino_grad_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw);
+size_t mnv_wino_grad_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw, int R);
 // filter_diff {K, C, 3, 3} = the gradient; `accumulate`: added to what is there; `sgd_w`: the value
 // stored is sgd_w - sgd_scale * gradient.  `plan` (optional): nothing is launched, plan[0] =
 // rows of the tile, plan[1] = 1, plan[2] = workgroups of the equal-shares launch (0: the product
 // is too small for it and runs one workgroup per tile).
 int mnv_wino_filter_grad(const float* bottom, const float* top_diff, float* filter_diff, int N, int C,
-                         int K, int H, int W, int ph, int pw, int images, int accumulate,
+                         int K, int H, int W, int ph, int pw, int R, int images, int accumulate,
                          const float* sgd_w, float sgd_scale, void* workspace,
                          size_t workspace_bytes, hipStream_t s, int* plan);

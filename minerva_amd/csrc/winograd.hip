@@ -34,6 +34,9 @@
 // Roofline: the matrix products are MFMA-bound (2 * al^2 * Cout * Cin * tiles flops); the
 // transform kernels stream al^2 * 4 bytes per (channel, tile) and are HBM-bound.
 
+#include <mutex>
+#include <vector>
+
 #include "gemm_core.h"
 #include "winograd.h"
 
@@ -43,17 +46,17 @@ struct WinoGeom {
   int N, Cin, Cout, Coutp;  // Coutp: Cout rounded up to the tile width of the product
   int Hs, Ws, Hd, Wd;       // source and destination planes
   int pad_h, pad_w;         // of the correlation: d[a][b] = src[m th - pad_h + a][m tw - pad_w + b]
-  int al, m;                // points per dimension (4 or 6), outputs per tile and dimension (al - 2)
+  int al, r, m;             // points per dimension, filter extent, outputs per tile and dimension (al - r + 1)
   int TH, TW, P, Pp;        // tiles per plane, tiles in all, P rounded up to 4
   MnvFastDiv d_T, d_TW, d_Cin;
 };
 
 // The matrices of one tile size as compile-time functions, so that the unrolled transforms
 // below fold every coefficient (zeros cost nothing, +-1 no multiply).
-template <int AL>
+template <int AL, int R>
 struct WinoF;
 template <>
-struct WinoF<4> {
+struct WinoF<4, 3> {
   struct BT { static constexpr int R = 4, C = 4;
     __host__ __device__ static constexpr float at(int i, int j) {
       constexpr float t[4][4] = {{1, 0, -1, 0}, {0, 1, 1, 0}, {0, -1, 1, 0}, {0, 1, 0, -1}};
@@ -76,7 +79,7 @@ struct WinoF<4> {
       return t[i][j]; } };
 };
 template <>
-struct WinoF<6> {
+struct WinoF<6, 3> {
   struct BT { static constexpr int R = 6, C = 6;
     __host__ __device__ static constexpr float at(int i, int j) {
       constexpr float t[6][6] = {{1, 1.5f, -2, -1.5f, 1, 0},
@@ -103,6 +106,44 @@ struct WinoF<6> {
   struct AAT { static constexpr int R = 3, C = 6;
     __host__ __device__ static constexpr float at(int i, int j) {
       constexpr float t[3][6] = {{1, 1, 1, 1, 1, 0}, {0, 1, -1, 2, -.5f, 0}, {0, 1, 1, 4, .25f, 1}};
+      return t[i][j]; } };
+};
+// 5 x 5 filters, 4 x 4 outputs per tile: the points {0, 1, -1, 2, -2, 1/2, -1/2, inf}
+template <>
+struct WinoF<8, 5> {
+  struct BT { static constexpr int R = 8, C = 8;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[8][8] = {
+          {1, 0, -21.f / 4, 0, 21.f / 4, 0, -1, 0},
+          {0, -2.f / 9, -2.f / 9, 17.f / 18, 17.f / 18, -2.f / 9, -2.f / 9, 0},
+          {0, 2.f / 9, -2.f / 9, -17.f / 18, 17.f / 18, 2.f / 9, -2.f / 9, 0},
+          {0, 1.f / 180, 1.f / 360, -1.f / 36, -1.f / 72, 1.f / 45, 1.f / 90, 0},
+          {0, -1.f / 180, 1.f / 360, 1.f / 36, -1.f / 72, -1.f / 45, 1.f / 90, 0},
+          {0, 64.f / 45, 128.f / 45, -16.f / 9, -32.f / 9, 16.f / 45, 32.f / 45, 0},
+          {0, -64.f / 45, 128.f / 45, 16.f / 9, -32.f / 9, -16.f / 45, 32.f / 45, 0},
+          {0, -1, 0, 21.f / 4, 0, -21.f / 4, 0, 1}};
+      return t[i][j]; } };
+  struct G { static constexpr int R = 8, C = 5;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[8][5] = {{1, 0, 0, 0, 0}, {1, 1, 1, 1, 1}, {1, -1, 1, -1, 1}, {1, 2, 4, 8, 16},
+                                 {1, -2, 4, -8, 16}, {1, .5f, .25f, .125f, .0625f},
+                                 {1, -.5f, .25f, -.125f, .0625f}, {0, 0, 0, 0, 1}};
+      return t[i][j]; } };
+  struct AT { static constexpr int R = 4, C = 8;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[4][8] = {{1, 1, 1, 1, 1, 1, 1, 0}, {0, 1, -1, 2, -2, .5f, -.5f, 0},
+                                 {0, 1, 1, 4, 4, .25f, .25f, 0}, {0, 1, -1, 8, -8, .125f, -.125f, 1}};
+      return t[i][j]; } };
+  struct GG { static constexpr int R = 8, C = 4;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[8][4] = {{1, 0, 0, 0}, {1, 1, 1, 1}, {1, -1, 1, -1}, {1, 2, 4, 8}, {1, -2, 4, -8},
+                                 {1, .5f, .25f, .125f}, {1, -.5f, .25f, -.125f}, {0, 0, 0, 1}};
+      return t[i][j]; } };
+  struct AAT { static constexpr int R = 5, C = 8;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[5][8] = {{1, 1, 1, 1, 1, 1, 1, 0}, {0, 1, -1, 2, -2, .5f, -.5f, 0},
+                                 {0, 1, 1, 4, 4, .25f, .25f, 0}, {0, 1, -1, 8, -8, .125f, -.125f, 0},
+                                 {0, 1, 1, 16, 16, .0625f, .0625f, 1}};
       return t[i][j]; } };
 };
 
@@ -148,31 +189,31 @@ __device__ __forceinline__ void wino_cols(const float (&in)[K][L::C], float (&ou
     }
 }
 
-// U[point][co][ci] from filter[k][c][3][3].  Forward: co = k, ci = c, g[r][s] = f[2-r][2-s];
+// U[point][co][ci] from filter[k][c][R][R].  Forward: co = k, ci = c, g[r][s] = f[R-1-r][R-1-s];
 // data gradient (`transposed`): co = c, ci = k, g = f.  Rows co >= Cout are zero.
-template <int AL>
+template <int AL, int R>
 __global__ __launch_bounds__(256) void mnv_wino_filter_kernel(const float* __restrict__ filter,
                                                               float* __restrict__ U, WinoGeom g,
                                                               int K, int C, bool transposed) {
-  typedef WinoF<AL> F;
+  typedef WinoF<AL, R> F;
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= g.Coutp * g.Cin) return;
   const int co = mnv_fastdiv(t, g.d_Cin), ci = t - co * g.Cin;
-  float f[3][3];
+  float f[R][R];
   if (co < g.Cout) {
-    const float* src = transposed ? filter + ((size_t)ci * C + co) * 9 : filter + ((size_t)co * C + ci) * 9;
+    const float* src = transposed ? filter + ((size_t)ci * C + co) * (R * R) : filter + ((size_t)co * C + ci) * (R * R);
 #pragma unroll
-    for (int r = 0; r < 3; ++r)
+    for (int r = 0; r < R; ++r)
 #pragma unroll
-      for (int s = 0; s < 3; ++s) f[r][s] = transposed ? src[r * 3 + s] : src[(2 - r) * 3 + (2 - s)];
+      for (int s = 0; s < R; ++s) f[r][s] = transposed ? src[r * R + s] : src[(R - 1 - r) * R + (R - 1 - s)];
   } else {
 #pragma unroll
-    for (int r = 0; r < 3; ++r)
+    for (int r = 0; r < R; ++r)
 #pragma unroll
-      for (int s = 0; s < 3; ++s) f[r][s] = 0.f;
+      for (int s = 0; s < R; ++s) f[r][s] = 0.f;
   }
-  float h[AL][3], u[AL][AL];
-  wino_rows<typename F::G, 3>(f, h);
+  float h[AL][R], u[AL][AL];
+  wino_rows<typename F::G, R>(f, h);
   wino_cols<typename F::G, AL>(h, u);
   const size_t plane = (size_t)g.Coutp * g.Cin;
   float* out = U + (size_t)co * g.Cin + ci;
@@ -183,9 +224,9 @@ __global__ __launch_bounds__(256) void mnv_wino_filter_kernel(const float* __res
 }
 
 // V[point][ci][p] = (B^T d B)[point] of the al x al tile p of channel ci; p >= P writes zeros.
-template <int AL>
+template <int AL, int R>
 __device__ __forceinline__ void wino_store_v(float (&d)[AL][AL], float* __restrict__ out, size_t plane) {
-  typedef WinoF<AL> F;
+  typedef WinoF<AL, R> F;
   float h[AL][AL], v[AL][AL];
   wino_rows<typename F::BT, AL>(d, h);
   wino_cols<typename F::BT, AL>(h, v);
@@ -195,7 +236,7 @@ __device__ __forceinline__ void wino_store_v(float (&d)[AL][AL], float* __restri
     for (int nu = 0; nu < AL; ++nu) out[(xi * AL + nu) * plane] = v[xi][nu];
 }
 
-template <int AL>
+template <int AL, int R>
 __global__ __launch_bounds__(256) void mnv_wino_input_kernel(const float* __restrict__ src,
                                                              float* __restrict__ V, WinoGeom g) {
   const int p = blockIdx.x * 256 + threadIdx.x;
@@ -210,7 +251,7 @@ __global__ __launch_bounds__(256) void mnv_wino_input_kernel(const float* __rest
     const int img = mnv_fastdiv(p, g.d_T);
     const int t = p - img * (g.TH * g.TW);
     const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
-    const int y0 = (AL - 2) * th - g.pad_h, x0 = (AL - 2) * tw - g.pad_w;
+    const int y0 = (AL - R + 1) * th - g.pad_h, x0 = (AL - R + 1) * tw - g.pad_w;
     const float* plane = src + ((size_t)img * g.Cin + ci) * (g.Hs * g.Ws);
 #pragma unroll
     for (int a = 0; a < AL; ++a)
@@ -220,7 +261,7 @@ __global__ __launch_bounds__(256) void mnv_wino_input_kernel(const float* __rest
         if ((unsigned)y < (unsigned)g.Hs && (unsigned)x < (unsigned)g.Ws) d[a][b] = plane[y * g.Ws + x];
       }
   }
-  wino_store_v<AL>(d, V + (size_t)ci * g.Pp + p, (size_t)g.Cin * g.Pp);
+  wino_store_v<AL, R>(d, V + (size_t)ci * g.Pp + p, (size_t)g.Cin * g.Pp);
 }
 
 // The same through LDS, for planes small enough that the planes of the images a workgroup's
@@ -229,7 +270,7 @@ __global__ __launch_bounds__(256) void mnv_wino_input_kernel(const float* __rest
 // thread at a stride of a few bytes between neighbouring tiles (F(2 x 2) on 384 channels of
 // 256 x 13 x 13: 107 -> 80 us).  One channel per workgroup: four (the tile arithmetic done once
 // for four) measured 84.7 against 79.6 us.
-template <int AL>
+template <int AL, int R>
 __global__ __launch_bounds__(256) void mnv_wino_input_lds_kernel(const float* __restrict__ src,
                                                                  float* __restrict__ V, WinoGeom g,
                                                                  MnvFastDiv d_HW) {
@@ -255,7 +296,7 @@ __global__ __launch_bounds__(256) void mnv_wino_input_lds_kernel(const float* __
     const int img = mnv_fastdiv(p, g.d_T);
     const int t = p - img * (g.TH * g.TW);
     const int th = mnv_fastdiv(t, g.d_TW), tw = t - th * g.TW;
-    const int y0 = (AL - 2) * th - g.pad_h, x0 = (AL - 2) * tw - g.pad_w;
+    const int y0 = (AL - R + 1) * th - g.pad_h, x0 = (AL - R + 1) * tw - g.pad_w;
     const float* plane = planes + (img - img0) * HW;
 #pragma unroll
     for (int a = 0; a < AL; ++a)
@@ -265,20 +306,20 @@ __global__ __launch_bounds__(256) void mnv_wino_input_lds_kernel(const float* __
         if ((unsigned)y < (unsigned)g.Hs && (unsigned)x < (unsigned)g.Ws) d[a][b] = plane[y * g.Ws + x];
       }
   }
-  wino_store_v<AL>(d, V + (size_t)ci * g.Pp + p, (size_t)g.Cin * g.Pp);
+  wino_store_v<AL, R>(d, V + (size_t)ci * g.Pp + p, (size_t)g.Cin * g.Pp);
 }
 
 // dst[img][co][m th + a][m tw + b] = (A^T M A)[a][b] (+ bias[co]) (then max(., 0)) (then kept
 // only where gate > 0): the epilogues of the direct kernels, each the single operation of the
 // separate operator.
-template <int AL>
+template <int AL, int R>
 __global__ __launch_bounds__(256) void mnv_wino_output_kernel(const float* __restrict__ Mx,
                                                               const float* __restrict__ bias,
                                                               const float* __restrict__ gate,
                                                               float* __restrict__ dst, WinoGeom g,
                                                               int relu) {
-  typedef WinoF<AL> F;
-  constexpr int MO = AL - 2;
+  typedef WinoF<AL, R> F;
+  constexpr int MO = AL - R + 1;
   const int p = blockIdx.x * 256 + threadIdx.x;
   const int co = blockIdx.y;
   if (p >= g.P) return;
@@ -318,14 +359,14 @@ __global__ __launch_bounds__(256) void mnv_wino_output_kernel(const float* __res
 // stores every plane in runs of contiguous floats, where the kernel above stores m floats per
 // row and thread, neighbouring threads m floats apart (4 x 4 tiles on 384 channels of
 // 256 x 13 x 13: 95 us).  A pixel is stored by the workgroup that holds its tile.
-template <int AL>
+template <int AL, int R>
 __global__ __launch_bounds__(256) void mnv_wino_output_lds_kernel(const float* __restrict__ Mx,
                                                                   const float* __restrict__ bias,
                                                                   const float* __restrict__ gate,
                                                                   float* __restrict__ dst, WinoGeom g,
                                                                   int relu, MnvFastDiv d_HW, MnvFastDiv d_W) {
-  typedef WinoF<AL> F;
-  constexpr int MO = AL - 2;
+  typedef WinoF<AL, R> F;
+  constexpr int MO = AL - R + 1;
   extern __shared__ float planes[];
   const int p0 = blockIdx.x * 256, p = p0 + threadIdx.x;
   const int co = blockIdx.y;
@@ -431,11 +472,11 @@ struct WinoGemm {
 // ---- filter gradient
 // Yt[point][k][p] = (G' dy G'^T)[point] of the m x m tile p of channel k of top_diff; zeros
 // for p >= P and for the rows k >= Cout.
-template <int AL>
+template <int AL, int R>
 __global__ __launch_bounds__(256) void mnv_wino_grad_kernel(const float* __restrict__ top_diff,
                                                             float* __restrict__ Yt, WinoGeom g) {
-  typedef WinoF<AL> F;
-  constexpr int MO = AL - 2;
+  typedef WinoF<AL, R> F;
+  constexpr int MO = AL - R + 1;
   const int p = blockIdx.x * 256 + threadIdx.x;
   const int k = blockIdx.y;
   if (p >= g.Pp) return;
@@ -469,12 +510,12 @@ __global__ __launch_bounds__(256) void mnv_wino_grad_kernel(const float* __restr
 }
 
 // The same with the planes of top_diff fetched whole into LDS (see mnv_wino_input_lds_kernel).
-template <int AL>
+template <int AL, int R>
 __global__ __launch_bounds__(256) void mnv_wino_grad_lds_kernel(const float* __restrict__ top_diff,
                                                                 float* __restrict__ Yt, WinoGeom g,
                                                                 MnvFastDiv d_HW) {
-  typedef WinoF<AL> F;
-  constexpr int MO = AL - 2;
+  typedef WinoF<AL, R> F;
+  constexpr int MO = AL - R + 1;
   extern __shared__ float planes[];
   const int p0 = blockIdx.x * 256, p = p0 + threadIdx.x;
   const int k = blockIdx.y;
@@ -517,15 +558,15 @@ __global__ __launch_bounds__(256) void mnv_wino_grad_lds_kernel(const float* __r
     for (int nu = 0; nu < AL; ++nu) out[(xi * AL + nu) * plane] = v[xi][nu];
 }
 
-// filter_diff[k][c][2-r][2-s] = (A'^T Q A')[r][s] with the epilogues of the direct kernel's
+// filter_diff[k][c][R-1-r][R-1-s] = (A'^T Q A')[r][s] with the epilogues of the direct kernel's
 // store: the parameter update sgd_w - sgd_scale * ., or the sum with what is there.
-// (filter_diff may be sgd_w itself: a thread reads the nine parameters it then writes.)
-template <int AL>
+// (filter_diff may be sgd_w itself: a thread reads the R x R parameters it then writes.)
+template <int AL, int R>
 __global__ __launch_bounds__(256) void mnv_wino_grad_output_kernel(const float* __restrict__ Q,
                                                                    float* filter_diff, WinoGeom g,
                                                                    int accumulate, const float* sgd_w,
                                                                    float sgd_scale) {
-  typedef WinoF<AL> F;
+  typedef WinoF<AL, R> F;
   const int t = blockIdx.x * 256 + threadIdx.x;
   if (t >= g.Cout * g.Cin) return;
   const int k = mnv_fastdiv(t, g.d_Cin), c = t - k * g.Cin;
@@ -536,17 +577,17 @@ __global__ __launch_bounds__(256) void mnv_wino_grad_output_kernel(const float* 
   for (int xi = 0; xi < AL; ++xi)
 #pragma unroll
     for (int nu = 0; nu < AL; ++nu) q[xi][nu] = in[(xi * AL + nu) * plane];
-  float h[3][AL], dg[3][3];
+  float h[R][AL], dg[R][R];
   wino_rows<typename F::AAT, AL>(q, h);
-  wino_cols<typename F::AAT, 3>(h, dg);
-  float* out = filter_diff + (size_t)t * 9;
+  wino_cols<typename F::AAT, R>(h, dg);
+  float* out = filter_diff + (size_t)t * (R * R);
 #pragma unroll
-  for (int r = 0; r < 3; ++r)
+  for (int r = 0; r < R; ++r)
 #pragma unroll
-    for (int s = 0; s < 3; ++s) {
-      const int at = (2 - r) * 3 + (2 - s);
+    for (int s = 0; s < R; ++s) {
+      const int at = (R - 1 - r) * R + (R - 1 - s);
       float x = dg[r][s];
-      if (sgd_w) x = sgd_w[(size_t)t * 9 + at] - sgd_scale * x;
+      if (sgd_w) x = sgd_w[(size_t)t * (R * R) + at] - sgd_scale * x;
       else if (accumulate) x = out[at] + x;
       out[at] = x;
     }
@@ -602,6 +643,46 @@ struct WinoGradGemm {
 
 typedef MnvGemmTile<128, 128, 16, 2, 2> TileBig;
 
+// Measurement aid (mnv_conv_winograd_profile): while it is on, every launch of the products
+// is bracketed by an event pair on its stream, so that a benchmark can time the MFMA kernel of
+// a pass apart from the transform kernels around it.
+struct ProductProfile {
+  struct Rec {
+    hipEvent_t begin, end;
+    double flops;
+    int kind;  // 0: forward / data gradient, 1: filter gradient (with the reduction of its shares)
+  };
+  std::mutex mu;
+  bool on = false;
+  std::vector<Rec> recs;
+  void drop() {
+    for (auto& r : recs) {
+      (void)hipEventDestroy(r.begin);
+      (void)hipEventDestroy(r.end);
+    }
+    recs.clear();
+  }
+};
+ProductProfile g_profile;
+
+// the event pair of one launch, or false when the profile is off
+bool profile_begin(hipEvent_t* begin, hipEvent_t* end, hipStream_t s) {
+  std::lock_guard<std::mutex> lock(g_profile.mu);
+  if (!g_profile.on) return false;
+  if (hipEventCreate(begin) != hipSuccess) return false;
+  if (hipEventCreate(end) != hipSuccess) {
+    (void)hipEventDestroy(*begin);
+    return false;
+  }
+  (void)hipEventRecord(*begin, s);
+  return true;
+}
+void profile_end(hipEvent_t begin, hipEvent_t end, hipStream_t s, int kind, double flops) {
+  (void)hipEventRecord(end, s);
+  std::lock_guard<std::mutex> lock(g_profile.mu);
+  g_profile.recs.push_back({begin, end, flops, kind});
+}
+
 inline size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
 
 // Mode of mnv_conv_winograd_mode: 0 never, 1 where it pays, 2 wherever it applies, 3 / 4 as 2
@@ -611,7 +692,8 @@ std::atomic<int> g_mode{1};
 // Points per dimension for an Hd x Wd output plane: 6 (4 x 4 outputs per tile) when that needs
 // at most 85% of the products of 4 (2 x 2 outputs per tile); its results are a few times
 // further from the direct sum, so a near tie goes to the smaller tile.
-int pick_points(int Hd, int Wd, int mode) {
+int pick_points(int Hd, int Wd, int R, int mode) {
+  if (R == 5) return mode == 3 ? 0 : 8;  // 5 x 5 filters: 4 x 4 outputs per 8 x 8 tile or not at all
   if (mode == 3) return 4;
   if (mode == 4) return 6;
   const long long small = 16LL * ((Hd + 1) / 2) * ((Wd + 1) / 2);
@@ -620,14 +702,15 @@ int pick_points(int Hd, int Wd, int mode) {
 }
 
 int make_wino_geom(WinoGeom* g, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w,
-                   int al) {
-  if (N <= 0 || Cin <= 0 || Cout <= 0 || Hs <= 0 || Ws <= 0 || pad_h < 0 || pad_w < 0 || pad_h > 2 ||
-      pad_w > 2 || Hs + 2 * pad_h < 3 || Ws + 2 * pad_w < 3 || (al != 4 && al != 6))
+                   int al, int r) {
+  if (N <= 0 || Cin <= 0 || Cout <= 0 || Hs <= 0 || Ws <= 0 || pad_h < 0 || pad_w < 0 || pad_h > r - 1 ||
+      pad_w > r - 1 || Hs + 2 * pad_h < r || Ws + 2 * pad_w < r ||
+      !((r == 3 && (al == 4 || al == 6)) || (r == 5 && al == 8)))
     return MNV_ERR_INVALID;
   g->N = N; g->Cin = Cin; g->Cout = Cout; g->Coutp = (Cout + 127) / 128 * 128;
-  g->Hs = Hs; g->Ws = Ws; g->Hd = Hs + 2 * pad_h - 2; g->Wd = Ws + 2 * pad_w - 2;
+  g->Hs = Hs; g->Ws = Ws; g->Hd = Hs + 2 * pad_h - (r - 1); g->Wd = Ws + 2 * pad_w - (r - 1);
   g->pad_h = pad_h; g->pad_w = pad_w;
-  g->al = al; g->m = al - 2;
+  g->al = al; g->r = r; g->m = al - r + 1;
   g->TH = (g->Hd + g->m - 1) / g->m; g->TW = (g->Wd + g->m - 1) / g->m;
   const long long P = (long long)N * g->TH * g->TW;
   if (P > (1LL << 28)) return MNV_ERR_INVALID;
@@ -642,16 +725,16 @@ int make_wino_geom(WinoGeom* g, int N, int Cin, int Cout, int Hs, int Ws, int pa
 }
 
 // V of the group of images that `g` describes
-template <int AL>
+template <int AL, int R>
 int launch_input_transform(const float* src, float* V, const WinoGeom& g, hipStream_t s) {
   const int T = g.TH * g.TW, HW = g.Hs * g.Ws;
   // planes a workgroup's 256 consecutive tiles can touch
   const size_t lds = (size_t)(255 / T + 2) * HW * sizeof(float);
   if (lds <= 32 * 1024)
-    hipLaunchKernelGGL(mnv_wino_input_lds_kernel<AL>, dim3((g.Pp + 255) / 256, g.Cin), dim3(256), lds,
+    hipLaunchKernelGGL((mnv_wino_input_lds_kernel<AL, R>), dim3((g.Pp + 255) / 256, g.Cin), dim3(256), lds,
                        s, src, V, g, mnv_fastdiv_make(HW));
   else
-    hipLaunchKernelGGL(mnv_wino_input_kernel<AL>, dim3((g.Pp + 255) / 256, g.Cin), dim3(256), 0, s, src,
+    hipLaunchKernelGGL((mnv_wino_input_kernel<AL, R>), dim3((g.Pp + 255) / 256, g.Cin), dim3(256), 0, s, src,
                        V, g);
   return MNV_LAUNCH_STATUS();
 }
@@ -691,24 +774,37 @@ bool plan_geom(WinoGeom* g, int* mode_out, int N, int Cin, int Cout, int Hs, int
                int R, int S, int sv, int sh) {
   const int mode = g_mode.load(std::memory_order_relaxed);
   *mode_out = mode;
-  if (mode == 0 || R != 3 || S != 3 || sv != 1 || sh != 1 || pad_h < 0 || pad_w < 0 || pad_h > 2 ||
-      pad_w > 2 || Hs + 2 * pad_h < 3 || Ws + 2 * pad_w < 3)
+  if (mode == 0 || R != S || (R != 3 && R != 5) || sv != 1 || sh != 1 || pad_h < 0 || pad_w < 0 ||
+      pad_h > R - 1 || pad_w > R - 1 || Hs + 2 * pad_h < R || Ws + 2 * pad_w < R)
     return false;
-  const int al = pick_points(Hs + 2 * pad_h - 2, Ws + 2 * pad_w - 2, mode);
-  return make_wino_geom(g, N, Cin, Cout, Hs, Ws, pad_h, pad_w, al) == MNV_OK;
+  const int al = pick_points(Hs + 2 * pad_h - (R - 1), Ws + 2 * pad_w - (R - 1), R, mode);
+  return al && make_wino_geom(g, N, Cin, Cout, Hs, Ws, pad_h, pad_w, al, R) == MNV_OK;
 }
 
-// mode 1: enough channels to fill the tiles of the products, enough tiles, and output extents
-// whose rounding up to whole tiles wastes at most 40% (al = 4) -- with al = 6 the choice of
-// the tile size has already weighed the waste
-bool pays(const WinoGeom& g, int images, int m_extent) {
-  const long long tiles = (long long)images * g.TH * g.TW;
-  const bool fills = m_extent < 0 || m_extent * 4 >= (m_extent + 127) / 128 * 128 * 3;
-  return g.Cin >= 32 && fills && g.Cout * 4 >= g.Coutp * 3 && tiles * (g.al * g.al / 16) >= 1024 &&
-         (g.al == 6 || 4LL * g.TH * g.TW * 5 <= 7LL * g.Hd * g.Wd);
+// Mode 1: the path is taken where a cost estimate puts it at 80% of the direct kernel's time
+// or less, and the direct kernel's estimate is at least 100 us (four or five launches instead
+// of one).  Per output pixel and image, with pts = transformed values per output (al^2 / m^2,
+// times the waste of rounding the plane up to whole tiles):
+//   direct   2 r^2 Cin Cout flops at 130 TFLOP/s (what the direct kernels sustain);
+//   filtered pts (Cin + Coutp) values written and read once, 8 bytes each way, at 5 TB/s (the
+//            transform kernels), plus 2 pts Cin' Coutp flops at the rate this core reaches on
+//            the products: 157 TFLOP/s x k / (k + 64 slab-equivalents of prologue and store),
+//            k = Cin for forward / data gradient, 0.85 for the filter gradient's long k
+//            (Cin' = Cin rounded up to the 128-row tile there).
+// Checked against the batch-256 layers: 96 -> 256 channels under 5 x 5 filters 0.46 estimated,
+// 0.43 measured; 256 -> 384 under 3 x 3 on 13 x 13 planes 0.65 / 0.63.  Layers of 128 channels
+// and fewer stay direct: the transforms alone cost what the multiplies save.
+bool pays(const WinoGeom& g, int images, bool filter_gradient) {
+  const double px = (double)g.Hd * g.Wd;
+  const double pts = (double)g.al * g.al * g.TH * g.TW / px;
+  const double direct = 2.0 * g.r * g.r * g.Cin * g.Cout / 130e12;
+  const double rate = filter_gradient ? 0.85 : (double)g.Cin / (g.Cin + 64.0);
+  const double rows = filter_gradient ? (g.Cin + 127) / 128 * 128 : g.Cin;
+  const double filtered = pts * (g.Cin + g.Coutp) * 8.0 / 5e12 + 2.0 * pts * rows * g.Coutp / (rate * 157.3e12);
+  return filtered <= 0.8 * direct && direct * px * images >= 100e-6;
 }
 
-template <int AL>
+template <int AL, int R>
 int wino_conv(const WinoGeom& g0, const float* src, const float* filter, const float* bias,
               const float* gate, float* dst, int N, int transposed, int relu, int images,
               void* workspace, hipStream_t s) {
@@ -721,24 +817,28 @@ int wino_conv(const WinoGeom& g0, const float* src, const float* filter, const f
   w += align256((size_t)AL * AL * g.Pp * Cin * sizeof(float));
   float* Mx = reinterpret_cast<float*>(w);
   const int K = transposed ? Cin : Cout, C = transposed ? Cout : Cin;
-  hipLaunchKernelGGL(mnv_wino_filter_kernel<AL>, dim3((g.Coutp * Cin + 255) / 256), dim3(256), 0, s,
+  hipLaunchKernelGGL((mnv_wino_filter_kernel<AL, R>), dim3((g.Coutp * Cin + 255) / 256), dim3(256), 0, s,
                      filter, U, g, K, C, transposed != 0);
   int rc = MNV_LAUNCH_STATUS();
   if (rc) return rc;
   const size_t per_src = (size_t)Cin * g.Hs * g.Ws, per_dst = (size_t)Cout * g.Hd * g.Wd;
   for (int n0 = 0; n0 < N; n0 += images) {
     const int nn = N - n0 < images ? N - n0 : images;
-    if (nn != g.N && (rc = make_wino_geom(&g, nn, Cin, Cout, g.Hs, g.Ws, g.pad_h, g.pad_w, AL))) return rc;
-    if ((rc = launch_input_transform<AL>(src + n0 * per_src, V, g, s))) return rc;
+    if (nn != g.N && (rc = make_wino_geom(&g, nn, Cin, Cout, g.Hs, g.Ws, g.pad_h, g.pad_w, AL, R))) return rc;
+    if ((rc = launch_input_transform<AL, R>(src + n0 * per_src, V, g, s))) return rc;
     WinoGemm p{V, U, Mx, g.Pp, AL * AL * g.Coutp, Cin, Cin / 16, Cin / 16, g.Coutp, g.Coutp / 128};
-    if ((rc = mnv_gemm_launch<TileBig>(p, 1, nullptr, s))) return rc;
+    hipEvent_t e0, e1;
+    const bool timed = profile_begin(&e0, &e1, s);
+    rc = mnv_gemm_launch<TileBig>(p, 1, nullptr, s);
+    if (timed) profile_end(e0, e1, s, 0, 2.0 * AL * AL * Cout * Cin * g.P);
+    if (rc) return rc;
     const size_t lds = (size_t)(255 / (g.TH * g.TW) + 2) * g.Hd * g.Wd * sizeof(float);
     if (lds <= 32 * 1024)
-      hipLaunchKernelGGL(mnv_wino_output_lds_kernel<AL>, dim3((g.P + 255) / 256, Cout), dim3(256), lds, s,
+      hipLaunchKernelGGL((mnv_wino_output_lds_kernel<AL, R>), dim3((g.P + 255) / 256, Cout), dim3(256), lds, s,
                          Mx, bias, gate ? gate + n0 * per_dst : nullptr, dst + n0 * per_dst, g, relu,
                          mnv_fastdiv_make(g.Hd * g.Wd), mnv_fastdiv_make(g.Wd));
     else
-      hipLaunchKernelGGL(mnv_wino_output_kernel<AL>, dim3((g.P + 255) / 256, Cout), dim3(256), 0, s, Mx,
+      hipLaunchKernelGGL((mnv_wino_output_kernel<AL, R>), dim3((g.P + 255) / 256, Cout), dim3(256), 0, s, Mx,
                          bias, gate ? gate + n0 * per_dst : nullptr, dst + n0 * per_dst, g, relu);
     if ((rc = MNV_LAUNCH_STATUS())) return rc;
   }
@@ -748,7 +848,7 @@ int wino_conv(const WinoGeom& g0, const float* src, const float* filter, const f
 #ifndef MNV_WINO_SK_PF
 #define MNV_WINO_SK_PF 1
 #endif
-template <int AL>
+template <int AL, int R>
 int wino_filter_grad(const WinoGeom& g0, const float* bottom, const float* top_diff, float* filter_diff,
                      int N, int images, int accumulate, const float* sgd_w, float sgd_scale,
                      void* workspace, hipStream_t s, int* plan) {
@@ -775,23 +875,27 @@ int wino_filter_grad(const WinoGeom& g0, const float* bottom, const float* top_d
   const size_t per_bottom = (size_t)C * g.Hs * g.Ws, per_top = (size_t)K * g.Hd * g.Wd;
   for (int n0 = 0; n0 < N; n0 += images) {
     const int nn = N - n0 < images ? N - n0 : images;
-    if (nn != g.N && (rc = make_wino_geom(&g, nn, C, K, g.Hs, g.Ws, g.pad_h, g.pad_w, AL))) return rc;
-    if ((rc = launch_input_transform<AL>(bottom + n0 * per_bottom, V, g, s))) return rc;
+    if (nn != g.N && (rc = make_wino_geom(&g, nn, C, K, g.Hs, g.Ws, g.pad_h, g.pad_w, AL, R))) return rc;
+    if ((rc = launch_input_transform<AL, R>(bottom + n0 * per_bottom, V, g, s))) return rc;
     const size_t lds = (size_t)(255 / (g.TH * g.TW) + 2) * g.Hd * g.Wd * sizeof(float);
     if (lds <= 32 * 1024)
-      hipLaunchKernelGGL(mnv_wino_grad_lds_kernel<AL>, dim3((g.Pp + 255) / 256, g.Coutp), dim3(256), lds, s,
+      hipLaunchKernelGGL((mnv_wino_grad_lds_kernel<AL, R>), dim3((g.Pp + 255) / 256, g.Coutp), dim3(256), lds, s,
                          top_diff + n0 * per_top, Yt, g, mnv_fastdiv_make(g.Hd * g.Wd));
     else
-      hipLaunchKernelGGL(mnv_wino_grad_kernel<AL>, dim3((g.Pp + 255) / 256, g.Coutp), dim3(256), 0, s,
+      hipLaunchKernelGGL((mnv_wino_grad_kernel<AL, R>), dim3((g.Pp + 255) / 256, g.Coutp), dim3(256), 0, s,
                          top_diff + n0 * per_top, Yt, g);
     if ((rc = MNV_LAUNCH_STATUS())) return rc;
     WinoGradGemm p{V, Yt, Q, C, AL * AL * g.Coutp, g.Pp, (g.Pp + 15) / 16, g.Pp >= 16 ? g.Pp / 16 : 1,
                    g.Coutp, n0 > 0};
     bool done = false;
-    if ((rc = mnv_gemm_streamk_launch<TileBig, MNV_WINO_SK_PF>(p, w, sk_bytes, s, &done))) return rc;
-    if (!done && (rc = mnv_gemm_launch<TileBig>(p, 1, nullptr, s))) return rc;
+    hipEvent_t e0, e1;
+    const bool timed = profile_begin(&e0, &e1, s);
+    rc = mnv_gemm_streamk_launch<TileBig, MNV_WINO_SK_PF>(p, w, sk_bytes, s, &done);
+    if (!rc && !done) rc = mnv_gemm_launch<TileBig>(p, 1, nullptr, s);
+    if (timed) profile_end(e0, e1, s, 1, 2.0 * AL * AL * K * C * g.P);
+    if (rc) return rc;
   }
-  hipLaunchKernelGGL(mnv_wino_grad_output_kernel<AL>, dim3((K * C + 255) / 256), dim3(256), 0, s, Q,
+  hipLaunchKernelGGL((mnv_wino_grad_output_kernel<AL, R>), dim3((K * C + 255) / 256), dim3(256), 0, s, Q,
                      filter_diff, g, accumulate, sgd_w, sgd_scale);
   return MNV_LAUNCH_STATUS();
 }
@@ -803,10 +907,37 @@ extern "C" int mnv_conv_winograd_mode(int mode) {
   return g_mode.exchange(mode, std::memory_order_relaxed);
 }
 
-size_t mnv_wino_workspace_bytes(int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w) {
+extern "C" int mnv_conv_winograd_profile(int enable) {
+  std::lock_guard<std::mutex> lock(g_profile.mu);
+  if (enable) g_profile.drop();
+  g_profile.on = enable != 0;
+  return MNV_OK;
+}
+
+extern "C" int mnv_conv_winograd_profile_read(int kind, int* launches, double* milliseconds,
+                                              double* gflop) {
+  std::lock_guard<std::mutex> lock(g_profile.mu);
+  int n = 0;
+  double ms = 0, fl = 0;
+  for (auto& r : g_profile.recs) {
+    if (r.kind != kind) continue;
+    MNV_HIP_TRY(hipEventSynchronize(r.end));
+    float t = 0;
+    MNV_HIP_TRY(hipEventElapsedTime(&t, r.begin, r.end));
+    ++n;
+    ms += t;
+    fl += r.flops;
+  }
+  if (launches) *launches = n;
+  if (milliseconds) *milliseconds = ms;
+  if (gflop) *gflop = fl / 1e9;
+  return MNV_OK;
+}
+
+size_t mnv_wino_workspace_bytes(int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w, int R) {
   WinoGeom g;
   int mode;
-  if (!plan_geom(&g, &mode, N, Cin, Cout, Hs, Ws, pad_h, pad_w, 3, 3, 1, 1)) return 0;
+  if (!plan_geom(&g, &mode, N, Cin, Cout, Hs, Ws, pad_h, pad_w, R, R, 1, 1)) return 0;
   return u_bytes(g) + vm_bytes(g, N);
 }
 
@@ -818,27 +949,29 @@ int mnv_wino_images(int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad
   if (workspace_bytes < u_bytes(g)) return 0;
   const int images = images_that_fit(g, N, workspace_bytes - u_bytes(g));
   if (mode != 1 || images == 0) return images;
-  return pays(g, images, -1) ? images : 0;
+  return pays(g, images, false) ? images : 0;
 }
 
 int mnv_wino_conv(const float* src, const float* filter, const float* bias, const float* gate,
-                  float* dst, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w,
+                  float* dst, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w, int R,
                   int transposed, int relu, int images, void* workspace, size_t workspace_bytes,
                   hipStream_t s) {
   WinoGeom g;
   int mode;
   if (!src || !filter || !dst || images <= 0 || Cin % 16 != 0) return MNV_ERR_INVALID;
   if (images > N) images = N;
-  if (!plan_geom(&g, &mode, images, Cin, Cout, Hs, Ws, pad_h, pad_w, 3, 3, 1, 1)) return MNV_ERR_INVALID;
+  if (!plan_geom(&g, &mode, images, Cin, Cout, Hs, Ws, pad_h, pad_w, R, R, 1, 1)) return MNV_ERR_INVALID;
   if (!workspace || workspace_bytes < u_bytes(g) + vm_bytes(g, images)) return MNV_ERR_INVALID;
-  return g.al == 6 ? wino_conv<6>(g, src, filter, bias, gate, dst, N, transposed, relu, images, workspace, s)
-                   : wino_conv<4>(g, src, filter, bias, gate, dst, N, transposed, relu, images, workspace, s);
+  if (g.al == 8)
+    return wino_conv<8, 5>(g, src, filter, bias, gate, dst, N, transposed, relu, images, workspace, s);
+  return g.al == 6 ? wino_conv<6, 3>(g, src, filter, bias, gate, dst, N, transposed, relu, images, workspace, s)
+                   : wino_conv<4, 3>(g, src, filter, bias, gate, dst, N, transposed, relu, images, workspace, s);
 }
 
-size_t mnv_wino_grad_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw) {
+size_t mnv_wino_grad_workspace_bytes(int N, int C, int K, int H, int W, int ph, int pw, int R) {
   WinoGeom g;
   int mode;
-  if (!plan_geom(&g, &mode, N, C, K, H, W, ph, pw, 3, 3, 1, 1)) return 0;
+  if (!plan_geom(&g, &mode, N, C, K, H, W, ph, pw, R, R, 1, 1)) return 0;
   return u_bytes(g) + vm_bytes(g, N) + grad_sk_bytes(g);
 }
 
@@ -854,23 +987,26 @@ int mnv_wino_grad_images(int N, int C, int K, int H, int W, int ph, int pw, int 
   const long long most = ((1LL << 29) - 1) / ((long long)g.al * g.al * g.Coutp) / per_image;
   if (images > most) images = (int)most;
   if (mode != 1 || images == 0) return images;
-  return pays(g, images, C) ? images : 0;
+  return pays(g, images, true) ? images : 0;
 }
 
 int mnv_wino_filter_grad(const float* bottom, const float* top_diff, float* filter_diff, int N, int C,
-                         int K, int H, int W, int ph, int pw, int images, int accumulate,
+                         int K, int H, int W, int ph, int pw, int R, int images, int accumulate,
                          const float* sgd_w, float sgd_scale, void* workspace,
                          size_t workspace_bytes, hipStream_t s, int* plan) {
   WinoGeom g;
   int mode;
   if (images <= 0) return MNV_ERR_INVALID;
   if (images > N) images = N;
-  if (!plan_geom(&g, &mode, images, C, K, H, W, ph, pw, 3, 3, 1, 1)) return MNV_ERR_INVALID;
+  if (!plan_geom(&g, &mode, images, C, K, H, W, ph, pw, R, R, 1, 1)) return MNV_ERR_INVALID;
   if (!workspace || workspace_bytes < u_bytes(g) + vm_bytes(g, images) + grad_sk_bytes(g))
     return MNV_ERR_INVALID;
   if (!plan && (!bottom || !top_diff || !filter_diff)) return MNV_ERR_INVALID;
-  return g.al == 6 ? wino_filter_grad<6>(g, bottom, top_diff, filter_diff, N, images, accumulate, sgd_w,
-                                         sgd_scale, workspace, s, plan)
-                   : wino_filter_grad<4>(g, bottom, top_diff, filter_diff, N, images, accumulate, sgd_w,
-                                         sgd_scale, workspace, s, plan);
+  if (g.al == 8)
+    return wino_filter_grad<8, 5>(g, bottom, top_diff, filter_diff, N, images, accumulate, sgd_w, sgd_scale,
+                                  workspace, s, plan);
+  return g.al == 6 ? wino_filter_grad<6, 3>(g, bottom, top_diff, filter_diff, N, images, accumulate, sgd_w,
+                                            sgd_scale, workspace, s, plan)
+                   : wino_filter_grad<4, 3>(g, bottom, top_diff, filter_diff, N, images, accumulate, sgd_w,
+                                            sgd_scale, workspace, s, plan);
 }

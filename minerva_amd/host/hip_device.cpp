@@ -14,10 +14,11 @@ void Ok(int status, const char* what) {
 }
 // Scratch arena per worker stream: split-k partial sums of the skinny GEMMs and of the
 // convolution filter gradient (the kernels use as many k ranges as fit) and the transformed
-// tiles of the 3 x 3 convolutions (up to 702 MB for 384 -> 384 channels on 13 x 13 planes at
-// batch 256; with less those run in groups of images).  Allocated when a stream first runs an
+// tiles of the 3 x 3 and 5 x 5 convolutions by minimal filtering (up to 1.2 GB for 96 -> 256
+// channels under 5 x 5 filters on 27 x 27 planes at batch 256; with less those run in groups of
+// images).  Allocated when a stream first runs an
 // operator and kept: no operator allocates, so a recorded step never meets an allocation.
-constexpr size_t kWorkspaceBytes = (size_t)768 << 20;
+constexpr size_t kWorkspaceBytes = (size_t)1280 << 20;
 // Pinned staging per worker stream: two halves, one filled by the CPU while the other is
 // copied to the device.
 constexpr size_t kStagingBytes = (size_t)16 << 20;
