@@ -730,7 +730,7 @@ int launch_input_transform(const float* src, float* V, const WinoGeom& g, hipStr
   const int T = g.TH * g.TW, HW = g.Hs * g.Ws;
   // planes a workgroup's 256 consecutive tiles can touch
   const size_t lds = (size_t)(255 / T + 2) * HW * sizeof(float);
-  if (lds <= 32 * 1024)
+  if (lds <= 48 * 1024)
     hipLaunchKernelGGL((mnv_wino_input_lds_kernel<AL, R>), dim3((g.Pp + 255) / 256, g.Cin), dim3(256), lds,
                        s, src, V, g, mnv_fastdiv_make(HW));
   else
@@ -833,7 +833,7 @@ int wino_conv(const WinoGeom& g0, const float* src, const float* filter, const f
     if (timed) profile_end(e0, e1, s, 0, 2.0 * AL * AL * Cout * Cin * g.P);
     if (rc) return rc;
     const size_t lds = (size_t)(255 / (g.TH * g.TW) + 2) * g.Hd * g.Wd * sizeof(float);
-    if (lds <= 32 * 1024)
+    if (lds <= 48 * 1024)
       hipLaunchKernelGGL((mnv_wino_output_lds_kernel<AL, R>), dim3((g.P + 255) / 256, Cout), dim3(256), lds, s,
                          Mx, bias, gate ? gate + n0 * per_dst : nullptr, dst + n0 * per_dst, g, relu,
                          mnv_fastdiv_make(g.Hd * g.Wd), mnv_fastdiv_make(g.Wd));
@@ -878,7 +878,7 @@ int wino_filter_grad(const WinoGeom& g0, const float* bottom, const float* top_d
     if (nn != g.N && (rc = make_wino_geom(&g, nn, C, K, g.Hs, g.Ws, g.pad_h, g.pad_w, AL, R))) return rc;
     if ((rc = launch_input_transform<AL, R>(bottom + n0 * per_bottom, V, g, s))) return rc;
     const size_t lds = (size_t)(255 / (g.TH * g.TW) + 2) * g.Hd * g.Wd * sizeof(float);
-    if (lds <= 32 * 1024)
+    if (lds <= 48 * 1024)
       hipLaunchKernelGGL((mnv_wino_grad_lds_kernel<AL, R>), dim3((g.Pp + 255) / 256, g.Coutp), dim3(256), lds, s,
                          top_diff + n0 * per_top, Yt, g, mnv_fastdiv_make(g.Hd * g.Wd));
     else

@@ -145,6 +145,44 @@ def test_winograd_needs_a_16_byte_aligned_workspace(gpu, ora):
         assert np.any(gpu.down(top).view(np.uint32) != direct.view(np.uint32))
 
 
+def _random_winograd_geometries(count, seed):
+    """Seeded geometries for the forced path: both filter extents, every tile size, planes from
+    one output to 40 x 40 (past what the transform kernels stage in LDS), paddings up to the
+    filter's reach, channel counts around 16 and 128."""
+    rng = np.random.default_rng(seed)
+    menu = [16, 16, 32, 48, 64, 80, 128, 144]
+    out = []
+    while len(out) < count:
+        R = int(rng.choice([3, 3, 5]))
+        tile = F4 if R == 5 else int(rng.choice([F2, F4]))
+        N = int(rng.integers(1, 6))
+        C, K = int(rng.choice(menu)), int(rng.choice(menu + [20, 130]))
+        H, W = int(rng.integers(1, 41)), int(rng.integers(1, 41))
+        ph, pw = int(rng.integers(0, R)), int(rng.integers(0, R))
+        if H + 2 * ph < R or W + 2 * pw < R:
+            continue
+        Ho, Wo = H + 2 * ph - R + 1, W + 2 * pw - R + 1
+        if N * C * K * Ho * Wo * R * R > 120e6:
+            continue
+        out.append((N, C, K, H, W, ph, pw, R, tile))
+    return out
+
+
+@pytest.mark.parametrize("q", _random_winograd_geometries(36, 7), ids=lambda q: "x".join(map(str, q)))
+def test_winograd_random_geometries_against_oracle(gpu, ora, q):
+    N, C, K, H, W, ph, pw, R, tile = q
+    p = (N, C, K, H, W, ph, pw, 1, 1, R, R)
+    cv = Conv(gpu, *p)
+    bound = TIGHT5 if R == 5 else TIGHT
+    x, w, b = _rand(N * C * H * W, 60), _rand(K * C * R * R, 61, 0.2), _rand(K, 62)
+    dy = _rand(N * K * cv.Ho * cv.Wo, 63)
+    with mode(gpu, tile):
+        say("winograd, random geometry", q)
+        assert normwise(cv.fwd(x, w, b), ora.conv_fwd(x, w, b, *p)) <= bound
+        assert normwise(cv.bwd_data(dy, w), ora.conv_bwd_data(dy, w, *p)) <= bound
+        assert normwise(cv.bwd_filter(dy, x), ora.conv_bwd_filter(dy, x, *p)) <= bound
+
+
 def _points(Ho, Wo):
     """Points per dimension the library picks by itself: 6 (4 x 4 outputs per tile) when that
     takes at most 85% of the products of 4 (2 x 2 outputs per tile)."""
