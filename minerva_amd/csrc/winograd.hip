@@ -147,46 +147,127 @@ struct WinoF<8, 5> {
       return t[i][j]; } };
 };
 
-// out = L in (rows) and out = in L^T (columns), fully unrolled with the coefficients folded.
-template <class L, int K>
-__device__ __forceinline__ void wino_rows(const float (&in)[L::C][K], float (&out)[L::R][K]) {
-#pragma unroll
+// Points come in pairs +-p.  In B^T, G and G' (one row per point) the rows of such a pair agree
+// in their even columns and differ in sign in the odd ones: both are e + o and e - o of one
+// even and one odd partial sum.  In A^T and A'^T (one column per point) the columns of a pair
+// agree in the even rows and differ in sign in the odd ones: a row needs one product with
+// in[j] + in[j+1] or in[j] - in[j+1] instead of two.  Either way the pair costs about half the
+// multiplies; which rows / columns pair up is read off the matrix at compile time.
+template <class L>
+__host__ __device__ constexpr bool wino_row_pair(int i) {
+  if (i < 0 || i + 1 >= L::R) return false;
+  bool any = false;
+  for (int j = 0; j < L::C; ++j) {
+    const float a = L::at(i, j), b = L::at(i + 1, j);
+    if ((j & 1) ? (b != -a) : (b != a)) return false;
+    if (a != 0.f) any = true;
+  }
+  return any;
+}
+template <class L>
+__host__ __device__ constexpr bool wino_col_pair(int j) {
+  if (j < 0 || j + 1 >= L::C) return false;
+  bool any = false;
+  for (int i = 0; i < L::R; ++i) {
+    const float a = L::at(i, j), b = L::at(i, j + 1);
+    if ((i & 1) ? (b != -a) : (b != a)) return false;
+    if (a != 0.f) any = true;
+  }
+  return any;
+}
+// the first row / column of a pair (pairs are taken greedily from the top / left)
+template <class L>
+__host__ __device__ constexpr bool wino_row_first(int i) {
+  return i >= 0 && wino_row_pair<L>(i) && !wino_row_first<L>(i - 1);
+}
+template <class L>
+__host__ __device__ constexpr bool wino_col_first(int j) {
+  return j >= 0 && wino_col_pair<L>(j) && !wino_col_first<L>(j - 1);
+}
+template <class L>
+__host__ __device__ constexpr bool wino_has_row_pairs() {
   for (int i = 0; i < L::R; ++i)
+    if (wino_row_first<L>(i)) return true;
+  return false;
+}
+
+__device__ __forceinline__ float wino_term(float c, float x) { return c == 1.f ? x : c == -1.f ? -x : c * x; }
+
+// out = L in for one vector, fully unrolled with the coefficients folded (zeros cost nothing,
+// +-1 no multiply).
+template <class L>
+__device__ __forceinline__ void wino_apply(const float (&in)[L::C], float (&out)[L::R]) {
+  if constexpr (wino_has_row_pairs<L>()) {
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-      float acc = 0.f;
-      bool any = false;
+    for (int i = 0; i < L::R; ++i) {
+      if (wino_row_first<L>(i - 1)) continue;  // written with its partner
+      const bool pair = wino_row_first<L>(i);
+      float part[2] = {0.f, 0.f};  // pair: even- and odd-column sums; otherwise all in part[0]
+      bool any[2] = {false, false};
 #pragma unroll
       for (int j = 0; j < L::C; ++j) {
         const float c = L::at(i, j);
         if (c != 0.f) {
-          const float t = c == 1.f ? in[j][k] : c == -1.f ? -in[j][k] : c * in[j][k];
-          acc = any ? acc + t : t;
-          any = true;
+          const int w = pair ? (j & 1) : 0;
+          const float t = wino_term(c, in[j]);
+          part[w] = any[w] ? part[w] + t : t;
+          any[w] = true;
         }
       }
-      out[i][k] = acc;
+      if (pair) {
+        out[i] = part[0] + part[1];
+        out[i + 1] = part[0] - part[1];
+      } else {
+        out[i] = part[0];
+      }
     }
-}
-template <class L, int K>
-__device__ __forceinline__ void wino_cols(const float (&in)[K][L::C], float (&out)[K][L::R]) {
+  } else {
+    float sum[L::C], dif[L::C];
 #pragma unroll
-  for (int k = 0; k < K; ++k)
+    for (int j = 0; j < L::C; ++j) {
+      sum[j] = dif[j] = 0.f;
+      if (wino_col_first<L>(j)) {
+        sum[j] = in[j] + in[j + 1];
+        dif[j] = in[j] - in[j + 1];
+      }
+    }
 #pragma unroll
     for (int i = 0; i < L::R; ++i) {
       float acc = 0.f;
       bool any = false;
 #pragma unroll
       for (int j = 0; j < L::C; ++j) {
+        if (wino_col_first<L>(j - 1)) continue;  // taken with its partner
         const float c = L::at(i, j);
         if (c != 0.f) {
-          const float t = c == 1.f ? in[k][j] : c == -1.f ? -in[k][j] : c * in[k][j];
+          const float x = wino_col_first<L>(j) ? ((i & 1) ? dif[j] : sum[j]) : in[j];
+          const float t = wino_term(c, x);
           acc = any ? acc + t : t;
           any = true;
         }
       }
-      out[k][i] = acc;
+      out[i] = acc;
     }
+  }
+}
+
+// out = L in along the rows of a block, out = in L^T along its columns
+template <class L, int K>
+__device__ __forceinline__ void wino_rows(const float (&in)[L::C][K], float (&out)[L::R][K]) {
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    float a[L::C], b[L::R];
+#pragma unroll
+    for (int j = 0; j < L::C; ++j) a[j] = in[j][k];
+    wino_apply<L>(a, b);
+#pragma unroll
+    for (int i = 0; i < L::R; ++i) out[i][k] = b[i];
+  }
+}
+template <class L, int K>
+__device__ __forceinline__ void wino_cols(const float (&in)[K][L::C], float (&out)[K][L::R]) {
+#pragma unroll
+  for (int k = 0; k < K; ++k) wino_apply<L>(in[k], out[k]);
 }
 
 // U[point][co][ci] from filter[k][c][R][R].  Forward: co = k, ci = c, g[r][s] = f[R-1-r][R-1-s];
