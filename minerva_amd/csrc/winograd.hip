@@ -1,10 +1,13 @@
-// 3 x 3, unit-stride convolutions by minimal filtering (Winograd): an m x m block of outputs
-// of one channel pair costs (m + 2)^2 multiplies instead of 9 m^2.  Two tile sizes:
+// 3 x 3 and 5 x 5 unit-stride convolutions by minimal filtering (Winograd / Toom-Cook): an
+// m x m block of outputs of one channel pair costs (m + r - 1)^2 multiplies instead of r^2 m^2.
 //   F(2 x 2, 3 x 3): 4 x 4 input tiles at stride 2, 16 points, 16 multiplies per 4 outputs;
-//   F(4 x 4, 3 x 3): 6 x 6 input tiles at stride 4, 36 points, 36 multiplies per 16 outputs,
-// the second taken when it needs clearly fewer products for the plane at hand (13 x 13 outputs:
-// 4 x 4 tiles x 36 = 576 against 7 x 7 x 16 = 784).  The work becomes al^2 independent matrix
-// products, one per point (xi, nu) of the transformed al x al tile (al = m + 2),
+//   F(4 x 4, 3 x 3): 6 x 6 input tiles at stride 4, 36 points, 36 multiplies per 16 outputs, taken
+//                    when it needs clearly fewer products for the plane at hand (13 x 13
+//                    outputs: 4 x 4 tiles x 36 = 576 against 7 x 7 x 16 = 784);
+//   F(4 x 4, 5 x 5): 8 x 8 input tiles at stride 4, 64 points, 64 multiplies per 16 outputs
+//                    instead of 400.
+// The work becomes al^2 independent matrix products, one per point (xi, nu) of the transformed
+// al x al tile (al = m + r - 1),
 //     M[xi,nu][co][p] = sum_ci U[xi,nu][co][ci] * V[xi,nu][ci][p],      p = (image, tile row, tile col)
 // with U = G g G^T (filters), V = B^T d B (input tiles) and the outputs Y = A^T M A.  The
 // products run as ONE launch of the fp32 MFMA core (gemm_core.h): the point is folded into the
@@ -12,27 +15,31 @@
 // block_init.  Semantics are those of conv.hip: the forward pass correlates with the flipped
 // filter (cuDNN's CUDNN_CONVOLUTION as selected at minerva/op/impl/cuda/cuda_perform.cu:227-264),
 // the data gradient (cuda_perform.cu:266-291) is the same correlation of top_diff with the
-// unflipped filter, channels exchanged, under a padding of 2 - pad.  The filter gradient
-// (cuda_perform.cu:293-318) is F(3 x 3, m x m) on the same points: the m x m tiles of top_diff
+// unflipped filter, channels exchanged, under a padding of r - 1 - pad.  The filter gradient
+// (cuda_perform.cu:293-318) is F(r x r, m x m) on the same points: the m x m tiles of top_diff
 // take the filter's place, Yt = G' dy G'^T, the sum over images and tiles is the reduction
 // dimension of the products Q[xi,nu][k][c] = sum_p Yt[xi,nu][k][p] V[xi,nu][c][p], and the
 // gradient is A'^T Q A'.
 //
-// The matrices are those of the Toom-Cook construction on the points {0, 1, -1, inf} (al = 4)
-// and {0, 1, -1, 2, -1/2, inf} (al = 6): B^T depends on the points alone and serves all three
-// passes.  al = 4 (G and G' carry the halves):
+// The matrices are those of the Toom-Cook construction (evaluation at the points, interpolation
+// by the transposed inverse Vandermonde matrix) on {0, 1, -1, inf} (al = 4), {0, 1, -1, 2, -1/2,
+// inf} (al = 6) and {0, 1, -1, 2, -2, 1/2, -1/2, inf} (al = 8): B^T depends on the points alone
+// and serves all three passes.  al = 4 (G and G' carry the halves):
 //   B^T = | 1  0 -1  0 |   G = | 1    0    0  |   A^T = | 1  1  1  0 |   G' = | 1    0  |   A'^T = | 1  1  1  0 |
 //         | 0  1  1  0 |       | 1/2  1/2  1/2|         | 0  1 -1 -1 |        | 1/2  1/2|          | 0  1 -1  0 |
 //         | 0 -1  1  0 |       | 1/2 -1/2  1/2|                              | 1/2 -1/2|          | 0  1  1 -1 |
 //         | 0  1  0 -1 |       | 0    0    1  |                              | 0    1  |
-// al = 6: see WinoF<6> below (G, G', A^T, A'^T are powers of the points, exact in fp32; B^T
-// carries the fractions).
+// al = 6 and 8: see WinoF below (G, G', A^T, A'^T are powers of the points, exact in fp32; B^T
+// carries the fractions).  The point sets were chosen by an fp32 emulation of the whole pass:
+// for al = 6 the customary {0, +-1, +-2} gave 2.6 times the error of the set above.
 //
 // Rounding: the transforms are short sums with small constants, the products are summed in
 // fp32 in k order; against the direct sum the results differ by a few 1e-6 of the output's
-// norm (al = 4) and up to about 1e-5 (al = 6); the bound of the convolutions is 1e-4.
-// Roofline: the matrix products are MFMA-bound (2 * al^2 * Cout * Cin * tiles flops); the
-// transform kernels stream al^2 * 4 bytes per (channel, tile) and are HBM-bound.
+// largest element (al = 4), up to about 6e-6 (al = 6) and up to about 2.5e-5 (al = 8, filter
+// gradient over 12544 tiles); the bound of the convolutions is 1e-4.
+// Roofline: the matrix products are MFMA-bound (2 * al^2 * Cout * Cin * tiles flops; with few
+// input channels they approach the bandwidth bound of their al^2 * (Cin + Cout) * tiles * 4
+// bytes); the transform kernels stream al^2 * 4 bytes per (channel, tile) and are HBM-bound.
 
 #include <mutex>
 #include <vector>
