@@ -791,8 +791,9 @@ int pick_points(int Hd, int Wd, int R, int mode) {
 
 int make_wino_geom(WinoGeom* g, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w,
                    int al, int r) {
-  if (N <= 0 || Cin <= 0 || Cout <= 0 || Hs <= 0 || Ws <= 0 || pad_h < 0 || pad_w < 0 || pad_h > r - 1 ||
-      pad_w > r - 1 || Hs + 2 * pad_h < r || Ws + 2 * pad_w < r ||
+  // (channel counts are grid extents of the transform kernels)
+  if (N <= 0 || Cin <= 0 || Cout <= 0 || Cin > 65535 || Cout > 65535 - 127 || Hs <= 0 || Ws <= 0 ||
+      pad_h < 0 || pad_w < 0 || pad_h > r - 1 || pad_w > r - 1 || Hs + 2 * pad_h < r || Ws + 2 * pad_w < r ||
       !((r == 3 && (al == 4 || al == 6)) || (r == 5 && al == 8)))
     return MNV_ERR_INVALID;
   g->N = N; g->Cin = Cin; g->Cout = Cout; g->Coutp = (Cout + 127) / 128 * 128;
