@@ -934,9 +934,13 @@ int wino_conv(const WinoGeom& g0, const float* src, const float* filter, const f
   return MNV_OK;
 }
 
+// Slabs the filter-gradient products' loads run ahead (see mnv_gemm_kernel): two; the kernel
+// still holds four workgroups per CU (conv2 / conv4 at batch 256: 387 -> 377 us on average).
 #ifndef MNV_WINO_SK_PF
-#define MNV_WINO_SK_PF 1
+#define MNV_WINO_SK_PF 2
 #endif
+// (the forward / data-gradient products gain nothing from it: 388 / 474 / 435 against 388 / 474 /
+// 426 us.)
 template <int AL, int R>
 int wino_filter_grad(const WinoGeom& g0, const float* bottom, const float* top_diff, float* filter_diff,
                      int N, int images, int accumulate, const float* sgd_w, float sgd_scale,
