@@ -36,10 +36,10 @@ CONV_GFLOP = [53.97, 229.32, 76.55, 114.83, 76.55]
 STEP_GFLOP = 1689.8  # convolutions (fwd, bwd-filter, bwd-data except conv1) + three FC layers
 # What the matrix pipe executes: the three passes of conv2..conv5 run by minimal filtering.
 # conv2 (5 x 5): 64 multiplies per 4 x 4 outputs of a channel pair on 7 x 7 tiles per 27 x 27
-# plane; conv3..5 (3 x 3): 36 per 4 x 4 outputs on 4 x 4 tiles per 13 x 13 plane; the filter
+# plane; conv3..5 (3 x 3): 49 per 5 x 5 outputs on 3 x 3 tiles per 13 x 13 plane; the filter
 # gradients the same counts with the tiles of top_diff in the filter's place.
 WINOGRAD_GFLOP = [2 * 64 * 256 * 96 * 256 * 49 / 1e9] + \
-                 [2 * 36 * k * c * 256 * 16 / 1e9 for (c, k) in ((256, 384), (384, 384), (384, 256))]
+                 [2 * 49 * k * c * 256 * 9 / 1e9 for (c, k) in ((256, 384), (384, 384), (384, 256))]
 STEP_EXECUTED_GFLOP = round(STEP_GFLOP - 3 * sum(CONV_GFLOP[1:]) + 3 * sum(WINOGRAD_GFLOP), 1)
 
 
@@ -757,13 +757,20 @@ def parity_report():
     # library would not choose it by itself)
     L.mnv_conv_winograd_mode(2)
     try:
+        close("conv forward, F(5x5,3x3)", run(lambda o: L.mnv_conv_fwd(dcx.p, dcw.p, dcb.p, o.p, *p, ws.p, z, S), N * K * H * W),
+              ora.conv_fwd(cx, cw, cb, *p))
+        close("conv backward data, F(5x5,3x3)", run(lambda o: L.mnv_conv_bwd_data(dcdy.p, dcw.p, o.p, *p, ws.p, z, S), N * C * H * W),
+              ora.conv_bwd_data(cdy, cw, *p))
+        close("conv backward filter, F(3x3,5x5)", run(lambda o: L.mnv_conv_bwd_filter(dcx.p, dcdy.p, o.p, *p, ws.p, z, S), K * C * 9),
+              ora.conv_bwd_filter(cdy, cx, *p))
+        L.mnv_conv_winograd_mode(4)  # the smaller tiles, which planes with fewer outputs take
         close("conv forward, F(4x4,3x3)", run(lambda o: L.mnv_conv_fwd(dcx.p, dcw.p, dcb.p, o.p, *p, ws.p, z, S), N * K * H * W),
               ora.conv_fwd(cx, cw, cb, *p))
         close("conv backward data, F(4x4,3x3)", run(lambda o: L.mnv_conv_bwd_data(dcdy.p, dcw.p, o.p, *p, ws.p, z, S), N * C * H * W),
               ora.conv_bwd_data(cdy, cw, *p))
         close("conv backward filter, F(3x3,4x4)", run(lambda o: L.mnv_conv_bwd_filter(dcx.p, dcdy.p, o.p, *p, ws.p, z, S), K * C * 9),
               ora.conv_bwd_filter(cdy, cx, *p))
-        L.mnv_conv_winograd_mode(3)  # the smaller tile, which planes with few outputs take
+        L.mnv_conv_winograd_mode(3)
         close("conv forward, F(2x2,3x3)", run(lambda o: L.mnv_conv_fwd(dcx.p, dcw.p, dcb.p, o.p, *p, ws.p, z, S), N * K * H * W),
               ora.conv_fwd(cx, cw, cb, *p))
         close("conv backward data, F(2x2,3x3)", run(lambda o: L.mnv_conv_bwd_data(dcdy.p, dcw.p, o.p, *p, ws.p, z, S), N * C * H * W),
@@ -855,7 +862,7 @@ def main():
             "median_ms_per_step": round(main_run["median_ms_per_step"], 3),
             "step_mfma_frac": round(STEP_GFLOP / main_run["ms_per_step"] / PEAK_FP32_MFMA_TFLOPS, 4),
             "step_mfma_frac_note": "algorithmic (direct-sum) flops of the step / time / fp32 MFMA peak; "
-                                   "conv2 executes 4/25 x (28/27)^2 of its, the 3 x 3 layers 1/4 x (16/13)^2 of theirs",
+                                   "conv2 executes 4/25 x (28/27)^2 of its, the 3 x 3 layers 49/225 x (15/13)^2 of theirs",
             "step_executed_gflop": STEP_EXECUTED_GFLOP,
             "step_executed_mfma_frac": round(STEP_EXECUTED_GFLOP / main_run["ms_per_step"] /
                                              PEAK_FP32_MFMA_TFLOPS, 4),

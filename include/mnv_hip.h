@@ -236,23 +236,24 @@ int mnv_softmax_channel_bwd(const float* top_diff, const float* top, float* bott
  * several launches over chunks of images, the filter gradient accumulating chunk by chunk;
  * only a single image or a filter of 2^29 elements and more is refused (MNV_ERR_INVALID).
  * 3 x 3 and 5 x 5 filters at unit stride may run by minimal filtering (Winograd): F(2 x 2, 3 x 3),
- * 16 multiplies per 2 x 2 outputs of a channel pair instead of 36, or F(4 x 4, 3 x 3), 36 per
- * 4 x 4 outputs instead of 144 -- whichever needs fewer products for the plane at hand, the
- * smaller tile on a near tie --, F(4 x 4, 5 x 5), 64 per 4 x 4 outputs instead of 400: as 16 / 36 /
- * 64 matrix products between transforms of 4 x 4 / 6 x 6 / 8 x 8 tiles, summed in fp32;
- * backward_filter by F(3 x 3, m x m) / F(5 x 5, 4 x 4) with the sum over the tiles as the products'
- * reduction.  Results differ from the direct sum by a few 1e-6 of the output's norm (up to
- * about 6e-6 with 6 x 6 tiles, up to about 2.5e-5 with 8 x 8 tiles; the bound of the
- * convolutions is 1e-4).  forward / backward_data need a bottom / top
+ * 16 multiplies per 2 x 2 outputs of a channel pair instead of 36, F(4 x 4, 3 x 3), 36 per 4 x 4
+ * outputs, or F(5 x 5, 3 x 3), 49 per 5 x 5 outputs -- whichever needs fewer products for the
+ * plane at hand, a smaller tile on a near tie --, F(4 x 4, 5 x 5), 64 per 4 x 4 outputs instead
+ * of 400: as 16 / 36 / 49 / 64 matrix products between transforms of 4 x 4 ... 8 x 8 tiles, summed
+ * in fp32; backward_filter by F(3 x 3, m x m) / F(5 x 5, 4 x 4) with the sum over the tiles as the
+ * products' reduction.  Results differ from the direct sum by a few 1e-6 of the output's
+ * largest element (up to about 6e-6 with 6 x 6 tiles, up to about 2.5e-5 with 7 x 7 and 8 x 8
+ * tiles; the bound of the convolutions is 1e-4).  forward / backward_data need a bottom / top
  * channel count that is a multiple of 16.  The path wants the workspace the size queries
- * report (16 / 36 / 64 transformed values per tile and channel of both tensors), 16-byte aligned;
+ * report (16 ... 64 transformed values per tile and channel of both tensors), 16-byte aligned;
  * with less it runs in groups of images, with less than one image needs the direct kernels
  * run. ---- */
 /* Selects when the three passes take the minimal-filtering path.  0: never; 1 (initial):
  * where a cost estimate from the extents (multiplies saved against transformed values moved;
  * in practice layers of about 200 channels and more whose direct pass takes over 100 us)
- * puts it at 80% of the direct kernels' time or less; 2: wherever it applies; 3 / 4: as 2
- * with the tile pinned to 2 x 2 / 4 x 4 outputs (3: 5 x 5 filters stay direct).
+ * puts it at 80% of the direct kernels' time or less; 2: wherever it applies; 3 / 4 / 5: as 2
+ * with the tile of 3 x 3 filters pinned to 2 x 2 / 4 x 4 / 5 x 5 outputs (3: 5 x 5 filters stay
+ * direct; the most accurate setting that still uses the path).
  * Process-wide; returns the previous mode; any other value only queries.  No reference
  * counterpart: cuDNN picks its algorithm out of sight (CUDNN_CONVOLUTION_FWD_PREFER_FASTEST,
  * cuda_perform.cu:227-264). */

@@ -4,6 +4,8 @@
 //   F(4 x 4, 3 x 3): 6 x 6 input tiles at stride 4, 36 points, 36 multiplies per 16 outputs, taken
 //                    when it needs clearly fewer products for the plane at hand (13 x 13
 //                    outputs: 4 x 4 tiles x 36 = 576 against 7 x 7 x 16 = 784);
+//   F(5 x 5, 3 x 3): 7 x 7 input tiles at stride 5, 49 points, 49 multiplies per 25 outputs (13 x 13
+//                    outputs: 3 x 3 tiles x 49 = 441);
 //   F(4 x 4, 5 x 5): 8 x 8 input tiles at stride 4, 64 points, 64 multiplies per 16 outputs
 //                    instead of 400.
 // The work becomes al^2 independent matrix products, one per point (xi, nu) of the transformed
@@ -23,7 +25,7 @@
 //
 // The matrices are those of the Toom-Cook construction (evaluation at the points, interpolation
 // by the transposed inverse Vandermonde matrix) on {0, 1, -1, inf} (al = 4), {0, 1, -1, 2, -1/2,
-// inf} (al = 6) and {0, 1, -1, 2, -2, 1/2, -1/2, inf} (al = 8): B^T depends on the points alone
+// inf} (al = 6), {0, 1, -1, 2, -2, -1/2, inf} (al = 7) and {0, 1, -1, 2, -2, 1/2, -1/2, inf} (al = 8): B^T depends on the points alone
 // and serves all three passes.  al = 4 (G and G' carry the halves):
 //   B^T = | 1  0 -1  0 |   G = | 1    0    0  |   A^T = | 1  1  1  0 |   G' = | 1    0  |   A'^T = | 1  1  1  0 |
 //         | 0  1  1  0 |       | 1/2  1/2  1/2|         | 0  1 -1 -1 |        | 1/2  1/2|          | 0  1 -1  0 |
@@ -35,8 +37,10 @@
 //
 // Rounding: the transforms are short sums with small constants, the products are summed in
 // fp32 in k order; against the direct sum the results differ by a few 1e-6 of the output's
-// largest element (al = 4), up to about 6e-6 (al = 6) and up to about 2.5e-5 (al = 8, filter
-// gradient over 12544 tiles); the bound of the convolutions is 1e-4.
+// largest element (al = 4), up to about 6e-6 (al = 6) and up to about 2.5e-5 (al = 7 and 8);
+// the bound of the convolutions is 1e-4.  A whole AlexNet-shaped backward pass at batch 256 is
+// 2e-5 from the oracle's with the larger tiles (set by the 8 x 8 tiles of the 5 x 5 layer; the
+// tile of the 3 x 3 layers does not move it), 4e-6 on the direct kernels.
 // Roofline: the matrix products are MFMA-bound (2 * al^2 * Cout * Cin * tiles flops; with few
 // input channels they approach the bandwidth bound of their al^2 * (Cin + Cout) * tiles * 4
 // bytes); the transform kernels stream al^2 * 4 bytes per (channel, tile) and are HBM-bound.
@@ -113,6 +117,38 @@ struct WinoF<6, 3> {
   struct AAT { static constexpr int R = 3, C = 6;
     __host__ __device__ static constexpr float at(int i, int j) {
       constexpr float t[3][6] = {{1, 1, 1, 1, 1, 0}, {0, 1, -1, 2, -.5f, 0}, {0, 1, 1, 4, .25f, 1}};
+      return t[i][j]; } };
+};
+// 3 x 3 filters, 5 x 5 outputs per tile: the points {0, 1, -1, 2, -2, -1/2, inf}
+template <>
+struct WinoF<7, 3> {
+  struct BT { static constexpr int R = 7, C = 7;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[7][7] = {{1, 2, -5.f / 4, -5.f / 2, 1.f / 4, 1.f / 2, 0},
+                                 {0, 2.f / 9, 2.f / 3, 7.f / 18, -1.f / 6, -1.f / 9, 0},
+                                 {0, 2.f / 3, 2.f / 3, -3.f / 2, -1.f / 6, 1.f / 3, 0},
+                                 {0, -1.f / 60, -1.f / 24, 0, 1.f / 24, 1.f / 60, 0},
+                                 {0, -1.f / 36, -1.f / 24, 1.f / 18, 1.f / 24, -1.f / 36, 0},
+                                 {0, -128.f / 45, 0, 32.f / 9, 0, -32.f / 45, 0},
+                                 {0, 2, 4, -5.f / 2, -5, 1.f / 2, 1}};
+      return t[i][j]; } };
+  struct G { static constexpr int R = 7, C = 3;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[7][3] = {{1, 0, 0}, {1, 1, 1}, {1, -1, 1}, {1, 2, 4}, {1, -2, 4}, {1, -.5f, .25f}, {0, 0, 1}};
+      return t[i][j]; } };
+  struct AT { static constexpr int R = 5, C = 7;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[5][7] = {{1, 1, 1, 1, 1, 1, 0}, {0, 1, -1, 2, -2, -.5f, 0}, {0, 1, 1, 4, 4, .25f, 0},
+                                 {0, 1, -1, 8, -8, -.125f, 0}, {0, 1, 1, 16, 16, .0625f, 1}};
+      return t[i][j]; } };
+  struct GG { static constexpr int R = 7, C = 5;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[7][5] = {{1, 0, 0, 0, 0}, {1, 1, 1, 1, 1}, {1, -1, 1, -1, 1}, {1, 2, 4, 8, 16},
+                                 {1, -2, 4, -8, 16}, {1, -.5f, .25f, -.125f, .0625f}, {0, 0, 0, 0, 1}};
+      return t[i][j]; } };
+  struct AAT { static constexpr int R = 3, C = 7;
+    __host__ __device__ static constexpr float at(int i, int j) {
+      constexpr float t[3][7] = {{1, 1, 1, 1, 1, 1, 0}, {0, 1, -1, 2, -2, -.5f, 0}, {0, 1, 1, 4, 4, .25f, 1}};
       return t[i][j]; } };
 };
 // 5 x 5 filters, 4 x 4 outputs per tile: the points {0, 1, -1, 2, -2, 1/2, -1/2, inf}
@@ -773,20 +809,29 @@ void profile_end(hipEvent_t begin, hipEvent_t end, hipStream_t s, int kind, doub
 
 inline size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
 
-// Mode of mnv_conv_winograd_mode: 0 never, 1 where it pays, 2 wherever it applies, 3 / 4 as 2
-// with the tile size pinned to F(2 x 2) / F(4 x 4).
+// Mode of mnv_conv_winograd_mode: 0 never, 1 where it pays, 2 wherever it applies, 3 / 4 / 5 as 2
+// with the tile size pinned to 2 x 2 / 4 x 4 / 5 x 5 outputs.
 std::atomic<int> g_mode{1};
 
-// Points per dimension for an Hd x Wd output plane: 6 (4 x 4 outputs per tile) when that needs
-// at most 85% of the products of 4 (2 x 2 outputs per tile); its results are a few times
-// further from the direct sum, so a near tie goes to the smaller tile.
+// Points per dimension for an Hd x Wd output plane under r x r filters.  3 x 3: 4, 6 or 7 (2 x 2,
+// 4 x 4 or 5 x 5 outputs per tile): a larger tile is taken when it needs at most 85% of the
+// products of the best smaller one; its results are a few times further from the direct sum,
+// so a near tie goes to the smaller tile.  5 x 5: 8 (4 x 4 outputs per tile) or not at all.
 int pick_points(int Hd, int Wd, int R, int mode) {
-  if (R == 5) return mode == 3 ? 0 : 8;  // 5 x 5 filters: 4 x 4 outputs per 8 x 8 tile or not at all
+  if (R == 5) return mode == 3 ? 0 : 8;
   if (mode == 3) return 4;
   if (mode == 4) return 6;
-  const long long small = 16LL * ((Hd + 1) / 2) * ((Wd + 1) / 2);
-  const long long large = 36LL * ((Hd + 3) / 4) * ((Wd + 3) / 4);
-  return large * 100 <= small * 85 ? 6 : 4;
+  if (mode == 5) return 7;
+  long long best = 16LL * ((Hd + 1) / 2) * ((Wd + 1) / 2);
+  int al = 4;
+  const long long six = 36LL * ((Hd + 3) / 4) * ((Wd + 3) / 4);
+  if (six * 100 <= best * 85) {
+    best = six;
+    al = 6;
+  }
+  const long long seven = 49LL * ((Hd + 4) / 5) * ((Wd + 4) / 5);
+  if (seven * 100 <= best * 85) al = 7;
+  return al;
 }
 
 int make_wino_geom(WinoGeom* g, int N, int Cin, int Cout, int Hs, int Ws, int pad_h, int pad_w,
@@ -794,7 +839,7 @@ int make_wino_geom(WinoGeom* g, int N, int Cin, int Cout, int Hs, int Ws, int pa
   // (channel counts are grid extents of the transform kernels)
   if (N <= 0 || Cin <= 0 || Cout <= 0 || Cin > 65535 || Cout > 65535 - 127 || Hs <= 0 || Ws <= 0 ||
       pad_h < 0 || pad_w < 0 || pad_h > r - 1 || pad_w > r - 1 || Hs + 2 * pad_h < r || Ws + 2 * pad_w < r ||
-      !((r == 3 && (al == 4 || al == 6)) || (r == 5 && al == 8)))
+      !((r == 3 && (al == 4 || al == 6 || al == 7)) || (r == 5 && al == 8)))
     return MNV_ERR_INVALID;
   g->N = N; g->Cin = Cin; g->Cout = Cout; g->Coutp = (Cout + 127) / 128 * 128;
   g->Hs = Hs; g->Ws = Ws; g->Hd = Hs + 2 * pad_h - (r - 1); g->Wd = Ws + 2 * pad_w - (r - 1);
@@ -996,7 +1041,7 @@ int wino_filter_grad(const WinoGeom& g0, const float* bottom, const float* top_d
 }  // namespace
 
 extern "C" int mnv_conv_winograd_mode(int mode) {
-  if (mode < 0 || mode > 4) return g_mode.load(std::memory_order_relaxed);
+  if (mode < 0 || mode > 5) return g_mode.load(std::memory_order_relaxed);
   return g_mode.exchange(mode, std::memory_order_relaxed);
 }
 
@@ -1057,6 +1102,8 @@ int mnv_wino_conv(const float* src, const float* filter, const float* bias, cons
   if (!workspace || workspace_bytes < u_bytes(g) + vm_bytes(g, images)) return MNV_ERR_INVALID;
   if (g.al == 8)
     return wino_conv<8, 5>(g, src, filter, bias, gate, dst, N, transposed, relu, images, workspace, s);
+  if (g.al == 7)
+    return wino_conv<7, 3>(g, src, filter, bias, gate, dst, N, transposed, relu, images, workspace, s);
   return g.al == 6 ? wino_conv<6, 3>(g, src, filter, bias, gate, dst, N, transposed, relu, images, workspace, s)
                    : wino_conv<4, 3>(g, src, filter, bias, gate, dst, N, transposed, relu, images, workspace, s);
 }
@@ -1097,6 +1144,9 @@ int mnv_wino_filter_grad(const float* bottom, const float* top_diff, float* filt
   if (!plan && (!bottom || !top_diff || !filter_diff)) return MNV_ERR_INVALID;
   if (g.al == 8)
     return wino_filter_grad<8, 5>(g, bottom, top_diff, filter_diff, N, images, accumulate, sgd_w, sgd_scale,
+                                  workspace, s, plan);
+  if (g.al == 7)
+    return wino_filter_grad<7, 3>(g, bottom, top_diff, filter_diff, N, images, accumulate, sgd_w, sgd_scale,
                                   workspace, s, plan);
   return g.al == 6 ? wino_filter_grad<6, 3>(g, bottom, top_diff, filter_diff, N, images, accumulate, sgd_w,
                                             sgd_scale, workspace, s, plan)

@@ -58,9 +58,9 @@ def test_pure_host_entry_points():
 def test_winograd_switch_and_size_queries():
     """The path switch is process-wide host state and the size queries follow it (pure
     arithmetic): the 384 -> 384 channel layer on 13 x 13 planes at batch 256 asks for its
-    transformed tensors only while the path is on (36 values per 6 x 6 tile and channel on
-    4 x 4 tiles per plane, 474 MB; 16 per 4 x 4 tile on 7 x 7 tiles, 597 MB, with the tile
-    size pinned); the 5 x 5 layer (96 -> 256 channels on 27 x 27 planes) 64 values per 8 x 8 tile
+    transformed tensors only while the path is on (49 values per 7 x 7 tile and channel on
+    3 x 3 tiles per plane, 376 MB; 16 per 4 x 4 tile on 7 x 7 tiles, 597 MB, or 36 per 6 x 6 tile
+    on 4 x 4 tiles, 474 MB, with the tile size pinned); the 5 x 5 layer (96 -> 256 channels on 27 x 27 planes) 64 values per 8 x 8 tile
     on 7 x 7 tiles per plane, 1137 MB, unless the tile is pinned to 2 x 2 outputs."""
     from minerva_amd import capi
     L = capi.lib()
@@ -69,8 +69,8 @@ def test_winograd_switch_and_size_queries():
     assert L.mnv_conv_winograd_mode(-1) == 1
     try:
         on = L.mnv_conv_fwd_workspace_bytes(*conv4)
-        tiles = 256 * 4 * 4
-        assert on == 36 * 384 * 384 * 4 + 2 * 36 * tiles * 384 * 4
+        tiles = 256 * 3 * 3
+        assert on == 49 * 384 * 384 * 4 + 2 * 49 * tiles * 384 * 4
         assert L.mnv_conv_bwd_data_workspace_bytes(*conv4) == on
         five = L.mnv_conv_fwd_workspace_bytes(*conv2)
         assert five == 64 * 256 * 96 * 4 + 64 * 256 * 49 * (96 + 256) * 4
@@ -85,8 +85,11 @@ def test_winograd_switch_and_size_queries():
         assert L.mnv_conv_fwd_workspace_bytes(*conv4) == 16 * 384 * 384 * 4 + 2 * 16 * 256 * 49 * 384 * 4
         assert L.mnv_conv_fwd_workspace_bytes(*conv2) == direct_five
         assert L.mnv_conv_winograd_mode(4) == 3      # 4 x 4 output tiles only
+        assert L.mnv_conv_fwd_workspace_bytes(*conv4) == 36 * 384 * 384 * 4 + 2 * 36 * 256 * 16 * 384 * 4
+        assert L.mnv_conv_fwd_workspace_bytes(*conv2) == five
+        assert L.mnv_conv_winograd_mode(5) == 4      # 5 x 5 output tiles only
         assert L.mnv_conv_fwd_workspace_bytes(*conv4) == on
-        assert L.mnv_conv_winograd_mode(7) == 4      # out of range: a query
+        assert L.mnv_conv_winograd_mode(7) == 5      # out of range: a query
     finally:
         L.mnv_conv_winograd_mode(1)
 
