@@ -920,8 +920,8 @@ static int conv_fwd_impl(const float* bottom, const float* filter, const float* 
   if (rc) return rc;
   int gm = N * g.HoWo, gn = K, gk = g.CRS;
   hipStream_t s = mnv_stream(stream);
-  // 3 x 3 unit-stride layers with enough channels and tiles: F(2 x 2, 3 x 3), see winograd.hip
-  // (its transformed tensors are read and written in 16-byte vectors)
+  // 3 x 3 and 5 x 5 unit-stride layers with enough channels and tiles: minimal filtering, see
+  // winograd.hip (its transformed tensors are read and written in 16-byte vectors)
   if (const int images = mnv_wino_images(N, C, K, H, W, ph, pw, R, S, sv, sh,
                                          workspace && mnv_aligned16(workspace) ? workspace_bytes : 0))
     return mnv_wino_conv(bottom, filter, bias, nullptr, top, N, C, K, H, W, ph, pw, R, 0, relu, images,
@@ -1108,7 +1108,8 @@ static int conv_bwd_filter_impl(const float* bottom, const float* top_diff, floa
   if (rc) return rc;
   int gm = g.CRS, gn = K, gk = N * g.HoWo;
   hipStream_t s = mnv_stream(stream);
-  // 3 x 3 unit-stride layers with enough channels and tiles: F(3 x 3, 2 x 2), see winograd.hip
+  // 3 x 3 and 5 x 5 unit-stride layers with enough channels and tiles: minimal filtering of the
+  // filter gradient, F(r x r, m x m), see winograd.hip
   if (const int images = mnv_wino_grad_images(N, C, K, H, W, ph, pw, R, S, sv, sh,
                                               workspace && (plan || mnv_aligned16(workspace)) ? workspace_bytes : 0))
     return mnv_wino_filter_grad(bottom, top_diff, filter_diff, N, C, K, H, W, ph, pw, R, images,
