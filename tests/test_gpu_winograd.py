@@ -285,6 +285,55 @@ def test_winograd_fused_epilogues_have_the_bits_of_the_chain(gpu, tile):
         assert_bits_equal(gpu.down(dwb), want, "filter gradient + update in place")
 
 
+def _profile_read(gpu, kind):
+    n, ms, gf = ctypes.c_int(), ctypes.c_double(), ctypes.c_double()
+    assert gpu.L.mnv_conv_winograd_profile_read(kind, ctypes.byref(n), ctypes.byref(ms), ctypes.byref(gf)) == 0
+    return n.value, ms.value, gf.value
+
+
+def test_winograd_product_profile_counts_launches_and_flops(gpu):
+    """The measurement aid brackets the products of a pass with events: one record per group
+    of images, of the pass's kind, carrying 2 x points x Cout x Cin x tiles flops; results
+    have the same bits with and without it; enabling drops earlier records, disabling keeps
+    them readable."""
+    N, C, K, H, W = 12, 32, 64, 13, 13
+    p = (N, C, K, H, W, 1, 1, 1, 1, 3, 3)
+    cv = Conv(gpu, *p)
+    x, w, b = _rand(N * C * H * W, 60), _rand(K * C * 9, 61, 0.2), _rand(K, 62)
+    dy = _rand(N * K * H * W, 63)
+    points, tiles = 36, N * 4 * 4        # 4 x 4 outputs per tile on 13 x 13 planes
+    with mode(gpu, F4):
+        plain = cv.fwd(x, w, b), cv.bwd_data(dy, w), cv.bwd_filter(dy, x)
+        assert gpu.L.mnv_conv_winograd_profile(1) == 0
+        try:
+            assert _profile_read(gpu, 0) == (0, 0.0, 0.0) and _profile_read(gpu, 1) == (0, 0.0, 0.0)
+            timed = cv.fwd(x, w, b), cv.bwd_data(dy, w), cv.bwd_filter(dy, x)
+            n0, ms0, gf0 = _profile_read(gpu, 0)
+            n1, ms1, gf1 = _profile_read(gpu, 1)
+            assert (n0, n1) == (2, 1) and ms0 > 0 and ms1 > 0
+            assert gf0 == pytest.approx(2 * 2.0 * points * K * C * tiles / 1e9, rel=1e-12)
+            assert gf1 == pytest.approx(2.0 * points * K * C * tiles / 1e9, rel=1e-12)
+            for got, want, what in zip(timed, plain, ("forward", "data gradient", "filter gradient")):
+                assert_bits_equal(got, want, what + " with the profile on")
+            # a workspace of five images: three groups, a record each
+            nbytes = _wino_bytes(5, C, K, H, W, POINTS[F4]) + 1024
+            ws, dxb, dwb, dbb = gpu.empty(nbytes // 4 + 64), gpu.up(x), gpu.up(w), gpu.up(b)
+            top = gpu.empty(N * K * H * W)
+            assert gpu.L.mnv_conv_winograd_profile(1) == 0      # drops the three records
+            assert _profile_read(gpu, 0)[0] == 0
+            gpu.call("mnv_conv_fwd", dxb.p, dwb.p, dbb.p, top.p, *p, ws.p, ctypes.c_size_t(nbytes))
+            n0, _, gf0 = _profile_read(gpu, 0)
+            assert n0 == 3 and gf0 == pytest.approx(2.0 * points * K * C * tiles / 1e9, rel=1e-12)
+            assert_bits_equal(gpu.down(top), plain[0], "forward in three groups")
+        finally:
+            assert gpu.L.mnv_conv_winograd_profile(0) == 0
+        assert _profile_read(gpu, 0)[0] == 3          # still readable after switching off
+        cv.fwd(x, w, b)
+        assert _profile_read(gpu, 0)[0] == 3          # and nothing is recorded while it is off
+        assert gpu.L.mnv_conv_winograd_profile(1) == 0 and gpu.L.mnv_conv_winograd_profile(0) == 0
+        assert _profile_read(gpu, 0)[0] == 0
+
+
 def test_winograd_is_taken_by_itself_where_it_pays(gpu):
     """In the initial mode a 3 x 3 layer whose multiplies outweigh the transformed tensors'
     traffic takes the path without being asked (256 -> 256 channels, 72 images of 13 x 13); the
